@@ -1,0 +1,256 @@
+/*
+ * rmlk_hip.h -- C ABI of librmlk_hip, the gfx950 (MI355X / CDNA4) kernel library that stands where
+ * the reference's `rmlk-cuda` kernel crate stands: below the runtime's operator dispatch.
+ *
+ * Each entry point names the reference interface it replaces as `ref: file:line` (paths relative
+ * to the reference repository root).
+ *
+ * Conventions (all entry points):
+ *   - Returns an int32 status: 0 = ok; > 0 = a hipError_t raised by the launch; < 0 = an argument
+ *     error from `rmlk_status`.
+ *   - Every pointer named `a`, `b`, `in`, `out`, `data`, ... is DEVICE memory owned by the caller.
+ *     `rmlk_dims` / attribute arrays are HOST memory, read before the call returns.
+ *   - Work is enqueued on `stream` (a hipStream_t; NULL = the default stream). No entry point
+ *     synchronises, allocates device memory or keeps a reference to host arguments after it returns
+ *     (the memory helpers at the end are the exception and say so).
+ *   - Tensors are dense row-major unless a stride argument says otherwise. Strides are in ELEMENTS.
+ *   - A call whose output has zero elements returns 0 without launching.
+ *   - No global mutable state: calls on distinct streams may be made from distinct threads.
+ */
+#ifndef RMLK_HIP_H
+#define RMLK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RMLK_MAX_RANK 8 /* ref: cuda/src/kernels/slice.rs:88 (rank <= 8) */
+
+typedef void *rmlk_stream_t; /* hipStream_t */
+
+typedef enum rmlk_status {
+    RMLK_OK = 0,
+    RMLK_ERR_BAD_RANK = -1,        /* rank outside 1..RMLK_MAX_RANK */
+    RMLK_ERR_UNSUPPORTED = -2,     /* dtype / op combination has no kernel ("unsupported data type") */
+    RMLK_ERR_NULL_POINTER = -3,    /* null pointer with a non-zero length */
+    RMLK_ERR_SIZE_MISMATCH = -4,   /* shapes / lengths disagree */
+    RMLK_ERR_INVALID_ARGUMENT = -5,/* bad axis, perm, step 0, negative dim ... */
+    RMLK_ERR_WORKSPACE = -6,       /* workspace smaller than rmlk_hip_matmul_workspace_size says */
+    RMLK_ERR_TOO_LARGE = -7        /* more elements than the kernels index (>= 2^62) */
+} rmlk_status;
+
+/* Element types. Values are the ONNX TensorProto.DataType numbers the reference maps its
+ * `schema::DataType` to (ref: schema/src/tensor.rs:404-430). */
+typedef enum rmlk_dtype {
+    RMLK_FLOAT = 1,
+    RMLK_UINT8 = 2,
+    RMLK_INT8 = 3,
+    RMLK_UINT16 = 4,
+    RMLK_INT16 = 5,
+    RMLK_INT32 = 6,
+    RMLK_INT64 = 7,
+    RMLK_BOOL = 9, /* one byte, 0 or 1 on output; any non-zero byte is true on input */
+    RMLK_FLOAT16 = 10,
+    RMLK_DOUBLE = 11,
+    RMLK_UINT32 = 12,
+    RMLK_UINT64 = 13
+} rmlk_dtype;
+
+/* Shape or stride vector passed by value from the host; replaces the device `info` buffers the
+ * reference uploads per call (ref: runtime/src/providers/cuda/backend/binary.rs:114-131). */
+typedef struct rmlk_dims {
+    int32_t rank;
+    int64_t v[RMLK_MAX_RANK];
+} rmlk_dims;
+
+/* ---------------------------------------------------------------------------------------------
+ * Broadcast binary ops.
+ * ref: cuda/src/kernels/binary.rs:27-100 (compute / compute_with_diff_output / compute_with_types)
+ *      cuda/src/ptx/headers/binary_op_macros.cuh:14-42, ptx/{add,sub,mul,div,pow,equal,greater}.cu
+ * out[i] = a[ia] (op) b[ib]; `out_shape` is the broadcast shape, `a_stride` / `b_stride` hold the
+ * operand's element stride per output dim with 0 on broadcast dims (the meaning of the reference's
+ * info buffer, ref: runtime/src/utils/mod.rs:56-91). `out` is dense.
+ *   ADD SUB MUL DIV : dtype_a == dtype_b in {FLOAT, DOUBLE, INT32, INT64}; out dtype = dtype_a.
+ *                     Integer DIV truncates toward zero; x/0 yields 0 for integers (never traps).
+ *   POW             : dtype_a (base) in {FLOAT, DOUBLE, INT32, INT64}, dtype_b (exponent) in
+ *                     {FLOAT, DOUBLE, INT32, INT64}; out dtype = dtype_a. Float bases with exponent
+ *                     2, 3, 0.5 use x*x, x*x*x, sqrt(x); integer bases round llround(pow(double)).
+ *   EQUAL GREATER   : dtype_a == dtype_b in {FLOAT, DOUBLE, INT32, INT64}; out dtype = BOOL (0/1).
+ */
+typedef enum rmlk_binary_op {
+    RMLK_ADD = 0,
+    RMLK_SUB = 1,
+    RMLK_MUL = 2,
+    RMLK_DIV = 3,
+    RMLK_POW = 4,
+    RMLK_EQUAL = 5,
+    RMLK_GREATER = 6
+} rmlk_binary_op;
+
+int32_t rmlk_hip_binary(rmlk_stream_t stream, int32_t op, int32_t dtype_a, int32_t dtype_b,
+                        const rmlk_dims *out_shape, const rmlk_dims *a_stride,
+                        const rmlk_dims *b_stride, const void *a, const void *b, void *out);
+
+/* Where: out[i] = cond[ic] ? x[ix] : y[iy], three-way broadcast, pure move (NaN payloads kept).
+ * ref: cuda/src/kernels/whereop.rs:57-101, cuda/src/ptx/headers/ternary_op_macro.cuh:1-34.
+ * dtype (of x, y, out) in {FLOAT, DOUBLE, INT32, INT64, and any 1/2/4/8-byte type}; cond is BOOL. */
+int32_t rmlk_hip_where(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *out_shape,
+                       const rmlk_dims *x_stride, const rmlk_dims *y_stride,
+                       const rmlk_dims *cond_stride, const void *x, const void *y,
+                       const void *cond, void *out);
+
+/* Contiguous unary maps.
+ * ref: cuda/src/kernels/unary.rs:10-42, cuda/src/ptx/headers/unary_op_macro.cuh:1-11,
+ *      ptx/{sqrt,neg,sin,cos}.cu; sigmoid replaces cuDNN (cuda/src/kernels/sigmoid.rs:7-29).
+ * SQRT SIN COS SIGMOID: FLOAT, DOUBLE. NEG: FLOAT, DOUBLE, INT32, INT64 (sign flip). */
+typedef enum rmlk_unary_op {
+    RMLK_SQRT = 0,
+    RMLK_NEG = 1,
+    RMLK_SIN = 2,
+    RMLK_COS = 3,
+    RMLK_SIGMOID = 4
+} rmlk_unary_op;
+
+int32_t rmlk_hip_unary(rmlk_stream_t stream, int32_t op, int32_t dtype, int64_t n, const void *in,
+                       void *out);
+
+/* Cast: C static_cast semantics (float -> int truncates toward zero and saturates; to BOOL is
+ * x != 0; from BOOL is 0/1). Any pair over {FLOAT, DOUBLE, FLOAT16, INT8..INT64, UINT8..UINT64,
+ * BOOL}. ref: cuda/src/kernels/unary.rs:47-80, cuda/src/ptx/cast.cu:6-124. */
+int32_t rmlk_hip_cast(rmlk_stream_t stream, int32_t src_dtype, int32_t dst_dtype, int64_t n,
+                      const void *in, void *out);
+
+/* ReduceMean over `axes` (normalised, distinct, 0 <= axis < rank) of a dense tensor; `out` is dense
+ * over the kept dims in order (keepdims only changes the shape the host records). Accumulates in
+ * double like the reference. dtype in {FLOAT, DOUBLE}.
+ * ref: cuda/src/kernels/reduce_mean.rs:40-93, cuda/src/ptx/headers/aggregation_op_macros.cuh:1-49. */
+int32_t rmlk_hip_reduce_mean(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *in_shape,
+                             const int64_t *axes, int32_t n_axes, const void *in, void *out);
+
+/* Softmax along the middle axis of a dense [outer, axis_len, inner] view (inner == 1 is the
+ * last-axis case; outer=N, axis_len=C, inner=H*W is the reference's rank-4 channel mode).
+ * Max-subtracted: exp(x - max) / sum. dtype in {FLOAT, DOUBLE}.
+ * ref: cuda/src/kernels/softmax.rs:5-37 (cuDNN), runtime/src/providers/cuda/backend/softmax.rs:121-158 */
+int32_t rmlk_hip_softmax(rmlk_stream_t stream, int32_t dtype, int64_t outer, int64_t axis_len,
+                         int64_t inner, const void *in, void *out);
+
+/* Batched MatMul, row-major: C[b] = op(A[b]) . op(B[b]), op = transpose when trans_x != 0.
+ * A is m x k (k x m when trans_a) with leading dimension lda, B is k x n (n x k when trans_b) with
+ * ldb, C is m x n with ldc. stride_x is the element distance between batches; 0 broadcasts one
+ * matrix over the batch (the reference copies the operand `batch` times instead,
+ * ref: runtime/src/providers/cuda/backend/matmul.rs:48-86). fp32 in, fp32 accumulate. dtype FLOAT.
+ * `workspace` is device scratch of at least rmlk_hip_matmul_workspace_size(...) bytes (may be NULL
+ * when that is 0); it is only written and read inside the call's own stream order.
+ * ref: cuda/src/kernels/gemm.rs:112-136,191-232 (cublasGemmStridedBatchedEx). */
+int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t m, int64_t n,
+                        int64_t k, const void *a, int64_t lda, int64_t stride_a, int32_t trans_a,
+                        const void *b, int64_t ldb, int64_t stride_b, int32_t trans_b, void *c,
+                        int64_t ldc, int64_t stride_c, void *workspace, size_t workspace_bytes);
+
+size_t rmlk_hip_matmul_workspace_size(int32_t dtype, int64_t batch, int64_t m, int64_t n,
+                                      int64_t k);
+
+/* Transpose: out = permute(in, perm); out.shape[d] = in_shape[perm[d]]. Any 1/2/4/8-byte dtype.
+ * ref: cuda/src/kernels/transpose.rs:38-80, cuda/src/ptx/headers/transpose_op_macros.cuh:1-25. */
+int32_t rmlk_hip_transpose(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *in_shape,
+                           const int64_t *perm, const void *in, void *out);
+
+/* Expand: broadcast-copy `in` (in_shape, right-aligned, dims of 1 repeat) to dense `out_shape`.
+ * ref: cuda/src/kernels/expand.rs:35-76, cuda/src/ptx/headers/expand_op_macros.cuh:1-31. */
+int32_t rmlk_hip_expand(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *in_shape,
+                        const rmlk_dims *out_shape, const void *in, void *out);
+
+/* Slice with the ONNX clamp rules already applied by the host: for every dim d,
+ * out[.., o_d, ..] = in[.., starts[d] + o_d * steps[d], ..], 0 <= o_d < out_shape[d]. steps may be
+ * negative; the caller guarantees every addressed index lies in [0, in_shape[d]) (checked).
+ * ref: cuda/src/kernels/slice.rs:61-122, cuda/src/ptx/headers/slice_op_macros.cuh:1-97; the clamp
+ * rules the host applies are runtime/src/providers/cuda/backend/slice.rs:357-463. */
+int32_t rmlk_hip_slice(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *in_shape,
+                       const rmlk_dims *starts, const rmlk_dims *steps, const rmlk_dims *out_shape,
+                       const void *in, void *out);
+
+/* Concat, one call per input: copies dense `in` (in_shape) into dense `out` (out_shape) at
+ * `axis_offset` along `axis`. A zero-length input is legal and launches nothing.
+ * ref: runtime/src/providers/cuda/backend/concat.rs:28-76 (a host loop of memcpy_dtod). */
+int32_t rmlk_hip_concat(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *in_shape,
+                        const rmlk_dims *out_shape, int32_t axis, int64_t axis_offset,
+                        const void *in, void *out);
+
+/* Gather along `axis`: out[outer, j, inner] = data[outer, idx[j], inner], j < n_idx; negative
+ * indices wrap once. idx_dtype INT32 or INT64. An index outside [-dim, dim) writes zeros for that
+ * row and stores 1 to *err_flag (device int32, may be NULL); the host reads it when it chooses.
+ * ref: runtime/src/providers/cuda/backend/gather.rs:199-258 (index D2H + one memcpy_dtod per
+ * index), index rule runtime/src/utils/mod.rs:155-175. */
+int32_t rmlk_hip_gather(rmlk_stream_t stream, int32_t dtype, int32_t idx_dtype,
+                        const rmlk_dims *data_shape, int32_t axis, int64_t n_idx, const void *data,
+                        const void *idx, void *out, int32_t *err_flag);
+
+/* ScatterND. `out` must already hold a copy of `data` (or be `data` itself for an in-place
+ * update); this call writes only the addressed slices. idx is INT64 [n_tuples, tuple_size],
+ * updates is [n_tuples, slice_len] with slice_len = prod(data_shape[tuple_size:]). Negative
+ * indices wrap once; an index outside [-dim, dim) skips the tuple and stores 1 to *err_flag.
+ * NONE is plain assignment (the reference's `in + 0*out` turns Inf/NaN already in `data` into
+ * NaN; ONNX does not). ADD MUL MAX MIN are atomic per element, so duplicates combine in an
+ * unspecified order. dtype in {FLOAT, DOUBLE, INT32, INT64} (NONE: any 1/2/4/8-byte type).
+ * ref: cuda/src/kernels/scatter_nd.rs:91-210, cuda/src/ptx/headers/scatter_op_macros.cuh:19-93. */
+typedef enum rmlk_scatter_reduction {
+    RMLK_SCATTER_NONE = 0,
+    RMLK_SCATTER_ADD = 1,
+    RMLK_SCATTER_MUL = 2,
+    RMLK_SCATTER_MAX = 3,
+    RMLK_SCATTER_MIN = 4
+} rmlk_scatter_reduction;
+
+int32_t rmlk_hip_scatter_nd(rmlk_stream_t stream, int32_t reduction, int32_t dtype,
+                            const rmlk_dims *data_shape, int64_t n_tuples, int32_t tuple_size,
+                            const int64_t *idx, const void *updates, void *out,
+                            int32_t *err_flag);
+
+/* Trilu on a dense [batch, rows, cols] view: keeps the upper (col >= row + k) or lower
+ * (col <= row + k) triangle and WRITES ZERO elsewhere (the reference leaves those untouched).
+ * ref: cuda/src/kernels/trilu.rs:36-78, cuda/src/ptx/headers/trilu_op_macros.cuh:1-43. */
+int32_t rmlk_hip_trilu(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t rows,
+                       int64_t cols, int32_t upper, int64_t k, const void *in, void *out);
+
+/* Fill `n` elements of `out` with the element at host address `value` (size of dtype).
+ * ref: runtime/src/providers/cuda/backend/constant_of_shape.rs:59-62 (host vector + H2D). */
+int32_t rmlk_hip_fill(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *value,
+                      void *out);
+
+/* ---------------------------------------------------------------------------------------------
+ * Memory and stream helpers (what the provider used cudarc for,
+ * ref: runtime/src/providers/cuda/allocator.rs:96-139, data.rs:24-25, store.rs:385-416).
+ * These DO call the HIP allocator / synchronise as named. */
+int32_t rmlk_hip_malloc(void **ptr, size_t bytes);
+int32_t rmlk_hip_free(void *ptr);
+int32_t rmlk_hip_memcpy_htod(rmlk_stream_t stream, void *dst, const void *src, size_t bytes);
+int32_t rmlk_hip_memcpy_dtoh(rmlk_stream_t stream, void *dst, const void *src, size_t bytes);
+int32_t rmlk_hip_memcpy_dtod(rmlk_stream_t stream, void *dst, const void *src, size_t bytes);
+int32_t rmlk_hip_memset(rmlk_stream_t stream, void *dst, int32_t byte, size_t bytes);
+int32_t rmlk_hip_stream_sync(rmlk_stream_t stream);
+
+typedef struct rmlk_device_info {
+    char name[128];
+    char arch[64];
+    int32_t compute_units;
+    int32_t wavefront_size;
+    int32_t lds_bytes_per_block;
+    int32_t clock_khz;
+    int64_t total_mem_bytes;
+} rmlk_device_info;
+
+int32_t rmlk_hip_device_info(int32_t device, rmlk_device_info *info);
+
+/* Human-readable name of a status (static string). */
+const char *rmlk_hip_status_string(int32_t status);
+
+/* Library version, "major.minor.patch". */
+const char *rmlk_hip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RMLK_HIP_H */

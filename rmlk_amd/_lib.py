@@ -1,0 +1,118 @@
+"""ctypes binding of librmlk_hip.so (the C ABI declared in include/rmlk_hip.h)."""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_int32, c_int64, c_size_t, c_void_p
+
+MAX_RANK = 8
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+class LibraryNotBuilt(RuntimeError):
+    """librmlk_hip.so is missing: build it with `make -C rmlk_amd/csrc` (or __graft_entry__.build)."""
+
+
+class RmlkError(RuntimeError):
+    """A C-ABI entry point returned a non-zero status."""
+
+    def __init__(self, status: int, message: str, where: str):
+        super().__init__(f"{where}: {message} (status {status})")
+        self.status = status
+        self.message = message
+
+
+class Dims(ctypes.Structure):
+    """struct rmlk_dims"""
+    _fields_ = [("rank", c_int32), ("v", c_int64 * MAX_RANK)]
+
+    @staticmethod
+    def of(values) -> "Dims":
+        values = [int(v) for v in values]
+        if len(values) > MAX_RANK:
+            raise RmlkError(-1, "rank outside 1..8", "rmlk_dims")
+        d = Dims()
+        d.rank = len(values)
+        for i, v in enumerate(values):
+            d.v[i] = v
+        return d
+
+
+class DeviceInfo(ctypes.Structure):
+    """struct rmlk_device_info"""
+    _fields_ = [("name", ctypes.c_char * 128), ("arch", ctypes.c_char * 64),
+                ("compute_units", c_int32), ("wavefront_size", c_int32),
+                ("lds_bytes_per_block", c_int32), ("clock_khz", c_int32),
+                ("total_mem_bytes", c_int64)]
+
+
+def library_path() -> str:
+    return os.path.join(_HERE, "lib", "librmlk_hip.so")
+
+
+# name -> (restype, argtypes); every symbol include/rmlk_hip.h declares
+_PD = POINTER(Dims)
+SIGNATURES = {
+    "rmlk_hip_binary": (c_int32, [c_void_p, c_int32, c_int32, c_int32, _PD, _PD, _PD, c_void_p,
+                                  c_void_p, c_void_p]),
+    "rmlk_hip_where": (c_int32, [c_void_p, c_int32, _PD, _PD, _PD, _PD, c_void_p, c_void_p,
+                                 c_void_p, c_void_p]),
+    "rmlk_hip_unary": (c_int32, [c_void_p, c_int32, c_int32, c_int64, c_void_p, c_void_p]),
+    "rmlk_hip_cast": (c_int32, [c_void_p, c_int32, c_int32, c_int64, c_void_p, c_void_p]),
+    "rmlk_hip_reduce_mean": (c_int32, [c_void_p, c_int32, _PD, POINTER(c_int64), c_int32, c_void_p,
+                                       c_void_p]),
+    "rmlk_hip_softmax": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p,
+                                   c_void_p]),
+    "rmlk_hip_matmul": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_void_p,
+                                  c_int64, c_int64, c_int32, c_void_p, c_int64, c_int64, c_int32,
+                                  c_void_p, c_int64, c_int64, c_void_p, c_size_t]),
+    "rmlk_hip_matmul_workspace_size": (c_size_t, [c_int32, c_int64, c_int64, c_int64, c_int64]),
+    "rmlk_hip_transpose": (c_int32, [c_void_p, c_int32, _PD, POINTER(c_int64), c_void_p,
+                                     c_void_p]),
+    "rmlk_hip_expand": (c_int32, [c_void_p, c_int32, _PD, _PD, c_void_p, c_void_p]),
+    "rmlk_hip_slice": (c_int32, [c_void_p, c_int32, _PD, _PD, _PD, _PD, c_void_p, c_void_p]),
+    "rmlk_hip_concat": (c_int32, [c_void_p, c_int32, _PD, _PD, c_int32, c_int64, c_void_p,
+                                  c_void_p]),
+    "rmlk_hip_gather": (c_int32, [c_void_p, c_int32, c_int32, _PD, c_int32, c_int64, c_void_p,
+                                  c_void_p, c_void_p, c_void_p]),
+    "rmlk_hip_scatter_nd": (c_int32, [c_void_p, c_int32, c_int32, _PD, c_int64, c_int32, c_void_p,
+                                      c_void_p, c_void_p, c_void_p]),
+    "rmlk_hip_trilu": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int32, c_int64,
+                                 c_void_p, c_void_p]),
+    "rmlk_hip_fill": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
+    "rmlk_hip_malloc": (c_int32, [POINTER(c_void_p), c_size_t]),
+    "rmlk_hip_free": (c_int32, [c_void_p]),
+    "rmlk_hip_memcpy_htod": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
+    "rmlk_hip_memcpy_dtoh": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
+    "rmlk_hip_memcpy_dtod": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
+    "rmlk_hip_memset": (c_int32, [c_void_p, c_void_p, c_int32, c_size_t]),
+    "rmlk_hip_stream_sync": (c_int32, [c_void_p]),
+    "rmlk_hip_device_info": (c_int32, [c_int32, POINTER(DeviceInfo)]),
+    "rmlk_hip_status_string": (c_char_p, [c_int32]),
+    "rmlk_hip_version": (c_char_p, []),
+}
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library; raises LibraryNotBuilt when the HIP extension has not been built."""
+    global _lib
+    if _lib is None:
+        path = library_path()
+        if not os.path.exists(path):
+            raise LibraryNotBuilt(f"{path} not found; there is no CPU fallback")
+        handle = ctypes.CDLL(path)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def check(status: int, where: str) -> None:
+    if status != 0:
+        msg = lib().rmlk_hip_status_string(status)
+        raise RmlkError(status, msg.decode() if msg else "unknown", where)

@@ -1,0 +1,91 @@
+// Memory, stream and device helpers of the C ABI, plus status strings.
+// What the reference's provider reaches through cudarc: allocation
+// (runtime/src/providers/cuda/allocator.rs:96-139), host/device copies
+// (runtime/src/providers/cuda/store.rs:385-416) and the blocking readback of outputs
+// (runtime/src/core/execution_state.rs:201-225).
+#include <cstring>
+
+#include "common.hpp"
+
+using namespace rmlk;
+
+extern "C" int32_t rmlk_hip_malloc(void **ptr, size_t bytes) {
+    if (!ptr) return RMLK_ERR_NULL_POINTER;
+    *ptr = nullptr;
+    if (bytes == 0) return RMLK_OK;
+    return static_cast<int32_t>(hipMalloc(ptr, bytes));
+}
+
+extern "C" int32_t rmlk_hip_free(void *ptr) {
+    if (!ptr) return RMLK_OK;
+    return static_cast<int32_t>(hipFree(ptr));
+}
+
+extern "C" int32_t rmlk_hip_memcpy_htod(rmlk_stream_t stream, void *dst, const void *src,
+                                        size_t bytes) {
+    if (bytes == 0) return RMLK_OK;
+    if (!dst || !src) return RMLK_ERR_NULL_POINTER;
+    return static_cast<int32_t>(
+        hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+}
+
+extern "C" int32_t rmlk_hip_memcpy_dtoh(rmlk_stream_t stream, void *dst, const void *src,
+                                        size_t bytes) {
+    if (bytes == 0) return RMLK_OK;
+    if (!dst || !src) return RMLK_ERR_NULL_POINTER;
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(stream));
+    if (e != hipSuccess) return static_cast<int32_t>(e);
+    return static_cast<int32_t>(hipStreamSynchronize(as_stream(stream)));
+}
+
+extern "C" int32_t rmlk_hip_memcpy_dtod(rmlk_stream_t stream, void *dst, const void *src,
+                                        size_t bytes) {
+    if (bytes == 0) return RMLK_OK;
+    if (!dst || !src) return RMLK_ERR_NULL_POINTER;
+    return static_cast<int32_t>(
+        hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+}
+
+extern "C" int32_t rmlk_hip_memset(rmlk_stream_t stream, void *dst, int32_t byte, size_t bytes) {
+    if (bytes == 0) return RMLK_OK;
+    if (!dst) return RMLK_ERR_NULL_POINTER;
+    return static_cast<int32_t>(hipMemsetAsync(dst, byte, bytes, as_stream(stream)));
+}
+
+extern "C" int32_t rmlk_hip_stream_sync(rmlk_stream_t stream) {
+    return static_cast<int32_t>(hipStreamSynchronize(as_stream(stream)));
+}
+
+extern "C" int32_t rmlk_hip_device_info(int32_t device, rmlk_device_info *info) {
+    if (!info) return RMLK_ERR_NULL_POINTER;
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return static_cast<int32_t>(e);
+    std::memset(info, 0, sizeof(*info));
+    std::strncpy(info->name, prop.name, sizeof(info->name) - 1);
+    std::strncpy(info->arch, prop.gcnArchName, sizeof(info->arch) - 1);
+    info->compute_units = prop.multiProcessorCount;
+    info->wavefront_size = prop.warpSize;
+    info->lds_bytes_per_block = static_cast<int32_t>(prop.sharedMemPerBlock);
+    info->clock_khz = prop.clockRate;
+    info->total_mem_bytes = static_cast<int64_t>(prop.totalGlobalMem);
+    return RMLK_OK;
+}
+
+extern "C" const char *rmlk_hip_status_string(int32_t status) {
+    switch (status) {
+        case RMLK_OK: return "ok";
+        case RMLK_ERR_BAD_RANK: return "rank outside 1..8";
+        case RMLK_ERR_UNSUPPORTED: return "unsupported data type";
+        case RMLK_ERR_NULL_POINTER: return "null pointer with non-zero length";
+        case RMLK_ERR_SIZE_MISMATCH: return "size mismatch";
+        case RMLK_ERR_INVALID_ARGUMENT: return "invalid argument";
+        case RMLK_ERR_WORKSPACE: return "workspace too small";
+        case RMLK_ERR_TOO_LARGE: return "tensor too large";
+        default:
+            if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
+            return "unknown status";
+    }
+}
+
+extern "C" const char *rmlk_hip_version(void) { return "0.1.0"; }

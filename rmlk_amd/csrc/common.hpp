@@ -1,0 +1,173 @@
+// Shared host/device helpers for the gfx950 kernel library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/rmlk_hip.h"
+
+namespace rmlk {
+
+constexpr int kMaxRank = RMLK_MAX_RANK;
+constexpr int kWave = 64;         // CDNA wavefront width
+constexpr int kNumCU = 256;       // MI355X compute units (8 XCDs x 32)
+constexpr int64_t kMaxElems = (int64_t)1 << 62;
+
+inline hipStream_t as_stream(rmlk_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Status of the launch just issued (hipError_t as a positive int, 0 when fine).
+inline int32_t launch_status() { return static_cast<int32_t>(hipGetLastError()); }
+
+inline int dtype_size(int32_t dt) {
+    switch (dt) {
+        case RMLK_BOOL:
+        case RMLK_UINT8:
+        case RMLK_INT8: return 1;
+        case RMLK_UINT16:
+        case RMLK_INT16:
+        case RMLK_FLOAT16: return 2;
+        case RMLK_FLOAT:
+        case RMLK_INT32:
+        case RMLK_UINT32: return 4;
+        case RMLK_DOUBLE:
+        case RMLK_INT64:
+        case RMLK_UINT64: return 8;
+        default: return 0;
+    }
+}
+
+inline bool dims_ok(const rmlk_dims *d) { return d && d->rank >= 1 && d->rank <= kMaxRank; }
+
+// Product of dims, -1 when a dim is negative or the product overflows kMaxElems.
+inline int64_t dims_numel(const rmlk_dims *d) {
+    int64_t n = 1;
+    for (int i = 0; i < d->rank; ++i) {
+        if (d->v[i] < 0) return -1;
+        if (d->v[i] == 0) return 0;
+    }
+    for (int i = 0; i < d->rank; ++i) {
+        if (n > kMaxElems / d->v[i]) return -1;
+        n *= d->v[i];
+    }
+    return n;
+}
+
+// Unsigned division by a runtime constant through one mul-high and a shift.
+// Exact for dividends below 2^31 (the kernels use it only on 32-bit index paths).
+struct FastDiv {
+    uint32_t d, mul, shr;
+    FastDiv() : d(1), mul(0), shr(0) {}
+    explicit FastDiv(uint32_t div) : d(div), mul(0), shr(0) {
+        if (div > 1) {
+            uint32_t lg = 0;
+            while ((1ull << lg) < div) ++lg;
+            uint32_t p = 31 + lg;
+            mul = static_cast<uint32_t>(((1ull << p) + div - 1) / div);
+            shr = p - 32;
+        }
+    }
+    __host__ __device__ __forceinline__ uint32_t div(uint32_t n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+        return d == 1 ? n : (__umulhi(n, mul) >> shr);
+#else
+        return d == 1 ? n : static_cast<uint32_t>((static_cast<uint64_t>(n) * mul) >> 32) >> shr;
+#endif
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// N-d iteration plan: one logical shape, element strides for up to NP operands (inputs and the
+// output alike). The host removes size-1 dims and merges dims that are jointly contiguous in every
+// operand, so dense same-shape work collapses to rank 1 and `[8,32,512,64] (.) [1,32,1,64]` keeps
+// four dims with a contiguous innermost run.
+template <int NP>
+struct NdPlan {
+    int32_t rank;                    // >= 1 after coalescing
+    uint32_t dim[kMaxRank];          // dim[rank-1] is innermost
+    int64_t dim64[kMaxRank];
+    FastDiv fdiv[kMaxRank];
+    int64_t stride[NP][kMaxRank];    // element strides, may be 0 or negative
+    int64_t numel;
+};
+
+// Build a coalesced plan. shape[rank], strides[p][rank]. Returns false when numel == 0.
+template <int NP>
+inline bool build_plan(NdPlan<NP> &pl, int rank, const int64_t *shape,
+                       const int64_t (*strides)[kMaxRank]) {
+    int64_t shp[kMaxRank];
+    int64_t st[NP][kMaxRank];
+    int r = 0;
+    int64_t numel = 1;
+    for (int d = 0; d < rank; ++d) numel *= shape[d];
+    pl.numel = numel;
+    if (numel == 0) return false;
+    for (int d = 0; d < rank; ++d) {
+        if (shape[d] == 1) continue;
+        shp[r] = shape[d];
+        for (int p = 0; p < NP; ++p) st[p][r] = strides[p][d];
+        ++r;
+    }
+    if (r == 0) {
+        r = 1;
+        shp[0] = 1;
+        for (int p = 0; p < NP; ++p) st[p][0] = 1;
+    }
+    // merge dim d into d+1 when every operand walks them as one run
+    int w = 0;  // write index of the current (outer-most so far) merged dim
+    int64_t mshp[kMaxRank];
+    int64_t mst[NP][kMaxRank];
+    mshp[0] = shp[0];
+    for (int p = 0; p < NP; ++p) mst[p][0] = st[p][0];
+    for (int d = 1; d < r; ++d) {
+        bool can = true;
+        for (int p = 0; p < NP; ++p)
+            if (mst[p][w] != st[p][d] * shp[d]) { can = false; break; }
+        if (can) {
+            mshp[w] *= shp[d];
+            for (int p = 0; p < NP; ++p) mst[p][w] = st[p][d];
+        } else {
+            ++w;
+            mshp[w] = shp[d];
+            for (int p = 0; p < NP; ++p) mst[p][w] = st[p][d];
+        }
+    }
+    pl.rank = w + 1;
+    for (int d = 0; d < pl.rank; ++d) {
+        pl.dim64[d] = mshp[d];
+        pl.dim[d] = static_cast<uint32_t>(mshp[d]);
+        pl.fdiv[d] = FastDiv(static_cast<uint32_t>(mshp[d] > 0x7fffffff ? 1 : mshp[d]));
+        for (int p = 0; p < NP; ++p) pl.stride[p][d] = mst[p][d];
+    }
+    for (int d = pl.rank; d < kMaxRank; ++d) {
+        pl.dim64[d] = 1;
+        pl.dim[d] = 1;
+        pl.fdiv[d] = FastDiv(1);
+        for (int p = 0; p < NP; ++p) pl.stride[p][d] = 0;
+    }
+    return true;
+}
+
+inline void dense_strides(int rank, const int64_t *shape, int64_t *stride) {
+    int64_t s = 1;
+    for (int d = rank - 1; d >= 0; --d) {
+        stride[d] = s;
+        s *= shape[d];
+    }
+}
+
+// Grid size for a grid-stride kernel: enough blocks to cover `work` items, capped so that a few
+// waves per SIMD stay resident on all 256 CUs.
+inline unsigned grid_for(int64_t work, int block, int max_blocks_per_cu = 8) {
+    int64_t need = (work + block - 1) / block;
+    int64_t cap = static_cast<int64_t>(kNumCU) * max_blocks_per_cu;
+    if (need < 1) need = 1;
+    return static_cast<unsigned>(need < cap ? need : cap);
+}
+
+// N elements moved as one access; alignment is capped at the widest (128-bit) memory operation.
+template <typename T, int N>
+struct alignas(sizeof(T) * N > 16 ? 16 : sizeof(T) * N) Vec {
+    T v[N];
+};
+
+}  // namespace rmlk

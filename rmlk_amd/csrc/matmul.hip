@@ -1,0 +1,609 @@
+// Batched fp32 MatMul for gfx950: MFMA tiles staged through LDS for M > 1, an HBM-streaming GEMV
+// for the M == 1 decode shape. Replaces the cublasGemmStridedBatchedEx call of the reference
+// (cuda/src/kernels/gemm.rs:191-232) and the operand copies its MatMul backend makes to
+// broadcast a 2-D operand over the batch (runtime/src/providers/cuda/backend/matmul.rs:48-86):
+// a batch stride of 0 broadcasts in place.
+//
+// MFMA kernel (row-major, A[M,K] . B[K,N]):
+//   - a 256-lane block (4 wavefronts) owns a BM x BN tile of C and walks K in steps of BK;
+//   - global -> registers -> LDS with the next K-step's global loads in flight while the current
+//     one is multiplied (two LDS buffers, one barrier per step);
+//   - each wavefront owns a WM x WN sub-tile as (WM/32) x (WN/32) v_mfma_f32_32x32x2_f32
+//     accumulators. MFMA's 2-deep K is fed with a K-permutation inside every 8-wide K chunk: lanes
+//     0-31 take k = 0..3 and lanes 32-63 take k = 4..7 of the chunk, for A and B alike, so one
+//     128-bit LDS read of A serves four MFMAs and the sum over K is unchanged;
+//   - split-K (grid z) writes partial tiles to the workspace, a second kernel adds them in a
+//     fixed order, so results do not depend on scheduling.
+#include "common.hpp"
+
+namespace rmlk {
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+struct GemmArgs {
+    const float *a;
+    const float *b;
+    float *c;
+    int32_t m, n, k;
+    int64_t lda, ldb, ldc;
+    int64_t stride_a, stride_b, stride_c;  // batch strides (elements)
+    int32_t k_per_split;                   // K range of one z-slice (multiple of BK)
+    int32_t tiles_m, tiles_n;
+};
+
+constexpr int kThreads = 256;
+constexpr int kPadA = 4;  // floats of padding per LDS row of A
+constexpr int kPadB = 8;  // floats of padding per LDS row of B
+
+template <int BM, int BN, int BK>
+struct SmemLayout {
+    static constexpr int kAStride = BK + kPadA;
+    static constexpr int kBStride = BN + kPadB;
+    static constexpr int kAFloats = BM * kAStride;
+    static constexpr int kBFloats = BK * kBStride;
+    static constexpr int kBytes = 2 * (kAFloats + kBFloats) * 4;
+};
+
+// tile index -> (tile_m, tile_n). Consecutive hardware block ids go round-robin over the 8 XCDs,
+// each with a private L2; blocks are renumbered so that one XCD works on a compact group of
+// tiles that share rows of A and columns of B.
+__device__ __forceinline__ void tile_coords(const GemmArgs &g, int &tm, int &tn) {
+    const int n_tiles = g.tiles_m * g.tiles_n;
+    int pid = blockIdx.x;
+    constexpr int kXcd = 8;
+    if (n_tiles % kXcd == 0) {
+        const int per = n_tiles / kXcd;
+        pid = (pid % kXcd) * per + pid / kXcd;
+    }
+    // groups of kGroupM tile-rows swept column by column
+    constexpr int kGroupM = 4;
+    const int width = kGroupM * g.tiles_n;
+    const int group = pid / width;
+    const int first_m = group * kGroupM;
+    const int gsz = g.tiles_m - first_m < kGroupM ? g.tiles_m - first_m : kGroupM;
+    const int in_group = pid - group * width;
+    tm = first_m + in_group % gsz;
+    tn = in_group / gsz;
+}
+
+template <int BM, int BN, int BK, int WM, int WN, bool ALIGNED>
+__global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
+    using L = SmemLayout<BM, BN, BK>;
+    extern __shared__ __align__(16) float smem[];
+    float *As = smem;                     // [2][BM][kAStride]
+    float *Bs = smem + 2 * L::kAFloats;   // [2][BK][kBStride]
+
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int WAVES_N = BN / WN;
+    static_assert((BM / WM) * (BN / WN) == kThreads / kWave, "four wavefronts per block");
+    static_assert(BK % 8 == 0, "K chunks of 8");
+
+    // global -> LDS staging shapes: float4 per lane
+    constexpr int A_VECS_PER_ROW = BK / 4;
+    constexpr int A_ROWS_PER_PASS = kThreads / A_VECS_PER_ROW;
+    constexpr int A_PASSES = BM / A_ROWS_PER_PASS;
+    constexpr int B_VECS_PER_ROW = BN / 4;
+    constexpr int B_ROWS_PER_PASS = kThreads / B_VECS_PER_ROW;
+    constexpr int B_PASSES = BK / B_ROWS_PER_PASS;
+    static_assert(A_PASSES >= 1 && B_PASSES >= 1, "tile too small for 256 lanes");
+
+    int tile_m, tile_n;
+    tile_coords(g, tile_m, tile_n);
+    const int batch = blockIdx.y;
+    const int split = blockIdx.z;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int k_begin = split * g.k_per_split;
+    const int k_end = min(g.k, k_begin + g.k_per_split);
+
+    const float *A = g.a + batch * g.stride_a;
+    const float *B = g.b + batch * g.stride_b;
+    float *C = g.c + (static_cast<int64_t>(split) * gridDim.y + batch) * g.stride_c;
+
+    const int tid = threadIdx.x;
+    const int lane = tid % kWave;
+    const int wave = tid / kWave;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int l32 = lane % 32, half = lane / 32;
+
+    const int a_vec = tid % A_VECS_PER_ROW, a_row = tid / A_VECS_PER_ROW;
+    const int b_vec = tid % B_VECS_PER_ROW, b_row = tid / B_VECS_PER_ROW;
+
+    v4f a_reg[A_PASSES], b_reg[B_PASSES];
+
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int p = 0; p < A_PASSES; ++p) {
+            const int r = m0 + a_row + p * A_ROWS_PER_PASS;
+            const int kk = k0 + a_vec * 4;
+            v4f v = {0.f, 0.f, 0.f, 0.f};
+            if (r < g.m) {
+                const float *src = A + static_cast<int64_t>(r) * g.lda + kk;
+                if (ALIGNED && kk + 3 < k_end) {
+                    v = *reinterpret_cast<const v4f *>(src);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (kk + j < k_end) v[j] = src[j];
+                }
+            }
+            a_reg[p] = v;
+        }
+#pragma unroll
+        for (int p = 0; p < B_PASSES; ++p) {
+            const int kk = k0 + b_row + p * B_ROWS_PER_PASS;
+            const int c = n0 + b_vec * 4;
+            v4f v = {0.f, 0.f, 0.f, 0.f};
+            if (kk < k_end) {
+                const float *src = B + static_cast<int64_t>(kk) * g.ldb + c;
+                if (ALIGNED && c + 3 < g.n) {
+                    v = *reinterpret_cast<const v4f *>(src);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (c + j < g.n) v[j] = src[j];
+                }
+            }
+            b_reg[p] = v;
+        }
+    };
+    auto store_lds = [&](int buf) {
+        float *as = As + buf * L::kAFloats;
+        float *bs = Bs + buf * L::kBFloats;
+#pragma unroll
+        for (int p = 0; p < A_PASSES; ++p)
+            *reinterpret_cast<v4f *>(as + (a_row + p * A_ROWS_PER_PASS) * L::kAStride +
+                                     a_vec * 4) = a_reg[p];
+#pragma unroll
+        for (int p = 0; p < B_PASSES; ++p)
+            *reinterpret_cast<v4f *>(bs + (b_row + p * B_ROWS_PER_PASS) * L::kBStride +
+                                     b_vec * 4) = b_reg[p];
+    };
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int n_steps = (k_end - k_begin + BK - 1) / BK;
+    if (n_steps > 0) {
+        load_global(k_begin);
+        store_lds(0);
+    }
+    __syncthreads();
+
+    for (int step = 0; step < n_steps; ++step) {
+        const int buf = step & 1;
+        const bool more = step + 1 < n_steps;
+        if (more) load_global(k_begin + (step + 1) * BK);
+
+        const float *as = As + buf * L::kAFloats + (wm * WM + l32) * L::kAStride + half * 4;
+        const float *bs = Bs + buf * L::kBFloats + (half * 4) * L::kBStride + wn * WN + l32;
+#pragma unroll
+        for (int kc = 0; kc < BK / 8; ++kc) {
+            v4f af[TM];
+            float bf[TN][4];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                af[i] = *reinterpret_cast<const v4f *>(as + i * 32 * L::kAStride + kc * 8);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) bf[j][s] = bs[(kc * 8 + s) * L::kBStride + j * 32];
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][s], bf[j][s],
+                                                                         acc[i][j], 0, 0, 0);
+        }
+        if (more) store_lds(buf ^ 1);
+        __syncthreads();
+    }
+
+    // C fragment: column = l32, row = 8 * (r / 4) + 4 * half + r % 4
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = n0 + wn * WN + j * 32 + l32;
+            if (col < g.n) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+                    if (row < g.m) C[static_cast<int64_t>(row) * g.ldc + col] = acc[i][j][r];
+                }
+            }
+        }
+    }
+}
+
+// Sum `splits` partial matrices laid out [split][batch][m][n] into C (fixed order).
+__global__ __launch_bounds__(kThreads) void splitk_reduce_kernel(const float *__restrict__ ws,
+                                                                 float *__restrict__ c, int splits,
+                                                                 int64_t batch, int32_t m,
+                                                                 int32_t n, int64_t ldc,
+                                                                 int64_t stride_c) {
+    const int64_t per = static_cast<int64_t>(m) * n;
+    const int64_t total = batch * per;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < total;
+         i += static_cast<int64_t>(gridDim.x) * kThreads) {
+        float s = 0.f;
+        for (int z = 0; z < splits; ++z) s += ws[z * total + i];
+        const int64_t b = i / per, rem = i - b * per;
+        const int64_t r = rem / n, col = rem - r * n;
+        c[b * stride_c + r * ldc + col] = s;
+    }
+}
+
+// ---- GEMV: y[n] = sum_k x[k] * W[k][n], W row-major -------------------------------------------
+// A block covers kThreads / 64 * ... columns: VEC columns per lane, 64 lanes per wavefront, and
+// the block's 4 wavefronts split the block's K slice; partial sums meet in LDS.
+struct GemvArgs {
+    const float *x;   // [batch][k], element stride x_inc
+    const float *w;
+    float *y;         // y or partial workspace [split][batch][n]
+    int32_t n, k;
+    int64_t x_inc, ldb;
+    int64_t stride_x, stride_w, stride_y;
+    int32_t k_per_split;
+};
+
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void gemv_kernel(GemvArgs g) {
+    constexpr int kWaves = kThreads / kWave;
+    constexpr int kCols = kWave * VEC;  // columns per block
+    __shared__ float red[kWaves][kCols];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int batch = blockIdx.y, split = blockIdx.z;
+    const int col = blockIdx.x * kCols + lane * VEC;
+    const int k_begin = split * g.k_per_split;
+    const int k_end = min(g.k, k_begin + g.k_per_split);
+    const float *x = g.x + batch * g.stride_x;
+    const float *w = g.w + batch * g.stride_w;
+
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+
+    // this wavefront's contiguous quarter of the slice
+    const int len = k_end - k_begin;
+    const int per_wave = (len + kWaves - 1) / kWaves;
+    const int kb = k_begin + wave * per_wave;
+    const int ke = min(k_end, kb + per_wave);
+    if (col < g.n) {
+        const float *wp = w + static_cast<int64_t>(kb) * g.ldb + col;
+        int kk = kb;
+        if constexpr (VEC == 4) {
+            constexpr int U = 8;
+            for (; kk + U <= ke; kk += U) {
+                v4f wv[U];
+                float xv[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    wv[u] = __builtin_nontemporal_load(
+                        reinterpret_cast<const v4f *>(wp + static_cast<int64_t>(u) * g.ldb));
+                    xv[u] = x[static_cast<int64_t>(kk + u) * g.x_inc];
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[j] = fmaf(xv[u], wv[u][j], acc[j]);
+                wp += static_cast<int64_t>(U) * g.ldb;
+            }
+            for (; kk < ke; ++kk) {
+                v4f wv = *reinterpret_cast<const v4f *>(wp);
+                float xv = x[static_cast<int64_t>(kk) * g.x_inc];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = fmaf(xv, wv[j], acc[j]);
+                wp += g.ldb;
+            }
+        } else {
+            constexpr int U = 8;
+            for (; kk + U <= ke; kk += U) {
+                float wv[U], xv[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    wv[u] = wp[static_cast<int64_t>(u) * g.ldb];
+                    xv[u] = x[static_cast<int64_t>(kk + u) * g.x_inc];
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) acc[0] = fmaf(xv[u], wv[u], acc[0]);
+                wp += static_cast<int64_t>(U) * g.ldb;
+            }
+            for (; kk < ke; ++kk) {
+                acc[0] = fmaf(x[static_cast<int64_t>(kk) * g.x_inc], *wp, acc[0]);
+                wp += g.ldb;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) red[wave][lane * VEC + j] = acc[j];
+    __syncthreads();
+    float *y = g.y + (static_cast<int64_t>(split) * gridDim.y + batch) * g.stride_y;
+    for (int c = threadIdx.x; c < kCols; c += kThreads) {
+        const int oc = blockIdx.x * kCols + c;
+        if (oc < g.n) {
+            float s = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < kWaves; ++wv) s += red[wv][c];
+            y[oc] = s;
+        }
+    }
+}
+
+// GEMV with W stored [n][k] (trans_b): a wavefront per output column, dot along contiguous k.
+__global__ __launch_bounds__(kThreads) void gemv_dot_kernel(GemvArgs g) {
+    const int lane = threadIdx.x % kWave;
+    const int batch = blockIdx.y;
+    const float *x = g.x + batch * g.stride_x;
+    const float *w = g.w + batch * g.stride_w;
+    float *y = g.y + batch * g.stride_y;
+    for (int n = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave; n < g.n;
+         n += gridDim.x * (kThreads / kWave)) {
+        const float *wr = w + static_cast<int64_t>(n) * g.ldb;
+        float acc = 0.f;
+        for (int kk = lane; kk < g.k; kk += kWave)
+            acc = fmaf(x[static_cast<int64_t>(kk) * g.x_inc], wr[kk], acc);
+#pragma unroll
+        for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, kWave);
+        if (lane == 0) y[n] = acc;
+    }
+}
+
+// Any-layout fallback (transposed operands with M > 1): one lane per C element.
+__global__ __launch_bounds__(kThreads) void gemm_naive_kernel(const float *__restrict__ a,
+                                                              const float *__restrict__ b,
+                                                              float *__restrict__ c, int64_t batch,
+                                                              int32_t m, int32_t n, int32_t k,
+                                                              int64_t a_rs, int64_t a_cs,
+                                                              int64_t b_rs, int64_t b_cs,
+                                                              int64_t ldc, int64_t stride_a,
+                                                              int64_t stride_b, int64_t stride_c) {
+    const int64_t per = static_cast<int64_t>(m) * n;
+    const int64_t total = batch * per;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < total;
+         i += static_cast<int64_t>(gridDim.x) * kThreads) {
+        const int64_t bb = i / per, rem = i - bb * per;
+        const int64_t r = rem / n, col = rem - r * n;
+        const float *pa = a + bb * stride_a + r * a_rs;
+        const float *pb = b + bb * stride_b + col * b_cs;
+        float s = 0.f;
+        for (int kk = 0; kk < k; ++kk) s = fmaf(pa[kk * a_cs], pb[kk * b_rs], s);
+        c[bb * stride_c + r * ldc + col] = s;
+    }
+}
+
+struct TileChoice {
+    int bm, bn;     // block tile
+    int splits;     // split-K factor
+    int k_per_split;
+};
+
+constexpr int kBK = 16;
+
+inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k) {
+    TileChoice t;
+    auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch; };
+    // big tiles when they alone fill the chip, else small tiles, else split K on top
+    if (tiles(128, 128) >= kNumCU) {
+        t.bm = 128;
+        t.bn = 128;
+    } else {
+        t.bm = 64;
+        t.bn = 64;
+    }
+    int64_t nt = tiles(t.bm, t.bn);
+    int splits = 1;
+    if (nt < kNumCU) {
+        splits = static_cast<int>((2 * kNumCU + nt - 1) / nt);
+        int64_t max_splits = k / (4 * kBK);
+        if (max_splits < 1) max_splits = 1;
+        if (splits > max_splits) splits = static_cast<int>(max_splits);
+        if (splits > 32) splits = 32;
+    }
+    int64_t kps = (k + splits - 1) / splits;
+    kps = (kps + kBK - 1) / kBK * kBK;
+    t.k_per_split = static_cast<int>(kps);
+    t.splits = static_cast<int>((k + kps - 1) / kps);
+    if (t.splits < 1) t.splits = 1;
+    return t;
+}
+
+inline int gemv_splits(int64_t batch, int64_t n, int64_t k, int cols_per_block, int *k_per_split) {
+    int64_t blocks = (n + cols_per_block - 1) / cols_per_block * batch;
+    int64_t splits = 1;
+    if (blocks < 4 * kNumCU) splits = (4 * kNumCU + blocks - 1) / blocks;
+    int64_t max_splits = k / 64;
+    if (max_splits < 1) max_splits = 1;
+    if (splits > max_splits) splits = max_splits;
+    if (splits > 64) splits = 64;
+    int64_t kps = (k + splits - 1) / splits;
+    kps = (kps + 7) / 8 * 8;
+    *k_per_split = static_cast<int>(kps);
+    return static_cast<int>((k + kps - 1) / kps);
+}
+
+template <int BM, int BN, int BK, int WM, int WN, bool ALIGNED>
+int32_t launch_mfma(hipStream_t s, const GemmArgs &g, int64_t batch, int splits) {
+    using L = SmemLayout<BM, BN, BK>;
+    auto kern = gemm_mfma_kernel<BM, BN, BK, WM, WN, ALIGNED>;
+    if (L::kBytes > 64 * 1024) {
+        static bool raised = false;  // benign race: same value from every thread
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               L::kBytes);
+            if (e != hipSuccess) return static_cast<int32_t>(e);
+            raised = true;
+        }
+    }
+    dim3 grid(static_cast<unsigned>(g.tiles_m * g.tiles_n), static_cast<unsigned>(batch),
+              static_cast<unsigned>(splits));
+    kern<<<grid, kThreads, L::kBytes, s>>>(g);
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace rmlk
+
+using namespace rmlk;
+
+extern "C" size_t rmlk_hip_matmul_workspace_size(int32_t dtype, int64_t batch, int64_t m,
+                                                 int64_t n, int64_t k) {
+    if (dtype != RMLK_FLOAT || batch <= 0 || m <= 0 || n <= 0 || k <= 0) return 0;
+    if (m == 1) {
+        // the larger of the two column widths the GEMV may pick
+        int kps;
+        int s4 = gemv_splits(batch, n, k, kWave * 4, &kps);
+        int s1 = gemv_splits(batch, n, k, kWave, &kps);
+        int sp = s4 > s1 ? s4 : s1;
+        return sp > 1 ? static_cast<size_t>(sp) * batch * n * sizeof(float) : 0;
+    }
+    TileChoice t = choose_tiles(batch, m, n, k);
+    return t.splits > 1 ? static_cast<size_t>(t.splits) * batch * m * n * sizeof(float) : 0;
+}
+
+extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t m,
+                                   int64_t n, int64_t k, const void *a, int64_t lda,
+                                   int64_t stride_a, int32_t trans_a, const void *b, int64_t ldb,
+                                   int64_t stride_b, int32_t trans_b, void *c, int64_t ldc,
+                                   int64_t stride_c, void *workspace, size_t workspace_bytes) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (batch < 0 || m < 0 || n < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (batch == 0 || m == 0 || n == 0) return RMLK_OK;
+    if (m >= (1ll << 31) || n >= (1ll << 31) || k >= (1ll << 31) || batch >= 65536)
+        return RMLK_ERR_TOO_LARGE;
+    if (!c) return RMLK_ERR_NULL_POINTER;
+    if (k > 0 && (!a || !b)) return RMLK_ERR_NULL_POINTER;
+    const int64_t a_cols = trans_a ? m : k, b_cols = trans_b ? k : n;
+    if (lda < a_cols || ldb < b_cols || ldc < n) return RMLK_ERR_SIZE_MISMATCH;
+    if (stride_a < 0 || stride_b < 0 || stride_c < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    hipStream_t s = as_stream(stream);
+    const float *pa = static_cast<const float *>(a);
+    const float *pb = static_cast<const float *>(b);
+    float *pc = static_cast<float *>(c);
+
+    if (k == 0) {
+        // empty sum: C = 0
+        float zero = 0.f;
+        for (int64_t bb = 0; bb < batch; ++bb)
+            for (int64_t r = 0; r < m; ++r) {
+                int32_t st = rmlk_hip_fill(stream, RMLK_FLOAT, n, &zero,
+                                           pc + bb * stride_c + r * ldc);
+                if (st) return st;
+            }
+        return RMLK_OK;
+    }
+
+    if (m == 1) {
+        GemvArgs g{};
+        g.x = pa;
+        g.w = pb;
+        g.n = static_cast<int32_t>(n);
+        g.k = static_cast<int32_t>(k);
+        g.x_inc = trans_a ? lda : 1;
+        g.ldb = ldb;
+        g.stride_x = stride_a;
+        g.stride_w = stride_b;
+        if (trans_b) {
+            g.y = pc;
+            g.stride_y = stride_c;
+            g.k_per_split = g.k;
+            int64_t blocks = (n + 3) / 4;
+            if (blocks > 8 * kNumCU) blocks = 8 * kNumCU;
+            dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch), 1);
+            gemv_dot_kernel<<<grid, kThreads, 0, s>>>(g);
+            return launch_status();
+        }
+        const bool vec = n % 4 == 0 && ldb % 4 == 0 && stride_b % 4 == 0 &&
+                         reinterpret_cast<uintptr_t>(pb) % 16 == 0;
+        const int cols = vec ? kWave * 4 : kWave;
+        int kps;
+        const int splits = gemv_splits(batch, n, k, cols, &kps);
+        g.k_per_split = kps;
+        if (splits > 1) {
+            const size_t need = static_cast<size_t>(splits) * batch * n * sizeof(float);
+            if (!workspace || workspace_bytes < need) return RMLK_ERR_WORKSPACE;
+            g.y = static_cast<float *>(workspace);
+            g.stride_y = n;
+        } else {
+            g.y = pc;
+            g.stride_y = stride_c;
+        }
+        dim3 grid(static_cast<unsigned>((n + cols - 1) / cols), static_cast<unsigned>(batch),
+                  static_cast<unsigned>(splits));
+        if (vec) gemv_kernel<4><<<grid, kThreads, 0, s>>>(g);
+        else gemv_kernel<1><<<grid, kThreads, 0, s>>>(g);
+        int32_t st = launch_status();
+        if (st) return st;
+        if (splits > 1) {
+            unsigned rg = grid_for(batch * n, kThreads, 8);
+            splitk_reduce_kernel<<<rg, kThreads, 0, s>>>(static_cast<const float *>(workspace), pc,
+                                                         splits, batch, 1, g.n, ldc, stride_c);
+            return launch_status();
+        }
+        return RMLK_OK;
+    }
+
+    if (trans_a || trans_b) {
+        unsigned grid = grid_for(batch * m * n, kThreads, 16);
+        gemm_naive_kernel<<<grid, kThreads, 0, s>>>(
+            pa, pb, pc, batch, static_cast<int32_t>(m), static_cast<int32_t>(n),
+            static_cast<int32_t>(k), trans_a ? 1 : lda, trans_a ? lda : 1, trans_b ? 1 : ldb,
+            trans_b ? ldb : 1, ldc, stride_a, stride_b, stride_c);
+        return launch_status();
+    }
+
+    TileChoice t = choose_tiles(batch, m, n, k);
+    GemmArgs g{};
+    g.a = pa;
+    g.b = pb;
+    g.m = static_cast<int32_t>(m);
+    g.n = static_cast<int32_t>(n);
+    g.k = static_cast<int32_t>(k);
+    g.lda = lda;
+    g.ldb = ldb;
+    g.stride_a = stride_a;
+    g.stride_b = stride_b;
+    g.k_per_split = t.k_per_split;
+    g.tiles_m = static_cast<int32_t>((m + t.bm - 1) / t.bm);
+    g.tiles_n = static_cast<int32_t>((n + t.bn - 1) / t.bn);
+    if (static_cast<int64_t>(g.tiles_m) * g.tiles_n >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
+    if (t.splits > 1) {
+        const size_t need = static_cast<size_t>(t.splits) * batch * m * n * sizeof(float);
+        if (!workspace || workspace_bytes < need) return RMLK_ERR_WORKSPACE;
+        g.c = static_cast<float *>(workspace);
+        g.ldc = n;
+        g.stride_c = m * n;
+    } else {
+        g.c = pc;
+        g.ldc = ldc;
+        g.stride_c = stride_c;
+    }
+    const bool aligned = lda % 4 == 0 && ldb % 4 == 0 && stride_a % 4 == 0 && stride_b % 4 == 0 &&
+                         reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(pb) % 16 == 0;
+    int32_t st;
+    if (t.bm == 128) {
+        st = aligned ? launch_mfma<128, 128, kBK, 64, 64, true>(s, g, batch, t.splits)
+                     : launch_mfma<128, 128, kBK, 64, 64, false>(s, g, batch, t.splits);
+    } else {
+        st = aligned ? launch_mfma<64, 64, kBK, 32, 32, true>(s, g, batch, t.splits)
+                     : launch_mfma<64, 64, kBK, 32, 32, false>(s, g, batch, t.splits);
+    }
+    if (st) return st;
+    if (t.splits > 1) {
+        unsigned rg = grid_for(batch * m * n, kThreads, 8);
+        splitk_reduce_kernel<<<rg, kThreads, 0, s>>>(static_cast<const float *>(workspace), pc,
+                                                     t.splits, batch, g.m, g.n, ldc, stride_c);
+        return launch_status();
+    }
+    return RMLK_OK;
+}

@@ -1,0 +1,403 @@
+// Row reductions: ReduceMean and Softmax.
+//
+// ReduceMean replaces cuda/src/ptx/reduce_mean.cu:5-9, whose kernel gives every output element to
+// one thread that walks the reduced elements serially (aggregation_op_macros.cuh:1-49). Here a
+// wavefront (or a block, for few long rows) owns a row, reads it with 128-bit loads, accumulates
+// in double like the reference and combines lanes with cross-lane shuffles.
+//
+// Softmax replaces the cuDNN call of cuda/src/kernels/softmax.rs:5-37. A wavefront keeps its whole
+// row in registers (one HBM read, one HBM write), max-subtracted.
+#include <type_traits>
+
+#include "nd_index.hpp"
+
+namespace rmlk {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+template <typename T>
+__device__ __forceinline__ T wave_max(T v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) {
+        T w = __shfl_xor(v, o, kWave);
+        v = w > v ? w : v;
+    }
+    return v;
+}
+
+// ---- ReduceMean over trailing contiguous elements: [rows, cols] -> [rows] ---------------------
+// kGroup lanes cooperate on a row: kWave (a wavefront per row) or kBlock (a block per row).
+template <typename T, int VEC, int kGroup>
+__global__ __launch_bounds__(kBlock) void mean_rows_kernel(const T *__restrict__ in,
+                                                           T *__restrict__ out, int64_t rows,
+                                                           int64_t cols) {
+    __shared__ double partial[kWavesPerBlock];
+    constexpr int kRowsPerBlock = kBlock / kGroup;
+    const int lane_in_group = threadIdx.x % kGroup;
+    const int group = threadIdx.x / kGroup;
+    for (int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + group; row < rows;
+         row += static_cast<int64_t>(gridDim.x) * kRowsPerBlock) {
+        const T *p = in + row * cols;
+        double acc = 0.0;
+        if constexpr (VEC == 1) {
+            for (int64_t c = lane_in_group; c < cols; c += kGroup) acc += static_cast<double>(p[c]);
+        } else {
+            using V = Vec<T, VEC>;
+            const int64_t nv = cols / VEC;
+            const V *pv = reinterpret_cast<const V *>(p);
+            int64_t c = lane_in_group;
+            for (; c + 3 * kGroup < nv; c += 4 * kGroup) {
+                V v0 = pv[c], v1 = pv[c + kGroup], v2 = pv[c + 2 * kGroup], v3 = pv[c + 3 * kGroup];
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    acc += (static_cast<double>(v0.v[j]) + static_cast<double>(v1.v[j])) +
+                           (static_cast<double>(v2.v[j]) + static_cast<double>(v3.v[j]));
+            }
+            for (; c < nv; c += kGroup) {
+                V v = pv[c];
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc += static_cast<double>(v.v[j]);
+            }
+        }
+        acc = wave_sum(acc);
+        if constexpr (kGroup == kWave) {
+            if (lane_in_group == 0) out[row] = static_cast<T>(acc / static_cast<double>(cols));
+        } else {
+            const int wave = threadIdx.x / kWave;
+            if ((threadIdx.x % kWave) == 0) partial[wave] = acc;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                double t = 0.0;
+#pragma unroll
+                for (int w = 0; w < kWavesPerBlock; ++w) t += partial[w];
+                out[row] = static_cast<T>(t / static_cast<double>(cols));
+            }
+            __syncthreads();
+        }
+    }
+}
+
+// ---- ReduceMean, any axes: a wavefront per output element -------------------------------------
+// kept / red are single-operand plans over the kept and the reduced dims of the input.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void mean_generic_kernel(NdPlan<1> kept, NdPlan<1> red,
+                                                              const T *__restrict__ in,
+                                                              T *__restrict__ out,
+                                                              uint32_t n_out, uint32_t n_red) {
+    const int lane = threadIdx.x % kWave;
+    const uint32_t wave0 = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+    for (uint32_t o = wave0; o < n_out; o += gridDim.x * kWavesPerBlock) {
+        int64_t base[1];
+        nd_offsets<1>(kept, o, base);
+        double acc = 0.0;
+        for (uint32_t r = lane; r < n_red; r += kWave) {
+            int64_t off[1];
+            nd_offsets<1>(red, r, off);
+            acc += static_cast<double>(in[base[0] + off[0]]);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) out[o] = static_cast<T>(acc / static_cast<double>(n_red));
+    }
+}
+
+// ---- Softmax, last axis, row held in registers ------------------------------------------------
+template <typename T>
+__device__ __forceinline__ T exp_t(T x) {
+    if constexpr (std::is_same<T, float>::value) return expf(x);
+    else return exp(x);
+}
+template <typename T>
+__device__ __forceinline__ T neg_inf() {
+    return -__builtin_huge_val();
+}
+template <>
+__device__ __forceinline__ float neg_inf<float>() {
+    return -__builtin_huge_valf();
+}
+
+// kGroup lanes own a row of up to kGroup * 4 * NV elements; cols % 4 == 0 and 16-byte aligned rows.
+template <typename T, int NV, int kGroup>
+__global__ __launch_bounds__(kBlock) void softmax_regs_kernel(const T *__restrict__ in,
+                                                              T *__restrict__ out, int64_t rows,
+                                                              int32_t cols) {
+    __shared__ T red_buf[2][kWavesPerBlock];
+    using V = Vec<T, 4>;
+    constexpr int kRowsPerBlock = kBlock / kGroup;
+    const int lane_in_group = threadIdx.x % kGroup;
+    const int group = threadIdx.x / kGroup;
+    const int nv = cols / 4;
+    for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock; row0 < rows;
+         row0 += static_cast<int64_t>(gridDim.x) * kRowsPerBlock) {
+        const int64_t row = row0 + group;
+        const bool live = row < rows;
+        const V *pv = reinterpret_cast<const V *>(in + row * cols);
+        V x[NV];
+        T m = neg_inf<T>();
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = lane_in_group + i * kGroup;
+            if (live && c < nv) {
+                x[i] = pv[c];
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) x[i].v[j] = neg_inf<T>();
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) m = x[i].v[j] > m ? x[i].v[j] : m;
+        }
+        m = wave_max(m);
+        if constexpr (kGroup == kBlock) {
+            const int wave = threadIdx.x / kWave;
+            if ((threadIdx.x % kWave) == 0) red_buf[0][wave] = m;
+            __syncthreads();
+#pragma unroll
+            for (int w = 0; w < kWavesPerBlock; ++w) m = red_buf[0][w] > m ? red_buf[0][w] : m;
+        }
+        T sum = 0;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                // padding lanes hold -inf: exp(-inf - m) = 0 unless m is -inf too (all-masked row),
+                // where IEEE gives NaN for real elements; keep padding at 0 in that case.
+                T e = exp_t<T>(x[i].v[j] - m);
+                const int c = lane_in_group + i * kGroup;
+                if (!(live && c < nv)) e = 0;
+                x[i].v[j] = e;
+                sum += e;
+            }
+        }
+        sum = wave_sum(sum);
+        if constexpr (kGroup == kBlock) {
+            const int wave = threadIdx.x / kWave;
+            if ((threadIdx.x % kWave) == 0) red_buf[1][wave] = sum;
+            __syncthreads();
+            sum = 0;
+#pragma unroll
+            for (int w = 0; w < kWavesPerBlock; ++w) sum += red_buf[1][w];
+            __syncthreads();
+        }
+        const T inv = static_cast<T>(1) / sum;
+        V *po = reinterpret_cast<V *>(out + row * cols);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = lane_in_group + i * kGroup;
+            if (live && c < nv) {
+                V y;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) y.v[j] = x[i].v[j] * inv;
+                po[c] = y;
+            }
+        }
+    }
+}
+
+// ---- Softmax fallback: [outer, n, inner], three passes over memory ----------------------------
+// inner == 1: a wavefront per row. inner > 1: a thread per (outer, inner) pair (coalesced along
+// inner), serial over the axis.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *__restrict__ in,
+                                                              T *__restrict__ out, int64_t rows,
+                                                              int64_t cols) {
+    const int lane = threadIdx.x % kWave;
+    for (int64_t row = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
+         row < rows; row += static_cast<int64_t>(gridDim.x) * kWavesPerBlock) {
+        const T *p = in + row * cols;
+        T *q = out + row * cols;
+        T m = neg_inf<T>();
+        for (int64_t c = lane; c < cols; c += kWave) m = p[c] > m ? p[c] : m;
+        m = wave_max(m);
+        T sum = 0;
+        for (int64_t c = lane; c < cols; c += kWave) sum += exp_t<T>(p[c] - m);
+        sum = wave_sum(sum);
+        const T inv = static_cast<T>(1) / sum;
+        for (int64_t c = lane; c < cols; c += kWave) q[c] = exp_t<T>(p[c] - m) * inv;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void softmax_strided_kernel(const T *__restrict__ in,
+                                                                 T *__restrict__ out,
+                                                                 int64_t outer, int64_t n,
+                                                                 int64_t inner) {
+    const int64_t total = outer * inner;
+    for (int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; t < total;
+         t += static_cast<int64_t>(gridDim.x) * kBlock) {
+        const int64_t o = t / inner, i = t - o * inner;
+        const T *p = in + o * n * inner + i;
+        T *q = out + o * n * inner + i;
+        T m = neg_inf<T>();
+        for (int64_t c = 0; c < n; ++c) m = p[c * inner] > m ? p[c * inner] : m;
+        T sum = 0;
+        for (int64_t c = 0; c < n; ++c) sum += exp_t<T>(p[c * inner] - m);
+        const T inv = static_cast<T>(1) / sum;
+        for (int64_t c = 0; c < n; ++c) q[c * inner] = exp_t<T>(p[c * inner] - m) * inv;
+    }
+}
+
+template <typename T, int NV, int kGroup>
+int32_t launch_softmax_regs(hipStream_t s, const T *in, T *out, int64_t rows, int32_t cols) {
+    constexpr int kRowsPerBlock = kBlock / kGroup;
+    int64_t blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+    const int64_t cap = static_cast<int64_t>(kNumCU) * 64;
+    if (blocks > cap) blocks = cap;
+    softmax_regs_kernel<T, NV, kGroup><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(in, out,
+                                                                                       rows, cols);
+    return launch_status();
+}
+
+template <typename T>
+int32_t softmax_typed(hipStream_t s, int64_t outer, int64_t n, int64_t inner, const T *in,
+                      T *out) {
+    if (inner == 1) {
+        const bool vec_ok = n % 4 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
+                            reinterpret_cast<uintptr_t>(out) % 16 == 0 && n <= 16384 &&
+                            sizeof(T) == 4;
+        if (vec_ok) {
+            const int32_t c = static_cast<int32_t>(n);
+            if (c <= 256) return launch_softmax_regs<T, 1, kWave>(s, in, out, outer, c);
+            if (c <= 512) return launch_softmax_regs<T, 2, kWave>(s, in, out, outer, c);
+            if (c <= 1024) return launch_softmax_regs<T, 4, kWave>(s, in, out, outer, c);
+            if (c <= 2048) return launch_softmax_regs<T, 8, kWave>(s, in, out, outer, c);
+            if (c <= 4096) return launch_softmax_regs<T, 4, kBlock>(s, in, out, outer, c);
+            if (c <= 8192) return launch_softmax_regs<T, 8, kBlock>(s, in, out, outer, c);
+            return launch_softmax_regs<T, 16, kBlock>(s, in, out, outer, c);
+        }
+        int64_t blocks = (outer + kWavesPerBlock - 1) / kWavesPerBlock;
+        const int64_t cap = static_cast<int64_t>(kNumCU) * 32;
+        if (blocks > cap) blocks = cap;
+        softmax_rows_kernel<T><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(in, out, outer, n);
+        return launch_status();
+    }
+    unsigned grid = grid_for(outer * inner, kBlock, 16);
+    softmax_strided_kernel<T><<<grid, kBlock, 0, s>>>(in, out, outer, n, inner);
+    return launch_status();
+}
+
+template <typename T>
+int32_t mean_typed(hipStream_t s, const rmlk_dims *shape, const bool *reduced, const T *in,
+                   T *out) {
+    const int rank = shape->rank;
+    int64_t st[kMaxRank];
+    dense_strides(rank, shape->v, st);
+    // trailing run of reduced dims?
+    int first_red = rank;
+    while (first_red > 0 && reduced[first_red - 1]) --first_red;
+    bool trailing = true;
+    for (int d = 0; d < first_red; ++d)
+        if (reduced[d]) trailing = false;
+    int64_t n_out = 1, n_red = 1;
+    for (int d = 0; d < rank; ++d) (reduced[d] ? n_red : n_out) *= shape->v[d];
+    if (trailing) {
+        const int64_t rows = n_out, cols = n_red;
+        const bool vec_ok = cols % 4 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
+                            sizeof(T) == 4;
+        const bool block_per_row = rows < 2048 && cols >= 8192;
+        if (block_per_row) {
+            unsigned grid = static_cast<unsigned>(rows < 65536 ? rows : 65536);
+            if (vec_ok) mean_rows_kernel<T, 4, kBlock><<<grid, kBlock, 0, s>>>(in, out, rows, cols);
+            else mean_rows_kernel<T, 1, kBlock><<<grid, kBlock, 0, s>>>(in, out, rows, cols);
+        } else {
+            int64_t blocks = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+            const int64_t cap = static_cast<int64_t>(kNumCU) * 32;
+            if (blocks > cap) blocks = cap;
+            unsigned grid = static_cast<unsigned>(blocks);
+            if (vec_ok) mean_rows_kernel<T, 4, kWave><<<grid, kBlock, 0, s>>>(in, out, rows, cols);
+            else mean_rows_kernel<T, 1, kWave><<<grid, kBlock, 0, s>>>(in, out, rows, cols);
+        }
+        return launch_status();
+    }
+    if (n_out >= ((int64_t)1 << 31) || n_red >= ((int64_t)1 << 31)) return RMLK_ERR_TOO_LARGE;
+    int64_t kshape[kMaxRank], kst[1][kMaxRank], rshape[kMaxRank], rst[1][kMaxRank];
+    int nk = 0, nr = 0;
+    for (int d = 0; d < rank; ++d) {
+        if (reduced[d]) {
+            rshape[nr] = shape->v[d];
+            rst[0][nr++] = st[d];
+        } else {
+            kshape[nk] = shape->v[d];
+            kst[0][nk++] = st[d];
+        }
+    }
+    if (nk == 0) {
+        kshape[0] = 1;
+        kst[0][0] = 0;
+        nk = 1;
+    }
+    NdPlan<1> kept, red;
+    build_plan<1>(kept, nk, kshape, kst);
+    build_plan<1>(red, nr, rshape, rst);
+    int64_t blocks = (n_out + kWavesPerBlock - 1) / kWavesPerBlock;
+    const int64_t cap = static_cast<int64_t>(kNumCU) * 32;
+    if (blocks > cap) blocks = cap;
+    mean_generic_kernel<T><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(
+        kept, red, in, out, static_cast<uint32_t>(n_out), static_cast<uint32_t>(n_red));
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace rmlk
+
+using namespace rmlk;
+
+extern "C" int32_t rmlk_hip_reduce_mean(rmlk_stream_t stream, int32_t dtype,
+                                        const rmlk_dims *in_shape, const int64_t *axes,
+                                        int32_t n_axes, const void *in, void *out) {
+    if (!dims_ok(in_shape)) return RMLK_ERR_BAD_RANK;
+    if (dtype != RMLK_FLOAT && dtype != RMLK_DOUBLE) return RMLK_ERR_UNSUPPORTED;
+    if (n_axes < 1 || n_axes > in_shape->rank) return RMLK_ERR_INVALID_ARGUMENT;
+    if (!axes) return RMLK_ERR_NULL_POINTER;
+    bool reduced[kMaxRank] = {false};
+    for (int i = 0; i < n_axes; ++i) {
+        if (axes[i] < 0 || axes[i] >= in_shape->rank || reduced[axes[i]])
+            return RMLK_ERR_INVALID_ARGUMENT;
+        reduced[axes[i]] = true;
+    }
+    int64_t numel = dims_numel(in_shape);
+    if (numel < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    int64_t n_out = 1;
+    for (int d = 0; d < in_shape->rank; ++d)
+        if (!reduced[d]) n_out *= in_shape->v[d];
+    if (n_out == 0) return RMLK_OK;
+    // A reduced dim of extent 0 leaves outputs that are means of nothing: NaN, as 0/0.
+    if (!out) return RMLK_ERR_NULL_POINTER;
+    if (numel == 0) {
+        if (dtype == RMLK_FLOAT) {
+            float nan = __builtin_nanf("");
+            return rmlk_hip_fill(stream, dtype, n_out, &nan, out);
+        }
+        double nan = __builtin_nan("");
+        return rmlk_hip_fill(stream, dtype, n_out, &nan, out);
+    }
+    if (!in) return RMLK_ERR_NULL_POINTER;
+    hipStream_t s = as_stream(stream);
+    if (dtype == RMLK_FLOAT)
+        return mean_typed<float>(s, in_shape, reduced, static_cast<const float *>(in),
+                                 static_cast<float *>(out));
+    return mean_typed<double>(s, in_shape, reduced, static_cast<const double *>(in),
+                              static_cast<double *>(out));
+}
+
+extern "C" int32_t rmlk_hip_softmax(rmlk_stream_t stream, int32_t dtype, int64_t outer,
+                                    int64_t axis_len, int64_t inner, const void *in, void *out) {
+    if (dtype != RMLK_FLOAT && dtype != RMLK_DOUBLE) return RMLK_ERR_UNSUPPORTED;
+    if (outer < 0 || axis_len < 0 || inner < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (outer == 0 || axis_len == 0 || inner == 0) return RMLK_OK;
+    if (outer > kMaxElems / axis_len || outer * axis_len > kMaxElems / inner)
+        return RMLK_ERR_TOO_LARGE;
+    if (!in || !out) return RMLK_ERR_NULL_POINTER;
+    hipStream_t s = as_stream(stream);
+    if (dtype == RMLK_FLOAT)
+        return softmax_typed<float>(s, outer, axis_len, inner, static_cast<const float *>(in),
+                                    static_cast<float *>(out));
+    return softmax_typed<double>(s, outer, axis_len, inner, static_cast<const double *>(in),
+                                 static_cast<double *>(out));
+}

@@ -1,0 +1,240 @@
+// Contiguous maps: Sqrt Neg Sin Cos Sigmoid, Cast, Fill.
+// Replaces cuda/src/ptx/{sqrt,neg,sin,cos,cast}.cu (cuda/src/ptx/headers/unary_op_macro.cuh:1-11,
+// cast_op_macro.cuh:1-11) and the cuDNN sigmoid call (cuda/src/kernels/activation.rs:6-39).
+#include <limits>
+#include <type_traits>
+
+#include "elementwise.hpp"
+
+namespace rmlk {
+namespace {
+
+template <typename F, typename TI, typename TO, int VEC>
+__global__ __launch_bounds__(kEwBlock) void map_flat_kernel(const TI *__restrict__ in,
+                                                            TO *__restrict__ out, uint32_t n) {
+    const uint32_t step = gridDim.x * kEwBlock;
+    if constexpr (VEC == 1) {
+        for (uint32_t i = blockIdx.x * kEwBlock + threadIdx.x; i < n; i += step)
+            out[i] = F::apply(in[i]);
+    } else {
+        const uint32_t n_vec = n / kEwVec;
+        for (uint32_t i = blockIdx.x * kEwBlock + threadIdx.x; i < n_vec; i += step) {
+            TI ri[kEwVec];
+            TO ro[kEwVec];
+            load_vec(in + static_cast<size_t>(i) * kEwVec, false, ri);
+#pragma unroll
+            for (int j = 0; j < kEwVec; ++j) ro[j] = F::apply(ri[j]);
+            store_vec(out + static_cast<size_t>(i) * kEwVec, ro);
+        }
+        if (blockIdx.x == 0 && threadIdx.x < (n - n_vec * kEwVec)) {
+            uint32_t i = n_vec * kEwVec + threadIdx.x;
+            out[i] = F::apply(in[i]);
+        }
+    }
+}
+
+template <typename F, typename TI, typename TO>
+int32_t launch_map(hipStream_t s, int64_t n, const void *in, void *out) {
+    constexpr int64_t kPiece = (int64_t)1 << 30;
+    for (int64_t off = 0; off < n; off += kPiece) {
+        const TI *pi = static_cast<const TI *>(in) + off;
+        TO *po = static_cast<TO *>(out) + off;
+        uint32_t m = static_cast<uint32_t>(n - off < kPiece ? n - off : kPiece);
+        size_t ai = sizeof(TI) * kEwVec > 16 ? 16 : sizeof(TI) * kEwVec;
+        size_t ao = sizeof(TO) * kEwVec > 16 ? 16 : sizeof(TO) * kEwVec;
+        bool aligned = reinterpret_cast<uintptr_t>(pi) % ai == 0 &&
+                       reinterpret_cast<uintptr_t>(po) % ao == 0;
+        if (aligned) {
+            unsigned grid = grid_for(m / kEwVec + 1, kEwBlock, 16);
+            map_flat_kernel<F, TI, TO, kEwVec><<<grid, kEwBlock, 0, s>>>(pi, po, m);
+        } else {
+            unsigned grid = grid_for(m, kEwBlock, 16);
+            map_flat_kernel<F, TI, TO, 1><<<grid, kEwBlock, 0, s>>>(pi, po, m);
+        }
+        int32_t st = launch_status();
+        if (st) return st;
+    }
+    return RMLK_OK;
+}
+
+template <typename T>
+struct SqrtF {
+    static __device__ __forceinline__ T apply(T x) {
+        if constexpr (std::is_same<T, float>::value) return sqrtf(x);
+        else return sqrt(x);
+    }
+};
+// The reference multiplies by -1 (cuda/src/ptx/neg.cu:6); a sign flip gives the same bits.
+template <typename T>
+struct NegF {
+    static __device__ __forceinline__ T apply(T x) {
+        if constexpr (std::is_integral<T>::value) {
+            using U = typename std::make_unsigned<T>::type;
+            return static_cast<T>(U(0) - static_cast<U>(x));
+        } else {
+            return -x;
+        }
+    }
+};
+template <typename T>
+struct SinF {
+    static __device__ __forceinline__ T apply(T x) {
+        if constexpr (std::is_same<T, float>::value) return sinf(x);
+        else return sin(x);
+    }
+};
+template <typename T>
+struct CosF {
+    static __device__ __forceinline__ T apply(T x) {
+        if constexpr (std::is_same<T, float>::value) return cosf(x);
+        else return cos(x);
+    }
+};
+template <typename T>
+struct SigmoidF {
+    static __device__ __forceinline__ T apply(T x) {
+        if constexpr (std::is_same<T, float>::value) return 1.0f / (1.0f + expf(-x));
+        else return 1.0 / (1.0 + exp(-x));
+    }
+};
+
+template <template <typename> class F>
+int32_t dispatch_float(hipStream_t s, int32_t dt, int64_t n, const void *in, void *out) {
+    switch (dt) {
+        case RMLK_FLOAT: return launch_map<F<float>, float, float>(s, n, in, out);
+        case RMLK_DOUBLE: return launch_map<F<double>, double, double>(s, n, in, out);
+        default: return RMLK_ERR_UNSUPPORTED;
+    }
+}
+
+// ---- cast ------------------------------------------------------------------------------------
+struct BoolTag {
+    uint8_t b;
+};
+
+template <typename TI, typename TO>
+struct CastF {
+    static __device__ __forceinline__ TO apply(TI x) {
+        constexpr bool in_bool = std::is_same<TI, BoolTag>::value;
+        constexpr bool out_bool = std::is_same<TO, BoolTag>::value;
+        if constexpr (in_bool && out_bool) {
+            return BoolTag{static_cast<uint8_t>(x.b ? 1 : 0)};
+        } else if constexpr (in_bool) {
+            return static_cast<TO>(x.b ? 1 : 0);
+        } else if constexpr (out_bool) {
+            return BoolTag{static_cast<uint8_t>(x != static_cast<TI>(0) ? 1 : 0)};
+        } else if constexpr (std::is_integral<TO>::value && !std::is_integral<TI>::value) {
+            // float -> int: truncate toward zero; NaN -> 0; out of range saturates.
+            double v = static_cast<double>(x);
+            if (v != v) return 0;
+            constexpr double lo = static_cast<double>(std::numeric_limits<TO>::min());
+            // max() of 64-bit types is not a double; 2^63 / 2^64 is the first value out of range.
+            constexpr double hi = static_cast<double>(std::numeric_limits<TO>::max());
+            if (v <= lo) return std::numeric_limits<TO>::min();
+            if (v >= hi) return std::numeric_limits<TO>::max();
+            return static_cast<TO>(v);
+        } else {
+            return static_cast<TO>(x);
+        }
+    }
+};
+
+template <typename TI>
+int32_t dispatch_cast_dst(hipStream_t s, int32_t dst, int64_t n, const void *in, void *out) {
+    switch (dst) {
+        case RMLK_FLOAT: return launch_map<CastF<TI, float>, TI, float>(s, n, in, out);
+        case RMLK_DOUBLE: return launch_map<CastF<TI, double>, TI, double>(s, n, in, out);
+        case RMLK_FLOAT16: return launch_map<CastF<TI, _Float16>, TI, _Float16>(s, n, in, out);
+        case RMLK_INT8: return launch_map<CastF<TI, int8_t>, TI, int8_t>(s, n, in, out);
+        case RMLK_INT16: return launch_map<CastF<TI, int16_t>, TI, int16_t>(s, n, in, out);
+        case RMLK_INT32: return launch_map<CastF<TI, int32_t>, TI, int32_t>(s, n, in, out);
+        case RMLK_INT64: return launch_map<CastF<TI, int64_t>, TI, int64_t>(s, n, in, out);
+        case RMLK_UINT8: return launch_map<CastF<TI, uint8_t>, TI, uint8_t>(s, n, in, out);
+        case RMLK_UINT16: return launch_map<CastF<TI, uint16_t>, TI, uint16_t>(s, n, in, out);
+        case RMLK_UINT32: return launch_map<CastF<TI, uint32_t>, TI, uint32_t>(s, n, in, out);
+        case RMLK_UINT64: return launch_map<CastF<TI, uint64_t>, TI, uint64_t>(s, n, in, out);
+        case RMLK_BOOL: return launch_map<CastF<TI, BoolTag>, TI, BoolTag>(s, n, in, out);
+        default: return RMLK_ERR_UNSUPPORTED;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kEwBlock) void fill_kernel(T *__restrict__ out, T value, uint64_t n) {
+    const uint64_t step = static_cast<uint64_t>(gridDim.x) * kEwBlock;
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kEwBlock + threadIdx.x; i < n; i += step)
+        out[i] = value;
+}
+
+}  // namespace
+}  // namespace rmlk
+
+using namespace rmlk;
+
+extern "C" int32_t rmlk_hip_unary(rmlk_stream_t stream, int32_t op, int32_t dtype, int64_t n,
+                                  const void *in, void *out) {
+    if (n < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n >= kMaxElems) return RMLK_ERR_TOO_LARGE;
+    if (op < RMLK_SQRT || op > RMLK_SIGMOID) return RMLK_ERR_INVALID_ARGUMENT;
+    if (dtype_size(dtype) == 0) return RMLK_ERR_UNSUPPORTED;
+    hipStream_t s = as_stream(stream);
+    bool is_float = dtype == RMLK_FLOAT || dtype == RMLK_DOUBLE;
+    bool neg_int = op == RMLK_NEG && (dtype == RMLK_INT32 || dtype == RMLK_INT64);
+    if (!is_float && !neg_int) return RMLK_ERR_UNSUPPORTED;
+    if (n == 0) return RMLK_OK;
+    if (!in || !out) return RMLK_ERR_NULL_POINTER;
+    switch (op) {
+        case RMLK_SQRT: return dispatch_float<SqrtF>(s, dtype, n, in, out);
+        case RMLK_SIN: return dispatch_float<SinF>(s, dtype, n, in, out);
+        case RMLK_COS: return dispatch_float<CosF>(s, dtype, n, in, out);
+        case RMLK_SIGMOID: return dispatch_float<SigmoidF>(s, dtype, n, in, out);
+        case RMLK_NEG:
+            if (dtype == RMLK_INT32) return launch_map<NegF<int32_t>, int32_t, int32_t>(s, n, in, out);
+            if (dtype == RMLK_INT64) return launch_map<NegF<int64_t>, int64_t, int64_t>(s, n, in, out);
+            return dispatch_float<NegF>(s, dtype, n, in, out);
+        default: return RMLK_ERR_INVALID_ARGUMENT;
+    }
+}
+
+extern "C" int32_t rmlk_hip_cast(rmlk_stream_t stream, int32_t src, int32_t dst, int64_t n,
+                                 const void *in, void *out) {
+    if (n < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n >= kMaxElems) return RMLK_ERR_TOO_LARGE;
+    if (dtype_size(src) == 0 || dtype_size(dst) == 0) return RMLK_ERR_UNSUPPORTED;
+    if (n == 0) return RMLK_OK;
+    if (!in || !out) return RMLK_ERR_NULL_POINTER;
+    hipStream_t s = as_stream(stream);
+    switch (src) {
+        case RMLK_FLOAT: return dispatch_cast_dst<float>(s, dst, n, in, out);
+        case RMLK_DOUBLE: return dispatch_cast_dst<double>(s, dst, n, in, out);
+        case RMLK_FLOAT16: return dispatch_cast_dst<_Float16>(s, dst, n, in, out);
+        case RMLK_INT8: return dispatch_cast_dst<int8_t>(s, dst, n, in, out);
+        case RMLK_INT16: return dispatch_cast_dst<int16_t>(s, dst, n, in, out);
+        case RMLK_INT32: return dispatch_cast_dst<int32_t>(s, dst, n, in, out);
+        case RMLK_INT64: return dispatch_cast_dst<int64_t>(s, dst, n, in, out);
+        case RMLK_UINT8: return dispatch_cast_dst<uint8_t>(s, dst, n, in, out);
+        case RMLK_UINT16: return dispatch_cast_dst<uint16_t>(s, dst, n, in, out);
+        case RMLK_UINT32: return dispatch_cast_dst<uint32_t>(s, dst, n, in, out);
+        case RMLK_UINT64: return dispatch_cast_dst<uint64_t>(s, dst, n, in, out);
+        case RMLK_BOOL: return dispatch_cast_dst<BoolTag>(s, dst, n, in, out);
+        default: return RMLK_ERR_UNSUPPORTED;
+    }
+}
+
+extern "C" int32_t rmlk_hip_fill(rmlk_stream_t stream, int32_t dtype, int64_t n,
+                                 const void *value, void *out) {
+    if (n < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n >= kMaxElems) return RMLK_ERR_TOO_LARGE;
+    int es = dtype_size(dtype);
+    if (es == 0) return RMLK_ERR_UNSUPPORTED;
+    if (n == 0) return RMLK_OK;
+    if (!value || !out) return RMLK_ERR_NULL_POINTER;
+    hipStream_t s = as_stream(stream);
+    unsigned grid = grid_for(n, kEwBlock, 16);
+    switch (es) {
+        case 1: fill_kernel<uint8_t><<<grid, kEwBlock, 0, s>>>(static_cast<uint8_t *>(out), *static_cast<const uint8_t *>(value), n); break;
+        case 2: fill_kernel<uint16_t><<<grid, kEwBlock, 0, s>>>(static_cast<uint16_t *>(out), *static_cast<const uint16_t *>(value), n); break;
+        case 4: fill_kernel<uint32_t><<<grid, kEwBlock, 0, s>>>(static_cast<uint32_t *>(out), *static_cast<const uint32_t *>(value), n); break;
+        default: fill_kernel<uint64_t><<<grid, kEwBlock, 0, s>>>(static_cast<uint64_t *>(out), *static_cast<const uint64_t *>(value), n); break;
+    }
+    return launch_status();
+}

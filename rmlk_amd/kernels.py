@@ -1,0 +1,174 @@
+"""Kernel-level wrappers over the C ABI: the Python mirror of the reference's kernel crate
+(`rmlk_cuda::kernels::<op>::compute`, cuda/src/kernels/mod.rs:1-29).
+
+Like the reference's wrappers, the caller owns every buffer: inputs and the pre-allocated output
+are torch tensors on the GPU (torch is only the owner of device memory and of the stream here);
+shape and stride vectors are host lists. Contract violations raise `AssertionError` (the
+reference's wrappers `assert!`), launch failures raise `RmlkError`.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from ._lib import Dims, RmlkError, check, lib
+
+# ONNX TensorProto.DataType numbers (include/rmlk_hip.h rmlk_dtype)
+FLOAT, UINT8, INT8, UINT16, INT16, INT32, INT64, BOOL, FLOAT16, DOUBLE, UINT32, UINT64 = (
+    1, 2, 3, 4, 5, 6, 7, 9, 10, 11, 12, 13)
+
+TORCH_TO_DTYPE = {
+    torch.float32: FLOAT, torch.uint8: UINT8, torch.int8: INT8, torch.int16: INT16,
+    torch.int32: INT32, torch.int64: INT64, torch.bool: BOOL, torch.float16: FLOAT16,
+    torch.float64: DOUBLE, torch.uint16: UINT16, torch.uint32: UINT32, torch.uint64: UINT64,
+}
+DTYPE_TO_TORCH = {v: k for k, v in TORCH_TO_DTYPE.items()}
+
+ADD, SUB, MUL, DIV, POW, EQUAL, GREATER = range(7)
+SQRT, NEG, SIN, COS, SIGMOID = range(5)
+SCATTER_NONE, SCATTER_ADD, SCATTER_MUL, SCATTER_MAX, SCATTER_MIN = range(5)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t) -> int:
+    if t is None:
+        return 0
+    assert t.is_cuda and t.is_contiguous(), "device tensors must be dense"
+    return t.data_ptr()
+
+
+def dtype_of(t: torch.Tensor) -> int:
+    return TORCH_TO_DTYPE[t.dtype]
+
+
+def binary(op: int, a, b, out, out_shape, a_stride, b_stride) -> None:
+    """ref: cuda/src/kernels/binary.rs:58-100 (compute_with_types). Strides are per output dim,
+    0 on broadcast dims."""
+    assert len(out_shape) == len(a_stride) == len(b_stride)
+    n = 1
+    for d in out_shape:
+        n *= d
+    assert out.numel() == n, "output length must equal the product of the output shape"
+    st = lib().rmlk_hip_binary(_stream(), op, dtype_of(a), dtype_of(b), Dims.of(out_shape),
+                               Dims.of(a_stride), Dims.of(b_stride), _ptr(a), _ptr(b), _ptr(out))
+    check(st, "rmlk_hip_binary")
+
+
+def where(x, y, cond, out, out_shape, x_stride, y_stride, cond_stride) -> None:
+    """ref: cuda/src/kernels/whereop.rs:57-101 (kernel operand order x, y, cond)."""
+    assert cond.dtype == torch.bool or cond.dtype == torch.uint8
+    st = lib().rmlk_hip_where(_stream(), dtype_of(x), Dims.of(out_shape), Dims.of(x_stride),
+                              Dims.of(y_stride), Dims.of(cond_stride), _ptr(x), _ptr(y),
+                              _ptr(cond), _ptr(out))
+    check(st, "rmlk_hip_where")
+
+
+def unary(op: int, x, out) -> None:
+    """ref: cuda/src/kernels/unary.rs:10-42."""
+    assert x.numel() == out.numel(), "input and output lengths must match"
+    check(lib().rmlk_hip_unary(_stream(), op, dtype_of(x), x.numel(), _ptr(x), _ptr(out)),
+          "rmlk_hip_unary")
+
+
+def cast(x, out) -> None:
+    """ref: cuda/src/kernels/unary.rs:47-80 (explicit_io_types_compute)."""
+    assert x.numel() == out.numel()
+    check(lib().rmlk_hip_cast(_stream(), dtype_of(x), dtype_of(out), x.numel(), _ptr(x),
+                              _ptr(out)), "rmlk_hip_cast")
+
+
+def reduce_mean(x, out, in_shape, axes) -> None:
+    """ref: cuda/src/kernels/reduce_mean.rs:40-93."""
+    arr = (ctypes.c_int64 * len(axes))(*[int(a) for a in axes])
+    check(lib().rmlk_hip_reduce_mean(_stream(), dtype_of(x), Dims.of(in_shape), arr, len(axes),
+                                     _ptr(x), _ptr(out)), "rmlk_hip_reduce_mean")
+
+
+def softmax(x, out, outer: int, axis_len: int, inner: int = 1) -> None:
+    """ref: cuda/src/kernels/softmax.rs:5-37."""
+    assert x.numel() == out.numel() == outer * axis_len * inner
+    check(lib().rmlk_hip_softmax(_stream(), dtype_of(x), outer, axis_len, inner, _ptr(x),
+                                 _ptr(out)), "rmlk_hip_softmax")
+
+
+def matmul_workspace_size(batch: int, m: int, n: int, k: int, dtype: int = FLOAT) -> int:
+    return int(lib().rmlk_hip_matmul_workspace_size(dtype, batch, m, n, k))
+
+
+def matmul(a, b, c, batch, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, trans_a=False,
+           trans_b=False, workspace=None) -> None:
+    """ref: cuda/src/kernels/gemm.rs:112-136 (compute with a StridedBatchedConfig)."""
+    need = matmul_workspace_size(batch, m, n, k, dtype_of(a))
+    if workspace is None and need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=a.device)
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    st = lib().rmlk_hip_matmul(_stream(), dtype_of(a), batch, m, n, k, _ptr(a), lda, stride_a,
+                               int(trans_a), _ptr(b), ldb, stride_b, int(trans_b), _ptr(c), ldc,
+                               stride_c, _ptr(workspace), ws_bytes)
+    check(st, "rmlk_hip_matmul")
+
+
+def transpose(x, out, in_shape, perm) -> None:
+    """ref: cuda/src/kernels/transpose.rs:38-80."""
+    arr = (ctypes.c_int64 * len(perm))(*[int(p) for p in perm])
+    check(lib().rmlk_hip_transpose(_stream(), dtype_of(x), Dims.of(in_shape), arr, _ptr(x),
+                                   _ptr(out)), "rmlk_hip_transpose")
+
+
+def expand(x, out, in_shape, out_shape) -> None:
+    """ref: cuda/src/kernels/expand.rs:35-76."""
+    check(lib().rmlk_hip_expand(_stream(), dtype_of(x), Dims.of(in_shape), Dims.of(out_shape),
+                                _ptr(x), _ptr(out)), "rmlk_hip_expand")
+
+
+def slice_(x, out, in_shape, starts, steps, out_shape) -> None:
+    """ref: cuda/src/kernels/slice.rs:61-122, with starts / steps already resolved per dim."""
+    check(lib().rmlk_hip_slice(_stream(), dtype_of(x), Dims.of(in_shape), Dims.of(starts),
+                               Dims.of(steps), Dims.of(out_shape), _ptr(x), _ptr(out)),
+          "rmlk_hip_slice")
+
+
+def concat_into(x, out, in_shape, out_shape, axis: int, axis_offset: int) -> None:
+    """ref: runtime/src/providers/cuda/backend/concat.rs:28-76 (one input)."""
+    check(lib().rmlk_hip_concat(_stream(), dtype_of(x), Dims.of(in_shape), Dims.of(out_shape),
+                                axis, axis_offset, _ptr(x), _ptr(out)), "rmlk_hip_concat")
+
+
+def gather(data, idx, out, data_shape, axis: int, err_flag=None) -> None:
+    """ref: runtime/src/providers/cuda/backend/gather.rs:199-258."""
+    check(lib().rmlk_hip_gather(_stream(), dtype_of(data), dtype_of(idx), Dims.of(data_shape),
+                                axis, idx.numel(), _ptr(data), _ptr(idx), _ptr(out),
+                                _ptr(err_flag)), "rmlk_hip_gather")
+
+
+def scatter_nd(idx, updates, out, data_shape, n_tuples: int, tuple_size: int,
+               reduction: int = SCATTER_NONE, err_flag=None) -> None:
+    """ref: cuda/src/kernels/scatter_nd.rs:91-210. `out` already holds the data."""
+    assert idx.dtype == torch.int64
+    check(lib().rmlk_hip_scatter_nd(_stream(), reduction, dtype_of(out), Dims.of(data_shape),
+                                    n_tuples, tuple_size, _ptr(idx), _ptr(updates), _ptr(out),
+                                    _ptr(err_flag)), "rmlk_hip_scatter_nd")
+
+
+def trilu(x, out, batch: int, rows: int, cols: int, upper: bool, k: int) -> None:
+    """ref: cuda/src/kernels/trilu.rs:36-78."""
+    assert x.numel() == out.numel() == batch * rows * cols
+    check(lib().rmlk_hip_trilu(_stream(), dtype_of(x), batch, rows, cols, int(upper), k, _ptr(x),
+                               _ptr(out)), "rmlk_hip_trilu")
+
+
+def device_info(device: int = 0) -> dict:
+    from ._lib import DeviceInfo
+    info = DeviceInfo()
+    check(lib().rmlk_hip_device_info(device, ctypes.byref(info)), "rmlk_hip_device_info")
+    return {"name": info.name.decode(), "arch": info.arch.decode(),
+            "compute_units": info.compute_units, "wavefront_size": info.wavefront_size,
+            "lds_bytes_per_block": info.lds_bytes_per_block, "clock_khz": info.clock_khz,
+            "total_mem_bytes": info.total_mem_bytes}
+
+
+__all__ = [n for n in dir() if not n.startswith("_")] + ["RmlkError"]

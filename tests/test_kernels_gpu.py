@@ -1,0 +1,561 @@
+"""Kernel-level parity: every C-ABI entry point against the CPU oracle on seeded inputs.
+
+Bars: integer / bool / pure-move results bit-exact; fp32 math within rtol 1e-4 / atol 1e-5 (the
+reference's per-op acceptance, runtime/tests/onnx_node/main.rs:26-27). Add/Sub/Mul/Div/Sqrt are
+IEEE-exact and are held to bit equality.
+"""
+import zlib
+
+import numpy as np
+import pytest
+
+from helpers import assert_close, assert_exact, bcast_strides, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def _k():
+    from rmlk_amd import kernels
+    return kernels
+
+
+def _ops():
+    from oracle import ops
+    return ops
+
+
+NP_BIN = {"add": 0, "sub": 1, "mul": 2, "div": 3, "pow": 4, "equal": 5, "greater": 6}
+
+BCAST_CASES = [
+    ((5,), (5,)),
+    ((1027,), (1027,)),              # flat with a scalar tail
+    ((4, 8), (1,)),                  # scalar operand
+    ((1,), (3, 5)),
+    ((2, 4, 1), (4, 3)),             # ref: backend/add.rs broadcast cases
+    ((2, 4, 3), (3,)),
+    ((8, 4, 16, 64), (1, 4, 1, 64)),  # the C2 pattern, small
+    ((2, 3, 5, 7), (2, 1, 5, 1)),
+    ((3, 1, 4), (1, 6, 1)),
+    ((2, 2, 2, 2, 2, 2, 2, 2), (2, 1, 2, 1, 2, 1, 2, 1)),  # rank 8
+    ((0, 4), (4,)),                  # empty
+]
+
+
+def run_binary(device, name, a, b):
+    k = _k()
+    out_shape = list(np.broadcast_shapes(a.shape, b.shape))
+    if name in ("equal", "greater"):
+        out = torch.empty(out_shape, dtype=torch.bool, device=device)
+    else:
+        out = torch.empty(out_shape, dtype=to_dev(a, device).dtype, device=device)
+    shp = out_shape or [1]
+    k.binary(NP_BIN[name], to_dev(a, device), to_dev(b, device), out, shp,
+             bcast_strides(a.shape or (1,), shp), bcast_strides(b.shape or (1,), shp))
+    return to_np(out)
+
+
+@pytest.mark.parametrize("name", ["add", "sub", "mul", "div"])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+@pytest.mark.parametrize("shapes", BCAST_CASES)
+def test_arith_broadcast(device, name, dtype, shapes):
+    rng = np.random.default_rng(zlib.crc32(repr((name, str(dtype), shapes)).encode()))
+    sa, sb = shapes
+    if np.issubdtype(dtype, np.integer):
+        a = rng.integers(-1000, 1000, size=sa).astype(dtype)
+        b = rng.integers(-50, 50, size=sb).astype(dtype)
+        if name == "div":
+            b[b == 0] = 7
+    else:
+        a = rng.standard_normal(sa).astype(dtype)
+        b = rng.standard_normal(sb).astype(dtype)
+    expected = getattr(_ops(), name)(a, b)
+    got = run_binary(device, name, a, b)
+    assert_exact(got, expected)
+
+
+def test_int_division_edges(device):
+    a = np.array([7, -7, 7, -7, 0, 5, np.iinfo(np.int32).min], dtype=np.int32)
+    b = np.array([2, 2, -2, -2, 3, 0, -1], dtype=np.int32)
+    got = run_binary(device, "div", a, b)
+    assert_exact(got, _ops().div(a, b))
+    assert list(got[:6]) == [3, -3, -3, 3, 0, 0]
+
+
+def test_float_specials(device):
+    a = np.array([np.inf, -np.inf, np.nan, 0.0, -0.0, 1e-45, 3.4e38, 1.0], dtype=np.float32)
+    b = np.array([1.0, np.inf, 1.0, -0.0, 0.0, 0.5, 3.4e38, 0.0], dtype=np.float32)
+    for name in ["add", "sub", "mul", "div"]:
+        assert_exact(run_binary(device, name, a, b), getattr(_ops(), name)(a, b))
+    assert_exact(run_binary(device, "equal", a, b), _ops().equal(a, b))
+    assert_exact(run_binary(device, "greater", a, b), _ops().greater(a, b))
+
+
+@pytest.mark.parametrize("name", ["equal", "greater"])
+@pytest.mark.parametrize("dtype", [np.float32, np.int32, np.int64, np.float64])
+@pytest.mark.parametrize("shapes", BCAST_CASES[:8])
+def test_compare(device, name, dtype, shapes):
+    rng = np.random.default_rng(11)
+    a = rng.integers(-3, 3, size=shapes[0]).astype(dtype)
+    b = rng.integers(-3, 3, size=shapes[1]).astype(dtype)
+    got = run_binary(device, name, a, b)
+    assert got.dtype == np.bool_
+    assert_exact(got, getattr(_ops(), name)(a, b))
+
+
+@pytest.mark.parametrize("base,exp", [(np.float32, np.float32), (np.float32, np.int32),
+                                      (np.float32, np.int64), (np.int32, np.int32),
+                                      (np.int32, np.int64), (np.int32, np.float32),
+                                      (np.int64, np.int32), (np.int64, np.int64),
+                                      (np.int64, np.float32)])
+def test_pow_pairs(device, base, exp):
+    """The nine (base, exponent) pairs the reference enables (backend/pow.rs:123-132)."""
+    rng = np.random.default_rng(5)
+    if np.issubdtype(base, np.integer):
+        a = rng.integers(-6, 7, size=(4, 33)).astype(base)
+        b = rng.integers(0, 5, size=(33,)).astype(exp)
+        assert_exact(run_binary(device, "pow", a, b), _ops().pow_(a, b))
+    else:
+        a = np.abs(rng.standard_normal((4, 33))).astype(base) + 0.1
+        b = rng.integers(-3, 4, size=(33,)).astype(exp)
+        assert_close(run_binary(device, "pow", a, b), _ops().pow_(a, b))
+
+
+def test_pow_special_exponents_exact(device):
+    rng = np.random.default_rng(6)
+    a = rng.standard_normal((128, 64)).astype(np.float32)
+    for e in (2.0, 3.0):
+        got = run_binary(device, "pow", a, np.array([e], dtype=np.float32))
+        assert_exact(got, _ops().pow_(a, np.array([e], dtype=np.float32)))
+    pos = np.abs(a)
+    assert_exact(run_binary(device, "pow", pos, np.array([0.5], dtype=np.float32)), np.sqrt(pos))
+    frac = run_binary(device, "pow", pos + 0.5, np.array([1.7], dtype=np.float32))
+    assert_close(frac, _ops().pow_(pos + 0.5, np.array([1.7], dtype=np.float32)))
+
+
+WHERE_CASES = [
+    ((4, 5), (4, 5), (4, 5)),
+    ((1031,), (1031,), (1,)),
+    ((8, 4, 16, 64), (8, 4, 16, 64), (1, 4, 1, 64)),  # C2 pattern
+    ((3, 1), (1, 4), (3, 4)),                          # ref: backend/whereop.rs 3-way broadcast
+    ((1,), (2, 3), (2, 1)),
+    ((2, 1, 8, 8), (1,), (2, 4, 8, 8)),               # causal-mask pattern
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.int64, np.int32, np.float64, np.uint8])
+@pytest.mark.parametrize("shapes", WHERE_CASES)
+def test_where(device, dtype, shapes):
+    k = _k()
+    rng = np.random.default_rng(21)
+    sc, sx, sy = shapes
+    cond = rng.random(sc) < 0.5
+    x = np.abs(rng.standard_normal(sx) * 10).astype(dtype)
+    y = np.abs(rng.standard_normal(sy) * 10).astype(dtype)
+    if dtype != np.uint8:
+        x, y = -x, y
+    if dtype == np.float32:
+        x.reshape(-1)[0] = np.nan
+        y.reshape(-1)[0] = -0.0
+    expected = _ops().where(cond, x, y)
+    shp = list(expected.shape)
+    out = torch.empty(shp, dtype=to_dev(x, device).dtype, device=device)
+    k.where(to_dev(x, device), to_dev(y, device), to_dev(cond, device), out, shp,
+            bcast_strides(sx, shp), bcast_strides(sy, shp), bcast_strides(sc, shp))
+    assert_exact(to_np(out), expected)
+
+
+@pytest.mark.parametrize("n", [1, 3, 128, 1025, 65536 + 3])
+@pytest.mark.parametrize("name", ["sqrt", "neg", "sin", "cos", "sigmoid"])
+def test_unary_f32(device, name, n):
+    k = _k()
+    rng = np.random.default_rng(31)
+    x = (rng.standard_normal(n) * 4).astype(np.float32)
+    if name == "sqrt":
+        x = np.abs(x)
+    if name in ("sin", "cos") and n > 8:
+        x[:8] = [0.0, np.pi, 3 * np.pi / 4, -np.pi / 2, 100.0, 2047.0, 8191.0, -8191.0]
+    if name == "sigmoid" and n > 4:
+        x[:4] = [100.0, -100.0, 0.0, -0.0]
+    op = {"sqrt": k.SQRT, "neg": k.NEG, "sin": k.SIN, "cos": k.COS, "sigmoid": k.SIGMOID}[name]
+    out = torch.empty(n, dtype=torch.float32, device=device)
+    k.unary(op, to_dev(x, device), out)
+    expected = getattr(_ops(), name)(x)
+    if name in ("sqrt", "neg"):
+        assert_exact(to_np(out), expected)
+    else:
+        assert_close(to_np(out), expected)
+
+
+def test_unary_other_dtypes(device):
+    k = _k()
+    for dt in (np.float64, np.int32, np.int64):
+        x = np.arange(-5, 6).astype(dt)
+        out = torch.empty(x.size, dtype=to_dev(x, device).dtype, device=device)
+        k.unary(k.NEG, to_dev(x, device), out)
+        assert_exact(to_np(out), -x)
+    with pytest.raises(k.RmlkError, match="unsupported"):
+        x = to_dev(np.arange(4, dtype=np.int32), device)
+        k.unary(k.SQRT, x, torch.empty_like(x))
+
+
+CAST_TYPES = [np.float32, np.float64, np.float16, np.int8, np.int16, np.int32, np.int64, np.uint8,
+              np.uint16, np.uint32, np.uint64, np.bool_]
+
+
+@pytest.mark.parametrize("src", CAST_TYPES)
+@pytest.mark.parametrize("dst", CAST_TYPES)
+def test_cast_pairs(device, src, dst):
+    k = _k()
+    from oracle.ops import NP_TO_ONNX
+    rng = np.random.default_rng(41)
+    if src == np.bool_:
+        x = rng.random(259) < 0.5
+    elif np.issubdtype(src, np.floating):
+        # values in range of every target (int8: |x| < 128; unsigned targets: non-negative)
+        x = (rng.random(259) * 120).astype(src)
+        if np.issubdtype(dst, np.signedinteger) or np.issubdtype(dst, np.floating):
+            x = (x - 60).astype(src)
+        x[:3] = [0.0, 2.1, 2.9]
+    else:
+        info = np.iinfo(src)
+        lo = max(info.min, -100) if not np.issubdtype(dst, np.unsignedinteger) else 0
+        x = rng.integers(lo, min(info.max, 100), size=259).astype(src)
+    expected = _ops().cast(x, NP_TO_ONNX[np.dtype(dst)])
+    out = torch.empty(x.size, dtype=to_dev(expected, device).dtype, device=device)
+    k.cast(to_dev(x, device), out)
+    assert_exact(to_np(out), expected)
+
+
+REDUCE_CASES = [
+    ((4, 8), [1]), ((4, 8), [0]), ((4, 8), [0, 1]),
+    ((2, 3, 4), [2]), ((2, 3, 4), [1]), ((2, 3, 4), [0, 2]), ((2, 3, 4), [1, 2]),
+    ((128, 2048), [1]), ((3, 5, 1031), [2]), ((2, 16384), [1]), ((7,), [0]),
+    ((2, 3, 4, 5), [1, 3]),
+]
+
+
+@pytest.mark.parametrize("case", REDUCE_CASES)
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_reduce_mean(device, case, dtype):
+    k = _k()
+    shape, axes = case
+    rng = np.random.default_rng(51)
+    x = (rng.standard_normal(shape) + 3.0).astype(dtype)
+    expected = _ops().reduce_mean(x, axes, keepdims=0)
+    out = torch.empty(int(np.prod(expected.shape)), dtype=to_dev(x, device).dtype, device=device)
+    k.reduce_mean(to_dev(x, device), out, list(shape), axes)
+    assert_close(to_np(out).reshape(expected.shape), expected, rtol=1e-6, atol=1e-7)
+
+
+SOFTMAX_CASES = [(4, 8, 1), (3, 7, 1), (16, 256, 1), (5, 1000, 1), (9, 2048, 1), (3, 4096, 1),
+                 (2, 8192, 1), (2, 16384, 1), (2, 20000, 1), (33, 513, 1), (2, 3, 4), (4, 6, 35)]
+
+
+@pytest.mark.parametrize("case", SOFTMAX_CASES)
+def test_softmax(device, case):
+    k = _k()
+    outer, n, inner = case
+    rng = np.random.default_rng(61)
+    x = (rng.standard_normal((outer, n, inner)) * 3).astype(np.float32)
+    expected = _ops().softmax(x, axis=1)
+    out = torch.empty(x.shape, dtype=torch.float32, device=device)
+    k.softmax(to_dev(x, device), out, outer, n, inner)
+    got = to_np(out)
+    assert_close(got, expected)
+    np.testing.assert_allclose(got.sum(axis=1), 1.0, rtol=0, atol=2e-6)
+
+
+def test_softmax_causal_mask(device):
+    """-inf strictly above the diagonal: masked entries exactly 0, rows sum to 1."""
+    k = _k()
+    s = 256
+    rng = np.random.default_rng(62)
+    x = rng.standard_normal((4, s, s)).astype(np.float32)
+    x = x + np.triu(np.full((s, s), -np.inf, dtype=np.float32), 1)
+    out = torch.empty(x.shape, dtype=torch.float32, device=device)
+    k.softmax(to_dev(x, device), out, 4 * s, s, 1)
+    got = to_np(out)
+    assert_close(got, _ops().softmax(x, axis=-1))
+    assert np.all(got[:, np.triu_indices(s, 1)[0], np.triu_indices(s, 1)[1]] == 0.0)
+    full_mask = np.full((2, 8), -np.inf, dtype=np.float32)
+    out2 = torch.empty(full_mask.shape, dtype=torch.float32, device=device)
+    k.softmax(to_dev(full_mask, device), out2, 2, 8, 1)
+    assert np.all(np.isnan(to_np(out2)))  # IEEE 0/0, as the oracle (and ONNX Runtime) give
+
+
+def run_matmul(device, a, b, trans_a=False, trans_b=False):
+    """a: [batch?, m, k] (or [k, m] per batch when trans_a), b likewise; 2-D operand = broadcast."""
+    k = _k()
+    am = a.shape[-2:] if not trans_a else a.shape[-2:][::-1]
+    bm = b.shape[-2:] if not trans_b else b.shape[-2:][::-1]
+    m, kk = am
+    n = bm[1]
+    batch = max(a.shape[0] if a.ndim == 3 else 1, b.shape[0] if b.ndim == 3 else 1)
+    c = torch.empty((batch, m, n), dtype=torch.float32, device=device)
+    k.matmul(to_dev(a, device), to_dev(b, device), c, batch, m, n, kk,
+             lda=a.shape[-1], ldb=b.shape[-1], ldc=n,
+             stride_a=a.shape[-1] * a.shape[-2] if a.ndim == 3 else 0,
+             stride_b=b.shape[-1] * b.shape[-2] if b.ndim == 3 else 0,
+             stride_c=m * n, trans_a=trans_a, trans_b=trans_b)
+    return to_np(c)
+
+
+MATMUL_CASES = [
+    (1, 2, 2, 2), (1, 7, 5, 3), (1, 64, 64, 64), (1, 128, 128, 16), (1, 130, 70, 33),
+    (1, 128, 2048, 256), (3, 96, 80, 40), (2, 256, 256, 128), (1, 512, 384, 2048),
+    (4, 1, 64, 300), (1, 1, 2048, 2048), (2, 1, 130, 77), (1, 1, 1, 5), (1, 300, 1, 64),
+    (1, 257, 129, 19),
+]
+
+
+@pytest.mark.parametrize("case", MATMUL_CASES)
+@pytest.mark.parametrize("bcast_b", [False, True])
+def test_matmul(device, case, bcast_b):
+    batch, m, n, kk = case
+    rng = np.random.default_rng(71)
+    a = rng.standard_normal((batch, m, kk)).astype(np.float32)
+    b = (rng.standard_normal((kk, n) if bcast_b else (batch, kk, n)) * 0.02).astype(np.float32)
+    expected = _ops().matmul(a, b)
+    got = run_matmul(device, a, b)
+    assert_close(got, expected, rtol=1e-4, atol=1e-5)
+
+
+def test_matmul_exact_integers(device):
+    """Integer-valued operands small enough that fp32 accumulation is exact in any order."""
+    rng = np.random.default_rng(72)
+    a = rng.integers(-8, 9, size=(2, 200, 96)).astype(np.float32)
+    b = rng.integers(-8, 9, size=(2, 96, 136)).astype(np.float32)
+    assert_exact(run_matmul(device, a, b), _ops().matmul(a, b))
+    assert_exact(run_matmul(device, a[:, :1], b), _ops().matmul(a[:, :1], b))  # GEMV path
+
+
+@pytest.mark.parametrize("trans", [(True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("m", [1, 37])
+def test_matmul_transposed(device, trans, m):
+    ta, tb = trans
+    rng = np.random.default_rng(73)
+    a = rng.standard_normal((2, m, 45)).astype(np.float32)
+    b = rng.standard_normal((2, 45, 28)).astype(np.float32)
+    expected = _ops().matmul(a, b)
+    a_in = np.ascontiguousarray(a.transpose(0, 2, 1)) if ta else a
+    b_in = np.ascontiguousarray(b.transpose(0, 2, 1)) if tb else b
+    assert_close(run_matmul(device, a_in, b_in, ta, tb), expected)
+
+
+TRANSPOSE_CASES = [
+    ((2, 3), [1, 0]), ((4, 5, 6), [2, 0, 1]), ((4, 5, 6), [0, 2, 1]), ((1, 64, 8, 16), [0, 2, 1, 3]),
+    ((1, 8, 64, 16), [0, 1, 3, 2]), ((3, 130, 70), [0, 2, 1]), ((2, 3, 4, 5), [3, 2, 1, 0]),
+    ((2, 3, 4, 5), [0, 1, 2, 3]), ((7, 1, 9), [2, 1, 0]), ((1, 300, 4, 64), [0, 2, 1, 3]),
+    ((65, 67), [1, 0]), ((2, 2, 2, 2, 2, 2, 2, 2), [7, 6, 5, 4, 3, 2, 1, 0]),
+]
+
+
+@pytest.mark.parametrize("case", TRANSPOSE_CASES)
+@pytest.mark.parametrize("dtype", [np.float32, np.int64, np.uint8, np.float16])
+def test_transpose(device, case, dtype):
+    k = _k()
+    shape, perm = case
+    x = np.arange(int(np.prod(shape))).reshape(shape).astype(dtype)
+    expected = _ops().transpose(x, perm)
+    out = torch.empty(expected.shape, dtype=to_dev(x, device).dtype, device=device)
+    k.transpose(to_dev(x, device), out, list(shape), perm)
+    assert_exact(to_np(out), expected)
+
+
+EXPAND_CASES = [((3, 1), (3, 4)), ((1,), (2, 3)), ((2, 1, 4), (2, 3, 4)), ((1, 8, 1, 16, 64), (1, 8, 4, 16, 64)),
+                ((4,), (2, 3, 4)), ((1, 1, 8, 8), (2, 4, 8, 8)), ((3, 4), (3, 4)), ((1, 3), (0, 3))]
+
+
+@pytest.mark.parametrize("case", EXPAND_CASES)
+@pytest.mark.parametrize("dtype", [np.float32, np.int64, np.bool_])
+def test_expand(device, case, dtype):
+    k = _k()
+    in_shape, out_shape = case
+    rng = np.random.default_rng(81)
+    x = (rng.standard_normal(in_shape) * 9).astype(dtype)
+    expected = _ops().expand(x, out_shape)
+    out = torch.empty(out_shape, dtype=to_dev(x, device).dtype, device=device)
+    k.expand(to_dev(x, device), out, list(in_shape), list(out_shape))
+    assert_exact(to_np(out), expected)
+
+
+SLICE_CASES = [
+    ((10,), [2], [7], None, None), ((10,), [-3], [100], None, None),
+    ((10,), [8], [1], [0], [-2]), ((10,), [-1], [-(2 ** 63)], [0], [-1]),
+    ((4, 6), [1, 2], [3, 5], None, None), ((4, 6), [0], [2 ** 63 - 1], [1], [2]),
+    ((2, 8, 16, 64), [0], [32], [3], None), ((2, 8, 16, 64), [32], [64], [-1], [1]),
+    ((1, 8, 40, 64), [3], [30], [2], [1]), ((5, 5), [4, 4], [0, 0], [0, 1], [-1, -2]),
+    ((3, 4), [2], [2], [0], None), ((1, 24, 27, 128), [0], [13], [2], None),
+]
+
+
+@pytest.mark.parametrize("case", SLICE_CASES)
+@pytest.mark.parametrize("dtype", [np.float32, np.int64])
+def test_slice(device, case, dtype):
+    k = _k()
+    shape, starts, ends, axes, steps = case
+    x = np.arange(int(np.prod(shape))).reshape(shape).astype(dtype)
+    expected = _ops().slice_(x, starts, ends, axes, steps)
+    res = _ops().slice_resolve(shape, starts, ends, axes, steps)
+    out = torch.empty(expected.shape, dtype=to_dev(x, device).dtype, device=device)
+    k.slice_(to_dev(x, device), out, list(shape), [r[0] if r[2] else 0 for r in res],
+             [r[1] for r in res], list(expected.shape))
+    assert_exact(to_np(out), expected)
+
+
+CONCAT_CASES = [([(2, 3), (2, 5)], 1), ([(2, 3), (4, 3), (1, 3)], 0), ([(1, 8, 0, 64), (1, 8, 5, 64)], 2),
+                ([(1, 8, 7, 64), (1, 8, 1, 64)], 2), ([(2, 4, 16, 32), (2, 4, 16, 32)], 3),
+                ([(3,), (4,)], 0)]
+
+
+@pytest.mark.parametrize("case", CONCAT_CASES)
+@pytest.mark.parametrize("dtype", [np.float32, np.int64])
+def test_concat(device, case, dtype):
+    k = _k()
+    shapes, axis = case
+    rng = np.random.default_rng(91)
+    xs = [(rng.standard_normal(s) * 100).astype(dtype) for s in shapes]
+    expected = _ops().concat(xs, axis)
+    out = torch.empty(expected.shape, dtype=to_dev(xs[0], device).dtype, device=device)
+    off = 0
+    for x in xs:
+        k.concat_into(to_dev(x, device), out, list(x.shape), list(expected.shape), axis, off)
+        off += x.shape[axis]
+    assert_exact(to_np(out), expected)
+
+
+GATHER_CASES = [((3, 4), 0, [0, 2]), ((3, 4), 0, [-3, -1]), ((3, 4), 1, [1, 3]), ((2, 3, 4), 1, [[1, 2], [0, -1]]),
+                ((500, 64), 0, list(range(0, 500, 7))), ((500, 2048), 0, [499, 0, 17, 17]),
+                ((4,), 0, [2]), ((6, 5), 1, [4, 0, 0]), ((3, 7, 3), 2, [2, 1])]
+
+
+@pytest.mark.parametrize("case", GATHER_CASES)
+@pytest.mark.parametrize("idx_dtype", [np.int32, np.int64])
+@pytest.mark.parametrize("dtype", [np.float32, np.int64, np.float16])
+def test_gather(device, case, idx_dtype, dtype):
+    k = _k()
+    shape, axis, idx = case
+    x = np.arange(int(np.prod(shape))).reshape(shape).astype(dtype)
+    idx = np.array(idx, dtype=idx_dtype)
+    expected = _ops().gather(x, idx, axis)
+    out = torch.empty(expected.shape, dtype=to_dev(x, device).dtype, device=device)
+    err = torch.zeros(1, dtype=torch.int32, device=device)
+    k.gather(to_dev(x, device), to_dev(idx, device), out, list(shape), axis, err)
+    assert_exact(to_np(out), expected)
+    assert int(err.item()) == 0
+
+
+def test_gather_out_of_range_sets_flag(device):
+    k = _k()
+    x = np.arange(12, dtype=np.float32).reshape(3, 4)
+    idx = np.array([0, 3, -4, 2], dtype=np.int64)   # 3 == dim (the reference would accept it) and -4
+    out = torch.full((4, 4), -1.0, dtype=torch.float32, device=device)
+    err = torch.zeros(1, dtype=torch.int32, device=device)
+    k.gather(to_dev(x, device), to_dev(idx, device), out, [3, 4], 0, err)
+    got = to_np(out)
+    assert int(err.item()) == 1
+    assert_exact(got[0], x[0])
+    assert_exact(got[3], x[2])
+    assert np.all(got[1:3] == 0.0)
+
+
+SCATTER_CASES = [
+    ((8,), [[4], [3], [1], [7]], None),                       # ONNX doc example 1
+    ((4, 4, 4), [[0], [2]], None),                            # ONNX doc example 2
+    ((1, 8, 32, 64), [[0, h, 5] for h in range(8)], None),    # KV-cache row write
+    ((5, 6), [[-1, -1], [0, 0]], None),
+]
+
+
+@pytest.mark.parametrize("case", SCATTER_CASES)
+@pytest.mark.parametrize("dtype", [np.float32, np.int64])
+def test_scatter_nd_none(device, case, dtype):
+    k = _k()
+    shape, idx, _ = case
+    rng = np.random.default_rng(101)
+    data = (rng.standard_normal(shape) * 10).astype(dtype)
+    if dtype == np.float32:
+        data.reshape(-1)[0] = np.inf  # the reference's in + 0*out would turn this into NaN
+    idx = np.array(idx, dtype=np.int64)
+    upd_shape = idx.shape[:-1] + tuple(shape[idx.shape[-1]:])
+    upd = (rng.standard_normal(upd_shape) * 10).astype(dtype)
+    expected = _ops().scatter_nd(data, idx, upd)
+    out = to_dev(data, device).clone()
+    err = torch.zeros(1, dtype=torch.int32, device=device)
+    k.scatter_nd(to_dev(idx, device), to_dev(upd, device), out, list(shape),
+                 int(np.prod(idx.shape[:-1])), idx.shape[-1], k.SCATTER_NONE, err)
+    assert_exact(to_np(out), expected)
+    assert int(err.item()) == 0
+
+
+@pytest.mark.parametrize("red", ["add", "mul", "max", "min"])
+@pytest.mark.parametrize("dtype", [np.float32, np.int32, np.int64, np.float64])
+def test_scatter_nd_reductions(device, red, dtype):
+    k = _k()
+    rng = np.random.default_rng(102)
+    data = rng.integers(1, 5, size=(6, 8)).astype(dtype)
+    idx = np.array([[0], [3], [0], [5], [3]], dtype=np.int64)  # duplicates combine
+    upd = rng.integers(1, 4, size=(5, 8)).astype(dtype)
+    expected = _ops().scatter_nd(data, idx, upd, red)
+    out = to_dev(data, device).clone()
+    code = {"add": k.SCATTER_ADD, "mul": k.SCATTER_MUL, "max": k.SCATTER_MAX, "min": k.SCATTER_MIN}
+    k.scatter_nd(to_dev(idx, device), to_dev(upd, device), out, [6, 8], 5, 1, code[red])
+    assert_exact(to_np(out), expected)  # small integers: exact in every order
+
+
+def test_scatter_nd_bad_index_flag(device):
+    k = _k()
+    data = np.zeros((4, 4), dtype=np.float32)
+    idx = np.array([[1], [4], [-5], [2]], dtype=np.int64)
+    upd = np.ones((4, 4), dtype=np.float32)
+    out = to_dev(data, device).clone()
+    err = torch.zeros(1, dtype=torch.int32, device=device)
+    k.scatter_nd(to_dev(idx, device), to_dev(upd, device), out, [4, 4], 4, 1, k.SCATTER_NONE, err)
+    got = to_np(out)
+    assert int(err.item()) == 1
+    assert np.all(got[1] == 1) and np.all(got[2] == 1) and np.all(got[0] == 0) and np.all(got[3] == 0)
+
+
+TRILU_CASES = [(1, 4, 5), (3, 7, 7), (2, 64, 64), (1, 33, 130), (1, 256, 256)]
+
+
+@pytest.mark.parametrize("shape", TRILU_CASES)
+@pytest.mark.parametrize("upper", [True, False])
+@pytest.mark.parametrize("kdiag", [0, 1, -1, 3, -100, 100, 2 ** 40, -(2 ** 40)])
+@pytest.mark.parametrize("dtype", [np.float32, np.int64])
+def test_trilu(device, shape, upper, kdiag, dtype):
+    k = _k()
+    rng = np.random.default_rng(111)
+    x = (rng.standard_normal(shape) * 10).astype(dtype)
+    if dtype == np.float32:
+        x[x == 0] = 1.0
+    expected = _ops().trilu(x, min(max(kdiag, -10 ** 6), 10 ** 6), upper)
+    out = torch.full(shape, 77, dtype=to_dev(x, device).dtype, device=device)  # zeros must be written
+    k.trilu(to_dev(x, device), out, shape[0], shape[1], shape[2], upper, kdiag)
+    assert_exact(to_np(out), expected)
+
+
+def test_trilu_neg_inf_mask(device):
+    """Trilu(upper, k=1) of a -inf matrix is the causal-mask builder of the Llama graph."""
+    k = _k()
+    s = 128
+    x = np.full((1, s, s), -np.inf, dtype=np.float32)
+    out = torch.empty((1, s, s), dtype=torch.float32, device=device)
+    k.trilu(to_dev(x, device), out, 1, s, s, True, 1)
+    assert_exact(to_np(out), np.triu(x[0], 1)[None])
+
+
+def test_status_codes(device):
+    k = _k()
+    x = torch.zeros(4, dtype=torch.float32, device=device)
+    with pytest.raises(k.RmlkError, match="unsupported"):
+        k.binary(k.ADD, x, x.to(torch.int32), x, [4], [1], [1])
+    with pytest.raises(k.RmlkError, match="invalid"):
+        k.transpose(x, x, [2, 2], [0, 0])
+    with pytest.raises(k.RmlkError, match="rank"):
+        from rmlk_amd._lib import Dims
+        Dims.of([1] * 9)
+    info = k.device_info(0)
+    assert info["wavefront_size"] == 64 and "gfx950" in info["arch"]
