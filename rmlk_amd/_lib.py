@@ -48,7 +48,8 @@ class DeviceInfo(ctypes.Structure):
 
 
 def library_path() -> str:
-    return os.path.join(_HERE, "lib", "librmlk_hip.so")
+    """In-tree build output, or the file RMLK_HIP_LIBRARY names."""
+    return os.environ.get("RMLK_HIP_LIBRARY") or os.path.join(_HERE, "lib", "librmlk_hip.so")
 
 
 # name -> (restype, argtypes); every symbol include/rmlk_hip.h declares

@@ -86,9 +86,12 @@ struct NdPlan {
     uint32_t dim[kMaxRank];          // dim[rank-1] is innermost
     int64_t dim64[kMaxRank];
     FastDiv fdiv[kMaxRank];
-    int64_t stride[NP][kMaxRank];    // element strides, may be 0 or negative
+    int32_t stride[NP][kMaxRank];    // element strides, may be 0 or negative; |stride| < 2^31
     int64_t numel;
 };
+
+constexpr int64_t kPieceElems = (int64_t)1 << 30;   // elements one launch indexes (32-bit math)
+constexpr int64_t kStrideLimit = (int64_t)1 << 31;  // strides a plan can hold
 
 // Build a coalesced plan. shape[rank], strides[p][rank]. Returns false when numel == 0.
 template <int NP>
@@ -136,7 +139,7 @@ inline bool build_plan(NdPlan<NP> &pl, int rank, const int64_t *shape,
         pl.dim64[d] = mshp[d];
         pl.dim[d] = static_cast<uint32_t>(mshp[d]);
         pl.fdiv[d] = FastDiv(static_cast<uint32_t>(mshp[d] > 0x7fffffff ? 1 : mshp[d]));
-        for (int p = 0; p < NP; ++p) pl.stride[p][d] = mst[p][d];
+        for (int p = 0; p < NP; ++p) pl.stride[p][d] = static_cast<int32_t>(mst[p][d]);
     }
     for (int d = pl.rank; d < kMaxRank; ++d) {
         pl.dim64[d] = 1;
@@ -153,6 +156,47 @@ inline void dense_strides(int rank, const int64_t *shape, int64_t *stride) {
         stride[d] = s;
         s *= shape[d];
     }
+}
+
+// Kernels index with 32-bit math: at most kPieceElems elements per launch and strides below
+// kStrideLimit. Larger work is cut along its outermost non-unit dim, recursively.
+// fn(shape, offsets) launches one piece; offsets[p] is the element offset of operand p.
+template <int NP, typename Fn>
+inline int32_t split_pieces(int rank, const int64_t *shape, const int64_t (*strides)[kMaxRank],
+                            const int64_t *offsets, Fn &&fn) {
+    int64_t numel = 1;
+    for (int d = 0; d < rank; ++d) {
+        if (shape[d] < 0) return RMLK_ERR_INVALID_ARGUMENT;
+        if (shape[d] == 0) return RMLK_OK;
+    }
+    for (int d = 0; d < rank; ++d) {
+        if (numel > kMaxElems / shape[d]) return RMLK_ERR_TOO_LARGE;
+        numel *= shape[d];
+    }
+    bool strides_fit = true;
+    for (int d = 0; d < rank; ++d)
+        if (shape[d] > 1)
+            for (int p = 0; p < NP; ++p)
+                if (strides[p][d] >= kStrideLimit || strides[p][d] <= -kStrideLimit)
+                    strides_fit = false;
+    if (numel <= kPieceElems && strides_fit) return fn(shape, offsets);
+    int d0 = 0;
+    while (d0 < rank - 1 && shape[d0] == 1) ++d0;
+    if (shape[d0] == 1) return RMLK_ERR_TOO_LARGE;  // a single element cannot be too large
+    const int64_t inner = numel / shape[d0];
+    int64_t rows_per = inner >= kPieceElems ? 1 : kPieceElems / inner;
+    for (int p = 0; p < NP; ++p)
+        if (strides[p][d0] >= kStrideLimit || strides[p][d0] <= -kStrideLimit) rows_per = 1;
+    int64_t sub[kMaxRank];
+    for (int d = 0; d < rank; ++d) sub[d] = shape[d];
+    for (int64_t r0 = 0; r0 < shape[d0]; r0 += rows_per) {
+        sub[d0] = shape[d0] - r0 < rows_per ? shape[d0] - r0 : rows_per;
+        int64_t offs[NP];
+        for (int p = 0; p < NP; ++p) offs[p] = offsets[p] + r0 * strides[p][d0];
+        int32_t st = split_pieces<NP>(rank, sub, strides, offs, fn);
+        if (st != RMLK_OK) return st;
+    }
+    return RMLK_OK;
 }
 
 // Grid size for a grid-stride kernel: enough blocks to cover `work` items, capped so that a few

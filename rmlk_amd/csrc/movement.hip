@@ -18,29 +18,30 @@ struct alignas(16) U128 {
 
 // ---------------------------------------------------------------------------------------------
 // strided N-d copy: plan operand 0 = in, 1 = out
+constexpr int kUnroll = 4;  // independent accesses in flight per lane
+
 template <typename U>
 __global__ __launch_bounds__(kBlock) void copy_nd_kernel(NdPlan<2> pl, const U *__restrict__ in,
                                                          U *__restrict__ out, uint32_t n) {
-    constexpr int kUnroll = 4;
     const uint32_t step = gridDim.x * kBlock;
-    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n; i += step * kUnroll) {
+    uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    for (; i + (kUnroll - 1) * step < n; i += step * kUnroll) {
         U r[kUnroll];
         int64_t oo[kUnroll];
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
-            uint32_t idx = i + j * step;
-            if (idx < n) {
-                int64_t offs[2];
-                nd_offsets<2>(pl, idx, offs);
-                r[j] = in[offs[0]];
-                oo[j] = offs[1];
-            }
+            int64_t offs[2];
+            nd_offsets<2>(pl, i + j * step, offs);
+            r[j] = in[offs[0]];
+            oo[j] = offs[1];
         }
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
-            uint32_t idx = i + j * step;
-            if (idx < n) out[oo[j]] = r[j];
-        }
+        for (int j = 0; j < kUnroll; ++j) out[oo[j]] = r[j];
+    }
+    for (; i < n; i += step) {
+        int64_t offs[2];
+        nd_offsets<2>(pl, i, offs);
+        out[offs[1]] = in[offs[0]];
     }
 }
 
@@ -48,27 +49,22 @@ __global__ __launch_bounds__(kBlock) void copy_nd_kernel(NdPlan<2> pl, const U *
 template <typename U>
 __global__ __launch_bounds__(kBlock) void copy_flat_kernel(const U *__restrict__ in,
                                                            U *__restrict__ out, uint32_t n) {
-    constexpr int kUnroll = 4;
     const uint32_t step = gridDim.x * kBlock;
-    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n; i += step * kUnroll) {
+    uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    for (; i + (kUnroll - 1) * step < n; i += step * kUnroll) {
         U r[kUnroll];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
-            uint32_t idx = i + j * step;
-            if (idx < n) r[j] = in[idx];
-        }
+        for (int j = 0; j < kUnroll; ++j) r[j] = in[i + j * step];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
-            uint32_t idx = i + j * step;
-            if (idx < n) out[idx] = r[j];
-        }
+        for (int j = 0; j < kUnroll; ++j) out[i + j * step] = r[j];
     }
+    for (; i < n; i += step) out[i] = in[i];
 }
 
 template <typename U>
 int32_t launch_copy_units(hipStream_t s, NdPlan<2> &pl, const void *in, void *out) {
     uint32_t n = static_cast<uint32_t>(pl.numel);
-    unsigned grid = grid_for((n + 3) / 4, kBlock, 16);
+    unsigned grid = grid_for(n / kUnroll + 1, kBlock, 8);
     if (pl.rank == 1 && pl.stride[0][0] == 1 && pl.stride[1][0] == 1) {
         copy_flat_kernel<U><<<grid, kBlock, 0, s>>>(static_cast<const U *>(in),
                                                     static_cast<U *>(out), n);
@@ -93,7 +89,7 @@ int32_t strided_copy_piece(hipStream_t s, int esize, int rank, const int64_t *sh
                       reinterpret_cast<uintptr_t>(out) % cand == 0;
             for (int d = 0; d < last && ok; ++d)
                 for (int p = 0; p < 2; ++p)
-                    if ((pl.stride[p][d] * esize) % cand) ok = false;
+                    if ((static_cast<int64_t>(pl.stride[p][d]) * esize) % cand) ok = false;
             if (ok) { unit = cand; break; }
         }
         if (unit != esize) {
@@ -115,37 +111,18 @@ int32_t strided_copy_piece(hipStream_t s, int esize, int rank, const int64_t *sh
     }
 }
 
-// Strided copy of any size: splits along the outermost dim to keep index math in 32 bits.
+// Strided copy of any size: pieces that the kernels' 32-bit index math can address.
 int32_t strided_copy(hipStream_t s, int esize, int rank, const int64_t *shape,
                      const int64_t (*strides)[kMaxRank], const void *in, void *out) {
-    int64_t numel = 1;
-    for (int d = 0; d < rank; ++d) {
-        if (shape[d] < 0) return RMLK_ERR_INVALID_ARGUMENT;
-        if (shape[d] == 0) return RMLK_OK;
-    }
-    for (int d = 0; d < rank; ++d) {
-        if (numel > kMaxElems / shape[d]) return RMLK_ERR_TOO_LARGE;
-        numel *= shape[d];
-    }
     const char *pin = static_cast<const char *>(in);
     char *pout = static_cast<char *>(out);
-    constexpr int64_t kLimit = (int64_t)1 << 30;
-    if (numel <= kLimit) return strided_copy_piece(s, esize, rank, shape, strides, pin, pout);
-    int d0 = 0;
-    while (d0 < rank - 1 && shape[d0] == 1) ++d0;
-    int64_t inner = numel / shape[d0];
-    if (inner > kLimit) return RMLK_ERR_TOO_LARGE;
-    int64_t rows_per = kLimit / inner;
-    int64_t sub[kMaxRank];
-    for (int d = 0; d < rank; ++d) sub[d] = shape[d];
-    for (int64_t r0 = 0; r0 < shape[d0]; r0 += rows_per) {
-        sub[d0] = shape[d0] - r0 < rows_per ? shape[d0] - r0 : rows_per;
-        int32_t st = strided_copy_piece(s, esize, rank, sub, strides,
-                                        pin + r0 * strides[0][d0] * esize,
-                                        pout + r0 * strides[1][d0] * esize);
-        if (st != RMLK_OK) return st;
-    }
-    return RMLK_OK;
+    int64_t zero[2] = {0, 0};
+    return split_pieces<2>(rank, shape, strides, zero,
+                           [&](const int64_t *shp, const int64_t *offs) {
+                               return strided_copy_piece(s, esize, rank, shp, strides,
+                                                         pin + offs[0] * esize,
+                                                         pout + offs[1] * esize);
+                           });
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -222,6 +199,24 @@ int32_t launch_tile(hipStream_t s, const TilePlan &tp, uint64_t blocks, const vo
 // Gather rows. Units of `U`; a row is `row_units` units. out row r = (outer, j) takes data row
 // (outer * axis_dim + idx[j]).
 template <typename U, typename I>
+__device__ __forceinline__ U gather_fetch(const U *__restrict__ data, const I *__restrict__ idx,
+                                          uint32_t e, uint32_t row_units, FastDiv row_div,
+                                          uint32_t n_idx, FastDiv idx_div, int64_t axis_dim,
+                                          int32_t *__restrict__ err) {
+    const uint32_t row = row_div.div(e);
+    const uint32_t c = e - row * row_units;
+    const uint32_t outer = idx_div.div(row);
+    const uint32_t jj = row - outer * n_idx;
+    int64_t ix = static_cast<int64_t>(idx[jj]);
+    if (ix < 0) ix += axis_dim;
+    if (ix < 0 || ix >= axis_dim) {
+        if (err) *err = 1;
+        return U{};
+    }
+    return data[(static_cast<int64_t>(outer) * axis_dim + ix) * row_units + c];
+}
+
+template <typename U, typename I>
 __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const U *__restrict__ data,
                                                              const I *__restrict__ idx,
                                                              U *__restrict__ out, uint32_t n_units,
@@ -229,41 +224,27 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const U *__restrict
                                                              uint32_t n_idx, FastDiv idx_div,
                                                              int64_t axis_dim,
                                                              int32_t *__restrict__ err) {
-    constexpr int kUnroll = 4;
     const uint32_t step = gridDim.x * kBlock;
-    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n_units; i += step * kUnroll) {
+    uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    for (; i + (kUnroll - 1) * step < n_units; i += step * kUnroll) {
         U r[kUnroll];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
-            uint32_t e = i + j * step;
-            if (e < n_units && e >= i) {
-                uint32_t row = row_div.div(e);
-                uint32_t c = e - row * row_units;
-                uint32_t outer = idx_div.div(row);
-                uint32_t jj = row - outer * n_idx;
-                int64_t ix = static_cast<int64_t>(idx[jj]);
-                if (ix < 0) ix += axis_dim;
-                if (ix < 0 || ix >= axis_dim) {
-                    if (err) *err = 1;
-                    r[j] = U{};
-                } else {
-                    r[j] = data[(static_cast<int64_t>(outer) * axis_dim + ix) * row_units + c];
-                }
-            }
-        }
+        for (int j = 0; j < kUnroll; ++j)
+            r[j] = gather_fetch<U, I>(data, idx, i + j * step, row_units, row_div, n_idx, idx_div,
+                                      axis_dim, err);
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
-            uint32_t e = i + j * step;
-            if (e < n_units && e >= i) out[e] = r[j];
-        }
+        for (int j = 0; j < kUnroll; ++j) out[i + j * step] = r[j];
     }
+    for (; i < n_units; i += step)
+        out[i] = gather_fetch<U, I>(data, idx, i, row_units, row_div, n_idx, idx_div, axis_dim,
+                                    err);
 }
 
 template <typename U>
 int32_t launch_gather(hipStream_t s, int32_t idx_dtype, const void *data, const void *idx,
                       void *out, uint32_t n_units, uint32_t row_units, uint32_t n_idx,
                       int64_t axis_dim, int32_t *err) {
-    unsigned grid = grid_for((n_units + 3) / 4, kBlock, 16);
+    unsigned grid = grid_for(n_units / kUnroll + 1, kBlock, 8);
     FastDiv rd(row_units), id(n_idx);
     if (idx_dtype == RMLK_INT64)
         gather_rows_kernel<U, int64_t><<<grid, kBlock, 0, s>>>(

@@ -18,11 +18,13 @@ __device__ __forceinline__ void nd_offsets(const NdPlan<NP> &pl, uint32_t idx, i
             uint32_t i = rem - q * pl.dim[d];
             rem = q;
 #pragma unroll
-            for (int p = 0; p < NP; ++p) offs[p] += static_cast<int64_t>(i) * pl.stride[p][d];
+            for (int p = 0; p < NP; ++p)
+                offs[p] += static_cast<int64_t>(static_cast<int32_t>(i)) * pl.stride[p][d];
         }
     }
 #pragma unroll
-    for (int p = 0; p < NP; ++p) offs[p] += static_cast<int64_t>(rem) * pl.stride[p][0];
+    for (int p = 0; p < NP; ++p)
+        offs[p] += static_cast<int64_t>(static_cast<int32_t>(rem)) * pl.stride[p][0];
 }
 
 }  // namespace rmlk

@@ -13,12 +13,25 @@ template <typename F, typename TI, typename TO, int VEC>
 __global__ __launch_bounds__(kEwBlock) void map_flat_kernel(const TI *__restrict__ in,
                                                             TO *__restrict__ out, uint32_t n) {
     const uint32_t step = gridDim.x * kEwBlock;
+    uint32_t i = blockIdx.x * kEwBlock + threadIdx.x;
     if constexpr (VEC == 1) {
-        for (uint32_t i = blockIdx.x * kEwBlock + threadIdx.x; i < n; i += step)
-            out[i] = F::apply(in[i]);
+        for (; i < n; i += step) out[i] = F::apply(in[i]);
     } else {
         const uint32_t n_vec = n / kEwVec;
-        for (uint32_t i = blockIdx.x * kEwBlock + threadIdx.x; i < n_vec; i += step) {
+        for (; i + (kEwUnroll - 1) * step < n_vec; i += kEwUnroll * step) {
+            TI ri[kEwUnroll][kEwVec];
+#pragma unroll
+            for (int u = 0; u < kEwUnroll; ++u)
+                load_vec(in + static_cast<size_t>(i + u * step) * kEwVec, false, ri[u]);
+#pragma unroll
+            for (int u = 0; u < kEwUnroll; ++u) {
+                TO ro[kEwVec];
+#pragma unroll
+                for (int j = 0; j < kEwVec; ++j) ro[j] = F::apply(ri[u][j]);
+                store_vec(out + static_cast<size_t>(i + u * step) * kEwVec, ro);
+            }
+        }
+        for (; i < n_vec; i += step) {
             TI ri[kEwVec];
             TO ro[kEwVec];
             load_vec(in + static_cast<size_t>(i) * kEwVec, false, ri);
@@ -27,8 +40,8 @@ __global__ __launch_bounds__(kEwBlock) void map_flat_kernel(const TI *__restrict
             store_vec(out + static_cast<size_t>(i) * kEwVec, ro);
         }
         if (blockIdx.x == 0 && threadIdx.x < (n - n_vec * kEwVec)) {
-            uint32_t i = n_vec * kEwVec + threadIdx.x;
-            out[i] = F::apply(in[i]);
+            uint32_t t = n_vec * kEwVec + threadIdx.x;
+            out[t] = F::apply(in[t]);
         }
     }
 }
@@ -45,7 +58,7 @@ int32_t launch_map(hipStream_t s, int64_t n, const void *in, void *out) {
         bool aligned = reinterpret_cast<uintptr_t>(pi) % ai == 0 &&
                        reinterpret_cast<uintptr_t>(po) % ao == 0;
         if (aligned) {
-            unsigned grid = grid_for(m / kEwVec + 1, kEwBlock, 16);
+            unsigned grid = grid_for(m / (kEwVec * kEwUnroll) + 1, kEwBlock, kEwBlocksPerCu);
             map_flat_kernel<F, TI, TO, kEwVec><<<grid, kEwBlock, 0, s>>>(pi, po, m);
         } else {
             unsigned grid = grid_for(m, kEwBlock, 16);

@@ -7,6 +7,15 @@ namespace rmlk {
 namespace {
 
 template <typename T>
+__device__ __forceinline__ void select_store(T *dst, const T (&x)[kEwVec], const T (&y)[kEwVec],
+                                             const uint8_t (&c)[kEwVec]) {
+    T ro[kEwVec];
+#pragma unroll
+    for (int j = 0; j < kEwVec; ++j) ro[j] = c[j] ? x[j] : y[j];
+    store_vec(dst, ro);
+}
+
+template <typename T>
 __global__ __launch_bounds__(kEwBlock) void where_flat_kernel(const T *__restrict__ x,
                                                               const T *__restrict__ y,
                                                               const uint8_t *__restrict__ c,
@@ -14,45 +23,86 @@ __global__ __launch_bounds__(kEwBlock) void where_flat_kernel(const T *__restric
                                                               int x_b, int y_b, int c_b) {
     const uint32_t n_vec = n / kEwVec;
     const uint32_t step = gridDim.x * kEwBlock;
-    for (uint32_t i = blockIdx.x * kEwBlock + threadIdx.x; i < n_vec; i += step) {
-        T rx[kEwVec], ry[kEwVec], ro[kEwVec];
+    uint32_t i = blockIdx.x * kEwBlock + threadIdx.x;
+    for (; i + (kEwUnroll - 1) * step < n_vec; i += kEwUnroll * step) {
+        T rx[kEwUnroll][kEwVec], ry[kEwUnroll][kEwVec];
+        uint8_t rc[kEwUnroll][kEwVec];
+#pragma unroll
+        for (int u = 0; u < kEwUnroll; ++u) {
+            const size_t e = static_cast<size_t>(i + u * step) * kEwVec;
+            load_vec(x_b ? x : x + e, x_b != 0, rx[u]);
+            load_vec(y_b ? y : y + e, y_b != 0, ry[u]);
+            load_vec(c_b ? c : c + e, c_b != 0, rc[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kEwUnroll; ++u)
+            select_store(out + static_cast<size_t>(i + u * step) * kEwVec, rx[u], ry[u], rc[u]);
+    }
+    for (; i < n_vec; i += step) {
+        T rx[kEwVec], ry[kEwVec];
         uint8_t rc[kEwVec];
-        size_t e = static_cast<size_t>(i) * kEwVec;
+        const size_t e = static_cast<size_t>(i) * kEwVec;
         load_vec(x_b ? x : x + e, x_b != 0, rx);
         load_vec(y_b ? y : y + e, y_b != 0, ry);
         load_vec(c_b ? c : c + e, c_b != 0, rc);
-#pragma unroll
-        for (int j = 0; j < kEwVec; ++j) ro[j] = rc[j] ? rx[j] : ry[j];
-        store_vec(out + e, ro);
+        select_store(out + e, rx, ry, rc);
     }
     if (blockIdx.x == 0 && threadIdx.x < (n - n_vec * kEwVec)) {
-        uint32_t i = n_vec * kEwVec + threadIdx.x;
-        out[i] = c[c_b ? 0 : i] ? x[x_b ? 0 : i] : y[y_b ? 0 : i];
+        uint32_t t = n_vec * kEwVec + threadIdx.x;
+        out[t] = c[c_b ? 0 : t] ? x[x_b ? 0 : t] : y[y_b ? 0 : t];
     }
 }
 
 // plan operands: 0 = x, 1 = y, 2 = cond, 3 = out
-template <typename T, int VEC>
-__global__ __launch_bounds__(kEwBlock) void where_nd_kernel(NdPlan<4> pl, const T *__restrict__ x,
+template <typename T, int VEC, int UNR>
+__global__ __launch_bounds__(kEwBlock) void where_nd_kernel(NdPlan<4> pl, EwUnrollDim<4> ud,
+                                                            const T *__restrict__ x,
                                                             const T *__restrict__ y,
                                                             const uint8_t *__restrict__ c,
                                                             T *__restrict__ out, uint32_t n_items,
                                                             int x0, int y0, int c0) {
     const uint32_t step = gridDim.x * kEwBlock;
-    for (uint32_t i = blockIdx.x * kEwBlock + threadIdx.x; i < n_items; i += step) {
-        int64_t offs[4];
-        nd_offsets<4>(pl, i, offs);
-        if constexpr (VEC == 1) {
+    uint32_t i = blockIdx.x * kEwBlock + threadIdx.x;
+    if constexpr (VEC == 1) {
+        for (; i < n_items; i += step) {
+            int64_t offs[4];
+            nd_offsets<4>(pl, i, offs);
             out[offs[3]] = c[offs[2]] ? x[offs[0]] : y[offs[1]];
-        } else {
-            T rx[kEwVec], ry[kEwVec], ro[kEwVec];
-            uint8_t rc[kEwVec];
-            load_vec(x + offs[0], x0 != 0, rx);
-            load_vec(y + offs[1], y0 != 0, ry);
-            load_vec(c + offs[2], c0 != 0, rc);
+        }
+    } else {
+        for (; i < n_items; i += step) {
+            int64_t offs[4];
+            nd_offsets<4>(pl, i, offs);
+            T rx[UNR][kEwVec], ry[UNR][kEwVec];
+            uint8_t rc[UNR][kEwVec];
+            load_vec(x + offs[0], x0 != 0, rx[0]);
+            load_vec(y + offs[1], y0 != 0, ry[0]);
+            load_vec(c + offs[2], c0 != 0, rc[0]);
 #pragma unroll
-            for (int j = 0; j < kEwVec; ++j) ro[j] = rc[j] ? rx[j] : ry[j];
-            store_vec(out + offs[3], ro);
+            for (int u = 1; u < UNR; ++u) {
+                if (ud.stride[0] != 0) {
+                    load_vec(x + offs[0] + static_cast<int64_t>(u) * ud.stride[0], x0 != 0, rx[u]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < kEwVec; ++j) rx[u][j] = rx[0][j];
+                }
+                if (ud.stride[1] != 0) {
+                    load_vec(y + offs[1] + static_cast<int64_t>(u) * ud.stride[1], y0 != 0, ry[u]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < kEwVec; ++j) ry[u][j] = ry[0][j];
+                }
+                if (ud.stride[2] != 0) {
+                    load_vec(c + offs[2] + static_cast<int64_t>(u) * ud.stride[2], c0 != 0, rc[u]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < kEwVec; ++j) rc[u][j] = rc[0][j];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UNR; ++u)
+                select_store(out + offs[3] + static_cast<int64_t>(u) * ud.stride[3], rx[u], ry[u],
+                             rc[u]);
         }
     }
 }
@@ -69,20 +119,26 @@ int32_t launch_where(hipStream_t stream, int rank, const int64_t *shape,
     unsigned grid;
     switch (dec.shape) {
         case EwShape::Flat:
-            grid = grid_for(dec.n_items / kEwVec + 1, kEwBlock, 16);
+            grid = grid_for(dec.n_items / (kEwVec * kEwUnroll) + 1, kEwBlock, kEwBlocksPerCu);
             where_flat_kernel<T><<<grid, kEwBlock, 0, stream>>>(x, y, c, out, dec.n_items,
                                                                 dec.inner0[0], dec.inner0[1],
                                                                 dec.inner0[2]);
             break;
         case EwShape::Nd4:
-            grid = grid_for(dec.n_items, kEwBlock, 16);
-            where_nd_kernel<T, kEwVec><<<grid, kEwBlock, 0, stream>>>(
-                dec.plan, x, y, c, out, dec.n_items, dec.inner0[0], dec.inner0[1], dec.inner0[2]);
+            grid = grid_for(dec.n_items, kEwBlock, kEwBlocksPerCu);
+            if (dec.unrolled)
+                where_nd_kernel<T, kEwVec, kEwUnroll><<<grid, kEwBlock, 0, stream>>>(
+                    dec.plan, dec.udim, x, y, c, out, dec.n_items, dec.inner0[0], dec.inner0[1],
+                    dec.inner0[2]);
+            else
+                where_nd_kernel<T, kEwVec, 1><<<grid, kEwBlock, 0, stream>>>(
+                    dec.plan, dec.udim, x, y, c, out, dec.n_items, dec.inner0[0], dec.inner0[1],
+                    dec.inner0[2]);
             break;
         case EwShape::Nd1:
             grid = grid_for(dec.n_items, kEwBlock, 16);
-            where_nd_kernel<T, 1><<<grid, kEwBlock, 0, stream>>>(dec.plan, x, y, c, out,
-                                                                 dec.n_items, 0, 0, 0);
+            where_nd_kernel<T, 1, 1><<<grid, kEwBlock, 0, stream>>>(dec.plan, dec.udim, x, y, c,
+                                                                    out, dec.n_items, 0, 0, 0);
             break;
     }
     return launch_status();
