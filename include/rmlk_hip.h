@@ -220,6 +220,17 @@ int32_t rmlk_hip_trilu(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64
 int32_t rmlk_hip_fill(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *value,
                       void *out);
 
+/* Range: out[i] = start + i * delta for i < n. `start` and `delta` are HOST scalars of `dtype`
+ * (FLOAT, DOUBLE, INT32, INT64). ref: runtime/src/providers/cuda/backend/range.rs:103-109 (the
+ * reference fills a host vector and uploads it). */
+int32_t rmlk_hip_range(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *start,
+                       const void *delta, void *out);
+
+/* Write up to 256 bytes from host memory `src` to device memory `dst`. The bytes travel as kernel
+ * arguments: no staging copy, nothing to keep alive, recordable into a HIP graph.
+ * ref: runtime/src/providers/cuda/backend/shape.rs:67-72 (host vector + H2D for tiny tensors). */
+int32_t rmlk_hip_write_small(rmlk_stream_t stream, void *dst, const void *src, size_t bytes);
+
 /* ---------------------------------------------------------------------------------------------
  * Memory and stream helpers (what the provider used cudarc for,
  * ref: runtime/src/providers/cuda/allocator.rs:96-139, data.rs:24-25, store.rs:385-416).

@@ -1,0 +1,124 @@
+/*
+ * rmlk_runtime.h -- C ABI of the host side that sits above the kernels of rmlk_hip.h: the graph
+ * builder, the operator dispatch and the sequential executor. It is the C++ stand-in for the
+ * reference's Rust layers on this path (no Rust toolchain ships with this build):
+ *
+ *   rmlk_graph_*    <->  schema::GraphBuilder             (ref: schema/src/builder.rs:49-260)
+ *   rmlk_session_*  <->  runtime::Builder / ModelInstance (ref: runtime/src/core/instance.rs:89-222)
+ *   operator table  <->  CudaKernel / OperationBackend    (ref: runtime/src/providers/cuda/backend/mod.rs:82-162)
+ *
+ * Every function returns 0 on success or a negative rmlk_status / positive hipError_t; the text of
+ * the last error of the calling thread is kept for rmlk_last_error(). Two texts are API, as in the
+ * reference (ref: runtime/src/core/error.rs:6,10): an unsupported element type reports a message
+ * that starts with "unsupported data type", an unsupported Cast pair one that starts with
+ * "unsupported cast".
+ */
+#ifndef RMLK_RUNTIME_H
+#define RMLK_RUNTIME_H
+
+#include "rmlk_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct rmlk_graph rmlk_graph;
+typedef struct rmlk_session rmlk_session;
+
+#define RMLK_ERR_GRAPH (-20)   /* graph construction error (duplicate / unknown name ...) */
+#define RMLK_ERR_OP (-21)      /* an operator rejected its inputs (shape, attribute, dtype) */
+#define RMLK_ERR_KERNEL (-22)  /* a kernel raised its device error flag (index out of range) */
+
+const char *rmlk_last_error(void);
+
+/* ---- graph building (ref: schema/src/builder.rs) ------------------------------------------- */
+int32_t rmlk_graph_create(rmlk_graph **out);
+void rmlk_graph_destroy(rmlk_graph *g);
+
+/* Graph input. dims may hold 0 for a dim only known at run time. ref: builder.rs:66-77 */
+int32_t rmlk_graph_input(rmlk_graph *g, const char *name, int32_t dtype, const int64_t *dims,
+                         int32_t rank);
+/* Initializer: `data` (host, dense, prod(dims) elements of dtype) is copied. ref: builder.rs:83-96 */
+int32_t rmlk_graph_constant(rmlk_graph *g, const char *name, int32_t dtype, const int64_t *dims,
+                            int32_t rank, const void *data);
+/* Append an operator node; `op` is the ONNX operator name ("MatMul", "ScatterND", ...). Inputs
+ * may be "" for an omitted optional input. Output values are declared implicitly.
+ * Returns the node index (>= 0) or an error (< 0). ref: builder.rs:128-190 */
+int32_t rmlk_graph_op(rmlk_graph *g, const char *op, const char *const *inputs, int32_t n_inputs,
+                      const char *const *outputs, int32_t n_outputs);
+/* Attributes of node `node` (ref: schema/src/attributes.rs AttributeType::{Int,Float,Ints,Floats,String,Tensor}) */
+int32_t rmlk_graph_attr_int(rmlk_graph *g, int32_t node, const char *name, int64_t value);
+int32_t rmlk_graph_attr_float(rmlk_graph *g, int32_t node, const char *name, float value);
+int32_t rmlk_graph_attr_ints(rmlk_graph *g, int32_t node, const char *name, const int64_t *values,
+                             int32_t n);
+int32_t rmlk_graph_attr_floats(rmlk_graph *g, int32_t node, const char *name, const float *values,
+                               int32_t n);
+int32_t rmlk_graph_attr_string(rmlk_graph *g, int32_t node, const char *name, const char *value);
+int32_t rmlk_graph_attr_tensor(rmlk_graph *g, int32_t node, const char *name, int32_t dtype,
+                               const int64_t *dims, int32_t rank, const void *data);
+/* Mark a value as graph output. ref: builder.rs:192-204 */
+int32_t rmlk_graph_output(rmlk_graph *g, const char *name);
+
+/* ---- sessions (ref: runtime/src/core/instance.rs) ------------------------------------------- */
+/* Validates the graph, uploads the initializers to `device`, creates the stream.
+ * ref: Builder::build, instance.rs:198-221 and TensorStore::init, providers/cuda/store.rs:95-261 */
+int32_t rmlk_session_create(const rmlk_graph *g, int32_t device, rmlk_session **out);
+void rmlk_session_destroy(rmlk_session *s);
+
+/* Feed a graph input from host memory (copied to a session-owned device buffer, H2D on the
+ * session stream). ref: ExecutionState::load_value, core/execution_state.rs:117-196 */
+int32_t rmlk_session_set_input(rmlk_session *s, const char *name, int32_t dtype,
+                               const int64_t *dims, int32_t rank, const void *host_data);
+/* Feed a graph input from device memory the caller owns (no copy; must stay valid until the run
+ * has finished). With `donate` != 0 an operator may update the buffer in place (ScatterND writing
+ * one row of a KV cache) instead of copying it first. */
+int32_t rmlk_session_bind_input(rmlk_session *s, const char *name, int32_t dtype,
+                                const int64_t *dims, int32_t rank, void *device_data,
+                                int32_t donate);
+/* Use output `out_name` of the previous run as input `in_name` of the next one without leaving
+ * the device (the reference's example round-trips every present.* through the host,
+ * ref: runtime/examples/llama.rs:96-117). */
+int32_t rmlk_session_feed_output(rmlk_session *s, const char *out_name, const char *in_name);
+
+/* Execute all nodes in stored order on the session stream; returns when everything is enqueued
+ * and the kernels' error flags have been checked (one small D2H at the end of the run).
+ * ref: ModelInstance::run, instance.rs:89-119 */
+int32_t rmlk_session_run(rmlk_session *s);
+
+/* Shape / dtype / device pointer of a graph output after a run. dims must hold RMLK_MAX_RANK. */
+int32_t rmlk_session_output_info(rmlk_session *s, const char *name, int32_t *dtype, int64_t *dims,
+                                 int32_t *rank, void **device_data);
+/* Blocking copy of a graph output to host memory (`bytes` must equal the output's size).
+ * ref: ExecutionState::get_value, core/execution_state.rs:201-225 */
+int32_t rmlk_session_read_output(rmlk_session *s, const char *name, void *host_data,
+                                 size_t bytes);
+
+/* Record the run for the current input shapes into a HIP graph, then replay it with
+ * rmlk_session_replay (inputs are re-read from the same buffers; set_input with unchanged shapes
+ * refreshes them in place). Needs one plain rmlk_session_run with the same shapes first. Shapes
+ * must not depend on input VALUES between replays. */
+int32_t rmlk_session_capture(rmlk_session *s);
+int32_t rmlk_session_replay(rmlk_session *s);
+
+int32_t rmlk_session_sync(rmlk_session *s);
+/* hipStream_t the session enqueues on */
+rmlk_stream_t rmlk_session_stream(rmlk_session *s);
+
+/* Per-node timing of the next runs with HIP events on the session stream (0 = off).
+ * rmlk_session_node_count / node_info describe node i: ONNX op name, last duration in
+ * microseconds (negative when not timed), bytes read + written and floating-point operations the
+ * operator's definition implies for the shapes of the last run. */
+int32_t rmlk_session_set_profiling(rmlk_session *s, int32_t enabled);
+int32_t rmlk_session_node_count(rmlk_session *s);
+int32_t rmlk_session_node_info(rmlk_session *s, int32_t node, const char **op, double *micros,
+                               double *bytes, double *flops);
+
+/* Device bytes the session's buffer pool holds, and how many times it went to the HIP
+ * allocator (steady state: a run allocates nothing new). */
+int32_t rmlk_session_memory_stats(rmlk_session *s, int64_t *pool_bytes, int64_t *hip_mallocs,
+                                  int64_t *device_syncs);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RMLK_RUNTIME_H */

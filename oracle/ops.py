@@ -238,7 +238,7 @@ def transpose(x, perm=None):
     x = np.asarray(x)
     if perm is None:
         perm = list(range(x.ndim))[::-1]
-    return np.ascontiguousarray(np.transpose(x, [int(p) for p in perm]))
+    return np.asarray(order="C", a=np.transpose(x, [int(p) for p in perm]))
 
 
 def expand(x, shape):
@@ -248,7 +248,7 @@ def expand(x, shape):
         out_shape = np.broadcast_shapes(x.shape, tuple(int(s) for s in shape))
     except ValueError as e:
         raise OracleError("incompatible shapes for expand") from e
-    return np.ascontiguousarray(np.broadcast_to(x, out_shape))
+    return np.asarray(order="C", a=np.broadcast_to(x, out_shape))
 
 
 def slice_resolve(shape, starts, ends, axes=None, steps=None):
@@ -262,6 +262,8 @@ def slice_resolve(shape, starts, ends, axes=None, steps=None):
         steps = [1] * len(starts)
     if len(steps) != len(axes):
         raise OracleError("StepsAndAxesLengthMismatch")
+    if len(axes) != len(starts) or len(starts) != len(ends):
+        raise OracleError("axes must have the same length as starts")
     res = [(0, 1, int(shape[d])) for d in range(rank)]
     for i, raw_axis in enumerate(axes):
         axis = int(raw_axis)
@@ -308,7 +310,7 @@ def slice_(x, starts, ends, axes=None, steps=None):
                         None if axes is None else list(np.asarray(axes).reshape(-1)),
                         None if steps is None else list(np.asarray(steps).reshape(-1)))
     idx = tuple(np.arange(c, dtype=np.int64) * st + s for (s, st, c) in res)
-    return np.ascontiguousarray(x[np.ix_(*idx)]) if x.ndim else x.copy()
+    return np.asarray(order="C", a=x[np.ix_(*idx)]) if x.ndim else x.copy()
 
 
 def concat(xs, axis):
@@ -336,7 +338,7 @@ def gather(data, indices, axis=0):
     dim = data.shape[ax]
     flat = [normalize_index(i, dim) for i in indices.reshape(-1)]
     idx = np.array(flat, dtype=np.int64).reshape(indices.shape)
-    return np.ascontiguousarray(np.take(data, idx, axis=ax))
+    return np.asarray(order="C", a=np.take(data, idx, axis=ax))
 
 
 def scatter_nd(data, indices, updates, reduction="none"):

@@ -82,6 +82,8 @@ SIGNATURES = {
     "rmlk_hip_trilu": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int32, c_int64,
                                  c_void_p, c_void_p]),
     "rmlk_hip_fill": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
+    "rmlk_hip_range": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p]),
+    "rmlk_hip_write_small": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "rmlk_hip_malloc": (c_int32, [POINTER(c_void_p), c_size_t]),
     "rmlk_hip_free": (c_int32, [c_void_p]),
     "rmlk_hip_memcpy_htod": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
@@ -92,6 +94,46 @@ SIGNATURES = {
     "rmlk_hip_device_info": (c_int32, [c_int32, POINTER(DeviceInfo)]),
     "rmlk_hip_status_string": (c_char_p, [c_int32]),
     "rmlk_hip_version": (c_char_p, []),
+    # include/rmlk_runtime.h
+    "rmlk_last_error": (c_char_p, []),
+    "rmlk_graph_create": (c_int32, [POINTER(c_void_p)]),
+    "rmlk_graph_destroy": (None, [c_void_p]),
+    "rmlk_graph_input": (c_int32, [c_void_p, c_char_p, c_int32, POINTER(c_int64), c_int32]),
+    "rmlk_graph_constant": (c_int32, [c_void_p, c_char_p, c_int32, POINTER(c_int64), c_int32,
+                                      c_void_p]),
+    "rmlk_graph_op": (c_int32, [c_void_p, c_char_p, POINTER(c_char_p), c_int32, POINTER(c_char_p),
+                                c_int32]),
+    "rmlk_graph_attr_int": (c_int32, [c_void_p, c_int32, c_char_p, c_int64]),
+    "rmlk_graph_attr_float": (c_int32, [c_void_p, c_int32, c_char_p, ctypes.c_float]),
+    "rmlk_graph_attr_ints": (c_int32, [c_void_p, c_int32, c_char_p, POINTER(c_int64), c_int32]),
+    "rmlk_graph_attr_floats": (c_int32, [c_void_p, c_int32, c_char_p, POINTER(ctypes.c_float),
+                                         c_int32]),
+    "rmlk_graph_attr_string": (c_int32, [c_void_p, c_int32, c_char_p, c_char_p]),
+    "rmlk_graph_attr_tensor": (c_int32, [c_void_p, c_int32, c_char_p, c_int32, POINTER(c_int64),
+                                         c_int32, c_void_p]),
+    "rmlk_graph_output": (c_int32, [c_void_p, c_char_p]),
+    "rmlk_session_create": (c_int32, [c_void_p, c_int32, POINTER(c_void_p)]),
+    "rmlk_session_destroy": (None, [c_void_p]),
+    "rmlk_session_set_input": (c_int32, [c_void_p, c_char_p, c_int32, POINTER(c_int64), c_int32,
+                                         c_void_p]),
+    "rmlk_session_bind_input": (c_int32, [c_void_p, c_char_p, c_int32, POINTER(c_int64), c_int32,
+                                          c_void_p, c_int32]),
+    "rmlk_session_feed_output": (c_int32, [c_void_p, c_char_p, c_char_p]),
+    "rmlk_session_run": (c_int32, [c_void_p]),
+    "rmlk_session_output_info": (c_int32, [c_void_p, c_char_p, POINTER(c_int32), POINTER(c_int64),
+                                           POINTER(c_int32), POINTER(c_void_p)]),
+    "rmlk_session_read_output": (c_int32, [c_void_p, c_char_p, c_void_p, c_size_t]),
+    "rmlk_session_capture": (c_int32, [c_void_p]),
+    "rmlk_session_replay": (c_int32, [c_void_p]),
+    "rmlk_session_sync": (c_int32, [c_void_p]),
+    "rmlk_session_stream": (c_void_p, [c_void_p]),
+    "rmlk_session_set_profiling": (c_int32, [c_void_p, c_int32]),
+    "rmlk_session_node_count": (c_int32, [c_void_p]),
+    "rmlk_session_node_info": (c_int32, [c_void_p, c_int32, POINTER(c_char_p),
+                                         POINTER(ctypes.c_double), POINTER(ctypes.c_double),
+                                         POINTER(ctypes.c_double)]),
+    "rmlk_session_memory_stats": (c_int32, [c_void_p, POINTER(c_int64), POINTER(c_int64),
+                                            POINTER(c_int64)]),
 }
 
 _lib = None

@@ -1,0 +1,240 @@
+// Host-side runtime above the kernel C ABI: tensors, the device buffer pool, graphs, sessions.
+// C++ stand-in for the reference's provider layer (runtime/src/providers/cuda/*.rs) and for the
+// sequential executor of runtime/src/core/instance.rs.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../../include/rmlk_runtime.h"
+
+namespace rmlk {
+namespace rt {
+
+// ---- errors -----------------------------------------------------------------------------------
+struct RtError : std::runtime_error {
+    int32_t code;
+    RtError(int32_t c, const std::string &m) : std::runtime_error(m), code(c) {}
+};
+
+// Rust `Debug` spelling of schema::DataType, used in the two error texts that are API
+// (runtime/src/core/error.rs:6,10,24-28).
+const char *dtype_name(int32_t dt);
+size_t dtype_size(int32_t dt);
+[[noreturn]] void fail_unsupported(int32_t dt);
+[[noreturn]] void fail_op(const std::string &msg);
+void check_status(int32_t st, const char *where);
+void check_hip(hipError_t e, const char *where);
+
+// ---- device memory ----------------------------------------------------------------------------
+// Caching pool: sizes are rounded to a bucket, freed blocks are kept per bucket and handed out
+// again in LIFO order, so a run with the same shapes meets the same addresses again and never
+// reaches hipMalloc after the first time. (The reference bumps inside two 4 KiB arenas and falls
+// back to cuMemAlloc for almost every tensor, providers/cuda/allocator.rs:96-139.)
+class Pool {
+public:
+    ~Pool();
+    void *alloc(size_t bytes);
+    void release(void *p, size_t bytes);
+    static size_t bucket(size_t bytes);
+    int64_t pool_bytes = 0;
+    int64_t hip_mallocs = 0;
+    bool forbid_malloc = false;  // set while a HIP graph is being captured
+
+private:
+    std::map<size_t, std::vector<void *>> free_;
+    std::vector<void *> all_;
+};
+
+struct Buffer {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+    Pool *pool = nullptr;   // null: memory the session does not own (bound by the caller)
+    bool owned_raw = false; // hipMalloc'ed outside the pool (initializers)
+    bool donated = false;   // an operator may overwrite it in place
+    ~Buffer();
+};
+using BufferRef = std::shared_ptr<Buffer>;
+
+// ---- small tensors mirrored on the host ---------------------------------------------------------
+// Shape arithmetic (Shape -> Gather -> Concat -> Reshape ...) runs on the device like any other
+// operator; operators additionally keep the VALUES of small integer tensors on the host when all
+// their inputs are known there, so that a later Reshape / Slice / Expand / Range does not have to
+// stall the stream with a device-to-host read (the reference reads back every time,
+// e.g. backend/reshape.rs:102-103, backend/slice.rs:262-335).
+constexpr int64_t kHostMirrorMax = 64;
+struct HostVal {
+    bool is_float = false;
+    std::vector<int64_t> i;  // integer / bool values
+    std::vector<double> f;   // floating values
+    size_t size() const { return is_float ? f.size() : i.size(); }
+    int64_t as_int(size_t k) const { return is_float ? static_cast<int64_t>(f[k]) : i[k]; }
+    double as_double(size_t k) const { return is_float ? f[k] : static_cast<double>(i[k]); }
+};
+
+struct Tensor {
+    int32_t dtype = 0;
+    std::vector<int64_t> shape;
+    BufferRef buf;
+    size_t offset = 0;  // bytes into buf
+    std::shared_ptr<HostVal> host;
+
+    bool defined() const { return dtype != 0; }
+    int64_t numel() const {
+        int64_t n = 1;
+        for (int64_t d : shape) n *= d;
+        return n;
+    }
+    size_t nbytes() const { return static_cast<size_t>(numel()) * dtype_size(dtype); }
+    void *data() const { return buf ? static_cast<char *>(buf->ptr) + offset : nullptr; }
+    int rank() const { return static_cast<int>(shape.size()); }
+    void reset() {
+        dtype = 0;
+        shape.clear();
+        buf.reset();
+        offset = 0;
+        host.reset();
+    }
+};
+
+rmlk_dims to_dims(const std::vector<int64_t> &v);          // rank-0 becomes [1]
+std::vector<int64_t> dense_strides(const std::vector<int64_t> &shape);
+int64_t normalize_axis(int64_t axis, int64_t rank, const char *what);
+
+// ---- graph ------------------------------------------------------------------------------------
+struct HostTensor {
+    int32_t dtype = 0;
+    std::vector<int64_t> shape;
+    std::vector<uint8_t> data;
+    int64_t numel() const {
+        int64_t n = 1;
+        for (int64_t d : shape) n *= d;
+        return n;
+    }
+};
+
+struct Attr {
+    enum Kind { Int, Float, Ints, Floats, String, TensorK } kind = Int;
+    int64_t i = 0;
+    float f = 0.f;
+    std::vector<int64_t> ints;
+    std::vector<float> floats;
+    std::string s;
+    HostTensor t;
+};
+
+struct Node {
+    std::string op;
+    std::vector<int> inputs;   // value ids, -1 = omitted optional input
+    std::vector<int> outputs;
+    std::unordered_map<std::string, Attr> attrs;
+};
+
+struct Value {
+    std::string name;
+    int32_t dtype = 0;             // declared (0 = inferred at run time)
+    std::vector<int64_t> shape;    // declared
+    bool is_input = false, is_initializer = false, is_output = false;
+    int producer = -1;             // node index
+    HostTensor init;               // initializer payload
+};
+
+}  // namespace rt
+}  // namespace rmlk
+
+struct rmlk_graph {
+    std::vector<rmlk::rt::Value> values;
+    std::vector<rmlk::rt::Node> nodes;
+    std::unordered_map<std::string, int> by_name;
+    std::vector<int> inputs, outputs;
+    int value_id(const std::string &name, bool create);
+};
+
+namespace rmlk {
+namespace rt {
+
+struct Session;
+
+// What an operator sees (ref: runtime/src/core/context.rs:41-145).
+struct OpContext {
+    Session &session;
+    const Node &node;
+    int node_index;
+    std::vector<Tensor *> in;   // nullptr for an omitted optional input
+    std::vector<Tensor *> out;
+    hipStream_t stream;
+
+    int n_inputs() const { return static_cast<int>(in.size()); }
+    bool has_input(int i) const { return i < n_inputs() && in[i] && in[i]->defined(); }
+    const Tensor &input(int i) const;
+    // Allocate output i (dense) from the pool.
+    Tensor &alloc_output(int i, int32_t dtype, const std::vector<int64_t> &shape);
+    // Output i shares the memory of `src` with a new shape (Reshape, Unsqueeze).
+    Tensor &view_output(int i, const Tensor &src, const std::vector<int64_t> &shape);
+
+    const Attr *attr(const char *name) const;
+    int64_t attr_int(const char *name, int64_t dflt) const;
+    std::vector<int64_t> attr_ints(const char *name, bool *present = nullptr) const;
+    std::string attr_string(const char *name, const std::string &dflt) const;
+
+    // Values of a small integer / float input on the host: the mirror when present, otherwise a
+    // blocking device-to-host copy (counted in the session's sync statistics).
+    HostVal host_values(int i) const;
+    int32_t *error_flag() const;
+    void *scratch(size_t bytes) const;  // per-run device scratch (MatMul split-K partials)
+};
+
+using OpFn = void (*)(OpContext &);
+OpFn find_op(const std::string &name);
+
+struct CapturedPlan {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    std::vector<Tensor> pinned;  // every value alive at the end of the captured run
+    ~CapturedPlan();
+};
+
+struct Session {
+    const rmlk_graph *g = nullptr;  // copied at creation
+    rmlk_graph graph_copy;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    Pool pool;
+    std::vector<Tensor> values;      // by value id
+    std::vector<int> last_use;       // node index of the last consumer, -1 = never read
+    std::vector<BufferRef> scratch_bufs;
+    int32_t *err_flag = nullptr;     // device
+    int32_t *err_host = nullptr;     // pinned host
+    bool capturing = false;
+    bool profiling = false;
+    int64_t device_syncs = 0;
+    std::unique_ptr<CapturedPlan> plan;
+    struct NodeStat {
+        double micros = -1.0, bytes = 0.0, flops = 0.0;
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+    };
+    std::vector<NodeStat> stats;
+
+    ~Session();
+    void build(const rmlk_graph &graph, int dev);
+    void run_nodes();
+    void run();
+    void capture();
+    void replay();
+    void check_error_flag();
+};
+
+}  // namespace rt
+}  // namespace rmlk
+
+struct rmlk_session {
+    rmlk::rt::Session impl;
+};

@@ -1,6 +1,7 @@
 // Contiguous maps: Sqrt Neg Sin Cos Sigmoid, Cast, Fill.
 // Replaces cuda/src/ptx/{sqrt,neg,sin,cos,cast}.cu (cuda/src/ptx/headers/unary_op_macro.cuh:1-11,
 // cast_op_macro.cuh:1-11) and the cuDNN sigmoid call (cuda/src/kernels/activation.rs:6-39).
+#include <cstring>
 #include <limits>
 #include <type_traits>
 
@@ -178,10 +179,66 @@ __global__ __launch_bounds__(kEwBlock) void fill_kernel(T *__restrict__ out, T v
         out[i] = value;
 }
 
+template <typename T>
+__global__ __launch_bounds__(kEwBlock) void range_kernel(T *__restrict__ out, T start, T delta,
+                                                         uint64_t n) {
+    const uint64_t step = static_cast<uint64_t>(gridDim.x) * kEwBlock;
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kEwBlock + threadIdx.x; i < n; i += step) {
+        if constexpr (std::is_integral<T>::value) {
+            using U = typename std::make_unsigned<T>::type;
+            out[i] = static_cast<T>(static_cast<U>(start) + static_cast<U>(i) * static_cast<U>(delta));
+        } else {
+            out[i] = static_cast<T>(static_cast<double>(start) +
+                                    static_cast<double>(i) * static_cast<double>(delta));
+        }
+    }
+}
+
+struct SmallPayload {
+    uint32_t w[64];
+};
+
+__global__ void write_small_kernel(uint8_t *__restrict__ dst, SmallPayload p, uint32_t bytes) {
+    const uint8_t *src = reinterpret_cast<const uint8_t *>(p.w);
+    for (uint32_t i = threadIdx.x; i < bytes; i += blockDim.x) dst[i] = src[i];
+}
+
 }  // namespace
 }  // namespace rmlk
 
 using namespace rmlk;
+
+extern "C" int32_t rmlk_hip_range(rmlk_stream_t stream, int32_t dtype, int64_t n,
+                                  const void *start, const void *delta, void *out) {
+    if (n < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n >= kMaxElems) return RMLK_ERR_TOO_LARGE;
+    if (dtype != RMLK_FLOAT && dtype != RMLK_DOUBLE && dtype != RMLK_INT32 && dtype != RMLK_INT64)
+        return RMLK_ERR_UNSUPPORTED;
+    if (n == 0) return RMLK_OK;
+    if (!start || !delta || !out) return RMLK_ERR_NULL_POINTER;
+    hipStream_t s = as_stream(stream);
+    unsigned grid = grid_for(n, kEwBlock, 16);
+    switch (dtype) {
+        case RMLK_FLOAT: range_kernel<float><<<grid, kEwBlock, 0, s>>>(static_cast<float *>(out), *static_cast<const float *>(start), *static_cast<const float *>(delta), n); break;
+        case RMLK_DOUBLE: range_kernel<double><<<grid, kEwBlock, 0, s>>>(static_cast<double *>(out), *static_cast<const double *>(start), *static_cast<const double *>(delta), n); break;
+        case RMLK_INT32: range_kernel<int32_t><<<grid, kEwBlock, 0, s>>>(static_cast<int32_t *>(out), *static_cast<const int32_t *>(start), *static_cast<const int32_t *>(delta), n); break;
+        default: range_kernel<int64_t><<<grid, kEwBlock, 0, s>>>(static_cast<int64_t *>(out), *static_cast<const int64_t *>(start), *static_cast<const int64_t *>(delta), n); break;
+    }
+    return launch_status();
+}
+
+extern "C" int32_t rmlk_hip_write_small(rmlk_stream_t stream, void *dst, const void *src,
+                                        size_t bytes) {
+    if (bytes == 0) return RMLK_OK;
+    if (bytes > sizeof(SmallPayload)) return RMLK_ERR_INVALID_ARGUMENT;
+    if (!dst || !src) return RMLK_ERR_NULL_POINTER;
+    SmallPayload p;
+    std::memset(&p, 0, sizeof(p));
+    std::memcpy(&p, src, bytes);
+    write_small_kernel<<<1, 64, 0, as_stream(stream)>>>(static_cast<uint8_t *>(dst), p,
+                                                        static_cast<uint32_t>(bytes));
+    return launch_status();
+}
 
 extern "C" int32_t rmlk_hip_unary(rmlk_stream_t stream, int32_t op, int32_t dtype, int64_t n,
                                   const void *in, void *out) {

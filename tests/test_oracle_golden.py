@@ -1,0 +1,264 @@
+"""CPU: the oracle against every known-answer vector extracted from the reference's own tests
+(tests/golden/reference_cases.json), the ONNX-Runtime-produced attention fixture the reference
+holds, and the loop restatement of the reference kernels. Nothing here touches the GPU."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from optest import decode
+from oracle import graph as ograph
+from oracle import loops, ops
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CASES = json.load(open(os.path.join(HERE, "golden", "reference_cases.json")))
+PROVIDER = [c for c in CASES["provider_cases"]]
+
+
+class _Node:
+    def __init__(self, op, inputs, outputs, attrs):
+        self.op, self.inputs, self.outputs, self.attrs = op, inputs, outputs, attrs
+
+
+class _Graph:
+    def __init__(self, nodes, inits, outputs):
+        self.nodes, self.initializers, self.outputs = nodes, inits, outputs
+
+
+def case_attrs(case):
+    attrs = {}
+    for k, v in case["attrs"].items():
+        if isinstance(v, dict) and "tensor" in v:
+            t = v["tensor"]
+            attrs[k] = decode(t["data"], t["dtype"] or "float32").reshape(t["dims"])
+        elif isinstance(v, dict) and "floats" in v:
+            attrs[k] = [float(x) for x in v["floats"]]
+        else:
+            attrs[k] = v
+    return attrs
+
+
+def one_op_graph(case):
+    names, env = [], {}
+    for i, f in enumerate(case["feeds"]):
+        env[f"v{i}"] = decode(f["data"], f["dtype"]).reshape(f["dims"])
+        names.append(f"v{i}")
+    attrs = case_attrs(case)
+    op = case["op"]
+    return _Graph([_Node(op, names, ["y"], attrs)], {}, ["y"]), env
+
+
+def expected_of(case, got):
+    return decode(case["expected"], got.dtype)
+
+
+@pytest.mark.parametrize("case", PROVIDER, ids=[f"{c['op']}-{c['test']}" for c in PROVIDER])
+def test_oracle_matches_reference_provider_vectors(case):
+    g, env = one_op_graph(case)
+    if case.get("expect_error"):
+        # dtype gates are properties of the operator dispatch, not of the arithmetic: only the
+        # shape / argument errors concern the oracle
+        if any("unsupported" in s for s in case.get("error_contains", [])):
+            pytest.skip("element-type gate: checked against the runtime, not the oracle")
+        with pytest.raises(Exception):
+            ograph.run_graph(g, env)
+        return
+    got = np.asarray(ograph.run_graph(g, env)["y"])
+    exp = expected_of(case, got)
+    assert got.size == exp.size, (got.shape, exp.size)
+    tol = case["tolerance"]
+    if tol == 0.0 and got.dtype.kind != "f":
+        assert np.array_equal(got.reshape(-1), exp)
+    else:
+        np.testing.assert_allclose(got.reshape(-1), exp, rtol=1e-6, atol=max(tol, 1e-6),
+                                   equal_nan=True)
+
+
+@pytest.mark.parametrize("rule", CASES["slice_shape_rules"], ids=lambda r: r["test"])
+def test_slice_shape_rules(rule):
+    """backend/slice.rs:497-677: output-shape rules of compute_output_shape_helper."""
+    if not rule["expect_error"] and rule["expected_shape"] is None:
+        ops.slice_resolve(rule["shape"], rule["starts"], rule["ends"], rule["axes"], rule["steps"])
+        return  # the reference only requires that this does not fail
+    if rule["expect_error"]:
+        with pytest.raises(Exception):
+            res = ops.slice_resolve(rule["shape"], rule["starts"], rule["ends"], rule["axes"],
+                                    rule["steps"])
+            if len(set(a % len(rule["shape"]) for a in rule["axes"])) != len(rule["axes"]):
+                raise ops.OracleError("duplicate axes")
+        return
+    res = ops.slice_resolve(rule["shape"], rule["starts"], rule["ends"], rule["axes"], rule["steps"])
+    assert [r[2] for r in res] == rule["expected_shape"]
+    x = np.arange(int(np.prod(rule["shape"]))).reshape(rule["shape"])
+    out_shape, flat = loops.slice_loop(rule["shape"], rule["starts"], rule["ends"], rule["axes"],
+                                       rule["steps"], x.reshape(-1))
+    assert out_shape == rule["expected_shape"]
+    assert np.array_equal(np.array(flat, dtype=x.dtype).reshape(out_shape),
+                          ops.slice_(x, rule["starts"], rule["ends"], rule["axes"], rule["steps"]))
+
+
+@pytest.mark.parametrize("case", CASES["kernel_cases"]["reduce_mean"], ids=lambda c: c["test"])
+def test_reduce_mean_kernel_vectors(case):
+    """cuda/src/kernels/reduce_mean.rs:156-266"""
+    x = decode(case["data"], np.float32).reshape(case["shape"])
+    got = ops.reduce_mean(x, case["axes"], keepdims=1)
+    assert list(got.shape) == case["out_shape"]
+    np.testing.assert_allclose(got.reshape(-1), decode(case["expected"], np.float32), rtol=1e-6)
+    lp = loops.reduce_mean_loop(case["shape"], case["axes"], x.reshape(-1))
+    np.testing.assert_allclose(np.array(lp, dtype=np.float32), got.reshape(-1), rtol=1e-7)
+
+
+def load_f32(name):
+    return np.fromfile(os.path.join(HERE, "golden", name), dtype="<f4")
+
+
+def attention_graph():
+    """runtime/tests/graphs/attention.rs:15-41"""
+    nodes = [
+        _Node("Transpose", ["k"], ["kt"], {"perm": [0, 2, 1]}),
+        _Node("MatMul", ["q", "kt"], ["scores"], {}),
+        _Node("Div", ["scores", "scale"], ["scaled"], {}),
+        _Node("Trilu", ["scaled"], ["masked"], {"upper": 0}),
+        _Node("Softmax", ["masked"], ["probs"], {"axis": -1}),
+        _Node("MatMul", ["probs", "v"], ["out"], {}),
+    ]
+    return _Graph(nodes, {"scale": np.array(2.0, dtype=np.float32)}, ["out"])
+
+
+def test_attention_fixture_from_onnxruntime():
+    """The one ONNX-Runtime-CPU-generated golden in the reference tree (tolerance 1e-5,
+    runtime/tests/graphs/attention.rs:53-55). Pins Transpose + MatMul + Div(scalar) +
+    Trilu(lower, zero fill) + Softmax + MatMul together."""
+    q, k, v = (load_f32(f"attention_{n}.f32").reshape(1, 2, 4) for n in "qkv")
+    exp = load_f32("attention_out.f32")
+    assert exp.size == 8
+    out = ograph.run_graph(attention_graph(), {"q": q, "k": k, "v": v})["out"]
+    np.testing.assert_allclose(out.reshape(-1), exp, rtol=0, atol=1e-5)
+    # the f32-accumulate variant used for CPU timing must agree as well
+    out32 = ograph.run_graph(attention_graph(), {"q": q, "k": k, "v": v}, "f32")["out"]
+    np.testing.assert_allclose(out32.reshape(-1), exp, rtol=0, atol=1e-5)
+
+
+# ---- loop restatement vs numpy restatement ------------------------------------------------------
+@pytest.mark.parametrize("sa,sb", [((2, 4, 1), (4, 3)), ((2, 4, 3), (3,)), ((3, 1, 2), (1, 5, 1)),
+                                   ((1,), (2, 2)), ((2, 3), (2, 3))])
+def test_binary_loop_vs_numpy(sa, sb):
+    rng = np.random.default_rng(1)
+    a = rng.integers(-9, 9, size=sa).astype(np.int64)
+    b = rng.integers(1, 9, size=sb).astype(np.int64)
+    out_shape = loops.compute_broadcast_output_shape(list(sa), list(sb))
+    assert out_shape == list(np.broadcast_shapes(sa, sb))
+    ast = loops.compute_broadcast_stride(list(sa), out_shape)
+    bst = loops.compute_broadcast_stride(list(sb), out_shape)
+    for fn, ref in [(lambda x, y: x + y, ops.add), (lambda x, y: x - y, ops.sub),
+                    (lambda x, y: x * y, ops.mul), (lambda x, y: x > y, ops.greater),
+                    (lambda x, y: x == y, ops.equal),
+                    (lambda x, y: int(abs(x) // abs(y)) * (1 if (x >= 0) == (y >= 0) else -1), ops.div)]:
+        got = loops.binary_loop(fn, out_shape, ast, bst, a.reshape(-1), b.reshape(-1))
+        assert np.array_equal(np.array(got).reshape(out_shape), ref(a, b))
+    assert loops.compute_broadcast_output_shape([2, 3], [4, 3]) is None
+
+
+def test_where_loop_vs_numpy():
+    rng = np.random.default_rng(2)
+    c = rng.random((3, 1)) < 0.5
+    x = rng.integers(0, 9, size=(1, 4))
+    y = rng.integers(0, 9, size=(3, 4))
+    shp = [3, 4]
+    got = loops.ternary_loop(shp, loops.compute_broadcast_stride([1, 4], shp),
+                             loops.compute_broadcast_stride([3, 4], shp),
+                             loops.compute_broadcast_stride([3, 1], shp), x.reshape(-1),
+                             y.reshape(-1), c.reshape(-1))
+    assert np.array_equal(np.array(got).reshape(shp), ops.where(c, x, y))
+
+
+def test_movement_loops_vs_numpy():
+    x = np.arange(2 * 3 * 4 * 5).reshape(2, 3, 4, 5)
+    for perm in ([0, 2, 1, 3], [3, 2, 1, 0], [1, 0, 3, 2], [0, 1, 3, 2]):
+        got = loops.transpose_loop(list(x.shape), perm, x.reshape(-1))
+        assert np.array_equal(np.array(got).reshape([x.shape[p] for p in perm]),
+                              ops.transpose(x, perm))
+    e = np.arange(6).reshape(1, 3, 1, 2)
+    got = loops.expand_loop([1, 3, 1, 2], [4, 3, 5, 2], e.reshape(-1))
+    assert np.array_equal(np.array(got).reshape(4, 3, 5, 2), ops.expand(e, [4, 3, 5, 2]))
+    got = loops.gather_loop([2, 3, 4], 1, [2, -3, 1], x[:, :3, :4, 0].reshape(-1))
+    assert np.array_equal(np.array(got).reshape(2, 3, 4),
+                          ops.gather(x[:, :3, :4, 0], np.array([2, -3, 1]), 1))
+    parts = [x[:, :, :1], x[:, :, 1:1], x[:, :, 1:]]
+    got = loops.concat_loop([list(p.shape) for p in parts], 2, [p.reshape(-1) for p in parts])
+    assert np.array_equal(np.array(got).reshape(x.shape), ops.concat(parts, 2))
+    for upper in (0, 1):
+        for k in (-2, 0, 1, 7):
+            m = np.arange(1, 2 * 4 * 5 + 1).reshape(2, 4, 5)
+            got = loops.trilu_loop(2, 4, 5, upper, k, m.reshape(-1))
+            assert np.array_equal(np.array(got).reshape(2, 4, 5), ops.trilu(m, k, upper))
+
+
+def test_scatter_loop_vs_numpy_and_onnx_examples():
+    data = np.array([1, 2, 3, 4, 5, 6, 7, 8], dtype=np.float32)
+    idx = np.array([[4], [3], [1], [7]], dtype=np.int64)
+    upd = np.array([9, 10, 11, 12], dtype=np.float32)
+    exp = np.array([1, 11, 3, 10, 9, 6, 7, 12], dtype=np.float32)  # ONNX ScatterND example 1
+    assert np.array_equal(ops.scatter_nd(data, idx, upd), exp)
+    got, err = loops.scatter_nd_loop([8], [4, 1], idx.reshape(-1), upd, data)
+    assert err == 0 and np.array_equal(np.array(got, dtype=np.float32), exp)
+    _, err = loops.scatter_nd_loop([8], [1, 1], [8], [0.0], data)
+    assert err == 1
+    with pytest.raises(ops.OracleError):
+        ops.scatter_nd(data, np.array([[8]]), np.array([0.0], dtype=np.float32))
+    d3 = np.arange(4 * 4 * 4, dtype=np.float32).reshape(4, 4, 4)
+    i3 = np.array([[0], [2]], dtype=np.int64)
+    u3 = -np.ones((2, 4, 4), dtype=np.float32)
+    for red in ("none", "add", "mul", "max", "min"):
+        got, err = loops.scatter_nd_loop([4, 4, 4], [2, 1], i3.reshape(-1), u3.reshape(-1),
+                                         d3.reshape(-1), red)
+        assert err == 0
+        assert np.array_equal(np.array(got, dtype=np.float32).reshape(4, 4, 4),
+                              ops.scatter_nd(d3, i3, u3, red))
+
+
+def test_matmul_and_softmax_closed_forms():
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal((3, 5)).astype(np.float32)
+    b = rng.standard_normal((5, 4)).astype(np.float32)
+    np.testing.assert_allclose(ops.matmul(a, b), loops.matmul_loop(a.reshape(-1), b.reshape(-1), 3, 5, 4),
+                               rtol=1e-6)
+    # batched 4-D of constants: every element is k * 1 * 13 (backend/matmul.rs d4_shape_and_values)
+    out = ops.matmul(np.ones((1, 24, 6, 6), np.float32), np.full((1, 24, 6, 128), 13.0, np.float32))
+    assert out.shape == (1, 24, 6, 128) and np.all(out == 78.0)
+    x = rng.standard_normal((4, 7)).astype(np.float32)
+    np.testing.assert_allclose(ops.softmax(x).reshape(-1), loops.softmax_loop(4, 7, x.reshape(-1)),
+                               rtol=1e-6)
+    # uniform row -> 1/n; shift invariance; -10000 mask -> exact 0 (backend/softmax.rs:259-275)
+    np.testing.assert_allclose(ops.softmax(np.full((2, 8), 3.0, np.float32)), 1 / 8, rtol=1e-7)
+    np.testing.assert_allclose(ops.softmax(x + 100.0), ops.softmax(x), rtol=2e-5)
+    m = ops.softmax(np.array([[0.0, -10000.0, 0.5]], dtype=np.float32))
+    assert m[0, 1] == 0.0 and abs(m.sum() - 1.0) < 1e-6
+    # 4096-wide row with its own closed form (backend/softmax.rs:299-313): geometric weights
+    n = 4096
+    row = (np.arange(n, dtype=np.float32) % 2)
+    s = ops.softmax(row[None])[0]
+    e = np.exp(1.0)
+    np.testing.assert_allclose(s[1] / s[0], e, rtol=1e-6)
+    np.testing.assert_allclose(s.sum(), 1.0, rtol=1e-6)
+
+
+def test_pow_and_cast_and_intdiv_semantics():
+    x = np.array([1.5, -2.0, 0.0, 3.0], dtype=np.float32)
+    assert np.array_equal(ops.pow_(x, np.float32(2.0)), x * x)
+    assert np.array_equal(ops.pow_(np.abs(x), np.float32(0.5)), np.sqrt(np.abs(x)))
+    assert np.array_equal(ops.pow_(np.array([2, -3, 5], dtype=np.int64), np.array([10, 3, 0])),
+                          np.array([1024, -27, 1]))
+    # llround: half away from zero (2^-1 = 0.5 -> 1)
+    assert ops.pow_(np.array([2], dtype=np.int32), np.array([-1], dtype=np.int32))[0] == 1
+    assert np.array_equal(ops.cast(np.array([2.9, -2.9, 0.4], dtype=np.float32), 6), [2, -2, 0])
+    assert np.array_equal(ops.cast(np.array([0.0, -0.0, 1e-9, np.nan], dtype=np.float32), 9),
+                          [False, False, True, True])
+    assert np.array_equal(ops.cast(np.array([True, False]), 1), np.array([1.0, 0.0], np.float32))
+    assert np.array_equal(ops.div(np.array([7, -7, 7, -7], dtype=np.int32),
+                                  np.array([2, 2, -2, -2], dtype=np.int32)), [3, -3, -3, 3])
+    assert np.array_equal(ops.range_(np.int64(2), np.int64(11), np.int64(3)), [2, 5, 8])
+    assert np.array_equal(ops.range_(np.int64(10), np.int64(1), np.int64(-4)), [10, 6, 2])
+    assert ops.range_(np.float32(0), np.float32(1), np.float32(0.25)).tolist() == [0, 0.25, 0.5, 0.75]
+    assert np.array_equal(ops.reduce_mean(np.full((3, 4), 2.5, np.float32), [1]), np.full((3, 1), 2.5))
