@@ -1,0 +1,320 @@
+#!/usr/bin/env python3
+"""Benchmark of the operator path on one MI355X.
+
+Default workload (BASELINE.json configs[3], the configuration the headline metric is quoted on):
+the full Llama-3.2-1B-shaped fp32 graph (16 layers, hidden 2048, 32/8 heads of 64, FFN 8192,
+vocab 128256, random-init weights ~ N(0, 0.02), synthetic token ids), fixed-length KV caches
+updated by ScatterND. One "step" is one prefill pass over a 512-token prompt; after the timed
+prefill steps, 128 greedy decode steps are timed as well (a decode step is one replay of the
+recorded HIP graph plus the host argmax over the logits).
+
+Prints ONE JSON line: value = prefill tokens/s (inputs resident in HBM, K steps timed between
+stream synchronisations), plus decode ms/token, the roofline of the dominant kernel (fp32 MFMA
+GEMM) measured with HIP events, and the CPU oracle timed on the host cores on a bounded sample.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--prompt 512] [--decode 128]
+    python bench.py --suite ops        # per-kernel launches of the op microbench shapes (for rocprofv3)
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def cpu_baseline(graph, cfg, graphs, n_tokens, max_len, seed):
+    """The numpy oracle (fp32 BLAS matmuls) on the host: prefill of the first n_tokens of the same
+    prompt through the same graph."""
+    import numpy as np
+    from oracle import graph as og
+    rng = np.random.default_rng(seed)
+    prompt = rng.integers(0, cfg.vocab, size=512)[:n_tokens]
+    feeds = {"input_ids": prompt.reshape(1, -1).astype(np.int64),
+             "position_ids": np.arange(n_tokens, dtype=np.int64).reshape(1, -1)}
+    for l in range(cfg.layers):
+        for kv in ("key", "value"):
+            feeds[f"cache.{l}.{kv}"] = np.zeros((1, cfg.kv_heads, max_len, cfg.head_dim), np.float32)
+    t0 = time.perf_counter()
+    out = og.run_graph(graph, feeds, matmul_accumulate="f32")
+    dt = time.perf_counter() - t0
+    return n_tokens / dt, dt, out["logits"][0, -1]
+
+
+def run_llama(args):
+    import numpy as np
+    import torch
+    from rmlk_amd import graphs, kernels, runtime
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    info = kernels.device_info(0)
+    cfg = graphs.LlamaConfig() if not args.tiny else graphs.LlamaConfig.tiny()
+    prompt_len, decode_steps = args.prompt, args.decode
+    max_len = prompt_len + decode_steps
+    t0 = time.perf_counter()
+    graph = graphs.llama_graph(cfg, seed=4, style="scatter", max_len=max_len)
+    log(f"[bench] graph built in {time.perf_counter() - t0:.1f}s: {len(graph.nodes)} nodes")
+    t0 = time.perf_counter()
+    inst = runtime.Builder.from_graph(graph).build(0)
+    log(f"[bench] session created (weights uploaded) in {time.perf_counter() - t0:.1f}s")
+
+    rng = np.random.default_rng(4)
+    prompt = rng.integers(0, cfg.vocab, size=prompt_len)
+    caches = {f"cache.{l}.{kv}": np.zeros((1, cfg.kv_heads, max_len, cfg.head_dim), np.float32)
+              for l in range(cfg.layers) for kv in ("key", "value")}
+
+    def feed_prefill():
+        inst.set_input("input_ids", prompt.reshape(1, -1).astype(np.int64))
+        inst.set_input("position_ids", np.arange(prompt_len, dtype=np.int64).reshape(1, -1))
+        for name, arr in caches.items():
+            inst.set_input(name, arr)
+
+    # ---- prefill: warm-up, then K timed steps (replays of the recorded graph) ------------------
+    feed_prefill()
+    inst.execute()                       # first run: fills the buffer pool
+    first_logits = inst.output("logits")[0, -1].copy()
+    inst.capture()
+    for _ in range(args.warmup):
+        inst.replay()
+    inst.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        inst.replay()
+    inst.sync()
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    ms_per_step = prefill_s / args.steps * 1e3
+    tok_s = prompt_len * args.steps / prefill_s
+    replay_logits = inst.output("logits")[0, -1].copy()
+    assert np.array_equal(first_logits, replay_logits), "replayed prefill differs from the eager run"
+    mem = inst.memory_stats()
+    log(f"[bench] prefill {prompt_len} tokens: {ms_per_step:.2f} ms/step, {tok_s:.0f} tok/s")
+
+    # ---- roofline of the MatMul kernels: one extra eager pass with HIP events per node ----------
+    feed_prefill()
+    inst.set_profiling(True)
+    inst.execute()
+    inst.set_profiling(False)
+    stats = inst.node_stats()
+    # classify each MatMul node by the kernel the library picks for its shape
+    shapes = matmul_shapes(cfg, prompt_len, max_len)
+    mm_nodes = [s for s in stats if s["op"] == "MatMul"]
+    assert len(mm_nodes) == len(shapes), (len(mm_nodes), len(shapes))
+    by_kind, per_op = {}, {}
+    for s, (batch, m, n, k) in zip(mm_nodes, shapes):
+        kind = kernels.matmul_describe(batch, m, n, k)
+        d = by_kind.setdefault(kind, {"launches": 0, "us": 0.0, "flops": 0.0})
+        d["launches"] += 1
+        d["us"] += s["micros"]
+        d["flops"] += 2.0 * batch * m * n * k
+    for s in stats:
+        if s["micros"] > 0:
+            d = per_op.setdefault(s["op"], {"n": 0, "us": 0.0, "bytes": 0.0})
+            d["n"] += 1
+            d["us"] += s["micros"]
+            d["bytes"] += s["bytes"]
+    eager_us = sum(d["us"] for d in per_op.values())
+    dom_kind = max(by_kind, key=lambda kd: by_kind[kd]["us"])
+    dom = by_kind[dom_kind]
+    achieved = dom["flops"] / (dom["us"] * 1e-6) / 1e12
+    roofline = {
+        "bound": "mfma", "kernel": f"gemm_mfma_kernel ({dom_kind})",
+        "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+        "launches": dom["launches"], "avg_launch_us": round(dom["us"] / dom["launches"], 2),
+        "flops_per_launch": dom["flops"] / dom["launches"],
+        "measured": "HIP events around every MatMul node of one eager prefill pass after the timed steps",
+    }
+    all_mm_flops = sum(d["flops"] for d in by_kind.values())
+    all_mm_us = sum(d["us"] for d in by_kind.values())
+    matmul_all = {"tflops": round(all_mm_flops / (all_mm_us * 1e-6) / 1e12, 2),
+                  "frac_of_fp32_mfma_peak": round(all_mm_flops / (all_mm_us * 1e-6) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                  "share_of_prefill_time": round(all_mm_us / eager_us, 3),
+                  "by_kernel": {k_: {"launches": v["launches"], "us": round(v["us"], 1),
+                                     "tflops": round(v["flops"] / (v["us"] * 1e-6) / 1e12, 2)}
+                                for k_, v in by_kind.items()}}
+    op_breakdown = {op: {"n": d["n"], "us": round(d["us"], 1),
+                         "gbs": round(d["bytes"] / (d["us"] * 1e-6) / 1e9, 1) if d["us"] > 0 else 0}
+                    for op, d in sorted(per_op.items(), key=lambda kv: -kv[1]["us"])}
+
+    # ---- decode: recorded HIP graph of one step, replayed decode_steps times -------------------
+    decode_ms, tokens = None, []
+    if decode_steps > 0:
+        for l in range(cfg.layers):
+            for kv in ("key", "value"):
+                inst.feed_output(f"cache_out.{l}.{kv}", f"cache.{l}.{kv}")
+        tok = int(np.argmax(first_logits))
+        pos = prompt_len
+        inst.set_input("input_ids", np.array([[tok]], dtype=np.int64))
+        inst.set_input("position_ids", np.array([[pos]], dtype=np.int64))
+        inst.capture()
+        logits_buf = np.empty((1, 1, cfg.vocab), dtype=np.float32)
+        inst.sync()
+        t0 = time.perf_counter()
+        for _ in range(decode_steps):
+            inst.set_input("input_ids", np.array([[tok]], dtype=np.int64))
+            inst.set_input("position_ids", np.array([[pos]], dtype=np.int64))
+            inst.replay()
+            tok = int(np.argmax(inst.output("logits")))
+            tokens.append(tok)
+            pos += 1
+        inst.sync()
+        decode_ms = (time.perf_counter() - t0) / decode_steps * 1e3
+        # device-only time of a step: replays without the host round trip
+        inst.sync()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            inst.replay()
+        inst.sync()
+        decode_dev_ms = (time.perf_counter() - t0) / 20 * 1e3
+        weight_bytes = decode_weight_bytes(cfg)
+        log(f"[bench] decode: {decode_ms:.3f} ms/token end to end, {decode_dev_ms:.3f} ms/token "
+            f"device replay ({weight_bytes / decode_dev_ms / 1e6:.0f} GB/s of weights)")
+    else:
+        decode_dev_ms, weight_bytes = None, decode_weight_bytes(cfg)
+
+    # ---- CPU baseline: the oracle on a bounded sample -------------------------------------------
+    cpu = None
+    if not args.no_cpu:
+        n_cpu = min(args.cpu_tokens, prompt_len)
+        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        cpu_tok_s, cpu_s, cpu_logits = cpu_baseline(graph, cfg, graphs, n_cpu, max_len, 4)
+        cpu = {"value": round(cpu_tok_s, 2), "unit": "tok/s", "cores": cores,
+               "kind": "port",
+               "sample": f"prefill of the first {n_cpu} prompt tokens through the same graph with the "
+                         f"numpy oracle (fp32 BLAS matmuls), {cpu_s:.1f} s; ONNX Runtime is not installed"}
+        log(f"[bench] cpu oracle: {cpu_tok_s:.1f} tok/s over {n_cpu} tokens ({cpu_s:.1f}s)")
+
+    result = {
+        "metric": "llama3.2-1b-shape fp32 prefill tok/s (decode ms/tok alongside)",
+        "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[3]: full Llama-3.2-1B-shaped ONNX-op graph, fp32, "
+                               f"prefill {prompt_len} tokens + {decode_steps} greedy decode steps, batch 1, "
+                               "KV cache updated by ScatterND, random-init weights N(0,0.02)",
+                   "layers": cfg.layers, "hidden": cfg.hidden, "vocab": cfg.vocab,
+                   "prompt_tokens": prompt_len, "graph_nodes": len(graph.nodes),
+                   "execution": "recorded HIP graph replay per step"},
+        "decode_ms_per_token": None if decode_ms is None else round(decode_ms, 4),
+        "decode_device_ms_per_token": None if decode_dev_ms is None else round(decode_dev_ms, 4),
+        "decode_weight_gbs": None if decode_dev_ms is None else round(weight_bytes / decode_dev_ms / 1e6, 1),
+        "decode_frac_of_hbm_peak": None if decode_dev_ms is None else round(weight_bytes / decode_dev_ms / 1e6 / PEAK_HBM_GBS, 4),
+        "roofline": roofline, "matmul_all": matmul_all, "ops": op_breakdown,
+        "cpu_baseline": cpu,
+        "memory": mem, "device": info["name"], "arch": info["arch"],
+    }
+    inst.close()
+    return result
+
+
+def decode_weight_bytes(cfg):
+    """Weights streamed once per decoded token (fp32): per layer q,o,k,v,gate,up,down + lm-head."""
+    kvd = cfg.kv_heads * cfg.head_dim
+    per_layer = (2 * cfg.hidden * cfg.heads * cfg.head_dim + 2 * cfg.hidden * kvd +
+                 3 * cfg.hidden * cfg.ffn)
+    return 4.0 * (cfg.layers * per_layer + cfg.hidden * cfg.vocab)
+
+
+def matmul_shapes(cfg, s, max_len):
+    """(batch, m, n, k) of every MatMul node of the scatter-style graph in node order."""
+    h, kvd, d = cfg.hidden, cfg.kv_heads * cfg.head_dim, cfg.head_dim
+    out = []
+    for _ in range(cfg.layers):
+        out += [(1, s, cfg.heads * d, h), (1, s, kvd, h), (1, s, kvd, h),
+                (cfg.heads, s, max_len, d), (cfg.heads, s, d, max_len),
+                (1, s, h, cfg.heads * d), (1, s, cfg.ffn, h), (1, s, cfg.ffn, h), (1, s, h, cfg.ffn)]
+    out.append((1, s, cfg.vocab, h))
+    return out
+
+
+def run_ops_suite(args):
+    """BASELINE configs[1]: each op of the microbench launched repeatedly over rotating buffer sets
+    (working set above the 256 MB Infinity Cache), for `rocprofv3 --kernel-trace --stats`."""
+    import numpy as np
+    import torch
+    from rmlk_amd import kernels as k
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(2)
+    ns = 6
+    shp, n = [8, 32, 512, 64], 8 * 32 * 512 * 64
+    xs = [torch.randn(n, device=dev, generator=g) for _ in range(ns)]
+    ys = [torch.empty(n, device=dev) for _ in range(ns)]
+    bs = [torch.randn(32 * 64, device=dev, generator=g) for _ in range(ns)]
+    conds = [(torch.rand(n, device=dev, generator=g) < 0.5) for _ in range(ns)]
+    dense, bst = [1048576, 32768, 64, 1], [0, 64, 0, 1]
+    reps = args.steps * 10
+    results = {}
+
+    def timed(name, fn, nset, bytes_):
+        for i in range(3):
+            fn(i % nset)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(reps):
+            fn(i % nset)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / reps * 1e3
+        results[name] = {"us_per_launch_incl_launch_gaps": round(us, 2), "algorithmic_bytes": bytes_}
+
+    timed("add", lambda i: k.binary(k.ADD, xs[i], bs[i], ys[i], shp, dense, bst), ns, 2 * n * 4 + 8192)
+    timed("mul", lambda i: k.binary(k.MUL, xs[i], bs[i], ys[i], shp, dense, bst), ns, 2 * n * 4 + 8192)
+    timed("div", lambda i: k.binary(k.DIV, xs[i], bs[i], ys[i], shp, dense, bst), ns, 2 * n * 4 + 8192)
+    timed("where", lambda i: k.where(xs[i], bs[i], conds[i], ys[i], shp, dense, bst, dense), ns,
+          2 * n * 4 + n + 8192)
+    rm_out = torch.empty(4096, device=dev)
+    timed("reduce_mean", lambda i: k.reduce_mean(xs[i], rm_out, [4096, 2048], [1]), ns, n * 4 + 16384)
+    timed("transpose", lambda i: k.transpose(xs[i], ys[i], [1, 2048, 32, 64], [0, 2, 1, 3]), ns,
+          2 * 2048 * 32 * 64 * 4)
+    table = torch.randn(128256, 2048, device=dev, generator=g)
+    idx = [torch.randint(0, 128256, (2048,), device=dev, generator=g) for _ in range(ns)]
+    timed("gather", lambda i: k.gather(table, idx[i], ys[i], [128256, 2048], 0), ns,
+          2 * 2048 * 2048 * 4 + 2048 * 8)
+    del table
+    sx = [torch.randn(32 * 2048, 2048, device=dev, generator=g) for _ in range(2)]
+    mask = torch.triu(torch.full((2048, 2048), float("-inf"), device=dev), 1)
+    for t in sx:
+        t.view(32, 2048, 2048).add_(mask)
+    so = [torch.empty_like(sx[0]) for _ in range(2)]
+    timed("softmax", lambda i: k.softmax(sx[i], so[i], 65536, 2048, 1), 2, 2 * sx[0].numel() * 4)
+    print(json.dumps({"suite": "ops", "note": "per-kernel durations come from rocprofv3 of this command",
+                      "results": results}))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--decode", type=int, default=128)
+    ap.add_argument("--cpu-tokens", type=int, default=64)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--tiny", action="store_true", help="2-layer toy shape (plumbing check only)")
+    ap.add_argument("--suite", default="llama", choices=["llama", "ops"])
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one MI355X: the operator path has no multi-GPU part "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if args.suite == "ops":
+        run_ops_suite(args)
+        return
+    print(json.dumps(run_llama(args)))
+
+
+if __name__ == "__main__":
+    main()

@@ -153,6 +153,12 @@ int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t batch, int6
 size_t rmlk_hip_matmul_workspace_size(int32_t dtype, int64_t batch, int64_t m, int64_t n,
                                       int64_t k);
 
+/* Which kernel rmlk_hip_matmul picks for a row-major problem of this size, as text
+ * ("mfma128x128 splitk=1", "mfma64x64 splitk=8", "gemv splitk=32"); for profiles and reports.
+ * Writes at most `size` bytes including the terminator; returns the length needed. */
+int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_t m, int64_t n, int64_t k,
+                                 char *buf, int32_t size);
+
 /* Transpose: out = permute(in, perm); out.shape[d] = in_shape[perm[d]]. Any 1/2/4/8-byte dtype.
  * ref: cuda/src/kernels/transpose.rs:38-80, cuda/src/ptx/headers/transpose_op_macros.cuh:1-25. */
 int32_t rmlk_hip_transpose(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *in_shape,

@@ -69,6 +69,8 @@ SIGNATURES = {
                                   c_int64, c_int64, c_int32, c_void_p, c_int64, c_int64, c_int32,
                                   c_void_p, c_int64, c_int64, c_void_p, c_size_t]),
     "rmlk_hip_matmul_workspace_size": (c_size_t, [c_int32, c_int64, c_int64, c_int64, c_int64]),
+    "rmlk_hip_matmul_describe": (c_int32, [c_int32, c_int64, c_int64, c_int64, c_int64, c_char_p,
+                                           c_int32]),
     "rmlk_hip_transpose": (c_int32, [c_void_p, c_int32, _PD, POINTER(c_int64), c_void_p,
                                      c_void_p]),
     "rmlk_hip_expand": (c_int32, [c_void_p, c_int32, _PD, _PD, c_void_p, c_void_p]),

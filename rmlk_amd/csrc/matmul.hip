@@ -14,6 +14,9 @@
 //     128-bit LDS read of A serves four MFMAs and the sum over K is unchanged;
 //   - split-K (grid z) writes partial tiles to the workspace, a second kernel adds them in a
 //     fixed order, so results do not depend on scheduling.
+#include <cstdio>
+#include <cstring>
+
 #include "common.hpp"
 
 namespace rmlk {
@@ -468,6 +471,28 @@ extern "C" size_t rmlk_hip_matmul_workspace_size(int32_t dtype, int64_t batch, i
     }
     TileChoice t = choose_tiles(batch, m, n, k);
     return t.splits > 1 ? static_cast<size_t>(t.splits) * batch * m * n * sizeof(float) : 0;
+}
+
+extern "C" int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_t m, int64_t n,
+                                            int64_t k, char *buf, int32_t size) {
+    char tmp[64];
+    if (dtype != RMLK_FLOAT || batch <= 0 || m <= 0 || n <= 0 || k <= 0) {
+        snprintf(tmp, sizeof(tmp), "none");
+    } else if (m == 1) {
+        int kps;
+        const bool vec = n % 4 == 0;
+        snprintf(tmp, sizeof(tmp), "gemv%s splitk=%d", vec ? "x4" : "x1",
+                 gemv_splits(batch, n, k, vec ? kWave * 4 : kWave, &kps));
+    } else {
+        TileChoice t = choose_tiles(batch, m, n, k);
+        snprintf(tmp, sizeof(tmp), "mfma%dx%d splitk=%d", t.bm, t.bn, t.splits);
+    }
+    const int32_t len = static_cast<int32_t>(strlen(tmp));
+    if (buf && size > 0) {
+        strncpy(buf, tmp, size - 1);
+        buf[size - 1] = 0;
+    }
+    return len + 1;
 }
 
 extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t m,

@@ -305,6 +305,11 @@ void Session::build(const rmlk_graph &graph, int dev) {
     // (ref: TensorStore::init, providers/cuda/store.rs:95-261)
     for (size_t v = 0; v < g->values.size(); ++v)
         if (g->values[v].is_initializer) values[v] = upload_initializer(g->values[v].init, stream);
+    check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+    // the host copies of large initializers are not needed once they are on the device
+    for (size_t v = 0; v < graph_copy.values.size(); ++v)
+        if (graph_copy.values[v].is_initializer && graph_copy.values[v].init.data.size() > 4096)
+            std::vector<uint8_t>().swap(graph_copy.values[v].init.data);
     for (size_t n = 0; n < g->nodes.size(); ++n) {
         const Node &node = g->nodes[n];
         if (node.op != "Constant") continue;

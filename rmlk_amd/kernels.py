@@ -99,6 +99,12 @@ def matmul_workspace_size(batch: int, m: int, n: int, k: int, dtype: int = FLOAT
     return int(lib().rmlk_hip_matmul_workspace_size(dtype, batch, m, n, k))
 
 
+def matmul_describe(batch: int, m: int, n: int, k: int, dtype: int = FLOAT) -> str:
+    buf = ctypes.create_string_buffer(64)
+    lib().rmlk_hip_matmul_describe(dtype, batch, m, n, k, buf, 64)
+    return buf.value.decode()
+
+
 def matmul(a, b, c, batch, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, trans_a=False,
            trans_b=False, workspace=None) -> None:
     """ref: cuda/src/kernels/gemm.rs:112-136 (compute with a StridedBatchedConfig)."""
