@@ -34,6 +34,7 @@ struct GemmArgs {
     int64_t stride_a, stride_b, stride_c;  // batch strides (elements)
     int32_t k_per_split;                   // K range of one z-slice (multiple of BK)
     int32_t tiles_m, tiles_n;
+    int32_t aligned;                       // rows of A and B start on 16-byte boundaries
 };
 
 constexpr int kThreads = 256;
@@ -71,7 +72,11 @@ __device__ __forceinline__ void tile_coords(const GemmArgs &g, int &tm, int &tn)
     tn = in_group / gsz;
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool ALIGNED>
+// EDGE == false: every tile is full (m % BM == 0, n % BN == 0, the K range of a split is a
+// multiple of BK) and rows are 16-byte aligned, so the main loop has no bounds checks at all.
+// EDGE == true: guarded loads (zero fill) and guarded stores; `aligned` still allows 128-bit
+// loads where a whole vector is in range.
+template <int BM, int BN, int BK, int WM, int WN, bool EDGE>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
     using L = SmemLayout<BM, BN, BK>;
     extern __shared__ __align__(16) float smem[];
@@ -115,41 +120,60 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
 
     v4f a_reg[A_PASSES], b_reg[B_PASSES];
 
+    // per-lane source pointers of the first K step; they advance by BK (A) and BK rows (B)
+    const float *a_src = A + static_cast<int64_t>(m0 + a_row) * g.lda + k_begin + a_vec * 4;
+    const float *b_src = B + static_cast<int64_t>(k_begin + b_row) * g.ldb + n0 + b_vec * 4;
+    const int64_t a_pass_stride = static_cast<int64_t>(A_ROWS_PER_PASS) * g.lda;
+    const int64_t b_pass_stride = static_cast<int64_t>(B_ROWS_PER_PASS) * g.ldb;
+    const int64_t b_step_stride = static_cast<int64_t>(BK) * g.ldb;
+    const bool vec_ok = g.aligned != 0;
+
     auto load_global = [&](int k0) {
+        if constexpr (!EDGE) {
 #pragma unroll
-        for (int p = 0; p < A_PASSES; ++p) {
-            const int r = m0 + a_row + p * A_ROWS_PER_PASS;
-            const int kk = k0 + a_vec * 4;
-            v4f v = {0.f, 0.f, 0.f, 0.f};
-            if (r < g.m) {
-                const float *src = A + static_cast<int64_t>(r) * g.lda + kk;
-                if (ALIGNED && kk + 3 < k_end) {
-                    v = *reinterpret_cast<const v4f *>(src);
-                } else {
+            for (int p = 0; p < A_PASSES; ++p)
+                a_reg[p] = *reinterpret_cast<const v4f *>(a_src + p * a_pass_stride);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (kk + j < k_end) v[j] = src[j];
+            for (int p = 0; p < B_PASSES; ++p)
+                b_reg[p] = *reinterpret_cast<const v4f *>(b_src + p * b_pass_stride);
+        } else {
+#pragma unroll
+            for (int p = 0; p < A_PASSES; ++p) {
+                const int r = m0 + a_row + p * A_ROWS_PER_PASS;
+                const int kk = k0 + a_vec * 4;
+                v4f v = {0.f, 0.f, 0.f, 0.f};
+                if (r < g.m) {
+                    const float *src = a_src + p * a_pass_stride;
+                    if (vec_ok && kk + 3 < k_end) {
+                        v = *reinterpret_cast<const v4f *>(src);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (kk + j < k_end) v[j] = src[j];
+                    }
                 }
+                a_reg[p] = v;
             }
-            a_reg[p] = v;
-        }
 #pragma unroll
-        for (int p = 0; p < B_PASSES; ++p) {
-            const int kk = k0 + b_row + p * B_ROWS_PER_PASS;
-            const int c = n0 + b_vec * 4;
-            v4f v = {0.f, 0.f, 0.f, 0.f};
-            if (kk < k_end) {
-                const float *src = B + static_cast<int64_t>(kk) * g.ldb + c;
-                if (ALIGNED && c + 3 < g.n) {
-                    v = *reinterpret_cast<const v4f *>(src);
-                } else {
+            for (int p = 0; p < B_PASSES; ++p) {
+                const int kk = k0 + b_row + p * B_ROWS_PER_PASS;
+                const int c = n0 + b_vec * 4;
+                v4f v = {0.f, 0.f, 0.f, 0.f};
+                if (kk < k_end) {
+                    const float *src = b_src + p * b_pass_stride;
+                    if (vec_ok && c + 3 < g.n) {
+                        v = *reinterpret_cast<const v4f *>(src);
+                    } else {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (c + j < g.n) v[j] = src[j];
+                        for (int j = 0; j < 4; ++j)
+                            if (c + j < g.n) v[j] = src[j];
+                    }
                 }
+                b_reg[p] = v;
             }
-            b_reg[p] = v;
         }
+        a_src += BK;
+        b_src += b_step_stride;
     };
     auto store_lds = [&](int buf) {
         float *as = As + buf * L::kAFloats;
@@ -179,13 +203,15 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
     }
     __syncthreads();
 
+    const int a_frag = (wm * WM + l32) * L::kAStride + half * 4;
+    const int b_frag = (half * 4) * L::kBStride + wn * WN + l32;
     for (int step = 0; step < n_steps; ++step) {
         const int buf = step & 1;
         const bool more = step + 1 < n_steps;
         if (more) load_global(k_begin + (step + 1) * BK);
 
-        const float *as = As + buf * L::kAFloats + (wm * WM + l32) * L::kAStride + half * 4;
-        const float *bs = Bs + buf * L::kBFloats + (half * 4) * L::kBStride + wn * WN + l32;
+        const float *as = As + buf * L::kAFloats + a_frag;
+        const float *bs = Bs + buf * L::kBFloats + b_frag;
 #pragma unroll
         for (int kc = 0; kc < BK / 8; ++kc) {
             v4f af[TM];
@@ -216,11 +242,12 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const int col = n0 + wn * WN + j * 32 + l32;
-            if (col < g.n) {
+            if (!EDGE || col < g.n) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                    if (row < g.m) C[static_cast<int64_t>(row) * g.ldc + col] = acc[i][j][r];
+                    if (!EDGE || row < g.m)
+                        C[static_cast<int64_t>(row) * g.ldc + col] = acc[i][j][r];
                 }
             }
         }
@@ -385,34 +412,47 @@ __global__ __launch_bounds__(kThreads) void gemm_naive_kernel(const float *__res
 
 struct TileChoice {
     int bm, bn;     // block tile
+    int bk;         // K step
     int splits;     // split-K factor
     int k_per_split;
 };
 
-constexpr int kBK = 16;
+#ifndef RMLK_GEMM_SPLIT_TARGET
+#define RMLK_GEMM_SPLIT_TARGET 2
+#endif
 
 inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k) {
     TileChoice t;
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch; };
-    // big tiles when they alone fill the chip, else small tiles, else split K on top
-    if (tiles(128, 128) >= kNumCU) {
+    // A 64 x 64 wavefront tile (four MFMA accumulators) keeps the matrix pipe busiest, so the
+    // 128 x 128 block (256 x 64 for narrow outputs) is preferred and K is split until the chip is
+    // covered; 64 x 64 blocks remain for small problems. Long K uses the deeper K step.
+    t.splits = 1;
+    if (n <= 64 && tiles(256, 64) >= kNumCU) {
+        t.bm = 256;
+        t.bn = 64;
+    } else if (tiles(128, 128) >= kNumCU) {
+        t.bm = 128;
+        t.bn = 128;
+    } else if (m >= 128 && n >= 128 && k >= 1024 && tiles(128, 128) * 8 >= kNumCU) {
         t.bm = 128;
         t.bn = 128;
     } else {
         t.bm = 64;
         t.bn = 64;
     }
+    t.bk = k >= 256 ? 32 : 16;
     int64_t nt = tiles(t.bm, t.bn);
     int splits = 1;
     if (nt < kNumCU) {
-        splits = static_cast<int>((2 * kNumCU + nt - 1) / nt);
-        int64_t max_splits = k / (4 * kBK);
+        splits = static_cast<int>((RMLK_GEMM_SPLIT_TARGET * kNumCU + nt - 1) / nt);
+        int64_t max_splits = k / (8 * t.bk);
         if (max_splits < 1) max_splits = 1;
         if (splits > max_splits) splits = static_cast<int>(max_splits);
         if (splits > 32) splits = 32;
     }
     int64_t kps = (k + splits - 1) / splits;
-    kps = (kps + kBK - 1) / kBK * kBK;
+    kps = (kps + t.bk - 1) / t.bk * t.bk;
     t.k_per_split = static_cast<int>(kps);
     t.splits = static_cast<int>((k + kps - 1) / kps);
     if (t.splits < 1) t.splits = 1;
@@ -433,10 +473,10 @@ inline int gemv_splits(int64_t batch, int64_t n, int64_t k, int cols_per_block, 
     return static_cast<int>((k + kps - 1) / kps);
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool ALIGNED>
+template <int BM, int BN, int BK, int WM, int WN, bool EDGE>
 int32_t launch_mfma(hipStream_t s, const GemmArgs &g, int64_t batch, int splits) {
     using L = SmemLayout<BM, BN, BK>;
-    auto kern = gemm_mfma_kernel<BM, BN, BK, WM, WN, ALIGNED>;
+    auto kern = gemm_mfma_kernel<BM, BN, BK, WM, WN, EDGE>;
     if (L::kBytes > 64 * 1024) {
         static bool raised = false;  // benign race: same value from every thread
         if (!raised) {
@@ -485,7 +525,7 @@ extern "C" int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_
                  gemv_splits(batch, n, k, vec ? kWave * 4 : kWave, &kps));
     } else {
         TileChoice t = choose_tiles(batch, m, n, k);
-        snprintf(tmp, sizeof(tmp), "mfma%dx%d splitk=%d", t.bm, t.bn, t.splits);
+        snprintf(tmp, sizeof(tmp), "mfma%dx%dx%d splitk=%d", t.bm, t.bn, t.bk, t.splits);
     }
     const int32_t len = static_cast<int32_t>(strlen(tmp));
     if (buf && size > 0) {
@@ -615,14 +655,19 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
     const bool aligned = lda % 4 == 0 && ldb % 4 == 0 && stride_a % 4 == 0 && stride_b % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
                          reinterpret_cast<uintptr_t>(pb) % 16 == 0;
+    g.aligned = aligned ? 1 : 0;
+    const bool full = aligned && m % t.bm == 0 && n % t.bn == 0 && t.k_per_split % t.bk == 0 &&
+                      k % t.k_per_split == 0;
     int32_t st;
-    if (t.bm == 128) {
-        st = aligned ? launch_mfma<128, 128, kBK, 64, 64, true>(s, g, batch, t.splits)
-                     : launch_mfma<128, 128, kBK, 64, 64, false>(s, g, batch, t.splits);
-    } else {
-        st = aligned ? launch_mfma<64, 64, kBK, 32, 32, true>(s, g, batch, t.splits)
-                     : launch_mfma<64, 64, kBK, 32, 32, false>(s, g, batch, t.splits);
-    }
+#define RMLK_LAUNCH(BM_, BN_, WM_, WN_)                                                        \
+    (t.bk == 32 ? (full ? launch_mfma<BM_, BN_, 32, WM_, WN_, false>(s, g, batch, t.splits)     \
+                        : launch_mfma<BM_, BN_, 32, WM_, WN_, true>(s, g, batch, t.splits))     \
+                : (full ? launch_mfma<BM_, BN_, 16, WM_, WN_, false>(s, g, batch, t.splits)     \
+                        : launch_mfma<BM_, BN_, 16, WM_, WN_, true>(s, g, batch, t.splits)))
+    if (t.bm == 256) st = RMLK_LAUNCH(256, 64, 64, 64);
+    else if (t.bm == 128) st = RMLK_LAUNCH(128, 128, 64, 64);
+    else st = RMLK_LAUNCH(64, 64, 32, 32);
+#undef RMLK_LAUNCH
     if (st) return st;
     if (t.splits > 1) {
         unsigned rg = grid_for(batch * m * n, kThreads, 8);

@@ -307,6 +307,13 @@ MATMUL_CASES = [
     (1, 128, 2048, 256), (3, 96, 80, 40), (2, 256, 256, 128), (1, 512, 384, 2048),
     (4, 1, 64, 300), (1, 1, 2048, 2048), (2, 1, 130, 77), (1, 1, 1, 5), (1, 300, 1, 64),
     (1, 257, 129, 19),
+    (1, 512, 2048, 2048),     # 128 x 128 tiles with split-K
+    (1, 128, 1024, 2048),     # small M, split-K
+    (32, 512, 64, 640),       # narrow output, 64 x 64 tiles
+    (32, 2048, 64, 256),      # narrow output, 256 x 64 tiles
+    (3, 300, 64, 100),        # narrow output with edges
+    (1, 2048, 2048, 64),      # short K (K step 16)
+    (8, 256, 256, 250),       # K not a multiple of the K step, batched
 ]
 
 
