@@ -143,7 +143,8 @@ int32_t rmlk_hip_softmax(rmlk_stream_t stream, int32_t dtype, int64_t outer, int
  * matrix over the batch (the reference copies the operand `batch` times instead,
  * ref: runtime/src/providers/cuda/backend/matmul.rs:48-86). fp32 in, fp32 accumulate. dtype FLOAT.
  * `workspace` is device scratch of at least rmlk_hip_matmul_workspace_size(...) bytes (may be NULL
- * when that is 0); it is only written and read inside the call's own stream order.
+ * when that is 0); it is only written and read inside the call's own stream order
+ * (calls that share one workspace must not overlap in time); its contents on entry do not matter.
  * ref: cuda/src/kernels/gemm.rs:112-136,191-232 (cublasGemmStridedBatchedEx). */
 int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t m, int64_t n,
                         int64_t k, const void *a, int64_t lda, int64_t stride_a, int32_t trans_a,

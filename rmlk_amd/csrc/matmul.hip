@@ -285,6 +285,8 @@ struct GemvArgs {
     int32_t k_per_split;
 };
 
+
+
 template <int VEC>
 __global__ __launch_bounds__(kThreads) void gemv_kernel(GemvArgs g) {
     constexpr int kWaves = kThreads / kWave;
@@ -356,6 +358,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(GemvArgs g) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) red[wave][lane * VEC + j] = acc[j];
     __syncthreads();
+    // one split: y itself; several: this split's slab of the workspace [split][batch][n]
     float *y = g.y + (static_cast<int64_t>(split) * gridDim.y + batch) * g.stride_y;
     for (int c = threadIdx.x; c < kCols; c += kThreads) {
         const int oc = blockIdx.x * kCols + c;
@@ -365,6 +368,27 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(GemvArgs g) {
             for (int wv = 0; wv < kWaves; ++wv) s += red[wv][c];
             y[oc] = s;
         }
+    }
+}
+
+// Combine GEMV partials [split][total] -> y: 64 outputs per block, 4 lanes per output take the
+// splits round-robin, then the four sums meet in LDS in a fixed order.
+__global__ __launch_bounds__(kThreads) void gemv_reduce_kernel(const float *__restrict__ ws,
+                                                               float *__restrict__ y, int splits,
+                                                               int64_t batch, int32_t n,
+                                                               int64_t stride_y) {
+    __shared__ float part[4][64];
+    const int64_t total = batch * n;
+    const int ox = threadIdx.x % 64, sy = threadIdx.x / 64;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 64 + ox;
+    float s = 0.f;
+    if (i < total)
+        for (int z = sy; z < splits; z += 4) s += ws[z * total + i];
+    part[sy][ox] = s;
+    __syncthreads();
+    if (sy == 0 && i < total) {
+        const int64_t b = i / n, col = i - b * n;
+        y[b * stride_y + col] = (part[0][ox] + part[1][ox]) + (part[2][ox] + part[3][ox]);
     }
 }
 
@@ -510,7 +534,8 @@ extern "C" size_t rmlk_hip_matmul_workspace_size(int32_t dtype, int64_t batch, i
         return sp > 1 ? static_cast<size_t>(sp) * batch * n * sizeof(float) : 0;
     }
     TileChoice t = choose_tiles(batch, m, n, k);
-    return t.splits > 1 ? static_cast<size_t>(t.splits) * batch * m * n * sizeof(float) : 0;
+    return t.splits > 1 ? static_cast<size_t>(t.splits) * batch * m * n * sizeof(float)
+                        : 0;
 }
 
 extern "C" int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_t m, int64_t n,
@@ -609,9 +634,9 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
         int32_t st = launch_status();
         if (st) return st;
         if (splits > 1) {
-            unsigned rg = grid_for(batch * n, kThreads, 8);
-            splitk_reduce_kernel<<<rg, kThreads, 0, s>>>(static_cast<const float *>(workspace), pc,
-                                                         splits, batch, 1, g.n, ldc, stride_c);
+            const int64_t total = batch * n;
+            gemv_reduce_kernel<<<static_cast<unsigned>((total + 63) / 64), kThreads, 0, s>>>(
+                static_cast<const float *>(workspace), pc, splits, batch, g.n, stride_c);
             return launch_status();
         }
         return RMLK_OK;
@@ -671,8 +696,8 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
     if (st) return st;
     if (t.splits > 1) {
         unsigned rg = grid_for(batch * m * n, kThreads, 8);
-        splitk_reduce_kernel<<<rg, kThreads, 0, s>>>(static_cast<const float *>(workspace), pc,
-                                                     t.splits, batch, g.m, g.n, ldc, stride_c);
+        splitk_reduce_kernel<<<rg, kThreads, 0, s>>>(g.c, pc, t.splits, batch, g.m, g.n, ldc,
+                                                     stride_c);
         return launch_status();
     }
     return RMLK_OK;

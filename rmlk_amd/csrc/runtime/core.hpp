@@ -189,7 +189,8 @@ struct OpContext {
     // blocking device-to-host copy (counted in the session's sync statistics).
     HostVal host_values(int i) const;
     int32_t *error_flag() const;
-    void *scratch(size_t bytes) const;  // per-run device scratch (MatMul split-K partials)
+    // The session's MatMul workspace (split-K partials): one persistent buffer, grown on demand.
+    void *scratch(size_t bytes) const;
 };
 
 using OpFn = void (*)(OpContext &);
@@ -211,11 +212,14 @@ struct Session {
     std::vector<Tensor> values;      // by value id
     std::vector<int> last_use;       // node index of the last consumer, -1 = never read
     std::vector<BufferRef> scratch_bufs;
+    void *workspace = nullptr;       // persistent MatMul workspace (raw allocation)
+    size_t workspace_bytes = 0;
     int32_t *err_flag = nullptr;     // device
     int32_t *err_host = nullptr;     // pinned host
     bool capturing = false;
     bool profiling = false;
-    int64_t device_syncs = 0;
+    int64_t device_syncs = 0;            // blocking reads of shape-like tensors
+    int64_t device_syncs_workspace = 0;  // stream syncs taken to grow the MatMul workspace
     std::unique_ptr<CapturedPlan> plan;
     struct NodeStat {
         double micros = -1.0, bytes = 0.0, flops = 0.0;

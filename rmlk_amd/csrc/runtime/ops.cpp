@@ -398,11 +398,20 @@ void op_transpose(OpContext &c) {
         perm[d] = normalize_axis(perm[d], x.rank(), "Transpose perm");
         out_shape[d] = x.shape[perm[d]];
     }
-    Tensor &y = c.alloc_output(0, x.dtype, out_shape);
-    if (x.rank() == 0) {
-        check_status(rmlk_hip_memcpy_dtod(c.stream, y.data(), x.data(), x.nbytes()), "Transpose");
+    // A permutation that only moves size-1 dims leaves the element order unchanged: the output
+    // is a view of the input (decode-time [1,1,H,D] <-> [1,H,1,D] head splits).
+    bool same_order = true;
+    int64_t prev = -1;
+    for (size_t d = 0; d < perm.size(); ++d) {
+        if (x.shape[perm[d]] == 1) continue;
+        if (perm[d] < prev) same_order = false;
+        prev = perm[d];
+    }
+    if (same_order) {
+        c.view_output(0, x, out_shape);
         return;
     }
+    Tensor &y = c.alloc_output(0, x.dtype, out_shape);
     rmlk_dims id = to_dims(x.shape);
     check_status(rmlk_hip_transpose(c.stream, x.dtype, &id, perm.data(), x.data(), y.data()),
                  "Transpose");

@@ -228,12 +228,21 @@ HostVal OpContext::host_values(int i) const {
 int32_t *OpContext::error_flag() const { return session.err_flag; }
 
 void *OpContext::scratch(size_t bytes) const {
-    auto b = std::make_shared<Buffer>();
-    b->bytes = bytes;
-    b->pool = &session.pool;
-    b->ptr = session.pool.alloc(bytes);
-    session.scratch_bufs.push_back(b);  // returned to the pool when the run's nodes are done
-    return b->ptr;
+    Session &ss = session;
+    if (bytes <= ss.workspace_bytes) return ss.workspace;
+    if (ss.capturing)
+        throw RtError(RMLK_ERR_OP, "MatMul workspace would grow while recording a HIP graph");
+    // grow: nothing that uses the old buffer is still queued behind this point of the stream
+    // once it is synchronised
+    check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+    ++ss.device_syncs_workspace;
+    if (ss.workspace) check_hip(hipFree(ss.workspace), "hipFree");
+    ss.workspace = nullptr;
+    size_t want = bytes + bytes / 4;
+    check_hip(hipMalloc(&ss.workspace, want), "hipMalloc (workspace)");
+    ss.workspace_bytes = want;
+    ++ss.pool.hip_mallocs;
+    return ss.workspace;
 }
 
 // ---- session ----------------------------------------------------------------------------------
@@ -245,6 +254,7 @@ Session::~Session() {
     }
     values.clear();
     scratch_bufs.clear();
+    if (workspace) (void)hipFree(workspace);
     if (err_flag) (void)hipFree(err_flag);
     if (err_host) (void)hipHostFree(err_host);
     if (stream) (void)hipStreamDestroy(stream);

@@ -110,7 +110,7 @@ def matmul(a, b, c, batch, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c,
     """ref: cuda/src/kernels/gemm.rs:112-136 (compute with a StridedBatchedConfig)."""
     need = matmul_workspace_size(batch, m, n, k, dtype_of(a))
     if workspace is None and need:
-        workspace = torch.empty(need, dtype=torch.uint8, device=a.device)
+        workspace = torch.zeros(need, dtype=torch.uint8, device=a.device)  # counters start at 0
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
     st = lib().rmlk_hip_matmul(_stream(), dtype_of(a), batch, m, n, k, _ptr(a), lda, stride_a,
                                int(trans_a), _ptr(b), ldb, stride_b, int(trans_b), _ptr(c), ldc,
