@@ -27,6 +27,23 @@ if ROOT not in sys.path:
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+CALIBRATION_COPY_BYTES = 256 << 20
+
+# HBM-side traffic of one gemm_mfma_kernel launch per MatMul shape (batch, m, n, k) of the default
+# workload, in KiB: (fetched, written). Read with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
+# (one run each) over `python3 bench.py --no-cpu --steps 1 --warmup 0 --decode 2`, scaled by what the
+# same counters read for the 256 MiB calibration copy below (FETCH_SIZE 131092 -> x2.0,
+# WRITE_SIZE 262144 -> x1.0). Split-K launches write partial sums to the workspace; the combine
+# kernel's own traffic is not included.
+PMC_TRAFFIC_KIB = {
+    (1, 512, 2048, 2048): (49262, 32768),
+    (1, 512, 512, 2048): (24632, 8192),
+    (32, 512, 640, 64): (28722, 35361),
+    (32, 512, 64, 640): (67787, 4096),
+    (1, 512, 8192, 2048): (98402, 16384),
+    (1, 512, 2048, 8192): (196706, 32768),
+    (1, 512, 128256, 2048): (1388996, 256512),
+}
 
 
 def log(*a):
@@ -67,6 +84,14 @@ def run_llama(args):
     t0 = time.perf_counter()
     inst = runtime.Builder.from_graph(graph).build(0)
     log(f"[bench] session created (weights uploaded) in {time.perf_counter() - t0:.1f}s")
+
+    # A plain copy of known size (256 MiB read + 256 MiB written by copy_flat_kernel): the unit
+    # that rocprofv3's FETCH_SIZE / WRITE_SIZE readings of the other kernels are scaled by.
+    calib = torch.empty(2 * CALIBRATION_COPY_BYTES // 4, dtype=torch.float32, device="cuda:0")
+    n_cal = CALIBRATION_COPY_BYTES // 4
+    kernels.concat_into(calib[:n_cal], calib[n_cal:], [n_cal], [n_cal], 0, 0)
+    torch.cuda.synchronize()
+    del calib
 
     rng = np.random.default_rng(4)
     prompt = rng.integers(0, cfg.vocab, size=prompt_len)
@@ -114,10 +139,14 @@ def run_llama(args):
     by_kind, per_op = {}, {}
     for s, (batch, m, n, k) in zip(mm_nodes, shapes):
         kind = kernels.matmul_describe(batch, m, n, k)
-        d = by_kind.setdefault(kind, {"launches": 0, "us": 0.0, "flops": 0.0})
+        d = by_kind.setdefault(kind, {"launches": 0, "us": 0.0, "flops": 0.0, "alg_bytes": 0.0,
+                                      "traffic": 0.0})
         d["launches"] += 1
         d["us"] += s["micros"]
         d["flops"] += 2.0 * batch * m * n * k
+        d["alg_bytes"] += 4.0 * batch * (m * k + k * n + m * n)
+        pmc = PMC_TRAFFIC_KIB.get((batch, m, n, k))
+        d["traffic"] = None if pmc is None or d["traffic"] is None else d["traffic"] + 1024.0 * sum(pmc)
     for s in stats:
         if s["micros"] > 0:
             d = per_op.setdefault(s["op"], {"n": 0, "us": 0.0, "bytes": 0.0})
@@ -131,7 +160,10 @@ def run_llama(args):
     roofline = {
         "bound": "mfma", "kernel": f"gemm_mfma_kernel ({dom_kind})",
         "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+        "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+        "traffic": None if dom["traffic"] is None else round(dom["traffic"] / dom["launches"]),
+        "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated)",
+        "algorithmic_bytes_per_launch": round(dom["alg_bytes"] / dom["launches"]),
         "launches": dom["launches"], "avg_launch_us": round(dom["us"] / dom["launches"], 2),
         "flops_per_launch": dom["flops"] / dom["launches"],
         "measured": "HIP events around every MatMul node of one eager prefill pass after the timed steps",
@@ -245,6 +277,7 @@ def run_ops_suite(args):
     import numpy as np
     import torch
     from rmlk_amd import kernels as k
+    from rmlk_amd._lib import check, lib
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev).manual_seed(2)
     ns = 6
@@ -290,6 +323,52 @@ def run_ops_suite(args):
         t.view(32, 2048, 2048).add_(mask)
     so = [torch.empty_like(sx[0]) for _ in range(2)]
     timed("softmax", lambda i: k.softmax(sx[i], so[i], 65536, 2048, 1), 2, 2 * sx[0].numel() * 4)
+    # ---- config 5 shapes: KV-cache / indexing stress ---------------------------------------------
+    kv_n = 8 * 8192 * 64
+    caches = [torch.randn(kv_n, device=dev, generator=g) for _ in range(ns * 3)]
+    outs = [torch.empty(kv_n, device=dev) for _ in range(ns * 3)]
+    rows = [torch.randn(8 * 64, device=dev, generator=g) for _ in range(ns)]
+    sidx = [torch.tensor([[0, h, int(p)] for h in range(8)], device=dev, dtype=torch.int64)
+            for p in np.random.default_rng(5).integers(0, 8192, size=ns)]
+    nk = ns * 3
+
+    def scatter_copy(i):
+        j = i % nk
+        check(lib().rmlk_hip_memcpy_dtod(torch.cuda.current_stream().cuda_stream, outs[j].data_ptr(),
+                                         caches[j].data_ptr(), kv_n * 4), "rmlk_hip_memcpy_dtod")
+        k.scatter_nd(sidx[i % ns], rows[i % ns], outs[j], [1, 8, 8192, 64], 8, 3)
+    timed("scatter_nd_copy", scatter_copy, nk, 2 * kv_n * 4 + 8 * 64 * 4 + 192)
+    timed("scatter_nd_inplace", lambda i: k.scatter_nd(sidx[i % ns], rows[i % ns], caches[i % nk],
+                                                       [1, 8, 8192, 64], 8, 3), nk, 8 * 64 * 4 + 192)
+    timed("slice_kv", lambda i: k.slice_(caches[i % nk], outs[i % nk], [1, 8, 8192, 64], [0, 0, 0, 0],
+                                         [1, 1, 1, 1], [1, 8, 8191, 64]), nk, 2 * 8 * 8191 * 64 * 4)
+
+    def concat_kv(i):
+        j = i % nk
+        k.concat_into(caches[j][:8 * 8191 * 64], outs[j], [1, 8, 8191, 64], [1, 8, 8192, 64], 2, 0)
+        k.concat_into(rows[i % ns], outs[j], [1, 8, 1, 64], [1, 8, 8192, 64], 2, 8191)
+    timed("concat_kv", concat_kv, nk, 2 * kv_n * 4)
+    del caches, outs
+    table = torch.randn(128256, 2048, device=dev, generator=g)
+    idx4 = [torch.randint(0, 128256, (4096,), device=dev, generator=g) for _ in range(ns)]
+    g4 = [torch.empty(4096 * 2048, device=dev) for _ in range(ns)]
+    timed("gather_4096", lambda i: k.gather(table, idx4[i], g4[i], [128256, 2048], 0), ns,
+          2 * 4096 * 2048 * 4 + 4096 * 8)
+    del table, g4
+    tri_in = [t.view(-1)[:8192 * 8192] for t in sx]
+    tri_out = [t.view(-1)[:8192 * 8192] for t in so]
+    timed("trilu_8192", lambda i: k.trilu(tri_in[i], tri_out[i], 1, 8192, 8192, True, 1), 2,
+          2 * 8192 * 8192 * 4)
+    eq_out = torch.empty(8192 * 8192, dtype=torch.bool, device=dev)
+    full = [8192, 8192]
+    dn = [8192, 1]
+    timed("equal_f32_8192", lambda i: k.binary(k.EQUAL, tri_in[i], tri_in[1 - i], eq_out, full, dn, dn),
+          2, 2 * 8192 * 8192 * 4 + 8192 * 8192)
+    timed("greater_f32_8192", lambda i: k.binary(k.GREATER, tri_in[i], tri_in[1 - i], eq_out, full, dn, dn),
+          2, 2 * 8192 * 8192 * 4 + 8192 * 8192)
+    i64a = [torch.randint(0, 100, (8192 * 8192,), device=dev, generator=g) for _ in range(2)]
+    timed("equal_i64_8192", lambda i: k.binary(k.EQUAL, i64a[i], i64a[1 - i], eq_out, full, dn, dn), 2,
+          2 * 8192 * 8192 * 8 + 8192 * 8192)
     print(json.dumps({"suite": "ops", "note": "per-kernel durations come from rocprofv3 of this command",
                       "results": results}))
 
