@@ -222,6 +222,50 @@ int32_t rmlk_hip_scatter_nd(rmlk_stream_t stream, int32_t reduction, int32_t dty
 int32_t rmlk_hip_trilu(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t rows,
                        int64_t cols, int32_t upper, int64_t k, const void *in, void *out);
 
+/* ---- fused operator chains --------------------------------------------------------------------
+ * The reference launches one kernel per ONNX node (runtime/src/providers/cuda/backend/<op>.rs); the
+ * four entry points below have no single counterpart there. Each computes, in one pass over
+ * memory, the chain of nodes named in its comment, and rounds every intermediate exactly as the
+ * separate kernels do, so a graph gives the same result either way. They support fp32 and return
+ * RMLK_ERR_UNSUPPORTED for layouts they do not cover (the caller then runs the separate kernels).
+ */
+
+/* y[r, :] = x[r, :] / sqrt(mean(x[r, :]^2) + eps) * gamma   (reciprocal_form == 0), or
+ * y[r, :] = x[r, :] * (1 / sqrt(mean(x[r, :]^2) + eps)) * gamma   (reciprocal_form != 0).
+ * Chain: Pow(x, 2) -> ReduceMean(axis -1, keepdims) -> Add(eps) -> Sqrt -> Div -> Mul(gamma)
+ * (ref kernels: cuda/src/kernels/binary.rs:58-100, reduce_mean.rs:40-93, unary.rs:10-42).
+ * x, out dense [rows, cols]; gamma [cols]; cols % 4 == 0, cols <= 8192, 16-byte aligned. */
+int32_t rmlk_hip_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t rows, int64_t cols,
+                         const void *x, const void *gamma, float eps, int32_t reciprocal_form,
+                         void *out);
+
+/* out = Softmax(x / scale + mask) (scale_is_mul == 0) or Softmax(x * scale + mask) over the last
+ * axis. `shape` is x's (and out's) dense shape; `mask_stride` gives the mask's element stride per
+ * dim of `shape` (0 on broadcast dims, 1 on the last dim).
+ * Chain: Div|Mul(x, scalar) -> Add(mask) -> Softmax(axis -1)
+ * (ref kernels: cuda/src/kernels/binary.rs:58-100, softmax.rs:5-37). */
+int32_t rmlk_hip_scale_mask_softmax(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *shape,
+                                    const rmlk_dims *mask_stride, int32_t scale_is_mul,
+                                    float scale, const void *x, const void *mask, void *out);
+
+/* out = (gate * sigmoid(gate)) * up over n elements.
+ * Chain: Sigmoid(gate) -> Mul(gate, .) -> Mul(., up)
+ * (ref kernels: cuda/src/kernels/unary.rs:10-42 via cuDNN sigmoid, binary.rs:58-100). */
+int32_t rmlk_hip_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *gate,
+                        const void *up, void *out);
+
+/* Rotary position embedding, half-rotation form, over x of logical shape [B, H, S, D]:
+ * out = x * cos + concat(-x[..., D/2:], x[..., :D/2]) * sin, out dense [B, H, S, D].
+ * x, cos and sin are read through element strides per dim of `shape` (innermost stride 1; 0 on
+ * broadcast dims), so a [B, S, H, D] projection output can be rotated and transposed in one pass.
+ * Chain: Slice, Slice, Neg, Concat, Mul, Mul, Add (optionally after Transpose perm 0,2,1,3)
+ * (ref kernels: cuda/src/kernels/slice.rs:61-122, unary.rs:10-42, binary.rs:58-100,
+ * transpose.rs:38-80). */
+int32_t rmlk_hip_rotary(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *shape,
+                        const rmlk_dims *x_stride, const rmlk_dims *cos_stride,
+                        const rmlk_dims *sin_stride, const void *x, const void *cos,
+                        const void *sin, void *out);
+
 /* Fill `n` elements of `out` with the element at host address `value` (size of dtype).
  * ref: runtime/src/providers/cuda/backend/constant_of_shape.rs:59-62 (host vector + H2D). */
 int32_t rmlk_hip_fill(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *value,

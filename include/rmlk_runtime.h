@@ -63,6 +63,16 @@ int32_t rmlk_graph_output(rmlk_graph *g, const char *name);
 /* Validates the graph, uploads the initializers to `device`, creates the stream.
  * ref: Builder::build, instance.rs:198-221 and TensorStore::init, providers/cuda/store.rs:95-261 */
 int32_t rmlk_session_create(const rmlk_graph *g, int32_t device, rmlk_session **out);
+/* The same with option flags. By default a session replaces four chains of small nodes that
+ * decoder graphs repeat per layer (decomposed RMSNorm, rotary embedding, SwiGLU, scale + mask +
+ * softmax) by single nodes backed by fused kernels with identical rounding;
+ * RMLK_SESSION_NO_FUSION keeps one kernel per ONNX node as the reference executes it
+ * (runtime/src/core/instance.rs:25-37). rmlk_session_create passes flags = 0. */
+#define RMLK_SESSION_NO_FUSION 1u
+int32_t rmlk_session_create_ex(const rmlk_graph *g, int32_t device, uint32_t flags,
+                               rmlk_session **out);
+/* Number of fused nodes the session formed while it was built. */
+int32_t rmlk_session_fused_nodes(const rmlk_session *s);
 void rmlk_session_destroy(rmlk_session *s);
 
 /* Feed a graph input from host memory (copied to a session-owned device buffer, H2D on the

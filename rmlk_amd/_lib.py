@@ -83,6 +83,13 @@ SIGNATURES = {
                                       c_void_p, c_void_p, c_void_p]),
     "rmlk_hip_trilu": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int32, c_int64,
                                  c_void_p, c_void_p]),
+    "rmlk_hip_rmsnorm": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p,
+                                   ctypes.c_float, c_int32, c_void_p]),
+    "rmlk_hip_scale_mask_softmax": (c_int32, [c_void_p, c_int32, _PD, _PD, c_int32, ctypes.c_float,
+                                              c_void_p, c_void_p, c_void_p]),
+    "rmlk_hip_swiglu": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p]),
+    "rmlk_hip_rotary": (c_int32, [c_void_p, c_int32, _PD, _PD, _PD, _PD, c_void_p, c_void_p,
+                                  c_void_p, c_void_p]),
     "rmlk_hip_fill": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
     "rmlk_hip_range": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p]),
     "rmlk_hip_write_small": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
@@ -115,6 +122,8 @@ SIGNATURES = {
                                          c_int32, c_void_p]),
     "rmlk_graph_output": (c_int32, [c_void_p, c_char_p]),
     "rmlk_session_create": (c_int32, [c_void_p, c_int32, POINTER(c_void_p)]),
+    "rmlk_session_create_ex": (c_int32, [c_void_p, c_int32, ctypes.c_uint32, POINTER(c_void_p)]),
+    "rmlk_session_fused_nodes": (c_int32, [c_void_p]),
     "rmlk_session_destroy": (None, [c_void_p]),
     "rmlk_session_set_input": (c_int32, [c_void_p, c_char_p, c_int32, POINTER(c_int64), c_int32,
                                          c_void_p]),

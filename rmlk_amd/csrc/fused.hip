@@ -1,0 +1,211 @@
+// Fused element-wise forms of operator chains that exported decoder graphs repeat in every layer.
+// The reference runs each ONNX node as its own kernel (runtime/src/providers/cuda/backend/<op>.rs);
+// these kernels compute the same chains in one pass over memory, with every intermediate rounded
+// exactly like the separate kernel would round it (no contraction into fma), so a graph gives the
+// same bits with or without them.
+//
+//   SwiGLU:  Mul(Mul(g, Sigmoid(g)), u)
+//   Rotary:  Add(Mul(x, cos), Mul(Concat(Neg(Slice(x, D/2..D)), Slice(x, 0..D/2)), sin))
+#include "common.hpp"
+
+namespace rmlk {
+namespace {
+
+constexpr int kBlock = 256;
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+__global__ __launch_bounds__(kBlock) void swiglu_kernel(const float *__restrict__ gate,
+                                                        const float *__restrict__ up,
+                                                        float *__restrict__ out, uint32_t n_vec) {
+    using V = Vec<float, 4>;
+    const V *g = reinterpret_cast<const V *>(gate);
+    const V *u = reinterpret_cast<const V *>(up);
+    V *o = reinterpret_cast<V *>(out);
+    constexpr uint32_t U = 4;
+    const uint32_t stride = gridDim.x * kBlock;
+    uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    for (; i + (U - 1) * stride < n_vec; i += U * stride) {
+        V gv[U], uv[U];
+#pragma unroll
+        for (uint32_t k = 0; k < U; ++k) {
+            gv[k] = g[i + k * stride];
+            uv[k] = u[i + k * stride];
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < U; ++k) {
+            V y;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float silu = gv[k].v[j] * sigmoid_f(gv[k].v[j]);
+                y.v[j] = silu * uv[k].v[j];
+            }
+            o[i + k * stride] = y;
+        }
+    }
+    for (; i < n_vec; i += stride) {
+        V gv = g[i], uv = u[i], y;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float silu = gv.v[j] * sigmoid_f(gv.v[j]);
+            y.v[j] = silu * uv.v[j];
+        }
+        o[i] = y;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void swiglu_tail_kernel(const float *__restrict__ gate,
+                                                             const float *__restrict__ up,
+                                                             float *__restrict__ out, int64_t begin,
+                                                             int64_t n) {
+    const int64_t i = begin + static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i < n) {
+        const float silu = gate[i] * sigmoid_f(gate[i]);
+        out[i] = silu * up[i];
+    }
+}
+
+// Rotary embedding over x [B,H,S,D] read through element strides (the innermost stride is 1), so a
+// [B,S,H,D] projection output is rotated and laid out [B,H,S,D] in the same pass. One lane takes W
+// neighbouring elements of the first half of a row together with their partners in the second half.
+struct RotaryArgs {
+    const float *x, *cos, *sin;
+    float *out;
+    FastDiv div_s, div_h, div_q;     // S, H, lanes per row
+    uint32_t n_s, n_h, n_q, half;
+    int64_t xs[3], cs[3], ss[3];     // strides of (b, h, s)
+    uint32_t total;                  // B * H * S * n_q
+};
+
+template <int W>
+__global__ __launch_bounds__(kBlock) void rotary_kernel(RotaryArgs a) {
+    using V = Vec<float, W>;
+    for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t < a.total; t += gridDim.x * kBlock) {
+        const uint32_t row = a.div_q.div(t), q = t - row * a.n_q;
+        const uint32_t bh = a.div_s.div(row), s = row - bh * a.n_s;
+        const uint32_t b = a.div_h.div(bh), h = bh - b * a.n_h;
+        const int64_t xo = b * a.xs[0] + h * a.xs[1] + s * a.xs[2];
+        const int64_t co = b * a.cs[0] + h * a.cs[1] + s * a.cs[2];
+        const int64_t so = b * a.ss[0] + h * a.ss[1] + s * a.ss[2];
+        const uint32_t d = q * W;
+        const V x1 = *reinterpret_cast<const V *>(a.x + xo + d);
+        const V x2 = *reinterpret_cast<const V *>(a.x + xo + d + a.half);
+        const V c1 = *reinterpret_cast<const V *>(a.cos + co + d);
+        const V c2 = *reinterpret_cast<const V *>(a.cos + co + d + a.half);
+        const V s1 = *reinterpret_cast<const V *>(a.sin + so + d);
+        const V s2 = *reinterpret_cast<const V *>(a.sin + so + d + a.half);
+        V y1, y2;
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+            const float a1 = x1.v[j] * c1.v[j];
+            const float r1 = (-x2.v[j]) * s1.v[j];
+            y1.v[j] = a1 + r1;
+            const float a2 = x2.v[j] * c2.v[j];
+            const float r2 = x1.v[j] * s2.v[j];
+            y2.v[j] = a2 + r2;
+        }
+        float *o = a.out + static_cast<int64_t>(row) * (2 * a.half) + d;
+        *reinterpret_cast<V *>(o) = y1;
+        *reinterpret_cast<V *>(o + a.half) = y2;
+    }
+}
+
+}  // namespace
+}  // namespace rmlk
+
+using namespace rmlk;
+
+extern "C" int32_t rmlk_hip_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *gate,
+                                   const void *up, void *out) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (n < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n == 0) return RMLK_OK;
+    if (!gate || !up || !out) return RMLK_ERR_NULL_POINTER;
+    if (n > kMaxElems) return RMLK_ERR_TOO_LARGE;
+    hipStream_t s = as_stream(stream);
+    const float *g = static_cast<const float *>(gate), *u = static_cast<const float *>(up);
+    float *o = static_cast<float *>(out);
+    const bool aligned = reinterpret_cast<uintptr_t>(g) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(u) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(o) % 16 == 0;
+    int64_t done = 0;
+    if (aligned) {
+        // pieces of at most 2^30 vectors keep the 32-bit index arithmetic in range
+        const int64_t n_vec = n / 4;
+        for (int64_t v0 = 0; v0 < n_vec; v0 += (int64_t)1 << 30) {
+            const int64_t cnt = n_vec - v0 < ((int64_t)1 << 30) ? n_vec - v0 : (int64_t)1 << 30;
+            swiglu_kernel<<<grid_for(cnt, kBlock * 4, 8), kBlock, 0, s>>>(
+                g + v0 * 4, u + v0 * 4, o + v0 * 4, static_cast<uint32_t>(cnt));
+        }
+        done = n_vec * 4;
+    }
+    if (done < n) {
+        const int64_t rest = n - done;
+        const int64_t blocks = (rest + kBlock - 1) / kBlock;
+        if (blocks >= ((int64_t)1 << 31)) return RMLK_ERR_TOO_LARGE;
+        swiglu_tail_kernel<<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(g, u, o, done, n);
+    }
+    return launch_status();
+}
+
+extern "C" int32_t rmlk_hip_rotary(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *shape,
+                                   const rmlk_dims *x_stride, const rmlk_dims *cos_stride,
+                                   const rmlk_dims *sin_stride, const void *x, const void *cos,
+                                   const void *sin, void *out) {
+    if (!dims_ok(shape) || !dims_ok(x_stride) || !dims_ok(cos_stride) || !dims_ok(sin_stride))
+        return RMLK_ERR_BAD_RANK;
+    if (shape->rank != 4 || x_stride->rank != 4 || cos_stride->rank != 4 || sin_stride->rank != 4)
+        return RMLK_ERR_BAD_RANK;
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    const int64_t numel = dims_numel(shape);
+    if (numel < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (numel == 0) return RMLK_OK;
+    if (!x || !cos || !sin || !out) return RMLK_ERR_NULL_POINTER;
+    const int64_t d = shape->v[3];
+    if (d % 2 != 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (x_stride->v[3] != 1 || cos_stride->v[3] != 1 || sin_stride->v[3] != 1)
+        return RMLK_ERR_UNSUPPORTED;
+    const int64_t half = d / 2;
+    const int64_t rows = numel / d;
+    for (int i = 0; i < 3; ++i)
+        if (x_stride->v[i] < 0 || cos_stride->v[i] < 0 || sin_stride->v[i] < 0)
+            return RMLK_ERR_INVALID_ARGUMENT;
+    // widest lane width that keeps every access aligned
+    auto ok = [&](int w) {
+        if (half % w) return false;
+        const uintptr_t mask = static_cast<uintptr_t>(w) * 4 - 1;
+        if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(cos) |
+             reinterpret_cast<uintptr_t>(sin) | reinterpret_cast<uintptr_t>(out)) & mask)
+            return false;
+        for (int i = 0; i < 3; ++i)
+            if (x_stride->v[i] % w || cos_stride->v[i] % w || sin_stride->v[i] % w) return false;
+        return true;
+    };
+    const int w = ok(4) ? 4 : ok(2) ? 2 : 1;
+    const int64_t total = rows * (half / w);
+    if (total >= ((int64_t)1 << 31) || numel >= ((int64_t)1 << 32)) return RMLK_ERR_TOO_LARGE;
+    RotaryArgs a;
+    a.x = static_cast<const float *>(x);
+    a.cos = static_cast<const float *>(cos);
+    a.sin = static_cast<const float *>(sin);
+    a.out = static_cast<float *>(out);
+    a.n_s = static_cast<uint32_t>(shape->v[2]);
+    a.n_h = static_cast<uint32_t>(shape->v[1]);
+    a.n_q = static_cast<uint32_t>(half / w);
+    a.half = static_cast<uint32_t>(half);
+    a.div_s = FastDiv(a.n_s);
+    a.div_h = FastDiv(a.n_h);
+    a.div_q = FastDiv(a.n_q);
+    for (int i = 0; i < 3; ++i) {
+        a.xs[i] = x_stride->v[i];
+        a.cs[i] = cos_stride->v[i];
+        a.ss[i] = sin_stride->v[i];
+    }
+    a.total = static_cast<uint32_t>(total);
+    hipStream_t s = as_stream(stream);
+    const unsigned grid = grid_for(total, kBlock, 16);
+    if (w == 4) rotary_kernel<4><<<grid, kBlock, 0, s>>>(a);
+    else if (w == 2) rotary_kernel<2><<<grid, kBlock, 0, s>>>(a);
+    else rotary_kernel<1><<<grid, kBlock, 0, s>>>(a);
+    return launch_status();
+}

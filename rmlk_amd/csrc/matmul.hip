@@ -371,24 +371,39 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(GemvArgs g) {
     }
 }
 
-// Combine GEMV partials [split][total] -> y: 64 outputs per block, 4 lanes per output take the
-// splits round-robin, then the four sums meet in LDS in a fixed order.
+// Combine GEMV partials [split][total] -> y: 32 outputs per block, 8 lanes per output take the
+// splits round-robin with four independent loads in flight, then the eight sums meet in LDS in
+// a fixed order (the result depends on `splits` only, never on timing).
 __global__ __launch_bounds__(kThreads) void gemv_reduce_kernel(const float *__restrict__ ws,
                                                                float *__restrict__ y, int splits,
                                                                int64_t batch, int32_t n,
                                                                int64_t stride_y) {
-    __shared__ float part[4][64];
+    constexpr int kOut = 32, kGroups = kThreads / kOut;
+    __shared__ float part[kGroups][kOut];
     const int64_t total = batch * n;
-    const int ox = threadIdx.x % 64, sy = threadIdx.x / 64;
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * 64 + ox;
+    const int ox = threadIdx.x % kOut, sy = threadIdx.x / kOut;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kOut + ox;
     float s = 0.f;
-    if (i < total)
-        for (int z = sy; z < splits; z += 4) s += ws[z * total + i];
+    if (i < total) {
+        const float *p = ws + i;
+        int z = sy;
+        for (; z + 3 * kGroups < splits; z += 4 * kGroups) {
+            const float v0 = p[static_cast<int64_t>(z) * total];
+            const float v1 = p[static_cast<int64_t>(z + kGroups) * total];
+            const float v2 = p[static_cast<int64_t>(z + 2 * kGroups) * total];
+            const float v3 = p[static_cast<int64_t>(z + 3 * kGroups) * total];
+            s += (v0 + v1) + (v2 + v3);
+        }
+        for (; z < splits; z += kGroups) s += p[static_cast<int64_t>(z) * total];
+    }
     part[sy][ox] = s;
     __syncthreads();
     if (sy == 0 && i < total) {
         const int64_t b = i / n, col = i - b * n;
-        y[b * stride_y + col] = (part[0][ox] + part[1][ox]) + (part[2][ox] + part[3][ox]);
+        float r = 0.f;
+#pragma unroll
+        for (int q = 0; q < kGroups; ++q) r += part[q][ox];
+        y[b * stride_y + col] = r;
     }
 }
 
@@ -635,7 +650,7 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
         if (st) return st;
         if (splits > 1) {
             const int64_t total = batch * n;
-            gemv_reduce_kernel<<<static_cast<unsigned>((total + 63) / 64), kThreads, 0, s>>>(
+            gemv_reduce_kernel<<<static_cast<unsigned>((total + 31) / 32), kThreads, 0, s>>>(
                 static_cast<const float *>(workspace), pc, splits, batch, g.n, stride_c);
             return launch_status();
         }

@@ -123,11 +123,51 @@ __device__ __forceinline__ float neg_inf<float>() {
     return -__builtin_huge_valf();
 }
 
+// Where a softmax row comes from: plain memory, or (x / c + mask) resp. (x * c + mask) computed on
+// the fly with exactly the roundings of the separate Div (Mul) and Add kernels.
+template <typename T>
+struct PlainRows {
+    const T *in;
+    __device__ __forceinline__ Vec<T, 4> load(int64_t row, int c, int32_t cols) const {
+        return reinterpret_cast<const Vec<T, 4> *>(in + row * cols)[c];
+    }
+};
+
+// row -> offset into a mask that is broadcast over some of the leading dims
+struct RowMap {
+    FastDiv d1, d2;       // extents of the two inner row dims
+    uint32_t n1, n2;
+    int64_t s0, s1, s2;   // mask element strides of the three row dims
+    __device__ __forceinline__ int64_t offset(uint32_t row) const {
+        const uint32_t t = d2.div(row), i2 = row - t * n2;
+        const uint32_t i0 = d1.div(t), i1 = t - i0 * n1;
+        return i0 * s0 + i1 * s1 + i2 * s2;
+    }
+};
+
+template <typename T, bool MUL>
+struct ScaledMaskedRows {
+    const T *in;
+    const T *mask;
+    T scale;
+    RowMap map;
+    __device__ __forceinline__ Vec<T, 4> load(int64_t row, int c, int32_t cols) const {
+        Vec<T, 4> x = reinterpret_cast<const Vec<T, 4> *>(in + row * cols)[c];
+        Vec<T, 4> m = reinterpret_cast<const Vec<T, 4> *>(
+            mask + map.offset(static_cast<uint32_t>(row)))[c];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const T scaled = MUL ? x.v[j] * scale : x.v[j] / scale;
+            x.v[j] = scaled + m.v[j];
+        }
+        return x;
+    }
+};
+
 // kGroup lanes own a row of up to kGroup * 4 * NV elements; cols % 4 == 0 and 16-byte aligned rows.
-template <typename T, int NV, int kGroup>
-__global__ __launch_bounds__(kBlock) void softmax_regs_kernel(const T *__restrict__ in,
-                                                              T *__restrict__ out, int64_t rows,
-                                                              int32_t cols) {
+template <typename T, int NV, int kGroup, typename Rows>
+__global__ __launch_bounds__(kBlock) void softmax_regs_kernel(Rows src, T *__restrict__ out,
+                                                              int64_t rows, int32_t cols) {
     __shared__ T red_buf[2][kWavesPerBlock];
     using V = Vec<T, 4>;
     constexpr int kRowsPerBlock = kBlock / kGroup;
@@ -138,14 +178,13 @@ __global__ __launch_bounds__(kBlock) void softmax_regs_kernel(const T *__restric
          row0 += static_cast<int64_t>(gridDim.x) * kRowsPerBlock) {
         const int64_t row = row0 + group;
         const bool live = row < rows;
-        const V *pv = reinterpret_cast<const V *>(in + row * cols);
         V x[NV];
         T m = neg_inf<T>();
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int c = lane_in_group + i * kGroup;
             if (live && c < nv) {
-                x[i] = pv[c];
+                x[i] = src.load(row, c, cols);
             } else {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) x[i].v[j] = neg_inf<T>();
@@ -243,15 +282,27 @@ __global__ __launch_bounds__(kBlock) void softmax_strided_kernel(const T *__rest
     }
 }
 
-template <typename T, int NV, int kGroup>
-int32_t launch_softmax_regs(hipStream_t s, const T *in, T *out, int64_t rows, int32_t cols) {
+template <typename T, int NV, int kGroup, typename Rows>
+int32_t launch_softmax_regs(hipStream_t s, const Rows &src, T *out, int64_t rows, int32_t cols) {
     constexpr int kRowsPerBlock = kBlock / kGroup;
     int64_t blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
     const int64_t cap = static_cast<int64_t>(kNumCU) * 64;
     if (blocks > cap) blocks = cap;
-    softmax_regs_kernel<T, NV, kGroup><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(in, out,
-                                                                                       rows, cols);
+    softmax_regs_kernel<T, NV, kGroup, Rows><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(
+        src, out, rows, cols);
     return launch_status();
+}
+
+// Same row-length ladder for the plain and the fused softmax, so both give the same bits.
+template <typename T, typename Rows>
+int32_t softmax_regs_dispatch(hipStream_t s, const Rows &src, T *out, int64_t rows, int32_t c) {
+    if (c <= 256) return launch_softmax_regs<T, 1, kWave>(s, src, out, rows, c);
+    if (c <= 512) return launch_softmax_regs<T, 2, kWave>(s, src, out, rows, c);
+    if (c <= 1024) return launch_softmax_regs<T, 4, kWave>(s, src, out, rows, c);
+    if (c <= 2048) return launch_softmax_regs<T, 8, kWave>(s, src, out, rows, c);
+    if (c <= 4096) return launch_softmax_regs<T, 4, kBlock>(s, src, out, rows, c);
+    if (c <= 8192) return launch_softmax_regs<T, 8, kBlock>(s, src, out, rows, c);
+    return launch_softmax_regs<T, 16, kBlock>(s, src, out, rows, c);
 }
 
 template <typename T>
@@ -261,16 +312,8 @@ int32_t softmax_typed(hipStream_t s, int64_t outer, int64_t n, int64_t inner, co
         const bool vec_ok = n % 4 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
                             reinterpret_cast<uintptr_t>(out) % 16 == 0 && n <= 16384 &&
                             sizeof(T) == 4;
-        if (vec_ok) {
-            const int32_t c = static_cast<int32_t>(n);
-            if (c <= 256) return launch_softmax_regs<T, 1, kWave>(s, in, out, outer, c);
-            if (c <= 512) return launch_softmax_regs<T, 2, kWave>(s, in, out, outer, c);
-            if (c <= 1024) return launch_softmax_regs<T, 4, kWave>(s, in, out, outer, c);
-            if (c <= 2048) return launch_softmax_regs<T, 8, kWave>(s, in, out, outer, c);
-            if (c <= 4096) return launch_softmax_regs<T, 4, kBlock>(s, in, out, outer, c);
-            if (c <= 8192) return launch_softmax_regs<T, 8, kBlock>(s, in, out, outer, c);
-            return launch_softmax_regs<T, 16, kBlock>(s, in, out, outer, c);
-        }
+        if (vec_ok)
+            return softmax_regs_dispatch<T>(s, PlainRows<T>{in}, out, outer, static_cast<int32_t>(n));
         int64_t blocks = (outer + kWavesPerBlock - 1) / kWavesPerBlock;
         const int64_t cap = static_cast<int64_t>(kNumCU) * 32;
         if (blocks > cap) blocks = cap;
@@ -279,6 +322,90 @@ int32_t softmax_typed(hipStream_t s, int64_t outer, int64_t n, int64_t inner, co
     }
     unsigned grid = grid_for(outer * inner, kBlock, 16);
     softmax_strided_kernel<T><<<grid, kBlock, 0, s>>>(in, out, outer, n, inner);
+    return launch_status();
+}
+
+// ---- RMSNorm: y = x / sqrt(mean(x^2) + eps) * gamma, one pass, the row held in registers --------
+// The fused form of Pow(2) -> ReduceMean(-1) -> Add(eps) -> Sqrt -> Div -> Mul(gamma): squares are
+// rounded to float before the double accumulation and every later step rounds like the separate
+// kernel does. RECIP selects the exported variant x * (1 / sqrt(..)) * gamma.
+template <int NV, int kGroup, bool RECIP>
+__global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const float *__restrict__ x,
+                                                         const float *__restrict__ gamma,
+                                                         float *__restrict__ out, int64_t rows,
+                                                         int32_t cols, float eps) {
+    __shared__ double partial[kWavesPerBlock];
+    using V = Vec<float, 4>;
+    constexpr int kRowsPerBlock = kBlock / kGroup;
+    const int lane_in_group = threadIdx.x % kGroup;
+    const int group = threadIdx.x / kGroup;
+    const int nv = cols / 4;
+    V g[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = lane_in_group + i * kGroup;
+        if (c < nv) g[i] = reinterpret_cast<const V *>(gamma)[c];
+    }
+    for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock; row0 < rows;
+         row0 += static_cast<int64_t>(gridDim.x) * kRowsPerBlock) {
+        const int64_t row = row0 + group;
+        const bool live = row < rows;
+        const V *pv = reinterpret_cast<const V *>(x + row * cols);
+        V xv[NV];
+        double acc = 0.0;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = lane_in_group + i * kGroup;
+            if (live && c < nv) {
+                xv[i] = pv[c];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float sq = xv[i].v[j] * xv[i].v[j];
+                    acc += static_cast<double>(sq);
+                }
+            }
+        }
+        acc = wave_sum(acc);
+        if constexpr (kGroup == kBlock) {
+            const int wave = threadIdx.x / kWave;
+            if ((threadIdx.x % kWave) == 0) partial[wave] = acc;
+            __syncthreads();
+            acc = 0.0;
+#pragma unroll
+            for (int w = 0; w < kWavesPerBlock; ++w) acc += partial[w];
+            __syncthreads();
+        }
+        const float mean = static_cast<float>(acc / static_cast<double>(cols));
+        const float var = mean + eps;
+        const float r = sqrtf(var);
+        const float inv = 1.0f / r;
+        V *po = reinterpret_cast<V *>(out + row * cols);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = lane_in_group + i * kGroup;
+            if (live && c < nv) {
+                V y;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float normed = RECIP ? xv[i].v[j] * inv : xv[i].v[j] / r;
+                    y.v[j] = normed * g[i].v[j];
+                }
+                po[c] = y;
+            }
+        }
+    }
+}
+
+template <int NV, int kGroup>
+int32_t launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *out, int64_t rows,
+                       int32_t cols, float eps, bool recip) {
+    constexpr int kRowsPerBlock = kBlock / kGroup;
+    int64_t blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+    const int64_t cap = static_cast<int64_t>(kNumCU) * 32;
+    if (blocks > cap) blocks = cap;
+    const unsigned grid = static_cast<unsigned>(blocks);
+    if (recip) rmsnorm_kernel<NV, kGroup, true><<<grid, kBlock, 0, s>>>(x, gamma, out, rows, cols, eps);
+    else rmsnorm_kernel<NV, kGroup, false><<<grid, kBlock, 0, s>>>(x, gamma, out, rows, cols, eps);
     return launch_status();
 }
 
@@ -400,4 +527,95 @@ extern "C" int32_t rmlk_hip_softmax(rmlk_stream_t stream, int32_t dtype, int64_t
                                     static_cast<float *>(out));
     return softmax_typed<double>(s, outer, axis_len, inner, static_cast<const double *>(in),
                                  static_cast<double *>(out));
+}
+
+extern "C" int32_t rmlk_hip_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t rows, int64_t cols,
+                                    const void *x, const void *gamma, float eps,
+                                    int32_t reciprocal_form, void *out) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (rows < 0 || cols < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (rows == 0 || cols == 0) return RMLK_OK;
+    if (!x || !gamma || !out) return RMLK_ERR_NULL_POINTER;
+    if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
+    const bool vec_ok = cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                        reinterpret_cast<uintptr_t>(gamma) % 16 == 0 &&
+                        reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    if (!vec_ok || cols > kBlock * 4 * 8) return RMLK_ERR_UNSUPPORTED;
+    hipStream_t s = as_stream(stream);
+    const float *xp = static_cast<const float *>(x), *gp = static_cast<const float *>(gamma);
+    float *op = static_cast<float *>(out);
+    const int32_t c = static_cast<int32_t>(cols);
+    const bool recip = reciprocal_form != 0;
+    if (rows >= 1024 && c <= kWave * 4 * 8) {  // many rows: a wavefront per row
+        if (c <= 256) return launch_rmsnorm<1, kWave>(s, xp, gp, op, rows, c, eps, recip);
+        if (c <= 512) return launch_rmsnorm<2, kWave>(s, xp, gp, op, rows, c, eps, recip);
+        if (c <= 1024) return launch_rmsnorm<4, kWave>(s, xp, gp, op, rows, c, eps, recip);
+        return launch_rmsnorm<8, kWave>(s, xp, gp, op, rows, c, eps, recip);
+    }
+    if (c <= 1024) return launch_rmsnorm<1, kBlock>(s, xp, gp, op, rows, c, eps, recip);
+    if (c <= 2048) return launch_rmsnorm<2, kBlock>(s, xp, gp, op, rows, c, eps, recip);
+    if (c <= 4096) return launch_rmsnorm<4, kBlock>(s, xp, gp, op, rows, c, eps, recip);
+    return launch_rmsnorm<8, kBlock>(s, xp, gp, op, rows, c, eps, recip);
+}
+
+extern "C" int32_t rmlk_hip_scale_mask_softmax(rmlk_stream_t stream, int32_t dtype,
+                                               const rmlk_dims *shape,
+                                               const rmlk_dims *mask_stride, int32_t scale_is_mul,
+                                               float scale, const void *x, const void *mask,
+                                               void *out) {
+    if (!dims_ok(shape) || !dims_ok(mask_stride) || mask_stride->rank != shape->rank)
+        return RMLK_ERR_BAD_RANK;
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    const int rank = shape->rank;
+    const int64_t numel = dims_numel(shape);
+    if (numel < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (numel == 0) return RMLK_OK;
+    if (!x || !mask || !out) return RMLK_ERR_NULL_POINTER;
+    const int64_t cols = shape->v[rank - 1], rows = numel / cols;
+    if (mask_stride->v[rank - 1] != 1 && cols != 1) return RMLK_ERR_UNSUPPORTED;
+    if (rows >= ((int64_t)1 << 31) || cols > 16384 || cols % 4 != 0) return RMLK_ERR_UNSUPPORTED;
+    // leading dims -> at most three (extent, mask stride) pairs: drop extent 1, merge neighbours
+    int64_t ext[kMaxRank], str[kMaxRank];
+    int nd = 0;
+    for (int d = 0; d < rank - 1; ++d) {
+        if (shape->v[d] == 1) continue;
+        const int64_t st = mask_stride->v[d];
+        if (st < 0) return RMLK_ERR_INVALID_ARGUMENT;
+        if (nd > 0 && str[nd - 1] == st * shape->v[d]) {
+            ext[nd - 1] *= shape->v[d];
+            str[nd - 1] = st;
+        } else {
+            ext[nd] = shape->v[d];
+            str[nd++] = st;
+        }
+    }
+    if (nd > 3) return RMLK_ERR_UNSUPPORTED;
+    for (int d = 0; d < nd; ++d)
+        if (str[d] % 4 != 0) return RMLK_ERR_UNSUPPORTED;
+    if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(mask) % 16 ||
+        reinterpret_cast<uintptr_t>(out) % 16)
+        return RMLK_ERR_UNSUPPORTED;
+    // right-align into (i0, i1, i2)
+    int64_t e3[3] = {1, 1, 1}, s3[3] = {0, 0, 0};
+    for (int d = 0; d < nd; ++d) {
+        e3[3 - nd + d] = ext[d];
+        s3[3 - nd + d] = str[d];
+    }
+    RowMap map;
+    map.n1 = static_cast<uint32_t>(e3[1]);
+    map.n2 = static_cast<uint32_t>(e3[2]);
+    map.d1 = FastDiv(map.n1);
+    map.d2 = FastDiv(map.n2);
+    map.s0 = s3[0];
+    map.s1 = s3[1];
+    map.s2 = s3[2];
+    hipStream_t s = as_stream(stream);
+    const float *xp = static_cast<const float *>(x), *mp = static_cast<const float *>(mask);
+    float *op = static_cast<float *>(out);
+    const int32_t c = static_cast<int32_t>(cols);
+    if (scale_is_mul)
+        return softmax_regs_dispatch<float>(s, ScaledMaskedRows<float, true>{xp, mp, scale, map}, op,
+                                            rows, c);
+    return softmax_regs_dispatch<float>(s, ScaledMaskedRows<float, false>{xp, mp, scale, map}, op,
+                                        rows, c);
 }

@@ -248,6 +248,19 @@ int32_t rmlk_session_create(const rmlk_graph *g, int32_t device, rmlk_session **
     });
 }
 
+int32_t rmlk_session_create_ex(const rmlk_graph *g, int32_t device, uint32_t flags,
+                               rmlk_session **out) {
+    return guarded([&] {
+        if (!g || !out) throw RtError(RMLK_ERR_NULL_POINTER, "null argument");
+        auto s = std::make_unique<rmlk_session>();
+        s->impl.fuse = (flags & RMLK_SESSION_NO_FUSION) == 0;
+        s->impl.build(*g, device);
+        *out = s.release();
+    });
+}
+
+int32_t rmlk_session_fused_nodes(const rmlk_session *s) { return s ? s->impl.fused_nodes : 0; }
+
 void rmlk_session_destroy(rmlk_session *s) {
     if (!s) return;
     (void)hipSetDevice(s->impl.device);

@@ -136,6 +136,7 @@ struct Node {
     std::vector<int> inputs;   // value ids, -1 = omitted optional input
     std::vector<int> outputs;
     std::unordered_map<std::string, Attr> attrs;
+    std::vector<Node> body;    // fused nodes only: the nodes this one replaced, in graph order
 };
 
 struct Value {
@@ -196,6 +197,13 @@ struct OpContext {
 using OpFn = void (*)(OpContext &);
 OpFn find_op(const std::string &name);
 
+// Pattern fusion (fusion.cpp): rewrites session.graph_copy.nodes, returns the number of fused nodes.
+int fuse_patterns(Session &s);
+void op_fused_rmsnorm(OpContext &c);
+void op_fused_swiglu(OpContext &c);
+void op_fused_softmax(OpContext &c);
+void op_fused_rotary(OpContext &c);
+
 struct CapturedPlan {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
@@ -218,6 +226,8 @@ struct Session {
     int32_t *err_host = nullptr;     // pinned host
     bool capturing = false;
     bool profiling = false;
+    bool fuse = true;                // form fused nodes while building
+    int fused_nodes = 0;
     int64_t device_syncs = 0;            // blocking reads of shape-like tensors
     int64_t device_syncs_workspace = 0;  // stream syncs taken to grow the MatMul workspace
     std::unique_ptr<CapturedPlan> plan;

@@ -1,0 +1,535 @@
+// Pattern fusion over the node list of a session's graph.
+//
+// The reference executes an ONNX graph node by node, one kernel each
+// (runtime/src/core/instance.rs:25-37). Decoder graphs repeat a few chains of small element-wise
+// nodes in every layer; on this GPU each launch costs ~2 us whatever it moves, so those chains
+// dominate a decode step. This pass finds four of them and replaces each by ONE node backed by a
+// fused kernel that rounds every intermediate like the separate kernels do:
+//
+//   rmlk.RMSNorm           Pow(x,2) ReduceMean(-1) Add(eps) Sqrt Div|(Div(1,.) Mul) Mul(gamma)
+//   rmlk.SwiGLU            Sigmoid(g) Mul(g,.) Mul(.,u)
+//   rmlk.ScaleMaskSoftmax  Div|Mul(x,c) Add(mask) Softmax(-1)
+//   rmlk.Rotary            [Transpose(0,2,1,3)] Slice Slice Neg Concat Mul Mul Add
+//
+// A fused node keeps the nodes it replaced as its `body`. What cannot be decided while building
+// (shapes are only known at run time) is checked when the node runs; if the fused kernel does not
+// cover the case, the body runs instead, node by node, so the graph's meaning never changes.
+#include <algorithm>
+#include <cmath>
+#include <set>
+
+#include "core.hpp"
+
+namespace rmlk {
+namespace rt {
+
+namespace {
+
+struct Matcher {
+    Session &s;
+    rmlk_graph &g;
+    std::vector<std::vector<int>> users;   // value id -> consumer node indices
+    std::vector<bool> removed;
+
+    explicit Matcher(Session &session) : s(session), g(session.graph_copy) {
+        users.assign(g.values.size(), {});
+        removed.assign(g.nodes.size(), false);
+        for (size_t n = 0; n < g.nodes.size(); ++n)
+            for (int v : g.nodes[n].inputs)
+                if (v >= 0) users[v].push_back(static_cast<int>(n));
+    }
+
+    int producer(int v) const {
+        if (v < 0) return -1;
+        const Value &val = g.values[v];
+        if (val.is_input || val.is_initializer) return -1;
+        int p = val.producer;
+        return p >= 0 && !removed[p] ? p : -1;
+    }
+    const Node *produced_by(int v, const char *op) const {
+        int p = producer(v);
+        return p >= 0 && g.nodes[p].op == op ? &g.nodes[p] : nullptr;
+    }
+    // every consumer of v is one of `inside`, and v is not a graph output
+    bool only_used_by(int v, std::initializer_list<const Node *> inside) const {
+        if (g.values[v].is_output) return false;
+        for (int u : users[v]) {
+            bool ok = false;
+            for (const Node *n : inside)
+                if (n == &g.nodes[u]) ok = true;
+            if (!ok) return false;
+        }
+        return true;
+    }
+    bool const_float(int v, float *out) const {
+        if (v < 0 || !g.values[v].is_initializer) return false;
+        const Tensor &t = s.values[v];
+        if (t.dtype != RMLK_FLOAT || t.numel() != 1 || !t.host || !t.host->is_float) return false;
+        *out = static_cast<float>(t.host->f[0]);
+        return true;
+    }
+    bool const_ints(int v, std::vector<int64_t> *out) const {
+        if (v < 0 || !g.values[v].is_initializer) return false;
+        const Tensor &t = s.values[v];
+        if (!t.host || t.host->is_float) return false;
+        if (t.dtype != RMLK_INT64 && t.dtype != RMLK_INT32) return false;
+        *out = t.host->i;
+        return true;
+    }
+    static int64_t attr_int(const Node &n, const char *name, int64_t dflt) {
+        auto it = n.attrs.find(name);
+        return it == n.attrs.end() ? dflt : it->second.i;
+    }
+    int index_of(const Node *n) const { return static_cast<int>(n - g.nodes.data()); }
+
+    // Replace `parts` (graph order) by one node at the position of the last of them.
+    void replace(const std::vector<const Node *> &parts, Node fused) {
+        std::vector<int> idx;
+        for (const Node *n : parts) idx.push_back(index_of(n));
+        std::sort(idx.begin(), idx.end());
+        for (int i : idx) fused.body.push_back(g.nodes[i]);
+        for (int i : idx) {
+            removed[i] = true;
+            for (int v : g.nodes[i].inputs) {
+                if (v < 0) continue;
+                auto &u = users[v];
+                u.erase(std::remove(u.begin(), u.end(), i), u.end());
+            }
+        }
+        const int at = idx.back();
+        g.nodes[at] = std::move(fused);
+        removed[at] = false;
+        // consumers: the fused node now reads its inputs at `at`
+        for (int v : g.nodes[at].inputs)
+            if (v >= 0) users[v].push_back(at);
+        for (int v : g.nodes[at].outputs) g.values[v].producer = at;
+    }
+
+    static Attr a_int(int64_t v) {
+        Attr a;
+        a.kind = Attr::Int;
+        a.i = v;
+        return a;
+    }
+    static Attr a_float(float v) {
+        Attr a;
+        a.kind = Attr::Float;
+        a.f = v;
+        return a;
+    }
+
+    // ---- RMSNorm, anchored at the final Mul ------------------------------------------------------
+    bool match_rmsnorm(const Node &m2) {
+        if (m2.op != "Mul" || m2.inputs.size() != 2) return false;
+        for (int side = 0; side < 2; ++side) {
+            const int normed = m2.inputs[side], gamma = m2.inputs[1 - side];
+            if (normed < 0 || gamma < 0) continue;
+            const Node *sqrt_n = nullptr, *div_n = nullptr, *mul_n = nullptr;
+            int x = -1;
+            bool recip = false;
+            if (const Node *d = produced_by(normed, "Div")) {
+                // x / sqrt(var)
+                if (d->inputs.size() != 2) continue;
+                sqrt_n = produced_by(d->inputs[1], "Sqrt");
+                if (!sqrt_n) continue;
+                div_n = d;
+                x = d->inputs[0];
+            } else if (const Node *m = produced_by(normed, "Mul")) {
+                // x * (1 / sqrt(var))
+                if (m->inputs.size() != 2) continue;
+                for (int k = 0; k < 2 && !div_n; ++k) {
+                    const Node *d = produced_by(m->inputs[k], "Div");
+                    float one;
+                    if (d && d->inputs.size() == 2 && const_float(d->inputs[0], &one) &&
+                        one == 1.0f && (sqrt_n = produced_by(d->inputs[1], "Sqrt"))) {
+                        div_n = d;
+                        mul_n = m;
+                        x = m->inputs[1 - k];
+                    }
+                }
+                if (!div_n) continue;
+                recip = true;
+            } else {
+                continue;
+            }
+            const Node *add_n = produced_by(sqrt_n->inputs[0], "Add");
+            if (!add_n || add_n->inputs.size() != 2) continue;
+            float eps = 0.f;
+            const Node *mean_n = nullptr;
+            for (int k = 0; k < 2 && !mean_n; ++k)
+                if (const_float(add_n->inputs[1 - k], &eps))
+                    mean_n = produced_by(add_n->inputs[k], "ReduceMean");
+            if (!mean_n) continue;
+            if (attr_int(*mean_n, "keepdims", 1) != 1) continue;
+            int64_t axis = 0;
+            {
+                std::vector<int64_t> axes;
+                auto it = mean_n->attrs.find("axes");
+                if (it != mean_n->attrs.end()) axes = it->second.ints;
+                else if (mean_n->inputs.size() > 1 && !const_ints(mean_n->inputs[1], &axes)) continue;
+                if (axes.size() != 1) continue;
+                axis = axes[0];
+            }
+            const Node *pow_n = produced_by(mean_n->inputs[0], "Pow");
+            float two;
+            if (!pow_n || pow_n->inputs.size() != 2 || pow_n->inputs[0] != x ||
+                !const_float(pow_n->inputs[1], &two) || two != 2.0f)
+                continue;
+            // every intermediate feeds the chain only
+            if (!only_used_by(pow_n->outputs[0], {mean_n}) ||
+                !only_used_by(mean_n->outputs[0], {add_n}) ||
+                !only_used_by(add_n->outputs[0], {sqrt_n}) ||
+                !only_used_by(sqrt_n->outputs[0], {div_n}))
+                continue;
+            if (recip) {
+                if (!only_used_by(div_n->outputs[0], {mul_n}) ||
+                    !only_used_by(mul_n->outputs[0], {&m2}))
+                    continue;
+            } else if (!only_used_by(div_n->outputs[0], {&m2})) {
+                continue;
+            }
+            Node f;
+            f.op = "rmlk.RMSNorm";
+            f.inputs = {x, gamma};
+            f.outputs = m2.outputs;
+            f.attrs["epsilon"] = a_float(eps);
+            f.attrs["reciprocal"] = a_int(recip ? 1 : 0);
+            f.attrs["axis"] = a_int(axis);
+            std::vector<const Node *> parts = {pow_n, mean_n, add_n, sqrt_n, div_n, &m2};
+            if (mul_n) parts.push_back(mul_n);
+            replace(parts, std::move(f));
+            return true;
+        }
+        return false;
+    }
+
+    // ---- SwiGLU, anchored at the outer Mul -------------------------------------------------------
+    bool match_swiglu(const Node &m2) {
+        if (m2.op != "Mul" || m2.inputs.size() != 2) return false;
+        for (int side = 0; side < 2; ++side) {
+            const int silu = m2.inputs[side], up = m2.inputs[1 - side];
+            const Node *m1 = produced_by(silu, "Mul");
+            if (!m1 || m1->inputs.size() != 2 || up < 0) continue;
+            for (int k = 0; k < 2; ++k) {
+                const Node *sg = produced_by(m1->inputs[k], "Sigmoid");
+                const int gate = m1->inputs[1 - k];
+                if (!sg || sg->inputs[0] != gate) continue;
+                if (!only_used_by(sg->outputs[0], {m1}) || !only_used_by(m1->outputs[0], {&m2}))
+                    continue;
+                Node f;
+                f.op = "rmlk.SwiGLU";
+                f.inputs = {gate, up};
+                f.outputs = m2.outputs;
+                replace({sg, m1, &m2}, std::move(f));
+                return true;
+            }
+        }
+        return false;
+    }
+
+    // ---- scale + mask + softmax, anchored at Softmax ----------------------------------------------
+    bool match_softmax(const Node &sm) {
+        if (sm.op != "Softmax" || sm.inputs.size() != 1) return false;
+        const Node *add_n = produced_by(sm.inputs[0], "Add");
+        if (!add_n || add_n->inputs.size() != 2) return false;
+        for (int side = 0; side < 2; ++side) {
+            const int scaled = add_n->inputs[side], mask = add_n->inputs[1 - side];
+            if (mask < 0) continue;
+            const Node *sc = produced_by(scaled, "Div");
+            bool is_mul = false;
+            int x = -1;
+            float c = 0.f;
+            if (sc) {
+                if (sc->inputs.size() != 2 || !const_float(sc->inputs[1], &c)) continue;
+                x = sc->inputs[0];
+            } else if ((sc = produced_by(scaled, "Mul"))) {
+                if (sc->inputs.size() != 2) continue;
+                if (const_float(sc->inputs[1], &c)) x = sc->inputs[0];
+                else if (const_float(sc->inputs[0], &c)) x = sc->inputs[1];
+                else continue;
+                is_mul = true;
+            } else {
+                continue;
+            }
+            if (x < 0) continue;
+            if (!only_used_by(sc->outputs[0], {add_n}) || !only_used_by(add_n->outputs[0], {&sm}))
+                continue;
+            Node f;
+            f.op = "rmlk.ScaleMaskSoftmax";
+            f.inputs = {x, mask};
+            f.outputs = sm.outputs;
+            f.attrs["scale"] = a_float(c);
+            f.attrs["scale_is_mul"] = a_int(is_mul ? 1 : 0);
+            f.attrs["axis"] = a_int(attr_int(sm, "axis", -1));
+            replace({sc, add_n, &sm}, std::move(f));
+            return true;
+        }
+        return false;
+    }
+
+    // one-element constant input `i` of a Slice
+    bool slice_param(const Node &sl, size_t i, int64_t *out) const {
+        std::vector<int64_t> v;
+        if (sl.inputs.size() <= i || !const_ints(sl.inputs[i], &v) || v.size() != 1) return false;
+        *out = v[0];
+        return true;
+    }
+
+    // ---- rotary embedding, anchored at the final Add ---------------------------------------------
+    bool match_rotary(const Node &add) {
+        if (add.op != "Add" || add.inputs.size() != 2) return false;
+        for (int side = 0; side < 2; ++side) {
+            const Node *ma = produced_by(add.inputs[side], "Mul");       // x * cos
+            const Node *mr = produced_by(add.inputs[1 - side], "Mul");   // rotate_half(x) * sin
+            if (!ma || !mr || ma == mr || ma->inputs.size() != 2 || mr->inputs.size() != 2) continue;
+            for (int k = 0; k < 2; ++k) {
+                const Node *cat = produced_by(mr->inputs[k], "Concat");
+                const int sin_v = mr->inputs[1 - k];
+                if (!cat || cat->inputs.size() != 2 || sin_v < 0) continue;
+                const Node *neg = produced_by(cat->inputs[0], "Neg");
+                const Node *s1 = produced_by(cat->inputs[1], "Slice");
+                if (!neg || !s1) continue;
+                const Node *s2 = produced_by(neg->inputs[0], "Slice");
+                if (!s2 || s1 == s2) continue;
+                const int x = s1->inputs[0];
+                if (x < 0 || s2->inputs[0] != x) continue;
+                int cos_v = -1;
+                if (ma->inputs[0] == x) cos_v = ma->inputs[1];
+                else if (ma->inputs[1] == x) cos_v = ma->inputs[0];
+                if (cos_v < 0 || cos_v == x) continue;
+                // Slice(x, [0], [h], [ax]) and Slice(x, [h], [>= 2h], [ax]), unit steps
+                int64_t b1, e1, a1, b2, e2, a2, st;
+                if (!slice_param(*s1, 1, &b1) || !slice_param(*s1, 2, &e1) ||
+                    !slice_param(*s1, 3, &a1) || !slice_param(*s2, 1, &b2) ||
+                    !slice_param(*s2, 2, &e2) || !slice_param(*s2, 3, &a2))
+                    continue;
+                if (s1->inputs.size() > 4 && s1->inputs[4] >= 0 &&
+                    (!slice_param(*s1, 4, &st) || st != 1))
+                    continue;
+                if (s2->inputs.size() > 4 && s2->inputs[4] >= 0 &&
+                    (!slice_param(*s2, 4, &st) || st != 1))
+                    continue;
+                if (b1 != 0 || e1 <= 0 || b2 != e1 || e2 < 2 * e1 || a1 != a2) continue;
+                const int64_t cat_axis = attr_int(*cat, "axis", 0);
+                if (!only_used_by(s1->outputs[0], {cat}) || !only_used_by(s2->outputs[0], {neg}) ||
+                    !only_used_by(neg->outputs[0], {cat}) || !only_used_by(cat->outputs[0], {mr}) ||
+                    !only_used_by(ma->outputs[0], {&add}) || !only_used_by(mr->outputs[0], {&add}))
+                    continue;
+                std::vector<const Node *> parts = {s1, s2, neg, cat, ma, mr, &add};
+                int src = x;
+                int64_t pre = 0;
+                // a head-split Transpose feeding only this pattern is read through strides instead
+                if (const Node *tr = produced_by(x, "Transpose")) {
+                    auto it = tr->attrs.find("perm");
+                    const std::vector<int64_t> want = {0, 2, 1, 3};
+                    if (it != tr->attrs.end() && it->second.ints == want &&
+                        only_used_by(x, {s1, s2, ma})) {
+                        parts.push_back(tr);
+                        src = tr->inputs[0];
+                        pre = 1;
+                    }
+                }
+                Node f;
+                f.op = "rmlk.Rotary";
+                f.inputs = {src, cos_v, sin_v};
+                f.outputs = add.outputs;
+                f.attrs["half"] = a_int(e1);
+                f.attrs["end"] = a_int(e2);
+                f.attrs["slice_axis"] = a_int(a1);
+                f.attrs["concat_axis"] = a_int(cat_axis);
+                f.attrs["transposed_input"] = a_int(pre);
+                replace(parts, std::move(f));
+                return true;
+            }
+        }
+        return false;
+    }
+};
+
+// Run the nodes a fused node replaced, one kernel each.
+void run_body(OpContext &c) {
+    Session &s = c.session;
+    std::unordered_map<int, Tensor> local;
+    auto lookup = [&](int v) -> Tensor * {
+        auto it = local.find(v);
+        return it != local.end() ? &it->second : &s.values[v];
+    };
+    for (const Node &n : c.node.body) {
+        OpContext sub{s, n, c.node_index, {}, {}, c.stream};
+        for (int v : n.inputs) sub.in.push_back(v < 0 ? nullptr : lookup(v));
+        std::vector<Tensor> outs(n.outputs.size());
+        for (size_t o = 0; o < outs.size(); ++o) sub.out.push_back(&outs[o]);
+        find_op(n.op)(sub);
+        for (size_t o = 0; o < outs.size(); ++o) local[n.outputs[o]] = outs[o];
+    }
+    for (size_t o = 0; o < c.node.outputs.size(); ++o) *c.out[o] = local[c.node.outputs[o]];
+}
+
+float attr_float(const OpContext &c, const char *name) {
+    const Attr *a = c.attr(name);
+    return a ? a->f : 0.f;
+}
+
+// status of a fused kernel: UNSUPPORTED means "not this layout", anything else is an error
+bool took_fast_path(int32_t st, const char *what) {
+    if (st == RMLK_ERR_UNSUPPORTED) return false;
+    check_status(st, what);
+    return true;
+}
+
+}  // namespace
+
+void op_fused_rmsnorm(OpContext &c) {
+    const Tensor &x = c.input(0), &gamma = c.input(1);
+    const int rank = x.rank();
+    bool ok = x.dtype == RMLK_FLOAT && gamma.dtype == RMLK_FLOAT && rank >= 1 && x.numel() > 0;
+    if (ok) {
+        const int64_t axis = c.attr_int("axis", -1);
+        ok = axis == -1 || axis == rank - 1;
+    }
+    if (ok) {
+        // gamma broadcasts along the rows only: [cols] or [1, .., 1, cols]
+        ok = gamma.rank() >= 1 && gamma.rank() <= rank && gamma.shape.back() == x.shape.back() &&
+             gamma.numel() == x.shape.back();
+    }
+    if (ok) {
+        const int64_t cols = x.shape.back(), rows = x.numel() / cols;
+        Tensor &y = c.alloc_output(0, RMLK_FLOAT, x.shape);
+        if (took_fast_path(rmlk_hip_rmsnorm(c.stream, RMLK_FLOAT, rows, cols, x.data(), gamma.data(),
+                                            attr_float(c, "epsilon"),
+                                            static_cast<int32_t>(c.attr_int("reciprocal", 0)),
+                                            y.data()),
+                           "rmlk.RMSNorm"))
+            return;
+    }
+    run_body(c);
+}
+
+void op_fused_swiglu(OpContext &c) {
+    const Tensor &g = c.input(0), &u = c.input(1);
+    if (g.dtype == RMLK_FLOAT && u.dtype == RMLK_FLOAT && g.shape == u.shape) {
+        Tensor &y = c.alloc_output(0, RMLK_FLOAT, g.shape);
+        if (took_fast_path(rmlk_hip_swiglu(c.stream, RMLK_FLOAT, g.numel(), g.data(), u.data(),
+                                           y.data()),
+                           "rmlk.SwiGLU"))
+            return;
+    }
+    run_body(c);
+}
+
+void op_fused_softmax(OpContext &c) {
+    const Tensor &x = c.input(0), &mask = c.input(1);
+    const int rank = x.rank();
+    bool ok = x.dtype == RMLK_FLOAT && mask.dtype == RMLK_FLOAT && rank >= 1 &&
+              mask.rank() <= rank && x.numel() > 0;
+    if (ok) {
+        const int64_t axis = c.attr_int("axis", -1);
+        ok = axis == -1 || axis == rank - 1;
+    }
+    rmlk_dims ms{};
+    if (ok) {
+        // the mask must broadcast INTO x's shape, with a full last dim
+        std::vector<int64_t> st(rank, 0), dense = dense_strides(mask.shape);
+        const int shift = rank - mask.rank();
+        for (int d = 0; d < mask.rank() && ok; ++d) {
+            const int64_t md = mask.shape[d], xd = x.shape[d + shift];
+            if (md == xd) st[d + shift] = md == 1 ? 0 : dense[d];
+            else if (md == 1) st[d + shift] = 0;
+            else ok = false;
+        }
+        if (ok && (mask.rank() == 0 || mask.shape.back() != x.shape.back())) ok = false;
+        if (ok) {
+            st[rank - 1] = 1;
+            ms = to_dims(st);
+        }
+    }
+    if (ok) {
+        rmlk_dims xs = to_dims(x.shape);
+        Tensor &y = c.alloc_output(0, RMLK_FLOAT, x.shape);
+        if (took_fast_path(rmlk_hip_scale_mask_softmax(
+                               c.stream, RMLK_FLOAT, &xs, &ms,
+                               static_cast<int32_t>(c.attr_int("scale_is_mul", 0)),
+                               attr_float(c, "scale"), x.data(), mask.data(), y.data()),
+                           "rmlk.ScaleMaskSoftmax"))
+            return;
+    }
+    run_body(c);
+}
+
+void op_fused_rotary(OpContext &c) {
+    const Tensor &src = c.input(0), &cos_t = c.input(1), &sin_t = c.input(2);
+    const bool pre = c.attr_int("transposed_input", 0) != 0;
+    bool ok = src.dtype == RMLK_FLOAT && cos_t.dtype == RMLK_FLOAT && sin_t.dtype == RMLK_FLOAT &&
+              src.rank() == 4 && cos_t.rank() <= 4 && sin_t.rank() <= 4 && src.numel() > 0;
+    std::vector<int64_t> shape, xst;
+    if (ok) {
+        std::vector<int64_t> dense = dense_strides(src.shape);
+        if (pre) {  // logical x = Transpose(src, 0,2,1,3)
+            shape = {src.shape[0], src.shape[2], src.shape[1], src.shape[3]};
+            xst = {dense[0], dense[2], dense[1], dense[3]};
+        } else {
+            shape = src.shape;
+            xst = dense;
+        }
+        const int64_t d = shape[3], half = c.attr_int("half", 0);
+        auto axis_ok = [](int64_t a) { return a == 3 || a == -1; };
+        ok = d == 2 * half && c.attr_int("end", 0) >= d && axis_ok(c.attr_int("slice_axis", 0)) &&
+             axis_ok(c.attr_int("concat_axis", 0));
+    }
+    auto table_strides = [&](const Tensor &t, rmlk_dims *out) {
+        // broadcast INTO `shape`, last dim full
+        std::vector<int64_t> st(4, 0), dense = dense_strides(t.shape);
+        const int shift = 4 - t.rank();
+        for (int d = 0; d < t.rank(); ++d) {
+            const int64_t td = t.shape[d], xd = shape[d + shift];
+            if (td == xd) st[d + shift] = td == 1 ? 0 : dense[d];
+            else if (td != 1) return false;
+        }
+        if (t.rank() == 0 || t.shape.back() != shape[3]) return false;
+        st[3] = 1;
+        *out = to_dims(st);
+        return true;
+    };
+    rmlk_dims cs{}, ss{};
+    if (ok) ok = table_strides(cos_t, &cs) && table_strides(sin_t, &ss);
+    if (ok) {
+        rmlk_dims sd = to_dims(shape), xs = to_dims(xst);
+        Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
+        if (took_fast_path(rmlk_hip_rotary(c.stream, RMLK_FLOAT, &sd, &xs, &cs, &ss, src.data(),
+                                           cos_t.data(), sin_t.data(), y.data()),
+                           "rmlk.Rotary"))
+            return;
+    }
+    run_body(c);
+}
+
+// Rewrite the session's node list; returns how many fused nodes were formed.
+int fuse_patterns(Session &s) {
+    Matcher m(s);
+    int formed = 0;
+    for (size_t n = 0; n < m.g.nodes.size(); ++n) {
+        if (m.removed[n]) continue;
+        // the node object may be overwritten by replace(): match on a copy of its header
+        const Node &node = m.g.nodes[n];
+        if (node.op == "Mul") {
+            if (m.match_rmsnorm(node) || m.match_swiglu(node)) ++formed;
+        } else if (node.op == "Softmax") {
+            if (m.match_softmax(node)) ++formed;
+        } else if (node.op == "Add") {
+            if (m.match_rotary(node)) ++formed;
+        }
+    }
+    if (!formed) return 0;
+    std::vector<Node> kept;
+    kept.reserve(m.g.nodes.size());
+    for (size_t n = 0; n < m.g.nodes.size(); ++n)
+        if (!m.removed[n]) kept.push_back(std::move(m.g.nodes[n]));
+    m.g.nodes = std::move(kept);
+    for (Value &v : m.g.values) v.producer = -1;
+    for (size_t n = 0; n < m.g.nodes.size(); ++n)
+        for (int v : m.g.nodes[n].outputs) m.g.values[v].producer = static_cast<int>(n);
+    return formed;
+}
+
+}  // namespace rt
+}  // namespace rmlk

@@ -823,6 +823,10 @@ const std::unordered_map<std::string, OpFn> &registry() {
         {"Shape", op_shape},     {"Range", op_range},
         {"ConstantOfShape", op_constant_of_shape},
         {"Constant", op_constant},
+        {"rmlk.RMSNorm", op_fused_rmsnorm},
+        {"rmlk.SwiGLU", op_fused_swiglu},
+        {"rmlk.ScaleMaskSoftmax", op_fused_softmax},
+        {"rmlk.Rotary", op_fused_rotary},
     };
     return table;
 }

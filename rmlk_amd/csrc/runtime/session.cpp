@@ -290,11 +290,9 @@ void Session::build(const rmlk_graph &graph, int dev) {
     *err_host = 0;
     if (g->outputs.empty()) throw RtError(RMLK_ERR_GRAPH, "graph has no outputs");
     values.assign(g->values.size(), Tensor());
-    last_use.assign(g->values.size(), -1);
-    stats.assign(g->nodes.size(), NodeStat());
     for (size_t n = 0; n < g->nodes.size(); ++n) {
         const Node &node = g->nodes[n];
-        if (!find_op(node.op))
+        if (!find_op(node.op) || node.op.rfind("rmlk.", 0) == 0)
             throw RtError(RMLK_ERR_OP, "unsupported operator `" + node.op + "`");
         for (int v : node.inputs) {
             if (v < 0) continue;
@@ -303,7 +301,6 @@ void Session::build(const rmlk_graph &graph, int dev) {
                 throw RtError(RMLK_ERR_GRAPH, "node " + std::to_string(n) + " (" + node.op +
                                                   ") reads `" + val.name +
                                                   "` before anything produces it");
-            last_use[v] = static_cast<int>(n);
         }
     }
     for (int o : g->outputs) {
@@ -351,6 +348,13 @@ void Session::build(const rmlk_graph &graph, int dev) {
         values[node.outputs[0]] = upload_initializer(ht, stream);
     }
     check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+    if (fuse) fused_nodes = fuse_patterns(*this);
+    // liveness over the final node list
+    last_use.assign(g->values.size(), -1);
+    stats.assign(g->nodes.size(), NodeStat());
+    for (size_t n = 0; n < g->nodes.size(); ++n)
+        for (int v : g->nodes[n].inputs)
+            if (v >= 0) last_use[v] = static_cast<int>(n);
 }
 
 void Session::run_nodes() {

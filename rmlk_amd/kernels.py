@@ -110,7 +110,7 @@ def matmul(a, b, c, batch, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c,
     """ref: cuda/src/kernels/gemm.rs:112-136 (compute with a StridedBatchedConfig)."""
     need = matmul_workspace_size(batch, m, n, k, dtype_of(a))
     if workspace is None and need:
-        workspace = torch.zeros(need, dtype=torch.uint8, device=a.device)  # counters start at 0
+        workspace = torch.empty(need, dtype=torch.uint8, device=a.device)
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
     st = lib().rmlk_hip_matmul(_stream(), dtype_of(a), batch, m, n, k, _ptr(a), lda, stride_a,
                                int(trans_a), _ptr(b), ldb, stride_b, int(trans_b), _ptr(c), ldc,
@@ -165,6 +165,35 @@ def trilu(x, out, batch: int, rows: int, cols: int, upper: bool, k: int) -> None
     assert x.numel() == out.numel() == batch * rows * cols
     check(lib().rmlk_hip_trilu(_stream(), dtype_of(x), batch, rows, cols, int(upper), k, _ptr(x),
                                _ptr(out)), "rmlk_hip_trilu")
+
+
+def rmsnorm(x, gamma, out, rows: int, cols: int, eps: float, reciprocal_form: bool = False) -> None:
+    """Fused Pow(2) -> ReduceMean(-1) -> Add(eps) -> Sqrt -> Div -> Mul(gamma)."""
+    assert x.numel() == out.numel() == rows * cols and gamma.numel() == cols
+    check(lib().rmlk_hip_rmsnorm(_stream(), dtype_of(x), rows, cols, _ptr(x), _ptr(gamma),
+                                 float(eps), int(reciprocal_form), _ptr(out)), "rmlk_hip_rmsnorm")
+
+
+def scale_mask_softmax(x, mask, out, shape, mask_stride, scale: float, scale_is_mul=False) -> None:
+    """Fused Div|Mul(x, scale) -> Add(mask) -> Softmax(axis -1)."""
+    check(lib().rmlk_hip_scale_mask_softmax(_stream(), dtype_of(x), Dims.of(shape),
+                                            Dims.of(mask_stride), int(scale_is_mul), float(scale),
+                                            _ptr(x), _ptr(mask), _ptr(out)),
+          "rmlk_hip_scale_mask_softmax")
+
+
+def swiglu(gate, up, out) -> None:
+    """Fused Sigmoid -> Mul -> Mul: (gate * sigmoid(gate)) * up."""
+    assert gate.numel() == up.numel() == out.numel()
+    check(lib().rmlk_hip_swiglu(_stream(), dtype_of(gate), gate.numel(), _ptr(gate), _ptr(up),
+                                _ptr(out)), "rmlk_hip_swiglu")
+
+
+def rotary(x, cos, sin, out, shape, x_stride, cos_stride, sin_stride) -> None:
+    """Fused half-rotation rotary embedding over a strided [B,H,S,D] view of x."""
+    check(lib().rmlk_hip_rotary(_stream(), dtype_of(x), Dims.of(shape), Dims.of(x_stride),
+                                Dims.of(cos_stride), Dims.of(sin_stride), _ptr(x), _ptr(cos),
+                                _ptr(sin), _ptr(out)), "rmlk_hip_rotary")
 
 
 def device_info(device: int = 0) -> dict:

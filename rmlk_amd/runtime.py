@@ -179,12 +179,17 @@ class GraphBuilder:
 class ModelInstance:
     """ref: runtime/src/core/instance.rs:20-119"""
 
-    def __init__(self, graph: Graph, device: int = 0):
+    def __init__(self, graph: Graph, device: int = 0, fuse: bool = True):
         self.graph = graph
         h = ctypes.c_void_p()
-        _check(lib().rmlk_session_create(graph.handle, device, ctypes.byref(h)),
+        _check(lib().rmlk_session_create_ex(graph.handle, device, 0 if fuse else 1, ctypes.byref(h)),
                "Builder.build")
         self._h = h
+
+    @property
+    def fused_nodes(self) -> int:
+        """Fused nodes formed while building (0 with fuse=False)."""
+        return int(lib().rmlk_session_fused_nodes(self._h))
 
     # -- inputs -------------------------------------------------------------------------------
     def set_input(self, name: str, array) -> None:
@@ -291,5 +296,6 @@ class Builder:
     def from_graph(graph: Graph) -> "Builder":
         return Builder(graph)
 
-    def build(self, device: int = 0) -> ModelInstance:
-        return ModelInstance(self._graph, device)
+    def build(self, device: int = 0, fuse: bool = True) -> ModelInstance:
+        """fuse=False keeps one kernel per node, as the reference executes a graph."""
+        return ModelInstance(self._graph, device, fuse)

@@ -1,0 +1,372 @@
+"""Fused kernels and the pattern-fusion pass, on the GPU.
+
+The reference has no fused kernels: it runs one kernel per ONNX node. The bar here is therefore the
+un-fused path itself — a fused kernel must give the BITS of the chain of separate kernels it
+replaces (RMSNorm: the row mean is a double-precision sum taken in a different order, so a result
+may differ in the last place on rare rows; the test allows 2 ulp there and requires 99.9 % of the
+elements to be identical) — plus the CPU oracle at the per-op tolerance (rtol 1e-4 / atol 1e-5).
+Session tests build every graph twice (fused / one kernel per node) and compare outputs."""
+import numpy as np
+import pytest
+
+from helpers import assert_close, assert_exact, bcast_strides, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _k():
+    from rmlk_amd import kernels
+    return kernels
+
+
+def _dense(shape):
+    return bcast_strides(shape, shape)
+
+
+# ---- kernel level: fused kernel vs the chain of separate kernels through the C ABI --------------
+
+@pytest.mark.parametrize("rows,cols", [(1, 2048), (7, 64), (512, 2048), (1500, 256), (3, 8192),
+                                       (2048, 1024), (5, 4)])
+@pytest.mark.parametrize("recip", [False, True])
+def test_rmsnorm_matches_separate_kernels(device, rows, cols, recip):
+    import torch
+    k = _k()
+    rng = np.random.default_rng(rows * 31 + cols)
+    x = to_dev(rng.standard_normal((rows, cols), dtype=np.float32) * 3, device)
+    gamma = to_dev(rng.uniform(0.5, 1.5, size=(cols,)).astype(np.float32), device)
+    eps = 1e-5
+    # separate kernels: Pow, ReduceMean, Add, Sqrt, Div (or Div(1, .) and Mul), Mul
+    two = torch.tensor([2.0], device=device)
+    epst = torch.tensor([eps], dtype=torch.float32, device=device)
+    one = torch.tensor([1.0], device=device)
+    sq = torch.empty_like(x)
+    k.binary(k.POW, x, two, sq, [rows, cols], [cols, 1], [0, 0])
+    mean = torch.empty(rows, device=device)
+    k.reduce_mean(sq, mean, [rows, cols], [1])
+    var = torch.empty_like(mean)
+    k.binary(k.ADD, mean, epst, var, [rows], [1], [0])
+    r = torch.empty_like(mean)
+    k.unary(k.SQRT, var, r)
+    normed = torch.empty_like(x)
+    if recip:
+        inv = torch.empty_like(r)
+        k.binary(k.DIV, one, r, inv, [rows], [0], [1])
+        k.binary(k.MUL, x, inv, normed, [rows, cols], [cols, 1], [1, 0])
+    else:
+        k.binary(k.DIV, x, r, normed, [rows, cols], [cols, 1], [1, 0])
+    exp = torch.empty_like(x)
+    k.binary(k.MUL, normed, gamma, exp, [rows, cols], [cols, 1], [0, 1])
+    got = torch.empty_like(x)
+    k.rmsnorm(x, gamma, got, rows, cols, eps, recip)
+    g, e = to_np(got), to_np(exp)
+    same = np.mean(g.view(np.uint32) == e.view(np.uint32))
+    assert same >= 0.999, same
+    np.testing.assert_allclose(g, e, rtol=3e-7, atol=0)
+    # oracle
+    xn = to_np(x).astype(np.float64)
+    ref = xn / np.sqrt((xn * xn).mean(-1, keepdims=True) + eps) * to_np(gamma)
+    assert_close(g, ref.astype(np.float32), rtol=1e-4, atol=1e-5)
+
+
+def test_rmsnorm_rejects_layouts_it_does_not_cover(device):
+    import torch
+    from rmlk_amd import RmlkError
+    k = _k()
+    x = torch.ones(2, 6, device=device)
+    with pytest.raises(RmlkError):
+        k.rmsnorm(x, torch.ones(6, device=device), torch.empty_like(x), 2, 6, 1e-5)
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 8192, 512 * 8192, 1000003])
+def test_swiglu_matches_separate_kernels(device, n):
+    import torch
+    k = _k()
+    rng = np.random.default_rng(n)
+    g = to_dev(rng.standard_normal(n, dtype=np.float32) * 4, device)
+    u = to_dev(rng.standard_normal(n, dtype=np.float32), device)
+    sig, silu, exp, got = (torch.empty_like(g) for _ in range(4))
+    k.unary(k.SIGMOID, g, sig)
+    k.binary(k.MUL, g, sig, silu, [n], [1], [1])
+    k.binary(k.MUL, silu, u, exp, [n], [1], [1])
+    k.swiglu(g, u, got)
+    assert_exact(to_np(got), to_np(exp))
+    gn = to_np(g).astype(np.float64)
+    ref = gn / (1 + np.exp(-gn)) * to_np(u)
+    assert_close(to_np(got), ref.astype(np.float32), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("shape,mask_shape,mul", [
+    ([1, 32, 512, 640], [1, 1, 512, 640], False),
+    ([1, 32, 1, 640], [1, 1, 1, 640], False),
+    ([2, 4, 16, 128], [2, 1, 16, 128], True),
+    ([2, 4, 16, 128], [128], False),
+    ([3, 5000], [3, 5000], False),
+    ([2, 3, 4, 8], [3, 1, 8], True),
+    ([2, 3, 4, 5, 8], [1, 1, 4, 5, 8], True),
+])
+def test_scale_mask_softmax_matches_separate_kernels(device, shape, mask_shape, mul):
+    import torch
+    k = _k()
+    rng = np.random.default_rng(sum(shape))
+    x = to_dev(rng.standard_normal(shape, dtype=np.float32) * 5, device)
+    mask_np = np.where(rng.random(mask_shape) < 0.3, -np.inf, 0.0).astype(np.float32)
+    mask_np[..., 0] = 0.0   # no fully masked row
+    mask = to_dev(mask_np, device)
+    scale = 0.125 if mul else 8.0
+    st = torch.tensor([scale], device=device)
+    n = x.numel()
+    scaled, masked, exp, got = (torch.empty_like(x) for _ in range(4))
+    zeros = [0] * len(shape)
+    k.binary(k.MUL if mul else k.DIV, x, st, scaled, shape, _dense(shape), zeros)
+    ms = bcast_strides(mask_shape, shape)
+    k.binary(k.ADD, scaled, mask, masked, shape, _dense(shape), ms)
+    k.softmax(masked, exp, n // shape[-1], shape[-1], 1)
+    ms_fused = list(ms)
+    ms_fused[-1] = 1
+    k.scale_mask_softmax(x, mask, got, shape, ms_fused, scale, mul)
+    assert_exact(to_np(got), to_np(exp))
+    xn = to_np(x).astype(np.float64)
+    z = (xn * scale if mul else xn / scale) + mask_np
+    z = z - z.max(-1, keepdims=True)
+    ref = np.exp(z) / np.exp(z).sum(-1, keepdims=True)
+    assert_close(to_np(got), ref.astype(np.float32), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("b,h,s,d,transposed", [
+    (1, 32, 512, 64, True), (1, 8, 1, 64, True), (1, 8, 1, 64, False), (2, 3, 5, 8, False),
+    (2, 3, 5, 6, True), (1, 2, 7, 2, False), (1, 4, 9, 128, True),
+])
+def test_rotary_matches_separate_kernels(device, b, h, s, d, transposed):
+    import torch
+    k = _k()
+    rng = np.random.default_rng(b + h + s + d)
+    shape = [b, h, s, d]
+    half = d // 2
+    if transposed:   # storage [B,S,H,D], logical x = Transpose(0,2,1,3)
+        store = to_dev(rng.standard_normal((b, s, h, d), dtype=np.float32), device)
+        x = torch.empty(b * h * s * d, device=device)
+        k.transpose(store, x, [b, s, h, d], [0, 2, 1, 3])
+        x_stride = [s * h * d, d, h * d, 1]
+        src = store
+    else:
+        x = to_dev(rng.standard_normal(shape, dtype=np.float32), device).reshape(-1)
+        x_stride = _dense(shape)
+        src = x
+    cos = to_dev(rng.uniform(-1, 1, size=(1, 1, s, d)).astype(np.float32), device)
+    sin = to_dev(rng.uniform(-1, 1, size=(1, 1, s, d)).astype(np.float32), device)
+    cs = bcast_strides([1, 1, s, d], shape)
+    cs[-1] = 1
+    n = b * h * s * d
+    hs = [b, h, s, half]
+    x1, x2, neg = (torch.empty(n // 2, device=device) for _ in range(3))
+    k.slice_(x, x1, shape, [0, 0, 0, 0], [1, 1, 1, 1], hs)
+    k.slice_(x, x2, shape, [0, 0, 0, half], [1, 1, 1, 1], hs)
+    k.unary(k.NEG, x2, neg)
+    rot, a, r, exp, got = (torch.empty(n, device=device) for _ in range(5))
+    k.concat_into(neg, rot, hs, shape, 3, 0)
+    k.concat_into(x1, rot, hs, shape, 3, half)
+    bc = bcast_strides([1, 1, s, d], shape)
+    k.binary(k.MUL, x, cos, a, shape, _dense(shape), bc)
+    k.binary(k.MUL, rot, sin, r, shape, _dense(shape), bc)
+    k.binary(k.ADD, a, r, exp, shape, _dense(shape), _dense(shape))
+    k.rotary(src, cos, sin, got, shape, x_stride, cs, cs)
+    assert_exact(to_np(got), to_np(exp))
+
+
+# ---- session level: the fusion pass ------------------------------------------------------------
+
+def _run_both(graph, feeds, outputs=None):
+    from rmlk_amd import runtime
+    fused = runtime.Builder.from_graph(graph).build(fuse=True)
+    plain = runtime.Builder.from_graph(graph).build(fuse=False)
+    assert plain.fused_nodes == 0
+    a, b = fused.run(feeds), plain.run(feeds)
+    n = fused.fused_nodes
+    ops = [d["op"] for d in fused.node_stats()] if hasattr(fused, "node_stats") else []
+    fused.close()
+    plain.close()
+    return a, b, n, ops
+
+
+def _same(a, b, loose=()):
+    assert a.keys() == b.keys()
+    for name in a:
+        if a[name].dtype.kind == "f" and name in loose:
+            np.testing.assert_allclose(a[name], b[name], rtol=2e-6, atol=1e-7)
+        else:
+            assert_exact(a[name], b[name])
+
+
+def test_pass_forms_the_expected_nodes_on_the_llama_graph(device):
+    from rmlk_amd import graphs
+    cfg = graphs.LlamaConfig.tiny()
+    graph = graphs.llama_graph(cfg, seed=4, style="scatter", max_len=24)
+    rng = np.random.default_rng(0)
+    s = 8
+    feeds = {"input_ids": rng.integers(0, cfg.vocab, size=(1, s)),
+             "position_ids": np.arange(s, dtype=np.int64).reshape(1, s)}
+    for l in range(cfg.layers):
+        for kv in ("key", "value"):
+            feeds[f"cache.{l}.{kv}"] = np.zeros((1, cfg.kv_heads, 24, cfg.head_dim), np.float32)
+    a, b, n, _ = _run_both(graph, feeds)
+    # per layer: 2 RMSNorm, 2 rotary, 1 SwiGLU, 1 softmax; plus the final RMSNorm
+    assert n == cfg.layers * 6 + 1
+    # RMSNorm's mean may differ in the last place; everything downstream inherits that
+    _same(a, b, loose=set(a.keys()))
+    assert np.array_equal(np.argmax(a["logits"][0], -1), np.argmax(b["logits"][0], -1))
+
+
+def test_fused_llama_concat_style_against_oracle(device):
+    from oracle import graph as og
+    from rmlk_amd import graphs, runtime
+    cfg = graphs.LlamaConfig.tiny()
+    graph = graphs.llama_graph(cfg, seed=4, style="concat")
+    feeds = graphs.llama_concat_inputs(cfg, np.random.default_rng(1).integers(0, cfg.vocab, 9), None, 0)
+    inst = runtime.Builder.from_graph(graph).build()
+    assert inst.fused_nodes == cfg.layers * 6 + 1
+    got = inst.run(feeds)
+    exp = og.run_graph(graph, feeds)
+    for name in exp:
+        assert_close(got[name], exp[name], rtol=1e-3, atol=1e-4)
+    inst.close()
+
+
+def test_fused_decoder_layer_full_width(device):
+    from rmlk_amd import graphs
+    graph, feeds = graphs.decoder_layer_graph(seed=3, seq=96)
+    a, b, n, _ = _run_both(graph, feeds)
+    assert n == 6
+    _same(a, b, loose={"y"})
+
+
+def test_capture_and_replay_with_fused_nodes(device):
+    from rmlk_amd import graphs, runtime
+    graph, feeds = graphs.decoder_layer_graph(seed=3, seq=32)
+    inst = runtime.Builder.from_graph(graph).build()
+    eager = inst.run(feeds)["y"].copy()
+    for name, arr in feeds.items():
+        inst.set_input(name, arr)
+    inst.execute()
+    inst.capture()
+    for _ in range(3):
+        inst.replay()
+        inst.sync()
+        assert_exact(inst.output("y"), eager)
+    inst.close()
+
+
+def _builder():
+    from rmlk_amd import runtime
+    return runtime.GraphBuilder()
+
+
+def _rmsnorm_nodes(g, x, gamma, out, recip=False, axis=-1, expose_mean=False):
+    g.constant("two", np.array(2.0, np.float32))
+    g.constant("eps", np.array(1e-5, np.float32))
+    g.op("Pow", [x, "two"], ["sq"])
+    g.op("ReduceMean", ["sq"], ["mean"]).attr("axes", [axis]).attr("keepdims", 1)
+    g.op("Add", ["mean", "eps"], ["var"])
+    g.op("Sqrt", ["var"], ["rms"])
+    if recip:
+        g.constant("one", np.array(1.0, np.float32))
+        g.op("Div", ["one", "rms"], ["inv"])
+        g.op("Mul", [x, "inv"], ["normed"])
+    else:
+        g.op("Div", [x, "rms"], ["normed"])
+    g.op("Mul", [gamma, "normed"], [out])
+    g.output(out)
+    if expose_mean:
+        g.output("mean")
+
+
+@pytest.mark.parametrize("shape,recip,n_fused", [
+    ([2, 5, 64], False, 1), ([2, 5, 64], True, 1),
+    ([3, 6], False, 1),            # cols % 4 != 0: the node is formed, its body runs
+    ([4, 16384], False, 1),        # row longer than the fused kernel holds: body runs
+])
+def test_rmsnorm_pattern_variants_and_fallback(device, shape, recip, n_fused):
+    from oracle import graph as og
+    g = _builder()
+    g.input("x", np.float32, shape)
+    rng = np.random.default_rng(len(shape))
+    g.constant("gamma", rng.uniform(0.5, 1.5, size=(shape[-1],)).astype(np.float32))
+    _rmsnorm_nodes(g, "x", "gamma", "y", recip)
+    graph = g.build()
+    feeds = {"x": rng.standard_normal(shape, dtype=np.float32)}
+    a, b, n, _ = _run_both(graph, feeds)
+    assert n == n_fused
+    _same(a, b, loose={"y"})
+    assert_close(a["y"], og.run_graph(graph, feeds)["y"], rtol=1e-4, atol=1e-5)
+
+
+def test_rmsnorm_over_a_middle_axis_runs_the_body(device):
+    g = _builder()
+    g.input("x", np.float32, [2, 8, 4])
+    g.constant("gamma", np.ones((4,), np.float32))
+    _rmsnorm_nodes(g, "x", "gamma", "y", axis=1)
+    feeds = {"x": np.random.default_rng(3).standard_normal((2, 8, 4), dtype=np.float32)}
+    a, b, n, _ = _run_both(g.build(), feeds)
+    assert n == 1
+    _same(a, b)
+
+
+def test_intermediate_that_is_a_graph_output_blocks_fusion(device):
+    g = _builder()
+    g.input("x", np.float32, [2, 64])
+    g.constant("gamma", np.ones((64,), np.float32))
+    _rmsnorm_nodes(g, "x", "gamma", "y", expose_mean=True)
+    feeds = {"x": np.random.default_rng(4).standard_normal((2, 64), dtype=np.float32)}
+    a, b, n, _ = _run_both(g.build(), feeds)
+    assert n == 0
+    _same(a, b)
+
+
+def test_softmax_pattern_with_mask_broadcast_on_last_dim_runs_the_body(device):
+    g = _builder()
+    g.input("x", np.float32, [2, 4, 8])
+    g.input("m", np.float32, [2, 4, 1])
+    g.constant("c", np.array(4.0, np.float32))
+    g.op("Div", ["x", "c"], ["sc"])
+    g.op("Add", ["m", "sc"], ["z"])
+    g.op("Softmax", ["z"], ["p"]).attr("axis", -1)
+    g.output("p")
+    rng = np.random.default_rng(5)
+    feeds = {"x": rng.standard_normal((2, 4, 8), dtype=np.float32),
+             "m": rng.standard_normal((2, 4, 1), dtype=np.float32)}
+    a, b, n, _ = _run_both(g.build(), feeds)
+    assert n == 1
+    _same(a, b)
+
+
+def test_rotary_pattern_on_rank3_runs_the_body(device):
+    g = _builder()
+    g.input("x", np.float32, [3, 5, 8])
+    g.input("cos", np.float32, [5, 8])
+    g.input("sin", np.float32, [5, 8])
+    for name, v in (("z0", [0]), ("h", [4]), ("e", [8]), ("ax", [2])):
+        g.constant(name, np.array(v, np.int64))
+    g.op("Slice", ["x", "z0", "h", "ax"], ["x1"])
+    g.op("Slice", ["x", "h", "e", "ax"], ["x2"])
+    g.op("Neg", ["x2"], ["n2"])
+    g.op("Concat", ["n2", "x1"], ["rot"]).attr("axis", -1)
+    g.op("Mul", ["x", "cos"], ["a"])
+    g.op("Mul", ["rot", "sin"], ["r"])
+    g.op("Add", ["a", "r"], ["y"])
+    g.output("y")
+    rng = np.random.default_rng(6)
+    feeds = {"x": rng.standard_normal((3, 5, 8), dtype=np.float32),
+             "cos": rng.standard_normal((5, 8), dtype=np.float32),
+             "sin": rng.standard_normal((5, 8), dtype=np.float32)}
+    a, b, n, _ = _run_both(g.build(), feeds)
+    assert n == 1
+    _same(a, b)
+
+
+def test_user_graph_cannot_name_internal_ops(device):
+    from rmlk_amd import runtime
+    g = _builder()
+    g.input("x", np.float32, [4])
+    g.op("rmlk.SwiGLU", ["x", "x"], ["y"])
+    g.output("y")
+    with pytest.raises(Exception, match="unsupported operator"):
+        runtime.Builder.from_graph(g.build()).build()
