@@ -134,7 +134,7 @@ def run_llama(args):
     stats = inst.node_stats()
     # classify each MatMul node by the kernel the library picks for its shape
     shapes = matmul_shapes(cfg, prompt_len, max_len)
-    mm_nodes = [s for s in stats if s["op"] == "MatMul"]
+    mm_nodes = [s for s in stats if s["op"] in ("MatMul", "rmlk.AttnMatMul")]
     assert len(mm_nodes) == len(shapes), (len(mm_nodes), len(shapes))
     by_kind, per_op = {}, {}
     for s, (batch, m, n, k) in zip(mm_nodes, shapes):
@@ -262,10 +262,12 @@ def decode_weight_bytes(cfg):
 def matmul_shapes(cfg, s, max_len):
     """(batch, m, n, k) of every MatMul node of the scatter-style graph in node order."""
     h, kvd, d = cfg.hidden, cfg.kv_heads * cfg.head_dim, cfg.head_dim
+    rep = cfg.heads // cfg.kv_heads
     out = []
     for _ in range(cfg.layers):
+        # the two attention products run as one strided GEMM per KV head over its group of q heads
         out += [(1, s, cfg.heads * d, h), (1, s, kvd, h), (1, s, kvd, h),
-                (cfg.heads, s, max_len, d), (cfg.heads, s, d, max_len),
+                (cfg.kv_heads, rep * s, max_len, d), (cfg.kv_heads, rep * s, d, max_len),
                 (1, s, h, cfg.heads * d), (1, s, cfg.ffn, h), (1, s, cfg.ffn, h), (1, s, h, cfg.ffn)]
     out.append((1, s, cfg.vocab, h))
     return out

@@ -41,12 +41,13 @@ constexpr int kThreads = 256;
 constexpr int kPadA = 4;  // floats of padding per LDS row of A
 constexpr int kPadB = 8;  // floats of padding per LDS row of B
 
-template <int BM, int BN, int BK>
+// TB: B is stored [N][K] (K contiguous) and staged in LDS exactly like A, [BN][BK + pad].
+template <int BM, int BN, int BK, bool TB = false>
 struct SmemLayout {
     static constexpr int kAStride = BK + kPadA;
-    static constexpr int kBStride = BN + kPadB;
+    static constexpr int kBStride = TB ? BK + kPadA : BN + kPadB;
     static constexpr int kAFloats = BM * kAStride;
-    static constexpr int kBFloats = BK * kBStride;
+    static constexpr int kBFloats = TB ? BN * kBStride : BK * kBStride;
     static constexpr int kBytes = 2 * (kAFloats + kBFloats) * 4;
 };
 
@@ -76,9 +77,11 @@ __device__ __forceinline__ void tile_coords(const GemmArgs &g, int &tm, int &tn)
 // multiple of BK) and rows are 16-byte aligned, so the main loop has no bounds checks at all.
 // EDGE == true: guarded loads (zero fill) and guarded stores; `aligned` still allows 128-bit
 // loads where a whole vector is in range.
-template <int BM, int BN, int BK, int WM, int WN, bool EDGE>
+// TB == true: B is given as [N][K] rows (C = A . B^T); both operands are then K-contiguous and the
+// B fragment is one 128-bit LDS read like A's.
+template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool TB = false>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
-    using L = SmemLayout<BM, BN, BK>;
+    using L = SmemLayout<BM, BN, BK, TB>;
     extern __shared__ __align__(16) float smem[];
     float *As = smem;                     // [2][BM][kAStride]
     float *Bs = smem + 2 * L::kAFloats;   // [2][BK][kBStride]
@@ -92,9 +95,9 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
     constexpr int A_VECS_PER_ROW = BK / 4;
     constexpr int A_ROWS_PER_PASS = kThreads / A_VECS_PER_ROW;
     constexpr int A_PASSES = BM / A_ROWS_PER_PASS;
-    constexpr int B_VECS_PER_ROW = BN / 4;
+    constexpr int B_VECS_PER_ROW = (TB ? BK : BN) / 4;
     constexpr int B_ROWS_PER_PASS = kThreads / B_VECS_PER_ROW;
-    constexpr int B_PASSES = BK / B_ROWS_PER_PASS;
+    constexpr int B_PASSES = (TB ? BN : BK) / B_ROWS_PER_PASS;
     static_assert(A_PASSES >= 1 && B_PASSES >= 1, "tile too small for 256 lanes");
 
     int tile_m, tile_n;
@@ -122,10 +125,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
 
     // per-lane source pointers of the first K step; they advance by BK (A) and BK rows (B)
     const float *a_src = A + static_cast<int64_t>(m0 + a_row) * g.lda + k_begin + a_vec * 4;
-    const float *b_src = B + static_cast<int64_t>(k_begin + b_row) * g.ldb + n0 + b_vec * 4;
+    const float *b_src = TB ? B + static_cast<int64_t>(n0 + b_row) * g.ldb + k_begin + b_vec * 4
+                            : B + static_cast<int64_t>(k_begin + b_row) * g.ldb + n0 + b_vec * 4;
     const int64_t a_pass_stride = static_cast<int64_t>(A_ROWS_PER_PASS) * g.lda;
     const int64_t b_pass_stride = static_cast<int64_t>(B_ROWS_PER_PASS) * g.ldb;
-    const int64_t b_step_stride = static_cast<int64_t>(BK) * g.ldb;
+    const int64_t b_step_stride = TB ? BK : static_cast<int64_t>(BK) * g.ldb;
     const bool vec_ok = g.aligned != 0;
 
     auto load_global = [&](int k0) {
@@ -156,6 +160,23 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
             }
 #pragma unroll
             for (int p = 0; p < B_PASSES; ++p) {
+                if constexpr (TB) {
+                    const int r = n0 + b_row + p * B_ROWS_PER_PASS;
+                    const int kk = k0 + b_vec * 4;
+                    v4f v = {0.f, 0.f, 0.f, 0.f};
+                    if (r < g.n) {
+                        const float *src = b_src + p * b_pass_stride;
+                        if (vec_ok && kk + 3 < k_end) {
+                            v = *reinterpret_cast<const v4f *>(src);
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < 4; ++j)
+                                if (kk + j < k_end) v[j] = src[j];
+                        }
+                    }
+                    b_reg[p] = v;
+                    continue;
+                }
                 const int kk = k0 + b_row + p * B_ROWS_PER_PASS;
                 const int c = n0 + b_vec * 4;
                 v4f v = {0.f, 0.f, 0.f, 0.f};
@@ -204,7 +225,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
     __syncthreads();
 
     const int a_frag = (wm * WM + l32) * L::kAStride + half * 4;
-    const int b_frag = (half * 4) * L::kBStride + wn * WN + l32;
+    const int b_frag = TB ? (wn * WN + l32) * L::kBStride + half * 4
+                          : (half * 4) * L::kBStride + wn * WN + l32;
     for (int step = 0; step < n_steps; ++step) {
         const int buf = step & 1;
         const bool more = step + 1 < n_steps;
@@ -219,10 +241,21 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
             for (int i = 0; i < TM; ++i)
                 af[i] = *reinterpret_cast<const v4f *>(as + i * 32 * L::kAStride + kc * 8);
+            if constexpr (TB) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s)
+                for (int j = 0; j < TN; ++j) {
+                    const v4f bv =
+                        *reinterpret_cast<const v4f *>(bs + j * 32 * L::kBStride + kc * 8);
 #pragma unroll
-                for (int j = 0; j < TN; ++j) bf[j][s] = bs[(kc * 8 + s) * L::kBStride + j * 32];
+                    for (int s = 0; s < 4; ++s) bf[j][s] = bv[s];
+                }
+            } else {
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        bf[j][s] = bs[(kc * 8 + s) * L::kBStride + j * 32];
+            }
 #pragma unroll
             for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -512,10 +545,10 @@ inline int gemv_splits(int64_t batch, int64_t n, int64_t k, int cols_per_block, 
     return static_cast<int>((k + kps - 1) / kps);
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool EDGE>
+template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool TB = false>
 int32_t launch_mfma(hipStream_t s, const GemmArgs &g, int64_t batch, int splits) {
-    using L = SmemLayout<BM, BN, BK>;
-    auto kern = gemm_mfma_kernel<BM, BN, BK, WM, WN, EDGE>;
+    using L = SmemLayout<BM, BN, BK, TB>;
+    auto kern = gemm_mfma_kernel<BM, BN, BK, WM, WN, EDGE, TB>;
     if (L::kBytes > 64 * 1024) {
         static bool raised = false;  // benign race: same value from every thread
         if (!raised) {
@@ -657,7 +690,7 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
         return RMLK_OK;
     }
 
-    if (trans_a || trans_b) {
+    if (trans_a) {
         unsigned grid = grid_for(batch * m * n, kThreads, 16);
         gemm_naive_kernel<<<grid, kThreads, 0, s>>>(
             pa, pb, pc, batch, static_cast<int32_t>(m), static_cast<int32_t>(n),
@@ -699,15 +732,19 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
     const bool full = aligned && m % t.bm == 0 && n % t.bn == 0 && t.k_per_split % t.bk == 0 &&
                       k % t.k_per_split == 0;
     int32_t st;
-#define RMLK_LAUNCH(BM_, BN_, WM_, WN_)                                                        \
-    (t.bk == 32 ? (full ? launch_mfma<BM_, BN_, 32, WM_, WN_, false>(s, g, batch, t.splits)     \
-                        : launch_mfma<BM_, BN_, 32, WM_, WN_, true>(s, g, batch, t.splits))     \
-                : (full ? launch_mfma<BM_, BN_, 16, WM_, WN_, false>(s, g, batch, t.splits)     \
-                        : launch_mfma<BM_, BN_, 16, WM_, WN_, true>(s, g, batch, t.splits)))
+#define RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, TB_)                                                   \
+    (t.bk == 32                                                                                  \
+         ? (full ? launch_mfma<BM_, BN_, 32, WM_, WN_, false, TB_>(s, g, batch, t.splits)        \
+                 : launch_mfma<BM_, BN_, 32, WM_, WN_, true, TB_>(s, g, batch, t.splits))        \
+         : (full ? launch_mfma<BM_, BN_, 16, WM_, WN_, false, TB_>(s, g, batch, t.splits)        \
+                 : launch_mfma<BM_, BN_, 16, WM_, WN_, true, TB_>(s, g, batch, t.splits)))
+#define RMLK_LAUNCH(BM_, BN_, WM_, WN_)                                                          \
+    (trans_b ? RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, true) : RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, false))
     if (t.bm == 256) st = RMLK_LAUNCH(256, 64, 64, 64);
     else if (t.bm == 128) st = RMLK_LAUNCH(128, 128, 64, 64);
     else st = RMLK_LAUNCH(64, 64, 32, 32);
 #undef RMLK_LAUNCH
+#undef RMLK_LAUNCH_TB
     if (st) return st;
     if (t.splits > 1) {
         unsigned rg = grid_for(batch * m * n, kThreads, 8);

@@ -203,6 +203,7 @@ void op_fused_rmsnorm(OpContext &c);
 void op_fused_swiglu(OpContext &c);
 void op_fused_softmax(OpContext &c);
 void op_fused_rotary(OpContext &c);
+void op_fused_attn_matmul(OpContext &c);
 
 struct CapturedPlan {
     hipGraph_t graph = nullptr;

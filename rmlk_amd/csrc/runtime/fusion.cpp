@@ -4,12 +4,14 @@
 // (runtime/src/core/instance.rs:25-37). Decoder graphs repeat a few chains of small element-wise
 // nodes in every layer; on this GPU each launch costs ~2 us whatever it moves, so those chains
 // dominate a decode step. This pass finds four of them and replaces each by ONE node backed by a
-// fused kernel that rounds every intermediate like the separate kernels do:
+// fused kernel that rounds every intermediate like the separate kernels do (the attention MatMul
+// instead drops two copies: the grouped-query Expand and the K transpose become GEMM strides):
 //
 //   rmlk.RMSNorm           Pow(x,2) ReduceMean(-1) Add(eps) Sqrt Div|(Div(1,.) Mul) Mul(gamma)
 //   rmlk.SwiGLU            Sigmoid(g) Mul(g,.) Mul(.,u)
 //   rmlk.ScaleMaskSoftmax  Div|Mul(x,c) Add(mask) Softmax(-1)
 //   rmlk.Rotary            [Transpose(0,2,1,3)] Slice Slice Neg Concat Mul Mul Add
+//   rmlk.AttnMatMul        MatMul(a, [Transpose(0,1,3,2)] [Reshape Expand Unsqueeze] (kv))
 //
 // A fused node keeps the nodes it replaced as its `body`. What cannot be decided while building
 // (shapes are only known at run time) is checked when the node runs; if the fused kernel does not
@@ -344,6 +346,68 @@ struct Matcher {
         }
         return false;
     }
+
+    static Attr a_ints(const std::vector<int64_t> &v) {
+        Attr a;
+        a.kind = Attr::Ints;
+        a.ints = v;
+        return a;
+    }
+
+    // ---- attention MatMul whose second operand is a transposed and / or group-expanded cache -------
+    bool match_attn_matmul(const Node &mm) {
+        if (mm.op != "MatMul" || mm.inputs.size() != 2 || mm.inputs[0] < 0) return false;
+        std::vector<const Node *> parts;
+        int cur = mm.inputs[1];
+        const Node *user = &mm;
+        bool transposed = false, expanded = false;
+        std::vector<int64_t> expand_shape, reshape_shape;
+        if (const Node *tr = produced_by(cur, "Transpose")) {
+            auto it = tr->attrs.find("perm");
+            const std::vector<int64_t> want = {0, 1, 3, 2};
+            if (it != tr->attrs.end() && it->second.ints == want && only_used_by(cur, {user})) {
+                transposed = true;
+                parts.push_back(tr);
+                cur = tr->inputs[0];
+                user = tr;
+            }
+        }
+        if (const Node *rs = produced_by(cur, "Reshape")) {
+            const Node *ex = rs->inputs.size() == 2 ? produced_by(rs->inputs[0], "Expand") : nullptr;
+            const Node *us = ex && ex->inputs.size() == 2 ? produced_by(ex->inputs[0], "Unsqueeze")
+                                                          : nullptr;
+            std::vector<int64_t> axes;
+            bool axes_ok = false;
+            if (us) {
+                auto it = us->attrs.find("axes");
+                if (it != us->attrs.end()) axes = it->second.ints;
+                else if (us->inputs.size() > 1) const_ints(us->inputs[1], &axes);
+                axes_ok = axes.size() == 1 && (axes[0] == 2 || axes[0] == -3);
+            }
+            if (us && axes_ok && attr_int(*rs, "allowzero", 0) == 0 &&
+                const_ints(ex->inputs[1], &expand_shape) && const_ints(rs->inputs[1], &reshape_shape) &&
+                only_used_by(cur, {user}) && only_used_by(rs->inputs[0], {rs}) &&
+                only_used_by(ex->inputs[0], {ex})) {
+                expanded = true;
+                parts.push_back(rs);
+                parts.push_back(ex);
+                parts.push_back(us);
+                cur = us->inputs[0];
+            }
+        }
+        if (!transposed && !expanded) return false;
+        parts.push_back(&mm);
+        Node f;
+        f.op = "rmlk.AttnMatMul";
+        f.inputs = {mm.inputs[0], cur};
+        f.outputs = mm.outputs;
+        f.attrs["transposed"] = a_int(transposed ? 1 : 0);
+        f.attrs["expanded"] = a_int(expanded ? 1 : 0);
+        f.attrs["expand_shape"] = a_ints(expand_shape);
+        f.attrs["reshape_shape"] = a_ints(reshape_shape);
+        replace(parts, std::move(f));
+        return true;
+    }
 };
 
 // Run the nodes a fused node replaced, one kernel each.
@@ -503,6 +567,75 @@ void op_fused_rotary(OpContext &c) {
     run_body(c);
 }
 
+// MatMul(a [B,H,S,K], f(kv [B,G,L,D])) where f repeats every cache head H / G times (Unsqueeze,
+// Expand, Reshape) and / or swaps the last two dims: one strided GEMM with batch B * G and
+// M = (H / G) * S reads the cache in place; neither the repeated nor the transposed copy is made.
+void op_fused_attn_matmul(OpContext &c) {
+    const Tensor &a = c.input(0), &kv = c.input(1);
+    const bool transposed = c.attr_int("transposed", 0) != 0;
+    const bool expanded = c.attr_int("expanded", 0) != 0;
+    bool ok = a.dtype == RMLK_FLOAT && kv.dtype == RMLK_FLOAT && a.rank() == 4 && kv.rank() == 4 &&
+              a.numel() > 0 && kv.numel() > 0;
+    int64_t rep = 1;
+    if (ok && expanded) {
+        const std::vector<int64_t> e = c.attr_ints("expand_shape"), r = c.attr_ints("reshape_shape");
+        const int64_t in5[5] = {kv.shape[0], kv.shape[1], 1, kv.shape[2], kv.shape[3]};
+        ok = e.size() == 5 && r.size() == 4;
+        for (int d = 0; d < 5 && ok; ++d)
+            if (d != 2 && e[d] != 1 && e[d] != in5[d]) ok = false;
+        if (ok) {
+            rep = e[2];
+            ok = rep >= 1;
+        }
+        if (ok) {
+            // the Reshape must give [B, G * rep, L, D] (0 copies a dim, one -1 is inferred)
+            const int64_t ex5[5] = {in5[0], in5[1], rep, in5[3], in5[4]};
+            const int64_t want[4] = {ex5[0], ex5[1] * rep, ex5[3], ex5[4]};
+            int64_t total = 1, known = 1;
+            for (int64_t d : ex5) total *= d;
+            int infer = -1;
+            int64_t got[4];
+            for (int d = 0; d < 4 && ok; ++d) {
+                if (r[d] == -1) {
+                    if (infer >= 0) ok = false;
+                    infer = d;
+                    got[d] = 1;
+                } else if (r[d] == 0) {
+                    got[d] = ex5[d];
+                    known *= got[d];
+                } else {
+                    got[d] = r[d];
+                    known *= got[d];
+                }
+            }
+            if (ok && infer >= 0) {
+                ok = known > 0 && total % known == 0;
+                if (ok) got[infer] = total / known;
+            }
+            for (int d = 0; d < 4 && ok; ++d)
+                if (got[d] != want[d]) ok = false;
+        }
+    }
+    if (ok) {
+        const int64_t bsz = kv.shape[0], grp = kv.shape[1], len = kv.shape[2], dim = kv.shape[3];
+        const int64_t heads = a.shape[1], seq = a.shape[2], ka = a.shape[3];
+        const int64_t n = transposed ? len : dim, k = transposed ? dim : len;
+        ok = a.shape[0] == bsz && heads == grp * rep && ka == k;
+        if (ok) {
+            const int64_t batch = bsz * grp, m = rep * seq;
+            Tensor &y = c.alloc_output(0, RMLK_FLOAT, {bsz, heads, seq, n});
+            const size_t ws_bytes = rmlk_hip_matmul_workspace_size(RMLK_FLOAT, batch, m, n, k);
+            void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
+            check_status(rmlk_hip_matmul(c.stream, RMLK_FLOAT, batch, m, n, k, a.data(), k, m * k, 0,
+                                         kv.data(), dim, len * dim, transposed ? 1 : 0, y.data(), n,
+                                         m * n, ws, ws_bytes),
+                         "rmlk.AttnMatMul");
+            return;
+        }
+    }
+    run_body(c);
+}
+
 // Rewrite the session's node list; returns how many fused nodes were formed.
 int fuse_patterns(Session &s) {
     Matcher m(s);
@@ -517,6 +650,8 @@ int fuse_patterns(Session &s) {
             if (m.match_softmax(node)) ++formed;
         } else if (node.op == "Add") {
             if (m.match_rotary(node)) ++formed;
+        } else if (node.op == "MatMul") {
+            if (m.match_attn_matmul(node)) ++formed;
         }
     }
     if (!formed) return 0;

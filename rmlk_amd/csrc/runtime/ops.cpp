@@ -827,6 +827,7 @@ const std::unordered_map<std::string, OpFn> &registry() {
         {"rmlk.SwiGLU", op_fused_swiglu},
         {"rmlk.ScaleMaskSoftmax", op_fused_softmax},
         {"rmlk.Rotary", op_fused_rotary},
+        {"rmlk.AttnMatMul", op_fused_attn_matmul},
     };
     return table;
 }

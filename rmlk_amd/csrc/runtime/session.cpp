@@ -420,7 +420,8 @@ void Session::run_nodes() {
             }
             if (node.op == "ScatterND" && !any_new) bytes += static_cast<double>(ctx.in[2]->nbytes());
         }
-        if (node.op == "MatMul" && ctx.in[0] && !ctx.in[0]->shape.empty())
+        if ((node.op == "MatMul" || node.op == "rmlk.AttnMatMul") && ctx.in[0] &&
+            !ctx.in[0]->shape.empty())
             flops = 2.0 * static_cast<double>(outs[0].numel()) *
                     static_cast<double>(ctx.in[0]->shape.back());
         st.bytes = bytes;

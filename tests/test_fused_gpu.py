@@ -209,8 +209,8 @@ def test_pass_forms_the_expected_nodes_on_the_llama_graph(device):
         for kv in ("key", "value"):
             feeds[f"cache.{l}.{kv}"] = np.zeros((1, cfg.kv_heads, 24, cfg.head_dim), np.float32)
     a, b, n, _ = _run_both(graph, feeds)
-    # per layer: 2 RMSNorm, 2 rotary, 1 SwiGLU, 1 softmax; plus the final RMSNorm
-    assert n == cfg.layers * 6 + 1
+    # per layer: 2 RMSNorm, 2 rotary, 1 SwiGLU, 1 softmax, 2 attention MatMuls; plus the final RMSNorm
+    assert n == cfg.layers * 8 + 1
     # RMSNorm's mean may differ in the last place; everything downstream inherits that
     _same(a, b, loose=set(a.keys()))
     assert np.array_equal(np.argmax(a["logits"][0], -1), np.argmax(b["logits"][0], -1))
@@ -223,7 +223,7 @@ def test_fused_llama_concat_style_against_oracle(device):
     graph = graphs.llama_graph(cfg, seed=4, style="concat")
     feeds = graphs.llama_concat_inputs(cfg, np.random.default_rng(1).integers(0, cfg.vocab, 9), None, 0)
     inst = runtime.Builder.from_graph(graph).build()
-    assert inst.fused_nodes == cfg.layers * 6 + 1
+    assert inst.fused_nodes == cfg.layers * 8 + 1
     got = inst.run(feeds)
     exp = og.run_graph(graph, feeds)
     for name in exp:
@@ -235,7 +235,7 @@ def test_fused_decoder_layer_full_width(device):
     from rmlk_amd import graphs
     graph, feeds = graphs.decoder_layer_graph(seed=3, seq=96)
     a, b, n, _ = _run_both(graph, feeds)
-    assert n == 6
+    assert n == 8
     _same(a, b, loose={"y"})
 
 
@@ -360,6 +360,73 @@ def test_rotary_pattern_on_rank3_runs_the_body(device):
     a, b, n, _ = _run_both(g.build(), feeds)
     assert n == 1
     _same(a, b)
+
+
+@pytest.mark.parametrize("b,g,rep,s,l,d", [(1, 8, 4, 512, 640, 64), (1, 8, 4, 1, 640, 64),
+                                            (2, 2, 3, 5, 7, 8), (1, 4, 1, 6, 9, 16),
+                                            (1, 1, 1, 1, 33, 8)])
+def test_attention_matmuls_read_the_cache_in_place(device, b, g, rep, s, l, d):
+    """scores = q . K^T and ctx = p . V with the grouped-query repeat (Unsqueeze, Expand, Reshape)
+    and the K transpose folded into GEMM strides; against the one-kernel-per-node session (fp32
+    tolerance: the strided GEMM may pick another tile / GEMV kernel than the separate MatMul) and
+    the oracle."""
+    from oracle import graph as og
+    h = g * rep
+    gb = _builder()
+    gb.input("q", np.float32, [b, h, s, d])
+    gb.input("p", np.float32, [b, h, s, l])
+    gb.input("k", np.float32, [b, g, l, d])
+    gb.input("v", np.float32, [b, g, l, d])
+    gb.constant("ax", np.array([2], np.int64))
+    gb.constant("eshape", np.array([1, g, rep, 1, 1], np.int64))
+    gb.constant("rshape", np.array([b, h, -1, d], np.int64))
+    for t in ("k", "v"):
+        if rep > 1:
+            gb.op("Unsqueeze", [t, "ax"], [t + "u"])
+            gb.op("Expand", [t + "u", "eshape"], [t + "e"])
+            gb.op("Reshape", [t + "e", "rshape"], [t + "x"])
+        else:
+            gb.op("Neg", [t], [t + "n"])
+            gb.op("Neg", [t + "n"], [t + "x"])
+    gb.op("Transpose", ["kx"], ["kt"]).attr("perm", [0, 1, 3, 2])
+    gb.op("MatMul", ["q", "kt"], ["scores"])
+    gb.op("MatMul", ["p", "vx"], ["ctx"])
+    gb.output("scores")
+    gb.output("ctx")
+    graph = gb.build()
+    rng = np.random.default_rng(b + g + rep + s + l + d)
+    feeds = {"q": rng.standard_normal((b, h, s, d), dtype=np.float32),
+             "p": rng.random((b, h, s, l), dtype=np.float32),
+             "k": rng.standard_normal((b, g, l, d), dtype=np.float32),
+             "v": rng.standard_normal((b, g, l, d), dtype=np.float32)}
+    a_, b_, n, _ = _run_both(graph, feeds)
+    assert n == (2 if rep > 1 else 1)
+    exp = og.run_graph(graph, feeds)
+    for name in ("scores", "ctx"):
+        assert_close(a_[name], b_[name], rtol=1e-4, atol=1e-4)
+        assert_close(a_[name], exp[name], rtol=1e-4, atol=1e-4)
+
+
+def test_attn_matmul_with_unexpected_expand_runs_the_body(device):
+    """Expand that also grows the batch dim: the pattern is formed, the run-time check refuses it."""
+    gb = _builder()
+    gb.input("q", np.float32, [2, 4, 3, 8])
+    gb.input("k", np.float32, [1, 2, 5, 8])
+    gb.constant("ax", np.array([2], np.int64))
+    gb.constant("eshape", np.array([2, 2, 2, 1, 1], np.int64))
+    gb.constant("rshape", np.array([2, 4, 5, 8], np.int64))
+    gb.op("Unsqueeze", ["k", "ax"], ["ku"])
+    gb.op("Expand", ["ku", "eshape"], ["ke"])
+    gb.op("Reshape", ["ke", "rshape"], ["kx"])
+    gb.op("Transpose", ["kx"], ["kt"]).attr("perm", [0, 1, 3, 2])
+    gb.op("MatMul", ["q", "kt"], ["scores"])
+    gb.output("scores")
+    rng = np.random.default_rng(9)
+    feeds = {"q": rng.standard_normal((2, 4, 3, 8), dtype=np.float32),
+             "k": rng.standard_normal((1, 2, 5, 8), dtype=np.float32)}
+    a_, b_, n, _ = _run_both(gb.build(), feeds)
+    assert n == 1
+    _same(a_, b_)
 
 
 def test_user_graph_cannot_name_internal_ops(device):

@@ -329,6 +329,21 @@ def test_matmul(device, case, bcast_b):
     assert_close(got, expected, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("case", MATMUL_CASES + [(8, 2048, 640, 64), (8, 4, 640, 64), (2, 100, 36, 52)])
+def test_matmul_b_transposed_mfma(device, case):
+    """B given as [N][K] rows (C = A . B^T): the K-contiguous staging path of the MFMA kernel,
+    bit-identical to the row-major path on the same values (same tiles, same K order)."""
+    batch, m, n, kk = case
+    rng = np.random.default_rng(74)
+    a = rng.standard_normal((batch, m, kk)).astype(np.float32)
+    b = (rng.standard_normal((batch, kk, n)) * 0.02).astype(np.float32)
+    bt = np.ascontiguousarray(b.transpose(0, 2, 1))
+    got = run_matmul(device, a, bt, False, True)
+    assert_close(got, _ops().matmul(a, b), rtol=1e-4, atol=1e-5)
+    if m > 1:
+        assert_exact(got, run_matmul(device, a, b))
+
+
 def test_matmul_exact_integers(device):
     """Integer-valued operands small enough that fp32 accumulation is exact in any order."""
     rng = np.random.default_rng(72)
