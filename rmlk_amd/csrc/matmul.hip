@@ -12,6 +12,8 @@
 //     accumulators. MFMA's 2-deep K is fed with a K-permutation inside every 8-wide K chunk: lanes
 //     0-31 take k = 0..3 and lanes 32-63 take k = 4..7 of the chunk, for A and B alike, so one
 //     128-bit LDS read of A serves four MFMAs and the sum over K is unchanged;
+//   - problems made of whole tiles with K steps of 32 take the variant whose K-step tiles go from
+//     global memory straight into LDS (global_load_lds_dwordx4), see gemm_mfma_direct_kernel;
 //   - split-K (grid z) writes partial tiles to the workspace, a second kernel adds them in a
 //     fixed order, so results do not depend on scheduling.
 #include <cstdio>
@@ -218,55 +220,94 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     const int n_steps = (k_end - k_begin + BK - 1) / BK;
-    if (n_steps > 0) {
-        load_global(k_begin);
-        store_lds(0);
-    }
-    __syncthreads();
-
     const int a_frag = (wm * WM + l32) * L::kAStride + half * 4;
     const int b_frag = TB ? (wn * WN + l32) * L::kBStride + half * 4
                           : (half * 4) * L::kBStride + wn * WN + l32;
-    for (int step = 0; step < n_steps; ++step) {
-        const int buf = step & 1;
-        const bool more = step + 1 < n_steps;
-        if (more) load_global(k_begin + (step + 1) * BK);
+    constexpr int KC = BK / 8;
+    static_assert(KC % 2 == 0, "fragment double buffering assumes an even number of K chunks");
 
+    // MFMA operands of one 8-wide K chunk, read from LDS buffer `buf`
+    v4f af[2][TM];
+    float bf[2][TN][4];
+    auto read_frags = [&](int buf, int kc, int slot) {
         const float *as = As + buf * L::kAFloats + a_frag;
         const float *bs = Bs + buf * L::kBFloats + b_frag;
 #pragma unroll
-        for (int kc = 0; kc < BK / 8; ++kc) {
-            v4f af[TM];
-            float bf[TN][4];
+        for (int i = 0; i < TM; ++i)
+            af[slot][i] = *reinterpret_cast<const v4f *>(as + i * 32 * L::kAStride + kc * 8);
+        if constexpr (TB) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-                af[i] = *reinterpret_cast<const v4f *>(as + i * 32 * L::kAStride + kc * 8);
-            if constexpr (TB) {
+            for (int j = 0; j < TN; ++j) {
+                const v4f bv = *reinterpret_cast<const v4f *>(bs + j * 32 * L::kBStride + kc * 8);
 #pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const v4f bv =
-                        *reinterpret_cast<const v4f *>(bs + j * 32 * L::kBStride + kc * 8);
-#pragma unroll
-                    for (int s = 0; s < 4; ++s) bf[j][s] = bv[s];
-                }
-            } else {
-#pragma unroll
-                for (int s = 0; s < 4; ++s)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        bf[j][s] = bs[(kc * 8 + s) * L::kBStride + j * 32];
+                for (int s = 0; s < 4; ++s) bf[slot][j][s] = bv[s];
             }
+        } else {
 #pragma unroll
             for (int s = 0; s < 4; ++s)
 #pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][s], bf[j][s],
-                                                                         acc[i][j], 0, 0, 0);
+                for (int j = 0; j < TN; ++j)
+                    bf[slot][j][s] = bs[(kc * 8 + s) * L::kBStride + j * 32];
         }
-        if (more) store_lds(buf ^ 1);
-        __syncthreads();
+    };
+    // LDS traffic of this wavefront has drained, then the block meets. (Global loads of a later
+    // K step stay in flight across the barrier.)
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    // Software pipeline over K steps s = 0 .. n_steps-1, LDS buffer s & 1. Program order inside a
+    // step (the scheduler is told not to move work across the marked points):
+    //   chunk 0         : after its first MFMAs, the tile of step s+1 (in registers since step s-1)
+    //                     goes to the other LDS buffer and the global loads of step s+2 are issued;
+    //   chunk kc        : request the operands of chunk kc+1 from LDS, then issue chunk kc's MFMAs
+    //                     (they run while the requests complete);
+    //   last chunk      : this wavefront's reads of the buffer are complete, the block meets
+    //                     (everyone's stores of step s+1 are long done), the first operands of
+    //                     step s+1 are requested, and the last chunk's MFMAs cover that latency.
+    if (n_steps > 0) {
+        load_global(k_begin);
+        store_lds(0);
+        if (n_steps > 1) load_global(k_begin + BK);
+        lds_barrier();
+        read_frags(0, 0, 0);
+    }
+    auto mfma_chunk = [&](int slot, int s_begin, int s_end) {
+#pragma unroll
+        for (int s = s_begin; s < s_end; ++s)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[slot][i][s], bf[slot][j][s],
+                                                                     acc[i][j], 0, 0, 0);
+    };
+    for (int step = 0; step < n_steps; ++step) {
+        const int buf = step & 1;
+        const bool more = step + 1 < n_steps;
+        // chunk 0: its first MFMAs go out before anything else (their operands were requested a
+        // whole chunk ago), the LDS stores and global loads issue in their shadow
+        mfma_chunk(0, 0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) {
+            store_lds(buf ^ 1);
+            if (step + 2 < n_steps) load_global(k_begin + (step + 2) * BK);
+        }
+        read_frags(buf, 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_chunk(0, 1, 4);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kc = 1; kc < KC; ++kc) {
+            const int slot = kc & 1;
+            if (kc + 1 < KC) {
+                read_frags(buf, kc + 1, slot ^ 1);
+            } else {
+                lds_barrier();
+                if (more) read_frags(buf ^ 1, 0, slot ^ 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_chunk(slot, 0, 4);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 
     // C fragment: column = l32, row = 8 * (r / 4) + 4 * half + r % 4
@@ -282,6 +323,203 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
                     if (!EDGE || row < g.m)
                         C[static_cast<int64_t>(row) * g.ldc + col] = acc[i][j][r];
                 }
+            }
+        }
+    }
+}
+
+// ---- full-tile kernel with direct global -> LDS loads ---------------------------------------------
+// For problems made of whole tiles (no bounds checks, 16-byte aligned rows, BK = 32) the K-step
+// tiles do not pass through registers: each wavefront issues `global_load_lds_dwordx4`, which
+// writes 64 lanes x 16 bytes as one contiguous 1 KiB piece of LDS while every lane picks its own
+// global address. Rows of 32 floats are therefore unpadded in LDS; bank conflicts on the
+// fragment reads of K-contiguous operands are avoided by a swizzle instead: the 16-byte unit q of
+// row r lives in unit q ^ (r & 7), applied on the global side when the unit is fetched and again
+// when it is read back. The loads are opaque to the compiler (inline asm), so completion is
+// awaited by hand (vmcnt) before the block-wide barrier that publishes a stage.
+template <int BM, int BN, int WM, int WN, bool TB, int STAGES>
+__global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) {
+    static_assert(STAGES == 2 || STAGES == 3, "two or three LDS stages");
+    constexpr int BK = 32;
+    constexpr int KC = BK / 8;
+    constexpr int kAFloats = BM * BK;   // one stage of A, floats
+    constexpr int kBFloats = BK * BN;
+    extern __shared__ __align__(16) float smem[];
+    float *As = smem;                        // [STAGES][BM][BK] swizzled
+    float *Bs = smem + STAGES * kAFloats;    // [STAGES][BK][BN], or [STAGES][BN][BK] swizzled (TB)
+
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int WAVES_N = BN / WN;
+    static_assert((BM / WM) * (BN / WN) == kThreads / kWave, "four wavefronts per block");
+    constexpr int A_PASSES = BM / 32;   // 1 KiB pieces (8 rows of A) per wavefront and stage
+    constexpr int B_PASSES = BN / 32;
+    constexpr int B_ROW_LANES = BN / 4;             // lanes per K-row of a row-major B tile
+    constexpr int B_ROWS_PER_PIECE = kWave / B_ROW_LANES > 0 ? kWave / B_ROW_LANES : 1;
+    static_assert(TB || B_ROW_LANES <= kWave, "a K-row of B must fit one 1 KiB piece");
+
+    int tile_m, tile_n;
+    tile_coords(g, tile_m, tile_n);
+    const int batch = blockIdx.y;
+    const int split = blockIdx.z;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int k_begin = split * g.k_per_split;
+    const int k_end = min(g.k, k_begin + g.k_per_split);
+    const int n_steps = (k_end - k_begin) / BK;
+
+    const float *A = g.a + batch * g.stride_a;
+    const float *B = g.b + batch * g.stride_b;
+    float *C = g.c + (static_cast<int64_t>(split) * gridDim.y + batch) * g.stride_c;
+
+    const int tid = threadIdx.x;
+    const int lane = tid % kWave;
+    const int wave = tid / kWave;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int l32 = lane % 32, half = lane / 32;
+
+    // this lane's global sources: piece (p * 4 + wave) of a stage, advanced by one K step per stage
+    const int sw_row = lane / 8, sw_unit = (lane % 8) ^ sw_row;
+    const float *a_src = A + static_cast<int64_t>(m0 + wave * 8 + sw_row) * g.lda + k_begin + sw_unit * 4;
+    const int64_t a_pass_stride = static_cast<int64_t>(32) * g.lda;
+    const float *b_src;
+    int64_t b_pass_stride, b_step_stride;
+    if constexpr (TB) {
+        b_src = B + static_cast<int64_t>(n0 + wave * 8 + sw_row) * g.ldb + k_begin + sw_unit * 4;
+        b_pass_stride = static_cast<int64_t>(32) * g.ldb;
+        b_step_stride = BK;
+    } else {
+        b_src = B + static_cast<int64_t>(k_begin + wave * B_ROWS_PER_PIECE + lane / B_ROW_LANES) * g.ldb +
+                n0 + (lane % B_ROW_LANES) * 4;
+        b_pass_stride = static_cast<int64_t>(4 * B_ROWS_PER_PIECE) * g.ldb;
+        b_step_stride = static_cast<int64_t>(BK) * g.ldb;
+    }
+    // LDS byte addresses of this wavefront's first piece of A and B in stage 0 (wave-uniform)
+    const uint32_t lds_a = __builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(As)) + wave * 1024u);
+    const uint32_t lds_b = __builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(Bs)) + wave * 1024u);
+
+    auto direct_load = [&](uint32_t lds_addr, const float *src) {
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off"
+                     :
+                     : "s"(lds_addr), "v"(src)
+                     : "memory", "m0");
+    };
+    auto issue_stage = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < A_PASSES; ++p)
+            direct_load(lds_a + static_cast<uint32_t>(buf * kAFloats * 4 + p * 4096),
+                        a_src + p * a_pass_stride);
+#pragma unroll
+        for (int p = 0; p < B_PASSES; ++p)
+            direct_load(lds_b + static_cast<uint32_t>(buf * kBFloats * 4 + p * 4096),
+                        b_src + p * b_pass_stride);
+        a_src += BK;
+        b_src += b_step_stride;
+    };
+
+    // fragment addressing
+    const int xr = l32 & 7;
+    const int a_row = (wm * WM + l32) * BK;
+    const int b_base = TB ? (wn * WN + l32) * BK : (half * 4) * BN + wn * WN + l32;
+    v4f af[2][TM];
+    float bf[2][TN][4];
+    auto read_frags = [&](int buf, int kc, int slot) {
+        const float *as = As + buf * kAFloats + a_row;
+        const float *bs = Bs + buf * kBFloats + b_base;
+        const int unit = ((kc * 2 + half) ^ xr) * 4;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            af[slot][i] = *reinterpret_cast<const v4f *>(as + i * 32 * BK + unit);
+        if constexpr (TB) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const v4f bv = *reinterpret_cast<const v4f *>(bs + j * 32 * BK + unit);
+#pragma unroll
+                for (int s = 0; s < 4; ++s) bf[slot][j][s] = bv[s];
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) bf[slot][j][s] = bs[(kc * 8 + s) * BN + j * 32];
+        }
+    };
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    auto mfma_chunk = [&](int slot, int s_begin, int s_end) {
+#pragma unroll
+        for (int s = s_begin; s < s_end; ++s)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[slot][i][s], bf[slot][j][s],
+                                                                     acc[i][j], 0, 0, 0);
+    };
+    // This wavefront's LDS reads are complete and its direct loads have landed, all of them or all
+    // but the newest stage's (loads complete in issue order); then the block meets.
+    constexpr int kLoadsPerStage = A_PASSES + B_PASSES;
+    auto stage_barrier = [&](bool newest_may_fly) {
+        if (newest_may_fly)
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kLoadsPerStage) : "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+
+    // Stage t lives in LDS buffer t % STAGES and is requested STAGES - 1 steps before its use; the
+    // buffer it overwrites was last read in the step before the request, and that step ended with
+    // the barrier.
+    constexpr int D = STAGES - 1;
+    int buf = 0, buf_next = STAGES > 2 ? 1 : 1 % STAGES, buf_load = D % STAGES;
+    if (n_steps > 0) {
+        issue_stage(0);
+        if (D == 2 && n_steps > 1) issue_stage(1);
+        stage_barrier(D == 2 && n_steps > 1);
+        read_frags(0, 0, 0);
+    }
+    for (int step = 0; step < n_steps; ++step) {
+        const bool more = step + 1 < n_steps;
+        const bool load = step + D < n_steps;
+        mfma_chunk(0, 0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (load) issue_stage(buf_load);
+        read_frags(buf, 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_chunk(0, 1, 4);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kc = 1; kc < KC; ++kc) {
+            const int slot = kc & 1;
+            if (kc + 1 < KC) {
+                read_frags(buf, kc + 1, slot ^ 1);
+            } else {
+                stage_barrier(D == 2 && load);
+                if (more) read_frags(buf_next, 0, slot ^ 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_chunk(slot, 0, 4);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        buf = buf_next;
+        buf_next = buf_next + 1 == STAGES ? 0 : buf_next + 1;
+        buf_load = buf_load + 1 == STAGES ? 0 : buf_load + 1;
+    }
+
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = n0 + wn * WN + j * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+                C[static_cast<int64_t>(row) * g.ldc + col] = acc[i][j][r];
             }
         }
     }
@@ -565,6 +803,25 @@ int32_t launch_mfma(hipStream_t s, const GemmArgs &g, int64_t batch, int splits)
     return launch_status();
 }
 
+template <int BM, int BN, int WM, int WN, bool TB, int STAGES>
+int32_t launch_direct(hipStream_t s, const GemmArgs &g, int64_t batch, int splits) {
+    constexpr int kBytes = STAGES * (BM * 32 + 32 * BN) * 4;
+    auto kern = gemm_mfma_direct_kernel<BM, BN, WM, WN, TB, STAGES>;
+    if (kBytes > 64 * 1024) {
+        static bool raised = false;  // benign race: same value from every thread
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
+            if (e != hipSuccess) return static_cast<int32_t>(e);
+            raised = true;
+        }
+    }
+    dim3 grid(static_cast<unsigned>(g.tiles_m * g.tiles_n), static_cast<unsigned>(batch),
+              static_cast<unsigned>(splits));
+    kern<<<grid, kThreads, kBytes, s>>>(g);
+    return launch_status();
+}
+
 }  // namespace
 }  // namespace rmlk
 
@@ -740,9 +997,21 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
                  : launch_mfma<BM_, BN_, 16, WM_, WN_, true, TB_>(s, g, batch, t.splits)))
 #define RMLK_LAUNCH(BM_, BN_, WM_, WN_)                                                          \
     (trans_b ? RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, true) : RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, false))
-    if (t.bm == 256) st = RMLK_LAUNCH(256, 64, 64, 64);
+#define RMLK_DIRECT_S(BM_, BN_, WM_, WN_, S_)                                                    \
+    (trans_b ? launch_direct<BM_, BN_, WM_, WN_, true, S_>(s, g, batch, t.splits)                \
+             : launch_direct<BM_, BN_, WM_, WN_, false, S_>(s, g, batch, t.splits))
+    // two LDS stages: a third (loads two K steps ahead) measured no faster and halves the blocks
+    // that fit a CU
+#define RMLK_DIRECT(BM_, BN_, WM_, WN_) RMLK_DIRECT_S(BM_, BN_, WM_, WN_, 2)
+    const bool direct = full && t.bk == 32;
+    if (direct && t.bm == 256) st = RMLK_DIRECT(256, 64, 64, 64);
+    else if (direct && t.bm == 128) st = RMLK_DIRECT(128, 128, 64, 64);
+    else if (direct) st = RMLK_DIRECT(64, 64, 32, 32);
+    else if (t.bm == 256) st = RMLK_LAUNCH(256, 64, 64, 64);
     else if (t.bm == 128) st = RMLK_LAUNCH(128, 128, 64, 64);
     else st = RMLK_LAUNCH(64, 64, 32, 32);
+#undef RMLK_DIRECT
+#undef RMLK_DIRECT_S
 #undef RMLK_LAUNCH
 #undef RMLK_LAUNCH_TB
     if (st) return st;
