@@ -728,7 +728,7 @@ struct TileChoice {
 };
 
 #ifndef RMLK_GEMM_SPLIT_TARGET
-#define RMLK_GEMM_SPLIT_TARGET 2
+#define RMLK_GEMM_SPLIT_TARGET 1
 #endif
 
 inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k) {
@@ -1002,8 +1002,14 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
              : launch_direct<BM_, BN_, WM_, WN_, false, S_>(s, g, batch, t.splits))
     // two LDS stages: a third (loads two K steps ahead) measured no faster and halves the blocks
     // that fit a CU
-#define RMLK_DIRECT(BM_, BN_, WM_, WN_) RMLK_DIRECT_S(BM_, BN_, WM_, WN_, 2)
-    const bool direct = full && t.bk == 32;
+#ifndef RMLK_GEMM_STAGES
+#define RMLK_GEMM_STAGES 2
+#endif
+#ifndef RMLK_GEMM_DIRECT
+#define RMLK_GEMM_DIRECT 1
+#endif
+#define RMLK_DIRECT(BM_, BN_, WM_, WN_) RMLK_DIRECT_S(BM_, BN_, WM_, WN_, RMLK_GEMM_STAGES)
+    const bool direct = RMLK_GEMM_DIRECT && full && t.bk == 32;
     if (direct && t.bm == 256) st = RMLK_DIRECT(256, 64, 64, 64);
     else if (direct && t.bm == 128) st = RMLK_DIRECT(128, 128, 64, 64);
     else if (direct) st = RMLK_DIRECT(64, 64, 32, 32);
