@@ -40,6 +40,7 @@ struct GemmArgs {
 };
 
 constexpr int kThreads = 256;
+constexpr int kSkinnyRows = 8;  // up to this many rows of A take the B-streaming kernels
 constexpr int kPadA = 4;  // floats of padding per LDS row of A
 constexpr int kPadB = 8;  // floats of padding per LDS row of B
 
@@ -647,11 +648,12 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(GemvArgs g) {
 // a fixed order (the result depends on `splits` only, never on timing).
 __global__ __launch_bounds__(kThreads) void gemv_reduce_kernel(const float *__restrict__ ws,
                                                                float *__restrict__ y, int splits,
-                                                               int64_t batch, int32_t n,
-                                                               int64_t stride_y) {
+                                                               int64_t batch, int32_t m, int32_t n,
+                                                               int64_t ldc, int64_t stride_y) {
     constexpr int kOut = 32, kGroups = kThreads / kOut;
     __shared__ float part[kGroups][kOut];
-    const int64_t total = batch * n;
+    const int64_t per = static_cast<int64_t>(m) * n;
+    const int64_t total = batch * per;
     const int ox = threadIdx.x % kOut, sy = threadIdx.x / kOut;
     const int64_t i = static_cast<int64_t>(blockIdx.x) * kOut + ox;
     float s = 0.f;
@@ -670,11 +672,132 @@ __global__ __launch_bounds__(kThreads) void gemv_reduce_kernel(const float *__re
     part[sy][ox] = s;
     __syncthreads();
     if (sy == 0 && i < total) {
-        const int64_t b = i / n, col = i - b * n;
+        const int64_t b = i / per, rem = i - b * per;
+        const int64_t row = rem / n, col = rem - row * n;
         float r = 0.f;
 #pragma unroll
         for (int q = 0; q < kGroups; ++q) r += part[q][ox];
-        y[b * stride_y + col] = r;
+        y[b * stride_y + row * ldc + col] = r;
+    }
+}
+
+// ---- skinny GEMM: 2..8 rows of A against a streamed B ---------------------------------------------
+// The decode-time shapes of grouped-query attention (the few query heads of one KV head against
+// its cache) and of small-batch projections: B is read from HBM once, every lane keeps ROWS x 4
+// accumulators. Same blocking as gemv_kernel<4>; rows beyond m are computed on row m-1 and dropped.
+struct SkinnyArgs {
+    const float *x;   // [batch][m][k] rows of lda
+    const float *w;   // [batch][k][n] rows of ldb, or [n][k] for the dot kernel
+    float *y;         // C, or partial workspace [split][batch][m][n]
+    int32_t m, n, k;
+    int64_t lda, ldb, ldy;
+    int64_t stride_x, stride_w, stride_y;
+    int32_t k_per_split;
+};
+
+template <int ROWS>
+__global__ __launch_bounds__(kThreads) void skinny_kernel(SkinnyArgs g) {
+    constexpr int kWaves = kThreads / kWave;
+    constexpr int kCols = kWave * 4;
+    __shared__ float red[kWaves][ROWS][kCols];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int batch = blockIdx.y, split = blockIdx.z;
+    const int col = blockIdx.x * kCols + lane * 4;
+    const int k_begin = split * g.k_per_split;
+    const int k_end = min(g.k, k_begin + g.k_per_split);
+    const float *x = g.x + batch * g.stride_x;
+    const float *w = g.w + batch * g.stride_w;
+    const float *xr[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) xr[r] = x + static_cast<int64_t>(min(r, g.m - 1)) * g.lda;
+
+    float acc[ROWS][4];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[r][j] = 0.f;
+
+    const int len = k_end - k_begin;
+    const int per_wave = (len + kWaves - 1) / kWaves;
+    const int kb = k_begin + wave * per_wave;
+    const int ke = min(k_end, kb + per_wave);
+    if (col < g.n) {
+        const float *wp = w + static_cast<int64_t>(kb) * g.ldb + col;
+        int kk = kb;
+        constexpr int U = 4;
+        for (; kk + U <= ke; kk += U) {
+            v4f wv[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                wv[u] = __builtin_nontemporal_load(
+                    reinterpret_cast<const v4f *>(wp + static_cast<int64_t>(u) * g.ldb));
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const float xv = xr[r][kk + u];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[r][j] = fmaf(xv, wv[u][j], acc[r][j]);
+                }
+            wp += static_cast<int64_t>(U) * g.ldb;
+        }
+        for (; kk < ke; ++kk) {
+            const v4f wv = *reinterpret_cast<const v4f *>(wp);
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                const float xv = xr[r][kk];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[r][j] = fmaf(xv, wv[j], acc[r][j]);
+            }
+            wp += g.ldb;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) red[wave][r][lane * 4 + j] = acc[r][j];
+    __syncthreads();
+    float *y = g.y + (static_cast<int64_t>(split) * gridDim.y + batch) * g.stride_y;
+    for (int t = threadIdx.x; t < ROWS * kCols; t += kThreads) {
+        const int r = t / kCols, c = t - r * kCols;
+        const int oc = blockIdx.x * kCols + c;
+        if (r < g.m && oc < g.n) {
+            float sum = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < kWaves; ++wv) sum += red[wv][r][c];
+            y[static_cast<int64_t>(r) * g.ldy + oc] = sum;
+        }
+    }
+}
+
+// B stored [n][k] (C = A . B^T): a wavefront per output column, ROWS dots along contiguous k.
+template <int ROWS>
+__global__ __launch_bounds__(kThreads) void skinny_dot_kernel(SkinnyArgs g) {
+    const int lane = threadIdx.x % kWave;
+    const int batch = blockIdx.y;
+    const float *x = g.x + batch * g.stride_x;
+    const float *w = g.w + batch * g.stride_w;
+    float *y = g.y + batch * g.stride_y;
+    const float *xr[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) xr[r] = x + static_cast<int64_t>(min(r, g.m - 1)) * g.lda;
+    for (int n = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave; n < g.n;
+         n += gridDim.x * (kThreads / kWave)) {
+        const float *wr = w + static_cast<int64_t>(n) * g.ldb;
+        float acc[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) acc[r] = 0.f;
+        for (int kk = lane; kk < g.k; kk += kWave) {
+            const float wv = wr[kk];
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) acc[r] = fmaf(xr[r][kk], wv, acc[r]);
+        }
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+#pragma unroll
+            for (int o = kWave / 2; o > 0; o >>= 1) acc[r] += __shfl_xor(acc[r], o, kWave);
+            if (lane == 0 && r < g.m) y[static_cast<int64_t>(r) * g.ldy + n] = acc[r];
+        }
     }
 }
 
@@ -839,8 +962,14 @@ extern "C" size_t rmlk_hip_matmul_workspace_size(int32_t dtype, int64_t batch, i
         return sp > 1 ? static_cast<size_t>(sp) * batch * n * sizeof(float) : 0;
     }
     TileChoice t = choose_tiles(batch, m, n, k);
-    return t.splits > 1 ? static_cast<size_t>(t.splits) * batch * m * n * sizeof(float)
-                        : 0;
+    size_t need = t.splits > 1 ? static_cast<size_t>(t.splits) * batch * m * n * sizeof(float) : 0;
+    if (m <= kSkinnyRows) {
+        int kps;
+        const int sp = gemv_splits(batch, n, k, kWave * 4, &kps);
+        const size_t skinny = sp > 1 ? static_cast<size_t>(sp) * batch * m * n * sizeof(float) : 0;
+        if (skinny > need) need = skinny;
+    }
+    return need;
 }
 
 extern "C" int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_t m, int64_t n,
@@ -853,9 +982,17 @@ extern "C" int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_
         const bool vec = n % 4 == 0;
         snprintf(tmp, sizeof(tmp), "gemv%s splitk=%d", vec ? "x4" : "x1",
                  gemv_splits(batch, n, k, vec ? kWave * 4 : kWave, &kps));
+    } else if (m <= kSkinnyRows && n % 4 == 0) {
+        int kps;
+        snprintf(tmp, sizeof(tmp), "skinny%d splitk=%d", m <= 2 ? 2 : m <= 4 ? 4 : 8,
+                 gemv_splits(batch, n, k, kWave * 4, &kps));
     } else {
         TileChoice t = choose_tiles(batch, m, n, k);
-        snprintf(tmp, sizeof(tmp), "mfma%dx%dx%d splitk=%d", t.bm, t.bn, t.bk, t.splits);
+        // dense row-major operands assumed (lda = k, ldb = n): whole tiles take the direct-to-LDS kernel
+        const bool whole = t.bk == 32 && m % t.bm == 0 && n % t.bn == 0 && k % 4 == 0 && n % 4 == 0 &&
+                           t.k_per_split % t.bk == 0 && k % t.k_per_split == 0;
+        snprintf(tmp, sizeof(tmp), "mfma%dx%dx%d%s splitk=%d", t.bm, t.bn, t.bk,
+                 whole ? " direct" : "", t.splits);
     }
     const int32_t len = static_cast<int32_t>(strlen(tmp));
     if (buf && size > 0) {
@@ -941,10 +1078,70 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
         if (splits > 1) {
             const int64_t total = batch * n;
             gemv_reduce_kernel<<<static_cast<unsigned>((total + 31) / 32), kThreads, 0, s>>>(
-                static_cast<const float *>(workspace), pc, splits, batch, g.n, stride_c);
+                static_cast<const float *>(workspace), pc, splits, batch, 1, g.n, ldc, stride_c);
             return launch_status();
         }
         return RMLK_OK;
+    }
+
+    if (m <= kSkinnyRows && !trans_a) {
+        SkinnyArgs g{};
+        g.x = pa;
+        g.w = pb;
+        g.m = static_cast<int32_t>(m);
+        g.n = static_cast<int32_t>(n);
+        g.k = static_cast<int32_t>(k);
+        g.lda = lda;
+        g.ldb = ldb;
+        g.stride_x = stride_a;
+        g.stride_w = stride_b;
+        if (trans_b) {
+            g.y = pc;
+            g.ldy = ldc;
+            g.stride_y = stride_c;
+            g.k_per_split = g.k;
+            int64_t blocks = (n + 3) / 4;
+            if (blocks > 8 * kNumCU) blocks = 8 * kNumCU;
+            dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch), 1);
+            if (m <= 2) skinny_dot_kernel<2><<<grid, kThreads, 0, s>>>(g);
+            else if (m <= 4) skinny_dot_kernel<4><<<grid, kThreads, 0, s>>>(g);
+            else skinny_dot_kernel<8><<<grid, kThreads, 0, s>>>(g);
+            return launch_status();
+        }
+        const bool vec = n % 4 == 0 && ldb % 4 == 0 && stride_b % 4 == 0 &&
+                         reinterpret_cast<uintptr_t>(pb) % 16 == 0;
+        if (vec) {
+            int kps;
+            const int splits = gemv_splits(batch, n, k, kWave * 4, &kps);
+            g.k_per_split = kps;
+            if (splits > 1) {
+                const size_t need = static_cast<size_t>(splits) * batch * m * n * sizeof(float);
+                if (!workspace || workspace_bytes < need) return RMLK_ERR_WORKSPACE;
+                g.y = static_cast<float *>(workspace);
+                g.ldy = n;
+                g.stride_y = m * n;
+            } else {
+                g.y = pc;
+                g.ldy = ldc;
+                g.stride_y = stride_c;
+            }
+            dim3 grid(static_cast<unsigned>((n + kWave * 4 - 1) / (kWave * 4)),
+                      static_cast<unsigned>(batch), static_cast<unsigned>(splits));
+            if (m <= 2) skinny_kernel<2><<<grid, kThreads, 0, s>>>(g);
+            else if (m <= 4) skinny_kernel<4><<<grid, kThreads, 0, s>>>(g);
+            else skinny_kernel<8><<<grid, kThreads, 0, s>>>(g);
+            int32_t st = launch_status();
+            if (st) return st;
+            if (splits > 1) {
+                const int64_t total = batch * m * n;
+                gemv_reduce_kernel<<<static_cast<unsigned>((total + 31) / 32), kThreads, 0, s>>>(
+                    static_cast<const float *>(workspace), pc, splits, batch, g.m, g.n, ldc,
+                    stride_c);
+                return launch_status();
+            }
+            return RMLK_OK;
+        }
+        // unaligned B: the MFMA kernel below handles it
     }
 
     if (trans_a) {

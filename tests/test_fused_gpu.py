@@ -192,7 +192,8 @@ def _same(a, b, loose=()):
     assert a.keys() == b.keys()
     for name in a:
         if a[name].dtype.kind == "f" and name in loose:
-            np.testing.assert_allclose(a[name], b[name], rtol=2e-6, atol=1e-7)
+            # the attention MatMul may run on another kernel (other summation order) once fused
+            np.testing.assert_allclose(a[name], b[name], rtol=1e-4, atol=1e-5)
         else:
             assert_exact(a[name], b[name])
 
