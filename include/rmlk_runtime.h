@@ -59,6 +59,25 @@ int32_t rmlk_graph_attr_tensor(rmlk_graph *g, int32_t node, const char *name, in
 /* Mark a value as graph output. ref: builder.rs:192-204 */
 int32_t rmlk_graph_output(rmlk_graph *g, const char *name);
 
+/* ---- ONNX files -------------------------------------------------------------------------------- */
+/* Build a graph from the bytes of an ONNX ModelProto (protobuf wire format). Follows the
+ * reference's importer: initializers first, then graph inputs (an input that shares its name with
+ * an initializer is a defaulted input: the constant stays), outputs, then the nodes in stored
+ * order; a symbolic or missing dim is dynamic (0); tensor payloads from raw_data, the typed
+ * repeated fields, or an external file (keys location / offset / length) resolved against
+ * `base_dir` (NULL or "": the working directory). Subgraph attributes, sparse and string tensors
+ * and non-tensor value types are rejected.
+ * ref: schema/src/onnx_import/transform.rs:76-260 (graph_from_onnx_bytes),
+ *      schema/src/onnx_import/traverse.rs:33-60, schema/src/tensor.rs:149-300 */
+int32_t rmlk_graph_load_onnx(const void *bytes, size_t size, const char *base_dir, rmlk_graph **out);
+/* The same from a file; external data is looked up next to it.
+ * ref: Builder::from_onnx_path, runtime/src/core/instance.rs:187-196 */
+int32_t rmlk_graph_load_onnx_file(const char *path, rmlk_graph **out);
+/* JSON text of a graph (inputs, initializers with an FNV-1a hash of their bytes, nodes with
+ * attributes, outputs), for tools and tests. Writes at most `size` bytes including the
+ * terminator; returns the length needed. */
+int64_t rmlk_graph_describe(const rmlk_graph *g, char *buf, int64_t size);
+
 /* ---- sessions (ref: runtime/src/core/instance.rs) ------------------------------------------- */
 /* Validates the graph, uploads the initializers to `device`, creates the stream.
  * ref: Builder::build, instance.rs:198-221 and TensorStore::init, providers/cuda/store.rs:95-261 */

@@ -121,6 +121,9 @@ SIGNATURES = {
     "rmlk_graph_attr_tensor": (c_int32, [c_void_p, c_int32, c_char_p, c_int32, POINTER(c_int64),
                                          c_int32, c_void_p]),
     "rmlk_graph_output": (c_int32, [c_void_p, c_char_p]),
+    "rmlk_graph_load_onnx": (c_int32, [c_void_p, c_size_t, c_char_p, POINTER(c_void_p)]),
+    "rmlk_graph_load_onnx_file": (c_int32, [c_char_p, POINTER(c_void_p)]),
+    "rmlk_graph_describe": (c_int64, [c_void_p, c_char_p, c_int64]),
     "rmlk_session_create": (c_int32, [c_void_p, c_int32, POINTER(c_void_p)]),
     "rmlk_session_create_ex": (c_int32, [c_void_p, c_int32, ctypes.c_uint32, POINTER(c_void_p)]),
     "rmlk_session_fused_nodes": (c_int32, [c_void_p]),

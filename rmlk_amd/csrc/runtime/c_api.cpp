@@ -92,6 +92,7 @@ int rmlk_graph::value_id(const std::string &name, bool create) {
 extern "C" {
 
 const char *rmlk_last_error(void) { return g_last_error.c_str(); }
+void rmlk_set_last_error(const char *message) { g_last_error = message ? message : ""; }
 
 int32_t rmlk_graph_create(rmlk_graph **out) {
     return guarded([&] {

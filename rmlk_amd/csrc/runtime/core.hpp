@@ -229,6 +229,7 @@ struct Session {
     bool profiling = false;
     bool fuse = true;                // form fused nodes while building
     int fused_nodes = 0;
+    int folded_nodes = 0;            // constant nodes evaluated while building
     int64_t device_syncs = 0;            // blocking reads of shape-like tensors
     int64_t device_syncs_workspace = 0;  // stream syncs taken to grow the MatMul workspace
     std::unique_ptr<CapturedPlan> plan;
@@ -249,6 +250,9 @@ struct Session {
 
 }  // namespace rt
 }  // namespace rmlk
+
+// Sets the calling thread's rmlk_last_error() text (for code outside c_api.cpp).
+extern "C" void rmlk_set_last_error(const char *message);
 
 struct rmlk_session {
     rmlk::rt::Session impl;

@@ -279,6 +279,63 @@ static Tensor upload_initializer(const HostTensor &ht, hipStream_t stream) {
     return t;
 }
 
+// Evaluate, once, the nodes whose inputs are all initializers (exported graphs compute Expand /
+// Reshape targets and masks from constants through ConstantOfShape, Mul, Equal, Where ...): their
+// outputs become initializers, with host mirrors where small, and the nodes leave the list. Nodes
+// that produce a graph output, more than 1 MiB, or an error now are left for run time.
+static int fold_constants(Session &s) {
+    rmlk_graph &g = s.graph_copy;
+    std::vector<bool> drop(g.nodes.size(), false);
+    int folded = 0;
+    for (size_t n = 0; n < g.nodes.size(); ++n) {
+        const Node &node = g.nodes[n];
+        if (node.op == "Constant") {   // already materialised by build()
+            drop[n] = true;
+            continue;
+        }
+        // Gather / ScatterND report bad indices through the device flag of a run: not folded
+        if (node.op == "Gather" || node.op == "ScatterND") continue;
+        bool constant = false;
+        for (int v : node.inputs) {
+            if (v < 0) continue;
+            constant = g.values[v].is_initializer && s.values[v].defined();
+            if (!constant) break;
+        }
+        for (int v : node.outputs)
+            if (g.values[v].is_output) constant = false;
+        if (!constant) continue;
+        OpContext ctx{s, node, static_cast<int>(n), {}, {}, s.stream};
+        for (int v : node.inputs) ctx.in.push_back(v < 0 ? nullptr : &s.values[v]);
+        std::vector<Tensor> outs(node.outputs.size());
+        for (size_t o = 0; o < outs.size(); ++o) ctx.out.push_back(&outs[o]);
+        try {
+            find_op(node.op)(ctx);
+        } catch (const RtError &) {
+            continue;
+        }
+        bool small = true;
+        for (const Tensor &t : outs)
+            if (!t.defined() || t.nbytes() > (1u << 20)) small = false;
+        if (!small) continue;
+        for (size_t o = 0; o < outs.size(); ++o) {
+            s.values[node.outputs[o]] = outs[o];
+            g.values[node.outputs[o]].is_initializer = true;
+        }
+        drop[n] = true;
+        ++folded;
+    }
+    check_hip(hipStreamSynchronize(s.stream), "hipStreamSynchronize");
+    s.scratch_bufs.clear();
+    std::vector<Node> kept;
+    for (size_t n = 0; n < g.nodes.size(); ++n)
+        if (!drop[n]) kept.push_back(std::move(g.nodes[n]));
+    g.nodes = std::move(kept);
+    for (Value &v : g.values) v.producer = -1;
+    for (size_t n = 0; n < g.nodes.size(); ++n)
+        for (int v : g.nodes[n].outputs) g.values[v].producer = static_cast<int>(n);
+    return folded;
+}
+
 void Session::build(const rmlk_graph &graph, int dev) {
     graph_copy = graph;
     g = &graph_copy;
@@ -348,7 +405,10 @@ void Session::build(const rmlk_graph &graph, int dev) {
         values[node.outputs[0]] = upload_initializer(ht, stream);
     }
     check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
-    if (fuse) fused_nodes = fuse_patterns(*this);
+    if (fuse) {
+        folded_nodes = fold_constants(*this);
+        fused_nodes = fuse_patterns(*this);
+    }
     // liveness over the final node list
     last_use.assign(g->values.size(), -1);
     stats.assign(g->nodes.size(), NodeStat());

@@ -296,6 +296,19 @@ class Builder:
     def from_graph(graph: Graph) -> "Builder":
         return Builder(graph)
 
+    @staticmethod
+    def from_onnx_path(path) -> "Builder":
+        """ref: Builder::from_onnx_path (runtime/src/core/instance.rs:187-196); external tensor
+        data is looked up next to the file."""
+        from .onnx_io import load_onnx
+        return Builder(load_onnx(path))
+
+    @staticmethod
+    def from_onnx_bytes(data: bytes, base_dir=None) -> "Builder":
+        """ref: graph_from_onnx_bytes (schema/src/onnx_import/transform.rs:249-258)."""
+        from .onnx_io import load_onnx_bytes
+        return Builder(load_onnx_bytes(data, base_dir))
+
     def build(self, device: int = 0, fuse: bool = True) -> ModelInstance:
         """fuse=False keeps one kernel per node, as the reference executes a graph."""
         return ModelInstance(self._graph, device, fuse)
