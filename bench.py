@@ -133,21 +133,24 @@ def run_llama(args):
     inst.set_profiling(False)
     stats = inst.node_stats()
     # classify each MatMul node by the kernel the library picks for its shape
-    shapes = matmul_shapes(cfg, prompt_len, max_len)
-    mm_nodes = [s for s in stats if s["op"] in ("MatMul", "rmlk.AttnMatMul")]
-    assert len(mm_nodes) == len(shapes), (len(mm_nodes), len(shapes))
+    launches = matmul_launches(cfg, prompt_len, max_len)
+    mm_nodes = [s for s in stats if s["op"] in ("MatMul", "rmlk.AttnMatMul", "rmlk.MatMulGroup")]
+    assert len(mm_nodes) == len(launches), (len(mm_nodes), len(launches))
     by_kind, per_op = {}, {}
-    for s, (batch, m, n, k) in zip(mm_nodes, shapes):
-        kind = kernels.matmul_describe(batch, m, n, k)
-        d = by_kind.setdefault(kind, {"launches": 0, "us": 0.0, "flops": 0.0, "alg_bytes": 0.0,
-                                      "traffic": 0.0, "shapes": {}})
-        d["launches"] += 1
-        d["shapes"][(batch, m, n, k)] = d["shapes"].get((batch, m, n, k), 0) + 1
-        d["us"] += s["micros"]
-        d["flops"] += 2.0 * batch * m * n * k
-        d["alg_bytes"] += 4.0 * batch * (m * k + k * n + m * n)
-        pmc = PMC_TRAFFIC_KIB.get((batch, m, n, k))
-        d["traffic"] = None if pmc is None or d["traffic"] is None else d["traffic"] + 1024.0 * sum(pmc)
+    for s, shapes in zip(mm_nodes, launches):
+        node_flops = sum(2.0 * b_ * m * n * k for b_, m, n, k in shapes)
+        for batch, m, n, k in shapes:
+            kind = kernels.matmul_describe(batch, m, n, k)
+            d = by_kind.setdefault(kind, {"launches": 0, "us": 0.0, "flops": 0.0, "alg_bytes": 0.0,
+                                          "traffic": 0.0, "shapes": {}})
+            d["launches"] += 1
+            d["shapes"][(batch, m, n, k)] = d["shapes"].get((batch, m, n, k), 0) + 1
+            flops = 2.0 * batch * m * n * k
+            d["us"] += s["micros"] * flops / node_flops     # a node of several launches: by flops
+            d["flops"] += flops
+            d["alg_bytes"] += 4.0 * batch * (m * k + k * n + m * n)
+            pmc = PMC_TRAFFIC_KIB.get((batch, m, n, k))
+            d["traffic"] = None if pmc is None or d["traffic"] is None else d["traffic"] + 1024.0 * sum(pmc)
     for s in stats:
         if s["micros"] > 0:
             d = per_op.setdefault(s["op"], {"n": 0, "us": 0.0, "bytes": 0.0})
@@ -301,17 +304,20 @@ def decode_weight_bytes(cfg):
     return 4.0 * (cfg.layers * per_layer + cfg.hidden * cfg.vocab)
 
 
-def matmul_shapes(cfg, s, max_len):
-    """(batch, m, n, k) of every MatMul node of the scatter-style graph in node order."""
+def matmul_launches(cfg, s, max_len):
+    """(batch, m, n, k) of the GEMM launches behind every MatMul-type node of the fused scatter-style
+    graph, in node order: [q, k, v] (one node), scores, context, o, [gate, up] (one node), down per
+    layer, then the lm-head."""
     h, kvd, d = cfg.hidden, cfg.kv_heads * cfg.head_dim, cfg.head_dim
     rep = cfg.heads // cfg.kv_heads
     out = []
     for _ in range(cfg.layers):
-        # the two attention products run as one strided GEMM per KV head over its group of q heads
-        out += [(1, s, cfg.heads * d, h), (1, s, kvd, h), (1, s, kvd, h),
-                (cfg.kv_heads, rep * s, max_len, d), (cfg.kv_heads, rep * s, d, max_len),
-                (1, s, h, cfg.heads * d), (1, s, cfg.ffn, h), (1, s, cfg.ffn, h), (1, s, h, cfg.ffn)]
-    out.append((1, s, cfg.vocab, h))
+        out += [[(1, s, cfg.heads * d, h), (1, s, kvd, h), (1, s, kvd, h)],
+                # the two attention products run as one strided GEMM per KV head over its q heads
+                [(cfg.kv_heads, rep * s, max_len, d)], [(cfg.kv_heads, rep * s, d, max_len)],
+                [(1, s, h, cfg.heads * d)], [(1, s, cfg.ffn, h), (1, s, cfg.ffn, h)],
+                [(1, s, h, cfg.ffn)]]
+    out.append([(1, s, cfg.vocab, h)])
     return out
 
 

@@ -12,6 +12,7 @@
 //   rmlk.ScaleMaskSoftmax  Div|Mul(x,c) Add(mask) Softmax(-1)
 //   rmlk.Rotary            [Transpose(0,2,1,3)] Slice Slice Neg Concat Mul Mul Add
 //   rmlk.AttnMatMul        MatMul(a, [Transpose(0,1,3,2)] [Reshape Expand Unsqueeze] (kv))
+//   rmlk.MatMulGroup       MatMul(a, W1), MatMul(a, W2), ... on the same a with constant 2-D weights
 //
 // A fused node keeps the nodes it replaced as its `body`. What cannot be decided while building
 // (shapes are only known at run time) is checked when the node runs; if the fused kernel does not
@@ -408,6 +409,102 @@ struct Matcher {
         replace(parts, std::move(f));
         return true;
     }
+
+    // ---- MatMuls that share their first operand and have constant 2-D weights (q/k/v, gate/up) ----
+    // The weights are laid side by side in ONE device matrix [K, N1 + N2 + ..] while building (the
+    // separate copies are released unless something else reads them). A one-row input then takes a
+    // single weight-streaming launch whose result is handed out as views; more rows take one GEMM
+    // per member on its column block of the joint matrix (leading dimension = the joint width), i.e.
+    // exactly the separate products. Nothing is left for a fallback body.
+    int form_matmul_groups() {
+        int formed = 0;
+        const size_t n_nodes = g.nodes.size();
+        for (size_t first = 0; first < n_nodes; ++first) {
+            if (removed[first] || g.nodes[first].op != "MatMul") continue;
+            auto weight_ok = [&](const Node &mm, int64_t *k, int64_t *n) {
+                if (mm.inputs.size() != 2 || mm.inputs[0] < 0 || mm.inputs[1] < 0) return false;
+                const int w = mm.inputs[1];
+                if (!g.values[w].is_initializer) return false;
+                const Tensor &t = s.values[w];
+                if (!t.defined() || t.dtype != RMLK_FLOAT || t.rank() != 2 || t.shape[1] % 4 != 0 ||
+                    t.shape[0] == 0 || t.shape[1] == 0)
+                    return false;
+                *k = t.shape[0];
+                *n = t.shape[1];
+                return true;
+            };
+            int64_t k0, n0;
+            if (!weight_ok(g.nodes[first], &k0, &n0)) continue;
+            const int a = g.nodes[first].inputs[0];
+            std::vector<size_t> members = {first};
+            std::vector<int64_t> widths = {n0};
+            for (size_t j = first + 1; j < n_nodes; ++j) {
+                if (removed[j] || g.nodes[j].op != "MatMul" || g.nodes[j].inputs.empty() ||
+                    g.nodes[j].inputs[0] != a)
+                    continue;
+                int64_t k, n;
+                if (!weight_ok(g.nodes[j], &k, &n) || k != k0) continue;
+                members.push_back(j);
+                widths.push_back(n);
+            }
+            if (members.size() < 2) continue;
+            int64_t total = 0;
+            for (int64_t w : widths) total += w;
+            // the joint weight matrix
+            Tensor joint;
+            joint.dtype = RMLK_FLOAT;
+            joint.shape = {k0, total};
+            auto buf = std::make_shared<Buffer>();
+            buf->bytes = joint.nbytes();
+            buf->owned_raw = true;
+            check_hip(hipMalloc(&buf->ptr, buf->bytes), "hipMalloc (joint weights)");
+            joint.buf = buf;
+            rmlk_dims out_shape = to_dims(joint.shape);
+            int64_t off = 0;
+            for (size_t i = 0; i < members.size(); ++i) {
+                const Tensor &w = s.values[g.nodes[members[i]].inputs[1]];
+                rmlk_dims in_shape = to_dims(w.shape);
+                check_status(rmlk_hip_concat(s.stream, RMLK_FLOAT, &in_shape, &out_shape, 1, off,
+                                             w.data(), joint.data()),
+                             "joint weights");
+                off += widths[i];
+            }
+            check_hip(hipStreamSynchronize(s.stream), "hipStreamSynchronize");
+            const int joint_id = static_cast<int>(g.values.size());
+            Value jv;
+            jv.name = "rmlk.joint_weights." + std::to_string(first);
+            jv.dtype = RMLK_FLOAT;
+            jv.shape = joint.shape;
+            jv.is_initializer = true;
+            g.values.push_back(jv);
+            g.by_name[jv.name] = joint_id;
+            s.values.push_back(joint);
+            users.emplace_back();
+            Node f;
+            f.op = "rmlk.MatMulGroup";
+            f.inputs = {a, joint_id};
+            f.attrs["widths"] = a_ints(widths);
+            for (size_t i = 0; i < members.size(); ++i) {
+                const Node &mm = g.nodes[members[i]];
+                f.outputs.push_back(mm.outputs[0]);
+                const int w = mm.inputs[1];
+                removed[members[i]] = true;
+                for (int v : mm.inputs) {
+                    auto &u = users[v];
+                    u.erase(std::remove(u.begin(), u.end(), static_cast<int>(members[i])), u.end());
+                }
+                // release a weight nobody else reads (another member may share it)
+                if (users[w].empty() && !g.values[w].is_output) s.values[w].reset();
+            }
+            g.nodes[first] = std::move(f);
+            removed[first] = false;
+            users[a].push_back(static_cast<int>(first));
+            users[joint_id].push_back(static_cast<int>(first));
+            for (int v : g.nodes[first].outputs) g.values[v].producer = static_cast<int>(first);
+            ++formed;
+        }
+        return formed;
+    }
 };
 
 // Run the nodes a fused node replaced, one kernel each.
@@ -427,6 +524,10 @@ void run_body(OpContext &c) {
         for (size_t o = 0; o < outs.size(); ++o) local[n.outputs[o]] = outs[o];
     }
     for (size_t o = 0; o < c.node.outputs.size(); ++o) *c.out[o] = local[c.node.outputs[o]];
+}
+
+void require_float(int32_t dt) {
+    if (dt != RMLK_FLOAT) fail_unsupported(dt);
 }
 
 float attr_float(const OpContext &c, const char *name) {
@@ -636,6 +737,59 @@ void op_fused_attn_matmul(OpContext &c) {
     run_body(c);
 }
 
+// MatMul(a, W_i) for every member of a group, W_i being column blocks of one joint matrix.
+void op_fused_matmul_group(OpContext &c) {
+    const Tensor &a = c.input(0), &w = c.input(1);
+    const std::vector<int64_t> widths = c.attr_ints("widths");
+    require_float(a.dtype);
+    if (a.rank() == 0) fail_op("ZeroRank");
+    const int64_t k = w.shape[0], total = w.shape[1];
+    if (a.shape.back() != k) fail_op("IncompatibleDimForMul");
+    const int64_t m = k ? a.numel() / k : 0;
+    std::vector<int64_t> lead(a.shape.begin(), a.shape.end() - 1);   // 1-D a: the row dim is dropped
+    auto out_shape = [&](int64_t n) {
+        std::vector<int64_t> sh = lead;
+        sh.push_back(n);
+        return sh;
+    };
+    auto run = [&](int64_t n, const void *b, void *out, int64_t ldc) {
+        const size_t ws_bytes = rmlk_hip_matmul_workspace_size(RMLK_FLOAT, 1, m, n, k);
+        void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
+        check_status(rmlk_hip_matmul(c.stream, RMLK_FLOAT, 1, m, n, k, a.data(), k, 0, 0, b, total, 0, 0,
+                                     out, ldc, 0, ws, ws_bytes),
+                     "rmlk.MatMulGroup");
+    };
+    if (m == 1) {
+        // one launch over the joint matrix; the members' results are slices of its output row
+        Tensor row;
+        {
+            std::vector<Tensor *> keep = c.out;
+            c.out = {&row};
+            c.alloc_output(0, RMLK_FLOAT, {total});
+            c.out = keep;
+        }
+        run(total, w.data(), row.data(), total);
+        int64_t off = 0;
+        for (size_t i = 0; i < widths.size(); ++i) {
+            Tensor v;
+            v.dtype = RMLK_FLOAT;
+            v.shape = out_shape(widths[i]);
+            v.buf = row.buf;
+            v.offset = row.offset + static_cast<size_t>(off) * sizeof(float);
+            *c.out[i] = v;
+            off += widths[i];
+        }
+        return;
+    }
+    int64_t off = 0;
+    for (size_t i = 0; i < widths.size(); ++i) {
+        Tensor &y = c.alloc_output(static_cast<int>(i), RMLK_FLOAT, out_shape(widths[i]));
+        if (y.numel() > 0)
+            run(widths[i], static_cast<const float *>(w.data()) + off, y.data(), widths[i]);
+        off += widths[i];
+    }
+}
+
 // Rewrite the session's node list; returns how many fused nodes were formed.
 int fuse_patterns(Session &s) {
     Matcher m(s);
@@ -654,6 +808,7 @@ int fuse_patterns(Session &s) {
             if (m.match_attn_matmul(node)) ++formed;
         }
     }
+    formed += m.form_matmul_groups();
     if (!formed) return 0;
     std::vector<Node> kept;
     kept.reserve(m.g.nodes.size());

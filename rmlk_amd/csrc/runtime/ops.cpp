@@ -828,6 +828,7 @@ const std::unordered_map<std::string, OpFn> &registry() {
         {"rmlk.ScaleMaskSoftmax", op_fused_softmax},
         {"rmlk.Rotary", op_fused_rotary},
         {"rmlk.AttnMatMul", op_fused_attn_matmul},
+        {"rmlk.MatMulGroup", op_fused_matmul_group},
     };
     return table;
 }

@@ -480,10 +480,12 @@ void Session::run_nodes() {
             }
             if (node.op == "ScatterND" && !any_new) bytes += static_cast<double>(ctx.in[2]->nbytes());
         }
-        if ((node.op == "MatMul" || node.op == "rmlk.AttnMatMul") && ctx.in[0] &&
-            !ctx.in[0]->shape.empty())
-            flops = 2.0 * static_cast<double>(outs[0].numel()) *
-                    static_cast<double>(ctx.in[0]->shape.back());
+        if ((node.op == "MatMul" || node.op == "rmlk.AttnMatMul" || node.op == "rmlk.MatMulGroup") &&
+            ctx.in[0] && !ctx.in[0]->shape.empty()) {
+            double out_elems = 0.0;
+            for (const Tensor &t : outs) out_elems += static_cast<double>(t.numel());
+            flops = 2.0 * out_elems * static_cast<double>(ctx.in[0]->shape.back());
+        }
         st.bytes = bytes;
         st.flops = flops;
         for (size_t o = 0; o < node.outputs.size(); ++o) values[node.outputs[o]] = outs[o];

@@ -210,8 +210,9 @@ def test_pass_forms_the_expected_nodes_on_the_llama_graph(device):
         for kv in ("key", "value"):
             feeds[f"cache.{l}.{kv}"] = np.zeros((1, cfg.kv_heads, 24, cfg.head_dim), np.float32)
     a, b, n, _ = _run_both(graph, feeds)
-    # per layer: 2 RMSNorm, 2 rotary, 1 SwiGLU, 1 softmax, 2 attention MatMuls; plus the final RMSNorm
-    assert n == cfg.layers * 8 + 1
+    # per layer: 2 RMSNorm, 2 rotary, 1 SwiGLU, 1 softmax, 2 attention MatMuls, the q/k/v and the
+    # gate/up MatMul groups; plus the final RMSNorm
+    assert n == cfg.layers * 10 + 1
     # RMSNorm's mean may differ in the last place; everything downstream inherits that
     _same(a, b, loose=set(a.keys()))
     assert np.array_equal(np.argmax(a["logits"][0], -1), np.argmax(b["logits"][0], -1))
@@ -224,7 +225,7 @@ def test_fused_llama_concat_style_against_oracle(device):
     graph = graphs.llama_graph(cfg, seed=4, style="concat")
     feeds = graphs.llama_concat_inputs(cfg, np.random.default_rng(1).integers(0, cfg.vocab, 9), None, 0)
     inst = runtime.Builder.from_graph(graph).build()
-    assert inst.fused_nodes == cfg.layers * 8 + 1
+    assert inst.fused_nodes == cfg.layers * 10 + 1
     got = inst.run(feeds)
     exp = og.run_graph(graph, feeds)
     for name in exp:
@@ -236,7 +237,7 @@ def test_fused_decoder_layer_full_width(device):
     from rmlk_amd import graphs
     graph, feeds = graphs.decoder_layer_graph(seed=3, seq=96)
     a, b, n, _ = _run_both(graph, feeds)
-    assert n == 8
+    assert n == 10
     _same(a, b, loose={"y"})
 
 
@@ -438,3 +439,50 @@ def test_user_graph_cannot_name_internal_ops(device):
     g.output("y")
     with pytest.raises(Exception, match="unsupported operator"):
         runtime.Builder.from_graph(g.build()).build()
+
+
+@pytest.mark.parametrize("rows", [1, 3, 40])
+def test_matmul_group_hands_out_the_separate_products(device, rows):
+    """Three MatMuls on one input with constant weights become one node; one input row takes a
+    single launch over the joint weight matrix (results are views of one row), more rows one GEMM
+    per member on its column block."""
+    from oracle import graph as og
+    gb = _builder()
+    gb.input("x", np.float32, [1, 0, 96])
+    rng = np.random.default_rng(rows)
+    for name, n in (("wq", 64), ("wk", 32), ("wv", 32)):
+        gb.constant(name, (rng.standard_normal((96, n)) * 0.1).astype(np.float32))
+    gb.op("MatMul", ["x", "wq"], ["q"])
+    gb.op("Neg", ["q"], ["qn"])               # a consumer between the members
+    gb.op("MatMul", ["x", "wk"], ["k"])
+    gb.op("MatMul", ["x", "wv"], ["v"])
+    gb.op("Add", ["k", "v"], ["kv"])
+    for o in ("qn", "k", "v", "kv"):
+        gb.output(o)
+    graph = gb.build()
+    feeds = {"x": rng.standard_normal((1, rows, 96), dtype=np.float32)}
+    a, b, n, _ = _run_both(graph, feeds)
+    assert n == 1
+    exp = og.run_graph(graph, feeds)
+    for name in a:
+        assert a[name].shape == b[name].shape == exp[name].shape
+        assert_close(a[name], b[name], rtol=1e-4, atol=1e-5)
+        assert_close(a[name], exp[name], rtol=1e-4, atol=1e-5)
+
+
+def test_matmul_group_keeps_a_weight_that_something_else_reads(device):
+    gb = _builder()
+    gb.input("x", np.float32, [2, 8])
+    rng = np.random.default_rng(1)
+    gb.constant("w1", rng.standard_normal((8, 8)).astype(np.float32))
+    gb.constant("w2", rng.standard_normal((8, 4)).astype(np.float32))
+    gb.op("MatMul", ["x", "w1"], ["a"])
+    gb.op("MatMul", ["x", "w2"], ["b"])
+    gb.op("MatMul", ["a", "w1"], ["c"])       # w1 again, on another input
+    for o in ("a", "b", "c"):
+        gb.output(o)
+    feeds = {"x": rng.standard_normal((2, 8), dtype=np.float32)}
+    a, b, n, _ = _run_both(gb.build(), feeds)
+    assert n == 1
+    for name in a:
+        assert_close(a[name], b[name], rtol=1e-4, atol=1e-5)
