@@ -224,7 +224,7 @@ int32_t rmlk_hip_trilu(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64
 
 /* ---- fused operator chains --------------------------------------------------------------------
  * The reference launches one kernel per ONNX node (runtime/src/providers/cuda/backend/<op>.rs); the
- * four entry points below have no single counterpart there. Each computes, in one pass over
+ * entry points below have no single counterpart there. Each computes, in one pass over
  * memory, the chain of nodes named in its comment, and rounds every intermediate exactly as the
  * separate kernels do, so a graph gives the same result either way. They support fp32 and return
  * RMLK_ERR_UNSUPPORTED for layouts they do not cover (the caller then runs the separate kernels).
@@ -238,6 +238,13 @@ int32_t rmlk_hip_trilu(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64
 int32_t rmlk_hip_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t rows, int64_t cols,
                          const void *x, const void *gamma, float eps, int32_t reciprocal_form,
                          void *out);
+
+/* sum_out = a + b (same dense [rows, cols] shape), out = RMSNorm(sum_out) as above, in one pass:
+ * the residual Add in front of a norm, whose result the residual stream reads again.
+ * Chain: Add -> the RMSNorm chain. */
+int32_t rmlk_hip_add_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t rows, int64_t cols,
+                             const void *a, const void *b, const void *gamma, float eps,
+                             int32_t reciprocal_form, void *sum_out, void *out);
 
 /* out = Softmax(x / scale + mask) (scale_is_mul == 0) or Softmax(x * scale + mask) over the last
  * axis. `shape` is x's (and out's) dense shape; `mask_stride` gives the mask's element stride per

@@ -85,6 +85,8 @@ SIGNATURES = {
                                  c_void_p, c_void_p]),
     "rmlk_hip_rmsnorm": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p,
                                    ctypes.c_float, c_int32, c_void_p]),
+    "rmlk_hip_add_rmsnorm": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p,
+                                       c_void_p, ctypes.c_float, c_int32, c_void_p, c_void_p]),
     "rmlk_hip_scale_mask_softmax": (c_int32, [c_void_p, c_int32, _PD, _PD, c_int32, ctypes.c_float,
                                               c_void_p, c_void_p, c_void_p]),
     "rmlk_hip_swiglu": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p]),

@@ -329,8 +329,20 @@ int32_t softmax_typed(hipStream_t s, int64_t outer, int64_t n, int64_t inner, co
 // The fused form of Pow(2) -> ReduceMean(-1) -> Add(eps) -> Sqrt -> Div -> Mul(gamma): squares are
 // rounded to float before the double accumulation and every later step rounds like the separate
 // kernel does. RECIP selects the exported variant x * (1 / sqrt(..)) * gamma.
+// The row may also be formed on the fly: x + add (the residual Add in front of the norm), or
+// residual + the sum of split-K partial slabs of a preceding GEMV; the formed row is then stored
+// to sum_out as well, because the residual stream reads it again later.
+struct RmsSource {
+    const float *x;       // the row, or the residual when add / ws is given
+    const float *add;     // second Add operand, or null
+    const float *ws;      // split-K partials [splits][slab], or null
+    int32_t splits;
+    int64_t slab;         // elements between consecutive partial slabs
+    float *sum_out;       // where the formed row goes (null: nowhere)
+};
+
 template <int NV, int kGroup, bool RECIP>
-__global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const float *__restrict__ x,
+__global__ __launch_bounds__(kBlock) void rmsnorm_kernel(RmsSource src,
                                                          const float *__restrict__ gamma,
                                                          float *__restrict__ out, int64_t rows,
                                                          int32_t cols, float eps) {
@@ -350,7 +362,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const float *__restrict
          row0 += static_cast<int64_t>(gridDim.x) * kRowsPerBlock) {
         const int64_t row = row0 + group;
         const bool live = row < rows;
-        const V *pv = reinterpret_cast<const V *>(x + row * cols);
+        const V *pv = reinterpret_cast<const V *>(src.x + row * cols);
         V xv[NV];
         double acc = 0.0;
 #pragma unroll
@@ -358,6 +370,23 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const float *__restrict
             const int c = lane_in_group + i * kGroup;
             if (live && c < nv) {
                 xv[i] = pv[c];
+                if (src.add) {
+                    const V av = reinterpret_cast<const V *>(src.add + row * cols)[c];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) xv[i].v[j] = xv[i].v[j] + av.v[j];
+                } else if (src.ws) {
+                    const V *pw = reinterpret_cast<const V *>(src.ws + row * cols) + c;
+                    V t = *pw;
+                    for (int z = 1; z < src.splits; ++z) {
+                        const V p = *reinterpret_cast<const V *>(
+                            reinterpret_cast<const float *>(pw) + z * src.slab);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) t.v[j] += p.v[j];
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) xv[i].v[j] = xv[i].v[j] + t.v[j];
+                }
+                if (src.sum_out) reinterpret_cast<V *>(src.sum_out + row * cols)[c] = xv[i];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const float sq = xv[i].v[j] * xv[i].v[j];
@@ -397,16 +426,35 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const float *__restrict
 }
 
 template <int NV, int kGroup>
-int32_t launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *out, int64_t rows,
-                       int32_t cols, float eps, bool recip) {
+int32_t launch_rmsnorm(hipStream_t s, const RmsSource &src, const float *gamma, float *out,
+                       int64_t rows, int32_t cols, float eps, bool recip) {
     constexpr int kRowsPerBlock = kBlock / kGroup;
     int64_t blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
     const int64_t cap = static_cast<int64_t>(kNumCU) * 32;
     if (blocks > cap) blocks = cap;
     const unsigned grid = static_cast<unsigned>(blocks);
-    if (recip) rmsnorm_kernel<NV, kGroup, true><<<grid, kBlock, 0, s>>>(x, gamma, out, rows, cols, eps);
-    else rmsnorm_kernel<NV, kGroup, false><<<grid, kBlock, 0, s>>>(x, gamma, out, rows, cols, eps);
+    if (recip) rmsnorm_kernel<NV, kGroup, true><<<grid, kBlock, 0, s>>>(src, gamma, out, rows, cols, eps);
+    else rmsnorm_kernel<NV, kGroup, false><<<grid, kBlock, 0, s>>>(src, gamma, out, rows, cols, eps);
     return launch_status();
+}
+
+int32_t rmsnorm_dispatch(hipStream_t s, const RmsSource &src, const float *gp, float *op, int64_t rows,
+                         int64_t cols, float eps, bool recip) {
+    auto aligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    const bool vec_ok = cols % 4 == 0 && aligned(src.x) && aligned(src.add) && aligned(src.ws) &&
+                        aligned(src.sum_out) && aligned(gp) && aligned(op) && src.slab % 4 == 0;
+    if (!vec_ok || cols > kBlock * 4 * 8) return RMLK_ERR_UNSUPPORTED;
+    const int32_t c = static_cast<int32_t>(cols);
+    if (rows >= 1024 && c <= kWave * 4 * 8) {  // many rows: a wavefront per row
+        if (c <= 256) return launch_rmsnorm<1, kWave>(s, src, gp, op, rows, c, eps, recip);
+        if (c <= 512) return launch_rmsnorm<2, kWave>(s, src, gp, op, rows, c, eps, recip);
+        if (c <= 1024) return launch_rmsnorm<4, kWave>(s, src, gp, op, rows, c, eps, recip);
+        return launch_rmsnorm<8, kWave>(s, src, gp, op, rows, c, eps, recip);
+    }
+    if (c <= 1024) return launch_rmsnorm<1, kBlock>(s, src, gp, op, rows, c, eps, recip);
+    if (c <= 2048) return launch_rmsnorm<2, kBlock>(s, src, gp, op, rows, c, eps, recip);
+    if (c <= 4096) return launch_rmsnorm<4, kBlock>(s, src, gp, op, rows, c, eps, recip);
+    return launch_rmsnorm<8, kBlock>(s, src, gp, op, rows, c, eps, recip);
 }
 
 template <typename T>
@@ -537,25 +585,24 @@ extern "C" int32_t rmlk_hip_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t
     if (rows == 0 || cols == 0) return RMLK_OK;
     if (!x || !gamma || !out) return RMLK_ERR_NULL_POINTER;
     if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
-    const bool vec_ok = cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
-                        reinterpret_cast<uintptr_t>(gamma) % 16 == 0 &&
-                        reinterpret_cast<uintptr_t>(out) % 16 == 0;
-    if (!vec_ok || cols > kBlock * 4 * 8) return RMLK_ERR_UNSUPPORTED;
-    hipStream_t s = as_stream(stream);
-    const float *xp = static_cast<const float *>(x), *gp = static_cast<const float *>(gamma);
-    float *op = static_cast<float *>(out);
-    const int32_t c = static_cast<int32_t>(cols);
-    const bool recip = reciprocal_form != 0;
-    if (rows >= 1024 && c <= kWave * 4 * 8) {  // many rows: a wavefront per row
-        if (c <= 256) return launch_rmsnorm<1, kWave>(s, xp, gp, op, rows, c, eps, recip);
-        if (c <= 512) return launch_rmsnorm<2, kWave>(s, xp, gp, op, rows, c, eps, recip);
-        if (c <= 1024) return launch_rmsnorm<4, kWave>(s, xp, gp, op, rows, c, eps, recip);
-        return launch_rmsnorm<8, kWave>(s, xp, gp, op, rows, c, eps, recip);
-    }
-    if (c <= 1024) return launch_rmsnorm<1, kBlock>(s, xp, gp, op, rows, c, eps, recip);
-    if (c <= 2048) return launch_rmsnorm<2, kBlock>(s, xp, gp, op, rows, c, eps, recip);
-    if (c <= 4096) return launch_rmsnorm<4, kBlock>(s, xp, gp, op, rows, c, eps, recip);
-    return launch_rmsnorm<8, kBlock>(s, xp, gp, op, rows, c, eps, recip);
+    RmsSource src{static_cast<const float *>(x), nullptr, nullptr, 0, 0, nullptr};
+    return rmsnorm_dispatch(as_stream(stream), src, static_cast<const float *>(gamma),
+                            static_cast<float *>(out), rows, cols, eps, reciprocal_form != 0);
+}
+
+extern "C" int32_t rmlk_hip_add_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t rows,
+                                        int64_t cols, const void *a, const void *b,
+                                        const void *gamma, float eps, int32_t reciprocal_form,
+                                        void *sum_out, void *out) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (rows < 0 || cols < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (rows == 0 || cols == 0) return RMLK_OK;
+    if (!a || !b || !gamma || !sum_out || !out) return RMLK_ERR_NULL_POINTER;
+    if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
+    RmsSource src{static_cast<const float *>(a), static_cast<const float *>(b), nullptr, 0, 0,
+                  static_cast<float *>(sum_out)};
+    return rmsnorm_dispatch(as_stream(stream), src, static_cast<const float *>(gamma),
+                            static_cast<float *>(out), rows, cols, eps, reciprocal_form != 0);
 }
 
 extern "C" int32_t rmlk_hip_scale_mask_softmax(rmlk_stream_t stream, int32_t dtype,

@@ -201,6 +201,7 @@ OpFn find_op(const std::string &name);
 int fuse_patterns(Session &s);
 void op_fused_rmsnorm(OpContext &c);
 void op_fused_swiglu(OpContext &c);
+void op_fused_add_rmsnorm(OpContext &c);
 void op_fused_softmax(OpContext &c);
 void op_fused_rotary(OpContext &c);
 void op_fused_attn_matmul(OpContext &c);

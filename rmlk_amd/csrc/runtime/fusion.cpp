@@ -8,6 +8,7 @@
 // instead drops two copies: the grouped-query Expand and the K transpose become GEMM strides):
 //
 //   rmlk.RMSNorm           Pow(x,2) ReduceMean(-1) Add(eps) Sqrt Div|(Div(1,.) Mul) Mul(gamma)
+//   rmlk.AddRMSNorm        Add(a,b) followed by rmlk.RMSNorm: the sum is an output too
 //   rmlk.SwiGLU            Sigmoid(g) Mul(g,.) Mul(.,u)
 //   rmlk.ScaleMaskSoftmax  Div|Mul(x,c) Add(mask) Softmax(-1)
 //   rmlk.Rotary            [Transpose(0,2,1,3)] Slice Slice Neg Concat Mul Mul Add
@@ -410,6 +411,38 @@ struct Matcher {
         return true;
     }
 
+    // ---- residual Add in front of an RMSNorm node: one pass, two outputs ---------------------------
+    int form_add_rmsnorm() {
+        int formed = 0;
+        for (size_t n = 0; n < g.nodes.size(); ++n) {
+            if (removed[n] || g.nodes[n].op != "rmlk.RMSNorm") continue;
+            const Node &norm = g.nodes[n];
+            const int x = norm.inputs[0], gamma = norm.inputs[1];
+            const Node *add = produced_by(x, "Add");
+            if (!add || add->inputs.size() != 2 || add->inputs[0] < 0 || add->inputs[1] < 0) continue;
+            // the fused node sits where the Add was: gamma must exist there already
+            const int at = index_of(add);
+            const Value &gv = g.values[gamma];
+            if (!gv.is_initializer && !gv.is_input && !(gv.producer >= 0 && gv.producer < at)) continue;
+            Node f;
+            f.op = "rmlk.AddRMSNorm";
+            f.inputs = {add->inputs[0], add->inputs[1], gamma};
+            f.outputs = {x, norm.outputs[0]};
+            f.attrs = norm.attrs;
+            f.body = {*add, norm};
+            auto &ux = users[x];
+            ux.erase(std::remove(ux.begin(), ux.end(), static_cast<int>(n)), ux.end());
+            auto &ug = users[gamma];
+            ug.erase(std::remove(ug.begin(), ug.end(), static_cast<int>(n)), ug.end());
+            ug.push_back(at);
+            removed[n] = true;
+            g.nodes[at] = std::move(f);
+            for (int v : g.nodes[at].outputs) g.values[v].producer = at;
+            ++formed;
+        }
+        return formed;
+    }
+
     // ---- MatMuls that share their first operand and have constant 2-D weights (q/k/v, gate/up) ----
     // The weights are laid side by side in ONE device matrix [K, N1 + N2 + ..] while building (the
     // separate copies are released unless something else reads them). A one-row input then takes a
@@ -511,6 +544,10 @@ struct Matcher {
 void run_body(OpContext &c) {
     Session &s = c.session;
     std::unordered_map<int, Tensor> local;
+    // the fused node's own inputs come from its context (a body may be nested inside another body,
+    // whose intermediates are not session values)
+    for (size_t i = 0; i < c.node.inputs.size(); ++i)
+        if (c.node.inputs[i] >= 0 && c.in[i]) local[c.node.inputs[i]] = *c.in[i];
     auto lookup = [&](int v) -> Tensor * {
         auto it = local.find(v);
         return it != local.end() ? &it->second : &s.values[v];
@@ -737,6 +774,30 @@ void op_fused_attn_matmul(OpContext &c) {
     run_body(c);
 }
 
+void op_fused_add_rmsnorm(OpContext &c) {
+    const Tensor &a = c.input(0), &b = c.input(1), &gamma = c.input(2);
+    const int rank = a.rank();
+    bool ok = a.dtype == RMLK_FLOAT && b.dtype == RMLK_FLOAT && gamma.dtype == RMLK_FLOAT &&
+              a.shape == b.shape && rank >= 1 && a.numel() > 0;
+    if (ok) {
+        const int64_t axis = c.attr_int("axis", -1);
+        ok = (axis == -1 || axis == rank - 1) && gamma.rank() >= 1 && gamma.rank() <= rank &&
+             gamma.shape.back() == a.shape.back() && gamma.numel() == a.shape.back();
+    }
+    if (ok) {
+        const int64_t cols = a.shape.back(), rows = a.numel() / cols;
+        Tensor &sum = c.alloc_output(0, RMLK_FLOAT, a.shape);
+        Tensor &y = c.alloc_output(1, RMLK_FLOAT, a.shape);
+        if (took_fast_path(rmlk_hip_add_rmsnorm(c.stream, RMLK_FLOAT, rows, cols, a.data(), b.data(),
+                                                gamma.data(), attr_float(c, "epsilon"),
+                                                static_cast<int32_t>(c.attr_int("reciprocal", 0)),
+                                                sum.data(), y.data()),
+                           "rmlk.AddRMSNorm"))
+            return;
+    }
+    run_body(c);
+}
+
 // MatMul(a, W_i) for every member of a group, W_i being column blocks of one joint matrix.
 void op_fused_matmul_group(OpContext &c) {
     const Tensor &a = c.input(0), &w = c.input(1);
@@ -808,6 +869,7 @@ int fuse_patterns(Session &s) {
             if (m.match_attn_matmul(node)) ++formed;
         }
     }
+    formed += m.form_add_rmsnorm();
     formed += m.form_matmul_groups();
     if (!formed) return 0;
     std::vector<Node> kept;

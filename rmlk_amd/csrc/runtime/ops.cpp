@@ -825,6 +825,7 @@ const std::unordered_map<std::string, OpFn> &registry() {
         {"Constant", op_constant},
         {"rmlk.RMSNorm", op_fused_rmsnorm},
         {"rmlk.SwiGLU", op_fused_swiglu},
+        {"rmlk.AddRMSNorm", op_fused_add_rmsnorm},
         {"rmlk.ScaleMaskSoftmax", op_fused_softmax},
         {"rmlk.Rotary", op_fused_rotary},
         {"rmlk.AttnMatMul", op_fused_attn_matmul},

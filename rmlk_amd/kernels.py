@@ -174,6 +174,15 @@ def rmsnorm(x, gamma, out, rows: int, cols: int, eps: float, reciprocal_form: bo
                                  float(eps), int(reciprocal_form), _ptr(out)), "rmlk_hip_rmsnorm")
 
 
+def add_rmsnorm(a, b, gamma, sum_out, out, rows: int, cols: int, eps: float,
+                reciprocal_form: bool = False) -> None:
+    """Fused Add -> RMSNorm chain: sum_out = a + b, out = RMSNorm(sum_out)."""
+    assert a.numel() == b.numel() == sum_out.numel() == out.numel() == rows * cols
+    check(lib().rmlk_hip_add_rmsnorm(_stream(), dtype_of(a), rows, cols, _ptr(a), _ptr(b),
+                                     _ptr(gamma), float(eps), int(reciprocal_form), _ptr(sum_out),
+                                     _ptr(out)), "rmlk_hip_add_rmsnorm")
+
+
 def scale_mask_softmax(x, mask, out, shape, mask_stride, scale: float, scale_is_mul=False) -> None:
     """Fused Div|Mul(x, scale) -> Add(mask) -> Softmax(axis -1)."""
     check(lib().rmlk_hip_scale_mask_softmax(_stream(), dtype_of(x), Dims.of(shape),

@@ -211,8 +211,8 @@ def test_pass_forms_the_expected_nodes_on_the_llama_graph(device):
             feeds[f"cache.{l}.{kv}"] = np.zeros((1, cfg.kv_heads, 24, cfg.head_dim), np.float32)
     a, b, n, _ = _run_both(graph, feeds)
     # per layer: 2 RMSNorm, 2 rotary, 1 SwiGLU, 1 softmax, 2 attention MatMuls, the q/k/v and the
-    # gate/up MatMul groups; plus the final RMSNorm
-    assert n == cfg.layers * 10 + 1
+    # gate/up MatMul groups, 2 residual Adds merged into the norm that follows; plus the final RMSNorm
+    assert n == cfg.layers * 12 + 1
     # RMSNorm's mean may differ in the last place; everything downstream inherits that
     _same(a, b, loose=set(a.keys()))
     assert np.array_equal(np.argmax(a["logits"][0], -1), np.argmax(b["logits"][0], -1))
@@ -225,7 +225,7 @@ def test_fused_llama_concat_style_against_oracle(device):
     graph = graphs.llama_graph(cfg, seed=4, style="concat")
     feeds = graphs.llama_concat_inputs(cfg, np.random.default_rng(1).integers(0, cfg.vocab, 9), None, 0)
     inst = runtime.Builder.from_graph(graph).build()
-    assert inst.fused_nodes == cfg.layers * 10 + 1
+    assert inst.fused_nodes == cfg.layers * 12 + 1
     got = inst.run(feeds)
     exp = og.run_graph(graph, feeds)
     for name in exp:
@@ -237,7 +237,7 @@ def test_fused_decoder_layer_full_width(device):
     from rmlk_amd import graphs
     graph, feeds = graphs.decoder_layer_graph(seed=3, seq=96)
     a, b, n, _ = _run_both(graph, feeds)
-    assert n == 10
+    assert n == 11
     _same(a, b, loose={"y"})
 
 
@@ -486,3 +486,48 @@ def test_matmul_group_keeps_a_weight_that_something_else_reads(device):
     assert n == 1
     for name in a:
         assert_close(a[name], b[name], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [[1, 1, 2048], [3, 40, 64], [2, 6]])
+def test_residual_add_merges_into_the_norm_and_stays_an_output(device, shape):
+    """h = a + b feeds an RMSNorm and is read again later (the residual stream): one node with two
+    outputs; [2, 6] (cols % 4 != 0) runs the body."""
+    from oracle import graph as og
+    gb = _builder()
+    gb.input("a", np.float32, shape)
+    gb.input("b", np.float32, shape)
+    rng = np.random.default_rng(len(shape) + shape[-1])
+    gb.constant("gamma", rng.uniform(0.5, 1.5, size=(shape[-1],)).astype(np.float32))
+    gb.op("Add", ["a", "b"], ["h"])
+    _rmsnorm_nodes(gb, "h", "gamma", "y")
+    gb.op("Mul", ["h", "y"], ["z"])
+    gb.output("z")
+    gb.output("h")
+    graph = gb.build()
+    feeds = {"a": rng.standard_normal(shape, dtype=np.float32),
+             "b": rng.standard_normal(shape, dtype=np.float32)}
+    a, b, n, _ = _run_both(graph, feeds)
+    assert n == 2          # the RMSNorm chain, then the Add merged into it
+    assert_exact(a["h"], b["h"])
+    _same(a, b, loose={"y", "z"})
+    exp = og.run_graph(graph, feeds)
+    for name in a:
+        assert_close(a[name], exp[name], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 2048), (512, 2048), (1500, 256), (5, 4)])
+def test_add_rmsnorm_kernel_matches_separate_kernels(device, rows, cols):
+    import torch
+    k = _k()
+    rng = np.random.default_rng(rows + cols)
+    a = to_dev(rng.standard_normal((rows, cols), dtype=np.float32), device)
+    b = to_dev(rng.standard_normal((rows, cols), dtype=np.float32), device)
+    gamma = to_dev(rng.uniform(0.5, 1.5, size=(cols,)).astype(np.float32), device)
+    h = torch.empty_like(a)
+    k.binary(k.ADD, a, b, h, [rows, cols], [cols, 1], [cols, 1])
+    exp = torch.empty_like(a)
+    k.rmsnorm(h, gamma, exp, rows, cols, 1e-5)
+    got_h, got = torch.empty_like(a), torch.empty_like(a)
+    k.add_rmsnorm(a, b, gamma, got_h, got, rows, cols, 1e-5)
+    assert_exact(to_np(got_h), to_np(h))
+    assert_exact(to_np(got), to_np(exp))
