@@ -261,6 +261,24 @@ int32_t rmlk_hip_scale_mask_softmax(rmlk_stream_t stream, int32_t dtype, const r
 int32_t rmlk_hip_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *gate,
                         const void *up, void *out);
 
+/* ---- one-row products whose split-K combine is left to the consumer -----------------------------
+ * A one-row MatMul (decode) streams its weights in K slabs and leaves one partial row per slab; these
+ * entry points let the kernel that consumes the product add the slabs up itself (ascending slab
+ * order), which saves the combine launch. No counterpart in the reference.
+ *
+ * rmlk_hip_gemv_partials: partial rows of x[k] . B[k, n] (B row-major, leading dimension ldb) into
+ * `workspace` as [splits][n]; *splits_out = number of slabs (>= 1). n % 4 == 0, 16-byte aligned B.
+ * rmlk_hip_gemv_partials_workspace_size: bytes the workspace must hold for that call. */
+size_t rmlk_hip_gemv_partials_workspace_size(int32_t dtype, int64_t n, int64_t k);
+int32_t rmlk_hip_gemv_partials(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
+                               const void *x, const void *b, int64_t ldb, void *workspace,
+                               size_t workspace_bytes, int32_t *splits_out);
+/* out[i] = swiglu(gate_i, up_i) with gate_i = sum of the slabs at element gate_offset + i and up_i
+ * likewise at up_offset + i (a joint [gate | up] product): rmlk_hip_swiglu on partial slabs. */
+int32_t rmlk_hip_splitk_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *partials,
+                               int32_t splits, int64_t slab, int64_t gate_offset, int64_t up_offset,
+                               void *out);
+
 /* Rotary position embedding, half-rotation form, over x of logical shape [B, H, S, D]:
  * out = x * cos + concat(-x[..., D/2:], x[..., :D/2]) * sin, out dense [B, H, S, D].
  * x, cos and sin are read through element strides per dim of `shape` (innermost stride 1; 0 on

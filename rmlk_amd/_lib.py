@@ -90,6 +90,11 @@ SIGNATURES = {
     "rmlk_hip_scale_mask_softmax": (c_int32, [c_void_p, c_int32, _PD, _PD, c_int32, ctypes.c_float,
                                               c_void_p, c_void_p, c_void_p]),
     "rmlk_hip_swiglu": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p]),
+    "rmlk_hip_gemv_partials_workspace_size": (c_size_t, [c_int32, c_int64, c_int64]),
+    "rmlk_hip_gemv_partials": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p,
+                                         c_int64, c_void_p, c_size_t, POINTER(c_int32)]),
+    "rmlk_hip_splitk_swiglu": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_int32, c_int64,
+                                         c_int64, c_int64, c_void_p]),
     "rmlk_hip_rotary": (c_int32, [c_void_p, c_int32, _PD, _PD, _PD, _PD, c_void_p, c_void_p,
                                   c_void_p, c_void_p]),
     "rmlk_hip_fill": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),

@@ -65,6 +65,47 @@ __global__ __launch_bounds__(kBlock) void swiglu_tail_kernel(const float *__rest
     }
 }
 
+// SwiGLU whose operands are still split-K partial rows of one GEMV over [gate | up] weights:
+// gate_i = sum_z p[z][i], up_i = sum_z p[z][n + i] (z ascending), then as above.
+__global__ __launch_bounds__(kBlock) void splitk_swiglu_kernel(const float *__restrict__ partials,
+                                                               int32_t splits, int64_t slab,
+                                                               float *__restrict__ out,
+                                                               uint32_t n_vec, uint32_t up_off) {
+    using V = Vec<float, 4>;
+    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n_vec; i += gridDim.x * kBlock) {
+        const float *pg = partials + static_cast<int64_t>(i) * 4;
+        V gv, uv;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) gv.v[j] = uv.v[j] = 0.f;
+        constexpr int kDepth = 8;   // slabs in ascending order, 16 loads in flight
+        for (int z0 = 0; z0 < splits; z0 += kDepth) {
+            V a[kDepth], b[kDepth];
+#pragma unroll
+            for (int u = 0; u < kDepth; ++u)
+                if (z0 + u < splits) {
+                    a[u] = *reinterpret_cast<const V *>(pg + (z0 + u) * slab);
+                    b[u] = *reinterpret_cast<const V *>(pg + (z0 + u) * slab + up_off);
+                }
+#pragma unroll
+            for (int u = 0; u < kDepth; ++u)
+                if (z0 + u < splits) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        gv.v[j] += a[u].v[j];
+                        uv.v[j] += b[u].v[j];
+                    }
+                }
+        }
+        V y;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float silu = gv.v[j] * sigmoid_f(gv.v[j]);
+            y.v[j] = silu * uv.v[j];
+        }
+        reinterpret_cast<V *>(out)[i] = y;
+    }
+}
+
 // Rotary embedding over x [B,H,S,D] read through element strides (the innermost stride is 1), so a
 // [B,S,H,D] projection output is rotated and laid out [B,H,S,D] in the same pass. One lane takes W
 // neighbouring elements of the first half of a row together with their partners in the second half.
@@ -145,6 +186,24 @@ extern "C" int32_t rmlk_hip_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t 
         if (blocks >= ((int64_t)1 << 31)) return RMLK_ERR_TOO_LARGE;
         swiglu_tail_kernel<<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(g, u, o, done, n);
     }
+    return launch_status();
+}
+
+extern "C" int32_t rmlk_hip_splitk_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n,
+                                          const void *partials, int32_t splits, int64_t slab,
+                                          int64_t gate_offset, int64_t up_offset, void *out) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (n < 0 || splits < 1 || gate_offset < 0 || up_offset < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n == 0) return RMLK_OK;
+    if (!partials || !out) return RMLK_ERR_NULL_POINTER;
+    const float *p = static_cast<const float *>(partials) + gate_offset;
+    const int64_t rel = up_offset - gate_offset;
+    if (n % 4 || slab % 4 || rel % 4 || rel < 0 || n >= ((int64_t)1 << 32) ||
+        reinterpret_cast<uintptr_t>(p) % 16 || reinterpret_cast<uintptr_t>(out) % 16)
+        return RMLK_ERR_UNSUPPORTED;
+    splitk_swiglu_kernel<<<grid_for(n / 4, kBlock, 8), kBlock, 0, as_stream(stream)>>>(
+        p, splits, slab, static_cast<float *>(out), static_cast<uint32_t>(n / 4),
+        static_cast<uint32_t>(rel));
     return launch_status();
 }
 

@@ -1226,3 +1226,40 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
     }
     return RMLK_OK;
 }
+
+extern "C" size_t rmlk_hip_gemv_partials_workspace_size(int32_t dtype, int64_t n, int64_t k) {
+    if (dtype != RMLK_FLOAT || n <= 0 || k <= 0 || n % 4 != 0) return 0;
+    int kps;
+    const int splits = gemv_splits(1, n, k, kWave * 4, &kps);
+    return static_cast<size_t>(splits) * n * sizeof(float);
+}
+
+extern "C" int32_t rmlk_hip_gemv_partials(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
+                                          const void *x, const void *b, int64_t ldb, void *workspace,
+                                          size_t workspace_bytes, int32_t *splits_out) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (n <= 0 || k <= 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n >= (1ll << 31) || k >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
+    if (!x || !b || !workspace || !splits_out) return RMLK_ERR_NULL_POINTER;
+    if (ldb < n) return RMLK_ERR_SIZE_MISMATCH;
+    if (n % 4 != 0 || ldb % 4 != 0 || reinterpret_cast<uintptr_t>(b) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+        return RMLK_ERR_UNSUPPORTED;
+    int kps;
+    const int splits = gemv_splits(1, n, k, kWave * 4, &kps);
+    if (workspace_bytes < static_cast<size_t>(splits) * n * sizeof(float)) return RMLK_ERR_WORKSPACE;
+    GemvArgs g{};
+    g.x = static_cast<const float *>(x);
+    g.w = static_cast<const float *>(b);
+    g.n = static_cast<int32_t>(n);
+    g.k = static_cast<int32_t>(k);
+    g.x_inc = 1;
+    g.ldb = ldb;
+    g.k_per_split = kps;
+    g.y = static_cast<float *>(workspace);
+    g.stride_y = n;
+    dim3 grid(static_cast<unsigned>((n + kWave * 4 - 1) / (kWave * 4)), 1, static_cast<unsigned>(splits));
+    gemv_kernel<4><<<grid, kThreads, 0, as_stream(stream)>>>(g);
+    *splits_out = splits;
+    return launch_status();
+}

@@ -329,15 +329,11 @@ int32_t softmax_typed(hipStream_t s, int64_t outer, int64_t n, int64_t inner, co
 // The fused form of Pow(2) -> ReduceMean(-1) -> Add(eps) -> Sqrt -> Div -> Mul(gamma): squares are
 // rounded to float before the double accumulation and every later step rounds like the separate
 // kernel does. RECIP selects the exported variant x * (1 / sqrt(..)) * gamma.
-// The row may also be formed on the fly: x + add (the residual Add in front of the norm), or
-// residual + the sum of split-K partial slabs of a preceding GEMV; the formed row is then stored
-// to sum_out as well, because the residual stream reads it again later.
+// The row may also be formed on the fly as x + add (the residual Add in front of the norm); the
+// formed row is then stored to sum_out as well, because the residual stream reads it again later.
 struct RmsSource {
-    const float *x;       // the row, or the residual when add / ws is given
+    const float *x;       // the row
     const float *add;     // second Add operand, or null
-    const float *ws;      // split-K partials [splits][slab], or null
-    int32_t splits;
-    int64_t slab;         // elements between consecutive partial slabs
     float *sum_out;       // where the formed row goes (null: nowhere)
 };
 
@@ -374,17 +370,6 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(RmsSource src,
                     const V av = reinterpret_cast<const V *>(src.add + row * cols)[c];
 #pragma unroll
                     for (int j = 0; j < 4; ++j) xv[i].v[j] = xv[i].v[j] + av.v[j];
-                } else if (src.ws) {
-                    const V *pw = reinterpret_cast<const V *>(src.ws + row * cols) + c;
-                    V t = *pw;
-                    for (int z = 1; z < src.splits; ++z) {
-                        const V p = *reinterpret_cast<const V *>(
-                            reinterpret_cast<const float *>(pw) + z * src.slab);
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) t.v[j] += p.v[j];
-                    }
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) xv[i].v[j] = xv[i].v[j] + t.v[j];
                 }
                 if (src.sum_out) reinterpret_cast<V *>(src.sum_out + row * cols)[c] = xv[i];
 #pragma unroll
@@ -441,8 +426,8 @@ int32_t launch_rmsnorm(hipStream_t s, const RmsSource &src, const float *gamma, 
 int32_t rmsnorm_dispatch(hipStream_t s, const RmsSource &src, const float *gp, float *op, int64_t rows,
                          int64_t cols, float eps, bool recip) {
     auto aligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-    const bool vec_ok = cols % 4 == 0 && aligned(src.x) && aligned(src.add) && aligned(src.ws) &&
-                        aligned(src.sum_out) && aligned(gp) && aligned(op) && src.slab % 4 == 0;
+    const bool vec_ok = cols % 4 == 0 && aligned(src.x) && aligned(src.add) &&
+                        aligned(src.sum_out) && aligned(gp) && aligned(op);
     if (!vec_ok || cols > kBlock * 4 * 8) return RMLK_ERR_UNSUPPORTED;
     const int32_t c = static_cast<int32_t>(cols);
     if (rows >= 1024 && c <= kWave * 4 * 8) {  // many rows: a wavefront per row
@@ -585,7 +570,7 @@ extern "C" int32_t rmlk_hip_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t
     if (rows == 0 || cols == 0) return RMLK_OK;
     if (!x || !gamma || !out) return RMLK_ERR_NULL_POINTER;
     if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
-    RmsSource src{static_cast<const float *>(x), nullptr, nullptr, 0, 0, nullptr};
+    RmsSource src{static_cast<const float *>(x), nullptr, nullptr};
     return rmsnorm_dispatch(as_stream(stream), src, static_cast<const float *>(gamma),
                             static_cast<float *>(out), rows, cols, eps, reciprocal_form != 0);
 }
@@ -599,7 +584,7 @@ extern "C" int32_t rmlk_hip_add_rmsnorm(rmlk_stream_t stream, int32_t dtype, int
     if (rows == 0 || cols == 0) return RMLK_OK;
     if (!a || !b || !gamma || !sum_out || !out) return RMLK_ERR_NULL_POINTER;
     if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
-    RmsSource src{static_cast<const float *>(a), static_cast<const float *>(b), nullptr, 0, 0,
+    RmsSource src{static_cast<const float *>(a), static_cast<const float *>(b),
                   static_cast<float *>(sum_out)};
     return rmsnorm_dispatch(as_stream(stream), src, static_cast<const float *>(gamma),
                             static_cast<float *>(out), rows, cols, eps, reciprocal_form != 0);

@@ -14,6 +14,8 @@
 //   rmlk.Rotary            [Transpose(0,2,1,3)] Slice Slice Neg Concat Mul Mul Add
 //   rmlk.AttnMatMul        MatMul(a, [Transpose(0,1,3,2)] [Reshape Expand Unsqueeze] (kv))
 //   rmlk.MatMulGroup       MatMul(a, W1), MatMul(a, W2), ... on the same a with constant 2-D weights
+//   rmlk.MatMulGroupSwiGLU a [gate | up] rmlk.MatMulGroup feeding only an rmlk.SwiGLU: a one-row a
+//                          leaves its split-K slabs to the SwiGLU kernel (no combine launch)
 //
 // A fused node keeps the nodes it replaced as its `body`. What cannot be decided while building
 // (shapes are only known at run time) is checked when the node runs; if the fused kernel does not
@@ -443,6 +445,43 @@ struct Matcher {
         return formed;
     }
 
+    // ---- a producer whose split-K combine can move into the consumer (one-row inputs) -------------
+    // (Tried as well for MatMul -> AddRMSNorm: the norm owns a row with ONE block, which then adds
+    // up 32-64 slabs by itself and is slower than the many-block combine kernel plus the norm.)
+    int form_splitk_epilogues() {
+        int formed = 0;
+        for (size_t n = 0; n < g.nodes.size(); ++n) {
+            if (removed[n]) continue;
+            const Node &cons = g.nodes[n];
+            if (cons.op == "rmlk.SwiGLU") {
+                const Node *grp = produced_by(cons.inputs[0], "rmlk.MatMulGroup");
+                if (!grp || grp != produced_by(cons.inputs[1], "rmlk.MatMulGroup") ||
+                    grp->outputs.size() != 2 || cons.inputs[0] == cons.inputs[1])
+                    continue;
+                if (!only_used_by(grp->outputs[0], {&cons}) || !only_used_by(grp->outputs[1], {&cons}))
+                    continue;
+                Node f;
+                f.op = "rmlk.MatMulGroupSwiGLU";
+                f.inputs = grp->inputs;
+                f.outputs = cons.outputs;
+                f.attrs = grp->attrs;
+                f.attrs["gate_first"] = a_int(cons.inputs[0] == grp->outputs[0] ? 1 : 0);
+                Node swiglu = cons;
+                f.body = {*grp, swiglu};
+                const int gi = index_of(grp);
+                for (int v : grp->inputs) {
+                    auto &u = users[v];
+                    u.erase(std::remove(u.begin(), u.end(), gi), u.end());
+                    u.push_back(static_cast<int>(n));
+                }
+                removed[gi] = true;
+                g.nodes[n] = std::move(f);
+                ++formed;
+            }
+        }
+        return formed;
+    }
+
     // ---- MatMuls that share their first operand and have constant 2-D weights (q/k/v, gate/up) ----
     // The weights are laid side by side in ONE device matrix [K, N1 + N2 + ..] while building (the
     // separate copies are released unless something else reads them). A one-row input then takes a
@@ -798,6 +837,42 @@ void op_fused_add_rmsnorm(OpContext &c) {
     run_body(c);
 }
 
+// Partial rows of a one-row product in the session workspace; false when the GEMV does not cover it.
+bool gemv_partials(OpContext &c, const Tensor &a, const Tensor &w, const void **ws_out, int32_t *splits) {
+    const int64_t k = w.shape[0], n = w.shape[1];
+    const size_t bytes = rmlk_hip_gemv_partials_workspace_size(RMLK_FLOAT, n, k);
+    if (!bytes) return false;
+    void *ws = c.scratch(bytes);
+    if (!took_fast_path(rmlk_hip_gemv_partials(c.stream, RMLK_FLOAT, n, k, a.data(), w.data(), n, ws,
+                                               bytes, splits),
+                        "one-row MatMul"))
+        return false;
+    *ws_out = ws;
+    return true;
+}
+
+void op_fused_matmul_group_swiglu(OpContext &c) {
+    const Tensor &a = c.input(0), &w = c.input(1);
+    const std::vector<int64_t> widths = c.attr_ints("widths");
+    const int64_t k = w.shape[0];
+    const bool ok = a.dtype == RMLK_FLOAT && a.rank() >= 1 && a.shape.back() == k && a.numel() == k &&
+                    widths.size() == 2 && widths[0] == widths[1];
+    const void *ws = nullptr;
+    int32_t splits = 0;
+    if (ok && gemv_partials(c, a, w, &ws, &splits)) {
+        const int64_t n = widths[0];
+        const bool gate_first = c.attr_int("gate_first", 1) != 0;
+        std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
+        shape.push_back(n);
+        Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
+        if (took_fast_path(rmlk_hip_splitk_swiglu(c.stream, RMLK_FLOAT, n, ws, splits, 2 * n,
+                                                  gate_first ? 0 : n, gate_first ? n : 0, y.data()),
+                           "rmlk.MatMulGroupSwiGLU"))
+            return;
+    }
+    run_body(c);
+}
+
 // MatMul(a, W_i) for every member of a group, W_i being column blocks of one joint matrix.
 void op_fused_matmul_group(OpContext &c) {
     const Tensor &a = c.input(0), &w = c.input(1);
@@ -871,6 +946,7 @@ int fuse_patterns(Session &s) {
     }
     formed += m.form_add_rmsnorm();
     formed += m.form_matmul_groups();
+    formed += m.form_splitk_epilogues();
     if (!formed) return 0;
     std::vector<Node> kept;
     kept.reserve(m.g.nodes.size());

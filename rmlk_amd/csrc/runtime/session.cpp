@@ -485,6 +485,11 @@ void Session::run_nodes() {
             double out_elems = 0.0;
             for (const Tensor &t : outs) out_elems += static_cast<double>(t.numel());
             flops = 2.0 * out_elems * static_cast<double>(ctx.in[0]->shape.back());
+        } else if (node.op == "rmlk.MatMulGroupSwiGLU" &&
+                   ctx.in[0] && ctx.in[1] && ctx.in[1]->rank() == 2 && ctx.in[1]->shape[0] > 0) {
+            // rows of a times the whole weight matrix
+            flops = 2.0 * static_cast<double>(ctx.in[0]->numel()) / static_cast<double>(ctx.in[1]->shape[0]) *
+                    static_cast<double>(ctx.in[1]->numel());
         }
         st.bytes = bytes;
         st.flops = flops;

@@ -211,8 +211,9 @@ def test_pass_forms_the_expected_nodes_on_the_llama_graph(device):
             feeds[f"cache.{l}.{kv}"] = np.zeros((1, cfg.kv_heads, 24, cfg.head_dim), np.float32)
     a, b, n, _ = _run_both(graph, feeds)
     # per layer: 2 RMSNorm, 2 rotary, 1 SwiGLU, 1 softmax, 2 attention MatMuls, the q/k/v and the
-    # gate/up MatMul groups, 2 residual Adds merged into the norm that follows; plus the final RMSNorm
-    assert n == cfg.layers * 12 + 1
+    # gate/up MatMul groups, 2 residual Adds merged into the norm that follows, the gate/up group
+    # merged with the SwiGLU; plus the final RMSNorm
+    assert n == cfg.layers * 13 + 1
     # RMSNorm's mean may differ in the last place; everything downstream inherits that
     _same(a, b, loose=set(a.keys()))
     assert np.array_equal(np.argmax(a["logits"][0], -1), np.argmax(b["logits"][0], -1))
@@ -225,7 +226,7 @@ def test_fused_llama_concat_style_against_oracle(device):
     graph = graphs.llama_graph(cfg, seed=4, style="concat")
     feeds = graphs.llama_concat_inputs(cfg, np.random.default_rng(1).integers(0, cfg.vocab, 9), None, 0)
     inst = runtime.Builder.from_graph(graph).build()
-    assert inst.fused_nodes == cfg.layers * 12 + 1
+    assert inst.fused_nodes == cfg.layers * 13 + 1
     got = inst.run(feeds)
     exp = og.run_graph(graph, feeds)
     for name in exp:
@@ -237,7 +238,7 @@ def test_fused_decoder_layer_full_width(device):
     from rmlk_amd import graphs
     graph, feeds = graphs.decoder_layer_graph(seed=3, seq=96)
     a, b, n, _ = _run_both(graph, feeds)
-    assert n == 11
+    assert n == 12
     _same(a, b, loose={"y"})
 
 
@@ -531,3 +532,39 @@ def test_add_rmsnorm_kernel_matches_separate_kernels(device, rows, cols):
     k.add_rmsnorm(a, b, gamma, got_h, got, rows, cols, 1e-5)
     assert_exact(to_np(got_h), to_np(h))
     assert_exact(to_np(got), to_np(exp))
+
+
+@pytest.mark.parametrize("rows", [1, 5])
+def test_one_row_products_leave_their_combine_to_the_consumer(device, rows):
+    """[gate | up] -> SwiGLU: with one input row the GEMV's split-K slabs are added up inside the
+    SwiGLU kernel; more rows run the body."""
+    from oracle import graph as og
+    hid, ffn = 256, 512
+    gb = _builder()
+    gb.input("x", np.float32, [1, 0, hid])
+    gb.input("res", np.float32, [1, 0, hid])
+    rng = np.random.default_rng(rows)
+    for name, shape in (("wo", (hid, hid)), ("wg", (hid, ffn)), ("wu", (hid, ffn)), ("wd", (ffn, hid))):
+        gb.constant(name, (rng.standard_normal(shape) * 0.05).astype(np.float32))
+    gb.constant("gamma", rng.uniform(0.5, 1.5, size=(hid,)).astype(np.float32))
+    gb.op("MatMul", ["x", "wo"], ["o"])
+    gb.op("Add", ["res", "o"], ["h"])
+    _rmsnorm_nodes(gb, "h", "gamma", "hn")
+    gb.op("MatMul", ["hn", "wg"], ["g"])
+    gb.op("MatMul", ["hn", "wu"], ["u"])
+    gb.op("Sigmoid", ["g"], ["sg"])
+    gb.op("Mul", ["g", "sg"], ["silu"])
+    gb.op("Mul", ["silu", "u"], ["act"])
+    gb.op("MatMul", ["act", "wd"], ["d"])
+    gb.op("Add", ["h", "d"], ["out"])
+    gb.output("out")
+    gb.output("h")
+    graph = gb.build()
+    feeds = {"x": rng.standard_normal((1, rows, hid), dtype=np.float32),
+             "res": rng.standard_normal((1, rows, hid), dtype=np.float32)}
+    a, b, n, _ = _run_both(graph, feeds)
+    assert n == 5      # RMSNorm, SwiGLU, AddRMSNorm, gate/up group, group + SwiGLU merge
+    exp = og.run_graph(graph, feeds)
+    for name in a:
+        assert_close(a[name], b[name], rtol=1e-4, atol=1e-5)
+        assert_close(a[name], exp[name], rtol=1e-4, atol=1e-5)
