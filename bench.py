@@ -374,6 +374,25 @@ def run_ops_suite(args):
         t.view(32, 2048, 2048).add_(mask)
     so = [torch.empty_like(sx[0]) for _ in range(2)]
     timed("softmax", lambda i: k.softmax(sx[i], so[i], 65536, 2048, 1), 2, 2 * sx[0].numel() * 4)
+    # ---- fused chains at the shapes they take in the Llama prefill (S = 2048) ---------------------
+    gam = torch.rand(2048, device=dev, generator=g) + 0.5
+    timed("fused_rmsnorm", lambda i: k.rmsnorm(xs[i], gam, ys[i], 4096, 2048, 1e-5), ns,
+          2 * n * 4 + 8192)
+    sums = [torch.empty(n, device=dev) for _ in range(2)]
+    timed("fused_add_rmsnorm", lambda i: k.add_rmsnorm(xs[i], xs[(i + 1) % ns], gam, sums[i % 2], ys[i],
+                                                       4096, 2048, 1e-5), ns, 4 * n * 4 + 8192)
+    timed("fused_swiglu", lambda i: k.swiglu(xs[i], xs[(i + 1) % ns], ys[i]), ns, 3 * n * 4)
+    cs_tab = torch.randn(2 * 2048 * 64, device=dev, generator=g)
+    rot_shape = [1, 64, 2048, 64]       # the [1, 2048, 64, 64] projection read head-major
+    timed("fused_rotary", lambda i: k.rotary(xs[i], cs_tab[:2048 * 64], cs_tab[2048 * 64:], ys[i], rot_shape,
+                                             [0, 64, 64 * 64, 1], [0, 0, 64, 1], [0, 0, 64, 1]), ns,
+          2 * n * 4 + 2 * 2048 * 64 * 4)
+    msk = torch.triu(torch.full((2048, 2048), float("-inf"), device=dev), 1)
+    plain = [torch.randn(32 * 2048, 2048, device=dev, generator=g) for _ in range(2)]
+    timed("fused_scale_mask_softmax",
+          lambda i: k.scale_mask_softmax(plain[i], msk, so[i], [1, 32, 2048, 2048], [0, 0, 2048, 1], 8.0),
+          2, 2 * plain[0].numel() * 4 + 2048 * 2048 * 4)
+    del plain
     # ---- config 5 shapes: KV-cache / indexing stress ---------------------------------------------
     kv_n = 8 * 8192 * 64
     caches = [torch.randn(kv_n, device=dev, generator=g) for _ in range(ns * 3)]

@@ -57,11 +57,21 @@ struct SmemLayout {
 // tile index -> (tile_m, tile_n). Consecutive hardware block ids go round-robin over the 8 XCDs,
 // each with a private L2; blocks are renumbered so that one XCD works on a compact group of
 // tiles that share rows of A and columns of B.
-__device__ __forceinline__ void tile_coords(const GemmArgs &g, int &tm, int &tn) {
+__device__ __forceinline__ void tile_coords(const GemmArgs &g, int &tm, int &tn, int &split) {
     const int n_tiles = g.tiles_m * g.tiles_n;
     int pid = blockIdx.x;
+    split = blockIdx.z;
     constexpr int kXcd = 8;
-    if (n_tiles % kXcd == 0) {
+    if (gridDim.y == 1 && gridDim.z > 1 && (n_tiles * gridDim.z) % kXcd == 0) {
+        // split-K of one matrix: the (split, tile) pairs are dealt to the XCDs in contiguous runs,
+        // split-major, so that an XCD works on ONE K slab where it can and fetches that slab of A
+        // once instead of every slab of A
+        const int linear = blockIdx.x + n_tiles * blockIdx.z;   // hardware order: x fastest
+        const int per = n_tiles * gridDim.z / kXcd;
+        const int item = (linear % kXcd) * per + linear / kXcd;
+        split = item / n_tiles;
+        pid = item - split * n_tiles;
+    } else if (n_tiles % kXcd == 0) {
         const int per = n_tiles / kXcd;
         pid = (pid % kXcd) * per + pid / kXcd;
     }
@@ -103,10 +113,9 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
     constexpr int B_PASSES = (TB ? BN : BK) / B_ROWS_PER_PASS;
     static_assert(A_PASSES >= 1 && B_PASSES >= 1, "tile too small for 256 lanes");
 
-    int tile_m, tile_n;
-    tile_coords(g, tile_m, tile_n);
+    int tile_m, tile_n, split;
+    tile_coords(g, tile_m, tile_n, split);
     const int batch = blockIdx.y;
-    const int split = blockIdx.z;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int k_begin = split * g.k_per_split;
     const int k_end = min(g.k, k_begin + g.k_per_split);
@@ -358,10 +367,9 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     constexpr int B_ROWS_PER_PIECE = kWave / B_ROW_LANES > 0 ? kWave / B_ROW_LANES : 1;
     static_assert(TB || B_ROW_LANES <= kWave, "a K-row of B must fit one 1 KiB piece");
 
-    int tile_m, tile_n;
-    tile_coords(g, tile_m, tile_n);
+    int tile_m, tile_n, split;
+    tile_coords(g, tile_m, tile_n, split);
     const int batch = blockIdx.y;
-    const int split = blockIdx.z;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int k_begin = split * g.k_per_split;
     const int k_end = min(g.k, k_begin + g.k_per_split);
