@@ -18,6 +18,7 @@
 //     fixed order, so results do not depend on scheduling.
 #include <cstdio>
 #include <cstring>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -555,6 +556,10 @@ __global__ __launch_bounds__(kThreads) void splitk_reduce_kernel(const float *__
 // ---- GEMV: y[n] = sum_k x[k] * W[k][n], W row-major -------------------------------------------
 // A block covers kThreads / 64 * ... columns: VEC columns per lane, 64 lanes per wavefront, and
 // the block's 4 wavefronts split the block's K slice; partial sums meet in LDS.
+#ifndef RMLK_GEMV_DEPTH
+#define RMLK_GEMV_DEPTH 16
+#endif
+
 struct GemvArgs {
     const float *x;   // [batch][k], element stride x_inc
     const float *w;
@@ -593,8 +598,10 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(GemvArgs g) {
         const float *wp = w + static_cast<int64_t>(kb) * g.ldb + col;
         int kk = kb;
         if constexpr (VEC == 4) {
-            constexpr int U = 8;
-            for (; kk + U <= ke; kk += U) {
+            // U rows of weights requested before any is used: a slab of 16 rows per wavefront is
+            // one round trip to HBM
+            auto rows = [&](auto u_tag) {
+                constexpr int U = decltype(u_tag)::value;
                 v4f wv[U];
                 float xv[U];
 #pragma unroll
@@ -608,7 +615,11 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(GemvArgs g) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) acc[j] = fmaf(xv[u], wv[u][j], acc[j]);
                 wp += static_cast<int64_t>(U) * g.ldb;
-            }
+                kk += U;
+            };
+            while (kk + RMLK_GEMV_DEPTH <= ke) rows(std::integral_constant<int, RMLK_GEMV_DEPTH>{});
+            if (RMLK_GEMV_DEPTH > 8 && kk + 8 <= ke) rows(std::integral_constant<int, 8>{});
+            if (kk + 4 <= ke) rows(std::integral_constant<int, 4>{});
             for (; kk < ke; ++kk) {
                 v4f wv = *reinterpret_cast<const v4f *>(wp);
                 float xv = x[static_cast<int64_t>(kk) * g.x_inc];
@@ -903,8 +914,15 @@ inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k) {
 inline int gemv_splits(int64_t batch, int64_t n, int64_t k, int cols_per_block, int *k_per_split) {
     int64_t blocks = (n + cols_per_block - 1) / cols_per_block * batch;
     int64_t splits = 1;
-    if (blocks < 4 * kNumCU) splits = (4 * kNumCU + blocks - 1) / blocks;
-    int64_t max_splits = k / 64;
+#ifndef RMLK_GEMV_BLOCKS_PER_CU
+#define RMLK_GEMV_BLOCKS_PER_CU 6
+#endif
+    if (blocks < RMLK_GEMV_BLOCKS_PER_CU * kNumCU)
+        splits = (RMLK_GEMV_BLOCKS_PER_CU * kNumCU + blocks - 1) / blocks;
+#ifndef RMLK_GEMV_MIN_ROWS
+#define RMLK_GEMV_MIN_ROWS 64
+#endif
+    int64_t max_splits = k / RMLK_GEMV_MIN_ROWS;
     if (max_splits < 1) max_splits = 1;
     if (splits > max_splits) splits = max_splits;
     if (splits > 64) splits = 64;
