@@ -446,8 +446,10 @@ struct Matcher {
     }
 
     // ---- a producer whose split-K combine can move into the consumer (one-row inputs) -------------
-    // (Tried as well for MatMul -> AddRMSNorm: the norm owns a row with ONE block, which then adds
-    // up 32-64 slabs by itself and is slower than the many-block combine kernel plus the norm.)
+    // (Tried as well and dropped, both slower than what they replace: MatMul -> AddRMSNorm, where the
+    // norm owns a row with ONE block that then adds up 32-64 slabs by itself; and one kernel for
+    // scores -> softmax -> context of a decode step with one block per KV head, where eight blocks
+    // cannot hide the HBM latency of a cold cache.)
     int form_splitk_epilogues() {
         int formed = 0;
         for (size_t n = 0; n < g.nodes.size(); ++n) {
