@@ -139,18 +139,20 @@ def run_llama(args):
     assert len(mm_nodes) == len(launches), (len(mm_nodes), len(launches))
     by_kind, per_op = {}, {}
     for s, shapes in zip(mm_nodes, launches):
-        node_flops = sum(2.0 * b_ * m * n * k for b_, m, n, k in shapes)
-        for batch, m, n, k in shapes:
+        node_flops = sum(2.0 * sh[0] * sh[1] * sh[2] * sh[3] for sh in shapes)
+        for shape in shapes:
+            batch, m, n, k = shape[:4]
+            swiglu = len(shape) > 4        # n counts the gate and the up columns; n / 2 are written
             kind = kernels.matmul_describe(batch, m, n, k)
             d = by_kind.setdefault(kind, {"launches": 0, "us": 0.0, "flops": 0.0, "alg_bytes": 0.0,
                                           "traffic": 0.0, "shapes": {}})
             d["launches"] += 1
-            d["shapes"][(batch, m, n, k)] = d["shapes"].get((batch, m, n, k), 0) + 1
+            d["shapes"][shape] = d["shapes"].get(shape, 0) + 1
             flops = 2.0 * batch * m * n * k
             d["us"] += s["micros"] * flops / node_flops     # a node of several launches: by flops
             d["flops"] += flops
-            d["alg_bytes"] += 4.0 * batch * (m * k + k * n + m * n)
-            pmc = PMC_TRAFFIC_KIB.get((batch, m, n, k))
+            d["alg_bytes"] += 4.0 * batch * (m * k + k * n + m * (n // 2 if swiglu else n))
+            pmc = PMC_TRAFFIC_KIB.get(shape)
             d["traffic"] = None if pmc is None or d["traffic"] is None else d["traffic"] + 1024.0 * sum(pmc)
     for s in stats:
         if s["micros"] > 0:
@@ -178,7 +180,8 @@ def run_llama(args):
         "launches": dom["launches"], "avg_launch_us": round(dom_us, 2),
         "avg_node_us_with_events": round(dom["us"] / dom["launches"], 2),
         "flops_per_launch": dom["flops"] / dom["launches"],
-        "shapes": {"x".join(map(str, k_)): v for k_, v in dom["shapes"].items()},
+        "shapes": {"x".join(map(str, k_[:4])) + ("".join(" " + t for t in k_[4:])): v
+                   for k_, v in dom["shapes"].items()},
         "measured": "one HIP event pair around the kernel's launches of one prefill pass (same shapes "
                     "and counts, cold weights), 3 repetitions, on the launching stream",
     }
@@ -271,21 +274,26 @@ def time_matmul_launches(kernels, torch, shape_counts, reps=3):
     exceed the 256 MB Infinity Cache, all between one pair of HIP events on the current stream."""
     dev = torch.device("cuda:0")
     plans, total = [], 0
-    for (batch, m, n, k), count in shape_counts.items():
+    for shape, count in shape_counts.items():
+        batch, m, n, k = shape[:4]
+        swiglu = len(shape) > 4
         a = torch.randn(batch, m, k, device=dev)
         nb = max(2, min(count, int(600e6 // (4 * k * n)) + 1))
         bs = [torch.randn(k, n, device=dev) * 0.02 for _ in range(nb)]
-        c = torch.empty(batch, m, n, device=dev)
+        c = torch.empty(batch, m, n // 2 if swiglu else n, device=dev)
         need = kernels.matmul_workspace_size(batch, m, n, k)
         ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
-        plans.append((batch, m, n, k, count, a, bs, c, ws))
+        plans.append((batch, m, n, k, swiglu, count, a, bs, c, ws))
         total += count
 
     def run_once():
-        for batch, m, n, k, count, a, bs, c, ws in plans:
+        for batch, m, n, k, swiglu, count, a, bs, c, ws in plans:
             for i in range(count):
-                kernels.matmul(a, bs[i % len(bs)], c, batch, m, n, k, k, n, n, m * k, 0, m * n,
-                               workspace=ws)
+                if swiglu:
+                    kernels.matmul_swiglu(a, bs[i % len(bs)], c, m, n // 2, k, n, 0, n // 2)
+                else:
+                    kernels.matmul(a, bs[i % len(bs)], c, batch, m, n, k, k, n, n, m * k, 0, m * n,
+                                   workspace=ws)
     run_once()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -306,18 +314,23 @@ def decode_weight_bytes(cfg):
 
 
 def matmul_launches(cfg, s, max_len):
-    """(batch, m, n, k) of the GEMM launches behind every MatMul-type node of the fused scatter-style
-    graph, in node order: [q, k, v] (one node), scores, context, o, [gate, up] (one node), down per
-    layer, then the lm-head."""
+    """(batch, m, n, k[, "swiglu"]) of the GEMM launches behind every MatMul-type node of the fused
+    scatter-style graph, in node order: q/k/v (one node, one launch over the joint weights), scores,
+    context, o, gate/up (one node, one launch with the SwiGLU epilogue; n counts both halves), down
+    per layer, then the lm-head."""
     h, kvd, d = cfg.hidden, cfg.kv_heads * cfg.head_dim, cfg.head_dim
     rep = cfg.heads // cfg.kv_heads
+    whole = s % 128 == 0 and h % 128 == 0 and kvd % 128 == 0 and cfg.ffn % 64 == 0
+    qkv = [(1, s, cfg.heads * d + 2 * kvd, h)] if whole else \
+        [(1, s, cfg.heads * d, h), (1, s, kvd, h), (1, s, kvd, h)]
+    gate_up = [(1, s, 2 * cfg.ffn, h, "swiglu")] if whole and (s // 128) * (cfg.ffn // 64) >= 256 else \
+        [(1, s, cfg.ffn, h), (1, s, cfg.ffn, h)]
     out = []
     for _ in range(cfg.layers):
-        out += [[(1, s, cfg.heads * d, h), (1, s, kvd, h), (1, s, kvd, h)],
+        out += [qkv,
                 # the two attention products run as one strided GEMM per KV head over its q heads
                 [(cfg.kv_heads, rep * s, max_len, d)], [(cfg.kv_heads, rep * s, d, max_len)],
-                [(1, s, h, cfg.heads * d)], [(1, s, cfg.ffn, h), (1, s, cfg.ffn, h)],
-                [(1, s, h, cfg.ffn)]]
+                [(1, s, h, cfg.heads * d)], gate_up, [(1, s, h, cfg.ffn)]]
     out.append([(1, s, cfg.vocab, h)])
     return out
 

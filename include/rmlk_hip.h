@@ -279,6 +279,28 @@ int32_t rmlk_hip_splitk_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, c
                                int32_t splits, int64_t slab, int64_t gate_offset, int64_t up_offset,
                                void *out);
 
+/* ---- products that share their first operand (q/k/v, gate/up) ----------------------------------
+ * The weights of such MatMuls (ref: one cublasGemmStridedBatchedEx each,
+ * cuda/src/kernels/gemm.rs:191-232) lie side by side in one row-major matrix B [k, sum(widths)].
+ *
+ * rmlk_hip_matmul_grouped: outs[i] (dense [m, widths[i]]) = A[m, k] . B[:, block i], block i being
+ * the next widths[i] columns. One launch covers all blocks where whole tiles allow it; otherwise
+ * the blocks are multiplied one after the other, with the same results as rmlk_hip_matmul on each.
+ * groups <= 4. The workspace must hold rmlk_hip_matmul_grouped_workspace_size bytes. */
+size_t rmlk_hip_matmul_grouped_workspace_size(int32_t dtype, int64_t m, int64_t k, int32_t groups,
+                                              const int64_t *widths);
+int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t k,
+                                const void *a, int64_t lda, const void *b, int64_t ldb,
+                                int32_t groups, const int64_t *widths, void *const *outs,
+                                void *workspace, size_t workspace_bytes);
+/* out[m, n] = swiglu(A . B[:, gate_offset .. +n], A . B[:, up_offset .. +n]) (see rmlk_hip_swiglu)
+ * in one launch, the activation applied to the accumulators. Covers m % 128 == 0, n % 64 == 0,
+ * k % 32 == 0, 16-byte aligned rows and at least one tile per compute unit; RMLK_ERR_UNSUPPORTED
+ * otherwise (the caller then multiplies and activates separately). */
+int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n, int64_t k,
+                               const void *a, int64_t lda, const void *b, int64_t ldb,
+                               int64_t gate_offset, int64_t up_offset, void *out, int64_t ldc);
+
 /* Rotary position embedding, half-rotation form, over x of logical shape [B, H, S, D]:
  * out = x * cos + concat(-x[..., D/2:], x[..., :D/2]) * sin, out dense [B, H, S, D].
  * x, cos and sin are read through element strides per dim of `shape` (innermost stride 1; 0 on

@@ -28,6 +28,18 @@ namespace {
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+constexpr int kMaxSegments = 4;
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant
+// expression inside the body.
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
 struct GemmArgs {
     const float *a;
     const float *b;
@@ -38,6 +50,15 @@ struct GemmArgs {
     int32_t k_per_split;                   // K range of one z-slice (multiple of BK)
     int32_t tiles_m, tiles_n;
     int32_t aligned;                       // rows of A and B start on 16-byte boundaries
+    // Column blocks of C with a destination each (grouped products): block i covers columns
+    // [seg_begin[i], seg_begin[i + 1]) and is written to seg_c[i] with leading dimension seg_ldc[i].
+    // n_seg == 0: plain C. Block boundaries are multiples of the tile width.
+    int32_t n_seg;
+    int32_t seg_begin[kMaxSegments + 1];
+    float *seg_c[kMaxSegments];
+    int64_t seg_ldc[kMaxSegments];
+    // SwiGLU epilogue: columns of the gate and of the up projection inside B
+    int32_t gate_offset, up_offset;
 };
 
 constexpr int kThreads = 256;
@@ -348,9 +369,14 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
 // row r lives in unit q ^ (r & 7), applied on the global side when the unit is fetched and again
 // when it is read back. The loads are opaque to the compiler (inline asm), so completion is
 // awaited by hand (vmcnt) before the block-wide barrier that publishes a stage.
-template <int BM, int BN, int WM, int WN, bool TB, int STAGES>
+//
+// SWIGLU: the block's B tile is half gate columns, half up columns of one joint weight matrix,
+// arranged so that a wavefront's first accumulator column holds gate values and its second the up
+// values of the SAME output columns; the epilogue writes silu(gate) * up, BN / 2 columns per tile.
+template <int BM, int BN, int WM, int WN, bool TB, int STAGES, bool SWIGLU = false>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) {
-    static_assert(STAGES == 2 || STAGES == 3, "two or three LDS stages");
+    static_assert(STAGES == 2, "two LDS stages");
+    static_assert(!SWIGLU || (!TB && WN == 64), "SwiGLU epilogue: row-major B, two accumulator columns");
     constexpr int BK = 32;
     constexpr int KC = BK / 8;
     constexpr int kAFloats = BM * BK;   // one stage of A, floats
@@ -386,19 +412,34 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int l32 = lane % 32, half = lane / 32;
 
-    // this lane's global sources: piece (p * 4 + wave) of a stage, advanced by one K step per stage
+    // Global sources of a stage: piece (p * 4 + wave) goes to this wavefront. The address is a
+    // wave-uniform base (scalar registers, advanced with scalar adds) plus a per-lane byte offset
+    // that never changes, so the loads cost no vector ALU work.
     const int sw_row = lane / 8, sw_unit = (lane % 8) ^ sw_row;
-    const float *a_src = A + static_cast<int64_t>(m0 + wave * 8 + sw_row) * g.lda + k_begin + sw_unit * 4;
+    const uint32_t a_voff =
+        static_cast<uint32_t>(((wave * 8 + sw_row) * g.lda + sw_unit * 4) * static_cast<int64_t>(4));
+    const float *a_ptr = A + static_cast<int64_t>(m0) * g.lda + k_begin;
     const int64_t a_pass_stride = static_cast<int64_t>(32) * g.lda;
-    const float *b_src;
+    uint32_t b_voff;
+    const float *b_ptr;
     int64_t b_pass_stride, b_step_stride;
     if constexpr (TB) {
-        b_src = B + static_cast<int64_t>(n0 + wave * 8 + sw_row) * g.ldb + k_begin + sw_unit * 4;
+        b_voff = static_cast<uint32_t>(((wave * 8 + sw_row) * g.ldb + sw_unit * 4) * static_cast<int64_t>(4));
+        b_ptr = B + static_cast<int64_t>(n0) * g.ldb + k_begin;
         b_pass_stride = static_cast<int64_t>(32) * g.ldb;
         b_step_stride = BK;
     } else {
-        b_src = B + static_cast<int64_t>(k_begin + wave * B_ROWS_PER_PIECE + lane / B_ROW_LANES) * g.ldb +
-                n0 + (lane % B_ROW_LANES) * 4;
+        const int krow = wave * B_ROWS_PER_PIECE + lane / B_ROW_LANES;
+        int col = (lane % B_ROW_LANES) * 4;    // LDS column of the tile this lane fills
+        if constexpr (SWIGLU) {
+            // LDS column c: wavefront column c / 64, accumulator (c % 64) / 32, lane c % 32
+            const int out_col = tile_n * (BN / 2) + (col / 64) * 32 + col % 32;
+            col = ((col % 64) / 32 ? g.up_offset : g.gate_offset) + out_col;
+            b_ptr = B + static_cast<int64_t>(k_begin) * g.ldb;
+        } else {
+            b_ptr = B + static_cast<int64_t>(k_begin) * g.ldb + n0;
+        }
+        b_voff = static_cast<uint32_t>((krow * g.ldb + col) * static_cast<int64_t>(4));
         b_pass_stride = static_cast<int64_t>(4 * B_ROWS_PER_PIECE) * g.ldb;
         b_step_stride = static_cast<int64_t>(BK) * g.ldb;
     }
@@ -408,23 +449,25 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     const uint32_t lds_b = __builtin_amdgcn_readfirstlane(
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>(Bs)) + wave * 1024u);
 
-    auto direct_load = [&](uint32_t lds_addr, const float *src) {
-        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off"
+    auto direct_load = [&](uint32_t lds_addr, const float *base, uint32_t voff) {
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
                      :
-                     : "s"(lds_addr), "v"(src)
+                     : "s"(lds_addr), "v"(voff), "s"(base)
                      : "memory", "m0");
     };
-    auto issue_stage = [&](int buf) {
-#pragma unroll
-        for (int p = 0; p < A_PASSES; ++p)
-            direct_load(lds_a + static_cast<uint32_t>(buf * kAFloats * 4 + p * 4096),
-                        a_src + p * a_pass_stride);
-#pragma unroll
-        for (int p = 0; p < B_PASSES; ++p)
-            direct_load(lds_b + static_cast<uint32_t>(buf * kBFloats * 4 + p * 4096),
-                        b_src + p * b_pass_stride);
-        a_src += BK;
-        b_src += b_step_stride;
+    constexpr int kLoadsPerStage = A_PASSES + B_PASSES;
+    // load number o of the stage that goes to LDS buffer `buf`
+    auto load_op = [&](int buf, int o) {
+        if (o < A_PASSES)
+            direct_load(lds_a + static_cast<uint32_t>(buf * kAFloats * 4 + o * 4096),
+                        a_ptr + o * a_pass_stride, a_voff);
+        else
+            direct_load(lds_b + static_cast<uint32_t>(buf * kBFloats * 4 + (o - A_PASSES) * 4096),
+                        b_ptr + (o - A_PASSES) * b_pass_stride, b_voff);
+    };
+    auto advance_sources = [&]() {
+        a_ptr += BK;
+        b_ptr += b_step_stride;
     };
 
     // fragment addressing
@@ -433,25 +476,23 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     const int b_base = TB ? (wn * WN + l32) * BK : (half * 4) * BN + wn * WN + l32;
     v4f af[2][TM];
     float bf[2][TN][4];
-    auto read_frags = [&](int buf, int kc, int slot) {
-        const float *as = As + buf * kAFloats + a_row;
-        const float *bs = Bs + buf * kBFloats + b_base;
+    // The fragments of one 8-wide K chunk are fetched by kFragOps LDS reads: TM 128-bit reads of A,
+    // then B as TN 128-bit reads (K-contiguous B) or 2 * TN pairs of 32-bit reads.
+    constexpr int kFragOps = TM + (TB ? TN : 2 * TN);
+    auto frag_op = [&](int buf, int kc, int slot, int o) {
         const int unit = ((kc * 2 + half) ^ xr) * 4;
+        if (o < TM) {
+            af[slot][o] = *reinterpret_cast<const v4f *>(As + buf * kAFloats + a_row + o * 32 * BK + unit);
+        } else if constexpr (TB) {
+            const int j = o - TM;
+            const v4f bv = *reinterpret_cast<const v4f *>(Bs + buf * kBFloats + b_base + j * 32 * BK + unit);
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
-            af[slot][i] = *reinterpret_cast<const v4f *>(as + i * 32 * BK + unit);
-        if constexpr (TB) {
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const v4f bv = *reinterpret_cast<const v4f *>(bs + j * 32 * BK + unit);
-#pragma unroll
-                for (int s = 0; s < 4; ++s) bf[slot][j][s] = bv[s];
-            }
+            for (int s = 0; s < 4; ++s) bf[slot][j][s] = bv[s];
         } else {
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) bf[slot][j][s] = bs[(kc * 8 + s) * BN + j * 32];
+            const int j = (o - TM) / 2, s0 = ((o - TM) % 2) * 2;
+            const float *bs = Bs + buf * kBFloats + b_base + j * 32;
+            bf[slot][j][s0] = bs[(kc * 8 + s0) * BN];
+            bf[slot][j][s0 + 1] = bs[(kc * 8 + s0 + 1) * BN];
         }
     };
 
@@ -462,74 +503,122 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    auto mfma_chunk = [&](int slot, int s_begin, int s_end) {
-#pragma unroll
-        for (int s = s_begin; s < s_end; ++s)
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[slot][i][s], bf[slot][j][s],
-                                                                     acc[i][j], 0, 0, 0);
-    };
-    // This wavefront's LDS reads are complete and its direct loads have landed, all of them or all
-    // but the newest stage's (loads complete in issue order); then the block meets.
-    constexpr int kLoadsPerStage = A_PASSES + B_PASSES;
-    auto stage_barrier = [&](bool newest_may_fly) {
-        if (newest_may_fly)
-            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kLoadsPerStage) : "memory");
-        else
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    // This wavefront's LDS reads are complete and its direct loads have landed; then the block
+    // meets: the stage just loaded may be read, the stage just read may be overwritten.
+    auto stage_barrier = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    // One K step. The matrix pipe takes a new MFMA every 64 cycles and the wavefront issues in
+    // order, so everything else -- the next chunk's fragment reads, the next stage's global loads,
+    // the barrier -- is dealt out between the MFMAs a few instructions at a time instead of in
+    // bursts that would let the pipe run dry. Chunks 0 .. KC-2 read the fragments of the chunk after
+    // them and issue the loads of the next stage; the last chunk meets the block a quarter of the
+    // way in and then reads chunk 0 of the next stage.
+    constexpr int NM = 4 * TM * TN;                  // MFMAs per chunk
+#ifndef RMLK_GEMM_LOAD_CHUNKS
+#define RMLK_GEMM_LOAD_CHUNKS 1
+#endif
+#ifndef RMLK_GEMM_BARRIER_AT
+#define RMLK_GEMM_BARRIER_AT 2
+#endif
+    constexpr int kLoadChunks = RMLK_GEMM_LOAD_CHUNKS;   // chunks (from the first) that carry the loads
+    constexpr int kLoadsPerChunk = (kLoadsPerStage + kLoadChunks - 1) / kLoadChunks;
+    constexpr int kBarrierAt = NM * RMLK_GEMM_BARRIER_AT / 4 < NM - 1 ? NM * RMLK_GEMM_BARRIER_AT / 4 : NM - 2;
+    auto k_step = [&](int buf, auto load_tag, auto more_tag) {
+        constexpr bool LOAD = decltype(load_tag)::value;   // another stage to fetch
+        constexpr bool MORE = decltype(more_tag)::value;   // another step follows
+        const int other = buf ^ 1;
+        static_for<KC>([&](auto kc_tag) {
+            constexpr int kc = decltype(kc_tag)::value;
+            constexpr int slot = kc & 1;
+            constexpr bool last = kc == KC - 1;
+            constexpr bool loads_here = LOAD && kc < kLoadChunks;
+            constexpr int load_lo = loads_here ? (kc * kLoadsPerChunk < kLoadsPerStage ? kc * kLoadsPerChunk
+                                                                                       : kLoadsPerStage)
+                                               : 0;
+            constexpr int load_hi =
+                loads_here ? ((kc + 1) * kLoadsPerChunk < kLoadsPerStage ? (kc + 1) * kLoadsPerChunk
+                                                                         : kLoadsPerStage)
+                           : 0;
+            constexpr int n_frag = last ? (MORE ? kFragOps : 0) : kFragOps;
+            constexpr int n_ops = n_frag + (load_hi - load_lo);
+            constexpr int first = last ? kBarrierAt + 1 : 0;     // first MFMA that carries an op
+            constexpr int room = NM - first;
+            static_for<NM>([&](auto q_tag) {
+                constexpr int q = decltype(q_tag)::value;
+                constexpr int s = q / (TM * TN), i = (q / TN) % TM, j = q % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[slot][i][s], bf[slot][j][s],
+                                                                 acc[i][j], 0, 0, 0);
+                if constexpr (last && MORE && q == kBarrierAt) stage_barrier();
+                static_for<n_ops>([&](auto o_tag) {
+                    constexpr int o = decltype(o_tag)::value;
+                    if constexpr (first + o * room / n_ops == q) {
+                        if constexpr (o < n_frag) {
+                            if constexpr (last) frag_op(other, 0, slot ^ 1, o);
+                            else frag_op(buf, kc + 1, slot ^ 1, o);
+                        } else {
+                            load_op(other, load_lo + o - n_frag);
+                        }
+                    }
+                });
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            if constexpr (LOAD && kc == kLoadChunks - 1) advance_sources();
+        });
     };
 
-    // Stage t lives in LDS buffer t % STAGES and is requested STAGES - 1 steps before its use; the
-    // buffer it overwrites was last read in the step before the request, and that step ended with
-    // the barrier.
-    constexpr int D = STAGES - 1;
-    int buf = 0, buf_next = STAGES > 2 ? 1 : 1 % STAGES, buf_load = D % STAGES;
     if (n_steps > 0) {
-        issue_stage(0);
-        if (D == 2 && n_steps > 1) issue_stage(1);
-        stage_barrier(D == 2 && n_steps > 1);
-        read_frags(0, 0, 0);
-    }
-    for (int step = 0; step < n_steps; ++step) {
-        const bool more = step + 1 < n_steps;
-        const bool load = step + D < n_steps;
-        mfma_chunk(0, 0, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        if (load) issue_stage(buf_load);
-        read_frags(buf, 1, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_chunk(0, 1, 4);
-        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int kc = 1; kc < KC; ++kc) {
-            const int slot = kc & 1;
-            if (kc + 1 < KC) {
-                read_frags(buf, kc + 1, slot ^ 1);
-            } else {
-                stage_barrier(D == 2 && load);
-                if (more) read_frags(buf_next, 0, slot ^ 1);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_chunk(slot, 0, 4);
-            __builtin_amdgcn_sched_barrier(0);
+        for (int o = 0; o < kLoadsPerStage; ++o) load_op(0, o);
+        advance_sources();
+        stage_barrier();
+#pragma unroll
+        for (int o = 0; o < kFragOps; ++o) frag_op(0, 0, 0, o);
+        int buf = 0;
+        for (int step = 0; step + 1 < n_steps; ++step) {
+            k_step(buf, std::true_type{}, std::true_type{});
+            buf ^= 1;
         }
-        buf = buf_next;
-        buf_next = buf_next + 1 == STAGES ? 0 : buf_next + 1;
-        buf_load = buf_load + 1 == STAGES ? 0 : buf_load + 1;
+        k_step(buf, std::false_type{}, std::false_type{});
     }
 
+    if constexpr (SWIGLU) {
+        const int col = tile_n * (BN / 2) + wn * 32 + l32;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+                const float gate = acc[i][0][r];
+                const float silu = gate * (1.0f / (1.0f + expf(-gate)));
+                C[static_cast<int64_t>(row) * g.ldc + col] = silu * acc[i][1][r];
+            }
+        }
+        return;
+    }
+    int64_t ldc = g.ldc;
+    int col0 = n0;
+    if (g.n_seg > 0 && gridDim.z == 1) {
+        // constant indices only: the argument struct stays in scalar registers
+        C = g.seg_c[0];
+        ldc = g.seg_ldc[0];
+#pragma unroll
+        for (int i = 1; i < kMaxSegments; ++i)
+            if (i < g.n_seg && n0 >= g.seg_begin[i]) {
+                C = g.seg_c[i];
+                ldc = g.seg_ldc[i];
+                col0 = n0 - g.seg_begin[i];
+            }
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const int col = n0 + wn * WN + j * 32 + l32;
+            const int col = col0 + wn * WN + j * 32 + l32;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                C[static_cast<int64_t>(row) * g.ldc + col] = acc[i][j][r];
+                C[static_cast<int64_t>(row) * ldc + col] = acc[i][j][r];
             }
         }
     }
@@ -550,6 +639,43 @@ __global__ __launch_bounds__(kThreads) void splitk_reduce_kernel(const float *__
         const int64_t b = i / per, rem = i - b * per;
         const int64_t r = rem / n, col = rem - r * n;
         c[b * stride_c + r * ldc + col] = s;
+    }
+}
+
+// Destinations of the column blocks of one [m][n] matrix (see GemmArgs).
+struct Segments {
+    int32_t n_seg;
+    int32_t begin[kMaxSegments + 1];
+    float *c[kMaxSegments];
+    int64_t ldc[kMaxSegments];
+};
+
+// The same sum, four columns per lane; n, every block boundary and every leading dimension are
+// multiples of 4 and all pointers 16-byte aligned. One matrix (batch 1).
+__global__ __launch_bounds__(kThreads) void splitk_reduce_vec_kernel(const float *__restrict__ ws,
+                                                                     Segments sg, int splits,
+                                                                     int32_t m, int32_t n) {
+    const int n4 = n / 4;
+    const int64_t total4 = static_cast<int64_t>(m) * n4;
+    const int64_t slab = static_cast<int64_t>(m) * n;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < total4;
+         i += static_cast<int64_t>(gridDim.x) * kThreads) {
+        const float *src = ws + i * 4;
+        v4f s = *reinterpret_cast<const v4f *>(src);
+        for (int z = 1; z < splits; ++z) s += *reinterpret_cast<const v4f *>(src + z * slab);
+        const int r = static_cast<int>(i / n4);
+        const int col = static_cast<int>(i - static_cast<int64_t>(r) * n4) * 4;
+        float *dst = sg.c[0];
+        int64_t ldc = sg.ldc[0];
+        int col0 = col;
+#pragma unroll
+        for (int j = 1; j < kMaxSegments; ++j)
+            if (j < sg.n_seg && col >= sg.begin[j]) {
+                dst = sg.c[j];
+                ldc = sg.ldc[j];
+                col0 = col - sg.begin[j];
+            }
+        *reinterpret_cast<v4f *>(dst + static_cast<int64_t>(r) * ldc + col0) = s;
     }
 }
 
@@ -902,6 +1028,12 @@ inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k) {
         if (max_splits < 1) max_splits = 1;
         if (splits > max_splits) splits = static_cast<int>(max_splits);
         if (splits > 32) splits = 32;
+        // a split count that cuts K into equal whole K steps keeps the kernel without bounds checks
+        for (int more = splits; more <= 2 * splits && more <= max_splits; ++more)
+            if (k % (static_cast<int64_t>(more) * t.bk) == 0) {
+                splits = more;
+                break;
+            }
     }
     int64_t kps = (k + splits - 1) / splits;
     kps = (kps + t.bk - 1) / t.bk * t.bk;
@@ -963,10 +1095,10 @@ int32_t launch_mfma(hipStream_t s, const GemmArgs &g, int64_t batch, int splits)
     return launch_status();
 }
 
-template <int BM, int BN, int WM, int WN, bool TB, int STAGES>
+template <int BM, int BN, int WM, int WN, bool TB, int STAGES, bool SWIGLU = false>
 int32_t launch_direct(hipStream_t s, const GemmArgs &g, int64_t batch, int splits) {
     constexpr int kBytes = STAGES * (BM * 32 + 32 * BN) * 4;
-    auto kern = gemm_mfma_direct_kernel<BM, BN, WM, WN, TB, STAGES>;
+    auto kern = gemm_mfma_direct_kernel<BM, BN, WM, WN, TB, STAGES, SWIGLU>;
     if (kBytes > 64 * 1024) {
         const int32_t st = allow_dynamic_lds(kern, kBytes);
         if (st) return st;
@@ -975,6 +1107,146 @@ int32_t launch_direct(hipStream_t s, const GemmArgs &g, int64_t batch, int split
               static_cast<unsigned>(splits));
     kern<<<grid, kThreads, kBytes, s>>>(g);
     return launch_status();
+}
+
+// The tiled MFMA path of a product (m > 1, A not transposed). `seg`: column blocks of C with their
+// own destinations (see Segments; their rows must be 16-byte aligned) instead of c/ldc; the call
+// then answers RMLK_ERR_UNSUPPORTED unless the whole-tile kernel applies.
+int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k, const float *pa,
+                   int64_t lda, int64_t stride_a, const float *pb, int64_t ldb, int64_t stride_b,
+                   int32_t trans_b, float *pc, int64_t ldc, int64_t stride_c, void *workspace,
+                   size_t workspace_bytes, const Segments *seg) {
+    TileChoice t = choose_tiles(batch, m, n, k);
+    GemmArgs g{};
+    g.a = pa;
+    g.b = pb;
+    g.m = static_cast<int32_t>(m);
+    g.n = static_cast<int32_t>(n);
+    g.k = static_cast<int32_t>(k);
+    g.lda = lda;
+    g.ldb = ldb;
+    g.stride_a = stride_a;
+    g.stride_b = stride_b;
+    g.k_per_split = t.k_per_split;
+    g.tiles_m = static_cast<int32_t>((m + t.bm - 1) / t.bm);
+    g.tiles_n = static_cast<int32_t>((n + t.bn - 1) / t.bn);
+    if (static_cast<int64_t>(g.tiles_m) * g.tiles_n >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
+    if (t.splits > 1) {
+        const size_t need = static_cast<size_t>(t.splits) * batch * m * n * sizeof(float);
+        if (!workspace || workspace_bytes < need) return RMLK_ERR_WORKSPACE;
+        g.c = static_cast<float *>(workspace);
+        g.ldc = n;
+        g.stride_c = m * n;
+    } else {
+        g.c = pc;
+        g.ldc = ldc;
+        g.stride_c = stride_c;
+        if (seg) {
+            g.n_seg = seg->n_seg;
+            for (int i = 0; i < seg->n_seg; ++i) {
+                g.seg_begin[i] = seg->begin[i];
+                g.seg_c[i] = seg->c[i];
+                g.seg_ldc[i] = seg->ldc[i];
+            }
+            g.seg_begin[seg->n_seg] = seg->begin[seg->n_seg];
+        }
+    }
+    const bool aligned = lda % 4 == 0 && ldb % 4 == 0 && stride_a % 4 == 0 && stride_b % 4 == 0 &&
+                         reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(pb) % 16 == 0;
+    g.aligned = aligned ? 1 : 0;
+    const bool full = aligned && m % t.bm == 0 && n % t.bn == 0 && t.k_per_split % t.bk == 0 &&
+                      k % t.k_per_split == 0;
+    int32_t st;
+#define RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, TB_)                                                   \
+    (t.bk == 32                                                                                  \
+         ? (full ? launch_mfma<BM_, BN_, 32, WM_, WN_, false, TB_>(s, g, batch, t.splits)        \
+                 : launch_mfma<BM_, BN_, 32, WM_, WN_, true, TB_>(s, g, batch, t.splits))        \
+         : (full ? launch_mfma<BM_, BN_, 16, WM_, WN_, false, TB_>(s, g, batch, t.splits)        \
+                 : launch_mfma<BM_, BN_, 16, WM_, WN_, true, TB_>(s, g, batch, t.splits)))
+#define RMLK_LAUNCH(BM_, BN_, WM_, WN_)                                                          \
+    (trans_b ? RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, true) : RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, false))
+#define RMLK_DIRECT_S(BM_, BN_, WM_, WN_, S_)                                                    \
+    (trans_b ? launch_direct<BM_, BN_, WM_, WN_, true, S_>(s, g, batch, t.splits)                \
+             : launch_direct<BM_, BN_, WM_, WN_, false, S_>(s, g, batch, t.splits))
+    // two LDS stages: a third (loads two K steps ahead) measured no faster and halves the blocks
+    // that fit a CU
+#ifndef RMLK_GEMM_STAGES
+#define RMLK_GEMM_STAGES 2
+#endif
+#ifndef RMLK_GEMM_DIRECT
+#define RMLK_GEMM_DIRECT 1
+#endif
+#define RMLK_DIRECT(BM_, BN_, WM_, WN_) RMLK_DIRECT_S(BM_, BN_, WM_, WN_, RMLK_GEMM_STAGES)
+    const bool direct = RMLK_GEMM_DIRECT && full && t.bk == 32;
+    if (seg) {
+        // column blocks with their own destinations: whole tiles only, no tile across a boundary
+        if (!direct || batch != 1) return RMLK_ERR_UNSUPPORTED;
+        for (int i = 0; i <= seg->n_seg; ++i)
+            if (seg->begin[i] % t.bn != 0) return RMLK_ERR_UNSUPPORTED;
+    }
+    if (direct && t.bm == 256) st = RMLK_DIRECT(256, 64, 64, 64);
+    else if (direct && t.bm == 128) st = RMLK_DIRECT(128, 128, 64, 64);
+    else if (direct) st = RMLK_DIRECT(64, 64, 32, 32);
+    else if (t.bm == 256) st = RMLK_LAUNCH(256, 64, 64, 64);
+    else if (t.bm == 128) st = RMLK_LAUNCH(128, 128, 64, 64);
+    else st = RMLK_LAUNCH(64, 64, 32, 32);
+#undef RMLK_DIRECT
+#undef RMLK_DIRECT_S
+#undef RMLK_LAUNCH
+#undef RMLK_LAUNCH_TB
+    if (st) return st;
+    if (t.splits > 1) {
+        Segments one{};
+        if (!seg && batch == 1 && n % 4 == 0 && ldc % 4 == 0 &&
+            reinterpret_cast<uintptr_t>(pc) % 16 == 0 && reinterpret_cast<uintptr_t>(g.c) % 16 == 0) {
+            one.n_seg = 1;
+            one.begin[1] = static_cast<int32_t>(n);
+            one.c[0] = pc;
+            one.ldc[0] = ldc;
+            seg = &one;
+        }
+        if (seg) {
+            unsigned rg = grid_for(m * n / 4, kThreads, 8);
+            splitk_reduce_vec_kernel<<<rg, kThreads, 0, s>>>(g.c, *seg, t.splits, g.m, g.n);
+        } else {
+            unsigned rg = grid_for(batch * m * n, kThreads, 8);
+            splitk_reduce_kernel<<<rg, kThreads, 0, s>>>(g.c, pc, t.splits, batch, g.m, g.n, ldc,
+                                                         stride_c);
+        }
+        return launch_status();
+    }
+    return RMLK_OK;
+}
+
+// silu(A . B[:, gate..]) * (A . B[:, up..]) in one launch: 128 x 128 tiles of 64 gate and 64 up
+// columns. Whole tiles, no split-K, enough tiles to cover the chip; otherwise UNSUPPORTED.
+int32_t gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float *pa, int64_t lda,
+                    const float *pb, int64_t ldb, int64_t gate_offset, int64_t up_offset, float *pc,
+                    int64_t ldc) {
+    const bool aligned = lda % 4 == 0 && ldb % 4 == 0 && gate_offset % 4 == 0 && up_offset % 4 == 0 &&
+                         reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(pb) % 16 == 0;
+    if (!aligned || m % 128 != 0 || n % 64 != 0 || k % 32 != 0 || k < 32) return RMLK_ERR_UNSUPPORTED;
+    const int64_t tiles = (m / 128) * (n / 64);
+    if (tiles < kNumCU || tiles >= (1ll << 31)) return RMLK_ERR_UNSUPPORTED;
+    GemmArgs g{};
+    g.a = pa;
+    g.b = pb;
+    g.c = pc;
+    g.m = static_cast<int32_t>(m);
+    g.n = static_cast<int32_t>(2 * n);
+    g.k = static_cast<int32_t>(k);
+    g.lda = lda;
+    g.ldb = ldb;
+    g.ldc = ldc;
+    g.k_per_split = g.k;
+    g.tiles_m = static_cast<int32_t>(m / 128);
+    g.tiles_n = static_cast<int32_t>(n / 64);
+    g.aligned = 1;
+    g.gate_offset = static_cast<int32_t>(gate_offset);
+    g.up_offset = static_cast<int32_t>(up_offset);
+    return launch_direct<128, 128, 64, 64, false, 2, true>(s, g, 1, 1);
 }
 
 }  // namespace
@@ -1185,78 +1457,8 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
         return launch_status();
     }
 
-    TileChoice t = choose_tiles(batch, m, n, k);
-    GemmArgs g{};
-    g.a = pa;
-    g.b = pb;
-    g.m = static_cast<int32_t>(m);
-    g.n = static_cast<int32_t>(n);
-    g.k = static_cast<int32_t>(k);
-    g.lda = lda;
-    g.ldb = ldb;
-    g.stride_a = stride_a;
-    g.stride_b = stride_b;
-    g.k_per_split = t.k_per_split;
-    g.tiles_m = static_cast<int32_t>((m + t.bm - 1) / t.bm);
-    g.tiles_n = static_cast<int32_t>((n + t.bn - 1) / t.bn);
-    if (static_cast<int64_t>(g.tiles_m) * g.tiles_n >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
-    if (t.splits > 1) {
-        const size_t need = static_cast<size_t>(t.splits) * batch * m * n * sizeof(float);
-        if (!workspace || workspace_bytes < need) return RMLK_ERR_WORKSPACE;
-        g.c = static_cast<float *>(workspace);
-        g.ldc = n;
-        g.stride_c = m * n;
-    } else {
-        g.c = pc;
-        g.ldc = ldc;
-        g.stride_c = stride_c;
-    }
-    const bool aligned = lda % 4 == 0 && ldb % 4 == 0 && stride_a % 4 == 0 && stride_b % 4 == 0 &&
-                         reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
-                         reinterpret_cast<uintptr_t>(pb) % 16 == 0;
-    g.aligned = aligned ? 1 : 0;
-    const bool full = aligned && m % t.bm == 0 && n % t.bn == 0 && t.k_per_split % t.bk == 0 &&
-                      k % t.k_per_split == 0;
-    int32_t st;
-#define RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, TB_)                                                   \
-    (t.bk == 32                                                                                  \
-         ? (full ? launch_mfma<BM_, BN_, 32, WM_, WN_, false, TB_>(s, g, batch, t.splits)        \
-                 : launch_mfma<BM_, BN_, 32, WM_, WN_, true, TB_>(s, g, batch, t.splits))        \
-         : (full ? launch_mfma<BM_, BN_, 16, WM_, WN_, false, TB_>(s, g, batch, t.splits)        \
-                 : launch_mfma<BM_, BN_, 16, WM_, WN_, true, TB_>(s, g, batch, t.splits)))
-#define RMLK_LAUNCH(BM_, BN_, WM_, WN_)                                                          \
-    (trans_b ? RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, true) : RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, false))
-#define RMLK_DIRECT_S(BM_, BN_, WM_, WN_, S_)                                                    \
-    (trans_b ? launch_direct<BM_, BN_, WM_, WN_, true, S_>(s, g, batch, t.splits)                \
-             : launch_direct<BM_, BN_, WM_, WN_, false, S_>(s, g, batch, t.splits))
-    // two LDS stages: a third (loads two K steps ahead) measured no faster and halves the blocks
-    // that fit a CU
-#ifndef RMLK_GEMM_STAGES
-#define RMLK_GEMM_STAGES 2
-#endif
-#ifndef RMLK_GEMM_DIRECT
-#define RMLK_GEMM_DIRECT 1
-#endif
-#define RMLK_DIRECT(BM_, BN_, WM_, WN_) RMLK_DIRECT_S(BM_, BN_, WM_, WN_, RMLK_GEMM_STAGES)
-    const bool direct = RMLK_GEMM_DIRECT && full && t.bk == 32;
-    if (direct && t.bm == 256) st = RMLK_DIRECT(256, 64, 64, 64);
-    else if (direct && t.bm == 128) st = RMLK_DIRECT(128, 128, 64, 64);
-    else if (direct) st = RMLK_DIRECT(64, 64, 32, 32);
-    else if (t.bm == 256) st = RMLK_LAUNCH(256, 64, 64, 64);
-    else if (t.bm == 128) st = RMLK_LAUNCH(128, 128, 64, 64);
-    else st = RMLK_LAUNCH(64, 64, 32, 32);
-#undef RMLK_DIRECT
-#undef RMLK_DIRECT_S
-#undef RMLK_LAUNCH
-#undef RMLK_LAUNCH_TB
-    if (st) return st;
-    if (t.splits > 1) {
-        unsigned rg = grid_for(batch * m * n, kThreads, 8);
-        splitk_reduce_kernel<<<rg, kThreads, 0, s>>>(g.c, pc, t.splits, batch, g.m, g.n, ldc,
-                                                     stride_c);
-        return launch_status();
-    }
-    return RMLK_OK;
+    return gemm_tiled(s, batch, m, n, k, pa, lda, stride_a, pb, ldb, stride_b, trans_b, pc, ldc, stride_c,
+                      workspace, workspace_bytes, nullptr);
 }
 
 extern "C" size_t rmlk_hip_gemv_partials_workspace_size(int32_t dtype, int64_t n, int64_t k) {
@@ -1294,4 +1496,82 @@ extern "C" int32_t rmlk_hip_gemv_partials(rmlk_stream_t stream, int32_t dtype, i
     gemv_kernel<4><<<grid, kThreads, 0, as_stream(stream)>>>(g);
     *splits_out = splits;
     return launch_status();
+}
+
+extern "C" size_t rmlk_hip_matmul_grouped_workspace_size(int32_t dtype, int64_t m, int64_t k,
+                                                         int32_t groups, const int64_t *widths) {
+    if (dtype != RMLK_FLOAT || !widths || groups <= 0 || groups > kMaxSegments) return 0;
+    int64_t total = 0;
+    size_t need = 0;
+    for (int i = 0; i < groups; ++i) {
+        if (widths[i] < 0) return 0;
+        total += widths[i];
+        const size_t one = rmlk_hip_matmul_workspace_size(dtype, 1, m, widths[i], k);
+        if (one > need) need = one;
+    }
+    const size_t joint = rmlk_hip_matmul_workspace_size(dtype, 1, m, total, k);
+    return joint > need ? joint : need;
+}
+
+extern "C" int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t k,
+                                           const void *a, int64_t lda, const void *b, int64_t ldb,
+                                           int32_t groups, const int64_t *widths, void *const *outs,
+                                           void *workspace, size_t workspace_bytes) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (!widths || !outs) return RMLK_ERR_NULL_POINTER;
+    if (groups <= 0 || groups > kMaxSegments || m < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    int64_t total = 0;
+    Segments sg{};
+    sg.n_seg = groups;
+    bool joint = m > kSkinnyRows && k > 0;
+    for (int i = 0; i < groups; ++i) {
+        if (widths[i] < 0) return RMLK_ERR_INVALID_ARGUMENT;
+        if (widths[i] > 0 && m > 0 && !outs[i]) return RMLK_ERR_NULL_POINTER;
+        sg.begin[i] = static_cast<int32_t>(total);
+        sg.c[i] = static_cast<float *>(outs[i]);
+        sg.ldc[i] = widths[i];
+        joint = joint && widths[i] > 0 && widths[i] % 4 == 0 &&
+                reinterpret_cast<uintptr_t>(outs[i]) % 16 == 0;
+        total += widths[i];
+    }
+    if (total >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
+    if (ldb < total) return RMLK_ERR_SIZE_MISMATCH;
+    sg.begin[groups] = static_cast<int32_t>(total);
+    if (m == 0 || total == 0) return RMLK_OK;
+    if (!a || !b) return RMLK_ERR_NULL_POINTER;
+    if (joint) {
+        const size_t need = rmlk_hip_matmul_workspace_size(dtype, 1, m, total, k);
+        if (need && (!workspace || workspace_bytes < need)) return RMLK_ERR_WORKSPACE;
+        const int32_t st = gemm_tiled(as_stream(stream), 1, m, total, k, static_cast<const float *>(a),
+                                      lda, 0, static_cast<const float *>(b), ldb, 0, 0, sg.c[0], sg.ldc[0],
+                                      0, workspace, workspace_bytes, &sg);
+        if (st != RMLK_ERR_UNSUPPORTED) return st;
+    }
+    int64_t off = 0;
+    for (int i = 0; i < groups; ++i) {
+        if (widths[i] > 0) {
+            const int32_t st = rmlk_hip_matmul(stream, dtype, 1, m, widths[i], k, a, lda, 0, 0,
+                                               static_cast<const float *>(b) + off, ldb, 0, 0, outs[i],
+                                               widths[i], 0, workspace, workspace_bytes);
+            if (st) return st;
+        }
+        off += widths[i];
+    }
+    return RMLK_OK;
+}
+
+extern "C" int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n,
+                                          int64_t k, const void *a, int64_t lda, const void *b,
+                                          int64_t ldb, int64_t gate_offset, int64_t up_offset, void *out,
+                                          int64_t ldc) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (m < 0 || n < 0 || k < 0 || gate_offset < 0 || up_offset < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (m >= (1ll << 31) || n >= (1ll << 30) || k >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
+    if (lda < k || ldc < n || ldb < gate_offset + n || ldb < up_offset + n) return RMLK_ERR_SIZE_MISMATCH;
+    if (m == 0 || n == 0) return RMLK_OK;
+    if (!a || !b || !out) return RMLK_ERR_NULL_POINTER;
+    if (reinterpret_cast<uintptr_t>(out) % 4 != 0) return RMLK_ERR_UNSUPPORTED;
+    return gemm_swiglu(as_stream(stream), m, n, k, static_cast<const float *>(a), lda,
+                       static_cast<const float *>(b), ldb, gate_offset, up_offset,
+                       static_cast<float *>(out), ldc);
 }

@@ -859,6 +859,21 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
     const int64_t k = w.shape[0];
     const bool ok = a.dtype == RMLK_FLOAT && a.rank() >= 1 && a.shape.back() == k && a.numel() == k &&
                     widths.size() == 2 && widths[0] == widths[1];
+    const bool same_width = a.dtype == RMLK_FLOAT && a.rank() >= 1 && a.shape.back() == k && k > 0 &&
+                            widths.size() == 2 && widths[0] == widths[1];
+    if (same_width && a.numel() / k >= 128) {
+        // many rows: one GEMM over [gate | up] with the activation applied to the accumulators
+        const int64_t n = widths[0], m = a.numel() / k;
+        const bool gate_first = c.attr_int("gate_first", 1) != 0;
+        std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
+        shape.push_back(n);
+        Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
+        if (took_fast_path(rmlk_hip_matmul_swiglu(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, w.data(),
+                                                  2 * n, gate_first ? 0 : n, gate_first ? n : 0, y.data(),
+                                                  n),
+                           "rmlk.MatMulGroupSwiGLU"))
+            return;
+    }
     const void *ws = nullptr;
     int32_t splits = 0;
     if (ok && gemv_partials(c, a, w, &ws, &splits)) {
@@ -917,6 +932,21 @@ void op_fused_matmul_group(OpContext &c) {
             *c.out[i] = v;
             off += widths[i];
         }
+        return;
+    }
+    if (widths.size() <= 4) {
+        // one launch whose tiles write to the members' outputs (or the members one by one, as the
+        // kernel library sees fit)
+        std::vector<void *> outs;
+        for (size_t i = 0; i < widths.size(); ++i)
+            outs.push_back(c.alloc_output(static_cast<int>(i), RMLK_FLOAT, out_shape(widths[i])).data());
+        const size_t ws_bytes = rmlk_hip_matmul_grouped_workspace_size(
+            RMLK_FLOAT, m, k, static_cast<int32_t>(widths.size()), widths.data());
+        void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
+        check_status(rmlk_hip_matmul_grouped(c.stream, RMLK_FLOAT, m, k, a.data(), k, w.data(), total,
+                                             static_cast<int32_t>(widths.size()), widths.data(),
+                                             outs.data(), ws, ws_bytes),
+                     "rmlk.MatMulGroup");
         return;
     }
     int64_t off = 0;

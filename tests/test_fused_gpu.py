@@ -568,3 +568,110 @@ def test_one_row_products_leave_their_combine_to_the_consumer(device, rows):
     for name in a:
         assert_close(a[name], b[name], rtol=1e-4, atol=1e-5)
         assert_close(a[name], exp[name], rtol=1e-4, atol=1e-5)
+
+
+# ---- products that share their first operand: one launch over the joint weight matrix -----------
+
+@pytest.mark.parametrize("m,k,widths", [
+    (512, 2048, [2048, 512, 512]),      # q/k/v of the 1B shape: split-K, blocks meet in the combine
+    (2048, 256, [1024, 256, 256]),      # enough tiles: the GEMM's own tiles write to the members
+    (256, 512, [128, 128]),
+    (512, 2048, [2048, 320, 512]),      # a boundary inside a tile: members one by one
+    (40, 96, [64, 32, 32]),             # ragged rows: members one by one
+    (5, 256, [128, 64]),                # skinny
+    (128, 64, [256, 0, 128, 128]),      # an empty member
+])
+def test_grouped_matmul_matches_separate_products(device, m, k, widths):
+    import torch
+    kk = _k()
+    rng = np.random.default_rng(m + k + len(widths))
+    a_np = rng.standard_normal((m, k), dtype=np.float32)
+    b_np = rng.standard_normal((k, sum(widths)), dtype=np.float32) * np.float32(0.02)
+    a, b = to_dev(a_np, device), to_dev(b_np, device)
+    outs = [torch.full((m, w), float("nan"), device=device) for w in widths]
+    kk.matmul_grouped(a, b, outs, m, k, widths)
+    off = 0
+    for w, got in zip(widths, outs):
+        if w:
+            sep = torch.empty(m, w, device=device)
+            kk.matmul(a, b[:, off:off + w].contiguous(), sep, 1, m, w, k, k, w, w, 0, 0, 0)
+            assert_close(to_np(got), to_np(sep), rtol=1e-4, atol=1e-5)
+            exp = a_np.astype(np.float64) @ b_np[:, off:off + w].astype(np.float64)
+            assert_close(to_np(got), exp.astype(np.float32), rtol=1e-4, atol=1e-5)
+        off += w
+
+
+def test_grouped_matmul_argument_checks(device):
+    import torch
+    from rmlk_amd import RmlkError
+    kk = _k()
+    a = torch.zeros(128, 64, device=device)
+    b = torch.zeros(64, 256, device=device)
+    outs = [torch.zeros(128, 64, device=device) for _ in range(5)]
+    with pytest.raises(RmlkError):
+        kk.matmul_grouped(a, b, outs, 128, 64, [64] * 5)       # more members than the entry takes
+    with pytest.raises(RmlkError):
+        kk.matmul_grouped(a, b, outs[:2], 128, 64, [64, -1])
+
+
+@pytest.mark.parametrize("m,n,k,gate_first", [(512, 8192, 2048, True), (256, 8192, 64, False),
+                                              (2048, 1024, 512, True)])
+def test_matmul_swiglu_matches_separate_kernels(device, m, n, k, gate_first):
+    import torch
+    kk = _k()
+    rng = np.random.default_rng(m + n + k)
+    a_np = rng.standard_normal((m, k), dtype=np.float32)
+    b_np = rng.standard_normal((k, 2 * n), dtype=np.float32) * np.float32(0.02)
+    a, b = to_dev(a_np, device), to_dev(b_np, device)
+    go, uo = (0, n) if gate_first else (n, 0)
+    got = torch.full((m, n), float("nan"), device=device)
+    kk.matmul_swiglu(a, b, got, m, n, k, 2 * n, go, uo)
+    gate, up = torch.empty(m, n, device=device), torch.empty(m, n, device=device)
+    kk.matmul(a, b[:, go:go + n].contiguous(), gate, 1, m, n, k, k, n, n, 0, 0, 0)
+    kk.matmul(a, b[:, uo:uo + n].contiguous(), up, 1, m, n, k, k, n, n, 0, 0, 0)
+    sep = torch.empty(m, n, device=device)
+    kk.swiglu(gate, up, sep)
+    assert_close(to_np(got), to_np(sep), rtol=1e-4, atol=1e-5)
+    g64 = a_np.astype(np.float64) @ b_np[:, go:go + n].astype(np.float64)
+    u64 = a_np.astype(np.float64) @ b_np[:, uo:uo + n].astype(np.float64)
+    exp = g64 / (1.0 + np.exp(-g64)) * u64
+    assert_close(to_np(got), exp.astype(np.float32), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 8192, 256), (512, 8200, 256), (512, 128, 256), (512, 8192, 48)])
+def test_matmul_swiglu_declines_what_it_does_not_cover(device, m, n, k):
+    import torch
+    from rmlk_amd import RmlkError
+    kk = _k()
+    a = torch.zeros(m, k, device=device)
+    b = torch.zeros(k, 2 * n, device=device)
+    out = torch.zeros(m, n, device=device)
+    with pytest.raises(RmlkError) as e:
+        kk.matmul_swiglu(a, b, out, m, n, k, 2 * n, 0, n)
+    assert e.value.status == -2
+
+
+@pytest.mark.parametrize("rows", [128, 384])
+def test_gate_up_swiglu_of_many_rows_is_one_launch(device, rows):
+    """[gate | up] -> SwiGLU with whole row tiles: the session's fused node takes the GEMM with the
+    activation in its epilogue; results against the one-kernel-per-node session and the oracle."""
+    from oracle import graph as og
+    hid, ffn = 128, 8192
+    gb = _builder()
+    gb.input("x", np.float32, [1, 0, hid])
+    rng = np.random.default_rng(rows)
+    for name in ("wg", "wu"):
+        gb.constant(name, (rng.standard_normal((hid, ffn)) * 0.1).astype(np.float32))
+    gb.op("MatMul", ["x", "wg"], ["g"])
+    gb.op("MatMul", ["x", "wu"], ["u"])
+    gb.op("Sigmoid", ["g"], ["sg"])
+    gb.op("Mul", ["g", "sg"], ["silu"])
+    gb.op("Mul", ["silu", "u"], ["act"])
+    gb.output("act")
+    graph = gb.build()
+    feeds = {"x": rng.standard_normal((1, rows, hid), dtype=np.float32)}
+    a, b, n, _ = _run_both(graph, feeds)
+    assert n == 3      # SwiGLU, the gate/up group, their merge
+    exp = og.run_graph(graph, feeds)
+    assert_close(a["act"], b["act"], rtol=1e-4, atol=1e-5)
+    assert_close(a["act"], exp["act"], rtol=1e-4, atol=1e-5)
