@@ -450,7 +450,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>(Bs)) + wave * 1024u);
 
     auto direct_load = [&](uint32_t lds_addr, const float *base, uint32_t voff) {
-        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+        // (one wait state between a scalar write of M0 and the LDS-bound load that reads it)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                      :
                      : "s"(lds_addr), "v"(voff), "s"(base)
                      : "memory", "m0");
@@ -479,17 +480,20 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     // The fragments of one 8-wide K chunk are fetched by kFragOps LDS reads: TM 128-bit reads of A,
     // then B as TN 128-bit reads (K-contiguous B) or 2 * TN pairs of 32-bit reads.
     constexpr int kFragOps = TM + (TB ? TN : 2 * TN);
+    // in the order the MFMAs want them: A row block 0, the first half of every B column block,
+    // the other A row blocks, the second halves of B
     auto frag_op = [&](int buf, int kc, int slot, int o) {
         const int unit = ((kc * 2 + half) ^ xr) * 4;
-        if (o < TM) {
-            af[slot][o] = *reinterpret_cast<const v4f *>(As + buf * kAFloats + a_row + o * 32 * BK + unit);
+        if (o == 0 || (o > TN && o < TN + TM)) {
+            const int i = o == 0 ? 0 : o - TN;
+            af[slot][i] = *reinterpret_cast<const v4f *>(As + buf * kAFloats + a_row + i * 32 * BK + unit);
         } else if constexpr (TB) {
-            const int j = o - TM;
+            const int j = o - 1;
             const v4f bv = *reinterpret_cast<const v4f *>(Bs + buf * kBFloats + b_base + j * 32 * BK + unit);
 #pragma unroll
             for (int s = 0; s < 4; ++s) bf[slot][j][s] = bv[s];
         } else {
-            const int j = (o - TM) / 2, s0 = ((o - TM) % 2) * 2;
+            const int j = o <= TN ? o - 1 : o - TN - TM, s0 = o <= TN ? 0 : 2;
             const float *bs = Bs + buf * kBFloats + b_base + j * 32;
             bf[slot][j][s0] = bs[(kc * 8 + s0) * BN];
             bf[slot][j][s0 + 1] = bs[(kc * 8 + s0 + 1) * BN];
@@ -552,7 +556,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
                 if constexpr (last && MORE && q == kBarrierAt) stage_barrier();
                 static_for<n_ops>([&](auto o_tag) {
                     constexpr int o = decltype(o_tag)::value;
-                    if constexpr (first + o * room / n_ops == q) {
+                    // one op per MFMA from `first` on while they fit, else spread evenly
+                    if constexpr ((n_ops <= room ? first + o : first + o * room / n_ops) == q) {
                         if constexpr (o < n_frag) {
                             if constexpr (last) frag_op(other, 0, slot ^ 1, o);
                             else frag_op(buf, kc + 1, slot ^ 1, o);
