@@ -38,8 +38,6 @@ CALIBRATION_COPY_BYTES = 256 << 20
 PMC_TRAFFIC_KIB = {
     (1, 512, 2048, 2048): (49257, 16384),
     (1, 512, 512, 2048): (24634, 4096),
-    (8, 2048, 640, 64): (13512, 35334),
-    (8, 2048, 64, 640): (42941, 4096),
     (1, 512, 8192, 2048): (98403, 16384),
     (1, 512, 2048, 8192): (196706, 16384),
     (1, 512, 128256, 2048): (2109895, 256512),
@@ -134,8 +132,7 @@ def run_llama(args):
     stats = inst.node_stats()
     # classify each MatMul node by the kernel the library picks for its shape
     launches = matmul_launches(cfg, prompt_len, max_len)
-    mm_nodes = [s for s in stats if s["op"] in ("MatMul", "rmlk.AttnMatMul", "rmlk.MatMulGroup",
-                                                "rmlk.MatMulGroupSwiGLU")]
+    mm_nodes = [s for s in stats if s["op"] in ("MatMul", "rmlk.MatMulGroup", "rmlk.MatMulGroupSwiGLU")]
     assert len(mm_nodes) == len(launches), (len(mm_nodes), len(launches))
     by_kind, per_op = {}, {}
     for s, shapes in zip(mm_nodes, launches):
@@ -315,11 +312,10 @@ def decode_weight_bytes(cfg):
 
 def matmul_launches(cfg, s, max_len):
     """(batch, m, n, k[, "swiglu"]) of the GEMM launches behind every MatMul-type node of the fused
-    scatter-style graph, in node order: q/k/v (one node, one launch over the joint weights), scores,
-    context, o, gate/up (one node, one launch with the SwiGLU epilogue; n counts both halves), down
-    per layer, then the lm-head."""
+    scatter-style graph, in node order: q/k/v (one node, one launch over the joint weights), o,
+    gate/up (one node, one launch with the SwiGLU epilogue; n counts both halves), down per layer,
+    then the lm-head. (Scores, softmax and context are one attention kernel, not a GEMM launch.)"""
     h, kvd, d = cfg.hidden, cfg.kv_heads * cfg.head_dim, cfg.head_dim
-    rep = cfg.heads // cfg.kv_heads
     whole = s % 128 == 0 and h % 128 == 0 and kvd % 128 == 0 and cfg.ffn % 64 == 0
     qkv = [(1, s, cfg.heads * d + 2 * kvd, h)] if whole else \
         [(1, s, cfg.heads * d, h), (1, s, kvd, h), (1, s, kvd, h)]
@@ -327,10 +323,7 @@ def matmul_launches(cfg, s, max_len):
         [(1, s, cfg.ffn, h), (1, s, cfg.ffn, h)]
     out = []
     for _ in range(cfg.layers):
-        out += [qkv,
-                # the two attention products run as one strided GEMM per KV head over its q heads
-                [(cfg.kv_heads, rep * s, max_len, d)], [(cfg.kv_heads, rep * s, d, max_len)],
-                [(1, s, h, cfg.heads * d)], gate_up, [(1, s, h, cfg.ffn)]]
+        out += [qkv, [(1, s, h, cfg.heads * d)], gate_up, [(1, s, h, cfg.ffn)]]
     out.append([(1, s, cfg.vocab, h)])
     return out
 

@@ -279,6 +279,23 @@ int32_t rmlk_hip_splitk_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, c
                                int32_t splits, int64_t slab, int64_t gate_offset, int64_t up_offset,
                                void *out);
 
+/* Grouped-query attention over many query rows in one kernel:
+ *   out[b, h, s, :] = Softmax_l(q[b, h, s, :] . k[b, h / rep, l, :] * scale + mask[b, h, s, l]) . v[b, h / rep, :, :]
+ * (scale_is_mul == 0: the scores are DIVIDED by `scale`). q and out are dense [batch, kv_heads * rep,
+ * q_len, head_dim], k and v dense [batch, kv_heads, kv_len, head_dim]; `mask_stride` gives the mask's
+ * element stride per dim of [batch, heads, q_len, kv_len] (0 on broadcast dims, 1 on the last).
+ * Chain: MatMul(q, k^T) -> Div|Mul(scalar) -> Add(mask) -> Softmax(axis -1) -> MatMul(., v) with the
+ * KV heads repeated over their query heads (ref kernels: cuda/src/kernels/gemm.rs:191-232,
+ * binary.rs:58-100, softmax.rs:5-37). The softmax is accumulated chunk by chunk over the keys with a
+ * running maximum, so results agree with the chain to rounding (about 1e-6 relative), not bit for bit.
+ * Covers head_dim == 64 and kv_len % 4 == 0 with 16-byte aligned operands; RMLK_ERR_UNSUPPORTED
+ * otherwise (the caller then runs the separate kernels). */
+int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t kv_heads,
+                           int64_t rep, int64_t q_len, int64_t kv_len, int64_t head_dim,
+                           const void *q, const void *k, const void *v, const void *mask,
+                           const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
+                           void *out);
+
 /* ---- products that share their first operand (q/k/v, gate/up) ----------------------------------
  * The weights of such MatMuls (ref: one cublasGemmStridedBatchedEx each,
  * cuda/src/kernels/gemm.rs:191-232) lie side by side in one row-major matrix B [k, sum(widths)].

@@ -1,0 +1,318 @@
+// Grouped-query attention over many query rows (prefill) in one kernel for gfx950:
+//   out = Softmax(q . k^T * scale + mask) . v,   q [B, G*rep, S, 64], k and v [B, G, L, 64].
+// Replaces three launches of the reference's one-kernel-per-node execution (MatMul via
+// cublasGemmStridedBatchedEx, cuda/src/kernels/gemm.rs:191-232; Div/Mul and Add,
+// cuda/src/kernels/binary.rs:58-100; Softmax, cuda/src/kernels/softmax.rs:5-37; MatMul again) and
+// the [rows, L] score and probability matrices they pass through memory.
+//
+// One block of four wavefronts owns 64 query rows of one KV head (the rep query heads that share
+// it lie one after the other, so they are rows of ONE matrix) and walks the keys in chunks of 64,
+// staged in LDS by direct global -> LDS loads, two buffers. Wavefront (wq, wk) takes query rows
+// wq*32.. and keys wk*32.. of every chunk, with its own running maximum, sum and output
+// accumulator (the two key halves are merged once, at the end, through LDS).
+//
+// Everything is computed TRANSPOSED so that a query stays in one lane from the scores to the
+// output: S^T = K . Q^T puts query l32 into lane column l32 of the 32x32 MFMA result, with 16 keys
+// in the lane's 16 accumulator registers. Those registers, exponentiated, ARE the B operand of
+// O^T += V^T . P^T (MFMA k index = lane half, the same key in both operands), and O^T again has the
+// query as its lane column. Row maxima and sums are therefore per-lane reductions over registers
+// plus one exchange between the two lane halves; no score ever goes through LDS.
+#include <cmath>
+
+#include "common.hpp"
+
+namespace rmlk {
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kAttnThreads = 256;
+constexpr int kHeadDim = 64;
+constexpr int kChunk = 64;                        // keys per step
+constexpr int kTile = kChunk * kHeadDim;          // floats of one staged K or V chunk
+constexpr int kAttnLdsBytes = 2 * 2 * kTile * 4;  // K and V, two buffers each
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct AttnArgs {
+    const float *q;
+    const float *k;
+    const float *v;
+    const float *mask;
+    float *out;
+    int32_t rows;      // rep * S query rows per KV head
+    int32_t seq;       // S
+    int32_t rep;       // query heads per KV head
+    int32_t kv_heads;  // G
+    int32_t len;       // L keys
+    int64_t mask_b, mask_h, mask_s;   // element strides of the mask over batch, head, query
+    float qscale;      // score scale times log2(e): the softmax runs on base-2 exponents
+};
+
+__global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g) {
+    extern __shared__ __align__(16) float smem[];
+    float *Ks = smem;               // [2][64 keys][16 units of 4 floats], unit u of key r at u ^ (r & 15)
+    float *Vs = smem + 2 * kTile;   // [2][64 keys][64], column c of key r at c ^ (32 * ((r >> 2) & 1))
+
+    const int tid = threadIdx.x;
+    const int lane = tid % kWave, wave = tid / kWave;
+    const int l32 = lane % 32, half = lane / 32;
+    const int wq = wave >> 1, wk = wave & 1;
+    const int bg = blockIdx.y;
+    const int b = bg / g.kv_heads, grp = bg - b * g.kv_heads;
+    const int r0 = blockIdx.x * 64;
+    const float *Kg = g.k + static_cast<int64_t>(bg) * g.len * kHeadDim;
+    const float *Vg = g.v + static_cast<int64_t>(bg) * g.len * kHeadDim;
+    const int n_chunks = (g.len + kChunk - 1) / kChunk;
+
+    // ---- staging: piece p * 4 + wave of a chunk (4 keys, 1 KiB) is this wavefront's p-th load -----
+    const int lrow = wave * 4 + lane / 16;   // key of this lane inside a group of 16 keys
+    const int lunit = lane % 16;
+    const uint32_t k_col = static_cast<uint32_t>((lunit ^ (lrow & 15)) * 4);
+    const uint32_t v_col = static_cast<uint32_t>((lunit ^ ((wave & 1) << 3)) * 4);
+    const uint32_t lds_k = __builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(Ks)) + wave * 1024u);
+    const uint32_t lds_v = __builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(Vs)) + wave * 1024u);
+    auto direct_load = [&](uint32_t lds_addr, const float *base, uint32_t voff) {
+        // (one wait state between a scalar write of M0 and the LDS-bound load that reads it)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_addr), "v"(voff), "s"(base)
+                     : "memory", "m0");
+    };
+    auto issue_chunk = [&](int c, int buf) {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int key = min(c * kChunk + p * 16 + lrow, g.len - 1);   // past the end: any valid row
+            direct_load(lds_k + static_cast<uint32_t>(buf * kTile * 4 + p * 4096), Kg,
+                        static_cast<uint32_t>(key * kHeadDim + k_col) * 4u);
+        }
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int key = min(c * kChunk + p * 16 + lrow, g.len - 1);
+            direct_load(lds_v + static_cast<uint32_t>(buf * kTile * 4 + p * 4096), Vg,
+                        static_cast<uint32_t>(key * kHeadDim + v_col) * 4u);
+        }
+    };
+
+    // ---- this lane's query: B operand of S^T, scaled once --------------------------------------
+    const int qrow = min(r0 + wq * 32 + l32, g.rows - 1);
+    const float *qp = g.q + (static_cast<int64_t>(bg) * g.rows + qrow) * kHeadDim + half * 4;
+    v4f qf[8];
+#pragma unroll
+    for (int kc = 0; kc < 8; ++kc) {
+        const v4f raw = *reinterpret_cast<const v4f *>(qp + kc * 8);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) qf[kc][s] = raw[s] * g.qscale;
+    }
+    // The query is in registers before any of the hand-issued loads below starts: the waits the
+    // compiler places for its own loads count only those.
+#pragma unroll
+    for (int kc = 0; kc < 8; ++kc) asm volatile("" : "+v"(qf[kc]));
+    const int head = grp * g.rep + qrow / g.seq, srow = qrow - (qrow / g.seq) * g.seq;
+    const float *mrow = g.mask + b * g.mask_b + head * g.mask_h + srow * g.mask_s;
+
+    const float kNegInf = -INFINITY;
+    float m_run = kNegInf, l_run = 0.f;
+    v16f o0, o1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        o0[r] = 0.f;
+        o1[r] = 0.f;
+    }
+
+    // The mask of this lane's 16 keys of a chunk (keys 8a + 4*half + 0..3 of the wavefront's 32) is
+    // fetched one chunk ahead, together with that chunk's K and V, and everything is awaited at once
+    // at the end of a step with vmcnt(0). (A partial wait in the middle of a step, "all but the
+    // eight newest loads", was tried first and read stale mask registers now and then: loads that
+    // return to registers and loads bound for LDS do not retire in one common order.)
+    auto load_mask = [&](v4f (&dst)[4], int c) {
+        const int key0 = c * kChunk + wk * 32 + 4 * half;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const float *mp = mrow + min(key0 + 8 * a, g.len - 4);
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst[a]) : "v"(mp) : "memory");
+        }
+    };
+    v4f mk[4], mk_next[4];
+    load_mask(mk, 0);
+    issue_chunk(0, 0);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier"
+                 : "+v"(mk[0]), "+v"(mk[1]), "+v"(mk[2]), "+v"(mk[3])
+                 :
+                 : "memory");
+
+    const int k_frag = (wk * 32 + l32) * kHeadDim;     // this lane's key row of a staged chunk
+    const int k_swz = l32 & 15;
+    const int v_frag0 = (wk * 32 + 4 * half) * kHeadDim + (half * 32 + l32);        // d =      l32
+    const int v_frag1 = (wk * 32 + 4 * half) * kHeadDim + ((half ^ 1) * 32 + l32);  // d = 32 + l32
+
+    for (int c = 0; c < n_chunks; ++c) {
+        const int buf = c & 1;
+        const bool more = c + 1 < n_chunks;
+        const int key0 = c * kChunk + wk * 32 + 4 * half;
+        if (more) {
+            load_mask(mk_next, c + 1);
+            issue_chunk(c + 1, buf ^ 1);
+        }
+
+        // S^T (32 keys x 32 queries) = K . Q^T over the 64 head dims
+        v16f st;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[r] = 0.f;
+        const float *ks = Ks + buf * kTile + k_frag;
+#pragma unroll
+        for (int kc = 0; kc < 8; ++kc) {
+            const v4f kf = *reinterpret_cast<const v4f *>(ks + (((kc * 2 + half) ^ k_swz) * 4));
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[s], qf[kc][s], st, 0, 0, 0);
+        }
+        float t[16];
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[4 * a + e] = fmaf(mk[a][e], kLog2e, st[4 * a + e]);
+        if ((c + 1) * kChunk > g.len) {
+            // keys past the end (their rows and mask values were read from valid but unrelated places)
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+                if (key0 + 8 * a >= g.len) {   // L is a multiple of 4: a lane's four keys go together
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) t[4 * a + e] = kNegInf;
+                }
+        }
+        float mx = t[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, t[r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_safe = m_new == kNegInf ? 0.f : m_new;   // a row with nothing visible so far
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+        float p[16], psum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            p[r] = __builtin_amdgcn_exp2f(t[r] - m_safe);
+            psum += p[r];
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            o0[r] *= alpha;
+            o1[r] *= alpha;
+        }
+
+        // O^T (64 dims x 32 queries) += V^T . P^T over this wavefront's 32 keys
+        const float *vs = Vs + buf * kTile;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key_off = (8 * (r / 4) + (r % 4)) * kHeadDim;
+            o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[v_frag0 + key_off], p[r], o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[v_frag1 + key_off], p[r], o1, 0, 0, 0);
+        }
+        // the next chunk and its mask have landed and nobody reads this chunk any more
+        if (more) {
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier"
+                         : "+v"(mk_next[0]), "+v"(mk_next[1]), "+v"(mk_next[2]), "+v"(mk_next[3])
+                         :
+                         : "memory");
+#pragma unroll
+            for (int a = 0; a < 4; ++a) mk[a] = mk_next[a];
+        } else {
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        }
+    }
+
+    // ---- merge the two key halves of every query tile and write ----------------------------------
+    l_run += __shfl_xor(l_run, 32);
+    float *cb = smem + wq * (34 * kWave);   // the staging buffers are free after the last barrier
+    if (wk == 1) {
+        cb[lane] = m_run;
+        cb[kWave + lane] = l_run;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            cb[(2 + r) * kWave + lane] = o0[r];
+            cb[(18 + r) * kWave + lane] = o1[r];
+        }
+    }
+    __syncthreads();
+    if (wk == 0) {
+        const float m1 = cb[lane], l1 = cb[kWave + lane];
+        const float m_f = fmaxf(m_run, m1);
+        const float m_safe = m_f == kNegInf ? 0.f : m_f;
+        const float a0 = __builtin_amdgcn_exp2f(m_run - m_safe), a1 = __builtin_amdgcn_exp2f(m1 - m_safe);
+        const float inv = 1.0f / (l_run * a0 + l1 * a1);   // nothing visible at all: 0 * inf = NaN, as Softmax
+        const int row = r0 + wq * 32 + l32;
+        if (row < g.rows) {
+            float *op = g.out + (static_cast<int64_t>(bg) * g.rows + row) * kHeadDim + 4 * half;
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                v4f w0, w1;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int r = 4 * a + e;
+                    w0[e] = (o0[r] * a0 + cb[(2 + r) * kWave + lane] * a1) * inv;
+                    w1[e] = (o1[r] * a0 + cb[(18 + r) * kWave + lane] * a1) * inv;
+                }
+                *reinterpret_cast<v4f *>(op + 8 * a) = w0;
+                *reinterpret_cast<v4f *>(op + 32 + 8 * a) = w1;
+            }
+        }
+    }
+}
+
+}  // namespace
+}  // namespace rmlk
+
+using namespace rmlk;
+
+extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                      int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
+                                      int64_t head_dim, const void *q, const void *k, const void *v,
+                                      const void *mask, const rmlk_dims *mask_stride,
+                                      int32_t scale_is_mul, float scale, void *out) {
+    if (!dims_ok(mask_stride) || mask_stride->rank != 4) return RMLK_ERR_BAD_RANK;
+    if (batch < 0 || kv_heads < 0 || rep < 0 || q_len < 0 || kv_len < 0 || head_dim < 0)
+        return RMLK_ERR_INVALID_ARGUMENT;
+    if (dtype != RMLK_FLOAT || head_dim != kHeadDim) return RMLK_ERR_UNSUPPORTED;
+    const int64_t rows = rep * q_len;
+    if (batch * kv_heads * rows == 0) return RMLK_OK;
+    if (kv_len == 0) return RMLK_ERR_UNSUPPORTED;   // Softmax over nothing: left to the separate kernels
+    if (!q || !k || !v || !mask || !out) return RMLK_ERR_NULL_POINTER;
+    for (int d = 0; d < 4; ++d)
+        if (mask_stride->v[d] < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    // 128-bit mask loads, 32-bit byte offsets into one KV head, grid limits
+    if (kv_len % 4 != 0 || mask_stride->v[3] != 1 || mask_stride->v[0] % 4 != 0 ||
+        mask_stride->v[1] % 4 != 0 || mask_stride->v[2] % 4 != 0)
+        return RMLK_ERR_UNSUPPORTED;
+    if (kv_len * kHeadDim >= (1ll << 29) || rows >= (1ll << 30) || batch * kv_heads >= 65536)
+        return RMLK_ERR_UNSUPPORTED;
+    if (reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(k) % 16 ||
+        reinterpret_cast<uintptr_t>(v) % 16 || reinterpret_cast<uintptr_t>(mask) % 16 ||
+        reinterpret_cast<uintptr_t>(out) % 16)
+        return RMLK_ERR_UNSUPPORTED;
+    if (scale_is_mul == 0 && scale == 0.f) return RMLK_ERR_UNSUPPORTED;   // x / 0: not this kernel's case
+    AttnArgs g{};
+    g.q = static_cast<const float *>(q);
+    g.k = static_cast<const float *>(k);
+    g.v = static_cast<const float *>(v);
+    g.mask = static_cast<const float *>(mask);
+    g.out = static_cast<float *>(out);
+    g.rows = static_cast<int32_t>(rows);
+    g.seq = static_cast<int32_t>(q_len);
+    g.rep = static_cast<int32_t>(rep);
+    g.kv_heads = static_cast<int32_t>(kv_heads);
+    g.len = static_cast<int32_t>(kv_len);
+    g.mask_b = mask_stride->v[0];
+    g.mask_h = mask_stride->v[1];
+    g.mask_s = mask_stride->v[2];
+    g.qscale = (scale_is_mul ? scale : 1.0f / scale) * kLog2e;
+    static DynamicLdsGrant grant;
+    const int32_t st = grant.ensure(attention_rows_kernel, kAttnLdsBytes);
+    if (st) return st;
+    dim3 grid(static_cast<unsigned>((rows + 63) / 64), static_cast<unsigned>(batch * kv_heads), 1);
+    attention_rows_kernel<<<grid, kAttnThreads, kAttnLdsBytes, as_stream(stream)>>>(g);
+    return launch_status();
+}

@@ -199,6 +199,27 @@ inline int32_t split_pieces(int rank, const int64_t *shape, const int64_t (*stri
     return RMLK_OK;
 }
 
+// A kernel that needs more than 64 KiB of dynamic LDS must be told so once per device. One object
+// per kernel (a function-local static of its launcher).
+struct DynamicLdsGrant {
+    static constexpr int kMaxDevices = 64;
+    bool raised[kMaxDevices] = {};   // benign race: every thread writes the same value
+
+    template <typename Kern>
+    int32_t ensure(Kern kern, int bytes) {
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return static_cast<int32_t>(e);
+        if (dev < 0 || dev >= kMaxDevices || !raised[dev]) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+            if (e != hipSuccess) return static_cast<int32_t>(e);
+            if (dev >= 0 && dev < kMaxDevices) raised[dev] = true;
+        }
+        return RMLK_OK;
+    }
+};
+
 // Grid size for a grid-stride kernel: enough blocks to cover `work` items, capped so that a few
 // waves per SIMD stay resident on all 256 CUs.
 inline unsigned grid_for(int64_t work, int block, int max_blocks_per_cu = 8) {

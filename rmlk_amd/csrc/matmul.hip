@@ -1069,29 +1069,13 @@ inline int gemv_splits(int64_t batch, int64_t n, int64_t k, int cols_per_block, 
     return static_cast<int>((k + kps - 1) / kps);
 }
 
-// Kernels that need more than 64 KiB of dynamic LDS must be told so once per device.
-template <typename Kern>
-int32_t allow_dynamic_lds(Kern kern, int bytes) {
-    constexpr int kMaxDevices = 64;
-    static bool raised[kMaxDevices] = {};   // benign race: every thread writes the same value
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return static_cast<int32_t>(e);
-    if (dev < 0 || dev >= kMaxDevices || !raised[dev]) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-        if (e != hipSuccess) return static_cast<int32_t>(e);
-        if (dev >= 0 && dev < kMaxDevices) raised[dev] = true;
-    }
-    return RMLK_OK;
-}
-
 template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool TB = false>
 int32_t launch_mfma(hipStream_t s, const GemmArgs &g, int64_t batch, int splits) {
     using L = SmemLayout<BM, BN, BK, TB>;
     auto kern = gemm_mfma_kernel<BM, BN, BK, WM, WN, EDGE, TB>;
     if (L::kBytes > 64 * 1024) {
-        const int32_t st = allow_dynamic_lds(kern, L::kBytes);
+        static DynamicLdsGrant grant;   // one per instantiation, i.e. per kernel
+        const int32_t st = grant.ensure(kern, L::kBytes);
         if (st) return st;
     }
     dim3 grid(static_cast<unsigned>(g.tiles_m * g.tiles_n), static_cast<unsigned>(batch),
@@ -1105,7 +1089,8 @@ int32_t launch_direct(hipStream_t s, const GemmArgs &g, int64_t batch, int split
     constexpr int kBytes = STAGES * (BM * 32 + 32 * BN) * 4;
     auto kern = gemm_mfma_direct_kernel<BM, BN, WM, WN, TB, STAGES, SWIGLU>;
     if (kBytes > 64 * 1024) {
-        const int32_t st = allow_dynamic_lds(kern, kBytes);
+        static DynamicLdsGrant grant;   // one per instantiation, i.e. per kernel
+        const int32_t st = grant.ensure(kern, kBytes);
         if (st) return st;
     }
     dim3 grid(static_cast<unsigned>(g.tiles_m * g.tiles_n), static_cast<unsigned>(batch),

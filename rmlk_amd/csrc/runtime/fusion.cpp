@@ -445,6 +445,39 @@ struct Matcher {
         return formed;
     }
 
+    // ---- scores -> softmax -> context, all three already fused nodes: one attention node -----------
+    int form_attention() {
+        int formed = 0;
+        for (size_t n = 0; n < g.nodes.size(); ++n) {
+            if (removed[n] || g.nodes[n].op != "rmlk.ScaleMaskSoftmax") continue;
+            const Node &sm = g.nodes[n];
+            const Node *qk = produced_by(sm.inputs[0], "rmlk.AttnMatMul");
+            if (!qk || attr_int(*qk, "transposed", 0) != 1 || !only_used_by(qk->outputs[0], {&sm}))
+                continue;
+            const int probs = sm.outputs[0];
+            if (g.values[probs].is_output || users[probs].size() != 1) continue;
+            const Node &pv = g.nodes[users[probs][0]];
+            // the context product: with the KV repeat folded in, or (one query head per KV head) plain
+            const bool plain = pv.op == "MatMul" && pv.inputs.size() == 2;
+            if (!plain && (pv.op != "rmlk.AttnMatMul" || attr_int(pv, "transposed", 0) != 0)) continue;
+            if (pv.inputs[0] != probs || pv.inputs[1] == probs || pv.inputs[1] < 0) continue;
+            Node f;
+            f.op = "rmlk.Attention";
+            f.inputs = {qk->inputs[0], qk->inputs[1], sm.inputs[1], pv.inputs[1]};
+            f.outputs = pv.outputs;
+            f.attrs["scale"] = sm.attrs.at("scale");
+            f.attrs["scale_is_mul"] = sm.attrs.at("scale_is_mul");
+            f.attrs["axis"] = sm.attrs.at("axis");
+            for (const char *name : {"expanded", "expand_shape", "reshape_shape"}) {
+                f.attrs[std::string("k_") + name] = qk->attrs.at(name);
+                if (!plain) f.attrs[std::string("v_") + name] = pv.attrs.at(name);
+            }
+            replace({qk, &sm, &pv}, std::move(f));
+            ++formed;
+        }
+        return formed;
+    }
+
     // ---- a producer whose split-K combine can move into the consumer (one-row inputs) -------------
     // (Tried as well and dropped, both slower than what they replace: MatMul -> AddRMSNorm, where the
     // norm owns a row with ONE block that then adds up 32-64 slabs by itself; and one kernel for
@@ -620,6 +653,63 @@ bool took_fast_path(int32_t st, const char *what) {
     return true;
 }
 
+// The Unsqueeze -> Expand -> Reshape chain folded into an attention product must repeat every KV
+// head of kv [B, G, L, D] `rep` times in place ([B, G * rep, L, D]); false when the recorded shapes
+// say anything else.
+bool kv_repeat(const std::vector<int64_t> &e, const std::vector<int64_t> &r, const Tensor &kv, int64_t *rep) {
+    const int64_t in5[5] = {kv.shape[0], kv.shape[1], 1, kv.shape[2], kv.shape[3]};
+    if (e.size() != 5 || r.size() != 4) return false;
+    for (int d = 0; d < 5; ++d)
+        if (d != 2 && e[d] != 1 && e[d] != in5[d]) return false;
+    *rep = e[2];
+    if (*rep < 1) return false;
+    // the Reshape must give [B, G * rep, L, D] (0 copies a dim, one -1 is inferred)
+    const int64_t ex5[5] = {in5[0], in5[1], *rep, in5[3], in5[4]};
+    const int64_t want[4] = {ex5[0], ex5[1] * *rep, ex5[3], ex5[4]};
+    int64_t total = 1, known = 1;
+    for (int64_t d : ex5) total *= d;
+    int infer = -1;
+    int64_t got[4];
+    for (int d = 0; d < 4; ++d) {
+        if (r[d] == -1) {
+            if (infer >= 0) return false;
+            infer = d;
+            got[d] = 1;
+        } else if (r[d] == 0) {
+            got[d] = ex5[d];
+            known *= got[d];
+        } else {
+            got[d] = r[d];
+            known *= got[d];
+        }
+    }
+    if (infer >= 0) {
+        if (known <= 0 || total % known != 0) return false;
+        got[infer] = total / known;
+    }
+    for (int d = 0; d < 4; ++d)
+        if (got[d] != want[d]) return false;
+    return true;
+}
+
+// Element strides of `mask` per dim of `shape` when it broadcasts INTO that shape with a full last
+// dim; false otherwise.
+bool mask_strides(const Tensor &mask, const std::vector<int64_t> &shape, rmlk_dims *out) {
+    const int rank = static_cast<int>(shape.size());
+    if (mask.rank() == 0 || mask.rank() > rank || mask.shape.back() != shape.back()) return false;
+    std::vector<int64_t> st(rank, 0), dense = dense_strides(mask.shape);
+    const int shift = rank - mask.rank();
+    for (int d = 0; d < mask.rank(); ++d) {
+        const int64_t md = mask.shape[d], xd = shape[d + shift];
+        if (md == xd) st[d + shift] = md == 1 ? 0 : dense[d];
+        else if (md == 1) st[d + shift] = 0;
+        else return false;
+    }
+    st[rank - 1] = 1;
+    *out = to_dims(st);
+    return true;
+}
+
 }  // namespace
 
 void op_fused_rmsnorm(OpContext &c) {
@@ -670,22 +760,7 @@ void op_fused_softmax(OpContext &c) {
         ok = axis == -1 || axis == rank - 1;
     }
     rmlk_dims ms{};
-    if (ok) {
-        // the mask must broadcast INTO x's shape, with a full last dim
-        std::vector<int64_t> st(rank, 0), dense = dense_strides(mask.shape);
-        const int shift = rank - mask.rank();
-        for (int d = 0; d < mask.rank() && ok; ++d) {
-            const int64_t md = mask.shape[d], xd = x.shape[d + shift];
-            if (md == xd) st[d + shift] = md == 1 ? 0 : dense[d];
-            else if (md == 1) st[d + shift] = 0;
-            else ok = false;
-        }
-        if (ok && (mask.rank() == 0 || mask.shape.back() != x.shape.back())) ok = false;
-        if (ok) {
-            st[rank - 1] = 1;
-            ms = to_dims(st);
-        }
-    }
+    if (ok) ok = mask_strides(mask, x.shape, &ms);
     if (ok) {
         rmlk_dims xs = to_dims(x.shape);
         Tensor &y = c.alloc_output(0, RMLK_FLOAT, x.shape);
@@ -756,45 +831,7 @@ void op_fused_attn_matmul(OpContext &c) {
     bool ok = a.dtype == RMLK_FLOAT && kv.dtype == RMLK_FLOAT && a.rank() == 4 && kv.rank() == 4 &&
               a.numel() > 0 && kv.numel() > 0;
     int64_t rep = 1;
-    if (ok && expanded) {
-        const std::vector<int64_t> e = c.attr_ints("expand_shape"), r = c.attr_ints("reshape_shape");
-        const int64_t in5[5] = {kv.shape[0], kv.shape[1], 1, kv.shape[2], kv.shape[3]};
-        ok = e.size() == 5 && r.size() == 4;
-        for (int d = 0; d < 5 && ok; ++d)
-            if (d != 2 && e[d] != 1 && e[d] != in5[d]) ok = false;
-        if (ok) {
-            rep = e[2];
-            ok = rep >= 1;
-        }
-        if (ok) {
-            // the Reshape must give [B, G * rep, L, D] (0 copies a dim, one -1 is inferred)
-            const int64_t ex5[5] = {in5[0], in5[1], rep, in5[3], in5[4]};
-            const int64_t want[4] = {ex5[0], ex5[1] * rep, ex5[3], ex5[4]};
-            int64_t total = 1, known = 1;
-            for (int64_t d : ex5) total *= d;
-            int infer = -1;
-            int64_t got[4];
-            for (int d = 0; d < 4 && ok; ++d) {
-                if (r[d] == -1) {
-                    if (infer >= 0) ok = false;
-                    infer = d;
-                    got[d] = 1;
-                } else if (r[d] == 0) {
-                    got[d] = ex5[d];
-                    known *= got[d];
-                } else {
-                    got[d] = r[d];
-                    known *= got[d];
-                }
-            }
-            if (ok && infer >= 0) {
-                ok = known > 0 && total % known == 0;
-                if (ok) got[infer] = total / known;
-            }
-            for (int d = 0; d < 4 && ok; ++d)
-                if (got[d] != want[d]) ok = false;
-        }
-    }
+    if (ok && expanded) ok = kv_repeat(c.attr_ints("expand_shape"), c.attr_ints("reshape_shape"), kv, &rep);
     if (ok) {
         const int64_t bsz = kv.shape[0], grp = kv.shape[1], len = kv.shape[2], dim = kv.shape[3];
         const int64_t heads = a.shape[1], seq = a.shape[2], ka = a.shape[3];
@@ -810,6 +847,41 @@ void op_fused_attn_matmul(OpContext &c) {
                                          m * n, ws, ws_bytes),
                          "rmlk.AttnMatMul");
             return;
+        }
+    }
+    run_body(c);
+}
+
+// scores -> scale, mask, softmax -> context of grouped-query attention in one kernel when there are
+// enough query rows to fill its tiles; a decode step (a handful of rows) runs the three nodes.
+void op_fused_attention(OpContext &c) {
+    const Tensor &q = c.input(0), &k = c.input(1), &mask = c.input(2), &v = c.input(3);
+    bool ok = q.dtype == RMLK_FLOAT && k.dtype == RMLK_FLOAT && v.dtype == RMLK_FLOAT &&
+              mask.dtype == RMLK_FLOAT && q.rank() == 4 && k.rank() == 4 && v.shape == k.shape &&
+              q.numel() > 0 && k.numel() > 0;
+    if (ok) {
+        const int64_t axis = c.attr_int("axis", -1);
+        ok = axis == -1 || axis == 3;
+    }
+    int64_t rep_k = 1, rep_v = 1;
+    if (ok && c.attr_int("k_expanded", 0) != 0)
+        ok = kv_repeat(c.attr_ints("k_expand_shape"), c.attr_ints("k_reshape_shape"), k, &rep_k);
+    if (ok && c.attr_int("v_expanded", 0) != 0)
+        ok = kv_repeat(c.attr_ints("v_expand_shape"), c.attr_ints("v_reshape_shape"), v, &rep_v);
+    rmlk_dims ms{};
+    if (ok) {
+        const int64_t bsz = k.shape[0], grp = k.shape[1], len = k.shape[2], dim = k.shape[3];
+        const int64_t heads = q.shape[1], seq = q.shape[2];
+        ok = rep_k == rep_v && q.shape[0] == bsz && heads == grp * rep_k && q.shape[3] == dim &&
+             rep_k * seq >= 32 && mask_strides(mask, {bsz, heads, seq, len}, &ms);
+        if (ok) {
+            Tensor &y = c.alloc_output(0, RMLK_FLOAT, {bsz, heads, seq, dim});
+            if (took_fast_path(rmlk_hip_attention(c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim,
+                                                  q.data(), k.data(), v.data(), mask.data(), &ms,
+                                                  static_cast<int32_t>(c.attr_int("scale_is_mul", 0)),
+                                                  attr_float(c, "scale"), y.data()),
+                               "rmlk.Attention"))
+                return;
         }
     }
     run_body(c);
@@ -976,6 +1048,7 @@ int fuse_patterns(Session &s) {
             if (m.match_attn_matmul(node)) ++formed;
         }
     }
+    formed += m.form_attention();
     formed += m.form_add_rmsnorm();
     formed += m.form_matmul_groups();
     formed += m.form_splitk_epilogues();

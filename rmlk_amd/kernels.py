@@ -198,6 +198,15 @@ def swiglu(gate, up, out) -> None:
                                 _ptr(out)), "rmlk_hip_swiglu")
 
 
+def attention(q, k, v, mask, out, batch: int, kv_heads: int, rep: int, q_len: int, kv_len: int,
+              head_dim: int, mask_stride, scale: float, scale_is_mul: bool = False) -> None:
+    """Fused grouped-query attention: Softmax(q . k^T (*|/) scale + mask) . v in one kernel."""
+    check(lib().rmlk_hip_attention(_stream(), dtype_of(q), batch, kv_heads, rep, q_len, kv_len,
+                                   head_dim, _ptr(q), _ptr(k), _ptr(v), _ptr(mask),
+                                   Dims.of(mask_stride), int(scale_is_mul), float(scale), _ptr(out)),
+          "rmlk_hip_attention")
+
+
 def matmul_grouped(a, b, outs, m: int, k: int, widths, workspace=None) -> None:
     """outs[i] = a[m, k] . (the next widths[i] columns of the row-major joint matrix b)."""
     n = len(widths)

@@ -210,10 +210,10 @@ def test_pass_forms_the_expected_nodes_on_the_llama_graph(device):
         for kv in ("key", "value"):
             feeds[f"cache.{l}.{kv}"] = np.zeros((1, cfg.kv_heads, 24, cfg.head_dim), np.float32)
     a, b, n, _ = _run_both(graph, feeds)
-    # per layer: 2 RMSNorm, 2 rotary, 1 SwiGLU, 1 softmax, 2 attention MatMuls, the q/k/v and the
-    # gate/up MatMul groups, 2 residual Adds merged into the norm that follows, the gate/up group
-    # merged with the SwiGLU; plus the final RMSNorm
-    assert n == cfg.layers * 13 + 1
+    # per layer: 2 RMSNorm, 2 rotary, 1 SwiGLU, 1 softmax, 2 attention MatMuls, those three merged
+    # into one attention node, the q/k/v and the gate/up MatMul groups, 2 residual Adds merged into
+    # the norm that follows, the gate/up group merged with the SwiGLU; plus the final RMSNorm
+    assert n == cfg.layers * 14 + 1
     # RMSNorm's mean may differ in the last place; everything downstream inherits that
     _same(a, b, loose=set(a.keys()))
     assert np.array_equal(np.argmax(a["logits"][0], -1), np.argmax(b["logits"][0], -1))
@@ -226,7 +226,7 @@ def test_fused_llama_concat_style_against_oracle(device):
     graph = graphs.llama_graph(cfg, seed=4, style="concat")
     feeds = graphs.llama_concat_inputs(cfg, np.random.default_rng(1).integers(0, cfg.vocab, 9), None, 0)
     inst = runtime.Builder.from_graph(graph).build()
-    assert inst.fused_nodes == cfg.layers * 13 + 1
+    assert inst.fused_nodes == cfg.layers * 14 + 1
     got = inst.run(feeds)
     exp = og.run_graph(graph, feeds)
     for name in exp:
@@ -238,7 +238,7 @@ def test_fused_decoder_layer_full_width(device):
     from rmlk_amd import graphs
     graph, feeds = graphs.decoder_layer_graph(seed=3, seq=96)
     a, b, n, _ = _run_both(graph, feeds)
-    assert n == 12
+    assert n == 13
     _same(a, b, loose={"y"})
 
 
@@ -675,3 +675,151 @@ def test_gate_up_swiglu_of_many_rows_is_one_launch(device, rows):
     exp = og.run_graph(graph, feeds)
     assert_close(a["act"], b["act"], rtol=1e-4, atol=1e-5)
     assert_close(a["act"], exp["act"], rtol=1e-4, atol=1e-5)
+
+
+# ---- attention over many query rows in one kernel -----------------------------------------------
+
+def _attention_reference(q, k, v, mask, scale, mul):
+    """float64 numpy: softmax(q k^T (*|/) scale + mask) v with KV heads repeated."""
+    b, h, s, d = q.shape
+    g = k.shape[1]
+    rep = h // g
+    kk = np.repeat(k.astype(np.float64), rep, axis=1)
+    vv = np.repeat(v.astype(np.float64), rep, axis=1)
+    sc = q.astype(np.float64) @ kk.transpose(0, 1, 3, 2)
+    sc = sc * scale if mul else sc / scale
+    sc = sc + np.broadcast_to(mask.astype(np.float64), sc.shape)
+    sc = sc - sc.max(axis=-1, keepdims=True)
+    p = np.exp(sc)
+    p = p / p.sum(axis=-1, keepdims=True)
+    return (p @ vv).astype(np.float32)
+
+
+@pytest.mark.parametrize("b,g,rep,s,l,mask_shape,mul", [
+    (1, 8, 4, 512, 640, (1, 1, 512, 640), False),     # the 1B prefill shape
+    (2, 2, 3, 70, 132, (2, 1, 70, 132), True),        # ragged rows and keys, per-batch mask
+    (1, 1, 1, 33, 4, (1, 1, 33, 4), False),           # fewer keys than one chunk
+    (1, 2, 2, 64, 256, (1, 4, 64, 256), True),        # per-head mask
+    (1, 3, 1, 200, 64, (1, 1, 1, 64), False),         # one mask row for every query
+])
+def test_attention_matches_separate_kernels(device, b, g, rep, s, l, mask_shape, mul):
+    import torch
+    kk = _k()
+    h, d = g * rep, 64
+    rng = np.random.default_rng(b * 1000 + s + l)
+    q_np = rng.standard_normal((b, h, s, d), dtype=np.float32)
+    k_np = rng.standard_normal((b, g, l, d), dtype=np.float32)
+    v_np = rng.standard_normal((b, g, l, d), dtype=np.float32)
+    # causal-style mask with -inf above the diagonal of the last s keys, plus some finite biases
+    m_np = rng.standard_normal(mask_shape, dtype=np.float32)
+    qi = np.arange(mask_shape[2])[:, None] + (l - mask_shape[2])
+    hidden = np.arange(l)[None, :] > np.maximum(qi, 0)
+    m_np = np.where(np.broadcast_to(hidden, mask_shape), np.float32(-np.inf), m_np).astype(np.float32)
+    scale = 8.0 if not mul else 0.125
+    q, k, v, m = (to_dev(x, device) for x in (q_np, k_np, v_np, m_np))
+    got = torch.full((b, h, s, d), float("nan"), device=device)
+    full = [b, h, s, l]
+    ms = bcast_strides(list(mask_shape), full)
+    kk.attention(q, k, v, m, got, b, g, rep, s, l, d, ms, scale, mul)
+    # the chain of separate kernels: scores per KV head (rows of its query heads), softmax, context
+    sc = torch.empty(b, h, s, l, device=device)
+    kk.matmul(q, k, sc, b * g, rep * s, l, d, d, d, l, rep * s * d, l * d, rep * s * l, trans_b=True)
+    pr = torch.empty_like(sc)
+    kk.scale_mask_softmax(sc, m, pr, full, ms, scale, mul)
+    sep = torch.empty(b, h, s, d, device=device)
+    kk.matmul(pr, v, sep, b * g, rep * s, d, l, l, d, d, rep * s * l, l * d, rep * s * d)
+    assert_close(to_np(got), to_np(sep), rtol=1e-4, atol=1e-5)
+    assert_close(to_np(got), _attention_reference(q_np, k_np, v_np, m_np, scale, mul), rtol=1e-4, atol=1e-5)
+
+
+def test_attention_row_with_nothing_visible_is_nan_like_softmax(device):
+    import torch
+    kk = _k()
+    b, g, rep, s, l, d = 1, 1, 1, 40, 128, 64
+    rng = np.random.default_rng(3)
+    q, k, v = (to_dev(rng.standard_normal(sh, dtype=np.float32), device)
+               for sh in ((b, g * rep, s, d), (b, g, l, d), (b, g, l, d)))
+    m_np = np.zeros((1, 1, s, l), dtype=np.float32)
+    m_np[0, 0, 7, :] = -np.inf        # nothing visible
+    m_np[0, 0, 9, :100] = -np.inf     # nothing visible in the first chunk
+    m = to_dev(m_np, device)
+    got = torch.empty(b, g * rep, s, d, device=device)
+    kk.attention(q, k, v, m, got, b, g, rep, s, l, d, [0, 0, l, 1], 8.0)
+    out = to_np(got)
+    assert np.isnan(out[0, 0, 7]).all()
+    assert np.isfinite(np.delete(out, 7, axis=2)).all()
+    exp = _attention_reference(to_np(q), to_np(k), to_np(v), np.where(np.isinf(m_np), -1e30, m_np).astype(np.float32), 8.0, False)
+    assert_close(np.delete(out, 7, axis=2), np.delete(exp, 7, axis=2), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("kw", [dict(d=32), dict(l=130), dict(last_stride=2)])
+def test_attention_declines_what_it_does_not_cover(device, kw):
+    import torch
+    from rmlk_amd import RmlkError
+    kk = _k()
+    d, l = kw.get("d", 64), kw.get("l", 128)
+    q = torch.zeros(1, 2, 64, d, device=device)
+    k = torch.zeros(1, 2, l, d, device=device)
+    m = torch.zeros(64, 2 * l, device=device)
+    out = torch.zeros_like(q)
+    with pytest.raises(RmlkError) as e:
+        kk.attention(q, k, k, m, out, 1, 2, 1, 64, l, d, [0, 0, 2 * l, kw.get("last_stride", 1)], 8.0)
+    assert e.value.status == -2
+
+
+@pytest.mark.parametrize("s,l,rep", [(200, 256, 4), (1, 256, 4), (48, 64, 1)])
+def test_attention_chain_becomes_one_node(device, s, l, rep):
+    """scores -> Div -> Add(mask) -> Softmax -> context over a grouped KV cache: one node; with
+    enough query rows it runs the one-kernel attention, a decode step runs the three nodes."""
+    from oracle import graph as og
+    b, g, d = 1, 2, 64
+    h = g * rep
+    gb = _builder()
+    gb.input("q", np.float32, [b, h, 0, d])
+    gb.input("k", np.float32, [b, g, l, d])
+    gb.input("v", np.float32, [b, g, l, d])
+    gb.input("mask", np.float32, [1, 1, 0, l])
+    gb.constant("ax", np.array([2], np.int64))
+    gb.constant("eshape", np.array([1, g, rep, 1, 1], np.int64))
+    gb.constant("rshape", np.array([b, h, -1, d], np.int64))
+    gb.constant("scale", np.array(8.0, np.float32))
+    for t in ("k", "v"):
+        if rep > 1:
+            gb.op("Unsqueeze", [t, "ax"], [t + "u"])
+            gb.op("Expand", [t + "u", "eshape"], [t + "e"])
+            gb.op("Reshape", [t + "e", "rshape"], [t + "x"])
+    kx, vx = ("kx", "vx") if rep > 1 else ("k", "v")
+    gb.op("Transpose", [kx], ["kt"]).attr("perm", [0, 1, 3, 2])
+    gb.op("MatMul", ["q", "kt"], ["scores"])
+    gb.op("Div", ["scores", "scale"], ["scaled"])
+    gb.op("Add", ["scaled", "mask"], ["masked"])
+    gb.op("Softmax", ["masked"], ["probs"]).attr("axis", -1)
+    gb.op("MatMul", ["probs", vx], ["ctx"])
+    gb.output("ctx")
+    graph = gb.build()
+    rng = np.random.default_rng(s + l)
+    mask = np.triu(np.full((s, l), -np.inf, dtype=np.float32), l - s + 1).reshape(1, 1, s, l)
+    feeds = {"q": rng.standard_normal((b, h, s, d), dtype=np.float32),
+             "k": rng.standard_normal((b, g, l, d), dtype=np.float32),
+             "v": rng.standard_normal((b, g, l, d), dtype=np.float32), "mask": mask}
+    a_, b_, n, _ = _run_both(graph, feeds)
+    # the scores product (K transpose, KV repeat), the softmax chain, the context product when it
+    # carries the KV repeat (plain MatMul otherwise), and the three merged
+    assert n == (4 if rep > 1 else 3)
+    exp = og.run_graph(graph, feeds)
+    assert_close(a_["ctx"], b_["ctx"], rtol=1e-4, atol=1e-5)
+    assert_close(a_["ctx"], exp["ctx"], rtol=1e-4, atol=1e-5)
+
+
+def test_decoder_layer_gives_the_same_bits_every_time(device):
+    """Every kernel sums in a fixed order and awaits its own loads: repeated runs of one session on
+    the same inputs are bit-identical (the recorded-graph replay depends on it)."""
+    from rmlk_amd import graphs, runtime
+    graph, feeds = graphs.decoder_layer_graph(seed=5, seq=512)
+    inst = runtime.Builder.from_graph(graph).build()
+    first = inst.run(feeds)
+    for _ in range(12):
+        again = inst.run(feeds)
+        for name in first:
+            assert_exact(again[name], first[name])
+    inst.close()
