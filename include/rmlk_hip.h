@@ -318,6 +318,23 @@ int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t m, i
                                const void *a, int64_t lda, const void *b, int64_t ldb,
                                int64_t gate_offset, int64_t up_offset, void *out, int64_t ldc);
 
+/* ---- many-row products whose split-K combine is left to the consumer ----------------------------
+ * rmlk_hip_matmul_partials: the tiled kernels of rmlk_hip_matmul for A[m, k] . B[k, n] (row-major,
+ * m > 8) without the combine: `workspace` receives *splits_out partial matrices [m, n] one after
+ * the other (*splits_out >= 1; their sum in ascending order is the product rmlk_hip_matmul returns).
+ * rmlk_hip_splitk_add_rmsnorm: rmlk_hip_add_rmsnorm whose first operand is that sum,
+ * a = partials[0] + partials[1] + ..; `slab` = elements from one partial matrix to the next.
+ * Together they save the combine launch of a projection that feeds a residual Add and a norm.
+ * No counterpart in the reference. */
+size_t rmlk_hip_matmul_partials_workspace_size(int32_t dtype, int64_t m, int64_t n, int64_t k);
+int32_t rmlk_hip_matmul_partials(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n, int64_t k,
+                                 const void *a, int64_t lda, const void *b, int64_t ldb,
+                                 void *workspace, size_t workspace_bytes, int32_t *splits_out);
+int32_t rmlk_hip_splitk_add_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t rows, int64_t cols,
+                                    const void *partials, int32_t splits, int64_t slab,
+                                    const void *b, const void *gamma, float eps,
+                                    int32_t reciprocal_form, void *sum_out, void *out);
+
 /* Rotary position embedding, half-rotation form, over x of logical shape [B, H, S, D]:
  * out = x * cos + concat(-x[..., D/2:], x[..., :D/2]) * sin, out dense [B, H, S, D].
  * x, cos and sin are read through element strides per dim of `shape` (innermost stride 1; 0 on

@@ -95,6 +95,13 @@ SIGNATURES = {
                                          c_int64, c_void_p, c_size_t, POINTER(c_int32)]),
     "rmlk_hip_splitk_swiglu": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                          c_int64, c_int64, c_void_p]),
+    "rmlk_hip_matmul_partials_workspace_size": (c_size_t, [c_int32, c_int64, c_int64, c_int64]),
+    "rmlk_hip_matmul_partials": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p,
+                                           c_int64, c_void_p, c_int64, c_void_p, c_size_t,
+                                           POINTER(c_int32)]),
+    "rmlk_hip_splitk_add_rmsnorm": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int32,
+                                              c_int64, c_void_p, c_void_p, ctypes.c_float, c_int32,
+                                              c_void_p, c_void_p]),
     "rmlk_hip_attention": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64,
                                      c_int64, c_void_p, c_void_p, c_void_p, c_void_p, _PD, c_int32,
                                      ctypes.c_float, c_void_p]),

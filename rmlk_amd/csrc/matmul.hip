@@ -1105,7 +1105,7 @@ int32_t launch_direct(hipStream_t s, const GemmArgs &g, int64_t batch, int split
 int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k, const float *pa,
                    int64_t lda, int64_t stride_a, const float *pb, int64_t ldb, int64_t stride_b,
                    int32_t trans_b, float *pc, int64_t ldc, int64_t stride_c, void *workspace,
-                   size_t workspace_bytes, const Segments *seg) {
+                   size_t workspace_bytes, const Segments *seg, int32_t *partial_splits = nullptr) {
     TileChoice t = choose_tiles(batch, m, n, k);
     GemmArgs g{};
     g.a = pa;
@@ -1121,7 +1121,9 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
     g.tiles_m = static_cast<int32_t>((m + t.bm - 1) / t.bm);
     g.tiles_n = static_cast<int32_t>((n + t.bn - 1) / t.bn);
     if (static_cast<int64_t>(g.tiles_m) * g.tiles_n >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
-    if (t.splits > 1) {
+    if (t.splits > 1 || partial_splits) {
+        // split-K slabs [split][batch][m][n]; with `partial_splits` they are the result (the caller's
+        // consumer adds them up), even when there is only one
         const size_t need = static_cast<size_t>(t.splits) * batch * m * n * sizeof(float);
         if (!workspace || workspace_bytes < need) return RMLK_ERR_WORKSPACE;
         g.c = static_cast<float *>(workspace);
@@ -1186,6 +1188,10 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
 #undef RMLK_LAUNCH
 #undef RMLK_LAUNCH_TB
     if (st) return st;
+    if (partial_splits) {
+        *partial_splits = t.splits;
+        return RMLK_OK;
+    }
     if (t.splits > 1) {
         Segments one{};
         if (!seg && batch == 1 && n % 4 == 0 && ldc % 4 == 0 &&
@@ -1564,4 +1570,26 @@ extern "C" int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, i
     return gemm_swiglu(as_stream(stream), m, n, k, static_cast<const float *>(a), lda,
                        static_cast<const float *>(b), ldb, gate_offset, up_offset,
                        static_cast<float *>(out), ldc);
+}
+
+extern "C" size_t rmlk_hip_matmul_partials_workspace_size(int32_t dtype, int64_t m, int64_t n, int64_t k) {
+    if (dtype != RMLK_FLOAT || m <= kSkinnyRows || n <= 0 || k <= 0) return 0;
+    const TileChoice t = choose_tiles(1, m, n, k);
+    return static_cast<size_t>(t.splits) * m * n * sizeof(float);
+}
+
+extern "C" int32_t rmlk_hip_matmul_partials(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n,
+                                            int64_t k, const void *a, int64_t lda, const void *b,
+                                            int64_t ldb, void *workspace, size_t workspace_bytes,
+                                            int32_t *splits_out) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (m < 0 || n < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (m >= (1ll << 31) || n >= (1ll << 31) || k >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
+    if (m <= kSkinnyRows || n == 0 || k == 0) return RMLK_ERR_UNSUPPORTED;   // not the tiled kernels' case
+    if (!a || !b || !workspace || !splits_out) return RMLK_ERR_NULL_POINTER;
+    if (lda < k || ldb < n) return RMLK_ERR_SIZE_MISMATCH;
+    if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return RMLK_ERR_UNSUPPORTED;
+    return gemm_tiled(as_stream(stream), 1, m, n, k, static_cast<const float *>(a), lda, 0,
+                      static_cast<const float *>(b), ldb, 0, 0, nullptr, n, 0, workspace,
+                      workspace_bytes, nullptr, splits_out);
 }

@@ -335,6 +335,8 @@ struct RmsSource {
     const float *x;       // the row
     const float *add;     // second Add operand, or null
     float *sum_out;       // where the formed row goes (null: nowhere)
+    int32_t slabs;        // x is the first of this many partial matrices (split-K), summed in order
+    int64_t slab;         // elements from one partial matrix to the next
 };
 
 template <int NV, int kGroup, bool RECIP>
@@ -366,6 +368,11 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(RmsSource src,
             const int c = lane_in_group + i * kGroup;
             if (live && c < nv) {
                 xv[i] = pv[c];
+                for (int z = 1; z < src.slabs; ++z) {
+                    const V more = reinterpret_cast<const V *>(src.x + z * src.slab + row * cols)[c];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) xv[i].v[j] = xv[i].v[j] + more.v[j];
+                }
                 if (src.add) {
                     const V av = reinterpret_cast<const V *>(src.add + row * cols)[c];
 #pragma unroll
@@ -570,7 +577,7 @@ extern "C" int32_t rmlk_hip_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t
     if (rows == 0 || cols == 0) return RMLK_OK;
     if (!x || !gamma || !out) return RMLK_ERR_NULL_POINTER;
     if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
-    RmsSource src{static_cast<const float *>(x), nullptr, nullptr};
+    RmsSource src{static_cast<const float *>(x), nullptr, nullptr, 1, 0};
     return rmsnorm_dispatch(as_stream(stream), src, static_cast<const float *>(gamma),
                             static_cast<float *>(out), rows, cols, eps, reciprocal_form != 0);
 }
@@ -585,7 +592,24 @@ extern "C" int32_t rmlk_hip_add_rmsnorm(rmlk_stream_t stream, int32_t dtype, int
     if (!a || !b || !gamma || !sum_out || !out) return RMLK_ERR_NULL_POINTER;
     if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
     RmsSource src{static_cast<const float *>(a), static_cast<const float *>(b),
-                  static_cast<float *>(sum_out)};
+                  static_cast<float *>(sum_out), 1, 0};
+    return rmsnorm_dispatch(as_stream(stream), src, static_cast<const float *>(gamma),
+                            static_cast<float *>(out), rows, cols, eps, reciprocal_form != 0);
+}
+
+extern "C" int32_t rmlk_hip_splitk_add_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t rows,
+                                               int64_t cols, const void *partials, int32_t splits,
+                                               int64_t slab, const void *b, const void *gamma,
+                                               float eps, int32_t reciprocal_form, void *sum_out,
+                                               void *out) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (rows < 0 || cols < 0 || splits < 1 || slab < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (rows == 0 || cols == 0) return RMLK_OK;
+    if (!partials || !b || !gamma || !sum_out || !out) return RMLK_ERR_NULL_POINTER;
+    if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
+    if (splits > 1 && (slab < rows * cols || slab % 4 != 0)) return RMLK_ERR_SIZE_MISMATCH;
+    RmsSource src{static_cast<const float *>(partials), static_cast<const float *>(b),
+                  static_cast<float *>(sum_out), splits, slab};
     return rmsnorm_dispatch(as_stream(stream), src, static_cast<const float *>(gamma),
                             static_cast<float *>(out), rows, cols, eps, reciprocal_form != 0);
 }

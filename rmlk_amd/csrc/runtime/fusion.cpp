@@ -478,16 +478,50 @@ struct Matcher {
         return formed;
     }
 
-    // ---- a producer whose split-K combine can move into the consumer (one-row inputs) -------------
-    // (Tried as well and dropped, both slower than what they replace: MatMul -> AddRMSNorm, where the
-    // norm owns a row with ONE block that then adds up 32-64 slabs by itself; and one kernel for
-    // scores -> softmax -> context of a decode step with one block per KV head, where eight blocks
-    // cannot hide the HBM latency of a cold cache.)
+    // ---- a producer whose split-K combine can move into the consumer -----------------------------
+    // (Tried for one-row inputs as well and dropped, both slower than what they replace: MatMul ->
+    // AddRMSNorm, where the norm owns a row with ONE block that then adds up 32-64 slabs by itself;
+    // and one kernel for scores -> softmax -> context of a decode step with one block per KV head,
+    // where eight blocks cannot hide the HBM latency of a cold cache.)
     int form_splitk_epilogues() {
         int formed = 0;
         for (size_t n = 0; n < g.nodes.size(); ++n) {
             if (removed[n]) continue;
             const Node &cons = g.nodes[n];
+            if (cons.op == "rmlk.AddRMSNorm") {
+                // a projection with constant 2-D weights feeding the residual Add: with many rows the
+                // GEMM's split-K slabs are added up by the norm kernel (a one-row product keeps its
+                // own combine, see above)
+                for (int side = 0; side < 2; ++side) {
+                    const Node *mm = produced_by(cons.inputs[side], "MatMul");
+                    if (!mm || mm->inputs.size() != 2 || mm->inputs[0] < 0 || mm->inputs[1] < 0) continue;
+                    const int w = mm->inputs[1];
+                    if (!g.values[w].is_initializer || !s.values[w].defined() ||
+                        s.values[w].dtype != RMLK_FLOAT || s.values[w].rank() != 2)
+                        continue;
+                    if (!only_used_by(mm->outputs[0], {&cons}) ||
+                        cons.inputs[0] == cons.inputs[1])
+                        continue;
+                    Node f;
+                    f.op = "rmlk.MatMulAddRMSNorm";
+                    f.inputs = {mm->inputs[0], w, cons.inputs[1 - side], cons.inputs[2]};
+                    f.outputs = cons.outputs;
+                    f.attrs = cons.attrs;
+                    Node norm = cons;
+                    f.body = {*mm, norm};
+                    const int mi = index_of(mm);
+                    for (int v : mm->inputs) {
+                        auto &u = users[v];
+                        u.erase(std::remove(u.begin(), u.end(), mi), u.end());
+                        u.push_back(static_cast<int>(n));
+                    }
+                    removed[mi] = true;
+                    g.nodes[n] = std::move(f);
+                    ++formed;
+                    break;
+                }
+                continue;
+            }
             if (cons.op == "rmlk.SwiGLU") {
                 const Node *grp = produced_by(cons.inputs[0], "rmlk.MatMulGroup");
                 if (!grp || grp != produced_by(cons.inputs[1], "rmlk.MatMulGroup") ||
@@ -907,6 +941,43 @@ void op_fused_add_rmsnorm(OpContext &c) {
                                                 sum.data(), y.data()),
                            "rmlk.AddRMSNorm"))
             return;
+    }
+    run_body(c);
+}
+
+// MatMul(a, W) -> Add(residual) -> RMSNorm for many rows: the GEMM leaves its split-K slabs in the
+// workspace and the norm kernel adds them up while it forms the residual row.
+void op_fused_matmul_add_rmsnorm(OpContext &c) {
+    const Tensor &a = c.input(0), &w = c.input(1), &res = c.input(2), &gamma = c.input(3);
+    bool ok = a.dtype == RMLK_FLOAT && w.dtype == RMLK_FLOAT && res.dtype == RMLK_FLOAT &&
+              gamma.dtype == RMLK_FLOAT && a.rank() >= 2 && w.rank() == 2 && a.numel() > 0 &&
+              w.numel() > 0 && a.shape.back() == w.shape[0];
+    if (ok) {
+        std::vector<int64_t> out_shape(a.shape.begin(), a.shape.end() - 1);
+        out_shape.push_back(w.shape[1]);
+        const int64_t axis = c.attr_int("axis", -1);
+        ok = res.shape == out_shape && (axis == -1 || axis == res.rank() - 1) && gamma.rank() >= 1 &&
+             gamma.rank() <= res.rank() && gamma.numel() == w.shape[1] && gamma.shape.back() == w.shape[1];
+    }
+    if (ok) {
+        const int64_t k = w.shape[0], n = w.shape[1], m = a.numel() / k;
+        const size_t bytes = rmlk_hip_matmul_partials_workspace_size(RMLK_FLOAT, m, n, k);
+        if (bytes) {
+            void *ws = c.scratch(bytes);
+            int32_t splits = 0;
+            if (took_fast_path(rmlk_hip_matmul_partials(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, w.data(),
+                                                        n, ws, bytes, &splits),
+                               "rmlk.MatMulAddRMSNorm")) {
+                Tensor &sum = c.alloc_output(0, RMLK_FLOAT, res.shape);
+                Tensor &y = c.alloc_output(1, RMLK_FLOAT, res.shape);
+                if (took_fast_path(rmlk_hip_splitk_add_rmsnorm(
+                                       c.stream, RMLK_FLOAT, m, n, ws, splits, m * n, res.data(), gamma.data(),
+                                       attr_float(c, "epsilon"),
+                                       static_cast<int32_t>(c.attr_int("reciprocal", 0)), sum.data(), y.data()),
+                                   "rmlk.MatMulAddRMSNorm"))
+                    return;
+            }
+        }
     }
     run_body(c);
 }

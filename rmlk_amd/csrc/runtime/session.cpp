@@ -485,6 +485,8 @@ void Session::run_nodes() {
             double out_elems = 0.0;
             for (const Tensor &t : outs) out_elems += static_cast<double>(t.numel());
             flops = 2.0 * out_elems * static_cast<double>(ctx.in[0]->shape.back());
+        } else if (node.op == "rmlk.MatMulAddRMSNorm" && ctx.in[0] && ctx.in[1] && ctx.in[1]->rank() == 2) {
+            flops = 2.0 * static_cast<double>(ctx.in[0]->numel()) * static_cast<double>(ctx.in[1]->shape[1]);
         } else if (node.op == "rmlk.Attention" && ctx.in[0] && ctx.in[1] && ctx.in[0]->rank() == 4 &&
                    ctx.in[1]->rank() == 4) {
             // scores and context: 2 * [B, H, S, L, D] multiply-adds

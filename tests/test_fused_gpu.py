@@ -212,8 +212,9 @@ def test_pass_forms_the_expected_nodes_on_the_llama_graph(device):
     a, b, n, _ = _run_both(graph, feeds)
     # per layer: 2 RMSNorm, 2 rotary, 1 SwiGLU, 1 softmax, 2 attention MatMuls, those three merged
     # into one attention node, the q/k/v and the gate/up MatMul groups, 2 residual Adds merged into
-    # the norm that follows, the gate/up group merged with the SwiGLU; plus the final RMSNorm
-    assert n == cfg.layers * 14 + 1
+    # the norm that follows and the o / down projections merged into those, the gate/up group
+    # merged with the SwiGLU; plus the final RMSNorm
+    assert n == cfg.layers * 16 + 1
     # RMSNorm's mean may differ in the last place; everything downstream inherits that
     _same(a, b, loose=set(a.keys()))
     assert np.array_equal(np.argmax(a["logits"][0], -1), np.argmax(b["logits"][0], -1))
@@ -226,7 +227,7 @@ def test_fused_llama_concat_style_against_oracle(device):
     graph = graphs.llama_graph(cfg, seed=4, style="concat")
     feeds = graphs.llama_concat_inputs(cfg, np.random.default_rng(1).integers(0, cfg.vocab, 9), None, 0)
     inst = runtime.Builder.from_graph(graph).build()
-    assert inst.fused_nodes == cfg.layers * 14 + 1
+    assert inst.fused_nodes == cfg.layers * 16 + 1
     got = inst.run(feeds)
     exp = og.run_graph(graph, feeds)
     for name in exp:
@@ -238,7 +239,7 @@ def test_fused_decoder_layer_full_width(device):
     from rmlk_amd import graphs
     graph, feeds = graphs.decoder_layer_graph(seed=3, seq=96)
     a, b, n, _ = _run_both(graph, feeds)
-    assert n == 13
+    assert n == 14
     _same(a, b, loose={"y"})
 
 
@@ -534,10 +535,11 @@ def test_add_rmsnorm_kernel_matches_separate_kernels(device, rows, cols):
     assert_exact(to_np(got), to_np(exp))
 
 
-@pytest.mark.parametrize("rows", [1, 5])
-def test_one_row_products_leave_their_combine_to_the_consumer(device, rows):
+@pytest.mark.parametrize("rows", [1, 5, 256, 300])
+def test_products_leave_their_combine_to_the_consumer(device, rows):
     """[gate | up] -> SwiGLU: with one input row the GEMV's split-K slabs are added up inside the
-    SwiGLU kernel; more rows run the body."""
+    SwiGLU kernel. o projection -> residual Add -> RMSNorm: with many rows the GEMM's split-K slabs
+    are added up inside the norm kernel. Other row counts run the bodies."""
     from oracle import graph as og
     hid, ffn = 256, 512
     gb = _builder()
@@ -563,7 +565,8 @@ def test_one_row_products_leave_their_combine_to_the_consumer(device, rows):
     feeds = {"x": rng.standard_normal((1, rows, hid), dtype=np.float32),
              "res": rng.standard_normal((1, rows, hid), dtype=np.float32)}
     a, b, n, _ = _run_both(graph, feeds)
-    assert n == 5      # RMSNorm, SwiGLU, AddRMSNorm, gate/up group, group + SwiGLU merge
+    # RMSNorm, SwiGLU, AddRMSNorm, gate/up group, group + SwiGLU merge, o projection + AddRMSNorm merge
+    assert n == 6
     exp = og.run_graph(graph, feeds)
     for name in a:
         assert_close(a[name], b[name], rtol=1e-4, atol=1e-5)
@@ -823,3 +826,38 @@ def test_decoder_layer_gives_the_same_bits_every_time(device):
         for name in first:
             assert_exact(again[name], first[name])
     inst.close()
+
+
+@pytest.mark.parametrize("m,n,k", [(512, 2048, 2048), (512, 2048, 8192), (300, 96, 200), (64, 256, 64)])
+def test_matmul_partials_feed_the_norm(device, m, n, k):
+    """rmlk_hip_matmul_partials + rmlk_hip_splitk_add_rmsnorm against rmlk_hip_matmul +
+    rmlk_hip_add_rmsnorm: the same slabs added in the same order, so the same bits."""
+    import ctypes
+    import torch
+    from rmlk_amd._lib import check, lib
+    kk = _k()
+    rng = np.random.default_rng(m + n + k)
+    a = to_dev(rng.standard_normal((m, k), dtype=np.float32), device)
+    w = to_dev(rng.standard_normal((k, n), dtype=np.float32) * np.float32(0.02), device)
+    res = to_dev(rng.standard_normal((m, n), dtype=np.float32), device)
+    gamma = to_dev(rng.uniform(0.5, 1.5, size=(n,)).astype(np.float32), device)
+    stream = torch.cuda.current_stream().cuda_stream
+    need = int(lib().rmlk_hip_matmul_partials_workspace_size(kk.FLOAT, m, n, k))
+    assert need >= m * n * 4
+    ws = torch.empty(need, dtype=torch.uint8, device=device)
+    splits = ctypes.c_int32(0)
+    check(lib().rmlk_hip_matmul_partials(stream, kk.FLOAT, m, n, k, a.data_ptr(), k, w.data_ptr(), n,
+                                         ws.data_ptr(), need, ctypes.byref(splits)),
+          "rmlk_hip_matmul_partials")
+    assert 1 <= splits.value and splits.value * m * n * 4 <= need
+    got_sum, got = torch.empty_like(res), torch.empty_like(res)
+    check(lib().rmlk_hip_splitk_add_rmsnorm(stream, kk.FLOAT, m, n, ws.data_ptr(), splits.value, m * n,
+                                            res.data_ptr(), gamma.data_ptr(), 1e-5, 0,
+                                            got_sum.data_ptr(), got.data_ptr()),
+          "rmlk_hip_splitk_add_rmsnorm")
+    prod = torch.empty(m, n, device=device)
+    kk.matmul(a, w, prod, 1, m, n, k, k, n, n, 0, 0, 0)
+    exp_sum, exp = torch.empty_like(res), torch.empty_like(res)
+    kk.add_rmsnorm(prod, res, gamma, exp_sum, exp, m, n, 1e-5)
+    assert_exact(to_np(got_sum), to_np(exp_sum))
+    assert_exact(to_np(got), to_np(exp))

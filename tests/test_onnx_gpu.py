@@ -24,9 +24,10 @@ def test_pytorch_export_matches_pytorch_output(device, name, fuse):
     assert inst.memory_stats()["device_syncs"] == 0
     if fuse and name == "torch_decoder_block":
         # 2 RMSNorm (reciprocal form), 2 rotary, SwiGLU, scale+mask+softmax, 2 attention products,
-        # the q/k/v and gate/up MatMul groups, one residual Add merged into the second norm, the
+        # those three merged into one attention node, the q/k/v and gate/up MatMul groups, one
+        # residual Add merged into the second norm and the o projection merged into that, the
         # gate/up group merged with the SwiGLU
-        assert inst.fused_nodes == 13
+        assert inst.fused_nodes == 14
     inst.close()
 
 
