@@ -288,13 +288,15 @@ int32_t rmlk_hip_splitk_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, c
  * KV heads repeated over their query heads (ref kernels: cuda/src/kernels/gemm.rs:191-232,
  * binary.rs:58-100, softmax.rs:5-37). The softmax is accumulated chunk by chunk over the keys with a
  * running maximum, so results agree with the chain to rounding (about 1e-6 relative), not bit for bit.
+ * out_seq_major != 0 writes out as [batch, q_len, heads, head_dim] instead, i.e. the
+ * Transpose(perm 0,2,1,3) that leads to the output projection (ref: cuda/src/kernels/transpose.rs:38-80).
  * Covers head_dim == 64 and kv_len % 4 == 0 with 16-byte aligned operands; RMLK_ERR_UNSUPPORTED
  * otherwise (the caller then runs the separate kernels). */
 int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t kv_heads,
                            int64_t rep, int64_t q_len, int64_t kv_len, int64_t head_dim,
                            const void *q, const void *k, const void *v, const void *mask,
                            const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
-                           void *out);
+                           int32_t out_seq_major, void *out);
 
 /* ---- products that share their first operand (q/k/v, gate/up) ----------------------------------
  * The weights of such MatMuls (ref: one cublasGemmStridedBatchedEx each,

@@ -46,6 +46,7 @@ struct AttnArgs {
     int32_t kv_heads;  // G
     int32_t len;       // L keys
     int64_t mask_b, mask_h, mask_s;   // element strides of the mask over batch, head, query
+    int64_t out_b, out_h, out_s;      // element strides of out over batch, head, query
     float qscale;      // score scale times log2(e): the softmax runs on base-2 exponents
 };
 
@@ -246,7 +247,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
         const float inv = 1.0f / (l_run * a0 + l1 * a1);   // nothing visible at all: 0 * inf = NaN, as Softmax
         const int row = r0 + wq * 32 + l32;
         if (row < g.rows) {
-            float *op = g.out + (static_cast<int64_t>(bg) * g.rows + row) * kHeadDim + 4 * half;
+            float *op = g.out + b * g.out_b + head * g.out_h + srow * g.out_s + 4 * half;   // row == qrow here
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
                 v4f w0, w1;
@@ -272,7 +273,8 @@ extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64
                                       int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
                                       int64_t head_dim, const void *q, const void *k, const void *v,
                                       const void *mask, const rmlk_dims *mask_stride,
-                                      int32_t scale_is_mul, float scale, void *out) {
+                                      int32_t scale_is_mul, float scale, int32_t out_seq_major,
+                                      void *out) {
     if (!dims_ok(mask_stride) || mask_stride->rank != 4) return RMLK_ERR_BAD_RANK;
     if (batch < 0 || kv_heads < 0 || rep < 0 || q_len < 0 || kv_len < 0 || head_dim < 0)
         return RMLK_ERR_INVALID_ARGUMENT;
@@ -309,6 +311,16 @@ extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64
     g.mask_h = mask_stride->v[1];
     g.mask_s = mask_stride->v[2];
     g.qscale = (scale_is_mul ? scale : 1.0f / scale) * kLog2e;
+    const int64_t heads = kv_heads * rep;
+    if (out_seq_major) {   // [batch, q_len, heads, head_dim]
+        g.out_b = q_len * heads * kHeadDim;
+        g.out_s = heads * kHeadDim;
+        g.out_h = kHeadDim;
+    } else {               // [batch, heads, q_len, head_dim]
+        g.out_b = heads * q_len * kHeadDim;
+        g.out_h = q_len * kHeadDim;
+        g.out_s = kHeadDim;
+    }
     static DynamicLdsGrant grant;
     const int32_t st = grant.ensure(attention_rows_kernel, kAttnLdsBytes);
     if (st) return st;

@@ -472,7 +472,21 @@ struct Matcher {
                 f.attrs[std::string("k_") + name] = qk->attrs.at(name);
                 if (!plain) f.attrs[std::string("v_") + name] = pv.attrs.at(name);
             }
-            replace({qk, &sm, &pv}, std::move(f));
+            // a Transpose to [B, S, H, D] behind the context (on the way to the output projection) is
+            // a matter of where the kernel writes
+            std::vector<const Node *> parts = {qk, &sm, &pv};
+            const int ctx = pv.outputs[0];
+            if (!g.values[ctx].is_output && users[ctx].size() == 1) {
+                const Node &tr = g.nodes[users[ctx][0]];
+                auto it = tr.attrs.find("perm");
+                const std::vector<int64_t> want = {0, 2, 1, 3};
+                if (tr.op == "Transpose" && it != tr.attrs.end() && it->second.ints == want) {
+                    f.outputs = tr.outputs;
+                    f.attrs["seq_major_output"] = a_int(1);
+                    parts.push_back(&tr);
+                }
+            }
+            replace(parts, std::move(f));
             ++formed;
         }
         return formed;
@@ -909,11 +923,13 @@ void op_fused_attention(OpContext &c) {
         ok = rep_k == rep_v && q.shape[0] == bsz && heads == grp * rep_k && q.shape[3] == dim &&
              rep_k * seq >= 32 && mask_strides(mask, {bsz, heads, seq, len}, &ms);
         if (ok) {
-            Tensor &y = c.alloc_output(0, RMLK_FLOAT, {bsz, heads, seq, dim});
+            const bool seq_major = c.attr_int("seq_major_output", 0) != 0;
+            Tensor &y = seq_major ? c.alloc_output(0, RMLK_FLOAT, {bsz, seq, heads, dim})
+                                  : c.alloc_output(0, RMLK_FLOAT, {bsz, heads, seq, dim});
             if (took_fast_path(rmlk_hip_attention(c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim,
                                                   q.data(), k.data(), v.data(), mask.data(), &ms,
                                                   static_cast<int32_t>(c.attr_int("scale_is_mul", 0)),
-                                                  attr_float(c, "scale"), y.data()),
+                                                  attr_float(c, "scale"), seq_major ? 1 : 0, y.data()),
                                "rmlk.Attention"))
                 return;
         }

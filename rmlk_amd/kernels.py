@@ -199,11 +199,14 @@ def swiglu(gate, up, out) -> None:
 
 
 def attention(q, k, v, mask, out, batch: int, kv_heads: int, rep: int, q_len: int, kv_len: int,
-              head_dim: int, mask_stride, scale: float, scale_is_mul: bool = False) -> None:
-    """Fused grouped-query attention: Softmax(q . k^T (*|/) scale + mask) . v in one kernel."""
+              head_dim: int, mask_stride, scale: float, scale_is_mul: bool = False,
+              out_seq_major: bool = False) -> None:
+    """Fused grouped-query attention: Softmax(q . k^T (*|/) scale + mask) . v in one kernel; out is
+    [B, H, S, D], or [B, S, H, D] with out_seq_major."""
     check(lib().rmlk_hip_attention(_stream(), dtype_of(q), batch, kv_heads, rep, q_len, kv_len,
                                    head_dim, _ptr(q), _ptr(k), _ptr(v), _ptr(mask),
-                                   Dims.of(mask_stride), int(scale_is_mul), float(scale), _ptr(out)),
+                                   Dims.of(mask_stride), int(scale_is_mul), float(scale),
+                                   int(out_seq_major), _ptr(out)),
           "rmlk_hip_attention")
 
 

@@ -733,6 +733,10 @@ def test_attention_matches_separate_kernels(device, b, g, rep, s, l, mask_shape,
     kk.matmul(pr, v, sep, b * g, rep * s, d, l, l, d, d, rep * s * l, l * d, rep * s * d)
     assert_close(to_np(got), to_np(sep), rtol=1e-4, atol=1e-5)
     assert_close(to_np(got), _attention_reference(q_np, k_np, v_np, m_np, scale, mul), rtol=1e-4, atol=1e-5)
+    # the same numbers written as [B, S, H, D]
+    moved = torch.full((b, s, h, d), float("nan"), device=device)
+    kk.attention(q, k, v, m, moved, b, g, rep, s, l, d, ms, scale, mul, out_seq_major=True)
+    assert_exact(to_np(moved), to_np(got).transpose(0, 2, 1, 3))
 
 
 def test_attention_row_with_nothing_visible_is_nan_like_softmax(device):
@@ -797,7 +801,8 @@ def test_attention_chain_becomes_one_node(device, s, l, rep):
     gb.op("Div", ["scores", "scale"], ["scaled"])
     gb.op("Add", ["scaled", "mask"], ["masked"])
     gb.op("Softmax", ["masked"], ["probs"]).attr("axis", -1)
-    gb.op("MatMul", ["probs", vx], ["ctx"])
+    gb.op("MatMul", ["probs", vx], ["ctx_heads"])
+    gb.op("Transpose", ["ctx_heads"], ["ctx"]).attr("perm", [0, 2, 1, 3])   # absorbed as well
     gb.output("ctx")
     graph = gb.build()
     rng = np.random.default_rng(s + l)
