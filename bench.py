@@ -320,7 +320,8 @@ def matmul_launches(cfg, s, max_len):
     whole = s % 128 == 0 and h % 128 == 0 and kvd % 128 == 0 and cfg.ffn % 64 == 0
     qkv = [(1, s, cfg.heads * d + 2 * kvd, h)] if whole else \
         [(1, s, cfg.heads * d, h), (1, s, kvd, h), (1, s, kvd, h)]
-    gate_up = [(1, s, 2 * cfg.ffn, h, "swiglu")] if whole and (s // 128) * (cfg.ffn // 64) >= 256 else \
+    gate_up = [(1, s, 2 * cfg.ffn, h, "swiglu")] if cfg.ffn % 64 == 0 and h % 32 == 0 and s >= 128 and \
+        ((s + 127) // 128) * (cfg.ffn // 64) >= 256 else \
         [(1, s, cfg.ffn, h), (1, s, cfg.ffn, h)]
     out = []
     for _ in range(cfg.layers):

@@ -313,8 +313,8 @@ int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, int64_t m, 
                                 int32_t groups, const int64_t *widths, void *const *outs,
                                 void *workspace, size_t workspace_bytes);
 /* out[m, n] = swiglu(A . B[:, gate_offset .. +n], A . B[:, up_offset .. +n]) (see rmlk_hip_swiglu)
- * in one launch, the activation applied to the accumulators. Covers m % 128 == 0, n % 64 == 0,
- * k % 32 == 0, 16-byte aligned rows and at least one tile per compute unit; RMLK_ERR_UNSUPPORTED
+ * in one launch, the activation applied to the accumulators. Covers n % 64 == 0, k % 32 == 0,
+ * 16-byte aligned rows and at least one 128 x 64 tile per compute unit; RMLK_ERR_UNSUPPORTED
  * otherwise (the caller then multiplies and activates separately). */
 int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n, int64_t k,
                                const void *a, int64_t lda, const void *b, int64_t ldb,

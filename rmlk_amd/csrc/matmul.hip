@@ -360,9 +360,9 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
     }
 }
 
-// ---- full-tile kernel with direct global -> LDS loads ---------------------------------------------
-// For problems made of whole tiles (no bounds checks, 16-byte aligned rows, BK = 32) the K-step
-// tiles do not pass through registers: each wavefront issues `global_load_lds_dwordx4`, which
+// ---- kernel with direct global -> LDS loads -------------------------------------------------------
+// For problems with whole K steps (BK = 32) and 16-byte aligned rows the K-step tiles do not pass
+// through registers: each wavefront issues `global_load_lds_dwordx4`, which
 // writes 64 lanes x 16 bytes as one contiguous 1 KiB piece of LDS while every lane picks its own
 // global address. Rows of 32 floats are therefore unpadded in LDS; bank conflicts on the
 // fragment reads of K-contiguous operands are avoided by a swizzle instead: the 16-byte unit q of
@@ -373,10 +373,15 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
 // SWIGLU: the block's B tile is half gate columns, half up columns of one joint weight matrix,
 // arranged so that a wavefront's first accumulator column holds gate values and its second the up
 // values of the SAME output columns; the epilogue writes silu(gate) * up, BN / 2 columns per tile.
-template <int BM, int BN, int WM, int WN, bool TB, int STAGES, bool SWIGLU = false>
+//
+// EDGE: m and n need not be whole tiles (K steps stay whole, rows 16-byte aligned). Rows and columns
+// past the end are fetched from the last valid row / 16-byte unit instead -- what they feed is
+// never stored -- so the main loop is the same; only the stores are guarded.
+template <int BM, int BN, int WM, int WN, bool TB, int STAGES, bool SWIGLU = false, bool EDGE = false>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) {
     static_assert(STAGES == 2, "two LDS stages");
-    static_assert(!SWIGLU || (!TB && WN == 64), "SwiGLU epilogue: row-major B, two accumulator columns");
+    static_assert(!SWIGLU || (!TB && WN == 64),
+                  "SwiGLU epilogue: row-major B, two accumulator columns (EDGE: partial tiles in m only)");
     constexpr int BK = 32;
     constexpr int KC = BK / 8;
     constexpr int kAFloats = BM * BK;   // one stage of A, floats
@@ -413,23 +418,29 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     const int l32 = lane % 32, half = lane / 32;
 
     // Global sources of a stage: piece (p * 4 + wave) goes to this wavefront. The address is a
-    // wave-uniform base (scalar registers, advanced with scalar adds) plus a per-lane byte offset
-    // that never changes, so the loads cost no vector ALU work.
+    // wave-uniform base (scalar registers, advanced by one K step with scalar adds) plus a per-lane
+    // byte offset per piece that never changes, so the loads cost no vector ALU work.
     const int sw_row = lane / 8, sw_unit = (lane % 8) ^ sw_row;
-    const uint32_t a_voff =
-        static_cast<uint32_t>(((wave * 8 + sw_row) * g.lda + sw_unit * 4) * static_cast<int64_t>(4));
+    uint32_t a_voff[A_PASSES], b_voff[B_PASSES];
     const float *a_ptr = A + static_cast<int64_t>(m0) * g.lda + k_begin;
-    const int64_t a_pass_stride = static_cast<int64_t>(32) * g.lda;
-    uint32_t b_voff;
+#pragma unroll
+    for (int p = 0; p < A_PASSES; ++p) {
+        int row = p * 32 + wave * 8 + sw_row;
+        if constexpr (EDGE) row = min(row, g.m - 1 - m0);
+        a_voff[p] = static_cast<uint32_t>((row * g.lda + sw_unit * 4) * static_cast<int64_t>(4));
+    }
     const float *b_ptr;
-    int64_t b_pass_stride, b_step_stride;
+    int64_t b_step_stride;
     if constexpr (TB) {
-        b_voff = static_cast<uint32_t>(((wave * 8 + sw_row) * g.ldb + sw_unit * 4) * static_cast<int64_t>(4));
         b_ptr = B + static_cast<int64_t>(n0) * g.ldb + k_begin;
-        b_pass_stride = static_cast<int64_t>(32) * g.ldb;
         b_step_stride = BK;
+#pragma unroll
+        for (int p = 0; p < B_PASSES; ++p) {
+            int row = p * 32 + wave * 8 + sw_row;
+            if constexpr (EDGE) row = min(row, g.n - 1 - n0);
+            b_voff[p] = static_cast<uint32_t>((row * g.ldb + sw_unit * 4) * static_cast<int64_t>(4));
+        }
     } else {
-        const int krow = wave * B_ROWS_PER_PIECE + lane / B_ROW_LANES;
         int col = (lane % B_ROW_LANES) * 4;    // LDS column of the tile this lane fills
         if constexpr (SWIGLU) {
             // LDS column c: wavefront column c / 64, accumulator (c % 64) / 32, lane c % 32
@@ -437,11 +448,15 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
             col = ((col % 64) / 32 ? g.up_offset : g.gate_offset) + out_col;
             b_ptr = B + static_cast<int64_t>(k_begin) * g.ldb;
         } else {
+            if constexpr (EDGE) col = min(col, g.n - 4 - n0);
             b_ptr = B + static_cast<int64_t>(k_begin) * g.ldb + n0;
         }
-        b_voff = static_cast<uint32_t>((krow * g.ldb + col) * static_cast<int64_t>(4));
-        b_pass_stride = static_cast<int64_t>(4 * B_ROWS_PER_PIECE) * g.ldb;
         b_step_stride = static_cast<int64_t>(BK) * g.ldb;
+#pragma unroll
+        for (int p = 0; p < B_PASSES; ++p) {
+            const int krow = (p * 4 + wave) * B_ROWS_PER_PIECE + lane / B_ROW_LANES;
+            b_voff[p] = static_cast<uint32_t>((krow * g.ldb + col) * static_cast<int64_t>(4));
+        }
     }
     // LDS byte addresses of this wavefront's first piece of A and B in stage 0 (wave-uniform)
     const uint32_t lds_a = __builtin_amdgcn_readfirstlane(
@@ -460,11 +475,10 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     // load number o of the stage that goes to LDS buffer `buf`
     auto load_op = [&](int buf, int o) {
         if (o < A_PASSES)
-            direct_load(lds_a + static_cast<uint32_t>(buf * kAFloats * 4 + o * 4096),
-                        a_ptr + o * a_pass_stride, a_voff);
+            direct_load(lds_a + static_cast<uint32_t>(buf * kAFloats * 4 + o * 4096), a_ptr, a_voff[o]);
         else
-            direct_load(lds_b + static_cast<uint32_t>(buf * kBFloats * 4 + (o - A_PASSES) * 4096),
-                        b_ptr + (o - A_PASSES) * b_pass_stride, b_voff);
+            direct_load(lds_b + static_cast<uint32_t>(buf * kBFloats * 4 + (o - A_PASSES) * 4096), b_ptr,
+                        b_voff[o - A_PASSES]);
     };
     auto advance_sources = [&]() {
         a_ptr += BK;
@@ -596,7 +610,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
                 const int row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
                 const float gate = acc[i][0][r];
                 const float silu = gate * (1.0f / (1.0f + expf(-gate)));
-                C[static_cast<int64_t>(row) * g.ldc + col] = silu * acc[i][1][r];
+                if (!EDGE || row < g.m) C[static_cast<int64_t>(row) * g.ldc + col] = silu * acc[i][1][r];
             }
         }
         return;
@@ -620,10 +634,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const int col = col0 + wn * WN + j * 32 + l32;
+            if (EDGE && n0 + wn * WN + j * 32 + l32 >= g.n) continue;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                C[static_cast<int64_t>(row) * ldc + col] = acc[i][j][r];
+                if (!EDGE || row < g.m) C[static_cast<int64_t>(row) * ldc + col] = acc[i][j][r];
             }
         }
     }
@@ -1084,10 +1099,10 @@ int32_t launch_mfma(hipStream_t s, const GemmArgs &g, int64_t batch, int splits)
     return launch_status();
 }
 
-template <int BM, int BN, int WM, int WN, bool TB, int STAGES, bool SWIGLU = false>
+template <int BM, int BN, int WM, int WN, bool TB, int STAGES, bool SWIGLU = false, bool EDGE = false>
 int32_t launch_direct(hipStream_t s, const GemmArgs &g, int64_t batch, int splits) {
     constexpr int kBytes = STAGES * (BM * 32 + 32 * BN) * 4;
-    auto kern = gemm_mfma_direct_kernel<BM, BN, WM, WN, TB, STAGES, SWIGLU>;
+    auto kern = gemm_mfma_direct_kernel<BM, BN, WM, WN, TB, STAGES, SWIGLU, EDGE>;
     if (kBytes > 64 * 1024) {
         static DynamicLdsGrant grant;   // one per instantiation, i.e. per kernel
         const int32_t st = grant.ensure(kern, kBytes);
@@ -1158,9 +1173,11 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
                  : launch_mfma<BM_, BN_, 16, WM_, WN_, true, TB_>(s, g, batch, t.splits)))
 #define RMLK_LAUNCH(BM_, BN_, WM_, WN_)                                                          \
     (trans_b ? RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, true) : RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, false))
+#define RMLK_DIRECT_E(BM_, BN_, WM_, WN_, S_, E_)                                                \
+    (trans_b ? launch_direct<BM_, BN_, WM_, WN_, true, S_, false, E_>(s, g, batch, t.splits)     \
+             : launch_direct<BM_, BN_, WM_, WN_, false, S_, false, E_>(s, g, batch, t.splits))
 #define RMLK_DIRECT_S(BM_, BN_, WM_, WN_, S_)                                                    \
-    (trans_b ? launch_direct<BM_, BN_, WM_, WN_, true, S_>(s, g, batch, t.splits)                \
-             : launch_direct<BM_, BN_, WM_, WN_, false, S_>(s, g, batch, t.splits))
+    (whole ? RMLK_DIRECT_E(BM_, BN_, WM_, WN_, S_, false) : RMLK_DIRECT_E(BM_, BN_, WM_, WN_, S_, true))
     // two LDS stages: a third (loads two K steps ahead) measured no faster and halves the blocks
     // that fit a CU
 #ifndef RMLK_GEMM_STAGES
@@ -1170,7 +1187,12 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
 #define RMLK_GEMM_DIRECT 1
 #endif
 #define RMLK_DIRECT(BM_, BN_, WM_, WN_) RMLK_DIRECT_S(BM_, BN_, WM_, WN_, RMLK_GEMM_STAGES)
-    const bool direct = RMLK_GEMM_DIRECT && full && t.bk == 32;
+    // the direct-to-LDS kernel: whole K steps and aligned rows; partial tiles in m and n are fine
+    // (for row-major B as long as n is a multiple of 4); per-lane byte offsets are 32-bit
+    const bool whole = m % t.bm == 0 && n % t.bn == 0;
+    const bool direct = RMLK_GEMM_DIRECT && t.bk == 32 && aligned && t.k_per_split % t.bk == 0 &&
+                        k % t.k_per_split == 0 && (trans_b || n % 4 == 0) && lda < (1ll << 21) &&
+                        ldb < (1ll << 21);
     if (seg) {
         // column blocks with their own destinations: whole tiles only, no tile across a boundary
         if (!direct || batch != 1) return RMLK_ERR_UNSUPPORTED;
@@ -1185,6 +1207,7 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
     else st = RMLK_LAUNCH(64, 64, 32, 32);
 #undef RMLK_DIRECT
 #undef RMLK_DIRECT_S
+#undef RMLK_DIRECT_E
 #undef RMLK_LAUNCH
 #undef RMLK_LAUNCH_TB
     if (st) return st;
@@ -1216,15 +1239,18 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
 }
 
 // silu(A . B[:, gate..]) * (A . B[:, up..]) in one launch: 128 x 128 tiles of 64 gate and 64 up
-// columns. Whole tiles, no split-K, enough tiles to cover the chip; otherwise UNSUPPORTED.
+// columns. Whole tiles in n and k, no split-K, enough tiles to cover the chip; otherwise UNSUPPORTED.
 int32_t gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float *pa, int64_t lda,
                     const float *pb, int64_t ldb, int64_t gate_offset, int64_t up_offset, float *pc,
                     int64_t ldc) {
     const bool aligned = lda % 4 == 0 && ldb % 4 == 0 && gate_offset % 4 == 0 && up_offset % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
                          reinterpret_cast<uintptr_t>(pb) % 16 == 0;
-    if (!aligned || m % 128 != 0 || n % 64 != 0 || k % 32 != 0 || k < 32) return RMLK_ERR_UNSUPPORTED;
-    const int64_t tiles = (m / 128) * (n / 64);
+    if (!aligned || n % 64 != 0 || k % 32 != 0 || k < 32 || lda >= (1ll << 21) || ldb >= (1ll << 21))
+        return RMLK_ERR_UNSUPPORTED;
+    if (m < 32) return RMLK_ERR_UNSUPPORTED;   // a 128-row tile would be nearly empty
+    const int64_t tiles_m = (m + 127) / 128;
+    const int64_t tiles = tiles_m * (n / 64);
     if (tiles < kNumCU || tiles >= (1ll << 31)) return RMLK_ERR_UNSUPPORTED;
     GemmArgs g{};
     g.a = pa;
@@ -1237,12 +1263,13 @@ int32_t gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float 
     g.ldb = ldb;
     g.ldc = ldc;
     g.k_per_split = g.k;
-    g.tiles_m = static_cast<int32_t>(m / 128);
+    g.tiles_m = static_cast<int32_t>(tiles_m);
     g.tiles_n = static_cast<int32_t>(n / 64);
     g.aligned = 1;
     g.gate_offset = static_cast<int32_t>(gate_offset);
     g.up_offset = static_cast<int32_t>(up_offset);
-    return launch_direct<128, 128, 64, 64, false, 2, true>(s, g, 1, 1);
+    if (m % 128 == 0) return launch_direct<128, 128, 64, 64, false, 2, true, false>(s, g, 1, 1);
+    return launch_direct<128, 128, 64, 64, false, 2, true, true>(s, g, 1, 1);
 }
 
 }  // namespace
@@ -1288,11 +1315,11 @@ extern "C" int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_
                  gemv_splits(batch, n, k, kWave * 4, &kps));
     } else {
         TileChoice t = choose_tiles(batch, m, n, k);
-        // dense row-major operands assumed (lda = k, ldb = n): whole tiles take the direct-to-LDS kernel
-        const bool whole = t.bk == 32 && m % t.bm == 0 && n % t.bn == 0 && k % 4 == 0 && n % 4 == 0 &&
-                           t.k_per_split % t.bk == 0 && k % t.k_per_split == 0;
+        // dense row-major operands assumed (lda = k, ldb = n): whole K steps take the direct-to-LDS kernel
+        const bool direct = t.bk == 32 && k % 4 == 0 && n % 4 == 0 && t.k_per_split % t.bk == 0 &&
+                            k % t.k_per_split == 0;
         snprintf(tmp, sizeof(tmp), "mfma%dx%dx%d%s splitk=%d", t.bm, t.bn, t.bk,
-                 whole ? " direct" : "", t.splits);
+                 direct ? " direct" : "", t.splits);
     }
     const int32_t len = static_cast<int32_t>(strlen(tmp));
     if (buf && size > 0) {

@@ -618,7 +618,8 @@ def test_grouped_matmul_argument_checks(device):
 
 
 @pytest.mark.parametrize("m,n,k,gate_first", [(512, 8192, 2048, True), (256, 8192, 64, False),
-                                              (2048, 1024, 512, True)])
+                                              (2048, 1024, 512, True), (500, 8192, 256, True),
+                                              (129, 8192, 128, False)])
 def test_matmul_swiglu_matches_separate_kernels(device, m, n, k, gate_first):
     import torch
     kk = _k()
@@ -641,7 +642,8 @@ def test_matmul_swiglu_matches_separate_kernels(device, m, n, k, gate_first):
     assert_close(to_np(got), exp.astype(np.float32), rtol=1e-4, atol=1e-5)
 
 
-@pytest.mark.parametrize("m,n,k", [(64, 8192, 256), (512, 8200, 256), (512, 128, 256), (512, 8192, 48)])
+@pytest.mark.parametrize("m,n,k", [(64, 8192, 256), (512, 8200, 256), (512, 128, 256), (512, 8192, 48),
+                                   (8, 32768, 256)])
 def test_matmul_swiglu_declines_what_it_does_not_cover(device, m, n, k):
     import torch
     from rmlk_amd import RmlkError

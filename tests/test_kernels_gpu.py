@@ -318,6 +318,9 @@ MATMUL_CASES = [
     (8, 4, 640, 64),          # skinny: scores of a KV group
     (1, 8, 2048, 2048),       # skinny with split-K
     (3, 5, 1024, 300), (2, 3, 132, 77), (1, 2, 8192, 2048), (2, 6, 4, 9),
+    # partial tiles in m and n with whole K steps: the direct-to-LDS kernel with guarded stores
+    (1, 500, 2048, 2048), (1, 130, 68, 256), (4, 100, 36, 512), (1, 129, 4100, 256),
+    (2, 257, 260, 288), (1, 9, 132, 1024),
 ]
 
 
