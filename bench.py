@@ -29,18 +29,18 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 CALIBRATION_COPY_BYTES = 256 << 20
 
-# HBM-side traffic of one gemm_mfma_kernel launch per MatMul shape (batch, m, n, k) of the default
-# workload, in KiB: (fetched, written). Read with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
-# (one run each) over `python3 bench.py --no-cpu --steps 1 --warmup 0 --decode 2`, scaled by what the
-# same counters read for the 256 MiB calibration copy below (FETCH_SIZE 131092 -> x2.0,
-# WRITE_SIZE 262144 -> x1.0). Split-K launches write partial sums to the workspace; the combine
-# kernel's own traffic is not included.
+# HBM-side traffic of one GEMM launch per shape (batch, m, n, k[, epilogue]) of the default workload,
+# in KiB: (fetched, written). Read with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (one run
+# each) over `python3 bench.py --no-cpu --steps 1 --warmup 0 --decode 4`, scaled by what the same
+# counters read for the 256 MiB calibration copy below (FETCH_SIZE 131092 -> x2.0, WRITE_SIZE
+# 262144 -> x1.0). Split-K launches write partial sums to the workspace; what their consumer (the
+# combine kernel or the norm kernel) moves is not included.
 PMC_TRAFFIC_KIB = {
-    (1, 512, 2048, 2048): (49257, 16384),
-    (1, 512, 512, 2048): (24634, 4096),
-    (1, 512, 8192, 2048): (98403, 16384),
-    (1, 512, 2048, 8192): (196706, 16384),
-    (1, 512, 128256, 2048): (2109895, 256512),
+    (1, 512, 3072, 2048): (32924, 24576),                 # q/k/v, split-K 4
+    (1, 512, 2048, 2048): (24719, 16384),                 # o, split-K 4
+    (1, 512, 2048, 8192): (98447, 16384),                 # down, split-K 4
+    (1, 512, 16384, 2048, "swiglu"): (164040, 16384),     # gate/up with the SwiGLU epilogue
+    (1, 512, 128256, 2048): (1492721, 256512),            # lm-head
 }
 
 

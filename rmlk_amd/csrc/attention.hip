@@ -34,6 +34,14 @@ constexpr int kTile = kChunk * kHeadDim;          // floats of one staged K or V
 constexpr int kAttnLdsBytes = 2 * 2 * kTile * 4;  // K and V, two buffers each
 constexpr float kLog2e = 1.4426950408889634f;
 
+// max / sum of a value over the two lanes (l, l + 32) that share a query, on all 64 lanes: one
+// v_permlane32_swap turns x into (lower half twice, upper half twice).
+__device__ __forceinline__ void half_pair(float x, float &lo, float &hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    lo = __uint_as_float(r[0]);
+    hi = __uint_as_float(r[1]);
+}
+
 struct AttnArgs {
     const float *q;
     const float *k;
@@ -159,9 +167,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
         }
 
         // S^T (32 keys x 32 queries) = K . Q^T over the 64 head dims
-        v16f st;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) st[r] = 0.f;
+        v16f st = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         const float *ks = Ks + buf * kTile + k_frag;
 #pragma unroll
         for (int kc = 0; kc < 8; ++kc) {
@@ -187,7 +193,11 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
         float mx = t[0];
 #pragma unroll
         for (int r = 1; r < 16; ++r) mx = fmaxf(mx, t[r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        {
+            float lo, hi;
+            half_pair(mx, lo, hi);
+            mx = fmaxf(lo, hi);
+        }
         const float m_new = fmaxf(m_run, mx);
         const float m_safe = m_new == kNegInf ? 0.f : m_new;   // a row with nothing visible so far
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
@@ -198,12 +208,16 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
             psum += p[r];
         }
         l_run = l_run * alpha + psum;
-        m_run = m_new;
+        // the output so far is rescaled only when some query of this wavefront met a new maximum
+        // (alpha is exactly 1 otherwise)
+        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            o0[r] *= alpha;
-            o1[r] *= alpha;
+            for (int r = 0; r < 16; ++r) {
+                o0[r] *= alpha;
+                o1[r] *= alpha;
+            }
         }
+        m_run = m_new;
 
         // O^T (64 dims x 32 queries) += V^T . P^T over this wavefront's 32 keys
         const float *vs = Vs + buf * kTile;
@@ -227,7 +241,11 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
     }
 
     // ---- merge the two key halves of every query tile and write ----------------------------------
-    l_run += __shfl_xor(l_run, 32);
+    {
+        float lo, hi;
+        half_pair(l_run, lo, hi);
+        l_run = lo + hi;
+    }
     float *cb = smem + wq * (34 * kWave);   // the staging buffers are free after the last barrier
     if (wk == 1) {
         cb[lane] = m_run;

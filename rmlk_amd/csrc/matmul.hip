@@ -52,7 +52,7 @@ struct GemmArgs {
     int32_t aligned;                       // rows of A and B start on 16-byte boundaries
     // Column blocks of C with a destination each (grouped products): block i covers columns
     // [seg_begin[i], seg_begin[i + 1]) and is written to seg_c[i] with leading dimension seg_ldc[i].
-    // n_seg == 0: plain C. Block boundaries are multiples of the tile width.
+    // n_seg == 0: plain C. Block boundaries are multiples of 32 (one MFMA result block).
     int32_t n_seg;
     int32_t seg_begin[kMaxSegments + 1];
     float *seg_c[kMaxSegments];
@@ -395,9 +395,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     static_assert((BM / WM) * (BN / WN) == kThreads / kWave, "four wavefronts per block");
     constexpr int A_PASSES = BM / 32;   // 1 KiB pieces (8 rows of A) per wavefront and stage
     constexpr int B_PASSES = BN / 32;
-    constexpr int B_ROW_LANES = BN / 4;             // lanes per K-row of a row-major B tile
-    constexpr int B_ROWS_PER_PIECE = kWave / B_ROW_LANES > 0 ? kWave / B_ROW_LANES : 1;
-    static_assert(TB || B_ROW_LANES <= kWave, "a K-row of B must fit one 1 KiB piece");
+    constexpr int B_ROW_UNITS = BN / 4;             // 16-byte units per K-row of a row-major B tile
 
     int tile_m, tile_n, split;
     tile_coords(g, tile_m, tile_n, split);
@@ -441,20 +439,21 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
             b_voff[p] = static_cast<uint32_t>((row * g.ldb + sw_unit * 4) * static_cast<int64_t>(4));
         }
     } else {
-        int col = (lane % B_ROW_LANES) * 4;    // LDS column of the tile this lane fills
-        if constexpr (SWIGLU) {
-            // LDS column c: wavefront column c / 64, accumulator (c % 64) / 32, lane c % 32
-            const int out_col = tile_n * (BN / 2) + (col / 64) * 32 + col % 32;
-            col = ((col % 64) / 32 ? g.up_offset : g.gate_offset) + out_col;
-            b_ptr = B + static_cast<int64_t>(k_begin) * g.ldb;
-        } else {
-            if constexpr (EDGE) col = min(col, g.n - 4 - n0);
-            b_ptr = B + static_cast<int64_t>(k_begin) * g.ldb + n0;
-        }
+        b_ptr = B + static_cast<int64_t>(k_begin) * g.ldb + (SWIGLU ? 0 : n0);
         b_step_stride = static_cast<int64_t>(BK) * g.ldb;
 #pragma unroll
         for (int p = 0; p < B_PASSES; ++p) {
-            const int krow = (p * 4 + wave) * B_ROWS_PER_PIECE + lane / B_ROW_LANES;
+            // the tile is [BK][BN] in LDS, filled in 1 KiB pieces of 64 consecutive 16-byte units
+            const int unit = (p * 4 + wave) * kWave + lane;
+            const int krow = unit / B_ROW_UNITS;
+            int col = (unit % B_ROW_UNITS) * 4;    // LDS column of the tile this lane fills
+            if constexpr (SWIGLU) {
+                // LDS column c: wavefront column c / 64, accumulator (c % 64) / 32, lane c % 32
+                const int out_col = tile_n * (BN / 2) + (col / 64) * 32 + col % 32;
+                col = ((col % 64) / 32 ? g.up_offset : g.gate_offset) + out_col;
+            } else if constexpr (EDGE) {
+                col = min(col, g.n - 4 - n0);
+            }
             b_voff[p] = static_cast<uint32_t>((krow * g.ldb + col) * static_cast<int64_t>(4));
         }
     }
@@ -615,30 +614,33 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
         }
         return;
     }
-    int64_t ldc = g.ldc;
-    int col0 = n0;
-    if (g.n_seg > 0 && gridDim.z == 1) {
-        // constant indices only: the argument struct stays in scalar registers
-        C = g.seg_c[0];
-        ldc = g.seg_ldc[0];
+    const bool segmented = g.n_seg > 0 && gridDim.z == 1;
 #pragma unroll
-        for (int i = 1; i < kMaxSegments; ++i)
-            if (i < g.n_seg && n0 >= g.seg_begin[i]) {
-                C = g.seg_c[i];
-                ldc = g.seg_ldc[i];
-                col0 = n0 - g.seg_begin[i];
-            }
-    }
+    for (int j = 0; j < TN; ++j) {
+        // destination of this 32-column block (block boundaries are multiples of 32)
+        const int cb = n0 + wn * WN + j * 32;
+        float *dst = C;
+        int64_t ldc = g.ldc;
+        int col = cb + l32;
+        if (segmented) {
+            // constant indices only: the argument struct stays in scalar registers
+            dst = g.seg_c[0];
+            ldc = g.seg_ldc[0];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+            for (int sgm = 1; sgm < kMaxSegments; ++sgm)
+                if (sgm < g.n_seg && cb >= g.seg_begin[sgm]) {
+                    dst = g.seg_c[sgm];
+                    ldc = g.seg_ldc[sgm];
+                    col = cb - g.seg_begin[sgm] + l32;
+                }
+        }
+        if (EDGE && cb + l32 >= g.n) continue;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int col = col0 + wn * WN + j * 32 + l32;
-            if (EDGE && n0 + wn * WN + j * 32 + l32 >= g.n) continue;
+        for (int i = 0; i < TM; ++i) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                if (!EDGE || row < g.m) C[static_cast<int64_t>(row) * ldc + col] = acc[i][j][r];
+                if (!EDGE || row < g.m) dst[static_cast<int64_t>(row) * ldc + col] = acc[i][j][r];
             }
         }
     }
@@ -1019,7 +1021,9 @@ struct TileChoice {
 #define RMLK_GEMM_SPLIT_TARGET 1
 #endif
 
-inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k) {
+// allow_wide: the 128 x 192 tile may be chosen (it exists for the direct-to-LDS kernel only; a caller
+// whose operands do not qualify asks again without it).
+inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k, bool allow_wide = true) {
     TileChoice t;
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch; };
     // A 64 x 64 wavefront tile (four MFMA accumulators) keeps the matrix pipe busiest, so the
@@ -1040,27 +1044,53 @@ inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k) {
         t.bn = 64;
     }
     t.bk = k >= 256 ? 32 : 16;
-    int64_t nt = tiles(t.bm, t.bn);
-    int splits = 1;
-    if (nt < kNumCU) {
-        splits = static_cast<int>((RMLK_GEMM_SPLIT_TARGET * kNumCU + nt - 1) / nt);
-        int64_t max_splits = k / (8 * t.bk);
-        if (max_splits < 1) max_splits = 1;
-        if (splits > max_splits) splits = static_cast<int>(max_splits);
-        if (splits > 32) splits = 32;
-        // a split count that cuts K into equal whole K steps keeps the kernel without bounds checks
-        for (int more = splits; more <= 2 * splits && more <= max_splits; ++more)
-            if (k % (static_cast<int64_t>(more) * t.bk) == 0) {
-                splits = more;
-                break;
-            }
+    auto split_for = [&](int bm, int bn, int *k_per_split) {
+        const int64_t nt = tiles(bm, bn);
+        int splits = 1;
+        if (nt < kNumCU) {
+            splits = static_cast<int>((RMLK_GEMM_SPLIT_TARGET * kNumCU + nt - 1) / nt);
+            int64_t max_splits = k / (8 * t.bk);
+            if (max_splits < 1) max_splits = 1;
+            if (splits > max_splits) splits = static_cast<int>(max_splits);
+            if (splits > 32) splits = 32;
+            // a split count that cuts K into equal whole K steps keeps the kernel without bounds checks
+            for (int more = splits; more <= 2 * splits && more <= max_splits; ++more)
+                if (k % (static_cast<int64_t>(more) * t.bk) == 0) {
+                    splits = more;
+                    break;
+                }
+        }
+        int64_t kps = (k + splits - 1) / splits;
+        kps = (kps + t.bk - 1) / t.bk * t.bk;
+        *k_per_split = static_cast<int>(kps);
+        splits = static_cast<int>((k + kps - 1) / kps);
+        return splits < 1 ? 1 : splits;
+    };
+    t.splits = split_for(t.bm, t.bn, &t.k_per_split);
+    // Widths that are 3 * 2^j (the joint q/k/v width of grouped-query attention) often leave the
+    // 128 x 128 tiling with a block count that covers the chip one and a half times; 128 x 192 tiles
+    // may cover it in whole rounds. Compare rounds x K steps x tile area (MFMA time) and take the
+    // wider tile only when it is clearly ahead.
+    if (allow_wide && t.bm == 128 && t.bn == 128 && t.bk == 32 && batch == 1 && n % 192 == 0) {
+        int kps_w;
+        const int splits_w = split_for(128, 192, &kps_w);
+        auto rounds = [&](int64_t blocks) { return (blocks + kNumCU - 1) / kNumCU; };
+        const int64_t cost = rounds(tiles(128, 128) * t.splits) * t.k_per_split * 2;
+        const int64_t cost_w = rounds(tiles(128, 192) * splits_w) * kps_w * 3;
+        if (cost_w * 10 <= cost * 9) {
+            t.bn = 192;
+            t.splits = splits_w;
+            t.k_per_split = kps_w;
+        }
     }
-    int64_t kps = (k + splits - 1) / splits;
-    kps = (kps + t.bk - 1) / t.bk * t.bk;
-    t.k_per_split = static_cast<int>(kps);
-    t.splits = static_cast<int>((k + kps - 1) / kps);
-    if (t.splits < 1) t.splits = 1;
     return t;
+}
+
+// the larger split-K factor of the two tilings a product may end up with
+inline int max_tile_splits(int64_t batch, int64_t m, int64_t n, int64_t k) {
+    const int wide = choose_tiles(batch, m, n, k, true).splits;
+    const int narrow = choose_tiles(batch, m, n, k, false).splits;
+    return wide > narrow ? wide : narrow;
 }
 
 inline int gemv_splits(int64_t batch, int64_t n, int64_t k, int cols_per_block, int *k_per_split) {
@@ -1114,6 +1144,10 @@ int32_t launch_direct(hipStream_t s, const GemmArgs &g, int64_t batch, int split
     return launch_status();
 }
 
+#ifndef RMLK_GEMM_DIRECT
+#define RMLK_GEMM_DIRECT 1
+#endif
+
 // The tiled MFMA path of a product (m > 1, A not transposed). `seg`: column blocks of C with their
 // own destinations (see Segments; their rows must be 16-byte aligned) instead of c/ldc; the call
 // then answers RMLK_ERR_UNSUPPORTED unless the whole-tile kernel applies.
@@ -1121,7 +1155,17 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
                    int64_t lda, int64_t stride_a, const float *pb, int64_t ldb, int64_t stride_b,
                    int32_t trans_b, float *pc, int64_t ldc, int64_t stride_c, void *workspace,
                    size_t workspace_bytes, const Segments *seg, int32_t *partial_splits = nullptr) {
+    const bool aligned = lda % 4 == 0 && ldb % 4 == 0 && stride_a % 4 == 0 && stride_b % 4 == 0 &&
+                         reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(pb) % 16 == 0;
+    // the direct-to-LDS kernel: whole K steps and aligned rows; partial tiles in m and n are fine
+    // (for row-major B as long as n is a multiple of 4); per-lane byte offsets are 32-bit
+    auto direct_ok = [&](const TileChoice &c) {
+        return RMLK_GEMM_DIRECT && c.bk == 32 && aligned && c.k_per_split % c.bk == 0 &&
+               k % c.k_per_split == 0 && (trans_b || n % 4 == 0) && lda < (1ll << 21) && ldb < (1ll << 21);
+    };
     TileChoice t = choose_tiles(batch, m, n, k);
+    if (t.bn == 192 && !direct_ok(t)) t = choose_tiles(batch, m, n, k, false);
     GemmArgs g{};
     g.a = pa;
     g.b = pb;
@@ -1158,9 +1202,6 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
             g.seg_begin[seg->n_seg] = seg->begin[seg->n_seg];
         }
     }
-    const bool aligned = lda % 4 == 0 && ldb % 4 == 0 && stride_a % 4 == 0 && stride_b % 4 == 0 &&
-                         reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
-                         reinterpret_cast<uintptr_t>(pb) % 16 == 0;
     g.aligned = aligned ? 1 : 0;
     const bool full = aligned && m % t.bm == 0 && n % t.bn == 0 && t.k_per_split % t.bk == 0 &&
                       k % t.k_per_split == 0;
@@ -1183,23 +1224,17 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
 #ifndef RMLK_GEMM_STAGES
 #define RMLK_GEMM_STAGES 2
 #endif
-#ifndef RMLK_GEMM_DIRECT
-#define RMLK_GEMM_DIRECT 1
-#endif
 #define RMLK_DIRECT(BM_, BN_, WM_, WN_) RMLK_DIRECT_S(BM_, BN_, WM_, WN_, RMLK_GEMM_STAGES)
-    // the direct-to-LDS kernel: whole K steps and aligned rows; partial tiles in m and n are fine
-    // (for row-major B as long as n is a multiple of 4); per-lane byte offsets are 32-bit
     const bool whole = m % t.bm == 0 && n % t.bn == 0;
-    const bool direct = RMLK_GEMM_DIRECT && t.bk == 32 && aligned && t.k_per_split % t.bk == 0 &&
-                        k % t.k_per_split == 0 && (trans_b || n % 4 == 0) && lda < (1ll << 21) &&
-                        ldb < (1ll << 21);
+    const bool direct = direct_ok(t);
     if (seg) {
         // column blocks with their own destinations: whole tiles only, no tile across a boundary
         if (!direct || batch != 1) return RMLK_ERR_UNSUPPORTED;
         for (int i = 0; i <= seg->n_seg; ++i)
-            if (seg->begin[i] % t.bn != 0) return RMLK_ERR_UNSUPPORTED;
+            if (seg->begin[i] % 32 != 0) return RMLK_ERR_UNSUPPORTED;
     }
     if (direct && t.bm == 256) st = RMLK_DIRECT(256, 64, 64, 64);
+    else if (direct && t.bn == 192) st = RMLK_DIRECT(128, 192, 64, 96);
     else if (direct && t.bm == 128) st = RMLK_DIRECT(128, 128, 64, 64);
     else if (direct) st = RMLK_DIRECT(64, 64, 32, 32);
     else if (t.bm == 256) st = RMLK_LAUNCH(256, 64, 64, 64);
@@ -1288,8 +1323,8 @@ extern "C" size_t rmlk_hip_matmul_workspace_size(int32_t dtype, int64_t batch, i
         int sp = s4 > s1 ? s4 : s1;
         return sp > 1 ? static_cast<size_t>(sp) * batch * n * sizeof(float) : 0;
     }
-    TileChoice t = choose_tiles(batch, m, n, k);
-    size_t need = t.splits > 1 ? static_cast<size_t>(t.splits) * batch * m * n * sizeof(float) : 0;
+    const int tile_splits = max_tile_splits(batch, m, n, k);
+    size_t need = tile_splits > 1 ? static_cast<size_t>(tile_splits) * batch * m * n * sizeof(float) : 0;
     if (m <= kSkinnyRows) {
         int kps;
         const int sp = gemv_splits(batch, n, k, kWave * 4, &kps);
@@ -1316,8 +1351,12 @@ extern "C" int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_
     } else {
         TileChoice t = choose_tiles(batch, m, n, k);
         // dense row-major operands assumed (lda = k, ldb = n): whole K steps take the direct-to-LDS kernel
-        const bool direct = t.bk == 32 && k % 4 == 0 && n % 4 == 0 && t.k_per_split % t.bk == 0 &&
-                            k % t.k_per_split == 0;
+        auto direct_ok = [&](const TileChoice &c) {
+            return c.bk == 32 && k % 4 == 0 && n % 4 == 0 && c.k_per_split % c.bk == 0 &&
+                   k % c.k_per_split == 0;
+        };
+        if (t.bn == 192 && !direct_ok(t)) t = choose_tiles(batch, m, n, k, false);
+        const bool direct = direct_ok(t);
         snprintf(tmp, sizeof(tmp), "mfma%dx%dx%d%s splitk=%d", t.bm, t.bn, t.bk,
                  direct ? " direct" : "", t.splits);
     }
@@ -1601,8 +1640,7 @@ extern "C" int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, i
 
 extern "C" size_t rmlk_hip_matmul_partials_workspace_size(int32_t dtype, int64_t m, int64_t n, int64_t k) {
     if (dtype != RMLK_FLOAT || m <= kSkinnyRows || n <= 0 || k <= 0) return 0;
-    const TileChoice t = choose_tiles(1, m, n, k);
-    return static_cast<size_t>(t.splits) * m * n * sizeof(float);
+    return static_cast<size_t>(max_tile_splits(1, m, n, k)) * m * n * sizeof(float);
 }
 
 extern "C" int32_t rmlk_hip_matmul_partials(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n,

@@ -321,6 +321,9 @@ MATMUL_CASES = [
     # partial tiles in m and n with whole K steps: the direct-to-LDS kernel with guarded stores
     (1, 500, 2048, 2048), (1, 130, 68, 256), (4, 100, 36, 512), (1, 129, 4100, 256),
     (2, 257, 260, 288), (1, 9, 132, 1024),
+    # widths of 3 * 2^j: 128 x 192 tiles (split-K, whole rounds, ragged rows, and the fallback when
+    # K has no whole steps)
+    (1, 512, 3072, 2048), (1, 2048, 3072, 256), (1, 500, 1536, 512), (1, 512, 3072, 2000),
 ]
 
 
