@@ -36,11 +36,11 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # 262144 -> x1.0). Split-K launches write partial sums to the workspace; what their consumer (the
 # combine kernel or the norm kernel) moves is not included.
 PMC_TRAFFIC_KIB = {
-    (1, 512, 3072, 2048): (32924, 24576),                 # q/k/v, split-K 4
+    (1, 512, 3072, 2048): (32997, 24576),                 # q/k/v (128 x 192 tiles), split-K 4
     (1, 512, 2048, 2048): (24719, 16384),                 # o, split-K 4
-    (1, 512, 2048, 8192): (98447, 16384),                 # down, split-K 4
-    (1, 512, 16384, 2048, "swiglu"): (164040, 16384),     # gate/up with the SwiGLU epilogue
-    (1, 512, 128256, 2048): (1492721, 256512),            # lm-head
+    (1, 512, 2048, 8192): (98476, 16384),                 # down, split-K 4
+    (1, 512, 16384, 2048, "swiglu"): (164057, 16384),     # gate/up with the SwiGLU epilogue
+    (1, 512, 128256, 2048): (1534894, 256512),            # lm-head
 }
 
 
