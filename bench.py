@@ -48,13 +48,12 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def cpu_baseline(graph, cfg, graphs, n_tokens, max_len, seed):
+def cpu_baseline(graph, cfg, graphs, prompt, n_tokens, max_len):
     """The numpy oracle (fp32 BLAS matmuls) on the host: prefill of the first n_tokens of the same
     prompt through the same graph."""
     import numpy as np
     from oracle import graph as og
-    rng = np.random.default_rng(seed)
-    prompt = rng.integers(0, cfg.vocab, size=512)[:n_tokens]
+    prompt = prompt[:n_tokens]
     feeds = {"input_ids": prompt.reshape(1, -1).astype(np.int64),
              "position_ids": np.arange(n_tokens, dtype=np.int64).reshape(1, -1)}
     for l in range(cfg.layers):
@@ -236,12 +235,25 @@ def run_llama(args):
     if not args.no_cpu:
         n_cpu = min(args.cpu_tokens, prompt_len)
         cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-        cpu_tok_s, cpu_s, cpu_logits = cpu_baseline(graph, cfg, graphs, n_cpu, max_len, 4)
+        cpu_tok_s, cpu_s, cpu_logits = cpu_baseline(graph, cfg, graphs, prompt, n_cpu, max_len)
+        # the same sample through the GPU session (eager), as a check of the measured path
+        inst.set_input("input_ids", prompt[:n_cpu].reshape(1, -1).astype(np.int64))
+        inst.set_input("position_ids", np.arange(n_cpu, dtype=np.int64).reshape(1, -1))
+        for name, arr in caches.items():
+            inst.set_input(name, arr)
+        inst.execute()
+        gpu_logits = inst.output("logits")[0, -1]
+        diff = float(np.max(np.abs(gpu_logits - cpu_logits)))
+        same_top1 = int(np.argmax(gpu_logits)) == int(np.argmax(cpu_logits))
+        assert diff <= 1e-2 and same_top1, f"GPU and oracle disagree on the sample: {diff}, top-1 {same_top1}"
         cpu = {"value": round(cpu_tok_s, 2), "unit": "tok/s", "cores": cores,
                "kind": "port",
                "sample": f"prefill of the first {n_cpu} prompt tokens through the same graph with the "
-                         f"numpy oracle (fp32 BLAS matmuls), {cpu_s:.1f} s; ONNX Runtime is not installed"}
-        log(f"[bench] cpu oracle: {cpu_tok_s:.1f} tok/s over {n_cpu} tokens ({cpu_s:.1f}s)")
+                         f"numpy oracle (fp32 BLAS matmuls), {cpu_s:.1f} s; ONNX Runtime is not installed",
+               "gpu_vs_oracle_on_sample": {"max_abs_logit_diff": round(diff, 6), "top1_equal": same_top1,
+                                           "bar": "1e-2 on logits, identical top-1"}}
+        log(f"[bench] cpu oracle: {cpu_tok_s:.1f} tok/s over {n_cpu} tokens ({cpu_s:.1f}s); "
+            f"GPU logits of the sample within {diff:.2e}, top-1 equal: {same_top1}")
 
     result = {
         "metric": "llama3.2-1b-shape fp32 prefill tok/s (decode ms/tok alongside)",
