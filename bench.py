@@ -470,7 +470,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--decode", type=int, default=128)
-    ap.add_argument("--cpu-tokens", type=int, default=64)
+    ap.add_argument("--cpu-tokens", type=int, default=512)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--tiny", action="store_true", help="2-layer toy shape (plumbing check only)")
     ap.add_argument("--suite", default="llama", choices=["llama", "ops"])
