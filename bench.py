@@ -469,8 +469,8 @@ def run_ops_suite(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--decode", type=int, default=128)
     ap.add_argument("--cpu-tokens", type=int, default=512)
