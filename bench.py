@@ -132,7 +132,7 @@ def run_llama(args):
     # classify each MatMul node by the kernel the library picks for its shape
     launches = matmul_launches(cfg, prompt_len, max_len)
     mm_nodes = [s for s in stats if s["op"] in ("MatMul", "rmlk.MatMulGroup", "rmlk.MatMulGroupSwiGLU",
-                                                "rmlk.MatMulAddRMSNorm")]
+                                                "rmlk.MatMulAddRMSNorm", "rmlk.MatMulConst")]
     assert len(mm_nodes) == len(launches), (len(mm_nodes), len(launches))
     by_kind, per_op = {}, {}
     for s, shapes in zip(mm_nodes, launches):

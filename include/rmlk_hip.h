@@ -320,6 +320,20 @@ int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t m, i
                                const void *a, int64_t lda, const void *b, int64_t ldb,
                                int64_t gate_offset, int64_t up_offset, void *out, int64_t ldc);
 
+/* One-row product with K-CONTIGUOUS weights: y[n] = sum_k x[k] * wt[n][k] (wt row-major [n, k],
+ * leading dimension ldw), i.e. rmlk_hip_matmul with m = 1 and trans_b. Every output column is
+ * finished inside one wavefront: no workspace and no combine launch, at any width. k % 4 == 0,
+ * 16-byte aligned operands; RMLK_ERR_UNSUPPORTED otherwise. The decode step of a session keeps a
+ * K-contiguous copy of constant weight matrices for it (ref: cublasGemmStridedBatchedEx with
+ * CUBLAS_OP_T on a transposed operand, cuda/src/kernels/gemm.rs:191-232). */
+int32_t rmlk_hip_gemv_kmajor(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k, const void *x,
+                        const void *wt, int64_t ldw, void *y);
+/* y[i] = swiglu(x . wt[gate_row + i, :], x . wt[up_row + i, :]) for i < n (see rmlk_hip_swiglu): the
+ * gate and the up projection of a one-row input and the activation in one launch. */
+int32_t rmlk_hip_gemv_kmajor_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
+                               const void *x, const void *wt, int64_t ldw, int64_t gate_row,
+                               int64_t up_row, void *y);
+
 /* ---- many-row products whose split-K combine is left to the consumer ----------------------------
  * rmlk_hip_matmul_partials: the tiled kernels of rmlk_hip_matmul for A[m, k] . B[k, n] (row-major,
  * m > 8) without the combine: `workspace` receives *splits_out partial matrices [m, n] one after

@@ -987,6 +987,63 @@ __global__ __launch_bounds__(kThreads) void gemv_dot_kernel(GemvArgs g) {
     }
 }
 
+// One-row product with K-contiguous weights, y[n] = sum_k x[k] * Wt[n][k]: a wavefront owns COLS
+// output columns and walks K in 128-bit units, eight units per lane and column in flight; the lanes'
+// partial sums meet in a shuffle tree. A column is finished inside its wavefront, so there is no
+// split-K, no workspace and no combine launch whatever the width.
+// SWIGLU: COLS is 2 and the wavefront's two rows of Wt are the gate and the up row of ONE output
+// (rows gate_row + i and up_row + i); it writes silu(gate) * up.
+template <int COLS, bool SWIGLU = false>
+__global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__restrict__ x,
+                                                          const float *__restrict__ wt,
+                                                          float *__restrict__ y, int32_t n, int32_t k,
+                                                          int64_t ldw, int32_t gate_row, int32_t up_row) {
+    static_assert(!SWIGLU || COLS == 2, "gate and up");
+    constexpr int kDepth = 8;
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int col0 = (blockIdx.x * (kThreads / kWave) + wave) * (SWIGLU ? 1 : COLS);
+    if (col0 >= n) return;
+    const int k4 = k / 4;
+    const v4f *xv = reinterpret_cast<const v4f *>(x);
+    const v4f *wv[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+        const int64_t row = SWIGLU ? (c == 0 ? gate_row : up_row) + col0 : min(col0 + c, n - 1);
+        wv[c] = reinterpret_cast<const v4f *>(wt + row * ldw);
+    }
+    float acc[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) acc[c] = 0.f;
+    for (int u0 = lane; u0 < k4; u0 += kWave * kDepth) {
+        v4f xr[kDepth], wr[kDepth][COLS];
+#pragma unroll
+        for (int j = 0; j < kDepth; ++j) {
+            const int u = u0 + j * kWave;
+            const bool live = u < k4;
+            xr[j] = live ? xv[u] : v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < COLS; ++c)
+                wr[j][c] = live ? __builtin_nontemporal_load(wv[c] + u) : v4f{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < kDepth; ++j)
+#pragma unroll
+            for (int c = 0; c < COLS; ++c)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[c] = fmaf(xr[j][e], wr[j][c][e], acc[c]);
+    }
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+#pragma unroll
+        for (int o = kWave / 2; o > 0; o >>= 1) acc[c] += __shfl_xor(acc[c], o, kWave);
+        if (!SWIGLU && lane == 0 && col0 + c < n) y[col0 + c] = acc[c];
+    }
+    if (SWIGLU && lane == 0) {
+        const float silu = acc[0] * (1.0f / (1.0f + expf(-acc[0])));
+        y[col0] = silu * acc[COLS - 1];
+    }
+}
+
 // Any-layout fallback (transposed operands with M > 1): one lane per C element.
 __global__ __launch_bounds__(kThreads) void gemm_naive_kernel(const float *__restrict__ a,
                                                               const float *__restrict__ b,
@@ -1657,4 +1714,54 @@ extern "C" int32_t rmlk_hip_matmul_partials(rmlk_stream_t stream, int32_t dtype,
     return gemm_tiled(as_stream(stream), 1, m, n, k, static_cast<const float *>(a), lda, 0,
                       static_cast<const float *>(b), ldb, 0, 0, nullptr, n, 0, workspace,
                       workspace_bytes, nullptr, splits_out);
+}
+
+extern "C" int32_t rmlk_hip_gemv_kmajor(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
+                                   const void *x, const void *wt, int64_t ldw, void *y) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (n < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n >= (1ll << 31) || k >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
+    if (n == 0) return RMLK_OK;
+    if (!y || (k > 0 && (!x || !wt))) return RMLK_ERR_NULL_POINTER;
+    if (ldw < k) return RMLK_ERR_SIZE_MISMATCH;
+    if (k % 4 != 0 || ldw % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(wt) % 16 != 0)
+        return RMLK_ERR_UNSUPPORTED;
+    const float *px = static_cast<const float *>(x), *pw = static_cast<const float *>(wt);
+    float *py = static_cast<float *>(y);
+    hipStream_t s = as_stream(stream);
+    constexpr int kWaves = kThreads / kWave;
+    // few columns: one per wavefront keeps every compute unit busy; many: four share the loads of x
+    if (n >= 16 * kNumCU * kWaves) {
+        const unsigned grid = static_cast<unsigned>((n + kWaves * 4 - 1) / (kWaves * 4));
+        gemv_kmajor_kernel<4><<<grid, kThreads, 0, s>>>(px, pw, py, static_cast<int32_t>(n), static_cast<int32_t>(k), ldw,
+                                                   0, 0);
+    } else {
+        const unsigned grid = static_cast<unsigned>((n + kWaves - 1) / kWaves);
+        gemv_kmajor_kernel<1><<<grid, kThreads, 0, s>>>(px, pw, py, static_cast<int32_t>(n), static_cast<int32_t>(k), ldw,
+                                                   0, 0);
+    }
+    return launch_status();
+}
+
+extern "C" int32_t rmlk_hip_gemv_kmajor_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
+                                          const void *x, const void *wt, int64_t ldw, int64_t gate_row,
+                                          int64_t up_row, void *y) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (n < 0 || k < 0 || gate_row < 0 || up_row < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n >= (1ll << 30) || k >= (1ll << 31) || gate_row >= (1ll << 30) || up_row >= (1ll << 30))
+        return RMLK_ERR_TOO_LARGE;
+    if (n == 0) return RMLK_OK;
+    if (!y || (k > 0 && (!x || !wt))) return RMLK_ERR_NULL_POINTER;
+    if (ldw < k) return RMLK_ERR_SIZE_MISMATCH;
+    if (k % 4 != 0 || ldw % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(wt) % 16 != 0)
+        return RMLK_ERR_UNSUPPORTED;
+    constexpr int kWaves = kThreads / kWave;
+    const unsigned grid = static_cast<unsigned>((n + kWaves - 1) / kWaves);
+    gemv_kmajor_kernel<2, true><<<grid, kThreads, 0, as_stream(stream)>>>(
+        static_cast<const float *>(x), static_cast<const float *>(wt), static_cast<float *>(y),
+        static_cast<int32_t>(n), static_cast<int32_t>(k), ldw, static_cast<int32_t>(gate_row),
+        static_cast<int32_t>(up_row));
+    return launch_status();
 }

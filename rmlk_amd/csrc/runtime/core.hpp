@@ -207,6 +207,7 @@ void op_fused_rotary(OpContext &c);
 void op_fused_attn_matmul(OpContext &c);
 void op_fused_attention(OpContext &c);
 void op_fused_matmul_add_rmsnorm(OpContext &c);
+void op_fused_matmul_const(OpContext &c);
 void op_fused_matmul_group(OpContext &c);
 void op_fused_matmul_group_swiglu(OpContext &c);
 

@@ -519,6 +519,11 @@ struct Matcher {
                     Node f;
                     f.op = "rmlk.MatMulAddRMSNorm";
                     f.inputs = {mm->inputs[0], w, cons.inputs[1 - side], cons.inputs[2]};
+                    const int wt = transposed_copy(w);
+                    if (wt >= 0) {
+                        f.inputs.push_back(wt);
+                        users[wt].push_back(static_cast<int>(n));
+                    }
                     f.outputs = cons.outputs;
                     f.attrs = cons.attrs;
                     Node norm = cons;
@@ -561,6 +566,66 @@ struct Matcher {
                 g.nodes[n] = std::move(f);
                 ++formed;
             }
+        }
+        return formed;
+    }
+
+    // A K-contiguous ([n][k]) device copy of the constant 2-D float matrix `w` ([k][n]) as a new
+    // initializer; -1 when w is not such a matrix. A one-row product reads it with a wavefront per
+    // output column and needs no split-K combine; the row-major original stays for the GEMM.
+    std::unordered_map<int, int> transposed_of;
+    int transposed_copy(int w) {
+        auto it = transposed_of.find(w);
+        if (it != transposed_of.end()) return it->second;
+        if (w < 0 || !g.values[w].is_initializer) return -1;
+        const Tensor &t = s.values[w];
+        if (!t.defined() || t.dtype != RMLK_FLOAT || t.rank() != 2 || t.shape[0] == 0 || t.shape[1] == 0 ||
+            t.shape[0] % 4 != 0)
+            return -1;
+        Tensor tt;
+        tt.dtype = RMLK_FLOAT;
+        tt.shape = {t.shape[1], t.shape[0]};
+        auto buf = std::make_shared<Buffer>();
+        buf->bytes = tt.nbytes();
+        buf->owned_raw = true;
+        check_hip(hipMalloc(&buf->ptr, buf->bytes), "hipMalloc (K-contiguous weights)");
+        tt.buf = buf;
+        rmlk_dims in_shape = to_dims(t.shape);
+        const int64_t perm[2] = {1, 0};
+        check_status(rmlk_hip_transpose(s.stream, RMLK_FLOAT, &in_shape, perm, t.data(), tt.data()),
+                     "K-contiguous weights");
+        check_hip(hipStreamSynchronize(s.stream), "hipStreamSynchronize");
+        const int id = static_cast<int>(g.values.size());
+        Value v;
+        v.name = "rmlk.k_contiguous." + std::to_string(w);
+        v.dtype = RMLK_FLOAT;
+        v.shape = tt.shape;
+        v.is_initializer = true;
+        g.values.push_back(v);
+        g.by_name[v.name] = id;
+        s.values.push_back(tt);
+        users.emplace_back();
+        transposed_of[w] = id;
+        return id;
+    }
+
+    // ---- remaining MatMuls with constant 2-D weights (the lm-head): a K-contiguous copy for one row ---
+    int form_const_matmuls() {
+        int formed = 0;
+        for (size_t n = 0; n < g.nodes.size(); ++n) {
+            if (removed[n] || g.nodes[n].op != "MatMul") continue;
+            const Node &mm = g.nodes[n];
+            if (mm.inputs.size() != 2 || mm.inputs[0] < 0) continue;
+            const int wt = transposed_copy(mm.inputs[1]);
+            if (wt < 0) continue;
+            Node f;
+            f.op = "rmlk.MatMulConst";
+            f.inputs = {mm.inputs[0], mm.inputs[1], wt};
+            f.outputs = mm.outputs;
+            f.body = {mm};
+            users[wt].push_back(static_cast<int>(n));
+            g.nodes[n] = std::move(f);
+            ++formed;
         }
         return formed;
     }
@@ -635,9 +700,11 @@ struct Matcher {
             g.by_name[jv.name] = joint_id;
             s.values.push_back(joint);
             users.emplace_back();
+            const int joint_t = transposed_copy(joint_id);
             Node f;
             f.op = "rmlk.MatMulGroup";
             f.inputs = {a, joint_id};
+            if (joint_t >= 0) f.inputs.push_back(joint_t);
             f.attrs["widths"] = a_ints(widths);
             for (size_t i = 0; i < members.size(); ++i) {
                 const Node &mm = g.nodes[members[i]];
@@ -655,6 +722,7 @@ struct Matcher {
             removed[first] = false;
             users[a].push_back(static_cast<int>(first));
             users[joint_id].push_back(static_cast<int>(first));
+            if (joint_t >= 0) users[joint_t].push_back(static_cast<int>(first));
             for (int v : g.nodes[first].outputs) g.values[v].producer = static_cast<int>(first);
             ++formed;
         }
@@ -975,6 +1043,22 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
         ok = res.shape == out_shape && (axis == -1 || axis == res.rank() - 1) && gamma.rank() >= 1 &&
              gamma.rank() <= res.rank() && gamma.numel() == w.shape[1] && gamma.shape.back() == w.shape[1];
     }
+    if (ok && a.numel() == w.shape[0] && c.has_input(4)) {
+        // one row: the product over the K-contiguous copy (no combine launch), then Add + norm
+        const int64_t k = w.shape[0], n = w.shape[1];
+        float *prod = static_cast<float *>(c.scratch(static_cast<size_t>(n) * sizeof(float)));
+        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, n, k, a.data(), c.input(4).data(), k, prod),
+                           "rmlk.MatMulAddRMSNorm")) {
+            Tensor &sum = c.alloc_output(0, RMLK_FLOAT, res.shape);
+            Tensor &y = c.alloc_output(1, RMLK_FLOAT, res.shape);
+            if (took_fast_path(rmlk_hip_add_rmsnorm(c.stream, RMLK_FLOAT, 1, n, prod, res.data(), gamma.data(),
+                                                    attr_float(c, "epsilon"),
+                                                    static_cast<int32_t>(c.attr_int("reciprocal", 0)),
+                                                    sum.data(), y.data()),
+                               "rmlk.MatMulAddRMSNorm"))
+                return;
+        }
+    }
     if (ok) {
         const int64_t k = w.shape[0], n = w.shape[1], m = a.numel() / k;
         const size_t bytes = rmlk_hip_matmul_partials_workspace_size(RMLK_FLOAT, m, n, k);
@@ -994,6 +1078,23 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
                     return;
             }
         }
+    }
+    run_body(c);
+}
+
+// MatMul(a, W) with constant 2-D W: a one-row input reads the K-contiguous copy of W (no split-K,
+// no combine launch); anything else is the plain MatMul.
+void op_fused_matmul_const(OpContext &c) {
+    const Tensor &a = c.input(0), &w = c.input(1), &wt = c.input(2);
+    if (a.dtype == RMLK_FLOAT && a.rank() >= 1 && w.rank() == 2 && a.shape.back() == w.shape[0] &&
+        a.numel() == w.shape[0] && w.shape[0] > 0) {
+        std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
+        shape.push_back(w.shape[1]);
+        Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
+        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, w.shape[1], w.shape[0], a.data(), wt.data(),
+                                           w.shape[0], y.data()),
+                           "rmlk.MatMulConst"))
+            return;
     }
     run_body(c);
 }
@@ -1030,6 +1131,18 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
         if (took_fast_path(rmlk_hip_matmul_swiglu(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, w.data(),
                                                   2 * n, gate_first ? 0 : n, gate_first ? n : 0, y.data(),
                                                   n),
+                           "rmlk.MatMulGroupSwiGLU"))
+            return;
+    }
+    if (ok && c.has_input(2)) {
+        // one row, K-contiguous weights: gate, up and the activation in one launch
+        const int64_t n = widths[0];
+        const bool gate_first = c.attr_int("gate_first", 1) != 0;
+        std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
+        shape.push_back(n);
+        Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
+        if (took_fast_path(rmlk_hip_gemv_kmajor_swiglu(c.stream, RMLK_FLOAT, n, k, a.data(), c.input(2).data(), k,
+                                                  gate_first ? 0 : n, gate_first ? n : 0, y.data()),
                            "rmlk.MatMulGroupSwiGLU"))
             return;
     }
@@ -1080,7 +1193,11 @@ void op_fused_matmul_group(OpContext &c) {
             c.alloc_output(0, RMLK_FLOAT, {total});
             c.out = keep;
         }
-        run(total, w.data(), row.data(), total);
+        // (over its K-contiguous copy when there is one: no split-K, no combine launch)
+        if (!(c.has_input(2) && took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, total, k, a.data(),
+                                                                c.input(2).data(), k, row.data()),
+                                               "rmlk.MatMulGroup")))
+            run(total, w.data(), row.data(), total);
         int64_t off = 0;
         for (size_t i = 0; i < widths.size(); ++i) {
             Tensor v;
@@ -1139,6 +1256,7 @@ int fuse_patterns(Session &s) {
     formed += m.form_add_rmsnorm();
     formed += m.form_matmul_groups();
     formed += m.form_splitk_epilogues();
+    formed += m.form_const_matmuls();
     if (!formed) return 0;
     std::vector<Node> kept;
     kept.reserve(m.g.nodes.size());

@@ -831,6 +831,7 @@ const std::unordered_map<std::string, OpFn> &registry() {
         {"rmlk.AttnMatMul", op_fused_attn_matmul},
         {"rmlk.Attention", op_fused_attention},
         {"rmlk.MatMulAddRMSNorm", op_fused_matmul_add_rmsnorm},
+        {"rmlk.MatMulConst", op_fused_matmul_const},
         {"rmlk.MatMulGroup", op_fused_matmul_group},
         {"rmlk.MatMulGroupSwiGLU", op_fused_matmul_group_swiglu},
     };

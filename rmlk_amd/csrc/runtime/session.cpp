@@ -480,7 +480,8 @@ void Session::run_nodes() {
             }
             if (node.op == "ScatterND" && !any_new) bytes += static_cast<double>(ctx.in[2]->nbytes());
         }
-        if ((node.op == "MatMul" || node.op == "rmlk.AttnMatMul" || node.op == "rmlk.MatMulGroup") &&
+        if ((node.op == "MatMul" || node.op == "rmlk.AttnMatMul" || node.op == "rmlk.MatMulGroup" ||
+             node.op == "rmlk.MatMulConst") &&
             ctx.in[0] && !ctx.in[0]->shape.empty()) {
             double out_elems = 0.0;
             for (const Tensor &t : outs) out_elems += static_cast<double>(t.numel());

@@ -210,6 +210,18 @@ def attention(q, k, v, mask, out, batch: int, kv_heads: int, rep: int, q_len: in
           "rmlk_hip_attention")
 
 
+def gemv_kmajor(x, wt, y, n: int, k: int) -> None:
+    """y[n] = sum_k x[k] * wt[n][k]: one-row product with K-contiguous weights, no combine launch."""
+    check(lib().rmlk_hip_gemv_kmajor(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(wt), k, _ptr(y)),
+          "rmlk_hip_gemv_kmajor")
+
+
+def gemv_kmajor_swiglu(x, wt, y, n: int, k: int, gate_row: int, up_row: int) -> None:
+    """y[i] = swiglu(x . wt[gate_row + i], x . wt[up_row + i]) in one launch (K-contiguous weights)."""
+    check(lib().rmlk_hip_gemv_kmajor_swiglu(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(wt), k, gate_row,
+                                       up_row, _ptr(y)), "rmlk_hip_gemv_kmajor_swiglu")
+
+
 def matmul_grouped(a, b, outs, m: int, k: int, widths, workspace=None) -> None:
     """outs[i] = a[m, k] . (the next widths[i] columns of the row-major joint matrix b)."""
     n = len(widths)

@@ -213,8 +213,9 @@ def test_pass_forms_the_expected_nodes_on_the_llama_graph(device):
     # per layer: 2 RMSNorm, 2 rotary, 1 SwiGLU, 1 softmax, 2 attention MatMuls, those three merged
     # into one attention node, the q/k/v and the gate/up MatMul groups, 2 residual Adds merged into
     # the norm that follows and the o / down projections merged into those, the gate/up group
-    # merged with the SwiGLU; plus the final RMSNorm
-    assert n == cfg.layers * 16 + 1
+    # merged with the SwiGLU; plus the final RMSNorm and the lm-head (a MatMul with constant
+    # weights gets a K-contiguous copy of them for one-row inputs)
+    assert n == cfg.layers * 16 + 2
     # RMSNorm's mean may differ in the last place; everything downstream inherits that
     _same(a, b, loose=set(a.keys()))
     assert np.array_equal(np.argmax(a["logits"][0], -1), np.argmax(b["logits"][0], -1))
@@ -227,7 +228,7 @@ def test_fused_llama_concat_style_against_oracle(device):
     graph = graphs.llama_graph(cfg, seed=4, style="concat")
     feeds = graphs.llama_concat_inputs(cfg, np.random.default_rng(1).integers(0, cfg.vocab, 9), None, 0)
     inst = runtime.Builder.from_graph(graph).build()
-    assert inst.fused_nodes == cfg.layers * 16 + 1
+    assert inst.fused_nodes == cfg.layers * 16 + 2
     got = inst.run(feeds)
     exp = og.run_graph(graph, feeds)
     for name in exp:
@@ -239,7 +240,7 @@ def test_fused_decoder_layer_full_width(device):
     from rmlk_amd import graphs
     graph, feeds = graphs.decoder_layer_graph(seed=3, seq=96)
     a, b, n, _ = _run_both(graph, feeds)
-    assert n == 14
+    assert n == 15
     _same(a, b, loose={"y"})
 
 
@@ -485,7 +486,7 @@ def test_matmul_group_keeps_a_weight_that_something_else_reads(device):
         gb.output(o)
     feeds = {"x": rng.standard_normal((2, 8), dtype=np.float32)}
     a, b, n, _ = _run_both(gb.build(), feeds)
-    assert n == 1
+    assert n == 2      # the group, and the third product (constant weights) on its own
     for name in a:
         assert_close(a[name], b[name], rtol=1e-4, atol=1e-5)
 
@@ -565,8 +566,9 @@ def test_products_leave_their_combine_to_the_consumer(device, rows):
     feeds = {"x": rng.standard_normal((1, rows, hid), dtype=np.float32),
              "res": rng.standard_normal((1, rows, hid), dtype=np.float32)}
     a, b, n, _ = _run_both(graph, feeds)
-    # RMSNorm, SwiGLU, AddRMSNorm, gate/up group, group + SwiGLU merge, o projection + AddRMSNorm merge
-    assert n == 6
+    # RMSNorm, SwiGLU, AddRMSNorm, gate/up group, group + SwiGLU merge, o projection + AddRMSNorm
+    # merge, the down projection (constant weights, K-contiguous copy for one row)
+    assert n == 7
     exp = og.run_graph(graph, feeds)
     for name in a:
         assert_close(a[name], b[name], rtol=1e-4, atol=1e-5)
@@ -868,3 +870,42 @@ def test_matmul_partials_feed_the_norm(device, m, n, k):
     kk.add_rmsnorm(prod, res, gamma, exp_sum, exp, m, n, 1e-5)
     assert_exact(to_np(got_sum), to_np(exp_sum))
     assert_exact(to_np(got), to_np(exp))
+
+
+@pytest.mark.parametrize("n,k", [(2048, 2048), (2048, 8192), (3072, 2048), (128256, 2048), (5, 8), (70, 132)])
+def test_one_row_product_over_k_contiguous_weights(device, n, k):
+    import torch
+    kk = _k()
+    rng = np.random.default_rng(n + k)
+    x_np = rng.standard_normal((k,), dtype=np.float32)
+    w_np = rng.standard_normal((k, n), dtype=np.float32) * np.float32(0.02)
+    x, w = to_dev(x_np, device), to_dev(w_np, device)
+    wt = to_dev(np.ascontiguousarray(w_np.T), device)
+    got = torch.full((n,), float("nan"), device=device)
+    kk.gemv_kmajor(x, wt, got, n, k)
+    sep = torch.empty(n, device=device)
+    kk.matmul(x, w, sep, 1, 1, n, k, k, n, n, 0, 0, 0)
+    assert_close(to_np(got), to_np(sep), rtol=1e-4, atol=1e-5)
+    exp = x_np.astype(np.float64) @ w_np.astype(np.float64)
+    assert_close(to_np(got), exp.astype(np.float32), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("n,k,gate_first", [(8192, 2048, True), (512, 256, False), (7, 64, True)])
+def test_one_row_gate_up_swiglu_over_k_contiguous_weights(device, n, k, gate_first):
+    import torch
+    kk = _k()
+    rng = np.random.default_rng(n + k)
+    x_np = rng.standard_normal((k,), dtype=np.float32)
+    wt_np = rng.standard_normal((2 * n, k), dtype=np.float32) * np.float32(0.05)
+    x, wt = to_dev(x_np, device), to_dev(wt_np, device)
+    go, uo = (0, n) if gate_first else (n, 0)
+    got = torch.full((n,), float("nan"), device=device)
+    kk.gemv_kmajor_swiglu(x, wt, got, n, k, go, uo)
+    both = torch.empty(2 * n, device=device)
+    kk.gemv_kmajor(x, wt, both, 2 * n, k)
+    sep = torch.empty(n, device=device)
+    kk.swiglu(both[go:go + n].contiguous(), both[uo:uo + n].contiguous(), sep)
+    assert_close(to_np(got), to_np(sep), rtol=1e-4, atol=1e-5)
+    g64 = wt_np[go:go + n].astype(np.float64) @ x_np.astype(np.float64)
+    u64 = wt_np[uo:uo + n].astype(np.float64) @ x_np.astype(np.float64)
+    assert_close(to_np(got), (g64 / (1.0 + np.exp(-g64)) * u64).astype(np.float32), rtol=1e-4, atol=1e-5)
