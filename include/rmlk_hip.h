@@ -298,6 +298,20 @@ int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch, i
                            const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
                            int32_t out_seq_major, void *out);
 
+/* The same attention for a handful of query rows per KV head (rep * q_len <= 16: a decode step),
+ * where there is no matrix work, only K and V to read: the keys are split over blocks in chunks of
+ * 64, every block leaves a partial softmax in `workspace`, a second small kernel merges them. Any
+ * kv_len; head_dim == 64; RMLK_ERR_UNSUPPORTED otherwise. */
+size_t rmlk_hip_attention_few_rows_workspace_size(int32_t dtype, int64_t batch, int64_t kv_heads,
+                                                  int64_t rep, int64_t q_len, int64_t kv_len,
+                                                  int64_t head_dim);
+int32_t rmlk_hip_attention_few_rows(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                    int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
+                                    int64_t head_dim, const void *q, const void *k, const void *v,
+                                    const void *mask, const rmlk_dims *mask_stride,
+                                    int32_t scale_is_mul, float scale, int32_t out_seq_major,
+                                    void *workspace, size_t workspace_bytes, void *out);
+
 /* ---- products that share their first operand (q/k/v, gate/up) ----------------------------------
  * The weights of such MatMuls (ref: one cublasGemmStridedBatchedEx each,
  * cuda/src/kernels/gemm.rs:191-232) lie side by side in one row-major matrix B [k, sum(widths)].

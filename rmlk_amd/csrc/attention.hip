@@ -282,36 +282,138 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
     }
 }
 
+// ---- a handful of query rows (a decode step): keys split over blocks ------------------------------
+// With one query row per head there is no matrix work to speak of, only the K and V rows to read:
+// block (chunk, kv head) takes 64 keys for all the query rows of that KV head (rep * q_len <= 16),
+// leaves a partial softmax (maximum, sum, unnormalised output) per row, and a second small kernel
+// merges the chunks. B * G * L / 64 blocks instead of B * G keep enough loads in flight.
+constexpr int kFewRowsMax = 16;
+constexpr int kPartial = kHeadDim + 2;   // floats per (row, chunk): output, maximum, sum
+
+__global__ __launch_bounds__(kAttnThreads) void attention_few_rows_kernel(AttnArgs g, float *__restrict__ ws,
+                                                                          float scale, int32_t scale_is_mul) {
+    __shared__ float Ks[kChunk][kHeadDim + 1];   // +1: lanes read different rows of one column
+    __shared__ __align__(16) float Vs[kChunk][kHeadDim];
+    __shared__ __align__(16) float qs[kFewRowsMax][kHeadDim];
+    __shared__ float ps[kFewRowsMax][kChunk];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int chunk = blockIdx.x, n_chunks = gridDim.x, bg = blockIdx.y;
+    const int b = bg / g.kv_heads, grp = bg - b * g.kv_heads;
+    const int rows = g.rows;
+    const float *Kg = g.k + static_cast<int64_t>(bg) * g.len * kHeadDim;
+    const float *Vg = g.v + static_cast<int64_t>(bg) * g.len * kHeadDim;
+    const float *Qg = g.q + static_cast<int64_t>(bg) * rows * kHeadDim;
+    // stage the chunk (rows past the end: the last valid row, masked below) and the queries
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int idx = tid + i * kAttnThreads;      // 16-byte unit of the 64 x 64 chunk
+        const int r = idx / 16, u = idx % 16;
+        const int key = min(chunk * kChunk + r, g.len - 1);
+        const v4f kv = *reinterpret_cast<const v4f *>(Kg + static_cast<int64_t>(key) * kHeadDim + u * 4);
+        const v4f vv = *reinterpret_cast<const v4f *>(Vg + static_cast<int64_t>(key) * kHeadDim + u * 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) Ks[r][u * 4 + e] = kv[e];
+        *reinterpret_cast<v4f *>(&Vs[r][u * 4]) = vv;
+    }
+    for (int idx = tid; idx < rows * 16; idx += kAttnThreads)
+        *reinterpret_cast<v4f *>(&qs[idx / 16][(idx % 16) * 4]) =
+            *reinterpret_cast<const v4f *>(Qg + static_cast<int64_t>(idx) * 4);
+    __syncthreads();
+    const int key = chunk * kChunk + lane;
+    for (int r = wave; r < rows; r += kAttnThreads / kWave) {
+        const int head = grp * g.rep + r / g.seq, srow = r - (r / g.seq) * g.seq;
+        float dot = 0.f;
+#pragma unroll 16
+        for (int d = 0; d < kHeadDim; ++d) dot = fmaf(qs[r][d], Ks[lane][d], dot);
+        float sc = -INFINITY;
+        if (key < g.len) {
+            const float m = g.mask[b * g.mask_b + head * g.mask_h + srow * g.mask_s + key];
+            sc = (scale_is_mul ? dot * scale : dot / scale) + m;
+        }
+        float mx = sc;
+#pragma unroll
+        for (int o = kWave / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+        const float m_safe = mx == -INFINITY ? 0.f : mx;
+        const float p = expf(sc - m_safe);
+        float sum = p;
+#pragma unroll
+        for (int o = kWave / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+        ps[r][lane] = p;   // read back by this wavefront only
+        __builtin_amdgcn_wave_barrier();
+        float acc = 0.f;   // lane = head dim
+#pragma unroll 16
+        for (int j = 0; j < kChunk; ++j) acc = fmaf(ps[r][j], Vs[j][lane], acc);
+        float *dst = ws + ((static_cast<int64_t>(bg) * n_chunks + chunk) * rows + r) * kPartial;
+        dst[lane] = acc;
+        if (lane == 0) {
+            dst[kHeadDim] = mx;
+            dst[kHeadDim + 1] = sum;
+        }
+    }
+}
+
+// out row = sum over chunks of the partial outputs, rescaled to the common maximum, over the
+// rescaled sums; a wavefront per (kv head, row), lane = head dim.
+__global__ __launch_bounds__(kAttnThreads) void attention_merge_kernel(AttnArgs g, const float *__restrict__ ws,
+                                                                       int32_t n_chunks, int32_t total_rows) {
+    const int lane = threadIdx.x % kWave;
+    const int item = blockIdx.x * (kAttnThreads / kWave) + threadIdx.x / kWave;
+    if (item >= total_rows) return;
+    const int rows = g.rows;
+    const int bg = item / rows, r = item - bg * rows;
+    const int b = bg / g.kv_heads, grp = bg - b * g.kv_heads;
+    const float *src = ws + (static_cast<int64_t>(bg) * n_chunks * rows + r) * kPartial;
+    const int64_t step = static_cast<int64_t>(rows) * kPartial;
+    float m = -INFINITY;
+    for (int c = 0; c < n_chunks; ++c) m = fmaxf(m, src[c * step + kHeadDim]);
+    const float m_safe = m == -INFINITY ? 0.f : m;
+    float acc = 0.f, sum = 0.f;
+    for (int c = 0; c < n_chunks; ++c) {
+        const float w = expf(src[c * step + kHeadDim] - m_safe);
+        acc = fmaf(src[c * step + lane], w, acc);
+        sum = fmaf(src[c * step + kHeadDim + 1], w, sum);
+    }
+    const int head = grp * g.rep + r / g.seq, srow = r - (r / g.seq) * g.seq;
+    g.out[b * g.out_b + head * g.out_h + srow * g.out_s + lane] = acc / sum;   // nothing visible: 0 / 0
+}
+
 }  // namespace
 }  // namespace rmlk
 
 using namespace rmlk;
 
-extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch,
-                                      int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
-                                      int64_t head_dim, const void *q, const void *k, const void *v,
-                                      const void *mask, const rmlk_dims *mask_stride,
-                                      int32_t scale_is_mul, float scale, int32_t out_seq_major,
-                                      void *out) {
+namespace {
+
+// Argument checks and the argument block shared by both attention entry points; RMLK_OK with
+// *empty set when there is nothing to compute.
+int32_t attention_args(int32_t dtype, int64_t batch, int64_t kv_heads, int64_t rep, int64_t q_len,
+                       int64_t kv_len, int64_t head_dim, const void *q, const void *k, const void *v,
+                       const void *mask, const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
+                       int32_t out_seq_major, void *out, bool vector_mask, AttnArgs *args, bool *empty) {
+    *empty = false;
     if (!dims_ok(mask_stride) || mask_stride->rank != 4) return RMLK_ERR_BAD_RANK;
     if (batch < 0 || kv_heads < 0 || rep < 0 || q_len < 0 || kv_len < 0 || head_dim < 0)
         return RMLK_ERR_INVALID_ARGUMENT;
     if (dtype != RMLK_FLOAT || head_dim != kHeadDim) return RMLK_ERR_UNSUPPORTED;
     const int64_t rows = rep * q_len;
-    if (batch * kv_heads * rows == 0) return RMLK_OK;
+    if (batch * kv_heads * rows == 0) {
+        *empty = true;
+        return RMLK_OK;
+    }
     if (kv_len == 0) return RMLK_ERR_UNSUPPORTED;   // Softmax over nothing: left to the separate kernels
     if (!q || !k || !v || !mask || !out) return RMLK_ERR_NULL_POINTER;
     for (int d = 0; d < 4; ++d)
         if (mask_stride->v[d] < 0) return RMLK_ERR_INVALID_ARGUMENT;
-    // 128-bit mask loads, 32-bit byte offsets into one KV head, grid limits
-    if (kv_len % 4 != 0 || mask_stride->v[3] != 1 || mask_stride->v[0] % 4 != 0 ||
-        mask_stride->v[1] % 4 != 0 || mask_stride->v[2] % 4 != 0)
+    if (mask_stride->v[3] != 1) return RMLK_ERR_UNSUPPORTED;
+    // 128-bit mask loads where the kernel makes them
+    if (vector_mask && (kv_len % 4 != 0 || mask_stride->v[0] % 4 != 0 || mask_stride->v[1] % 4 != 0 ||
+                        mask_stride->v[2] % 4 != 0 || reinterpret_cast<uintptr_t>(mask) % 16))
         return RMLK_ERR_UNSUPPORTED;
+    // 32-bit byte offsets into one KV head, grid limits
     if (kv_len * kHeadDim >= (1ll << 29) || rows >= (1ll << 30) || batch * kv_heads >= 65536)
         return RMLK_ERR_UNSUPPORTED;
     if (reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(k) % 16 ||
-        reinterpret_cast<uintptr_t>(v) % 16 || reinterpret_cast<uintptr_t>(mask) % 16 ||
-        reinterpret_cast<uintptr_t>(out) % 16)
+        reinterpret_cast<uintptr_t>(v) % 16 || reinterpret_cast<uintptr_t>(out) % 16)
         return RMLK_ERR_UNSUPPORTED;
     if (scale_is_mul == 0 && scale == 0.f) return RMLK_ERR_UNSUPPORTED;   // x / 0: not this kernel's case
     AttnArgs g{};
@@ -339,10 +441,68 @@ extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64
         g.out_h = q_len * kHeadDim;
         g.out_s = kHeadDim;
     }
+    *args = g;
+    return RMLK_OK;
+}
+
+}  // namespace
+
+extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                      int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
+                                      int64_t head_dim, const void *q, const void *k, const void *v,
+                                      const void *mask, const rmlk_dims *mask_stride,
+                                      int32_t scale_is_mul, float scale, int32_t out_seq_major,
+                                      void *out) {
+    AttnArgs g{};
+    bool empty = false;
+    const int32_t st = attention_args(dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
+                                      mask_stride, scale_is_mul, scale, out_seq_major, out, true, &g, &empty);
+    if (st || empty) return st;
     static DynamicLdsGrant grant;
-    const int32_t st = grant.ensure(attention_rows_kernel, kAttnLdsBytes);
-    if (st) return st;
-    dim3 grid(static_cast<unsigned>((rows + 63) / 64), static_cast<unsigned>(batch * kv_heads), 1);
+    const int32_t granted = grant.ensure(attention_rows_kernel, kAttnLdsBytes);
+    if (granted) return granted;
+    dim3 grid(static_cast<unsigned>((g.rows + 63) / 64), static_cast<unsigned>(batch * kv_heads), 1);
     attention_rows_kernel<<<grid, kAttnThreads, kAttnLdsBytes, as_stream(stream)>>>(g);
+    return launch_status();
+}
+
+extern "C" size_t rmlk_hip_attention_few_rows_workspace_size(int32_t dtype, int64_t batch, int64_t kv_heads,
+                                                             int64_t rep, int64_t q_len, int64_t kv_len,
+                                                             int64_t head_dim) {
+    if (dtype != RMLK_FLOAT || head_dim != kHeadDim || batch <= 0 || kv_heads <= 0 || rep <= 0 ||
+        q_len <= 0 || kv_len <= 0 || rep * q_len > kFewRowsMax)
+        return 0;
+    const int64_t chunks = (kv_len + kChunk - 1) / kChunk;
+    return static_cast<size_t>(batch * kv_heads * chunks * rep * q_len * kPartial) * sizeof(float);
+}
+
+extern "C" int32_t rmlk_hip_attention_few_rows(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                               int64_t kv_heads, int64_t rep, int64_t q_len,
+                                               int64_t kv_len, int64_t head_dim, const void *q,
+                                               const void *k, const void *v, const void *mask,
+                                               const rmlk_dims *mask_stride, int32_t scale_is_mul,
+                                               float scale, int32_t out_seq_major, void *workspace,
+                                               size_t workspace_bytes, void *out) {
+    AttnArgs g{};
+    bool empty = false;
+    const int32_t st = attention_args(dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
+                                      mask_stride, scale_is_mul, scale, out_seq_major, out, false, &g, &empty);
+    if (st || empty) return st;
+    if (g.rows > kFewRowsMax) return RMLK_ERR_UNSUPPORTED;
+    const size_t need = rmlk_hip_attention_few_rows_workspace_size(dtype, batch, kv_heads, rep, q_len, kv_len,
+                                                                   head_dim);
+    if (!workspace || workspace_bytes < need) return RMLK_ERR_WORKSPACE;
+    const int64_t chunks = (kv_len + kChunk - 1) / kChunk;
+    if (chunks >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
+    hipStream_t s = as_stream(stream);
+    float *ws = static_cast<float *>(workspace);
+    dim3 grid(static_cast<unsigned>(chunks), static_cast<unsigned>(batch * kv_heads), 1);
+    attention_few_rows_kernel<<<grid, kAttnThreads, 0, s>>>(g, ws, scale, scale_is_mul);
+    int32_t launched = launch_status();
+    if (launched) return launched;
+    const int64_t total_rows = batch * kv_heads * g.rows;
+    constexpr int kWaves = kAttnThreads / kWave;
+    attention_merge_kernel<<<static_cast<unsigned>((total_rows + kWaves - 1) / kWaves), kAttnThreads, 0, s>>>(
+        g, ws, static_cast<int32_t>(chunks), static_cast<int32_t>(total_rows));
     return launch_status();
 }

@@ -968,8 +968,9 @@ void op_fused_attn_matmul(OpContext &c) {
     run_body(c);
 }
 
-// scores -> scale, mask, softmax -> context of grouped-query attention in one kernel when there are
-// enough query rows to fill its tiles; a decode step (a handful of rows) runs the three nodes.
+// scores -> scale, mask, softmax -> context of grouped-query attention: one kernel when there are
+// enough query rows to fill its tiles, the split-key pair of kernels for a decode step (a handful
+// of rows), the three nodes otherwise.
 void op_fused_attention(OpContext &c) {
     const Tensor &q = c.input(0), &k = c.input(1), &mask = c.input(2), &v = c.input(3);
     bool ok = q.dtype == RMLK_FLOAT && k.dtype == RMLK_FLOAT && v.dtype == RMLK_FLOAT &&
@@ -989,7 +990,24 @@ void op_fused_attention(OpContext &c) {
         const int64_t bsz = k.shape[0], grp = k.shape[1], len = k.shape[2], dim = k.shape[3];
         const int64_t heads = q.shape[1], seq = q.shape[2];
         ok = rep_k == rep_v && q.shape[0] == bsz && heads == grp * rep_k && q.shape[3] == dim &&
-             rep_k * seq >= 32 && mask_strides(mask, {bsz, heads, seq, len}, &ms);
+             mask_strides(mask, {bsz, heads, seq, len}, &ms);
+        const size_t few_bytes =
+            ok ? rmlk_hip_attention_few_rows_workspace_size(RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim) : 0;
+        if (ok && few_bytes) {
+            // a decode step: keys split over blocks, partial softmaxes merged by a second kernel
+            const bool seq_major = c.attr_int("seq_major_output", 0) != 0;
+            void *ws = c.scratch(few_bytes);
+            Tensor &y = seq_major ? c.alloc_output(0, RMLK_FLOAT, {bsz, seq, heads, dim})
+                                  : c.alloc_output(0, RMLK_FLOAT, {bsz, heads, seq, dim});
+            if (took_fast_path(rmlk_hip_attention_few_rows(
+                                   c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, q.data(), k.data(),
+                                   v.data(), mask.data(), &ms,
+                                   static_cast<int32_t>(c.attr_int("scale_is_mul", 0)), attr_float(c, "scale"),
+                                   seq_major ? 1 : 0, ws, few_bytes, y.data()),
+                               "rmlk.Attention"))
+                return;
+        }
+        ok = ok && rep_k * seq >= 32;
         if (ok) {
             const bool seq_major = c.attr_int("seq_major_output", 0) != 0;
             Tensor &y = seq_major ? c.alloc_output(0, RMLK_FLOAT, {bsz, seq, heads, dim})

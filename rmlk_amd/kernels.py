@@ -210,6 +210,20 @@ def attention(q, k, v, mask, out, batch: int, kv_heads: int, rep: int, q_len: in
           "rmlk_hip_attention")
 
 
+def attention_few_rows(q, k, v, mask, out, batch: int, kv_heads: int, rep: int, q_len: int, kv_len: int,
+                       head_dim: int, mask_stride, scale: float, scale_is_mul: bool = False,
+                       out_seq_major: bool = False) -> None:
+    """The attention of a decode step (rep * q_len <= 16 query rows per KV head): keys split over blocks."""
+    need = int(lib().rmlk_hip_attention_few_rows_workspace_size(dtype_of(q), batch, kv_heads, rep, q_len,
+                                                                kv_len, head_dim))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    check(lib().rmlk_hip_attention_few_rows(_stream(), dtype_of(q), batch, kv_heads, rep, q_len, kv_len,
+                                            head_dim, _ptr(q), _ptr(k), _ptr(v), _ptr(mask),
+                                            Dims.of(mask_stride), int(scale_is_mul), float(scale),
+                                            int(out_seq_major), _ptr(ws), need, _ptr(out)),
+          "rmlk_hip_attention_few_rows")
+
+
 def gemv_kmajor(x, wt, y, n: int, k: int) -> None:
     """y[n] = sum_k x[k] * wt[n][k]: one-row product with K-contiguous weights, no combine launch."""
     check(lib().rmlk_hip_gemv_kmajor(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(wt), k, _ptr(y)),

@@ -909,3 +909,42 @@ def test_one_row_gate_up_swiglu_over_k_contiguous_weights(device, n, k, gate_fir
     g64 = wt_np[go:go + n].astype(np.float64) @ x_np.astype(np.float64)
     u64 = wt_np[uo:uo + n].astype(np.float64) @ x_np.astype(np.float64)
     assert_close(to_np(got), (g64 / (1.0 + np.exp(-g64)) * u64).astype(np.float32), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("b,g,rep,s,l,mask_shape,mul", [
+    (1, 8, 4, 1, 640, (1, 1, 1, 640), False),      # a decode step of the 1B shape
+    (2, 2, 3, 2, 130, (2, 1, 2, 130), True),       # ragged last chunk, per-batch mask, two query rows
+    (1, 1, 1, 1, 5, (1, 1, 1, 5), False),
+    (1, 2, 16, 1, 200, (1, 32, 1, 200), True),     # 16 query heads per KV head, per-head mask
+])
+def test_attention_few_rows_matches_separate_kernels(device, b, g, rep, s, l, mask_shape, mul):
+    import torch
+    kk = _k()
+    h, d = g * rep, 64
+    rng = np.random.default_rng(b * 100 + s + l)
+    q_np = rng.standard_normal((b, h, s, d), dtype=np.float32)
+    k_np = rng.standard_normal((b, g, l, d), dtype=np.float32)
+    v_np = rng.standard_normal((b, g, l, d), dtype=np.float32)
+    m_np = rng.standard_normal(mask_shape, dtype=np.float32)
+    m_np[..., l - l // 3:] = -np.inf          # the unwritten tail of a cache
+    scale = 8.0 if not mul else 0.125
+    q, k, v, m = (to_dev(x, device) for x in (q_np, k_np, v_np, m_np))
+    full = [b, h, s, l]
+    ms = bcast_strides(list(mask_shape), full)
+    got = torch.full((b, h, s, d), float("nan"), device=device)
+    kk.attention_few_rows(q, k, v, m, got, b, g, rep, s, l, d, ms, scale, mul)
+    assert_close(to_np(got), _attention_reference(q_np, k_np, v_np, m_np, scale, mul), rtol=1e-4, atol=1e-5)
+    moved = torch.full((b, s, h, d), float("nan"), device=device)
+    kk.attention_few_rows(q, k, v, m, moved, b, g, rep, s, l, d, ms, scale, mul, out_seq_major=True)
+    assert_exact(to_np(moved), to_np(got).transpose(0, 2, 1, 3))
+
+
+def test_attention_few_rows_declines_many_rows(device):
+    import torch
+    from rmlk_amd import RmlkError
+    kk = _k()
+    q = torch.zeros(1, 8, 5, 64, device=device)
+    k = torch.zeros(1, 2, 64, 64, device=device)
+    m = torch.zeros(5, 64, device=device)
+    with pytest.raises(RmlkError):
+        kk.attention_few_rows(q, k, k, m, torch.zeros_like(q), 1, 2, 4, 5, 64, 64, [0, 0, 64, 1], 8.0)
