@@ -364,15 +364,24 @@ __global__ __launch_bounds__(kAttnThreads) void attention_merge_kernel(AttnArgs 
     const int b = bg / g.kv_heads, grp = bg - b * g.kv_heads;
     const float *src = ws + (static_cast<int64_t>(bg) * n_chunks * rows + r) * kPartial;
     const int64_t step = static_cast<int64_t>(rows) * kPartial;
+    // maxima and sums: a chunk per lane (all loads in flight at once), then the outputs chunk by chunk
     float m = -INFINITY;
-    for (int c = 0; c < n_chunks; ++c) m = fmaxf(m, src[c * step + kHeadDim]);
+    for (int c0 = 0; c0 < n_chunks; c0 += kWave)
+        if (c0 + lane < n_chunks) m = fmaxf(m, src[(c0 + lane) * step + kHeadDim]);
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, kWave));
     const float m_safe = m == -INFINITY ? 0.f : m;
     float acc = 0.f, sum = 0.f;
-    for (int c = 0; c < n_chunks; ++c) {
-        const float w = expf(src[c * step + kHeadDim] - m_safe);
-        acc = fmaf(src[c * step + lane], w, acc);
-        sum = fmaf(src[c * step + kHeadDim + 1], w, sum);
+    for (int c0 = 0; c0 < n_chunks; c0 += kWave) {
+        const int c = c0 + lane;
+        const float w = c < n_chunks ? expf(src[c * step + kHeadDim] - m_safe) : 0.f;
+        if (c < n_chunks) sum = fmaf(src[c * step + kHeadDim + 1], w, sum);
+        const int here = min(kWave, n_chunks - c0);
+#pragma unroll 8
+        for (int j = 0; j < here; ++j) acc = fmaf(src[(c0 + j) * step + lane], __shfl(w, j, kWave), acc);
     }
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
     const int head = grp * g.rep + r / g.seq, srow = r - (r / g.seq) * g.seq;
     g.out[b * g.out_b + head * g.out_h + srow * g.out_s + lane] = acc / sum;   // nothing visible: 0 / 0
 }
