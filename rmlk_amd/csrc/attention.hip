@@ -133,16 +133,15 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
 
     // The mask of this lane's 16 keys of a chunk (keys 8a + 4*half + 0..3 of the wavefront's 32) is
     // fetched one chunk ahead, together with that chunk's K and V, and everything is awaited at once
-    // at the end of a step with vmcnt(0). (A partial wait in the middle of a step, "all but the
-    // eight newest loads", was tried first and read stale mask registers now and then: loads that
-    // return to registers and loads bound for LDS do not retire in one common order.)
+    // at the end of a step. These are ordinary loads on purpose: the compiler has to know that the
+    // registers are still in flight. (Issued from inline assembly they looked ready at once, and
+    // the register allocator copied them to other registers BEFORE the wait, which now and then
+    // picked up what the registers held before the data arrived.)
     auto load_mask = [&](v4f (&dst)[4], int c) {
         const int key0 = c * kChunk + wk * 32 + 4 * half;
 #pragma unroll
-        for (int a = 0; a < 4; ++a) {
-            const float *mp = mrow + min(key0 + 8 * a, g.len - 4);
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst[a]) : "v"(mp) : "memory");
-        }
+        for (int a = 0; a < 4; ++a)
+            dst[a] = *reinterpret_cast<const v4f *>(mrow + min(key0 + 8 * a, g.len - 4));
     };
     v4f mk[4], mk_next[4];
     load_mask(mk, 0);

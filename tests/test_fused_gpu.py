@@ -837,6 +837,35 @@ def test_decoder_layer_gives_the_same_bits_every_time(device):
     inst.close()
 
 
+def test_long_prompt_replays_give_the_bits_of_the_eager_run(device):
+    """A 2048-token prompt (the causal mask no longer fits the caches, so its loads are slow) through
+    a recorded graph: every replay equals the eager run bit for bit. The attention kernel once took
+    its prefetched mask from registers that the data had not reached yet, in about one replay of
+    twenty at this size."""
+    from rmlk_amd import graphs, runtime
+    cfg = graphs.LlamaConfig()
+    cfg.layers, cfg.vocab = 4, 8192
+    prompt_len, max_len = 2048, 2064
+    graph = graphs.llama_graph(cfg, seed=4, style="scatter", max_len=max_len)
+    inst = runtime.Builder.from_graph(graph).build()
+    rng = np.random.default_rng(4)
+    inst.set_input("input_ids", rng.integers(0, cfg.vocab, size=(1, prompt_len)).astype(np.int64))
+    inst.set_input("position_ids", np.arange(prompt_len, dtype=np.int64).reshape(1, -1))
+    for l in range(cfg.layers):
+        for kv in ("key", "value"):
+            inst.set_input(f"cache.{l}.{kv}", np.zeros((1, cfg.kv_heads, max_len, cfg.head_dim), np.float32))
+    names = [f"cache_out.{cfg.layers - 1}.key", "logits"]
+    inst.execute()
+    first = {n: inst.output(n).copy() for n in names}
+    inst.capture()
+    for _ in range(10):
+        inst.replay()
+        inst.sync()
+        for n in names:
+            assert_exact(inst.output(n), first[n])
+    inst.close()
+
+
 @pytest.mark.parametrize("m,n,k", [(512, 2048, 2048), (512, 2048, 8192), (300, 96, 200), (64, 256, 64)])
 def test_matmul_partials_feed_the_norm(device, m, n, k):
     """rmlk_hip_matmul_partials + rmlk_hip_splitk_add_rmsnorm against rmlk_hip_matmul +
