@@ -377,6 +377,38 @@ int32_t rmlk_hip_rotary(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *sh
                         const rmlk_dims *sin_stride, const void *x, const void *cos,
                         const void *sin, void *out);
 
+/* Several streams of head rows in one launch. Stream i reads rows of D elements of x, logical
+ * shape [B, H, S, D], through element strides (innermost 1), rotates them like rmlk_hip_rotary
+ * when cos and sin are given (both NULL: the rows are moved unchanged, i.e. a Transpose perm
+ * 0,2,1,3 read through strides) and writes them
+ *   idx == NULL: densely to out [B, H, S, D];
+ *   idx != NULL: to out = the data tensor of a ScatterND (reduction none) that already holds its
+ *                copy of the data, shape data_shape = [.., D] of rank tuple_size + 1, row r
+ *                (b, h, s order) going where the index tuple idx[r * tuple_size ..] points;
+ *                negative indices wrap, an index out of range sets *err_flag and skips the row
+ *                (as rmlk_hip_scatter_nd).
+ * One launch covers what a decoder layer does behind its q/k/v projection (q rotated, k rotated
+ * into the key cache, v moved into the value cache); the results equal the separate kernels'
+ * bit for bit. At most 4 streams, all with the same D; tuple_size <= 4.
+ * Chain per stream: [Transpose 0,2,1,3] [Slice Slice Neg Concat Mul Mul Add] [ScatterND]
+ * (ref: cuda/src/kernels/transpose.rs:38-80, slice.rs:61-122, unary.rs:10-42, binary.rs:58-100,
+ * scatter_nd.rs:11-77; runtime/src/providers/cuda/backend/scatter_nd.rs:78-225). */
+typedef struct rmlk_row_stream {
+    rmlk_dims shape;        /* logical [B, H, S, D] */
+    rmlk_dims x_stride;     /* element strides of x over those dims */
+    const void *x;
+    const void *cos;        /* NULL (with sin): move */
+    const void *sin;
+    rmlk_dims cos_stride;   /* read only when cos / sin are given */
+    rmlk_dims sin_stride;
+    void *out;
+    const int64_t *idx;     /* NULL: dense output */
+    int32_t tuple_size;     /* read only when idx is given */
+    rmlk_dims data_shape;
+} rmlk_row_stream;
+int32_t rmlk_hip_head_rows(rmlk_stream_t stream, int32_t dtype, int32_t n_streams,
+                           const rmlk_row_stream *streams, int32_t *err_flag);
+
 /* Fill `n` elements of `out` with the element at host address `value` (size of dtype).
  * ref: runtime/src/providers/cuda/backend/constant_of_shape.rs:59-62 (host vector + H2D). */
 int32_t rmlk_hip_fill(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *value,

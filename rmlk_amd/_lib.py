@@ -39,6 +39,13 @@ class Dims(ctypes.Structure):
         return d
 
 
+class RowStream(ctypes.Structure):
+    """struct rmlk_row_stream"""
+    _fields_ = [("shape", Dims), ("x_stride", Dims), ("x", c_void_p), ("cos", c_void_p),
+                ("sin", c_void_p), ("cos_stride", Dims), ("sin_stride", Dims), ("out", c_void_p),
+                ("idx", c_void_p), ("tuple_size", c_int32), ("data_shape", Dims)]
+
+
 class DeviceInfo(ctypes.Structure):
     """struct rmlk_device_info"""
     _fields_ = [("name", ctypes.c_char * 128), ("arch", ctypes.c_char * 64),
@@ -125,6 +132,7 @@ SIGNATURES = {
                                          c_int64]),
     "rmlk_hip_rotary": (c_int32, [c_void_p, c_int32, _PD, _PD, _PD, _PD, c_void_p, c_void_p,
                                   c_void_p, c_void_p]),
+    "rmlk_hip_head_rows": (c_int32, [c_void_p, c_int32, c_int32, POINTER(RowStream), c_void_p]),
     "rmlk_hip_fill": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
     "rmlk_hip_range": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p]),
     "rmlk_hip_write_small": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),

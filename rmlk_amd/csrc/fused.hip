@@ -151,6 +151,89 @@ __global__ __launch_bounds__(kBlock) void rotary_kernel(RotaryArgs a) {
     }
 }
 
+
+// Up to kMaxRowStreams independent streams of head rows in ONE launch (blockIdx.y picks the stream):
+// each reads rows of D elements through strides over (b, h, s) like rotary_kernel, rotates them
+// (same expressions, same rounding) or moves them unchanged, and writes them either densely as
+// [B,H,S,D] or to the rows of a ScatterND destination addressed by one index tuple per row
+// (bounds and negative indices as scatter_nd_kernel handles them). That is what a decoder layer
+// does behind its joint q/k/v projection: q rotated, k rotated into the key cache, v moved into
+// the value cache, five launches otherwise.
+constexpr int kMaxRowStreams = 4;
+constexpr int kMaxRowTuple = 4;
+
+struct RowStream {
+    const float *x, *cos, *sin;      // cos == nullptr: rows are moved unchanged
+    float *out;
+    const int64_t *idx;              // nullptr: dense output
+    FastDiv div_s, div_h;
+    uint32_t n_s, n_h;
+    uint32_t total;                  // B * H * S * n_q
+    int32_t tuple_size;
+    int64_t xs[3], cs[3], ss[3];     // strides of (b, h, s)
+    int64_t dim[kMaxRowTuple], stride[kMaxRowTuple];   // leading dims of the scatter destination, in rows
+};
+
+struct RowStreams {
+    RowStream s[kMaxRowStreams];
+    FastDiv div_q;                   // lanes per row
+    uint32_t n_q, half;
+    int32_t *err;
+};
+
+template <int W>
+__global__ __launch_bounds__(kBlock) void head_rows_kernel(RowStreams all) {
+    using V = Vec<float, W>;
+    const RowStream &a = all.s[blockIdx.y];
+    for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t < a.total; t += gridDim.x * kBlock) {
+        const uint32_t row = all.div_q.div(t), q = t - row * all.n_q;
+        const uint32_t bh = a.div_s.div(row), s = row - bh * a.n_s;
+        const uint32_t b = a.div_h.div(bh), h = bh - b * a.n_h;
+        const int64_t xo = b * a.xs[0] + h * a.xs[1] + s * a.xs[2];
+        const uint32_t d = q * W;
+        const V x1 = *reinterpret_cast<const V *>(a.x + xo + d);
+        const V x2 = *reinterpret_cast<const V *>(a.x + xo + d + all.half);
+        V y1 = x1, y2 = x2;
+        if (a.cos) {
+            const int64_t co = b * a.cs[0] + h * a.cs[1] + s * a.cs[2];
+            const int64_t so = b * a.ss[0] + h * a.ss[1] + s * a.ss[2];
+            const V c1 = *reinterpret_cast<const V *>(a.cos + co + d);
+            const V c2 = *reinterpret_cast<const V *>(a.cos + co + d + all.half);
+            const V s1 = *reinterpret_cast<const V *>(a.sin + so + d);
+            const V s2 = *reinterpret_cast<const V *>(a.sin + so + d + all.half);
+#pragma unroll
+            for (int j = 0; j < W; ++j) {
+                const float a1 = x1.v[j] * c1.v[j];
+                const float r1 = (-x2.v[j]) * s1.v[j];
+                y1.v[j] = a1 + r1;
+                const float a2 = x2.v[j] * c2.v[j];
+                const float r2 = x1.v[j] * s2.v[j];
+                y2.v[j] = a2 + r2;
+            }
+        }
+        int64_t out_row = row;
+        if (a.idx) {
+            out_row = 0;
+            bool bad = false;
+#pragma unroll
+            for (int k = 0; k < kMaxRowTuple; ++k)
+                if (k < a.tuple_size) {
+                    int64_t ix = a.idx[static_cast<int64_t>(row) * a.tuple_size + k];
+                    if (ix < 0) ix += a.dim[k];
+                    if (ix < 0 || ix >= a.dim[k]) bad = true;
+                    out_row += ix * a.stride[k];
+                }
+            if (bad) {
+                if (all.err) *all.err = 1;
+                continue;
+            }
+        }
+        float *o = a.out + out_row * (2 * all.half) + d;
+        *reinterpret_cast<V *>(o) = y1;
+        *reinterpret_cast<V *>(o + all.half) = y2;
+    }
+}
+
 }  // namespace
 }  // namespace rmlk
 
@@ -266,5 +349,104 @@ extern "C" int32_t rmlk_hip_rotary(rmlk_stream_t stream, int32_t dtype, const rm
     if (w == 4) rotary_kernel<4><<<grid, kBlock, 0, s>>>(a);
     else if (w == 2) rotary_kernel<2><<<grid, kBlock, 0, s>>>(a);
     else rotary_kernel<1><<<grid, kBlock, 0, s>>>(a);
+    return launch_status();
+}
+
+extern "C" int32_t rmlk_hip_head_rows(rmlk_stream_t stream, int32_t dtype, int32_t n_streams,
+                                      const rmlk_row_stream *streams, int32_t *err_flag) {
+    if (n_streams < 0 || n_streams > kMaxRowStreams) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n_streams == 0) return RMLK_OK;
+    if (!streams) return RMLK_ERR_NULL_POINTER;
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    RowStreams all{};
+    all.err = err_flag;
+    int64_t d_common = -1, max_total = 0;
+    int w = 4;
+    int n_live = 0;
+    for (int i = 0; i < n_streams; ++i) {
+        const rmlk_row_stream &in = streams[i];
+        const bool rotate = in.cos || in.sin;
+        if (!dims_ok(&in.shape) || !dims_ok(&in.x_stride) || in.shape.rank != 4 || in.x_stride.rank != 4)
+            return RMLK_ERR_BAD_RANK;
+        if (rotate && (!dims_ok(&in.cos_stride) || !dims_ok(&in.sin_stride) ||
+                       in.cos_stride.rank != 4 || in.sin_stride.rank != 4))
+            return RMLK_ERR_BAD_RANK;
+        const int64_t numel = dims_numel(&in.shape);
+        if (numel < 0) return RMLK_ERR_INVALID_ARGUMENT;
+        const int64_t d = in.shape.v[3];
+        if (in.idx) {
+            if (!dims_ok(&in.data_shape)) return RMLK_ERR_BAD_RANK;
+            if (in.tuple_size < 1 || in.tuple_size != in.data_shape.rank - 1)
+                return RMLK_ERR_INVALID_ARGUMENT;
+            if (in.tuple_size > kMaxRowTuple) return RMLK_ERR_UNSUPPORTED;
+            if (in.data_shape.v[in.tuple_size] != d || dims_numel(&in.data_shape) < 0)
+                return RMLK_ERR_INVALID_ARGUMENT;
+        }
+        if (numel == 0) continue;
+        if (!in.x || !in.out || (rotate && (!in.cos || !in.sin))) return RMLK_ERR_NULL_POINTER;
+        if (d % 2 != 0) return RMLK_ERR_INVALID_ARGUMENT;
+        if (d_common >= 0 && d != d_common) return RMLK_ERR_UNSUPPORTED;   // one row length per launch
+        d_common = d;
+        if (in.x_stride.v[3] != 1 || (rotate && (in.cos_stride.v[3] != 1 || in.sin_stride.v[3] != 1)))
+            return RMLK_ERR_UNSUPPORTED;
+        for (int k = 0; k < 3; ++k)
+            if (in.x_stride.v[k] < 0 || (rotate && (in.cos_stride.v[k] < 0 || in.sin_stride.v[k] < 0)))
+                return RMLK_ERR_INVALID_ARGUMENT;
+        if (in.idx && dims_numel(&in.data_shape) >= ((int64_t)1 << 40)) return RMLK_ERR_TOO_LARGE;
+        // widest lane width that keeps every access of every stream aligned
+        auto ok = [&](int lanes) {
+            if ((d / 2) % lanes) return false;
+            const uintptr_t mask = static_cast<uintptr_t>(lanes) * 4 - 1;
+            uintptr_t ptrs = reinterpret_cast<uintptr_t>(in.x) | reinterpret_cast<uintptr_t>(in.out);
+            if (rotate) ptrs |= reinterpret_cast<uintptr_t>(in.cos) | reinterpret_cast<uintptr_t>(in.sin);
+            if (ptrs & mask) return false;
+            for (int k = 0; k < 3; ++k) {
+                if (in.x_stride.v[k] % lanes) return false;
+                if (rotate && (in.cos_stride.v[k] % lanes || in.sin_stride.v[k] % lanes)) return false;
+            }
+            return true;
+        };
+        while (w > 1 && !ok(w)) w /= 2;
+        RowStream &a = all.s[n_live++];
+        a.x = static_cast<const float *>(in.x);
+        a.cos = rotate ? static_cast<const float *>(in.cos) : nullptr;
+        a.sin = rotate ? static_cast<const float *>(in.sin) : nullptr;
+        a.out = static_cast<float *>(in.out);
+        a.idx = in.idx;
+        a.n_s = static_cast<uint32_t>(in.shape.v[2]);
+        a.n_h = static_cast<uint32_t>(in.shape.v[1]);
+        a.div_s = FastDiv(a.n_s);
+        a.div_h = FastDiv(a.n_h);
+        for (int k = 0; k < 3; ++k) {
+            a.xs[k] = in.x_stride.v[k];
+            a.cs[k] = rotate ? in.cos_stride.v[k] : 0;
+            a.ss[k] = rotate ? in.sin_stride.v[k] : 0;
+        }
+        a.tuple_size = in.idx ? in.tuple_size : 0;
+        int64_t stride = 1;
+        for (int k = a.tuple_size - 1; k >= 0; --k) {
+            a.dim[k] = in.data_shape.v[k];
+            a.stride[k] = stride;
+            stride *= in.data_shape.v[k];
+        }
+        if (numel >= ((int64_t)1 << 32)) return RMLK_ERR_TOO_LARGE;
+        a.total = static_cast<uint32_t>(numel / d);   // rows for now; lanes per row follow
+    }
+    if (n_live == 0) return RMLK_OK;
+    const int64_t half = d_common / 2;
+    all.half = static_cast<uint32_t>(half);
+    all.n_q = static_cast<uint32_t>(half / w);
+    all.div_q = FastDiv(all.n_q);
+    for (int i = 0; i < n_live; ++i) {
+        const int64_t total = static_cast<int64_t>(all.s[i].total) * all.n_q;
+        if (total >= ((int64_t)1 << 31)) return RMLK_ERR_TOO_LARGE;
+        all.s[i].total = static_cast<uint32_t>(total);
+        max_total = total > max_total ? total : max_total;
+    }
+    const dim3 grid(grid_for(max_total, kBlock, 16), static_cast<unsigned>(n_live));
+    hipStream_t s = as_stream(stream);
+    if (w == 4) head_rows_kernel<4><<<grid, kBlock, 0, s>>>(all);
+    else if (w == 2) head_rows_kernel<2><<<grid, kBlock, 0, s>>>(all);
+    else head_rows_kernel<1><<<grid, kBlock, 0, s>>>(all);
     return launch_status();
 }

@@ -492,6 +492,122 @@ struct Matcher {
         return formed;
     }
 
+    // ---- streams of head rows behind a projection: one launch -------------------------------------
+    // A stream is an rmlk.Rotary node, or a ScatterND (reduction none) whose updates come from an
+    // rmlk.Rotary node or from a head Transpose (0,2,1,3) that feed nothing else. Streams that follow
+    // one another in the node list are gathered (up to four) into one rmlk.HeadRows node at the
+    // position of the last, as long as nothing in between reads the result of an earlier one.
+    int form_head_rows() {
+        struct Stream {
+            int kind;                  // see op_fused_head_rows
+            int last;                  // node index of the stream's last node
+            std::vector<int> nodes;
+            std::vector<int> inputs;
+            int output;
+            int64_t transposed, half, end, slice_axis, concat_axis;
+        };
+        std::vector<Stream> streams;
+        std::vector<bool> taken(g.nodes.size(), false);
+        auto rotary_stream = [&](const Node &rot, Stream *st) {
+            st->inputs = {rot.inputs[0], rot.inputs[1], rot.inputs[2]};
+            st->transposed = attr_int(rot, "transposed_input", 0);
+            st->half = attr_int(rot, "half", 0);
+            st->end = attr_int(rot, "end", 0);
+            st->slice_axis = attr_int(rot, "slice_axis", 0);
+            st->concat_axis = attr_int(rot, "concat_axis", 0);
+        };
+        for (size_t n = 0; n < g.nodes.size(); ++n) {
+            if (removed[n] || g.nodes[n].op != "ScatterND") continue;
+            const Node &sc = g.nodes[n];
+            auto red = sc.attrs.find("reduction");
+            if (red != sc.attrs.end() && red->second.s != "none") continue;
+            if (sc.inputs.size() != 3 || sc.inputs[0] < 0 || sc.inputs[1] < 0 || sc.inputs[2] < 0) continue;
+            const int upd = sc.inputs[2];
+            if (upd == sc.inputs[0] || upd == sc.inputs[1]) continue;
+            Stream st{};
+            st.last = static_cast<int>(n);
+            st.output = sc.outputs[0];
+            if (const Node *rot = produced_by(upd, "rmlk.Rotary")) {
+                if (!only_used_by(upd, {&sc})) continue;
+                st.kind = 1;
+                rotary_stream(*rot, &st);
+                st.nodes = {index_of(rot), static_cast<int>(n)};
+            } else if (const Node *tr = produced_by(upd, "Transpose")) {
+                auto it = tr->attrs.find("perm");
+                const std::vector<int64_t> want = {0, 2, 1, 3};
+                if (it == tr->attrs.end() || it->second.ints != want || !only_used_by(upd, {&sc}) ||
+                    tr->inputs[0] < 0)
+                    continue;
+                st.kind = 2;
+                st.transposed = 1;
+                st.inputs = {tr->inputs[0]};
+                st.nodes = {index_of(tr), static_cast<int>(n)};
+            } else {
+                continue;
+            }
+            st.inputs.push_back(sc.inputs[0]);
+            st.inputs.push_back(sc.inputs[1]);
+            taken[st.nodes[0]] = true;
+            streams.push_back(std::move(st));
+        }
+        for (size_t n = 0; n < g.nodes.size(); ++n) {
+            if (removed[n] || taken[n] || g.nodes[n].op != "rmlk.Rotary") continue;
+            Stream st{};
+            st.kind = 0;
+            st.last = static_cast<int>(n);
+            st.output = g.nodes[n].outputs[0];
+            rotary_stream(g.nodes[n], &st);
+            st.nodes = {static_cast<int>(n)};
+            streams.push_back(std::move(st));
+        }
+        std::sort(streams.begin(), streams.end(),
+                  [](const Stream &a, const Stream &b) { return a.last < b.last; });
+        int formed = 0;
+        size_t i = 0;
+        while (i < streams.size()) {
+            // grow the group while every earlier member's result is first read after the newcomer
+            size_t j = i + 1;
+            auto safe = [&](size_t upto) {
+                for (size_t m = i; m < upto; ++m) {
+                    for (int u : users[streams[m].output])
+                        if (u <= streams[upto].last) return false;
+                }
+                return true;
+            };
+            while (j < streams.size() && j - i < 4 && safe(j)) ++j;
+            const size_t count = j - i;
+            const bool worth = count > 1 || streams[i].kind != 0;
+            if (worth) {
+                Node f;
+                f.op = "rmlk.HeadRows";
+                std::vector<int64_t> kinds, tr, half, end, sa, ca;
+                std::vector<const Node *> parts;
+                for (size_t m = i; m < j; ++m) {
+                    const Stream &st = streams[m];
+                    kinds.push_back(st.kind);
+                    tr.push_back(st.transposed);
+                    half.push_back(st.half);
+                    end.push_back(st.end);
+                    sa.push_back(st.slice_axis);
+                    ca.push_back(st.concat_axis);
+                    f.inputs.insert(f.inputs.end(), st.inputs.begin(), st.inputs.end());
+                    f.outputs.push_back(st.output);
+                    for (int k : st.nodes) parts.push_back(&g.nodes[k]);
+                }
+                f.attrs["kinds"] = a_ints(kinds);
+                f.attrs["transposed"] = a_ints(tr);
+                f.attrs["half"] = a_ints(half);
+                f.attrs["end"] = a_ints(end);
+                f.attrs["slice_axis"] = a_ints(sa);
+                f.attrs["concat_axis"] = a_ints(ca);
+                replace(parts, std::move(f));
+                ++formed;
+            }
+            i = j;
+        }
+        return formed;
+    }
+
     // ---- a producer whose split-K combine can move into the consumer -----------------------------
     // (Tried for one-row inputs as well and dropped, both slower than what they replace: MatMul ->
     // AddRMSNorm, where the norm owns a row with ONE block that then adds up 32-64 slabs by itself;
@@ -890,50 +1006,148 @@ void op_fused_softmax(OpContext &c) {
     run_body(c);
 }
 
-void op_fused_rotary(OpContext &c) {
-    const Tensor &src = c.input(0), &cos_t = c.input(1), &sin_t = c.input(2);
-    const bool pre = c.attr_int("transposed_input", 0) != 0;
-    bool ok = src.dtype == RMLK_FLOAT && cos_t.dtype == RMLK_FLOAT && sin_t.dtype == RMLK_FLOAT &&
-              src.rank() == 4 && cos_t.rank() <= 4 && sin_t.rank() <= 4 && src.numel() > 0;
+namespace {
+
+// Layout of one stream of head rows: the logical [B,H,S,D] shape of `src` (seen through a
+// Transpose 0,2,1,3 when `pre`), its element strides, and, with rotary tables, their broadcast
+// strides into that shape. False when the rotary kernels do not cover the case.
+struct RowLayout {
     std::vector<int64_t> shape, xst;
-    if (ok) {
-        std::vector<int64_t> dense = dense_strides(src.shape);
-        if (pre) {  // logical x = Transpose(src, 0,2,1,3)
-            shape = {src.shape[0], src.shape[2], src.shape[1], src.shape[3]};
-            xst = {dense[0], dense[2], dense[1], dense[3]};
-        } else {
-            shape = src.shape;
-            xst = dense;
-        }
-        const int64_t d = shape[3], half = c.attr_int("half", 0);
-        auto axis_ok = [](int64_t a) { return a == 3 || a == -1; };
-        ok = d == 2 * half && c.attr_int("end", 0) >= d && axis_ok(c.attr_int("slice_axis", 0)) &&
-             axis_ok(c.attr_int("concat_axis", 0));
+    rmlk_dims cs{}, ss{};
+};
+bool row_layout(const Tensor &src, bool pre, RowLayout *out) {
+    if (src.dtype != RMLK_FLOAT || src.rank() != 4 || src.numel() == 0) return false;
+    std::vector<int64_t> dense = dense_strides(src.shape);
+    if (pre) {  // logical x = Transpose(src, 0,2,1,3)
+        out->shape = {src.shape[0], src.shape[2], src.shape[1], src.shape[3]};
+        out->xst = {dense[0], dense[2], dense[1], dense[3]};
+    } else {
+        out->shape = src.shape;
+        out->xst = dense;
     }
-    auto table_strides = [&](const Tensor &t, rmlk_dims *out) {
+    return true;
+}
+bool rotary_layout(const Tensor &src, const Tensor &cos_t, const Tensor &sin_t, bool pre, int64_t half,
+                   int64_t end, int64_t slice_axis, int64_t concat_axis, RowLayout *out) {
+    if (cos_t.dtype != RMLK_FLOAT || sin_t.dtype != RMLK_FLOAT || cos_t.rank() > 4 || sin_t.rank() > 4 ||
+        !row_layout(src, pre, out))
+        return false;
+    const std::vector<int64_t> &shape = out->shape;
+    const int64_t d = shape[3];
+    auto axis_ok = [](int64_t a) { return a == 3 || a == -1; };
+    if (d != 2 * half || end < d || !axis_ok(slice_axis) || !axis_ok(concat_axis)) return false;
+    auto table_strides = [&](const Tensor &t, rmlk_dims *st_out) {
         // broadcast INTO `shape`, last dim full
         std::vector<int64_t> st(4, 0), dense = dense_strides(t.shape);
         const int shift = 4 - t.rank();
-        for (int d = 0; d < t.rank(); ++d) {
-            const int64_t td = t.shape[d], xd = shape[d + shift];
-            if (td == xd) st[d + shift] = td == 1 ? 0 : dense[d];
+        for (int k = 0; k < t.rank(); ++k) {
+            const int64_t td = t.shape[k], xd = shape[k + shift];
+            if (td == xd) st[k + shift] = td == 1 ? 0 : dense[k];
             else if (td != 1) return false;
         }
         if (t.rank() == 0 || t.shape.back() != shape[3]) return false;
         st[3] = 1;
-        *out = to_dims(st);
+        *st_out = to_dims(st);
         return true;
     };
-    rmlk_dims cs{}, ss{};
-    if (ok) ok = table_strides(cos_t, &cs) && table_strides(sin_t, &ss);
-    if (ok) {
-        rmlk_dims sd = to_dims(shape), xs = to_dims(xst);
-        Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
-        if (took_fast_path(rmlk_hip_rotary(c.stream, RMLK_FLOAT, &sd, &xs, &cs, &ss, src.data(),
+    return table_strides(cos_t, &out->cs) && table_strides(sin_t, &out->ss);
+}
+
+}  // namespace
+
+void op_fused_rotary(OpContext &c) {
+    const Tensor &src = c.input(0), &cos_t = c.input(1), &sin_t = c.input(2);
+    RowLayout lay;
+    if (rotary_layout(src, cos_t, sin_t, c.attr_int("transposed_input", 0) != 0, c.attr_int("half", 0),
+                      c.attr_int("end", 0), c.attr_int("slice_axis", 0), c.attr_int("concat_axis", 0),
+                      &lay)) {
+        rmlk_dims sd = to_dims(lay.shape), xs = to_dims(lay.xst);
+        Tensor &y = c.alloc_output(0, RMLK_FLOAT, lay.shape);
+        if (took_fast_path(rmlk_hip_rotary(c.stream, RMLK_FLOAT, &sd, &xs, &lay.cs, &lay.ss, src.data(),
                                            cos_t.data(), sin_t.data(), y.data()),
                            "rmlk.Rotary"))
             return;
     }
+    run_body(c);
+}
+
+// Streams of head rows (rmlk.HeadRows): per stream, by `kinds`,
+//   0  rmlk.Rotary                                 inputs src, cos, sin
+//   1  rmlk.Rotary -> ScatterND(data, idx, .)      inputs src, cos, sin, data, idx
+//   2  Transpose(0,2,1,3) -> ScatterND(data, idx, .)   inputs src, data, idx
+// one output each, all in one launch. The ScatterND destinations follow op_scatter_nd (in place
+// where the data tensor may be overwritten, else a copy first).
+void op_fused_head_rows(OpContext &c) {
+    const std::vector<int64_t> kinds = c.attr_ints("kinds"), pre = c.attr_ints("transposed"),
+                               half = c.attr_ints("half"), end = c.attr_ints("end"),
+                               slice_axis = c.attr_ints("slice_axis"),
+                               concat_axis = c.attr_ints("concat_axis");
+    const size_t n = kinds.size();
+    std::vector<RowLayout> lay(n);
+    std::vector<int> first_input(n);
+    bool ok = n > 0 && n <= 4;
+    int at = 0;
+    int64_t d_common = -1;
+    for (size_t i = 0; i < n && ok; ++i) {
+        first_input[i] = at;
+        const Tensor &src = c.input(at);
+        int data_at = -1;
+        if (kinds[i] == 2) {
+            ok = row_layout(src, pre[i] != 0, &lay[i]);
+            data_at = at + 1;
+            at += 3;
+        } else {
+            ok = rotary_layout(src, c.input(at + 1), c.input(at + 2), pre[i] != 0, half[i], end[i],
+                               slice_axis[i], concat_axis[i], &lay[i]);
+            if (kinds[i] == 1) data_at = at + 3;
+            at += kinds[i] == 1 ? 5 : 3;
+        }
+        if (!ok) break;
+        const int64_t d = lay[i].shape[3];
+        ok = d % 2 == 0 && (d_common < 0 || d == d_common);
+        d_common = d;
+        if (ok && data_at >= 0) {
+            // ScatterND(reduction none) writing whole rows: one index tuple per row, in row order
+            const Tensor &data = c.input(data_at), &idx = c.input(data_at + 1);
+            ok = data.dtype == RMLK_FLOAT && idx.dtype == RMLK_INT64 && data.rank() >= 2 &&
+                 data.rank() <= 5 && idx.rank() == 4 && idx.shape[3] == data.rank() - 1 &&
+                 data.shape.back() == d && idx.shape[0] == lay[i].shape[0] &&
+                 idx.shape[1] == lay[i].shape[1] && idx.shape[2] == lay[i].shape[2] &&
+                 data.numel() > 0;
+        }
+    }
+    if (!ok) {
+        run_body(c);
+        return;
+    }
+    std::vector<rmlk_row_stream> streams(n);
+    for (size_t i = 0; i < n; ++i) {
+        rmlk_row_stream &st = streams[i];
+        st = rmlk_row_stream{};
+        int in = first_input[i];
+        st.shape = to_dims(lay[i].shape);
+        st.x_stride = to_dims(lay[i].xst);
+        st.x = c.input(in++).data();
+        if (kinds[i] != 2) {
+            st.cos = c.input(in++).data();
+            st.sin = c.input(in++).data();
+            st.cos_stride = lay[i].cs;
+            st.sin_stride = lay[i].ss;
+        }
+        if (kinds[i] == 0) {
+            st.out = c.alloc_output(static_cast<int>(i), RMLK_FLOAT, lay[i].shape).data();
+        } else {
+            const Tensor &data = c.input(in), &idx = c.input(in + 1);
+            st.data_shape = to_dims(data.shape);
+            st.tuple_size = static_cast<int32_t>(data.rank() - 1);
+            st.idx = static_cast<const int64_t *>(idx.data());
+            st.out = scatter_destination(c, in, static_cast<int>(i)).data();
+        }
+    }
+    if (took_fast_path(rmlk_hip_head_rows(c.stream, RMLK_FLOAT, static_cast<int32_t>(n), streams.data(),
+                                          c.error_flag()),
+                       "rmlk.HeadRows"))
+        return;
     run_body(c);
 }
 
@@ -1271,6 +1485,7 @@ int fuse_patterns(Session &s) {
         }
     }
     formed += m.form_attention();
+    formed += m.form_head_rows();
     formed += m.form_add_rmsnorm();
     formed += m.form_matmul_groups();
     formed += m.form_splitk_epilogues();

@@ -577,6 +577,28 @@ void op_gather(OpContext &c) {
     }
 }
 
+}  // namespace
+
+// Output `out_index` as the destination of a ScatterND over input `data_index`: the data tensor
+// itself when it may be updated in place (see op_scatter_nd), else a fresh copy of it.
+Tensor &scatter_destination(OpContext &c, int data_index, int out_index) {
+    const Tensor &data = c.input(data_index);
+    const int vid = c.node.inputs[data_index];
+    const Value &v = c.session.graph_copy.values[vid];
+    const bool last_reader = c.session.last_use[vid] == c.node_index;
+    const bool sole_owner = data.buf && data.buf.use_count() == 1;
+    const bool may_overwrite = data.buf && (v.is_input ? data.buf->donated
+                                                       : (data.buf->pool != nullptr));
+    if (last_reader && sole_owner && may_overwrite && !v.is_output && !v.is_initializer)
+        return c.view_output(out_index, data, data.shape);
+    Tensor &y = c.alloc_output(out_index, data.dtype, data.shape);
+    check_status(rmlk_hip_memcpy_dtod(c.stream, y.data(), data.data(), data.nbytes()),
+                 "ScatterND copy");
+    return y;
+}
+
+namespace {
+
 // ref: backend/scatter_nd.rs:78-225. The reference always copies data -> output first
 // (scatter_nd.rs:128-129). Here the copy is skipped and the update is done in place when nothing
 // else can observe the data tensor afterwards: this node is its last reader, no view shares its
@@ -608,20 +630,7 @@ void op_scatter_nd(OpContext &c) {
     int64_t n_tuples = 1;
     for (size_t d = 0; d + 1 < idx.shape.size(); ++d) n_tuples *= idx.shape[d];
 
-    const int vid = c.node.inputs[0];
-    const Value &v = c.session.graph_copy.values[vid];
-    const bool last_reader = c.session.last_use[vid] == c.node_index;
-    const bool sole_owner = data.buf && data.buf.use_count() == 1;
-    const bool may_overwrite = data.buf && (v.is_input ? data.buf->donated
-                                                       : (data.buf->pool != nullptr));
-    Tensor *y;
-    if (last_reader && sole_owner && may_overwrite && !v.is_output && !v.is_initializer) {
-        y = &c.view_output(0, data, data.shape);
-    } else {
-        y = &c.alloc_output(0, data.dtype, data.shape);
-        check_status(rmlk_hip_memcpy_dtod(c.stream, y->data(), data.data(), data.nbytes()),
-                     "ScatterND copy");
-    }
+    Tensor *y = &scatter_destination(c, 0, 0);
     rmlk_dims dd = to_dims(data.shape);
     check_status(rmlk_hip_scatter_nd(c.stream, rcode, data.dtype, &dd, n_tuples,
                                      static_cast<int32_t>(t),
@@ -828,6 +837,7 @@ const std::unordered_map<std::string, OpFn> &registry() {
         {"rmlk.AddRMSNorm", op_fused_add_rmsnorm},
         {"rmlk.ScaleMaskSoftmax", op_fused_softmax},
         {"rmlk.Rotary", op_fused_rotary},
+        {"rmlk.HeadRows", op_fused_head_rows},
         {"rmlk.AttnMatMul", op_fused_attn_matmul},
         {"rmlk.Attention", op_fused_attention},
         {"rmlk.MatMulAddRMSNorm", op_fused_matmul_add_rmsnorm},

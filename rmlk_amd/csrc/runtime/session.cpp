@@ -474,6 +474,10 @@ void Session::run_nodes() {
                     bytes += static_cast<double>(outs[0].nbytes());  // only the gathered rows
                 } else if (node.op == "ScatterND" && ti == ctx.in[0] && !any_new) {
                     continue;  // in place: only indices and updates move
+                } else if (node.op == "rmlk.HeadRows" && ti->buf &&
+                           std::any_of(outs.begin(), outs.end(),
+                                       [&](const Tensor &o) { return o.buf == ti->buf; })) {
+                    continue;  // a cache updated in place: only its new rows move (counted as read)
                 } else {
                     bytes += static_cast<double>(ti->nbytes());
                 }

@@ -264,6 +264,30 @@ def rotary(x, cos, sin, out, shape, x_stride, cos_stride, sin_stride) -> None:
                                 _ptr(sin), _ptr(out)), "rmlk_hip_rotary")
 
 
+def head_rows(streams, err_flag=None) -> None:
+    """Several streams of head rows in one launch. Each stream is a dict: x, shape [B,H,S,D],
+    x_stride, out, and optionally cos, sin, cos_stride, sin_stride (rotate) and idx, data_shape
+    (scatter the rows into `out` by index tuples)."""
+    from ._lib import RowStream
+    arr = (RowStream * len(streams))()
+    for st, d in zip(arr, streams):
+        st.shape = Dims.of(d["shape"])
+        st.x_stride = Dims.of(d["x_stride"])
+        st.x = _ptr(d["x"])
+        if d.get("cos") is not None:
+            st.cos, st.sin = _ptr(d["cos"]), _ptr(d["sin"])
+            st.cos_stride, st.sin_stride = Dims.of(d["cos_stride"]), Dims.of(d["sin_stride"])
+        st.out = _ptr(d["out"])
+        if d.get("idx") is not None:
+            st.idx = _ptr(d["idx"])
+            st.data_shape = Dims.of(d["data_shape"])
+            st.tuple_size = len(d["data_shape"]) - 1
+    dt = dtype_of(streams[0]["x"]) if streams else 1
+    check(lib().rmlk_hip_head_rows(_stream(), dt, len(streams), arr,
+                                   _ptr(err_flag) if err_flag is not None else None),
+          "rmlk_hip_head_rows")
+
+
 def device_info(device: int = 0) -> dict:
     from ._lib import DeviceInfo
     info = DeviceInfo()

@@ -173,6 +173,88 @@ def test_rotary_matches_separate_kernels(device, b, h, s, d, transposed):
     assert_exact(to_np(got), to_np(exp))
 
 
+@pytest.mark.parametrize("b,hq,hk,s,length,d", [
+    (1, 32, 8, 512, 640, 64), (1, 32, 8, 1, 640, 64), (2, 4, 2, 5, 9, 8), (1, 2, 1, 3, 4, 6), (1, 3, 3, 7, 7, 2),
+])
+def test_head_rows_match_separate_kernels(device, b, hq, hk, s, length, d):
+    """q rotated, k rotated into the key cache, v moved into the value cache in ONE launch equal the
+    five separate kernels (rotary x2, transpose, ScatterND x2) bit for bit."""
+    import torch
+    k = _k()
+    rng = np.random.default_rng(hq + s + d)
+    def proj(h):   # a projection output [B,S,H,D]; its logical [B,H,S,D] strides
+        return to_dev(rng.standard_normal((b, s, h, d), dtype=np.float32), device), [s * h * d, d, h * d, 1]
+    q_st, q_xs = proj(hq)
+    k_st, k_xs = proj(hk)
+    v_st, v_xs = proj(hk)
+    cos = to_dev(rng.uniform(-1, 1, size=(1, 1, s, d)).astype(np.float32), device)
+    sin = to_dev(rng.uniform(-1, 1, size=(1, 1, s, d)).astype(np.float32), device)
+    cache_shape = [b, hk, length, d]
+    kc = rng.standard_normal(cache_shape, dtype=np.float32)
+    vc = rng.standard_normal(cache_shape, dtype=np.float32)
+    pos = rng.permutation(length)[:s]
+    idx = np.zeros((b, hk, s, 3), np.int64)
+    idx[..., 0] = np.arange(b).reshape(b, 1, 1)
+    idx[..., 1] = np.arange(hk).reshape(1, hk, 1)
+    idx[..., 2] = pos.reshape(1, 1, s)
+    idx[0, 0, 0, 2] -= length                      # a negative index wraps
+    idx_d = to_dev(idx, device)
+    def table(h):
+        cs = bcast_strides([1, 1, s, d], [b, h, s, d])
+        cs[-1] = 1
+        return cs
+    # separate kernels
+    q_exp = torch.empty(b * hq * s * d, device=device)
+    k_rot = torch.empty(b * hk * s * d, device=device)
+    v_tr = torch.empty(b * hk * s * d, device=device)
+    k.rotary(q_st, cos, sin, q_exp, [b, hq, s, d], q_xs, table(hq), table(hq))
+    k.rotary(k_st, cos, sin, k_rot, [b, hk, s, d], k_xs, table(hk), table(hk))
+    k.transpose(v_st, v_tr, [b, s, hk, d], [0, 2, 1, 3])
+    kc_exp, vc_exp = to_dev(kc, device), to_dev(vc, device)
+    k.scatter_nd(idx_d, k_rot, kc_exp, cache_shape, b * hk * s, 3)
+    k.scatter_nd(idx_d, v_tr, vc_exp, cache_shape, b * hk * s, 3)
+    # one launch
+    q_got = torch.empty_like(q_exp)
+    kc_got, vc_got = to_dev(kc, device), to_dev(vc, device)
+    err = torch.zeros(1, dtype=torch.int32, device=device)
+    k.head_rows([
+        dict(x=q_st, shape=[b, hq, s, d], x_stride=q_xs, cos=cos, sin=sin, cos_stride=table(hq),
+             sin_stride=table(hq), out=q_got),
+        dict(x=k_st, shape=[b, hk, s, d], x_stride=k_xs, cos=cos, sin=sin, cos_stride=table(hk),
+             sin_stride=table(hk), out=kc_got, idx=idx_d, data_shape=cache_shape),
+        dict(x=v_st, shape=[b, hk, s, d], x_stride=v_xs, out=vc_got, idx=idx_d, data_shape=cache_shape),
+    ], err)
+    assert_exact(to_np(q_got), to_np(q_exp))
+    assert_exact(to_np(kc_got), to_np(kc_exp))
+    assert_exact(to_np(vc_got), to_np(vc_exp))
+    assert int(err.item()) == 0
+
+
+def test_head_rows_flag_an_index_out_of_range_and_check_their_arguments(device):
+    import torch
+    from rmlk_amd import RmlkError
+    k = _k()
+    x = to_dev(np.ones((1, 2, 3, 4), np.float32), device)
+    cache = to_dev(np.zeros((1, 2, 5, 4), np.float32), device)
+    idx = np.zeros((1, 2, 3, 3), np.int64)
+    idx[..., 1] = np.arange(2).reshape(1, 2, 1)
+    idx[..., 2] = np.array([0, 5, 2]).reshape(1, 1, 3)     # 5 is past the end of the cache
+    err = torch.zeros(1, dtype=torch.int32, device=device)
+    st = dict(x=x, shape=[1, 2, 3, 4], x_stride=[24, 12, 4, 1], out=cache, idx=to_dev(idx, device),
+              data_shape=[1, 2, 5, 4])
+    k.head_rows([st], err)
+    assert int(err.item()) == 1
+    got = to_np(cache)
+    assert got[0, :, [0, 2]].min() == 1.0 and got[0, :, [1, 3, 4]].max() == 0.0
+    with pytest.raises(RmlkError):       # tuple size must address whole rows
+        k.head_rows([dict(st, data_shape=[1, 2, 5, 8])], err)
+    with pytest.raises(RmlkError):       # more streams than one launch takes
+        k.head_rows([st] * 5, err)
+    with pytest.raises(RmlkError):       # streams of different row lengths
+        k.head_rows([st, dict(x=x, shape=[1, 2, 6, 2], x_stride=[24, 12, 2, 1], out=x)], err)
+    k.head_rows([], err)                 # nothing to do
+
+
 # ---- session level: the fusion pass ------------------------------------------------------------
 
 def _run_both(graph, feeds, outputs=None):
@@ -214,8 +296,9 @@ def test_pass_forms_the_expected_nodes_on_the_llama_graph(device):
     # into one attention node, the q/k/v and the gate/up MatMul groups, 2 residual Adds merged into
     # the norm that follows and the o / down projections merged into those, the gate/up group
     # merged with the SwiGLU; plus the final RMSNorm and the lm-head (a MatMul with constant
-    # weights gets a K-contiguous copy of them for one-row inputs)
-    assert n == cfg.layers * 16 + 2
+    # weights gets a K-contiguous copy of them for one-row inputs); the rotated q and the two cache
+    # updates of a layer (rotated k, transposed v) merged into one node of three row streams
+    assert n == cfg.layers * 17 + 2
     # RMSNorm's mean may differ in the last place; everything downstream inherits that
     _same(a, b, loose=set(a.keys()))
     assert np.array_equal(np.argmax(a["logits"][0], -1), np.argmax(b["logits"][0], -1))
@@ -228,7 +311,7 @@ def test_fused_llama_concat_style_against_oracle(device):
     graph = graphs.llama_graph(cfg, seed=4, style="concat")
     feeds = graphs.llama_concat_inputs(cfg, np.random.default_rng(1).integers(0, cfg.vocab, 9), None, 0)
     inst = runtime.Builder.from_graph(graph).build()
-    assert inst.fused_nodes == cfg.layers * 16 + 2
+    assert inst.fused_nodes == cfg.layers * 17 + 2   # rotated q and k of a layer: one node of two row streams
     got = inst.run(feeds)
     exp = og.run_graph(graph, feeds)
     for name in exp:
@@ -240,7 +323,7 @@ def test_fused_decoder_layer_full_width(device):
     from rmlk_amd import graphs
     graph, feeds = graphs.decoder_layer_graph(seed=3, seq=96)
     a, b, n, _ = _run_both(graph, feeds)
-    assert n == 15
+    assert n == 16
     _same(a, b, loose={"y"})
 
 
@@ -365,6 +448,66 @@ def test_rotary_pattern_on_rank3_runs_the_body(device):
     a, b, n, _ = _run_both(g.build(), feeds)
     assert n == 1
     _same(a, b)
+
+
+def _rope_chain(g, x, out, tag):
+    g.op("Slice", [x, "z", "h", "ax"], [tag + "x1"])
+    g.op("Slice", [x, "h", "e", "ax"], [tag + "x2"])
+    g.op("Neg", [tag + "x2"], [tag + "n2"])
+    g.op("Concat", [tag + "n2", tag + "x1"], [tag + "rot"]).attr("axis", -1)
+    g.op("Mul", [x, "cos"], [tag + "a"])
+    g.op("Mul", [tag + "rot", "sin"], [tag + "r"])
+    g.op("Add", [tag + "a", tag + "r"], [out])
+
+
+@pytest.mark.parametrize("s,early_reader", [(5, False), (1, False), (5, True)])
+def test_rows_behind_the_projections_become_one_node(device, s, early_reader):
+    """Rotary(q), Rotary(k) -> ScatterND and Transpose(v) -> ScatterND merge into one rmlk.HeadRows
+    node with the bits of the separate kernels; a node that reads the rotated q before the cache
+    updates keeps q out of the group."""
+    hq, hk, d, length = 4, 2, 8, 11
+    g = _builder()
+    g.input("q_in", np.float32, [1, s, hq * d])
+    g.input("k_in", np.float32, [1, s, hk * d])
+    g.input("v_in", np.float32, [1, s, hk * d])
+    g.input("cos", np.float32, [1, 1, s, d])
+    g.input("sin", np.float32, [1, 1, s, d])
+    g.input("cache_k", np.float32, [1, hk, length, d])
+    g.input("cache_v", np.float32, [1, hk, length, d])
+    g.input("idx", np.int64, [1, hk, s, 3])
+    for name, val in (("z", [0]), ("h", [d // 2]), ("e", [d]), ("ax", [3]),
+                      ("q_shape", [1, -1, hq, d]), ("kv_shape", [1, -1, hk, d])):
+        g.constant(name, np.array(val, np.int64))
+    for t, shp in (("q", "q_shape"), ("k", "kv_shape"), ("v", "kv_shape")):
+        g.op("Reshape", [t + "_in", shp], [t + "_r"])
+        g.op("Transpose", [t + "_r"], [t + "_t"]).attr("perm", [0, 2, 1, 3])
+    _rope_chain(g, "q_t", "q_rot", "q.")
+    if early_reader:
+        g.op("Neg", ["q_rot"], ["q_neg"])
+        g.output("q_neg")
+    _rope_chain(g, "k_t", "k_rot", "k.")
+    g.op("ScatterND", ["cache_k", "idx", "k_rot"], ["k_out"])
+    g.op("ScatterND", ["cache_v", "idx", "v_t"], ["v_out"])
+    for o in ("q_rot", "k_out", "v_out"):
+        g.output(o)
+    rng = np.random.default_rng(s)
+    idx = np.zeros((1, hk, s, 3), np.int64)
+    idx[..., 1] = np.arange(hk).reshape(1, hk, 1)
+    idx[..., 2] = rng.permutation(length)[:s].reshape(1, 1, s)
+    feeds = {"idx": idx}
+    for name, shape in (("q_in", (1, s, hq * d)), ("k_in", (1, s, hk * d)), ("v_in", (1, s, hk * d)),
+                        ("cos", (1, 1, s, d)), ("sin", (1, 1, s, d)),
+                        ("cache_k", (1, hk, length, d)), ("cache_v", (1, hk, length, d))):
+        feeds[name] = rng.standard_normal(shape, dtype=np.float32)
+    a, b, n, ops = _run_both(g.build(), feeds)
+    assert n == 3                       # two rotary chains, one group of streams
+    assert ops.count("rmlk.HeadRows") == 1 and "ScatterND" not in ops
+    assert ops.count("rmlk.Rotary") == (1 if early_reader else 0)
+    _same(a, b)
+    from oracle import graph as og
+    exp = og.run_graph(g.build(), feeds)
+    for name in exp:
+        assert_close(a[name], exp[name], rtol=1e-4, atol=1e-5)
 
 
 @pytest.mark.parametrize("b,g,rep,s,l,d", [(1, 8, 4, 512, 640, 64), (1, 8, 4, 1, 640, 64),
