@@ -5,11 +5,14 @@
 // cuda/src/kernels/binary.rs:58-100; Softmax, cuda/src/kernels/softmax.rs:5-37; MatMul again) and
 // the [rows, L] score and probability matrices they pass through memory.
 //
-// One block of four wavefronts owns 64 query rows of one KV head (the rep query heads that share
-// it lie one after the other, so they are rows of ONE matrix) and walks the keys in chunks of 64,
-// staged in LDS by direct global -> LDS loads, two buffers. Wavefront (wq, wk) takes query rows
+// One block owns 64 query rows of one KV head (the rep query heads that share it lie one after the
+// other, so they are rows of ONE matrix) and walks the keys in chunks of 32 * NK, staged in LDS by
+// direct global -> LDS loads, two buffers. Wavefront (wq, wk) of the 2 * NK takes query rows
 // wq*32.. and keys wk*32.. of every chunk, with its own running maximum, sum and output
-// accumulator (the two key halves are merged once, at the end, through LDS).
+// accumulator (the NK key parts are merged once, at the end, through LDS). NK = 2 (four
+// wavefronts, 64 KB of LDS, two blocks per CU) when there are blocks enough to fill the chip that
+// way; NK = 4 (eight wavefronts, 128 KB) otherwise, so that every SIMD still holds two wavefronts
+// and one's softmax arithmetic runs under the other's MFMAs.
 //
 // Everything is computed TRANSPOSED so that a query stays in one lane from the scores to the
 // output: S^T = K . Q^T puts query l32 into lane column l32 of the 32x32 MFMA result, with 16 keys
@@ -27,11 +30,21 @@ namespace {
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kAttnThreads = 256;
+// 0: always four wavefronts per block (to compare)
+#ifndef RMLK_ATTN_WIDE_BLOCKS
+#define RMLK_ATTN_WIDE_BLOCKS 1
+#endif
+
+constexpr int kAttnThreads = 256;                 // of the few-rows kernels
 constexpr int kHeadDim = 64;
-constexpr int kChunk = 64;                        // keys per step
-constexpr int kTile = kChunk * kHeadDim;          // floats of one staged K or V chunk
-constexpr int kAttnLdsBytes = 2 * 2 * kTile * 4;  // K and V, two buffers each
+constexpr int kChunk = 64;                        // keys per block of the few-rows kernel
+template <int NK>
+struct AttnShape {
+    static constexpr int kThreads = 2 * NK * kWave;
+    static constexpr int kKeys = 32 * NK;                  // keys per step
+    static constexpr int kTile = kKeys * kHeadDim;         // floats of one staged K or V chunk
+    static constexpr int kLdsBytes = 2 * 2 * kTile * 4;    // K and V, two buffers each
+};
 constexpr float kLog2e = 1.4426950408889634f;
 
 // max / sum of a value over the two lanes (l, l + 32) that share a query, on all 64 lanes: one
@@ -58,24 +71,26 @@ struct AttnArgs {
     float qscale;      // score scale times log2(e): the softmax runs on base-2 exponents
 };
 
-__global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g) {
+template <int NK>
+__global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel(AttnArgs g) {
+    constexpr int kKeys = AttnShape<NK>::kKeys, kTile = AttnShape<NK>::kTile;
     extern __shared__ __align__(16) float smem[];
-    float *Ks = smem;               // [2][64 keys][16 units of 4 floats], unit u of key r at u ^ (r & 15)
-    float *Vs = smem + 2 * kTile;   // [2][64 keys][64], column c of key r at c ^ (32 * ((r >> 2) & 1))
+    float *Ks = smem;               // [2][keys][16 units of 4 floats], unit u of key r at u ^ (r & 15)
+    float *Vs = smem + 2 * kTile;   // [2][keys][64], column c of key r at c ^ (32 * ((r >> 2) & 1))
 
     const int tid = threadIdx.x;
     const int lane = tid % kWave, wave = tid / kWave;
     const int l32 = lane % 32, half = lane / 32;
-    const int wq = wave >> 1, wk = wave & 1;
+    const int wq = wave / NK, wk = wave % NK;
     const int bg = blockIdx.y;
     const int b = bg / g.kv_heads, grp = bg - b * g.kv_heads;
     const int r0 = blockIdx.x * 64;
     const float *Kg = g.k + static_cast<int64_t>(bg) * g.len * kHeadDim;
     const float *Vg = g.v + static_cast<int64_t>(bg) * g.len * kHeadDim;
-    const int n_chunks = (g.len + kChunk - 1) / kChunk;
+    const int n_chunks = (g.len + kKeys - 1) / kKeys;
 
-    // ---- staging: piece p * 4 + wave of a chunk (4 keys, 1 KiB) is this wavefront's p-th load -----
-    const int lrow = wave * 4 + lane / 16;   // key of this lane inside a group of 16 keys
+    // ---- staging: piece p * 2 NK + wave of a chunk (4 keys, 1 KiB) is this wavefront's p-th load ---
+    const int lrow = wave * 4 + lane / 16;   // key of this lane inside a group of 8 NK keys
     const int lunit = lane % 16;
     const uint32_t k_col = static_cast<uint32_t>((lunit ^ (lrow & 15)) * 4);
     const uint32_t v_col = static_cast<uint32_t>((lunit ^ ((wave & 1) << 3)) * 4);
@@ -90,19 +105,14 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
                      : "s"(lds_addr), "v"(voff), "s"(base)
                      : "memory", "m0");
     };
-    auto issue_chunk = [&](int c, int buf) {
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            const int key = min(c * kChunk + p * 16 + lrow, g.len - 1);   // past the end: any valid row
-            direct_load(lds_k + static_cast<uint32_t>(buf * kTile * 4 + p * 4096), Kg,
-                        static_cast<uint32_t>(key * kHeadDim + k_col) * 4u);
-        }
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            const int key = min(c * kChunk + p * 16 + lrow, g.len - 1);
-            direct_load(lds_v + static_cast<uint32_t>(buf * kTile * 4 + p * 4096), Vg,
-                        static_cast<uint32_t>(key * kHeadDim + v_col) * 4u);
-        }
+    // piece p (0..3: K, 4..7: V) of chunk c into buffer buf
+    auto issue_piece = [&](int p, int c, int buf) {
+        const int key = min(c * kKeys + (p & 3) * 8 * NK + lrow, g.len - 1);   // past the end: any valid row
+        const uint32_t lds_at = static_cast<uint32_t>(buf * kTile * 4 + (p & 3) * 2048 * NK);
+        if (p < 4)
+            direct_load(lds_k + lds_at, Kg, static_cast<uint32_t>(key * kHeadDim + k_col) * 4u);
+        else
+            direct_load(lds_v + lds_at, Vg, static_cast<uint32_t>(key * kHeadDim + v_col) * 4u);
     };
 
     // ---- this lane's query: B operand of S^T, scaled once --------------------------------------
@@ -137,15 +147,15 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
     // registers are still in flight. (Issued from inline assembly they looked ready at once, and
     // the register allocator copied them to other registers BEFORE the wait, which now and then
     // picked up what the registers held before the data arrived.)
-    auto load_mask = [&](v4f (&dst)[4], int c) {
-        const int key0 = c * kChunk + wk * 32 + 4 * half;
-#pragma unroll
-        for (int a = 0; a < 4; ++a)
-            dst[a] = *reinterpret_cast<const v4f *>(mrow + min(key0 + 8 * a, g.len - 4));
+    auto load_mask = [&](int a, int c) {
+        const int key0 = c * kKeys + wk * 32 + 4 * half;
+        return *reinterpret_cast<const v4f *>(mrow + min(key0 + 8 * a, g.len - 4));
     };
     v4f mk[4], mk_next[4];
-    load_mask(mk, 0);
-    issue_chunk(0, 0);
+#pragma unroll
+    for (int a = 0; a < 4; ++a) mk[a] = load_mask(a, 0);
+#pragma unroll
+    for (int p = 0; p < 8; ++p) issue_piece(p, 0, 0);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier"
                  : "+v"(mk[0]), "+v"(mk[1]), "+v"(mk[2]), "+v"(mk[3])
                  :
@@ -156,31 +166,35 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
     const int v_frag0 = (wk * 32 + 4 * half) * kHeadDim + (half * 32 + l32);        // d =      l32
     const int v_frag1 = (wk * 32 + 4 * half) * kHeadDim + ((half ^ 1) * 32 + l32);  // d = 32 + l32
 
-    for (int c = 0; c < n_chunks; ++c) {
+    auto step = [&](int c, auto more_tag) {
+        constexpr bool MORE = decltype(more_tag)::value;
         const int buf = c & 1;
-        const bool more = c + 1 < n_chunks;
-        const int key0 = c * kChunk + wk * 32 + 4 * half;
-        if (more) {
-            load_mask(mk_next, c + 1);
-            issue_chunk(c + 1, buf ^ 1);
-        }
+        const int key0 = c * kKeys + wk * 32 + 4 * half;
 
         // S^T (32 keys x 32 queries) = K . Q^T over the 64 head dims
         v16f st = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         const float *ks = Ks + buf * kTile + k_frag;
-#pragma unroll
-        for (int kc = 0; kc < 8; ++kc) {
+        // The next chunk's eight pieces and its mask are requested one after each group of four
+        // MFMAs (all at the top of the step they kept the matrix pipe idle for some 1200 cycles of
+        // address arithmetic and load issue per step).
+        static_for<8>([&](auto kc_tag) {
+            constexpr int kc = decltype(kc_tag)::value;
             const v4f kf = *reinterpret_cast<const v4f *>(ks + (((kc * 2 + half) ^ k_swz) * 4));
 #pragma unroll
             for (int s = 0; s < 4; ++s)
                 st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[s], qf[kc][s], st, 0, 0, 0);
-        }
+            if constexpr (MORE) {
+                if constexpr (kc < 4) mk_next[kc] = load_mask(kc, c + 1);
+                issue_piece(kc, c + 1, buf ^ 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
         float t[16];
 #pragma unroll
         for (int a = 0; a < 4; ++a)
 #pragma unroll
             for (int e = 0; e < 4; ++e) t[4 * a + e] = fmaf(mk[a][e], kLog2e, st[4 * a + e]);
-        if ((c + 1) * kChunk > g.len) {
+        if ((c + 1) * kKeys > g.len) {
             // keys past the end (their rows and mask values were read from valid but unrelated places)
 #pragma unroll
             for (int a = 0; a < 4; ++a)
@@ -227,7 +241,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
             o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[v_frag1 + key_off], p[r], o1, 0, 0, 0);
         }
         // the next chunk and its mask have landed and nobody reads this chunk any more
-        if (more) {
+        if constexpr (MORE) {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier"
                          : "+v"(mk_next[0]), "+v"(mk_next[1]), "+v"(mk_next[2]), "+v"(mk_next[3])
                          :
@@ -237,31 +251,44 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
         } else {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }
-    }
+    };
+    for (int c = 0; c + 1 < n_chunks; ++c) step(c, std::true_type{});
+    step(n_chunks - 1, std::false_type{});
 
-    // ---- merge the two key halves of every query tile and write ----------------------------------
+    // ---- merge the NK key parts of every query tile and write -------------------------------------
     {
         float lo, hi;
         half_pair(l_run, lo, hi);
         l_run = lo + hi;
     }
-    float *cb = smem + wq * (34 * kWave);   // the staging buffers are free after the last barrier
-    if (wk == 1) {
-        cb[lane] = m_run;
-        cb[kWave + lane] = l_run;
+    // the staging buffers are free after the last barrier: part wk >= 1 of tile wq leaves its
+    // maximum, sum and output in slot (wq, wk - 1)
+    constexpr int kSlot = 34 * kWave;
+    float *cb = smem + wq * ((NK - 1) * kSlot);
+    if (wk != 0) {
+        float *mine = cb + (wk - 1) * kSlot;
+        mine[lane] = m_run;
+        mine[kWave + lane] = l_run;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            cb[(2 + r) * kWave + lane] = o0[r];
-            cb[(18 + r) * kWave + lane] = o1[r];
+            mine[(2 + r) * kWave + lane] = o0[r];
+            mine[(18 + r) * kWave + lane] = o1[r];
         }
     }
     __syncthreads();
     if (wk == 0) {
-        const float m1 = cb[lane], l1 = cb[kWave + lane];
-        const float m_f = fmaxf(m_run, m1);
+        float m_f = m_run;
+#pragma unroll
+        for (int j = 0; j < NK - 1; ++j) m_f = fmaxf(m_f, cb[j * kSlot + lane]);
         const float m_safe = m_f == kNegInf ? 0.f : m_f;
-        const float a0 = __builtin_amdgcn_exp2f(m_run - m_safe), a1 = __builtin_amdgcn_exp2f(m1 - m_safe);
-        const float inv = 1.0f / (l_run * a0 + l1 * a1);   // nothing visible at all: 0 * inf = NaN, as Softmax
+        const float a0 = __builtin_amdgcn_exp2f(m_run - m_safe);
+        float aj[NK - 1], total = l_run * a0;
+#pragma unroll
+        for (int j = 0; j < NK - 1; ++j) {
+            aj[j] = __builtin_amdgcn_exp2f(cb[j * kSlot + lane] - m_safe);
+            total += cb[j * kSlot + kWave + lane] * aj[j];
+        }
+        const float inv = 1.0f / total;   // nothing visible at all: 0 * inf = NaN, as Softmax
         const int row = r0 + wq * 32 + l32;
         if (row < g.rows) {
             float *op = g.out + b * g.out_b + head * g.out_h + srow * g.out_s + 4 * half;   // row == qrow here
@@ -271,8 +298,14 @@ __global__ __launch_bounds__(kAttnThreads) void attention_rows_kernel(AttnArgs g
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int r = 4 * a + e;
-                    w0[e] = (o0[r] * a0 + cb[(2 + r) * kWave + lane] * a1) * inv;
-                    w1[e] = (o1[r] * a0 + cb[(18 + r) * kWave + lane] * a1) * inv;
+                    float s0 = o0[r] * a0, s1 = o1[r] * a0;
+#pragma unroll
+                    for (int j = 0; j < NK - 1; ++j) {
+                        s0 += cb[j * kSlot + (2 + r) * kWave + lane] * aj[j];
+                        s1 += cb[j * kSlot + (18 + r) * kWave + lane] * aj[j];
+                    }
+                    w0[e] = s0 * inv;
+                    w1[e] = s1 * inv;
                 }
                 *reinterpret_cast<v4f *>(op + 8 * a) = w0;
                 *reinterpret_cast<v4f *>(op + 32 + 8 * a) = w1;
@@ -466,11 +499,19 @@ extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64
     const int32_t st = attention_args(dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
                                       mask_stride, scale_is_mul, scale, out_seq_major, out, true, &g, &empty);
     if (st || empty) return st;
-    static DynamicLdsGrant grant;
-    const int32_t granted = grant.ensure(attention_rows_kernel, kAttnLdsBytes);
-    if (granted) return granted;
     dim3 grid(static_cast<unsigned>((g.rows + 63) / 64), static_cast<unsigned>(batch * kv_heads), 1);
-    attention_rows_kernel<<<grid, kAttnThreads, kAttnLdsBytes, as_stream(stream)>>>(g);
+    // two blocks of four wavefronts per CU when there are that many, else one block of eight
+    if (!RMLK_ATTN_WIDE_BLOCKS || static_cast<int64_t>(grid.x) * grid.y > kNumCU) {
+        static DynamicLdsGrant grant;
+        const int32_t granted = grant.ensure(attention_rows_kernel<2>, AttnShape<2>::kLdsBytes);
+        if (granted) return granted;
+        attention_rows_kernel<2><<<grid, AttnShape<2>::kThreads, AttnShape<2>::kLdsBytes, as_stream(stream)>>>(g);
+    } else {
+        static DynamicLdsGrant grant;
+        const int32_t granted = grant.ensure(attention_rows_kernel<4>, AttnShape<4>::kLdsBytes);
+        if (granted) return granted;
+        attention_rows_kernel<4><<<grid, AttnShape<4>::kThreads, AttnShape<4>::kLdsBytes, as_stream(stream)>>>(g);
+    }
     return launch_status();
 }
 

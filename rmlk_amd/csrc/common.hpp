@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/rmlk_hip.h"
 
 namespace rmlk {
@@ -219,6 +221,16 @@ struct DynamicLdsGrant {
         return RMLK_OK;
     }
 };
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant
+// expression inside the body.
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
 
 // Grid size for a grid-stride kernel: enough blocks to cover `work` items, capped so that a few
 // waves per SIMD stay resident on all 256 CUs.

@@ -30,16 +30,6 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kMaxSegments = 4;
 
-// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant
-// expression inside the body.
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F &&f) {
-    if constexpr (N > 0) {
-        static_for<N - 1>(f);
-        f(std::integral_constant<int, N - 1>{});
-    }
-}
-
 struct GemmArgs {
     const float *a;
     const float *b;

@@ -851,6 +851,10 @@ def _attention_reference(q, k, v, mask, scale, mul):
     (1, 1, 1, 33, 4, (1, 1, 33, 4), False),           # fewer keys than one chunk
     (1, 2, 2, 64, 256, (1, 4, 64, 256), True),        # per-head mask
     (1, 3, 1, 200, 64, (1, 1, 1, 64), False),         # one mask row for every query
+    # more blocks than compute units: four wavefronts per block instead of eight
+    (1, 8, 4, 2048, 2064, (1, 1, 2048, 2064), False),
+    (2, 8, 3, 700, 132, (2, 1, 700, 132), True),      # the same with ragged rows and keys
+    (1, 8, 4, 512, 200, (1, 1, 512, 200), False),     # eight wavefronts, keys end inside a chunk of 128
 ])
 def test_attention_matches_separate_kernels(device, b, g, rep, s, l, mask_shape, mul):
     import torch
