@@ -194,6 +194,51 @@ def test_llama_tiny_scatter_style_equals_concat_style(device):
     assert stats_e["device_syncs"] == 0 and stats_g["device_syncs"] == 0
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,hidden,ffn", [
+    (6, 2, 64, 384, 640),      # head_dim 64: the attention kernels and the row-stream launch run
+    (4, 2, 128, 512, 768),     # head_dim 128: the attention chain falls back to its three kernels
+    (3, 3, 64, 192, 260),      # no grouped-query repeat, widths that are no multiple of a tile
+])
+def test_llama_other_widths_scatter_style_vs_oracle(device, heads, kv_heads, head_dim, hidden, ffn):
+    """Prefill of 70 tokens and four decode steps (caches fed back on the device) of Llama-shaped
+    graphs of other widths against the oracle, teacher-forced like e2e_ort/llama.rs."""
+    graphs, runtime = _rt()
+    og = _oracle()
+    cfg = graphs.LlamaConfig(layers=2, hidden=hidden, heads=heads, kv_heads=kv_heads, head_dim=head_dim,
+                             ffn=ffn, vocab=1000)
+    max_len = 100
+    graph = graphs.llama_graph(cfg, seed=7, style="scatter", max_len=max_len)
+    rng = np.random.default_rng(7)
+    prompt = rng.integers(0, cfg.vocab, size=70)
+    zeros = {f"cache.{l}.{kv}": np.zeros((1, cfg.kv_heads, max_len, cfg.head_dim), np.float32)
+             for l in range(cfg.layers) for kv in ("key", "value")}
+    inst = runtime.Builder.from_graph(graph).build()
+    got = inst.run(_scatter_feeds(cfg, prompt, 0, zeros))
+    exp = og.run_graph(graph, _scatter_feeds(cfg, prompt, 0, zeros))
+    assert_close(got["logits"], exp["logits"], rtol=1e-3, atol=1e-4)
+    for l in range(cfg.layers):
+        for kv in ("key", "value"):
+            assert_close(got[f"cache_out.{l}.{kv}"], exp[f"cache_out.{l}.{kv}"], rtol=1e-3, atol=1e-4)
+    pos = prompt.size
+    for _ in range(4):
+        tok = int(np.argmax(exp["logits"][0, -1]))
+        assert int(np.argmax(got["logits"][0, -1])) == tok
+        caches = {f"cache.{l}.{kv}": exp[f"cache_out.{l}.{kv}"] for l in range(cfg.layers)
+                  for kv in ("key", "value")}
+        exp = og.run_graph(graph, _scatter_feeds(cfg, np.array([tok]), pos, caches))
+        inst.set_input("input_ids", np.array([[tok]], dtype=np.int64))
+        inst.set_input("position_ids", np.array([[pos]], dtype=np.int64))
+        for l in range(cfg.layers):        # the caches stay on the device, updated in place
+            for kv in ("key", "value"):
+                inst.feed_output(f"cache_out.{l}.{kv}", f"cache.{l}.{kv}")
+        inst.execute()
+        got = {"logits": inst.output("logits")}
+        assert_close(got["logits"], exp["logits"], rtol=1e-3, atol=1e-4)
+        pos += 1
+    assert inst.memory_stats()["device_syncs"] == 0
+    inst.close()
+
+
 def test_config5_kv_stress_small_vs_oracle(device):
     graphs, runtime = _rt()
     graph, feeds = graphs.kv_stress_graph(seed=5, length=256, vocab=1000, hidden=128,
