@@ -589,7 +589,12 @@ Tensor &scatter_destination(OpContext &c, int data_index, int out_index) {
     const bool sole_owner = data.buf && data.buf.use_count() == 1;
     const bool may_overwrite = data.buf && (v.is_input ? data.buf->donated
                                                        : (data.buf->pool != nullptr));
-    if (last_reader && sole_owner && may_overwrite && !v.is_output && !v.is_initializer)
+    // the same value read through another input of this node (as updates, or by another row stream
+    // of the launch) must keep its contents
+    bool read_elsewhere = false;
+    for (size_t i = 0; i < c.node.inputs.size(); ++i)
+        if (static_cast<int>(i) != data_index && c.node.inputs[i] == vid) read_elsewhere = true;
+    if (last_reader && sole_owner && may_overwrite && !read_elsewhere && !v.is_output && !v.is_initializer)
         return c.view_output(out_index, data, data.shape);
     Tensor &y = c.alloc_output(out_index, data.dtype, data.shape);
     check_status(rmlk_hip_memcpy_dtod(c.stream, y.data(), data.data(), data.nbytes()),

@@ -460,6 +460,28 @@ def _rope_chain(g, x, out, tag):
     g.op("Add", [tag + "a", tag + "r"], [out])
 
 
+def test_scatter_whose_updates_are_its_own_data_is_not_done_in_place(device):
+    """ScatterND(d, idx, d) moves rows of an intermediate onto other rows of itself: the update in
+    place that an intermediate otherwise gets would read rows it has already overwritten."""
+    from oracle import graph as og
+    g = _builder()
+    g.input("x", np.float32, [1, 2, 64, 8])
+    g.input("idx", np.int64, [1, 2, 64, 3])
+    g.op("Neg", ["x"], ["d"])
+    g.op("ScatterND", ["d", "idx", "d"], ["y"])
+    g.output("y")
+    rng = np.random.default_rng(11)
+    idx = np.zeros((1, 2, 64, 3), np.int64)
+    idx[..., 1] = np.arange(2).reshape(1, 2, 1)
+    idx[0, 0, :, 2] = rng.permutation(64)
+    idx[0, 1, :, 2] = rng.permutation(64)
+    feeds = {"x": rng.standard_normal((1, 2, 64, 8), dtype=np.float32), "idx": idx}
+    a, b, _, _ = _run_both(g.build(), feeds)
+    exp = og.run_graph(g.build(), feeds)
+    assert_exact(a["y"], exp["y"])
+    assert_exact(b["y"], exp["y"])
+
+
 @pytest.mark.parametrize("s,early_reader", [(5, False), (1, False), (5, True)])
 def test_rows_behind_the_projections_become_one_node(device, s, early_reader):
     """Rotary(q), Rotary(k) -> ScatterND and Transpose(v) -> ScatterND merge into one rmlk.HeadRows
