@@ -347,6 +347,22 @@ int32_t rmlk_hip_gemv_kmajor(rmlk_stream_t stream, int32_t dtype, int64_t n, int
 int32_t rmlk_hip_gemv_kmajor_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
                                const void *x, const void *wt, int64_t ldw, int64_t gate_row,
                                int64_t up_row, void *y);
+/* rmlk_hip_gemv_kmajor with a residual row added to the result: y = x . wt^T + residual (the Add
+ * behind an output projection; ref kernels: gemm.rs:191-232, binary.rs:58-100). */
+int32_t rmlk_hip_gemv_kmajor_add(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k, const void *x,
+                                 const void *wt, int64_t ldw, const void *residual, void *y);
+/* The same products over RMSNorm(x) * gamma instead of x, the normalised row never stored: every
+ * wavefront works out the row's statistics with rmlk_hip_rmsnorm's arithmetic, so the results equal
+ * rmlk_hip_rmsnorm followed by the product bit for bit. k <= 8192, gamma 16-byte aligned, else
+ * RMLK_ERR_UNSUPPORTED. Chain: Pow, ReduceMean, Add, Sqrt, Div | Div(1,.) Mul, Mul, MatMul
+ * (ref kernels: unary.rs:10-42, reduce_mean.rs:5-36, binary.rs:58-100, gemm.rs:191-232). */
+int32_t rmlk_hip_gemv_kmajor_normed(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k, const void *x,
+                                    const void *gamma, float eps, int32_t reciprocal_form, const void *wt,
+                                    int64_t ldw, void *y);
+int32_t rmlk_hip_gemv_kmajor_swiglu_normed(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
+                                           const void *x, const void *gamma, float eps,
+                                           int32_t reciprocal_form, const void *wt, int64_t ldw,
+                                           int64_t gate_row, int64_t up_row, void *y);
 
 /* ---- many-row products whose split-K combine is left to the consumer ----------------------------
  * rmlk_hip_matmul_partials: the tiled kernels of rmlk_hip_matmul for A[m, k] . B[k, n] (row-major,

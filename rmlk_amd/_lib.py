@@ -113,6 +113,13 @@ SIGNATURES = {
                                   c_void_p]),
     "rmlk_hip_gemv_kmajor_swiglu": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p,
                                          c_int64, c_int64, c_int64, c_void_p]),
+    "rmlk_hip_gemv_kmajor_add": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p, c_int64,
+                                           c_void_p, c_void_p]),
+    "rmlk_hip_gemv_kmajor_normed": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p,
+                                              ctypes.c_float, c_int32, c_void_p, c_int64, c_void_p]),
+    "rmlk_hip_gemv_kmajor_swiglu_normed": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p,
+                                                     ctypes.c_float, c_int32, c_void_p, c_int64, c_int64,
+                                                     c_int64, c_void_p]),
     "rmlk_hip_attention": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64,
                                      c_int64, c_void_p, c_void_p, c_void_p, c_void_p, _PD, c_int32,
                                      ctypes.c_float, c_int32, c_void_p]),

@@ -983,24 +983,93 @@ __global__ __launch_bounds__(kThreads) void gemv_dot_kernel(GemvArgs g) {
 // split-K, no workspace and no combine launch whatever the width.
 // SWIGLU: COLS is 2 and the wavefront's two rows of Wt are the gate and the up row of ONE output
 // (rows gate_row + i and up_row + i); it writes silu(gate) * up.
-template <int COLS, bool SWIGLU = false>
+// NORM: x is the row BEFORE an RMSNorm and the product is taken with RMSNorm(x) * gamma, which is
+// never stored in memory: every block first normalises the row into LDS exactly as the norm
+// kernel's block-per-row form does (squares rounded to float, summed in double per lane, wavefront
+// and block in that kernel's order), so the result equals the norm kernel followed by the product
+// bit for bit. (Every WAVEFRONT normalising the row for itself was tried first: the arithmetic,
+// repeated for each output column, cost more than the launch it saves.)
+// `residual` (may be null) is added to the outputs (the Add behind an output projection).
+struct RowNormArgs {
+    const float *gamma;
+    float eps;
+    int32_t reciprocal;
+};
+
+template <int COLS, bool SWIGLU = false, bool NORM = false>
 __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__restrict__ x,
                                                           const float *__restrict__ wt,
                                                           float *__restrict__ y, int32_t n, int32_t k,
-                                                          int64_t ldw, int32_t gate_row, int32_t up_row) {
+                                                          int64_t ldw, int32_t gate_row, int32_t up_row,
+                                                          const float *__restrict__ residual,
+                                                          RowNormArgs norm) {
     static_assert(!SWIGLU || COLS == 2, "gate and up");
     constexpr int kDepth = 8;
+    constexpr int kWaves = kThreads / kWave;
+    // the normalised row of the block (NORM): k floats of dynamic LDS
+    extern __shared__ __align__(16) float xs[];
+    __shared__ double partial[kWaves];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    const int col0 = (blockIdx.x * (kThreads / kWave) + wave) * (SWIGLU ? 1 : COLS);
-    if (col0 >= n) return;
+    const int col0 = (blockIdx.x * kWaves + wave) * (SWIGLU ? 1 : COLS);
     const int k4 = k / 4;
     const v4f *xv = reinterpret_cast<const v4f *>(x);
+    // (a wavefront past the last column keeps valid addresses and takes part in the barriers)
+    const int col_c = min(col0, n - 1);
     const v4f *wv[COLS];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
-        const int64_t row = SWIGLU ? (c == 0 ? gate_row : up_row) + col0 : min(col0 + c, n - 1);
+        const int64_t row = SWIGLU ? (c == 0 ? gate_row : up_row) + col_c : min(col_c + c, n - 1);
         wv[c] = reinterpret_cast<const v4f *>(wt + row * ldw);
     }
+    // NORM: the first batch of weight loads is in flight while the block normalises the row
+    [[maybe_unused]] v4f w_first[kDepth][COLS];
+    if constexpr (NORM) {
+#pragma unroll
+        for (int j = 0; j < kDepth; ++j) {
+            const int u = lane + j * kWave;
+#pragma unroll
+            for (int c = 0; c < COLS; ++c)
+                w_first[j][c] = u < k4 ? __builtin_nontemporal_load(wv[c] + u) : v4f{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    if constexpr (NORM) {
+        // (two passes over the row, which the caches hold: keeping it in registers between them
+        // cost the wavefronts that stream the weights their occupancy)
+        double acc = 0.0;
+        for (int c = threadIdx.x; c < k4; c += kThreads) {
+            const v4f v = xv[c];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float sq = v[j] * v[j];
+                acc += static_cast<double>(sq);
+            }
+        }
+#pragma unroll
+        for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, kWave);
+        if (lane == 0) partial[wave] = acc;
+        __syncthreads();
+        acc = 0.0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) acc += partial[w];
+        const float mean = static_cast<float>(acc / static_cast<double>(k));
+        const float var = mean + norm.eps;
+        const float r = sqrtf(var);
+        const float inv = 1.0f / r;
+        const v4f *gv = reinterpret_cast<const v4f *>(norm.gamma);
+        for (int c = threadIdx.x; c < k4; c += kThreads) {
+            v4f v = xv[c];
+            const v4f g = gv[c];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float normed = norm.reciprocal ? v[j] * inv : v[j] / r;
+                v[j] = normed * g[j];
+            }
+            reinterpret_cast<v4f *>(xs)[c] = v;
+        }
+        __syncthreads();
+    }
+    if (col0 >= n) return;
+    auto load_x = [&](int u) { return NORM ? reinterpret_cast<const v4f *>(xs)[u] : xv[u]; };
     float acc[COLS];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) acc[c] = 0.f;
@@ -1010,10 +1079,12 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__re
         for (int j = 0; j < kDepth; ++j) {
             const int u = u0 + j * kWave;
             const bool live = u < k4;
-            xr[j] = live ? xv[u] : v4f{0.f, 0.f, 0.f, 0.f};
+            xr[j] = live ? load_x(u) : v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < COLS; ++c)
-                wr[j][c] = live ? __builtin_nontemporal_load(wv[c] + u) : v4f{0.f, 0.f, 0.f, 0.f};
+            for (int c = 0; c < COLS; ++c) {
+                if (NORM && u0 == lane) wr[j][c] = w_first[j][c];
+                else wr[j][c] = live ? __builtin_nontemporal_load(wv[c] + u) : v4f{0.f, 0.f, 0.f, 0.f};
+            }
         }
 #pragma unroll
         for (int j = 0; j < kDepth; ++j)
@@ -1026,7 +1097,8 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__re
     for (int c = 0; c < COLS; ++c) {
 #pragma unroll
         for (int o = kWave / 2; o > 0; o >>= 1) acc[c] += __shfl_xor(acc[c], o, kWave);
-        if (!SWIGLU && lane == 0 && col0 + c < n) y[col0 + c] = acc[c];
+        if (!SWIGLU && lane == 0 && col0 + c < n)
+            y[col0 + c] = residual ? acc[c] + residual[col0 + c] : acc[c];
     }
     if (SWIGLU && lane == 0) {
         const float silu = acc[0] * (1.0f / (1.0f + expf(-acc[0])));
@@ -1706,52 +1778,109 @@ extern "C" int32_t rmlk_hip_matmul_partials(rmlk_stream_t stream, int32_t dtype,
                       workspace_bytes, nullptr, splits_out);
 }
 
-extern "C" int32_t rmlk_hip_gemv_kmajor(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
-                                   const void *x, const void *wt, int64_t ldw, void *y) {
+namespace {
+
+// Shared argument checks and launches of the K-major one-row products. `norm`: x is normalised on
+// the fly (see gemv_kmajor_kernel); `residual`: added to the outputs.
+int32_t gemv_kmajor_launch(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k, const void *x,
+                           const void *wt, int64_t ldw, const void *residual, const RowNormArgs *norm,
+                           void *y) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
     if (n < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (n >= (1ll << 31) || k >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
     if (n == 0) return RMLK_OK;
-    if (!y || (k > 0 && (!x || !wt))) return RMLK_ERR_NULL_POINTER;
+    if (!y || (k > 0 && (!x || !wt)) || (norm && !norm->gamma)) return RMLK_ERR_NULL_POINTER;
     if (ldw < k) return RMLK_ERR_SIZE_MISMATCH;
     if (k % 4 != 0 || ldw % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
         reinterpret_cast<uintptr_t>(wt) % 16 != 0)
         return RMLK_ERR_UNSUPPORTED;
+    // the widths the norm kernel gives one block
+    if (norm && (k == 0 || k > kThreads * 4 * 8 || reinterpret_cast<uintptr_t>(norm->gamma) % 16 != 0))
+        return RMLK_ERR_UNSUPPORTED;
     const float *px = static_cast<const float *>(x), *pw = static_cast<const float *>(wt);
+    const float *pr = static_cast<const float *>(residual);
     float *py = static_cast<float *>(y);
     hipStream_t s = as_stream(stream);
     constexpr int kWaves = kThreads / kWave;
+    const int32_t ni = static_cast<int32_t>(n), ki = static_cast<int32_t>(k);
     // few columns: one per wavefront keeps every compute unit busy; many: four share the loads of x
     if (n >= 16 * kNumCU * kWaves) {
         const unsigned grid = static_cast<unsigned>((n + kWaves * 4 - 1) / (kWaves * 4));
-        gemv_kmajor_kernel<4><<<grid, kThreads, 0, s>>>(px, pw, py, static_cast<int32_t>(n), static_cast<int32_t>(k), ldw,
-                                                   0, 0);
+        if (norm) gemv_kmajor_kernel<4, false, true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
+        else gemv_kmajor_kernel<4><<<grid, kThreads, 0, s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, RowNormArgs{});
     } else {
         const unsigned grid = static_cast<unsigned>((n + kWaves - 1) / kWaves);
-        gemv_kmajor_kernel<1><<<grid, kThreads, 0, s>>>(px, pw, py, static_cast<int32_t>(n), static_cast<int32_t>(k), ldw,
-                                                   0, 0);
+        if (norm) gemv_kmajor_kernel<1, false, true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
+        else gemv_kmajor_kernel<1><<<grid, kThreads, 0, s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, RowNormArgs{});
     }
     return launch_status();
 }
 
-extern "C" int32_t rmlk_hip_gemv_kmajor_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
-                                          const void *x, const void *wt, int64_t ldw, int64_t gate_row,
-                                          int64_t up_row, void *y) {
+int32_t gemv_kmajor_swiglu_launch(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k, const void *x,
+                                  const void *wt, int64_t ldw, int64_t gate_row, int64_t up_row,
+                                  const RowNormArgs *norm, void *y) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
     if (n < 0 || k < 0 || gate_row < 0 || up_row < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (n >= (1ll << 30) || k >= (1ll << 31) || gate_row >= (1ll << 30) || up_row >= (1ll << 30))
         return RMLK_ERR_TOO_LARGE;
     if (n == 0) return RMLK_OK;
-    if (!y || (k > 0 && (!x || !wt))) return RMLK_ERR_NULL_POINTER;
+    if (!y || (k > 0 && (!x || !wt)) || (norm && !norm->gamma)) return RMLK_ERR_NULL_POINTER;
     if (ldw < k) return RMLK_ERR_SIZE_MISMATCH;
     if (k % 4 != 0 || ldw % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
         reinterpret_cast<uintptr_t>(wt) % 16 != 0)
         return RMLK_ERR_UNSUPPORTED;
+    if (norm && (k == 0 || k > kThreads * 4 * 8 || reinterpret_cast<uintptr_t>(norm->gamma) % 16 != 0))
+        return RMLK_ERR_UNSUPPORTED;
     constexpr int kWaves = kThreads / kWave;
     const unsigned grid = static_cast<unsigned>((n + kWaves - 1) / kWaves);
-    gemv_kmajor_kernel<2, true><<<grid, kThreads, 0, as_stream(stream)>>>(
-        static_cast<const float *>(x), static_cast<const float *>(wt), static_cast<float *>(y),
-        static_cast<int32_t>(n), static_cast<int32_t>(k), ldw, static_cast<int32_t>(gate_row),
-        static_cast<int32_t>(up_row));
+    const float *px = static_cast<const float *>(x), *pw = static_cast<const float *>(wt);
+    float *py = static_cast<float *>(y);
+    const int32_t ni = static_cast<int32_t>(n), ki = static_cast<int32_t>(k);
+    const int32_t gr = static_cast<int32_t>(gate_row), ur = static_cast<int32_t>(up_row);
+    if (norm)
+        gemv_kmajor_kernel<2, true, true><<<grid, kThreads, k * sizeof(float), as_stream(stream)>>>(
+            px, pw, py, ni, ki, ldw, gr, ur, nullptr, *norm);
+    else
+        gemv_kmajor_kernel<2, true><<<grid, kThreads, 0, as_stream(stream)>>>(px, pw, py, ni, ki, ldw, gr, ur,
+                                                                             nullptr, RowNormArgs{});
     return launch_status();
+}
+
+}  // namespace
+
+extern "C" int32_t rmlk_hip_gemv_kmajor(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
+                                   const void *x, const void *wt, int64_t ldw, void *y) {
+    return gemv_kmajor_launch(stream, dtype, n, k, x, wt, ldw, nullptr, nullptr, y);
+}
+
+extern "C" int32_t rmlk_hip_gemv_kmajor_add(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
+                                            const void *x, const void *wt, int64_t ldw,
+                                            const void *residual, void *y) {
+    if (n > 0 && !residual) return RMLK_ERR_NULL_POINTER;
+    return gemv_kmajor_launch(stream, dtype, n, k, x, wt, ldw, residual, nullptr, y);
+}
+
+extern "C" int32_t rmlk_hip_gemv_kmajor_normed(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
+                                               const void *x, const void *gamma, float eps,
+                                               int32_t reciprocal_form, const void *wt, int64_t ldw,
+                                               void *y) {
+    const RowNormArgs norm{static_cast<const float *>(gamma), eps, reciprocal_form};
+    if (n > 0 && !gamma) return RMLK_ERR_NULL_POINTER;
+    return gemv_kmajor_launch(stream, dtype, n, k, x, wt, ldw, nullptr, &norm, y);
+}
+
+extern "C" int32_t rmlk_hip_gemv_kmajor_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
+                                          const void *x, const void *wt, int64_t ldw, int64_t gate_row,
+                                          int64_t up_row, void *y) {
+    return gemv_kmajor_swiglu_launch(stream, dtype, n, k, x, wt, ldw, gate_row, up_row, nullptr, y);
+}
+
+extern "C" int32_t rmlk_hip_gemv_kmajor_swiglu_normed(rmlk_stream_t stream, int32_t dtype, int64_t n,
+                                                      int64_t k, const void *x, const void *gamma,
+                                                      float eps, int32_t reciprocal_form, const void *wt,
+                                                      int64_t ldw, int64_t gate_row, int64_t up_row,
+                                                      void *y) {
+    const RowNormArgs norm{static_cast<const float *>(gamma), eps, reciprocal_form};
+    if (n > 0 && !gamma) return RMLK_ERR_NULL_POINTER;
+    return gemv_kmajor_swiglu_launch(stream, dtype, n, k, x, wt, ldw, gate_row, up_row, &norm, y);
 }

@@ -80,12 +80,18 @@ struct HostVal {
     double as_double(size_t k) const { return is_float ? f[k] : static_cast<double>(i[k]); }
 };
 
+struct PendingNorm;
+
 struct Tensor {
     int32_t dtype = 0;
     std::vector<int64_t> shape;
     BufferRef buf;
     size_t offset = 0;  // bytes into buf
     std::shared_ptr<HostVal> host;
+    // Set on the result of a one-row RMSNorm that was NOT computed: the memory holds the row before
+    // the norm, and the one consumer (a one-row product, which the fusion pass has checked) applies
+    // the norm while it loads the row, or computes it first if it cannot.
+    std::shared_ptr<const PendingNorm> pending_norm;
 
     bool defined() const { return dtype != 0; }
     int64_t numel() const {
@@ -102,7 +108,14 @@ struct Tensor {
         buf.reset();
         offset = 0;
         host.reset();
+        pending_norm.reset();
     }
+};
+
+struct PendingNorm {
+    Tensor gamma;
+    float eps = 0.f;
+    int32_t reciprocal = 0;
 };
 
 rmlk_dims to_dims(const std::vector<int64_t> &v);          // rank-0 becomes [1]

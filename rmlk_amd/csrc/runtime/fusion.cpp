@@ -608,6 +608,28 @@ struct Matcher {
         return formed;
     }
 
+    // ---- norms whose only reader is a product that can apply them itself (one-row inputs) -----------
+    int mark_deferred_norms() {
+        int marked = 0;
+        for (size_t n = 0; n < g.nodes.size(); ++n) {
+            if (removed[n]) continue;
+            Node &p = g.nodes[n];
+            int normed = -1;
+            if (p.op == "rmlk.RMSNorm") normed = p.outputs[0];
+            else if (p.op == "rmlk.MatMulAddRMSNorm" && p.inputs.size() == 5) normed = p.outputs[1];
+            if (normed < 0 || g.values[normed].is_output || users[normed].size() != 1) continue;
+            const Node &cons = g.nodes[users[normed][0]];
+            const bool aware = (cons.op == "rmlk.MatMulGroup" || cons.op == "rmlk.MatMulGroupSwiGLU" ||
+                                cons.op == "rmlk.MatMulConst") &&
+                               cons.inputs.size() == 3 && cons.inputs[0] == normed &&
+                               cons.inputs[1] != normed && cons.inputs[2] != normed;
+            if (!aware) continue;
+            p.attrs["defer_norm"] = a_int(1);
+            ++marked;
+        }
+        return marked;
+    }
+
     // ---- a producer whose split-K combine can move into the consumer -----------------------------
     // (Tried for one-row inputs as well and dropped, both slower than what they replace: MatMul ->
     // AddRMSNorm, where the norm owns a row with ONE block that then adds up 32-64 slabs by itself;
@@ -873,6 +895,7 @@ void require_float(int32_t dt) {
     if (dt != RMLK_FLOAT) fail_unsupported(dt);
 }
 
+
 float attr_float(const OpContext &c, const char *name) {
     const Attr *a = c.attr(name);
     return a ? a->f : 0.f;
@@ -883,6 +906,51 @@ bool took_fast_path(int32_t st, const char *what) {
     if (st == RMLK_ERR_UNSUPPORTED) return false;
     check_status(st, what);
     return true;
+}
+
+// ---- one-row RMSNorm left to the product that reads it ------------------------------------------
+// A norm node marked `defer_norm` (its result feeds exactly one product over K-contiguous constant
+// weights) does not run for a one-row input: its output is a view of the row BEFORE the norm that
+// carries the norm's parameters (Tensor::pending_norm), and the product's kernel normalises the
+// row while it loads it (rmlk_hip_gemv_kmajor_normed). One launch less per norm of a decode step.
+constexpr int64_t kMaxDeferredNormCols = 8192;   // what the product kernels accept
+// 0: every norm runs as its own launch (to compare)
+#ifndef RMLK_DEFER_NORM
+#define RMLK_DEFER_NORM 1
+#endif
+
+bool may_defer_norm(const OpContext &c, const Tensor &row, const Tensor &gamma) {
+    const int64_t cols = row.shape.empty() ? 0 : row.shape.back();
+    return RMLK_DEFER_NORM && c.attr_int("defer_norm", 0) != 0 && row.dtype == RMLK_FLOAT && gamma.dtype == RMLK_FLOAT &&
+           cols > 0 && row.numel() == cols && cols % 4 == 0 && cols <= kMaxDeferredNormCols &&
+           gamma.numel() == cols;
+}
+
+void defer_norm(OpContext &c, int out_index, const Tensor &row, const Tensor &gamma) {
+    Tensor &y = c.view_output(out_index, row, row.shape);
+    auto pn = std::make_shared<PendingNorm>();
+    pn->gamma = gamma;
+    pn->eps = attr_float(c, "epsilon");
+    pn->reciprocal = static_cast<int32_t>(c.attr_int("reciprocal", 0));
+    y.pending_norm = pn;
+}
+
+// The consumer's side: input 0 with a pending norm is replaced by the computed norm (kept in
+// `store`) when the consumer is not going to apply it itself.
+void compute_pending_norm(OpContext &c, Tensor *store) {
+    const Tensor &row = c.input(0);
+    const PendingNorm &pn = *row.pending_norm;
+    {
+        std::vector<Tensor *> keep = c.out;
+        c.out = {store};
+        c.alloc_output(0, RMLK_FLOAT, row.shape);
+        c.out = keep;
+    }
+    const int64_t cols = row.shape.back();
+    check_status(rmlk_hip_rmsnorm(c.stream, RMLK_FLOAT, row.numel() / cols, cols, row.data(), pn.gamma.data(),
+                                  pn.eps, pn.reciprocal, store->data()),
+                 "rmlk.RMSNorm (deferred)");
+    c.in[0] = store;
 }
 
 // The Unsqueeze -> Expand -> Reshape chain folded into an attention product must repeat every KV
@@ -956,6 +1024,10 @@ void op_fused_rmsnorm(OpContext &c) {
         // gamma broadcasts along the rows only: [cols] or [1, .., 1, cols]
         ok = gamma.rank() >= 1 && gamma.rank() <= rank && gamma.shape.back() == x.shape.back() &&
              gamma.numel() == x.shape.back();
+    }
+    if (ok && may_defer_norm(c, x, gamma)) {
+        defer_norm(c, 0, x, gamma);
+        return;
     }
     if (ok) {
         const int64_t cols = x.shape.back(), rows = x.numel() / cols;
@@ -1278,6 +1350,17 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
     if (ok && a.numel() == w.shape[0] && c.has_input(4)) {
         // one row: the product over the K-contiguous copy (no combine launch), then Add + norm
         const int64_t k = w.shape[0], n = w.shape[1];
+        if (may_defer_norm(c, res, gamma)) {
+            // the product with the residual added is the row; the norm is left to the product
+            // that reads it
+            Tensor &sum = c.alloc_output(0, RMLK_FLOAT, res.shape);
+            if (took_fast_path(rmlk_hip_gemv_kmajor_add(c.stream, RMLK_FLOAT, n, k, a.data(), c.input(4).data(), k,
+                                                        res.data(), sum.data()),
+                               "rmlk.MatMulAddRMSNorm")) {
+                defer_norm(c, 1, sum, gamma);
+                return;
+            }
+        }
         float *prod = static_cast<float *>(c.scratch(static_cast<size_t>(n) * sizeof(float)));
         if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, n, k, a.data(), c.input(4).data(), k, prod),
                            "rmlk.MatMulAddRMSNorm")) {
@@ -1317,17 +1400,33 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
 // MatMul(a, W) with constant 2-D W: a one-row input reads the K-contiguous copy of W (no split-K,
 // no combine launch); anything else is the plain MatMul.
 void op_fused_matmul_const(OpContext &c) {
-    const Tensor &a = c.input(0), &w = c.input(1), &wt = c.input(2);
-    if (a.dtype == RMLK_FLOAT && a.rank() >= 1 && w.rank() == 2 && a.shape.back() == w.shape[0] &&
-        a.numel() == w.shape[0] && w.shape[0] > 0) {
+    const Tensor &w = c.input(1), &wt = c.input(2);
+    Tensor normed;   // of a row whose norm was left to this node and that it cannot apply itself
+    const bool one_row = [&] {
+        const Tensor &a = c.input(0);
+        return a.dtype == RMLK_FLOAT && a.rank() >= 1 && w.rank() == 2 && a.shape.back() == w.shape[0] &&
+               a.numel() == w.shape[0] && w.shape[0] > 0;
+    }();
+    if (one_row) {
+        const Tensor &a = c.input(0);
         std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
         shape.push_back(w.shape[1]);
         Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
-        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, w.shape[1], w.shape[0], a.data(), wt.data(),
-                                           w.shape[0], y.data()),
+        if (a.pending_norm) {
+            const PendingNorm &pn = *a.pending_norm;
+            if (took_fast_path(rmlk_hip_gemv_kmajor_normed(c.stream, RMLK_FLOAT, w.shape[1], w.shape[0], a.data(),
+                                                           pn.gamma.data(), pn.eps, pn.reciprocal, wt.data(),
+                                                           w.shape[0], y.data()),
+                               "rmlk.MatMulConst"))
+                return;
+            compute_pending_norm(c, &normed);
+        }
+        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, w.shape[1], w.shape[0], c.input(0).data(),
+                                                wt.data(), w.shape[0], y.data()),
                            "rmlk.MatMulConst"))
             return;
     }
+    if (c.input(0).pending_norm) compute_pending_norm(c, &normed);
     run_body(c);
 }
 
@@ -1346,9 +1445,29 @@ bool gemv_partials(OpContext &c, const Tensor &a, const Tensor &w, const void **
 }
 
 void op_fused_matmul_group_swiglu(OpContext &c) {
-    const Tensor &a = c.input(0), &w = c.input(1);
+    const Tensor &w = c.input(1);
     const std::vector<int64_t> widths = c.attr_ints("widths");
     const int64_t k = w.shape[0];
+    Tensor normed;   // of a row whose norm was left to this node and that it cannot apply itself
+    if (c.input(0).pending_norm) {
+        const Tensor &row = c.input(0);
+        const PendingNorm &pn = *row.pending_norm;
+        if (row.dtype == RMLK_FLOAT && row.rank() >= 1 && row.shape.back() == k && row.numel() == k &&
+            widths.size() == 2 && widths[0] == widths[1] && c.has_input(2)) {
+            const int64_t n = widths[0];
+            const bool gate_first = c.attr_int("gate_first", 1) != 0;
+            std::vector<int64_t> shape(row.shape.begin(), row.shape.end() - 1);
+            shape.push_back(n);
+            Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
+            if (took_fast_path(rmlk_hip_gemv_kmajor_swiglu_normed(
+                                   c.stream, RMLK_FLOAT, n, k, row.data(), pn.gamma.data(), pn.eps, pn.reciprocal,
+                                   c.input(2).data(), k, gate_first ? 0 : n, gate_first ? n : 0, y.data()),
+                               "rmlk.MatMulGroupSwiGLU"))
+                return;
+        }
+        compute_pending_norm(c, &normed);
+    }
+    const Tensor &a = c.input(0);
     const bool ok = a.dtype == RMLK_FLOAT && a.rank() >= 1 && a.shape.back() == k && a.numel() == k &&
                     widths.size() == 2 && widths[0] == widths[1];
     const bool same_width = a.dtype == RMLK_FLOAT && a.rank() >= 1 && a.shape.back() == k && k > 0 &&
@@ -1396,8 +1515,15 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
 
 // MatMul(a, W_i) for every member of a group, W_i being column blocks of one joint matrix.
 void op_fused_matmul_group(OpContext &c) {
-    const Tensor &a = c.input(0), &w = c.input(1);
+    const Tensor &w = c.input(1);
     const std::vector<int64_t> widths = c.attr_ints("widths");
+    Tensor normed;   // of a row whose norm was left to this node and that it cannot apply itself
+    std::shared_ptr<const PendingNorm> pending = c.input(0).pending_norm;
+    if (pending && !(c.has_input(2) && c.input(0).numel() == w.shape[0])) {
+        compute_pending_norm(c, &normed);
+        pending.reset();
+    }
+    const Tensor &a = c.input(0);
     require_float(a.dtype);
     if (a.rank() == 0) fail_op("ZeroRank");
     const int64_t k = w.shape[0], total = w.shape[1];
@@ -1412,8 +1538,8 @@ void op_fused_matmul_group(OpContext &c) {
     auto run = [&](int64_t n, const void *b, void *out, int64_t ldc) {
         const size_t ws_bytes = rmlk_hip_matmul_workspace_size(RMLK_FLOAT, 1, m, n, k);
         void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
-        check_status(rmlk_hip_matmul(c.stream, RMLK_FLOAT, 1, m, n, k, a.data(), k, 0, 0, b, total, 0, 0,
-                                     out, ldc, 0, ws, ws_bytes),
+        check_status(rmlk_hip_matmul(c.stream, RMLK_FLOAT, 1, m, n, k, c.input(0).data(), k, 0, 0, b, total, 0,
+                                     0, out, ldc, 0, ws, ws_bytes),
                      "rmlk.MatMulGroup");
     };
     if (m == 1) {
@@ -1426,9 +1552,20 @@ void op_fused_matmul_group(OpContext &c) {
             c.out = keep;
         }
         // (over its K-contiguous copy when there is one: no split-K, no combine launch)
-        if (!(c.has_input(2) && took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, total, k, a.data(),
-                                                                c.input(2).data(), k, row.data()),
-                                               "rmlk.MatMulGroup")))
+        bool done = false;
+        if (pending) {
+            done = took_fast_path(rmlk_hip_gemv_kmajor_normed(c.stream, RMLK_FLOAT, total, k, a.data(),
+                                                              pending->gamma.data(), pending->eps,
+                                                              pending->reciprocal, c.input(2).data(), k,
+                                                              row.data()),
+                                  "rmlk.MatMulGroup");
+            if (!done) compute_pending_norm(c, &normed);   // `run` reads input 0 through the context
+        }
+        const Tensor &a1 = c.input(0);
+        if (!done && !(c.has_input(2) &&
+                       took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, total, k, a1.data(),
+                                                           c.input(2).data(), k, row.data()),
+                                      "rmlk.MatMulGroup")))
             run(total, w.data(), row.data(), total);
         int64_t off = 0;
         for (size_t i = 0; i < widths.size(); ++i) {
@@ -1490,6 +1627,7 @@ int fuse_patterns(Session &s) {
     formed += m.form_matmul_groups();
     formed += m.form_splitk_epilogues();
     formed += m.form_const_matmuls();
+    if (formed) m.mark_deferred_norms();   // an attribute on existing fused nodes, not a node of its own
     if (!formed) return 0;
     std::vector<Node> kept;
     kept.reserve(m.g.nodes.size());

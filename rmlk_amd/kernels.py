@@ -236,6 +236,27 @@ def gemv_kmajor_swiglu(x, wt, y, n: int, k: int, gate_row: int, up_row: int) -> 
                                        up_row, _ptr(y)), "rmlk_hip_gemv_kmajor_swiglu")
 
 
+def gemv_kmajor_add(x, wt, residual, y, n: int, k: int) -> None:
+    """y = x . wt^T + residual (K-contiguous weights, one launch)."""
+    check(lib().rmlk_hip_gemv_kmajor_add(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(wt), k, _ptr(residual),
+                                         _ptr(y)), "rmlk_hip_gemv_kmajor_add")
+
+
+def gemv_kmajor_normed(x, gamma, wt, y, n: int, k: int, eps: float, reciprocal_form: bool = False) -> None:
+    """y = (RMSNorm(x) * gamma) . wt^T, the normalised row never stored."""
+    check(lib().rmlk_hip_gemv_kmajor_normed(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(gamma), eps,
+                                            int(reciprocal_form), _ptr(wt), k, _ptr(y)),
+          "rmlk_hip_gemv_kmajor_normed")
+
+
+def gemv_kmajor_swiglu_normed(x, gamma, wt, y, n: int, k: int, gate_row: int, up_row: int, eps: float,
+                              reciprocal_form: bool = False) -> None:
+    """gemv_kmajor_swiglu over RMSNorm(x) * gamma."""
+    check(lib().rmlk_hip_gemv_kmajor_swiglu_normed(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(gamma), eps,
+                                                   int(reciprocal_form), _ptr(wt), k, gate_row, up_row,
+                                                   _ptr(y)), "rmlk_hip_gemv_kmajor_swiglu_normed")
+
+
 def matmul_grouped(a, b, outs, m: int, k: int, widths, workspace=None) -> None:
     """outs[i] = a[m, k] . (the next widths[i] columns of the row-major joint matrix b)."""
     n = len(widths)

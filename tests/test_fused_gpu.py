@@ -1088,6 +1088,37 @@ def test_one_row_product_over_k_contiguous_weights(device, n, k):
     assert_close(to_np(got), exp.astype(np.float32), rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("n,k,recip", [(3072, 2048, False), (128256, 2048, True), (70, 132, False),
+                                       (512, 8192, True), (40, 8, False), (64, 1024, False)])
+def test_one_row_products_over_a_row_normalised_on_the_fly(device, n, k, recip):
+    """The K-major one-row products over RMSNorm(x) * gamma without storing the normalised row, and
+    with a residual added to the result: bit for bit what the norm kernel, the product kernel and
+    an Add give one after the other."""
+    import torch
+    kk = _k()
+    rng = np.random.default_rng(n + k)
+    x = to_dev(rng.standard_normal((k,), dtype=np.float32) * np.float32(3.0), device)
+    gamma = to_dev(rng.uniform(0.5, 1.5, size=(k,)).astype(np.float32), device)
+    wt = to_dev(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.05), device)
+    res = to_dev(rng.standard_normal((n,), dtype=np.float32), device)
+    normed, exp, got = torch.empty(k, device=device), torch.empty(n, device=device), torch.empty(n, device=device)
+    kk.rmsnorm(x, gamma, normed, 1, k, 1e-5, recip)
+    kk.gemv_kmajor(normed, wt, exp, n, k)
+    kk.gemv_kmajor_normed(x, gamma, wt, got, n, k, 1e-5, recip)
+    assert_exact(to_np(got), to_np(exp))
+    # residual epilogue
+    plain, summed = torch.empty(n, device=device), torch.empty(n, device=device)
+    kk.gemv_kmajor(x, wt, plain, n, k)
+    kk.binary(kk.ADD, plain, res, summed, [n], [1], [1])
+    kk.gemv_kmajor_add(x, wt, res, got, n, k)
+    assert_exact(to_np(got), to_np(summed))
+    if n % 2 == 0:
+        half = n // 2
+        kk.gemv_kmajor_swiglu(normed, wt, exp[:half], half, k, 0, half)
+        kk.gemv_kmajor_swiglu_normed(x, gamma, wt, got[:half], half, k, 0, half, 1e-5, recip)
+        assert_exact(to_np(got[:half]), to_np(exp[:half]))
+
+
 @pytest.mark.parametrize("n,k,gate_first", [(8192, 2048, True), (512, 256, False), (7, 64, True)])
 def test_one_row_gate_up_swiglu_over_k_contiguous_weights(device, n, k, gate_first):
     import torch
