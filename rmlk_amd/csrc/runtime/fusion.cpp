@@ -914,6 +914,7 @@ bool took_fast_path(int32_t st, const char *what) {
 // carries the norm's parameters (Tensor::pending_norm), and the product's kernel normalises the
 // row while it loads it (rmlk_hip_gemv_kmajor_normed). One launch less per norm of a decode step.
 constexpr int64_t kMaxDeferredNormCols = 8192;   // what the product kernels accept
+constexpr int64_t kMaxDeferredNormWidth = 16384; // output columns up to which a product applies the norm
 // 0: every norm runs as its own launch (to compare)
 #ifndef RMLK_DEFER_NORM
 #define RMLK_DEFER_NORM 1
@@ -1412,15 +1413,17 @@ void op_fused_matmul_const(OpContext &c) {
         std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
         shape.push_back(w.shape[1]);
         Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
-        if (a.pending_norm) {
+        // (a very wide product -- the lm-head -- has thousands of blocks that would each normalise
+        // the row: there the separate norm launch is cheaper)
+        if (a.pending_norm && w.shape[1] < kMaxDeferredNormWidth) {
             const PendingNorm &pn = *a.pending_norm;
             if (took_fast_path(rmlk_hip_gemv_kmajor_normed(c.stream, RMLK_FLOAT, w.shape[1], w.shape[0], a.data(),
                                                            pn.gamma.data(), pn.eps, pn.reciprocal, wt.data(),
                                                            w.shape[0], y.data()),
                                "rmlk.MatMulConst"))
                 return;
-            compute_pending_norm(c, &normed);
         }
+        if (c.input(0).pending_norm) compute_pending_norm(c, &normed);
         if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, w.shape[1], w.shape[0], c.input(0).data(),
                                                 wt.data(), w.shape[0], y.data()),
                            "rmlk.MatMulConst"))
@@ -1519,7 +1522,7 @@ void op_fused_matmul_group(OpContext &c) {
     const std::vector<int64_t> widths = c.attr_ints("widths");
     Tensor normed;   // of a row whose norm was left to this node and that it cannot apply itself
     std::shared_ptr<const PendingNorm> pending = c.input(0).pending_norm;
-    if (pending && !(c.has_input(2) && c.input(0).numel() == w.shape[0])) {
+    if (pending && !(c.has_input(2) && c.input(0).numel() == w.shape[0] && w.shape[1] < kMaxDeferredNormWidth)) {
         compute_pending_norm(c, &normed);
         pending.reset();
     }

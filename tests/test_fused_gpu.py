@@ -367,6 +367,48 @@ def _rmsnorm_nodes(g, x, gamma, out, recip=False, axis=-1, expose_mean=False):
         g.output("mean")
 
 
+@pytest.mark.parametrize("rows,k,n,recip", [
+    (1, 256, 96, False),       # one row: the norm is left to the product's kernel
+    (1, 256, 96, True),
+    (1, 64, 20000, False),     # very wide product: the norm is computed first, by its own launch
+    (1, 6, 8, False),          # row length no multiple of 4: nothing is deferred
+    (3, 256, 96, False),       # several rows: nothing is deferred
+])
+def test_norm_feeding_one_product_over_constant_weights(device, rows, k, n, recip):
+    """RMSNorm -> MatMul(constant W) where only the product reads the normalised row: same bits as
+    the session without fusion up to the norm's own last-place differences, and the oracle's values."""
+    from oracle import graph as og
+    g = _builder()
+    g.input("x", np.float32, [1, rows, k])
+    rng = np.random.default_rng(k + n)
+    g.constant("gamma", rng.uniform(0.5, 1.5, size=(k,)).astype(np.float32))
+    g.constant("w", (rng.standard_normal((k, n), dtype=np.float32) * np.float32(0.05)))
+    g.constant("two", np.array(2.0, np.float32))
+    g.constant("eps", np.array(1e-5, np.float32))
+    g.op("Pow", ["x", "two"], ["sq"])
+    g.op("ReduceMean", ["sq"], ["mean"]).attr("axes", [-1]).attr("keepdims", 1)
+    g.op("Add", ["mean", "eps"], ["var"])
+    g.op("Sqrt", ["var"], ["rms"])
+    if recip:
+        g.constant("one", np.array(1.0, np.float32))
+        g.op("Div", ["one", "rms"], ["inv"])
+        g.op("Mul", ["x", "inv"], ["normed"])
+    else:
+        g.op("Div", ["x", "rms"], ["normed"])
+    g.op("Mul", ["gamma", "normed"], ["h"])
+    g.op("MatMul", ["h", "w"], ["y"])
+    g.output("y")
+    feeds = {"x": rng.standard_normal((1, rows, k), dtype=np.float32) * np.float32(2.0)}
+    a, b, nf, ops = _run_both(g.build(), feeds)
+    if k % 4 == 0:
+        assert nf == 2 and ops == ["rmlk.RMSNorm", "rmlk.MatMulConst"]
+    else:   # no K-contiguous copy of such weights: the product stays a MatMul
+        assert nf == 1 and ops == ["rmlk.RMSNorm", "MatMul"]
+    _same(a, b, loose={"y"})
+    exp = og.run_graph(g.build(), feeds)
+    assert_close(a["y"], exp["y"], rtol=1e-4, atol=1e-5)
+
+
 @pytest.mark.parametrize("shape,recip,n_fused", [
     ([2, 5, 64], False, 1), ([2, 5, 64], True, 1),
     ([3, 6], False, 1),            # cols % 4 != 0: the node is formed, its body runs
