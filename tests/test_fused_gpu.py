@@ -1161,6 +1161,31 @@ def test_one_row_products_over_a_row_normalised_on_the_fly(device, n, k, recip):
         assert_exact(to_np(got[:half]), to_np(exp[:half]))
 
 
+def test_one_row_products_over_a_normalised_row_decline_what_they_do_not_cover(device):
+    import torch
+    from rmlk_amd import RmlkError
+    kk = _k()
+    n, k = 8, 16
+    x = torch.ones(k + 4, device=device)
+    wt = torch.ones(n * k, device=device)
+    gamma = torch.ones(k + 4, device=device)
+    y = torch.empty(n, device=device)
+    kk.gemv_kmajor_normed(x, gamma, wt, y, 0, k, 1e-5)                      # nothing to do
+    with pytest.raises(RmlkError):                                          # row longer than a block normalises
+        big = torch.ones(16384, device=device)
+        kk.gemv_kmajor_normed(big, big, torch.ones(4 * 16384, device=device), y[:4], 4, 16384, 1e-5)
+    with pytest.raises(RmlkError):                                          # K no multiple of 4
+        kk.gemv_kmajor_normed(x, gamma, wt, y, n, 14, 1e-5)
+    with pytest.raises(RmlkError):                                          # x not 16-byte aligned
+        kk.gemv_kmajor_normed(x[1:], gamma, wt, y, n, k, 1e-5)
+    with pytest.raises(RmlkError):                                          # gamma not 16-byte aligned
+        kk.gemv_kmajor_normed(x, gamma[1:], wt, y, n, k, 1e-5)
+    with pytest.raises(RmlkError):
+        kk.gemv_kmajor_swiglu_normed(x, gamma[1:], wt, y, n // 2, k, 0, n // 2, 1e-5)
+    with pytest.raises(RmlkError):                                          # x not 16-byte aligned
+        kk.gemv_kmajor_add(x[1:], wt, y, y, n, k)
+
+
 @pytest.mark.parametrize("n,k,gate_first", [(8192, 2048, True), (512, 256, False), (7, 64, True)])
 def test_one_row_gate_up_swiglu_over_k_contiguous_weights(device, n, k, gate_first):
     import torch
