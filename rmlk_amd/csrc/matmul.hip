@@ -1139,9 +1139,13 @@ struct TileChoice {
 #ifndef RMLK_GEMM_SPLIT_TARGET
 #define RMLK_GEMM_SPLIT_TARGET 1
 #endif
+// 0: split-K products keep 128 x 128 tiles (to compare)
+#ifndef RMLK_GEMM_NARROW_SPLIT
+#define RMLK_GEMM_NARROW_SPLIT 1
+#endif
 
-// allow_wide: the 128 x 192 tile may be chosen (it exists for the direct-to-LDS kernel only; a caller
-// whose operands do not qualify asks again without it).
+// allow_wide: the 128 x 192 and 128 x 64 tiles may be chosen (they exist for the direct-to-LDS kernel
+// only; a caller whose operands do not qualify asks again without it).
 inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k, bool allow_wide = true) {
     TileChoice t;
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch; };
@@ -1202,6 +1206,13 @@ inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k, b
             t.k_per_split = kps_w;
         }
     }
+#if RMLK_GEMM_NARROW_SPLIT
+    // split-K products whose 128 x 128 tiles give one block per CU: 128 x 64 tiles with the same
+    // split put two or three blocks on a CU, which overlap each other's first stage and epilogue
+    if (allow_wide && t.bm == 128 && t.bn == 128 && t.bk == 32 && t.splits > 1 && n % 64 == 0 &&
+        tiles(128, 128) * t.splits <= kNumCU)
+        t.bn = 64;
+#endif
     return t;
 }
 
@@ -1284,7 +1295,7 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
                k % c.k_per_split == 0 && (trans_b || n % 4 == 0) && lda < (1ll << 21) && ldb < (1ll << 21);
     };
     TileChoice t = choose_tiles(batch, m, n, k);
-    if (t.bn == 192 && !direct_ok(t)) t = choose_tiles(batch, m, n, k, false);
+    if ((t.bn == 192 || (t.bm == 128 && t.bn == 64)) && !direct_ok(t)) t = choose_tiles(batch, m, n, k, false);
     GemmArgs g{};
     g.a = pa;
     g.b = pb;
@@ -1354,6 +1365,7 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
     }
     if (direct && t.bm == 256) st = RMLK_DIRECT(256, 64, 64, 64);
     else if (direct && t.bn == 192) st = RMLK_DIRECT(128, 192, 64, 96);
+    else if (direct && t.bm == 128 && t.bn == 64) st = RMLK_DIRECT(128, 64, 64, 32);
     else if (direct && t.bm == 128) st = RMLK_DIRECT(128, 128, 64, 64);
     else if (direct) st = RMLK_DIRECT(64, 64, 32, 32);
     else if (t.bm == 256) st = RMLK_LAUNCH(256, 64, 64, 64);
@@ -1474,7 +1486,7 @@ extern "C" int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_
             return c.bk == 32 && k % 4 == 0 && n % 4 == 0 && c.k_per_split % c.bk == 0 &&
                    k % c.k_per_split == 0;
         };
-        if (t.bn == 192 && !direct_ok(t)) t = choose_tiles(batch, m, n, k, false);
+        if ((t.bn == 192 || (t.bm == 128 && t.bn == 64)) && !direct_ok(t)) t = choose_tiles(batch, m, n, k, false);
         const bool direct = direct_ok(t);
         snprintf(tmp, sizeof(tmp), "mfma%dx%dx%d%s splitk=%d", t.bm, t.bn, t.bk,
                  direct ? " direct" : "", t.splits);
