@@ -232,6 +232,27 @@ __device__ __forceinline__ void static_for(F &&f) {
     }
 }
 
+// Streaming (non-temporal) load of a vector of 4, 8 or n * 16 bytes, for data a kernel reads once.
+// It pays where measured (dense float operands of the element-wise kernels, the rows of Softmax)
+// and costs elsewhere (SwiGLU -8 %, Trilu -4 %, copies and 8-byte elements), so it is not a default.
+typedef uint32_t ew_u32x4 __attribute__((ext_vector_type(4)));
+template <typename V>
+__device__ __forceinline__ V nt_load(const V *p) {
+    V out;
+    if constexpr (sizeof(V) % 16 == 0) {
+#pragma unroll
+        for (size_t i = 0; i < sizeof(V) / 16; ++i)
+            reinterpret_cast<ew_u32x4 *>(&out)[i] =
+                __builtin_nontemporal_load(reinterpret_cast<const ew_u32x4 *>(p) + i);
+    } else if constexpr (sizeof(V) == 8) {
+        *reinterpret_cast<uint64_t *>(&out) = __builtin_nontemporal_load(reinterpret_cast<const uint64_t *>(p));
+    } else if constexpr (sizeof(V) == 4) {
+        *reinterpret_cast<uint32_t *>(&out) = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p));
+    } else {
+        out = *p;
+    }
+    return out;
+}
 // Grid size for a grid-stride kernel: enough blocks to cover `work` items, capped so that a few
 // waves per SIMD stay resident on all 256 CUs.
 inline unsigned grid_for(int64_t work, int block, int max_blocks_per_cu = 8) {

@@ -36,11 +36,11 @@ __device__ __forceinline__ void load_vec(const T *p, bool bcast, T (&r)[kEwVec])
         for (int j = 0; j < kEwVec; ++j) r[j] = s;
     } else {
         using V = Vec<T, kEwVec>;
-#ifdef RMLK_NT_LOAD
-        V v = __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
-#else
-        V v = *reinterpret_cast<const V *>(p);
-#endif
+        // Dense operands are read once: streaming loads for element sizes up to 4 bytes (two dense
+        // 256 MiB float inputs: 112 -> 96 us; 8-byte elements measured slower that way, 218 -> 238 us)
+        V v;
+        if constexpr (sizeof(T) <= 4) v = nt_load(reinterpret_cast<const V *>(p));
+        else v = *reinterpret_cast<const V *>(p);
 #pragma unroll
         for (int j = 0; j < kEwVec; ++j) r[j] = v.v[j];
     }
@@ -52,11 +52,7 @@ __device__ __forceinline__ void store_vec(T *p, const T (&r)[kEwVec]) {
     V v;
 #pragma unroll
     for (int j = 0; j < kEwVec; ++j) v.v[j] = r[j];
-#ifdef RMLK_NT_STORE
-    __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
-#else
-    *reinterpret_cast<V *>(p) = v;
-#endif
+    *reinterpret_cast<V *>(p) = v;   // (results are usually read next: ordinary stores)
 }
 
 // ---- two inputs ------------------------------------------------------------------------------
