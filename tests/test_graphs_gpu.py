@@ -239,6 +239,48 @@ def test_llama_other_widths_scatter_style_vs_oracle(device, heads, kv_heads, hea
     inst.close()
 
 
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_llama_shapes_with_and_without_fusion(device, seed):
+    """Llama-shaped graphs of random widths, head counts, sequence and cache lengths, both cache
+    styles: the session with pattern fusion agrees with the one-kernel-per-node session, and gives
+    the same bits when it runs again on recycled buffers."""
+    graphs, runtime = _rt()
+    rng = np.random.default_rng(seed)
+    for _ in range(8):
+        head_dim = int(rng.choice([4, 8, 16, 64, 64, 128]))
+        kv_heads = int(rng.choice([1, 2, 3, 4]))
+        heads = kv_heads * int(rng.choice([1, 2, 4, 5]))
+        hidden = heads * head_dim
+        if hidden > 2048:
+            continue
+        vocab = int(rng.choice([50, 300, 1000]))
+        style = str(rng.choice(["scatter", "concat"]))
+        seq = int(rng.choice([1, 2, 3, 7, 16, 33, 64, 70, 130]))
+        max_len = -(-(seq + int(rng.integers(1, 40))) // 4) * 4
+        cfg = graphs.LlamaConfig(layers=int(rng.choice([1, 2])), hidden=hidden, heads=heads, kv_heads=kv_heads,
+                                 head_dim=head_dim, ffn=int(rng.choice([64, 100, 256, 520])), vocab=vocab)
+        case = f"{cfg} {style} seq={seq} max_len={max_len}"
+        if style == "scatter":
+            graph = graphs.llama_graph(cfg, seed=seed, style="scatter", max_len=max_len)
+            feeds = {"input_ids": rng.integers(0, vocab, size=(1, seq)).astype(np.int64),
+                     "position_ids": np.arange(seq, dtype=np.int64).reshape(1, seq)}
+            for l in range(cfg.layers):
+                for kv in ("key", "value"):
+                    feeds[f"cache.{l}.{kv}"] = (rng.standard_normal((1, kv_heads, max_len, head_dim),
+                                                                    dtype=np.float32) * np.float32(0.1))
+        else:
+            graph = graphs.llama_graph(cfg, seed=seed, style="concat")
+            feeds = graphs.llama_concat_inputs(cfg, rng.integers(0, vocab, size=seq), None, 0)
+        fused = runtime.Builder.from_graph(graph).build(fuse=True)
+        plain = runtime.Builder.from_graph(graph).build(fuse=False)
+        a, b, again = fused.run(feeds), plain.run(feeds), fused.run(feeds)
+        for name in a:
+            np.testing.assert_allclose(a[name], b[name], rtol=2e-3, atol=2e-4, err_msg=f"{name} of {case}")
+            assert np.array_equal(a[name], again[name], equal_nan=True), f"{name} of {case} is not repeatable"
+        fused.close()
+        plain.close()
+
+
 def test_config5_kv_stress_small_vs_oracle(device):
     graphs, runtime = _rt()
     graph, feeds = graphs.kv_stress_graph(seed=5, length=256, vocab=1000, hidden=128,
