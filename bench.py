@@ -37,10 +37,10 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # combine kernel or the norm kernel) moves is not included.
 PMC_TRAFFIC_KIB = {
     (1, 512, 3072, 2048): (32997, 24576),                 # q/k/v (128 x 192 tiles), split-K 4
-    (1, 512, 2048, 2048): (24719, 16384),                 # o, split-K 4
-    (1, 512, 2048, 8192): (98476, 16384),                 # down, split-K 4
-    (1, 512, 16384, 2048, "swiglu"): (164057, 16384),     # gate/up with the SwiGLU epilogue
-    (1, 512, 128256, 2048): (1534894, 256512),            # lm-head
+    (1, 512, 2048, 2048): (24677, 16384),                 # o (128 x 64 tiles), split-K 4
+    (1, 512, 2048, 8192): (99094, 16384),                 # down (128 x 64 tiles), split-K 4
+    (1, 512, 16384, 2048, "swiglu"): (164044, 16384),     # gate/up with the SwiGLU epilogue
+    (1, 512, 128256, 2048): (1522548, 256512),            # lm-head
 }
 
 
