@@ -39,7 +39,9 @@ typedef enum rmlk_status {
     RMLK_ERR_SIZE_MISMATCH = -4,   /* shapes / lengths disagree */
     RMLK_ERR_INVALID_ARGUMENT = -5,/* bad axis, perm, step 0, negative dim ... */
     RMLK_ERR_WORKSPACE = -6,       /* workspace smaller than rmlk_hip_matmul_workspace_size says */
-    RMLK_ERR_TOO_LARGE = -7        /* more elements than the kernels index (>= 2^62) */
+    RMLK_ERR_TOO_LARGE = -7,       /* more elements than the kernels index (>= 2^62) */
+    RMLK_ERR_SCRATCH_LIMIT = -8    /* rmlk_hip_matmul_noalloc: the problem needs more scratch than the
+                                      library's fixed array holds */
 } rmlk_status;
 
 /* Element types. Values are the ONNX TensorProto.DataType numbers the reference maps its
@@ -159,6 +161,21 @@ size_t rmlk_hip_matmul_workspace_size(int32_t dtype, int64_t batch, int64_t m, i
  * Writes at most `size` bytes including the terminator; returns the length needed. */
 int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_t m, int64_t n, int64_t k,
                                  char *buf, int32_t size);
+
+/* rmlk_hip_matmul for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same
+ * arguments and results as rmlk_hip_matmul (bit for bit) without the workspace: the split-K partials
+ * go to a fixed device array of RMLK_HIP_MATMUL_NOALLOC_SCRATCH_BYTES that is part of the library's
+ * code object (every GPU the library runs on holds its copy until the process ends). A problem whose
+ * rmlk_hip_matmul_workspace_size exceeds that returns RMLK_ERR_SCRATCH_LIMIT and launches nothing.
+ * The call allocates nothing and frees nothing. All calls on one GPU share the array: calls that may
+ * overlap in time on one GPU (different streams, different threads) race on it and must be ordered
+ * by the caller; calls on one stream are ordered by the stream. */
+#define RMLK_HIP_MATMUL_NOALLOC_SCRATCH_BYTES (32 << 20)
+int32_t rmlk_hip_matmul_noalloc(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t m,
+                                int64_t n, int64_t k, const void *a, int64_t lda, int64_t stride_a,
+                                int32_t trans_a, const void *b, int64_t ldb, int64_t stride_b,
+                                int32_t trans_b, void *c, int64_t ldc, int64_t stride_c);
 
 /* Transpose: out = permute(in, perm); out.shape[d] = in_shape[perm[d]]. Any 1/2/4/8-byte dtype.
  * ref: cuda/src/kernels/transpose.rs:38-80, cuda/src/ptx/headers/transpose_op_macros.cuh:1-25. */

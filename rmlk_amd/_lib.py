@@ -75,6 +75,9 @@ SIGNATURES = {
     "rmlk_hip_matmul": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_void_p,
                                   c_int64, c_int64, c_int32, c_void_p, c_int64, c_int64, c_int32,
                                   c_void_p, c_int64, c_int64, c_void_p, c_size_t]),
+    "rmlk_hip_matmul_noalloc": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_void_p,
+                                          c_int64, c_int64, c_int32, c_void_p, c_int64, c_int64, c_int32,
+                                          c_void_p, c_int64, c_int64]),
     "rmlk_hip_matmul_workspace_size": (c_size_t, [c_int32, c_int64, c_int64, c_int64, c_int64]),
     "rmlk_hip_matmul_describe": (c_int32, [c_int32, c_int64, c_int64, c_int64, c_int64, c_char_p,
                                            c_int32]),

@@ -82,6 +82,7 @@ extern "C" const char *rmlk_hip_status_string(int32_t status) {
         case RMLK_ERR_INVALID_ARGUMENT: return "invalid argument";
         case RMLK_ERR_WORKSPACE: return "workspace too small";
         case RMLK_ERR_TOO_LARGE: return "tensor too large";
+        case RMLK_ERR_SCRATCH_LIMIT: return "problem needs more scratch memory than the no-allocation entry point holds";
         default:
             if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
             return "unknown status";

@@ -16,6 +16,7 @@
 //     global memory straight into LDS (global_load_lds_dwordx4), see gemm_mfma_direct_kernel;
 //   - split-K (grid z) writes partial tiles to the workspace, a second kernel adds them in a
 //     fixed order, so results do not depend on scheduling.
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <type_traits>
@@ -1895,4 +1896,54 @@ extern "C" int32_t rmlk_hip_gemv_kmajor_swiglu_normed(rmlk_stream_t stream, int3
     const RowNormArgs norm{static_cast<const float *>(gamma), eps, reciprocal_form};
     if (n > 0 && !gamma) return RMLK_ERR_NULL_POINTER;
     return gemv_kmajor_swiglu_launch(stream, dtype, n, k, x, wt, ldw, gate_row, up_row, &norm, y);
+}
+
+// ---- MatMul for callers that cannot allocate ----------------------------------------------------
+// The split-K partials of rmlk_hip_matmul live in a workspace the caller allocates. A caller under
+// HIP graph capture, in a tight serving loop or in a harness that forbids hipMalloc cannot do that:
+// for them the partials go to a fixed array in device memory that is part of the code object. Every
+// GPU the library runs on holds its own copy of the array, at its own address, until the process ends.
+static __device__ __align__(256) unsigned char scratch[RMLK_HIP_MATMUL_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+// Device address of `scratch` per GPU, looked up on the entry point's first call on that GPU (the
+// array's name is a host-side stand-in in host code, not an address a kernel can use).
+constexpr int kScratchDevices = 64;
+std::atomic<void *> g_scratch_ptr[kScratchDevices];
+
+int32_t scratch_for_current_device(void **out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int32_t>(e);
+    if (dev < 0 || dev >= kScratchDevices) return RMLK_ERR_INVALID_ARGUMENT;
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        // threads that race here all get the same answer for this device
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int32_t>(e);
+        if (!p) return RMLK_ERR_NULL_POINTER;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return RMLK_OK;
+}
+}  // namespace
+
+extern "C" int32_t rmlk_hip_matmul_noalloc(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t m,
+                                           int64_t n, int64_t k, const void *a, int64_t lda,
+                                           int64_t stride_a, int32_t trans_a, const void *b, int64_t ldb,
+                                           int64_t stride_b, int32_t trans_b, void *c, int64_t ldc,
+                                           int64_t stride_c) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (batch < 0 || m < 0 || n < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    const size_t need = rmlk_hip_matmul_workspace_size(dtype, batch, m, n, k);
+    if (need > static_cast<size_t>(RMLK_HIP_MATMUL_NOALLOC_SCRATCH_BYTES)) return RMLK_ERR_SCRATCH_LIMIT;
+    void *ws = nullptr;
+    if (need) {
+        // the partials are written before they are read: nothing in the array has to start at zero
+        const int32_t st = scratch_for_current_device(&ws);
+        if (st) return st;
+    }
+    return rmlk_hip_matmul(stream, dtype, batch, m, n, k, a, lda, stride_a, trans_a, b, ldb, stride_b,
+                           trans_b, c, ldc, stride_c, ws, need);
 }

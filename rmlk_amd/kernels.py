@@ -118,6 +118,16 @@ def matmul(a, b, c, batch, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c,
     check(st, "rmlk_hip_matmul")
 
 
+def matmul_noalloc(a, b, c, batch, m, n, k, lda, ldb, ldc, stride_a, stride_b, stride_c, trans_a=False,
+                   trans_b=False) -> None:
+    """rmlk_hip_matmul with the split-K partials in the library's fixed device array: the call
+    allocates nothing (no counterpart in the reference; for callers that cannot allocate)."""
+    st = lib().rmlk_hip_matmul_noalloc(_stream(), dtype_of(a), batch, m, n, k, _ptr(a), lda, stride_a,
+                                       int(trans_a), _ptr(b), ldb, stride_b, int(trans_b), _ptr(c), ldc,
+                                       stride_c)
+    check(st, "rmlk_hip_matmul_noalloc")
+
+
 def transpose(x, out, in_shape, perm) -> None:
     """ref: cuda/src/kernels/transpose.rs:38-80."""
     arr = (ctypes.c_int64 * len(perm))(*[int(p) for p in perm])
