@@ -46,10 +46,24 @@ extern "C" int32_t rmlk_hip_memcpy_dtod(rmlk_stream_t stream, void *dst, const v
         hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
 }
 
+// Byte fill through the fill kernels (never hipMemsetAsync): safe to record into a HIP graph, where
+// memset nodes have given wrong results on replays after the first. Head and tail bytes go one by one,
+// the 8-byte aligned middle as 64-bit words.
 extern "C" int32_t rmlk_hip_memset(rmlk_stream_t stream, void *dst, int32_t byte, size_t bytes) {
     if (bytes == 0) return RMLK_OK;
     if (!dst) return RMLK_ERR_NULL_POINTER;
-    return static_cast<int32_t>(hipMemsetAsync(dst, byte, bytes, as_stream(stream)));
+    const uint8_t b = static_cast<uint8_t>(byte);
+    uint8_t *p = static_cast<uint8_t *>(dst);
+    size_t head = (8 - reinterpret_cast<uintptr_t>(p) % 8) % 8;
+    if (head > bytes) head = bytes;
+    const size_t words = (bytes - head) / 8;
+    const size_t tail = bytes - head - words * 8;
+    const uint64_t word = 0x0101010101010101ull * b;
+    int32_t st = RMLK_OK;
+    if (head) st = rmlk_hip_fill(stream, RMLK_UINT8, static_cast<int64_t>(head), &b, p);
+    if (!st && words) st = rmlk_hip_fill(stream, RMLK_UINT64, static_cast<int64_t>(words), &word, p + head);
+    if (!st && tail) st = rmlk_hip_fill(stream, RMLK_UINT8, static_cast<int64_t>(tail), &b, p + head + words * 8);
+    return st;
 }
 
 extern "C" int32_t rmlk_hip_stream_sync(rmlk_stream_t stream) {

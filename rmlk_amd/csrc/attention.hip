@@ -68,7 +68,7 @@ struct AttnArgs {
     int32_t len;       // L keys
     int64_t mask_b, mask_h, mask_s;   // element strides of the mask over batch, head, query
     int64_t out_b, out_h, out_s;      // element strides of out over batch, head, query
-    float qscale;      // score scale times log2(e): the softmax runs on base-2 exponents
+    float qscale;      // score scale (folded into the query)
 };
 
 template <int NK>
@@ -189,11 +189,16 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
             }
             __builtin_amdgcn_sched_barrier(0);
         });
+        // The mask is added to the natural-log scores, as the Add node in front of a Softmax adds it,
+        // and only the difference to the running maximum is scaled by log2(e): a mask of the most
+        // negative finite float (what exported graphs use for "hidden") stays finite, so a row with
+        // nothing else visible comes out uniform like the separate kernels' (scaled by log2(e) first
+        // such a mask overflows to -inf and the row turns NaN).
         float t[16];
 #pragma unroll
         for (int a = 0; a < 4; ++a)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) t[4 * a + e] = fmaf(mk[a][e], kLog2e, st[4 * a + e]);
+            for (int e = 0; e < 4; ++e) t[4 * a + e] = st[4 * a + e] + mk[a][e];
         if ((c + 1) * kKeys > g.len) {
             // keys past the end (their rows and mask values were read from valid but unrelated places)
 #pragma unroll
@@ -213,11 +218,11 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
         }
         const float m_new = fmaxf(m_run, mx);
         const float m_safe = m_new == kNegInf ? 0.f : m_new;   // a row with nothing visible so far
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * kLog2e);
         float p[16], psum = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            p[r] = __builtin_amdgcn_exp2f(t[r] - m_safe);
+            p[r] = __builtin_amdgcn_exp2f((t[r] - m_safe) * kLog2e);
             psum += p[r];
         }
         l_run = l_run * alpha + psum;
@@ -281,11 +286,11 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
 #pragma unroll
         for (int j = 0; j < NK - 1; ++j) m_f = fmaxf(m_f, cb[j * kSlot + lane]);
         const float m_safe = m_f == kNegInf ? 0.f : m_f;
-        const float a0 = __builtin_amdgcn_exp2f(m_run - m_safe);
+        const float a0 = __builtin_amdgcn_exp2f((m_run - m_safe) * kLog2e);
         float aj[NK - 1], total = l_run * a0;
 #pragma unroll
         for (int j = 0; j < NK - 1; ++j) {
-            aj[j] = __builtin_amdgcn_exp2f(cb[j * kSlot + lane] - m_safe);
+            aj[j] = __builtin_amdgcn_exp2f((cb[j * kSlot + lane] - m_safe) * kLog2e);
             total += cb[j * kSlot + kWave + lane] * aj[j];
         }
         const float inv = 1.0f / total;   // nothing visible at all: 0 * inf = NaN, as Softmax
@@ -471,7 +476,7 @@ int32_t attention_args(int32_t dtype, int64_t batch, int64_t kv_heads, int64_t r
     g.mask_b = mask_stride->v[0];
     g.mask_h = mask_stride->v[1];
     g.mask_s = mask_stride->v[2];
-    g.qscale = (scale_is_mul ? scale : 1.0f / scale) * kLog2e;
+    g.qscale = scale_is_mul ? scale : 1.0f / scale;
     const int64_t heads = kv_heads * rep;
     if (out_seq_major) {   // [batch, q_len, heads, head_dim]
         g.out_b = q_len * heads * kHeadDim;

@@ -286,8 +286,26 @@ int32_t rmlk_session_set_input(rmlk_session *s, const char *name, int32_t dtype,
         }
         // same shape as before and a buffer of the session's own: refresh it in place, so that a
         // recorded HIP graph keeps reading the address it knows
-        const bool reuse = t.defined() && t.dtype == dtype && t.shape == shape && t.buf &&
-                           t.buf->pool == &ss.pool && !t.buf->donated && t.buf.use_count() <= 2;
+        // only when every owner of the buffer is accounted for. Without a recorded graph that is
+        // the input slot alone: a view of the input that the last run left among the values (a
+        // Reshape of an input as a graph output) must keep the old bytes, so a fresh buffer is
+        // taken. With a recorded graph the owners are the session's values that share the buffer
+        // and the plan's pins of them; the recorded kernels read this address, so it is refreshed
+        // in place (outputs of the last replay that are views of the input then show the new bytes
+        // until the next replay rewrites them). Any other owner drops the plan.
+        bool reuse = t.defined() && t.dtype == dtype && t.shape == shape && t.buf &&
+                     t.buf->pool == &ss.pool && !t.buf->donated;
+        if (reuse) {
+            long expected = 1;
+            if (ss.plan) {
+                expected = 0;
+                for (const Tensor &v : ss.values)
+                    if (v.buf == t.buf) ++expected;
+                for (const Tensor &v : ss.plan->pinned)
+                    if (v.buf == t.buf) ++expected;
+            }
+            reuse = t.buf.use_count() == expected;
+        }
         if (!reuse) {
             if (ss.plan) ss.plan.reset();
             t.reset();

@@ -188,6 +188,16 @@ std::string OpContext::attr_string(const char *name, const std::string &dflt) co
     return a ? a->s : dflt;
 }
 
+// Element types decode_host reads (integers, bool, float, double): only those get host mirrors.
+static bool host_decodable(int32_t dtype) {
+    switch (dtype) {
+        case RMLK_FLOAT: case RMLK_DOUBLE: case RMLK_INT64: case RMLK_UINT64: case RMLK_INT32:
+        case RMLK_UINT32: case RMLK_INT16: case RMLK_UINT16: case RMLK_INT8: case RMLK_UINT8:
+        case RMLK_BOOL: return true;
+        default: return false;
+    }
+}
+
 static HostVal decode_host(int32_t dtype, const uint8_t *p, size_t n) {
     HostVal h;
     switch (dtype) {
@@ -273,7 +283,7 @@ static Tensor upload_initializer(const HostTensor &ht, hipStream_t stream) {
                                  stream),
                   "hipMemcpyAsync H2D (initializer)");
     t.buf = b;
-    if (ht.numel() <= kHostMirrorMax && dtype_size(ht.dtype))
+    if (ht.numel() <= kHostMirrorMax && host_decodable(ht.dtype))
         t.host = std::make_shared<HostVal>(
             decode_host(ht.dtype, ht.data.data(), static_cast<size_t>(ht.numel())));
     return t;

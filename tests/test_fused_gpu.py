@@ -974,6 +974,45 @@ def test_attention_row_with_nothing_visible_is_nan_like_softmax(device):
     assert_close(np.delete(out, 7, axis=2), np.delete(exp, 7, axis=2), rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("s,l", [(64, 128), (200, 264)])
+def test_attention_with_most_negative_finite_mask_matches_separate_kernels(device, s, l):
+    """Exported graphs hide keys with an additive mask of float32's most negative finite value, not
+    -inf. In fp32 `score + that` is that value again, so a row with every key hidden is a uniform
+    average of V in the separate Add / Softmax kernels (finite), not NaN; the one-kernel attention has
+    to agree, also for rows that mix hidden and visible keys."""
+    import torch
+    kk = _k()
+    b, g, rep, d = 1, 2, 2, 64
+    h = g * rep
+    rng = np.random.default_rng(s + l)
+    q_np, k_np, v_np = (rng.standard_normal(sh, dtype=np.float32)
+                        for sh in ((b, h, s, d), (b, g, l, d), (b, g, l, d)))
+    lowest = np.finfo(np.float32).min
+    m_np = np.zeros((1, 1, s, l), dtype=np.float32)
+    qi = np.arange(s)[:, None] + (l - s)
+    m_np[0, 0][np.arange(l)[None, :] > qi] = lowest       # causal
+    m_np[0, 0, 5, :] = lowest                              # a padded row: nothing visible
+    m_np[0, 0, s - 1, :] = lowest
+    m_np[0, 0, 9, : l - 3] = lowest                        # visible keys only in the last chunk
+    q, k, v, m = (to_dev(x, device) for x in (q_np, k_np, v_np, m_np))
+    full, ms = [b, h, s, l], [0, 0, l, 1]
+    got = torch.full((b, h, s, d), float("nan"), device=device)
+    kk.attention(q, k, v, m, got, b, g, rep, s, l, d, ms, 8.0, False)
+    sc = torch.empty(b, h, s, l, device=device)
+    kk.matmul(q, k, sc, b * g, rep * s, l, d, d, d, l, rep * s * d, l * d, rep * s * l, trans_b=True)
+    pr = torch.empty_like(sc)
+    kk.scale_mask_softmax(sc, m, pr, full, ms, 8.0, False)
+    sep = torch.empty(b, h, s, d, device=device)
+    kk.matmul(pr, v, sep, b * g, rep * s, d, l, l, d, d, rep * s * l, l * d, rep * s * d)
+    out, exp = to_np(got), to_np(sep)
+    assert np.isfinite(exp).all() and np.isfinite(out).all()
+    assert_close(out, exp, rtol=1e-4, atol=1e-5)
+    # the rows with nothing visible are the plain average of their KV head's V rows
+    mean_v = np.repeat(v_np.astype(np.float64).mean(axis=2), rep, axis=1).astype(np.float32)
+    for row in (5, s - 1):
+        assert_close(out[:, :, row], mean_v, rtol=1e-4, atol=1e-5)
+
+
 @pytest.mark.parametrize("kw", [dict(d=32), dict(l=130), dict(last_stride=2)])
 def test_attention_declines_what_it_does_not_cover(device, kw):
     import torch

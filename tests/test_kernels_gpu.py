@@ -591,3 +591,33 @@ def test_status_codes(device):
         Dims.of([1] * 9)
     info = k.device_info(0)
     assert info["wavefront_size"] == 64 and "gfx950" in info["arch"]
+
+
+@pytest.mark.parametrize("offset,nbytes", [(0, 4096), (3, 1), (5, 2), (1, 4093), (7, 8), (2, 40)])
+def test_memset_is_a_kernel_fill_and_replays_in_a_graph(device, offset, nbytes):
+    """rmlk_hip_memset fills through kernels, so it can be recorded into a HIP graph: every replay,
+    with eager work in between, gives the eager result (head, aligned middle and tail bytes)."""
+    from rmlk_amd._lib import check, lib
+    buf = torch.zeros(4200, dtype=torch.uint8, device=device)
+    base = buf.data_ptr() + offset
+
+    def fill(byte):
+        check(lib().rmlk_hip_memset(torch.cuda.current_stream().cuda_stream, base, byte, nbytes),
+              "rmlk_hip_memset")
+
+    expected = np.zeros(4200, dtype=np.uint8)
+    expected[offset:offset + nbytes] = 0xAB
+    fill(0xAB)
+    assert_exact(to_np(buf), expected)
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            fill(0x5C)
+    expected[offset:offset + nbytes] = 0x5C
+    for _ in range(3):
+        buf.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_exact(to_np(buf), expected)

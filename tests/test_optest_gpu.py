@@ -223,3 +223,51 @@ def test_session_memory_steady_state(device):
     m1 = inst.memory_stats()
     assert m1["hip_mallocs"] == m0["hip_mallocs"] and m1["pool_bytes"] == m0["pool_bytes"]
     inst.close()
+
+
+def test_small_float16_initializer_builds_and_casts(device):
+    """A float16 constant of a few elements needs no host mirror (nothing reads half floats on the
+    host): the session must build, and Cast must read the constant on the device."""
+    from rmlk_amd.runtime import Builder, GraphBuilder
+    half = np.array([0.5, -2.0, 1024.0], dtype=np.float16)
+    gb = GraphBuilder()
+    gb.input("x", np.float32, [3])
+    gb.constant("h", half)
+    gb.op("Cast", ["h"], ["hf"]).attr("to", 1)
+    gb.op("Add", ["x", "hf"], ["y"])
+    gb.output("y")
+    inst = Builder.from_graph(gb.build()).build()
+    x = np.array([1.0, 2.0, 3.0], dtype=np.float32)
+    got = inst.run({"x": x})["y"]
+    assert_exact(got, x + half.astype(np.float32))
+    inst.close()
+
+
+def test_set_input_keeps_a_view_output_of_the_previous_run(device):
+    """A graph output that is a view of an input (Reshape shares the buffer) must keep the bytes of
+    the run that produced it when the next input is set, with and without a recorded graph."""
+    from rmlk_amd.runtime import Builder, GraphBuilder
+    gb = GraphBuilder()
+    gb.input("x", np.float32, [2, 3])
+    gb.constant("shape", np.array([3, 2], dtype=np.int64))
+    gb.op("Reshape", ["x", "shape"], ["v"])
+    gb.op("Neg", ["x"], ["n"])
+    gb.output("v").output("n")
+    inst = Builder.from_graph(gb.build()).build()
+    a = np.arange(6, dtype=np.float32).reshape(2, 3)
+    b = a + 100
+    inst.set_input("x", a)
+    inst.execute()
+    inst.set_input("x", b)                      # no run yet: the outputs are still those of `a`
+    assert_exact(inst.output("v"), a.reshape(3, 2))
+    assert_exact(inst.output("n"), -a)
+    inst.execute()
+    assert_exact(inst.output("v"), b.reshape(3, 2))
+    # with a recorded graph the input is refreshed in place and the replay gives the new results
+    inst.capture()
+    for arr in (a, b, a):
+        inst.set_input("x", arr)
+        inst.replay()
+        assert_exact(inst.output("v"), arr.reshape(3, 2))
+        assert_exact(inst.output("n"), -arr)
+    inst.close()
