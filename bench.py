@@ -361,21 +361,44 @@ def run_ops_suite(args):
     bs = [torch.randn(32 * 64, device=dev, generator=g) for _ in range(ns)]
     conds = [(torch.rand(n, device=dev, generator=g) < 0.5) for _ in range(ns)]
     dense, bst = [1048576, 32768, 64, 1], [0, 64, 0, 1]
-    reps = args.steps * 10
+    reps = max(100, args.steps * 10)     # launches per recorded graph, rotating over the buffer sets
     results = {}
+    side = torch.cuda.Stream()
 
     def timed(name, fn, nset, bytes_):
-        for i in range(3):
-            fn(i % nset)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for i in range(reps):
-            fn(i % nset)
-        e1.record()
-        torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) / reps * 1e3
-        results[name] = {"us_per_launch_incl_launch_gaps": round(us, 2), "algorithmic_bytes": bytes_}
+        """>= 10 eager warm-up launches, then `reps` launches recorded into ONE HIP graph (so that they
+        run back to back with no host in between), the graph replayed untimed until >= 30 ms of
+        continuous work have passed, then `args.warmup`+... timed replays between one pair of events
+        on the launching stream."""
+        with torch.cuda.stream(side):
+            for i in range(max(10, 2 * nset)):
+                fn(i % nset)
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(reps):
+                    fn(i % nset)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(side)
+            graph.replay()
+            e1.record(side)
+            side.synchronize()
+            first_ms = max(e0.elapsed_time(e1), 1e-3)
+            for _ in range(min(200, int(30.0 / first_ms) + 1)):
+                graph.replay()
+            n_timed = max(3, min(50, int(20.0 / first_ms)))
+            e0.record(side)
+            for _ in range(n_timed):
+                graph.replay()
+            e1.record(side)
+            side.synchronize()
+        us = e0.elapsed_time(e1) / (n_timed * reps) * 1e3
+        results[name] = {"us_per_launch": round(us, 2), "algorithmic_bytes": bytes_,
+                         "tb_per_s": round(bytes_ / us / 1e6, 3),
+                         "frac_of_hbm_peak": round(bytes_ / us / 1e6 / (PEAK_HBM_GBS / 1e3), 3),
+                         "launches_timed": n_timed * reps, "buffer_sets": nset}
+        log(f"[ops] {name}: {us:.2f} us/launch, {bytes_ / us / 1e6:.2f} TB/s")
+        del graph
 
     timed("add", lambda i: k.binary(k.ADD, xs[i], bs[i], ys[i], shp, dense, bst), ns, 2 * n * 4 + 8192)
     timed("mul", lambda i: k.binary(k.MUL, xs[i], bs[i], ys[i], shp, dense, bst), ns, 2 * n * 4 + 8192)
@@ -462,7 +485,9 @@ def run_ops_suite(args):
     i64a = [torch.randint(0, 100, (8192 * 8192,), device=dev, generator=g) for _ in range(2)]
     timed("equal_i64_8192", lambda i: k.binary(k.EQUAL, i64a[i], i64a[1 - i], eq_out, full, dn, dn), 2,
           2 * 8192 * 8192 * 8 + 8192 * 8192)
-    print(json.dumps({"suite": "ops", "note": "per-kernel durations come from rocprofv3 of this command",
+    print(json.dumps({"suite": "ops", "note": "us_per_launch: HIP events around back-to-back launches "
+                      "(replays of a recorded graph of rotating launches), launch gaps included; "
+                      "per-kernel durations come from rocprofv3 --kernel-trace of this command",
                       "results": results}))
 
 

@@ -38,14 +38,6 @@ extern "C" int32_t rmlk_hip_memcpy_dtoh(rmlk_stream_t stream, void *dst, const v
     return static_cast<int32_t>(hipStreamSynchronize(as_stream(stream)));
 }
 
-extern "C" int32_t rmlk_hip_memcpy_dtod(rmlk_stream_t stream, void *dst, const void *src,
-                                        size_t bytes) {
-    if (bytes == 0) return RMLK_OK;
-    if (!dst || !src) return RMLK_ERR_NULL_POINTER;
-    return static_cast<int32_t>(
-        hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
-}
-
 // Byte fill through the fill kernels (never hipMemsetAsync): safe to record into a HIP graph, where
 // memset nodes have given wrong results on replays after the first. Head and tail bytes go one by one,
 // the 8-byte aligned middle as 64-bit words.

@@ -253,6 +253,37 @@ __device__ __forceinline__ V nt_load(const V *p) {
     }
     return out;
 }
+// Streaming (non-temporal) store, the counterpart of nt_load: a large result leaves the chip as it
+// is produced instead of sitting in the L2s until the write-back at the end of the kernel
+// (a 16 MiB + 16 MiB copy: 7.7 -> 6.7 us; 256 MiB + 256 MiB: 95 -> 90 us).
+template <typename V>
+__device__ __forceinline__ void nt_store(V *p, const V &v) {
+    if constexpr (sizeof(V) % 16 == 0) {
+#pragma unroll
+        for (size_t i = 0; i < sizeof(V) / 16; ++i)
+            __builtin_nontemporal_store(reinterpret_cast<const ew_u32x4 *>(&v)[i],
+                                        reinterpret_cast<ew_u32x4 *>(p) + i);
+    } else if constexpr (sizeof(V) == 8) {
+        __builtin_nontemporal_store(*reinterpret_cast<const uint64_t *>(&v), reinterpret_cast<uint64_t *>(p));
+    } else if constexpr (sizeof(V) == 4) {
+        __builtin_nontemporal_store(*reinterpret_cast<const uint32_t *>(&v), reinterpret_cast<uint32_t *>(p));
+    } else {
+        *p = v;
+    }
+}
+
+// Streaming kernels walk their index space in chunks of block x unroll consecutive items: a block
+// takes a chunk, lane t of it the items t, t + block, t + 2 block, ..., so that the accesses a block
+// has in flight cover one contiguous 16 KiB piece of every dense operand (accesses a whole grid
+// apart, the usual grid-stride unrolling, reached 4.3 TB/s on a 256 MiB copy where this reaches 6.0).
+// Grid for `items` items in chunks of `chunk`: one trip up to 32 blocks per compute unit.
+inline unsigned chunk_grid(int64_t items, int chunk) {
+    int64_t need = (items + chunk - 1) / chunk;
+    const int64_t cap = static_cast<int64_t>(256) * 32;
+    if (need < 1) need = 1;
+    return static_cast<unsigned>(need < cap ? need : cap);
+}
+
 // Grid size for a grid-stride kernel: enough blocks to cover `work` items, capped so that a few
 // waves per SIMD stay resident on all 256 CUs.
 inline unsigned grid_for(int64_t work, int block, int max_blocks_per_cu = 8) {

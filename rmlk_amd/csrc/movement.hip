@@ -19,29 +19,46 @@ struct alignas(16) U128 {
 // ---------------------------------------------------------------------------------------------
 // strided N-d copy: plan operand 0 = in, 1 = out
 constexpr int kUnroll = 4;  // independent accesses in flight per lane
+constexpr int kChunk = kBlock * kUnroll;      // units a block takes per trip, consecutive in the output
 
+// Sources are read once and results are not found in a cache by whoever reads them next (the L2s of
+// the eight XCDs are written back at the end of a kernel): streaming loads and stores.
 template <typename U>
+__device__ __forceinline__ void put(U *p, const U &v) {
+    nt_store(p, v);
+}
+
+// REPEATS: the input is read more than once (repeated along some dim, as Expand's): ordinary loads
+template <bool REPEATS, typename U>
+__device__ __forceinline__ U get(const U *p) {
+    if constexpr (REPEATS) return *p;
+    else return nt_load(p);
+}
+
+template <typename U, bool REPEATS>
 __global__ __launch_bounds__(kBlock) void copy_nd_kernel(NdPlan<2> pl, const U *__restrict__ in,
                                                          U *__restrict__ out, uint32_t n) {
-    const uint32_t step = gridDim.x * kBlock;
-    uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-    for (; i + (kUnroll - 1) * step < n; i += step * kUnroll) {
-        U r[kUnroll];
-        int64_t oo[kUnroll];
+    for (uint32_t base = blockIdx.x * kChunk; base < n; base += gridDim.x * kChunk) {
+        const uint32_t i0 = base + threadIdx.x;
+        if (base + kChunk <= n) {
+            U r[kUnroll];
+            int64_t oo[kUnroll];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
-            int64_t offs[2];
-            nd_offsets<2>(pl, i + j * step, offs);
-            r[j] = in[offs[0]];
-            oo[j] = offs[1];
+            for (int j = 0; j < kUnroll; ++j) {
+                int64_t offs[2];
+                nd_offsets<2>(pl, i0 + j * kBlock, offs);
+                r[j] = get<REPEATS>(in + offs[0]);
+                oo[j] = offs[1];
+            }
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j) put(out + oo[j], r[j]);
+        } else {
+            for (uint32_t i = i0; i < n; i += kBlock) {
+                int64_t offs[2];
+                nd_offsets<2>(pl, i, offs);
+                put(out + offs[1], get<REPEATS>(in + offs[0]));
+            }
         }
-#pragma unroll
-        for (int j = 0; j < kUnroll; ++j) out[oo[j]] = r[j];
-    }
-    for (; i < n; i += step) {
-        int64_t offs[2];
-        nd_offsets<2>(pl, i, offs);
-        out[offs[1]] = in[offs[0]];
     }
 }
 
@@ -49,28 +66,37 @@ __global__ __launch_bounds__(kBlock) void copy_nd_kernel(NdPlan<2> pl, const U *
 template <typename U>
 __global__ __launch_bounds__(kBlock) void copy_flat_kernel(const U *__restrict__ in,
                                                            U *__restrict__ out, uint32_t n) {
-    const uint32_t step = gridDim.x * kBlock;
-    uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-    for (; i + (kUnroll - 1) * step < n; i += step * kUnroll) {
-        U r[kUnroll];
+    for (uint32_t base = blockIdx.x * kChunk; base < n; base += gridDim.x * kChunk) {
+        const uint32_t i0 = base + threadIdx.x;
+        if (base + kChunk <= n) {
+            U r[kUnroll];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) r[j] = in[i + j * step];
+            for (int j = 0; j < kUnroll; ++j) r[j] = nt_load(in + i0 + j * kBlock);
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) out[i + j * step] = r[j];
+            for (int j = 0; j < kUnroll; ++j) put(out + i0 + j * kBlock, r[j]);
+        } else {
+            for (uint32_t i = i0; i < n; i += kBlock) put(out + i, nt_load(in + i));
+        }
     }
-    for (; i < n; i += step) out[i] = in[i];
 }
 
 template <typename U>
 int32_t launch_copy_units(hipStream_t s, NdPlan<2> &pl, const void *in, void *out) {
     uint32_t n = static_cast<uint32_t>(pl.numel);
-    unsigned grid = grid_for(n / kUnroll + 1, kBlock, 8);
+    unsigned grid = chunk_grid(n, kChunk);
     if (pl.rank == 1 && pl.stride[0][0] == 1 && pl.stride[1][0] == 1) {
         copy_flat_kernel<U><<<grid, kBlock, 0, s>>>(static_cast<const U *>(in),
                                                     static_cast<U *>(out), n);
     } else {
-        copy_nd_kernel<U><<<grid, kBlock, 0, s>>>(pl, static_cast<const U *>(in),
-                                                  static_cast<U *>(out), n);
+        bool repeats = false;
+        for (int d = 0; d < pl.rank; ++d)
+            if (pl.stride[0][d] == 0 && pl.dim64[d] > 1) repeats = true;
+        if (repeats)
+            copy_nd_kernel<U, true><<<grid, kBlock, 0, s>>>(pl, static_cast<const U *>(in),
+                                                            static_cast<U *>(out), n);
+        else
+            copy_nd_kernel<U, false><<<grid, kBlock, 0, s>>>(pl, static_cast<const U *>(in),
+                                                             static_cast<U *>(out), n);
     }
     return launch_status();
 }
@@ -213,7 +239,7 @@ __device__ __forceinline__ U gather_fetch(const U *__restrict__ data, const I *_
         if (err) *err = 1;
         return U{};
     }
-    return data[(static_cast<int64_t>(outer) * axis_dim + ix) * row_units + c];
+    return nt_load(data + (static_cast<int64_t>(outer) * axis_dim + ix) * row_units + c);
 }
 
 template <typename U, typename I>
@@ -224,27 +250,28 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const U *__restrict
                                                              uint32_t n_idx, FastDiv idx_div,
                                                              int64_t axis_dim,
                                                              int32_t *__restrict__ err) {
-    const uint32_t step = gridDim.x * kBlock;
-    uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-    for (; i + (kUnroll - 1) * step < n_units; i += step * kUnroll) {
-        U r[kUnroll];
+    for (uint32_t base = blockIdx.x * kChunk; base < n_units; base += gridDim.x * kChunk) {
+        const uint32_t i0 = base + threadIdx.x;
+        if (base + kChunk <= n_units) {
+            U r[kUnroll];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j)
-            r[j] = gather_fetch<U, I>(data, idx, i + j * step, row_units, row_div, n_idx, idx_div,
-                                      axis_dim, err);
+            for (int j = 0; j < kUnroll; ++j)
+                r[j] = gather_fetch<U, I>(data, idx, i0 + j * kBlock, row_units, row_div, n_idx, idx_div,
+                                          axis_dim, err);
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) out[i + j * step] = r[j];
+            for (int j = 0; j < kUnroll; ++j) put(out + i0 + j * kBlock, r[j]);
+        } else {
+            for (uint32_t i = i0; i < n_units; i += kBlock)
+                put(out + i, gather_fetch<U, I>(data, idx, i, row_units, row_div, n_idx, idx_div, axis_dim, err));
+        }
     }
-    for (; i < n_units; i += step)
-        out[i] = gather_fetch<U, I>(data, idx, i, row_units, row_div, n_idx, idx_div, axis_dim,
-                                    err);
 }
 
 template <typename U>
 int32_t launch_gather(hipStream_t s, int32_t idx_dtype, const void *data, const void *idx,
                       void *out, uint32_t n_units, uint32_t row_units, uint32_t n_idx,
                       int64_t axis_dim, int32_t *err) {
-    unsigned grid = grid_for(n_units / kUnroll + 1, kBlock, 8);
+    unsigned grid = chunk_grid(n_units, kChunk);
     FastDiv rd(row_units), id(n_idx);
     if (idx_dtype == RMLK_INT64)
         gather_rows_kernel<U, int64_t><<<grid, kBlock, 0, s>>>(
@@ -338,33 +365,53 @@ __global__ __launch_bounds__(kBlock) void scatter_nd_kernel(ScatterPlan sp,
 // ---------------------------------------------------------------------------------------------
 // Trilu over [batch, rows, cols]; VEC units along cols
 template <typename U, int VEC>
+__device__ __forceinline__ Vec<U, VEC> trilu_item(const U *__restrict__ in, uint32_t i, uint32_t cols_v,
+                                                  FastDiv cols_div, uint32_t rows, FastDiv rows_div,
+                                                  int upper, int64_t k) {
+    const uint32_t rq = cols_div.div(i);
+    const uint32_t cv = i - rq * cols_v;
+    const uint32_t bq = rows_div.div(rq);
+    const int64_t row = rq - bq * rows;
+    const int64_t c0 = static_cast<int64_t>(cv) * VEC;
+    const int64_t diag = row + k;  // upper keeps col >= diag, lower keeps col <= diag
+    const bool any = upper ? (c0 + VEC - 1 >= diag) : (c0 <= diag);
+    Vec<U, VEC> v;
+    if (any) {   // vectors wholly outside the triangle are not read
+        v = nt_load(reinterpret_cast<const Vec<U, VEC> *>(in + static_cast<size_t>(i) * VEC));
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            const bool keep = upper ? (c0 + j >= diag) : (c0 + j <= diag);
+            if (!keep) v.v[j] = U{};
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v.v[j] = U{};
+    }
+    return v;
+}
+
+template <typename U, int VEC>
 __global__ __launch_bounds__(kBlock) void trilu_kernel(const U *__restrict__ in,
                                                        U *__restrict__ out, uint32_t n_items,
                                                        uint32_t cols_v, FastDiv cols_div,
                                                        uint32_t rows, FastDiv rows_div, int upper,
                                                        int64_t k) {
-    const uint32_t step = gridDim.x * kBlock;
-    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n_items; i += step) {
-        uint32_t rq = cols_div.div(i);
-        uint32_t cv = i - rq * cols_v;
-        uint32_t bq = rows_div.div(rq);
-        int64_t row = rq - bq * rows;
-        int64_t c0 = static_cast<int64_t>(cv) * VEC;
-        int64_t diag = row + k;  // upper keeps col >= diag, lower keeps col <= diag
-        bool any = upper ? (c0 + VEC - 1 >= diag) : (c0 <= diag);
-        Vec<U, VEC> v;
-        if (any) {
-            v = *reinterpret_cast<const Vec<U, VEC> *>(in + static_cast<size_t>(i) * VEC);
+    using V = Vec<U, VEC>;
+    for (uint32_t base = blockIdx.x * kChunk; base < n_items; base += gridDim.x * kChunk) {
+        const uint32_t i0 = base + threadIdx.x;
+        if (base + kChunk <= n_items) {
+            V r[kUnroll];
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) {
-                bool keep = upper ? (c0 + j >= diag) : (c0 + j <= diag);
-                if (!keep) v.v[j] = U{};
-            }
+            for (int j = 0; j < kUnroll; ++j)
+                r[j] = trilu_item<U, VEC>(in, i0 + j * kBlock, cols_v, cols_div, rows, rows_div, upper, k);
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j)
+                put(reinterpret_cast<V *>(out + static_cast<size_t>(i0 + j * kBlock) * VEC), r[j]);
         } else {
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) v.v[j] = U{};
+            for (uint32_t i = i0; i < n_items; i += kBlock)
+                put(reinterpret_cast<V *>(out + static_cast<size_t>(i) * VEC),
+                    trilu_item<U, VEC>(in, i, cols_v, cols_div, rows, rows_div, upper, k));
         }
-        *reinterpret_cast<Vec<U, VEC> *>(out + static_cast<size_t>(i) * VEC) = v;
     }
 }
 
@@ -384,7 +431,7 @@ int32_t launch_trilu(hipStream_t s, int64_t batch, int64_t rows, int64_t cols, i
         const U *pi = static_cast<const U *>(in) + b0 * rows * cols;
         U *po = static_cast<U *>(out) + b0 * rows * cols;
         const uint32_t n_items = static_cast<uint32_t>(nb * rows * cols_v);
-        const unsigned grid = grid_for(n_items, kBlock, 16);
+        const unsigned grid = chunk_grid(n_items, kChunk);
         const uint32_t cv = static_cast<uint32_t>(cols_v), rw = static_cast<uint32_t>(rows);
         if (vec == 4)
             trilu_kernel<U, 4><<<grid, kBlock, 0, s>>>(pi, po, n_items, cv, FastDiv(cv), rw,
@@ -402,6 +449,27 @@ int32_t launch_trilu(hipStream_t s, int64_t batch, int64_t rows, int64_t cols, i
 }  // namespace rmlk
 
 using namespace rmlk;
+
+// Device-to-device copy with the flat copy kernel when both ends and the length are multiples of 16
+// bytes (what the runtime copies: whole tensors from its pool), through the HIP runtime otherwise.
+extern "C" int32_t rmlk_hip_memcpy_dtod(rmlk_stream_t stream, void *dst, const void *src,
+                                        size_t bytes) {
+    if (bytes == 0) return RMLK_OK;
+    if (!dst || !src) return RMLK_ERR_NULL_POINTER;
+    hipStream_t s = as_stream(stream);
+    if (bytes % 16 || reinterpret_cast<uintptr_t>(dst) % 16 || reinterpret_cast<uintptr_t>(src) % 16)
+        return static_cast<int32_t>(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s));
+    constexpr size_t kPieceUnits = static_cast<size_t>(1) << 30;
+    const U128 *pi = static_cast<const U128 *>(src);
+    U128 *po = static_cast<U128 *>(dst);
+    for (size_t done = 0, units = bytes / 16; done < units; done += kPieceUnits) {
+        const uint32_t n = static_cast<uint32_t>(units - done < kPieceUnits ? units - done : kPieceUnits);
+        copy_flat_kernel<U128><<<chunk_grid(n, kChunk), kBlock, 0, s>>>(pi + done, po + done, n);
+        const int32_t st = launch_status();
+        if (st) return st;
+    }
+    return RMLK_OK;
+}
 
 extern "C" int32_t rmlk_hip_transpose(rmlk_stream_t stream, int32_t dtype,
                                       const rmlk_dims *in_shape, const int64_t *perm,

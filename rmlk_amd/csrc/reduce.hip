@@ -54,15 +54,28 @@ __global__ __launch_bounds__(kBlock) void mean_rows_kernel(const T *__restrict__
             const int64_t nv = cols / VEC;
             const V *pv = reinterpret_cast<const V *>(p);
             int64_t c = lane_in_group;
+            // the input is read once: streaming loads, eight in flight per lane while the row lasts
+            for (; c + 7 * kGroup < nv; c += 8 * kGroup) {
+                V v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = nt_load(pv + c + u * kGroup);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    acc += ((static_cast<double>(v[0].v[j]) + static_cast<double>(v[1].v[j])) +
+                            (static_cast<double>(v[2].v[j]) + static_cast<double>(v[3].v[j]))) +
+                           ((static_cast<double>(v[4].v[j]) + static_cast<double>(v[5].v[j])) +
+                            (static_cast<double>(v[6].v[j]) + static_cast<double>(v[7].v[j])));
+            }
             for (; c + 3 * kGroup < nv; c += 4 * kGroup) {
-                V v0 = pv[c], v1 = pv[c + kGroup], v2 = pv[c + 2 * kGroup], v3 = pv[c + 3 * kGroup];
+                V v0 = nt_load(pv + c), v1 = nt_load(pv + c + kGroup), v2 = nt_load(pv + c + 2 * kGroup),
+                  v3 = nt_load(pv + c + 3 * kGroup);
 #pragma unroll
                 for (int j = 0; j < VEC; ++j)
                     acc += (static_cast<double>(v0.v[j]) + static_cast<double>(v1.v[j])) +
                            (static_cast<double>(v2.v[j]) + static_cast<double>(v3.v[j]));
             }
             for (; c < nv; c += kGroup) {
-                V v = pv[c];
+                V v = nt_load(pv + c);
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) acc += static_cast<double>(v.v[j]);
             }

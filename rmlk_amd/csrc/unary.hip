@@ -13,32 +13,35 @@ namespace {
 template <typename F, typename TI, typename TO, int VEC>
 __global__ __launch_bounds__(kEwBlock) void map_flat_kernel(const TI *__restrict__ in,
                                                             TO *__restrict__ out, uint32_t n) {
-    const uint32_t step = gridDim.x * kEwBlock;
-    uint32_t i = blockIdx.x * kEwBlock + threadIdx.x;
     if constexpr (VEC == 1) {
-        for (; i < n; i += step) out[i] = F::apply(in[i]);
+        const uint32_t step = gridDim.x * kEwBlock;
+        for (uint32_t i = blockIdx.x * kEwBlock + threadIdx.x; i < n; i += step) out[i] = F::apply(in[i]);
     } else {
         const uint32_t n_vec = n / kEwVec;
-        for (; i + (kEwUnroll - 1) * step < n_vec; i += kEwUnroll * step) {
-            TI ri[kEwUnroll][kEwVec];
+        for (uint32_t base = blockIdx.x * kEwChunk; base < n_vec; base += gridDim.x * kEwChunk) {
+            const uint32_t i0 = base + threadIdx.x;
+            if (base + kEwChunk <= n_vec) {
+                TI ri[kEwUnroll][kEwVec];
 #pragma unroll
-            for (int u = 0; u < kEwUnroll; ++u)
-                load_vec(in + static_cast<size_t>(i + u * step) * kEwVec, false, ri[u]);
+                for (int u = 0; u < kEwUnroll; ++u)
+                    load_op<kEwDense, true>(in + static_cast<size_t>(i0 + u * kEwBlock) * kEwVec, ri[u]);
 #pragma unroll
-            for (int u = 0; u < kEwUnroll; ++u) {
-                TO ro[kEwVec];
+                for (int u = 0; u < kEwUnroll; ++u) {
+                    TO ro[kEwVec];
 #pragma unroll
-                for (int j = 0; j < kEwVec; ++j) ro[j] = F::apply(ri[u][j]);
-                store_vec(out + static_cast<size_t>(i + u * step) * kEwVec, ro);
+                    for (int j = 0; j < kEwVec; ++j) ro[j] = F::apply(ri[u][j]);
+                    store_vec(out + static_cast<size_t>(i0 + u * kEwBlock) * kEwVec, ro);
+                }
+            } else {
+                for (uint32_t i = i0; i < n_vec; i += kEwBlock) {
+                    TI ri[kEwVec];
+                    TO ro[kEwVec];
+                    load_op<kEwDense, true>(in + static_cast<size_t>(i) * kEwVec, ri);
+#pragma unroll
+                    for (int j = 0; j < kEwVec; ++j) ro[j] = F::apply(ri[j]);
+                    store_vec(out + static_cast<size_t>(i) * kEwVec, ro);
+                }
             }
-        }
-        for (; i < n_vec; i += step) {
-            TI ri[kEwVec];
-            TO ro[kEwVec];
-            load_vec(in + static_cast<size_t>(i) * kEwVec, false, ri);
-#pragma unroll
-            for (int j = 0; j < kEwVec; ++j) ro[j] = F::apply(ri[j]);
-            store_vec(out + static_cast<size_t>(i) * kEwVec, ro);
         }
         if (blockIdx.x == 0 && threadIdx.x < (n - n_vec * kEwVec)) {
             uint32_t t = n_vec * kEwVec + threadIdx.x;
@@ -59,7 +62,7 @@ int32_t launch_map(hipStream_t s, int64_t n, const void *in, void *out) {
         bool aligned = reinterpret_cast<uintptr_t>(pi) % ai == 0 &&
                        reinterpret_cast<uintptr_t>(po) % ao == 0;
         if (aligned) {
-            unsigned grid = grid_for(m / (kEwVec * kEwUnroll) + 1, kEwBlock, kEwBlocksPerCu);
+            unsigned grid = chunk_grid(m / kEwVec, kEwChunk);
             map_flat_kernel<F, TI, TO, kEwVec><<<grid, kEwBlock, 0, s>>>(pi, po, m);
         } else {
             unsigned grid = grid_for(m, kEwBlock, 16);

@@ -15,52 +15,55 @@ __device__ __forceinline__ void select_store(T *dst, const T (&x)[kEwVec], const
     store_vec(dst, ro);
 }
 
-template <typename T>
+// XM / YM: how x and y walk the output (kEwDense, or kEwRepeat: one element for all of it); the
+// condition is dense. Other combinations take the nd<1> kernel.
+template <typename T, int XM, int YM>
 __global__ __launch_bounds__(kEwBlock) void where_flat_kernel(const T *__restrict__ x,
                                                               const T *__restrict__ y,
                                                               const uint8_t *__restrict__ c,
-                                                              T *__restrict__ out, uint32_t n,
-                                                              int x_b, int y_b, int c_b) {
+                                                              T *__restrict__ out, uint32_t n) {
     const uint32_t n_vec = n / kEwVec;
-    const uint32_t step = gridDim.x * kEwBlock;
-    uint32_t i = blockIdx.x * kEwBlock + threadIdx.x;
-    for (; i + (kEwUnroll - 1) * step < n_vec; i += kEwUnroll * step) {
-        T rx[kEwUnroll][kEwVec], ry[kEwUnroll][kEwVec];
-        uint8_t rc[kEwUnroll][kEwVec];
+    for (uint32_t base = blockIdx.x * kEwChunk; base < n_vec; base += gridDim.x * kEwChunk) {
+        const uint32_t i0 = base + threadIdx.x;
+        if (base + kEwChunk <= n_vec) {
+            T rx[kEwUnroll][kEwVec], ry[kEwUnroll][kEwVec];
+            uint8_t rc[kEwUnroll][kEwVec];
 #pragma unroll
-        for (int u = 0; u < kEwUnroll; ++u) {
-            const size_t e = static_cast<size_t>(i + u * step) * kEwVec;
-            load_vec(x_b ? x : x + e, x_b != 0, rx[u]);
-            load_vec(y_b ? y : y + e, y_b != 0, ry[u]);
-            load_vec(c_b ? c : c + e, c_b != 0, rc[u]);
+            for (int u = 0; u < kEwUnroll; ++u) {
+                const size_t e = static_cast<size_t>(i0 + u * kEwBlock) * kEwVec;
+                load_op<XM, true>(XM == kEwRepeat ? x : x + e, rx[u]);
+                load_op<YM, true>(YM == kEwRepeat ? y : y + e, ry[u]);
+                load_op<kEwDense, true>(c + e, rc[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < kEwUnroll; ++u)
+                select_store(out + static_cast<size_t>(i0 + u * kEwBlock) * kEwVec, rx[u], ry[u], rc[u]);
+        } else {
+            for (uint32_t i = i0; i < n_vec; i += kEwBlock) {
+                T rx[kEwVec], ry[kEwVec];
+                uint8_t rc[kEwVec];
+                const size_t e = static_cast<size_t>(i) * kEwVec;
+                load_op<XM, true>(XM == kEwRepeat ? x : x + e, rx);
+                load_op<YM, true>(YM == kEwRepeat ? y : y + e, ry);
+                load_op<kEwDense, true>(c + e, rc);
+                select_store(out + e, rx, ry, rc);
+            }
         }
-#pragma unroll
-        for (int u = 0; u < kEwUnroll; ++u)
-            select_store(out + static_cast<size_t>(i + u * step) * kEwVec, rx[u], ry[u], rc[u]);
-    }
-    for (; i < n_vec; i += step) {
-        T rx[kEwVec], ry[kEwVec];
-        uint8_t rc[kEwVec];
-        const size_t e = static_cast<size_t>(i) * kEwVec;
-        load_vec(x_b ? x : x + e, x_b != 0, rx);
-        load_vec(y_b ? y : y + e, y_b != 0, ry);
-        load_vec(c_b ? c : c + e, c_b != 0, rc);
-        select_store(out + e, rx, ry, rc);
     }
     if (blockIdx.x == 0 && threadIdx.x < (n - n_vec * kEwVec)) {
         uint32_t t = n_vec * kEwVec + threadIdx.x;
-        out[t] = c[c_b ? 0 : t] ? x[x_b ? 0 : t] : y[y_b ? 0 : t];
+        out[t] = c[t] ? x[XM == kEwRepeat ? 0 : t] : y[YM == kEwRepeat ? 0 : t];
     }
 }
 
-// plan operands: 0 = x, 1 = y, 2 = cond, 3 = out
-template <typename T, int VEC, int UNR>
+// plan operands: 0 = x, 1 = y, 2 = cond, 3 = out. XM / YM: how x and y walk the innermost run
+// (VEC == 4 only; the condition walks it densely).
+template <typename T, int VEC, int UNR, int XM, int YM>
 __global__ __launch_bounds__(kEwBlock) void where_nd_kernel(NdPlan<4> pl, EwUnrollDim<4> ud,
                                                             const T *__restrict__ x,
                                                             const T *__restrict__ y,
                                                             const uint8_t *__restrict__ c,
-                                                            T *__restrict__ out, uint32_t n_items,
-                                                            int x0, int y0, int c0) {
+                                                            T *__restrict__ out, uint32_t n_items) {
     const uint32_t step = gridDim.x * kEwBlock;
     uint32_t i = blockIdx.x * kEwBlock + threadIdx.x;
     if constexpr (VEC == 1) {
@@ -75,35 +78,37 @@ __global__ __launch_bounds__(kEwBlock) void where_nd_kernel(NdPlan<4> pl, EwUnro
             nd_offsets<4>(pl, i, offs);
             T rx[UNR][kEwVec], ry[UNR][kEwVec];
             uint8_t rc[UNR][kEwVec];
-            load_vec(x + offs[0], x0 != 0, rx[0]);
-            load_vec(y + offs[1], y0 != 0, ry[0]);
-            load_vec(c + offs[2], c0 != 0, rc[0]);
 #pragma unroll
-            for (int u = 1; u < UNR; ++u) {
-                if (ud.stride[0] != 0) {
-                    load_vec(x + offs[0] + static_cast<int64_t>(u) * ud.stride[0], x0 != 0, rx[u]);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < kEwVec; ++j) rx[u][j] = rx[0][j];
-                }
-                if (ud.stride[1] != 0) {
-                    load_vec(y + offs[1] + static_cast<int64_t>(u) * ud.stride[1], y0 != 0, ry[u]);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < kEwVec; ++j) ry[u][j] = ry[0][j];
-                }
-                if (ud.stride[2] != 0) {
-                    load_vec(c + offs[2] + static_cast<int64_t>(u) * ud.stride[2], c0 != 0, rc[u]);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < kEwVec; ++j) rc[u][j] = rc[0][j];
-                }
+            for (int u = 0; u < UNR; ++u) {
+                load_op<XM, false>(x + offs[0] + static_cast<int64_t>(u) * ud.stride[0], rx[u]);
+                load_op<YM, false>(y + offs[1] + static_cast<int64_t>(u) * ud.stride[1], ry[u]);
+                load_op<kEwDense, false>(c + offs[2] + static_cast<int64_t>(u) * ud.stride[2], rc[u]);
             }
 #pragma unroll
             for (int u = 0; u < UNR; ++u)
                 select_store(out + offs[3] + static_cast<int64_t>(u) * ud.stride[3], rx[u], ry[u],
                              rc[u]);
         }
+    }
+}
+
+// bit 0: x repeats one element along the innermost run, bit 1: y does (the condition never)
+constexpr uint32_t kWhereModes = (1u << 0) | (1u << 1) | (1u << 2) | (1u << 3);
+
+template <typename T, int XM, int YM>
+void launch_where_mode(hipStream_t stream, const EwDecision<4> &dec, const T *x, const T *y,
+                       const uint8_t *c, T *out) {
+    if (dec.shape == EwShape::Flat) {
+        where_flat_kernel<T, XM, YM><<<chunk_grid(dec.n_items / kEwVec, kEwChunk), kEwBlock, 0, stream>>>(
+            x, y, c, out, dec.n_items);
+    } else {
+        const unsigned grid = grid_for(dec.n_items, kEwBlock, kEwBlocksPerCu);
+        if (dec.unrolled)
+            where_nd_kernel<T, kEwVec, kEwUnroll, XM, YM><<<grid, kEwBlock, 0, stream>>>(
+                dec.plan, dec.udim, x, y, c, out, dec.n_items);
+        else
+            where_nd_kernel<T, kEwVec, 1, XM, YM><<<grid, kEwBlock, 0, stream>>>(
+                dec.plan, dec.udim, x, y, c, out, dec.n_items);
     }
 }
 
@@ -115,31 +120,17 @@ int32_t launch_where(hipStream_t stream, int rank, const int64_t *shape,
     const void *ptrs[4] = {x, y, c, out};
     const int sizes[4] = {static_cast<int>(sizeof(T)), static_cast<int>(sizeof(T)), 1,
                           static_cast<int>(sizeof(T))};
-    if (!ew_decide<4>(dec, rank, shape, strides, ptrs, sizes)) return RMLK_OK;
-    unsigned grid;
-    switch (dec.shape) {
-        case EwShape::Flat:
-            grid = grid_for(dec.n_items / (kEwVec * kEwUnroll) + 1, kEwBlock, kEwBlocksPerCu);
-            where_flat_kernel<T><<<grid, kEwBlock, 0, stream>>>(x, y, c, out, dec.n_items,
-                                                                dec.inner0[0], dec.inner0[1],
-                                                                dec.inner0[2]);
-            break;
-        case EwShape::Nd4:
-            grid = grid_for(dec.n_items, kEwBlock, kEwBlocksPerCu);
-            if (dec.unrolled)
-                where_nd_kernel<T, kEwVec, kEwUnroll><<<grid, kEwBlock, 0, stream>>>(
-                    dec.plan, dec.udim, x, y, c, out, dec.n_items, dec.inner0[0], dec.inner0[1],
-                    dec.inner0[2]);
-            else
-                where_nd_kernel<T, kEwVec, 1><<<grid, kEwBlock, 0, stream>>>(
-                    dec.plan, dec.udim, x, y, c, out, dec.n_items, dec.inner0[0], dec.inner0[1],
-                    dec.inner0[2]);
-            break;
-        case EwShape::Nd1:
-            grid = grid_for(dec.n_items, kEwBlock, 16);
-            where_nd_kernel<T, 1, 1><<<grid, kEwBlock, 0, stream>>>(dec.plan, dec.udim, x, y, c,
-                                                                    out, dec.n_items, 0, 0, 0);
-            break;
+    if (!ew_decide<4>(dec, rank, shape, strides, ptrs, sizes, kWhereModes)) return RMLK_OK;
+    if (dec.shape == EwShape::Nd1) {
+        where_nd_kernel<T, 1, 1, kEwDense, kEwDense><<<grid_for(dec.n_items, kEwBlock, 16), kEwBlock, 0, stream>>>(
+            dec.plan, dec.udim, x, y, c, out, dec.n_items);
+    } else {
+        switch (dec.mode_bits) {
+            case 0: launch_where_mode<T, kEwDense, kEwDense>(stream, dec, x, y, c, out); break;
+            case 1: launch_where_mode<T, kEwRepeat, kEwDense>(stream, dec, x, y, c, out); break;
+            case 2: launch_where_mode<T, kEwDense, kEwRepeat>(stream, dec, x, y, c, out); break;
+            default: launch_where_mode<T, kEwRepeat, kEwRepeat>(stream, dec, x, y, c, out); break;
+        }
     }
     return launch_status();
 }
