@@ -346,32 +346,40 @@ def matmul_launches(cfg, s, max_len):
 
 
 def run_ops_suite(args):
-    """BASELINE configs[1]: each op of the microbench launched repeatedly over rotating buffer sets
-    (working set above the 256 MB Infinity Cache), for `rocprofv3 --kernel-trace --stats`."""
+    """BASELINE configs[1] and configs[4] operator shapes, each launched repeatedly over rotating buffer
+    sets (working set well above the 256 MB Infinity Cache, so that HBM is what is measured).
+    A one-block `write_small_kernel` launch marks the start of every op in a kernel trace:
+    `bench.py --summarize-ops` splits a `rocprofv3 --kernel-trace` (and `--pmc`) CSV of this command
+    at those markers."""
+    import ctypes
     import numpy as np
     import torch
     from rmlk_amd import kernels as k
     from rmlk_amd._lib import check, lib
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev).manual_seed(2)
-    ns = 6
+    ns = 16                             # 16 x 33.5 MB per operand
     shp, n = [8, 32, 512, 64], 8 * 32 * 512 * 64
     xs = [torch.randn(n, device=dev, generator=g) for _ in range(ns)]
     ys = [torch.empty(n, device=dev) for _ in range(ns)]
     bs = [torch.randn(32 * 64, device=dev, generator=g) for _ in range(ns)]
     conds = [(torch.rand(n, device=dev, generator=g) < 0.5) for _ in range(ns)]
     dense, bst = [1048576, 32768, 64, 1], [0, 64, 0, 1]
-    reps = max(100, args.steps * 10)     # launches per recorded graph, rotating over the buffer sets
+    reps = max(8, args.ops_launches)     # launches per recorded graph, rotating over the buffer sets
     results = {}
     side = torch.cuda.Stream()
+    marker = torch.zeros(4, dtype=torch.int32, device=dev)
+    one = ctypes.c_int32(1)
 
-    def timed(name, fn, nset, bytes_):
-        """>= 10 eager warm-up launches, then `reps` launches recorded into ONE HIP graph (so that they
-        run back to back with no host in between), the graph replayed untimed until >= 30 ms of
-        continuous work have passed, then `args.warmup`+... timed replays between one pair of events
-        on the launching stream."""
+    def timed(name, fn, nset, bytes_, kernels_per_call=1):
+        """A marker launch, >= 10 eager warm-up launches, then `reps` launches recorded into ONE HIP
+        graph (back to back, no host in between); the graph is replayed untimed until >= 30 ms of
+        continuous work have passed, then timed replays run between one pair of events on the
+        launching stream."""
         with torch.cuda.stream(side):
-            for i in range(max(10, 2 * nset)):
+            check(lib().rmlk_hip_write_small(side.cuda_stream, marker.data_ptr(), ctypes.byref(one), 4),
+                  "rmlk_hip_write_small")
+            for i in range(max(10, nset)):
                 fn(i % nset)
             side.synchronize()
             graph = torch.cuda.CUDAGraph()
@@ -384,22 +392,33 @@ def run_ops_suite(args):
             e1.record(side)
             side.synchronize()
             first_ms = max(e0.elapsed_time(e1), 1e-3)
-            for _ in range(min(200, int(30.0 / first_ms) + 1)):
+            n_warm = 0 if args.ops_quick else min(200, int(30.0 / first_ms) + 1)
+            for _ in range(n_warm):
                 graph.replay()
-            n_timed = max(3, min(50, int(20.0 / first_ms)))
+            n_timed = 1 if args.ops_quick else max(3, min(50, int(20.0 / first_ms)))
             e0.record(side)
             for _ in range(n_timed):
                 graph.replay()
             e1.record(side)
             side.synchronize()
         us = e0.elapsed_time(e1) / (n_timed * reps) * 1e3
-        results[name] = {"us_per_launch": round(us, 2), "algorithmic_bytes": bytes_,
-                         "tb_per_s": round(bytes_ / us / 1e6, 3),
-                         "frac_of_hbm_peak": round(bytes_ / us / 1e6 / (PEAK_HBM_GBS / 1e3), 3),
-                         "launches_timed": n_timed * reps, "buffer_sets": nset}
-        log(f"[ops] {name}: {us:.2f} us/launch, {bytes_ / us / 1e6:.2f} TB/s")
+        results[name] = {"us_per_call_with_launch_gaps": round(us, 2), "algorithmic_bytes": bytes_,
+                         "calls_timed": n_timed * reps, "kernels_per_call": kernels_per_call,
+                         "buffer_sets": nset}
+        log(f"[ops] {name}: {us:.2f} us/call with launch gaps, {bytes_ / us / 1e6:.2f} TB/s")
         del graph
 
+    # ---- yardsticks: an almost empty launch and a plain 256 MiB copy -------------------------------
+    timed("launch_floor", lambda i: check(lib().rmlk_hip_fill(side.cuda_stream, k.INT32, 1, ctypes.byref(one),
+                                                              marker.data_ptr()), "rmlk_hip_fill"), 1, 4)
+    big = [torch.empty(CALIBRATION_COPY_BYTES // 4, device=dev) for _ in range(4)]
+    for t in big:
+        t.normal_(generator=g)
+    timed("copy_256MiB", lambda i: check(lib().rmlk_hip_memcpy_dtod(
+        side.cuda_stream, big[2 + i % 2].data_ptr(), big[i % 2].data_ptr(), CALIBRATION_COPY_BYTES),
+        "rmlk_hip_memcpy_dtod"), 2, 2 * CALIBRATION_COPY_BYTES)
+    del big
+    # ---- configs[1] ---------------------------------------------------------------------------------
     timed("add", lambda i: k.binary(k.ADD, xs[i], bs[i], ys[i], shp, dense, bst), ns, 2 * n * 4 + 8192)
     timed("mul", lambda i: k.binary(k.MUL, xs[i], bs[i], ys[i], shp, dense, bst), ns, 2 * n * 4 + 8192)
     timed("div", lambda i: k.binary(k.DIV, xs[i], bs[i], ys[i], shp, dense, bst), ns, 2 * n * 4 + 8192)
@@ -424,9 +443,10 @@ def run_ops_suite(args):
     gam = torch.rand(2048, device=dev, generator=g) + 0.5
     timed("fused_rmsnorm", lambda i: k.rmsnorm(xs[i], gam, ys[i], 4096, 2048, 1e-5), ns,
           2 * n * 4 + 8192)
-    sums = [torch.empty(n, device=dev) for _ in range(2)]
-    timed("fused_add_rmsnorm", lambda i: k.add_rmsnorm(xs[i], xs[(i + 1) % ns], gam, sums[i % 2], ys[i],
+    sums = [torch.empty(n, device=dev) for _ in range(ns)]
+    timed("fused_add_rmsnorm", lambda i: k.add_rmsnorm(xs[i], xs[(i + 1) % ns], gam, sums[i], ys[i],
                                                        4096, 2048, 1e-5), ns, 4 * n * 4 + 8192)
+    del sums
     timed("fused_swiglu", lambda i: k.swiglu(xs[i], xs[(i + 1) % ns], ys[i]), ns, 3 * n * 4)
     cs_tab = torch.randn(2 * 2048 * 64, device=dev, generator=g)
     rot_shape = [1, 64, 2048, 64]       # the [1, 2048, 64, 64] projection read head-major
@@ -439,21 +459,21 @@ def run_ops_suite(args):
           lambda i: k.scale_mask_softmax(plain[i], msk, so[i], [1, 32, 2048, 2048], [0, 0, 2048, 1], 8.0),
           2, 2 * plain[0].numel() * 4 + 2048 * 2048 * 4)
     del plain
-    # ---- config 5 shapes: KV-cache / indexing stress ---------------------------------------------
+    # ---- configs[4] shapes: KV-cache / indexing stress ---------------------------------------------
     kv_n = 8 * 8192 * 64
-    caches = [torch.randn(kv_n, device=dev, generator=g) for _ in range(ns * 3)]
-    outs = [torch.empty(kv_n, device=dev) for _ in range(ns * 3)]
+    nk = ns * 2
+    caches = [torch.randn(kv_n, device=dev, generator=g) for _ in range(nk)]
+    outs = [torch.empty(kv_n, device=dev) for _ in range(nk)]
     rows = [torch.randn(8 * 64, device=dev, generator=g) for _ in range(ns)]
     sidx = [torch.tensor([[0, h, int(p)] for h in range(8)], device=dev, dtype=torch.int64)
             for p in np.random.default_rng(5).integers(0, 8192, size=ns)]
-    nk = ns * 3
 
     def scatter_copy(i):
         j = i % nk
         check(lib().rmlk_hip_memcpy_dtod(torch.cuda.current_stream().cuda_stream, outs[j].data_ptr(),
                                          caches[j].data_ptr(), kv_n * 4), "rmlk_hip_memcpy_dtod")
         k.scatter_nd(sidx[i % ns], rows[i % ns], outs[j], [1, 8, 8192, 64], 8, 3)
-    timed("scatter_nd_copy", scatter_copy, nk, 2 * kv_n * 4 + 8 * 64 * 4 + 192)
+    timed("scatter_nd_copy", scatter_copy, nk, 2 * kv_n * 4 + 8 * 64 * 4 + 192, kernels_per_call=2)
     timed("scatter_nd_inplace", lambda i: k.scatter_nd(sidx[i % ns], rows[i % ns], caches[i % nk],
                                                        [1, 8, 8192, 64], 8, 3), nk, 8 * 64 * 4 + 192)
     timed("slice_kv", lambda i: k.slice_(caches[i % nk], outs[i % nk], [1, 8, 8192, 64], [0, 0, 0, 0],
@@ -463,7 +483,7 @@ def run_ops_suite(args):
         j = i % nk
         k.concat_into(caches[j][:8 * 8191 * 64], outs[j], [1, 8, 8191, 64], [1, 8, 8192, 64], 2, 0)
         k.concat_into(rows[i % ns], outs[j], [1, 8, 1, 64], [1, 8, 8192, 64], 2, 8191)
-    timed("concat_kv", concat_kv, nk, 2 * kv_n * 4)
+    timed("concat_kv", concat_kv, nk, 2 * kv_n * 4, kernels_per_call=2)
     del caches, outs
     table = torch.randn(128256, 2048, device=dev, generator=g)
     idx4 = [torch.randint(0, 128256, (4096,), device=dev, generator=g) for _ in range(ns)]
@@ -485,10 +505,98 @@ def run_ops_suite(args):
     i64a = [torch.randint(0, 100, (8192 * 8192,), device=dev, generator=g) for _ in range(2)]
     timed("equal_i64_8192", lambda i: k.binary(k.EQUAL, i64a[i], i64a[1 - i], eq_out, full, dn, dn), 2,
           2 * 8192 * 8192 * 8 + 8192 * 8192)
-    print(json.dumps({"suite": "ops", "note": "us_per_launch: HIP events around back-to-back launches "
-                      "(replays of a recorded graph of rotating launches), launch gaps included; "
-                      "per-kernel durations come from rocprofv3 --kernel-trace of this command",
+    with torch.cuda.stream(side):          # closing marker: the last op's segment ends here
+        check(lib().rmlk_hip_write_small(side.cuda_stream, marker.data_ptr(), ctypes.byref(one), 4),
+              "rmlk_hip_write_small")
+        side.synchronize()
+    print(json.dumps({"suite": "ops", "note": "us_per_call_with_launch_gaps: HIP events around replays of a "
+                      "recorded graph of rotating launches; kernel durations come from rocprofv3 "
+                      "--kernel-trace of this command (bench.py --summarize-ops)",
                       "results": results}))
+
+
+OPS_MARKER_KERNEL = "write_small_kernel"
+
+
+def _ops_segments(csv_path):
+    """Dispatch rows of a rocprofv3 CSV (kernel trace or counter collection) of `--suite ops`, in
+    start order, cut at the marker launches: one list of this library's dispatches per op."""
+    import csv
+    rows = list(csv.DictReader(open(csv_path)))
+    rows.sort(key=lambda r: int(r["Start_Timestamp"]))
+    segments, cur = [], None
+    for r in rows:
+        name = r["Kernel_Name"]
+        if OPS_MARKER_KERNEL in name:
+            if cur is not None:
+                segments.append(cur)
+            cur = []
+        elif cur is not None and "rmlk::" in name:
+            cur.append(r)
+    return segments
+
+
+def _short_kernel_name(name):
+    import re
+    name = re.sub(r"rmlk::\(anonymous namespace\)::", "", name)
+    name = re.sub(r"^void ", "", name).replace("rmlk::", "")
+    cut = name.find("(")
+    return (name if cut < 0 else name[:cut])[:64]
+
+
+def summarize_ops(args):
+    """Markdown table per op of `--suite ops` from its JSON line and the rocprofv3 CSVs of the same
+    command: kernel-trace durations of the timed launches (the last calls_timed of each op), and,
+    when given, FETCH_SIZE / WRITE_SIZE per call scaled by what the counters read for the 256 MiB
+    copy of the same run."""
+    res = json.loads([l for l in open(args.summarize_ops) if l.startswith("{")][-1])["results"]
+    names = list(res)
+    segs = _ops_segments(args.kernel_trace)
+    assert len(segs) == len(names), (len(segs), len(names))
+    pmc = {}
+    for label, path in (("FETCH_SIZE", args.pmc_fetch), ("WRITE_SIZE", args.pmc_write)):
+        if not path:
+            continue
+        psegs = _ops_segments(path)
+        assert len(psegs) == len(names), (label, len(psegs), len(names))
+        per_call = {}
+        for nm, seg in zip(names, psegs):
+            vals = [float(r["Counter_Value"]) for r in seg if r["Counter_Name"] == label]
+            kpc = res[nm]["kernels_per_call"]
+            per_call[nm] = sum(vals) / (len(vals) / kpc) if vals else None
+        unit = (CALIBRATION_COPY_BYTES / 1024.0) / per_call["copy_256MiB"]
+        pmc[label] = ({nm: None if v is None else v * unit * 1024.0 for nm, v in per_call.items()}, unit)
+    floor = None
+    print("| op | kernel(s) | grid x block | timed launches | avg us | min us | algorithmic MB | TB/s | % of 8 TB/s"
+          + (" | fetched MB | written MB | moved / algorithmic" if pmc else "") + " |")
+    print("|---|---|---|---|---|---|---|---|---|" + ("---|---|---|" if pmc else ""))
+    for nm, seg in zip(names, segs):
+        r = res[nm]
+        kpc = r["kernels_per_call"]
+        timed_rows = seg[-r["calls_timed"] * kpc:]
+        durs = [int(x["End_Timestamp"]) - int(x["Start_Timestamp"]) for x in timed_rows]
+        calls = [sum(durs[i:i + kpc]) / 1e3 for i in range(0, len(durs), kpc)]
+        avg, mn = sum(calls) / len(calls), min(calls)
+        kernels = []
+        for x in timed_rows[:kpc]:
+            kn = _short_kernel_name(x["Kernel_Name"])
+            wg = int(x["Workgroup_Size_X"]) if "Workgroup_Size_X" in x else int(x["Workgroup_Size"])
+            gs = int(x["Grid_Size_X"]) if "Grid_Size_X" in x else int(x["Grid_Size"])
+            kernels.append((kn, f"{gs // wg} x {wg}"))
+        mb = r["algorithmic_bytes"] / 1e6
+        if nm == "launch_floor":
+            floor = avg
+        line = (f"| {nm} | {' + '.join(kk for kk, _ in kernels)} | {' + '.join(gg for _, gg in kernels)} | "
+                f"{len(calls)} | {avg:.2f} | {mn:.2f} | {mb:.1f} | {mb / avg:.2f} | {mb / avg / 8.0 * 100:.0f}")
+        if pmc:
+            f = pmc.get("FETCH_SIZE", ({}, 0))[0].get(nm)
+            w = pmc.get("WRITE_SIZE", ({}, 0))[0].get(nm)
+            moved = (f or 0) + (w or 0)
+            line += (f" | {'-' if f is None else f'{f / 1e6:.1f}'} | {'-' if w is None else f'{w / 1e6:.1f}'}"
+                     f" | {moved / r['algorithmic_bytes']:.2f}" if r["algorithmic_bytes"] > 4096 else " | - | - | -")
+        print(line + " |")
+    for label, (_, unit) in pmc.items():
+        print(f"\n{label}: one counter unit = {unit:.3f} KiB (from the 256 MiB copy of the same run).")
 
 
 def main():
@@ -502,7 +610,18 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--tiny", action="store_true", help="2-layer toy shape (plumbing check only)")
     ap.add_argument("--suite", default="llama", choices=["llama", "ops"])
+    ap.add_argument("--ops-launches", type=int, default=100, help="ops suite: launches per recorded graph")
+    ap.add_argument("--ops-quick", action="store_true",
+                    help="ops suite: one replay per op, no settling (for counter runs, which serialise launches)")
+    ap.add_argument("--summarize-ops", metavar="JSON", help="print the per-op table from an ops-suite JSON "
+                    "line and the rocprofv3 CSVs of the same command (no GPU needed)")
+    ap.add_argument("--kernel-trace", metavar="CSV")
+    ap.add_argument("--pmc-fetch", metavar="CSV")
+    ap.add_argument("--pmc-write", metavar="CSV")
     args = ap.parse_args()
+    if args.summarize_ops:
+        summarize_ops(args)
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one MI355X: the operator path has no multi-GPU part "
               "(run with --gpus 1)", file=sys.stderr)

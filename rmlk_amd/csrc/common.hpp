@@ -181,12 +181,25 @@ inline int32_t split_pieces(int rank, const int64_t *shape, const int64_t (*stri
             for (int p = 0; p < NP; ++p)
                 if (strides[p][d] >= kStrideLimit || strides[p][d] <= -kStrideLimit)
                     strides_fit = false;
-    if (numel <= kPieceElems && strides_fit) return fn(shape, offsets);
+    // the kernels may accumulate element offsets in 32 bits: the farthest element of every operand
+    // must lie within 2^31 elements of its first
+    bool extents_fit = true;
+    for (int p = 0; p < NP; ++p) {
+        int64_t reach_up = 0, reach_down = 0;
+        for (int d = 0; d < rank; ++d) {
+            if (shape[d] <= 1 || strides[p][d] == 0 || !strides_fit) continue;
+            const int64_t span = (shape[d] - 1) * strides[p][d];
+            if (span > 0) reach_up += span; else reach_down -= span;
+        }
+        if (reach_up >= kStrideLimit || reach_down >= kStrideLimit) extents_fit = false;
+    }
+    if (numel <= kPieceElems && strides_fit && extents_fit) return fn(shape, offsets);
     int d0 = 0;
     while (d0 < rank - 1 && shape[d0] == 1) ++d0;
     if (shape[d0] == 1) return RMLK_ERR_TOO_LARGE;  // a single element cannot be too large
     const int64_t inner = numel / shape[d0];
     int64_t rows_per = inner >= kPieceElems ? 1 : kPieceElems / inner;
+    if (rows_per >= shape[d0]) rows_per = (shape[d0] + 1) / 2;   // cut for the extents alone
     for (int p = 0; p < NP; ++p)
         if (strides[p][d0] >= kStrideLimit || strides[p][d0] <= -kStrideLimit) rows_per = 1;
     int64_t sub[kMaxRank];

@@ -16,6 +16,8 @@
 // The vector kernels write with streaming stores.
 #pragma once
 
+#include <type_traits>
+
 #include "nd_index.hpp"
 
 namespace rmlk {
@@ -23,7 +25,6 @@ namespace rmlk {
 constexpr int kEwBlock = 256;
 constexpr int kEwVec = 4;
 constexpr int kEwUnroll = 4;       // independent vector accesses in flight per lane and operand
-constexpr int kEwBlocksPerCu = 8;  // grid cap of the nd kernels (they loop beyond it)
 constexpr int kEwChunk = kEwBlock * kEwUnroll;      // vectors a block of the flat kernel takes per trip
 
 // An input's way through the innermost run.
@@ -126,37 +127,44 @@ struct EwUnrollDim {
 // plan operands: 0 = a, 1 = b, 2 = out. For VEC == 4 the host has divided the innermost dim by 4
 // and multiplied the innermost strides by 4; AM / BM say how the operand walks the innermost run.
 // UNR is kEwUnroll (positions along the unroll dim) or 1. VEC == 1 ignores AM / BM.
+template <int NP, int VEC>
+using EwIndexArg = std::conditional_t<VEC == 1, NdPlan<NP>, NdIndex4<NP>>;
+
 template <typename F, typename TA, typename TB, typename TO, int VEC, int UNR, int AM, int BM>
-__global__ __launch_bounds__(kEwBlock) void binary_nd_kernel(NdPlan<3> pl, EwUnrollDim<3> ud,
+__global__ __launch_bounds__(kEwBlock) void binary_nd_kernel(EwIndexArg<3, VEC> pl, EwUnrollDim<3> ud,
                                                              const TA *__restrict__ a,
                                                              const TB *__restrict__ b,
                                                              TO *__restrict__ out, uint32_t n_items) {
-    const uint32_t step = gridDim.x * kEwBlock;
-    uint32_t i = blockIdx.x * kEwBlock + threadIdx.x;
     if constexpr (VEC == 1) {
-        for (; i < n_items; i += step) {
+        const uint32_t step = gridDim.x * kEwBlock;
+        for (uint32_t i = blockIdx.x * kEwBlock + threadIdx.x; i < n_items; i += step) {
             int64_t offs[3];
             nd_offsets<3>(pl, i, offs);
             out[offs[2]] = F::apply(a[offs[0]], b[offs[1]]);
         }
     } else {
-        for (; i < n_items; i += step) {
-            int64_t offs[3];
-            nd_offsets<3>(pl, i, offs);
-            TA ra[UNR][kEwVec];
-            TB rb[UNR][kEwVec];
+        // one trip: the grid covers n_items (a loop here makes the compiler keep every choice of the
+        // index arithmetic live in scalar registers across it, more than there are)
+        // (lanes past the end work on item 0 and do not store: an early exit would put the load of
+        // n_items and a branch in front of every other kernel-argument load)
+        const uint32_t i_raw = blockIdx.x * kEwBlock + threadIdx.x;
+        const bool live = i_raw < n_items;
+        const uint32_t i = live ? i_raw : 0;
+        int32_t offs[3];
+        nd4_offsets<3>(pl, i, offs);
+        TA ra[UNR][kEwVec];
+        TB rb[UNR][kEwVec];
 #pragma unroll
-            for (int u = 0; u < UNR; ++u) {
-                load_op<AM, false>(a + offs[0] + static_cast<int64_t>(u) * ud.stride[0], ra[u]);
-                load_op<BM, false>(b + offs[1] + static_cast<int64_t>(u) * ud.stride[1], rb[u]);
-            }
+        for (int u = 0; u < UNR; ++u) {
+            load_op<AM, true>(a + (offs[0] + u * ud.stride[0]), ra[u]);
+            load_op<BM, true>(b + (offs[1] + u * ud.stride[1]), rb[u]);
+        }
 #pragma unroll
-            for (int u = 0; u < UNR; ++u) {
-                TO ro[kEwVec];
+        for (int u = 0; u < UNR; ++u) {
+            TO ro[kEwVec];
 #pragma unroll
-                for (int j = 0; j < kEwVec; ++j) ro[j] = F::apply(ra[u][j], rb[u][j]);
-                store_vec(out + offs[2] + static_cast<int64_t>(u) * ud.stride[2], ro);
-            }
+            for (int j = 0; j < kEwVec; ++j) ro[j] = F::apply(ra[u][j], rb[u][j]);
+            if (live) store_vec(out + (offs[2] + u * ud.stride[2]), ro);
         }
     }
 }
@@ -169,6 +177,7 @@ template <int NP>
 struct EwDecision {
     EwShape shape;
     NdPlan<NP> plan;
+    NdIndex4<NP> index; // what the nd<4> kernels take
     int inner0[NP];     // operand repeats one element along the innermost run
     int mode_bits;      // bit p set: input p repeats one element along the innermost run
     uint32_t n_items;   // loop trip count of the chosen kernel
@@ -212,7 +221,7 @@ inline bool ew_decide(EwDecision<NP> &dec, int rank, const int64_t *shape,
         dec.n_items = static_cast<uint32_t>(pl.numel);
         return true;
     }
-    if (pl.rank > 1 && vector_ok && pl.dim64[last] % kEwVec == 0) {
+    if (pl.rank > 1 && pl.rank <= kIndexRank && vector_ok && pl.dim64[last] % kEwVec == 0) {
         dec.shape = EwShape::Nd4;
         pl.dim64[last] /= kEwVec;
         pl.dim[last] = static_cast<uint32_t>(pl.dim64[last]);
@@ -246,6 +255,10 @@ inline bool ew_decide(EwDecision<NP> &dec, int rank, const int64_t *shape,
                 dec.n_items /= kEwUnroll;
             }
         }
+        static_assert(kEwVec == 4 && kEwUnroll == 4, "the shifts of the index");
+        int inner_shift[NP];
+        for (int p = 0; p < NP; ++p) inner_shift[p] = 2;
+        make_index4<NP>(dec.index, pl, inner_shift, dec.unrolled ? best : -1, 2);
         return true;
     }
     dec.shape = EwShape::Nd1;
@@ -264,13 +277,13 @@ inline void launch_binary_mode(hipStream_t stream, const EwDecision<3> &dec, con
         unsigned grid = chunk_grid(dec.n_items / kEwVec, kEwChunk);
         binary_flat_kernel<F, TA, TB, TO, AM, BM><<<grid, kEwBlock, 0, stream>>>(pa, pb, po, dec.n_items);
     } else {
-        unsigned grid = grid_for(dec.n_items, kEwBlock, kEwBlocksPerCu);
+        unsigned grid = (dec.n_items + kEwBlock - 1) / kEwBlock;      // one trip
         if (dec.unrolled)
             binary_nd_kernel<F, TA, TB, TO, kEwVec, kEwUnroll, AM, BM><<<grid, kEwBlock, 0, stream>>>(
-                dec.plan, dec.udim, pa, pb, po, dec.n_items);
+                dec.index, dec.udim, pa, pb, po, dec.n_items);
         else
             binary_nd_kernel<F, TA, TB, TO, kEwVec, 1, AM, BM><<<grid, kEwBlock, 0, stream>>>(
-                dec.plan, dec.udim, pa, pb, po, dec.n_items);
+                dec.index, dec.udim, pa, pb, po, dec.n_items);
     }
 }
 

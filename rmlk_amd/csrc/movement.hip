@@ -35,29 +35,38 @@ __device__ __forceinline__ U get(const U *p) {
     else return nt_load(p);
 }
 
-template <typename U, bool REPEATS>
-__global__ __launch_bounds__(kBlock) void copy_nd_kernel(NdPlan<2> pl, const U *__restrict__ in,
+template <typename OFF, typename PL>
+__device__ __forceinline__ void copy_offsets(const PL &pl, uint32_t i, OFF (&offs)[2]) {
+    if constexpr (std::is_same<PL, NdIndex4<2>>::value) nd4_offsets<2>(pl, i, offs);
+    else nd_offsets<2>(pl, i, offs);
+}
+
+// PL: NdIndex4<2> (at most four dims, 32-bit offsets, a dense side free of index arithmetic) or the
+// full NdPlan<2>.
+template <typename U, bool REPEATS, typename PL>
+__global__ __launch_bounds__(kBlock) void copy_nd_kernel(PL pl, const U *__restrict__ in,
                                                          U *__restrict__ out, uint32_t n) {
-    for (uint32_t base = blockIdx.x * kChunk; base < n; base += gridDim.x * kChunk) {
-        const uint32_t i0 = base + threadIdx.x;
-        if (base + kChunk <= n) {
-            U r[kUnroll];
-            int64_t oo[kUnroll];
+    using OFF = std::conditional_t<std::is_same<PL, NdIndex4<2>>::value, int32_t, int64_t>;
+    // one trip: the grid covers n in chunks (no loop for the compiler to hoist the index choices out of)
+    const uint32_t base = blockIdx.x * kChunk;
+    const uint32_t i0 = base + threadIdx.x;
+    if (base + kChunk <= n) {
+        U r[kUnroll];
+        OFF oo[kUnroll];
 #pragma unroll
-            for (int j = 0; j < kUnroll; ++j) {
-                int64_t offs[2];
-                nd_offsets<2>(pl, i0 + j * kBlock, offs);
-                r[j] = get<REPEATS>(in + offs[0]);
-                oo[j] = offs[1];
-            }
+        for (int j = 0; j < kUnroll; ++j) {
+            OFF offs[2];
+            copy_offsets(pl, i0 + j * kBlock, offs);
+            r[j] = get<REPEATS>(in + offs[0]);
+            oo[j] = offs[1];
+        }
 #pragma unroll
-            for (int j = 0; j < kUnroll; ++j) put(out + oo[j], r[j]);
-        } else {
-            for (uint32_t i = i0; i < n; i += kBlock) {
-                int64_t offs[2];
-                nd_offsets<2>(pl, i, offs);
-                put(out + offs[1], get<REPEATS>(in + offs[0]));
-            }
+        for (int j = 0; j < kUnroll; ++j) put(out + oo[j], r[j]);
+    } else {
+        for (uint32_t i = i0; i < n; i += kBlock) {
+            OFF offs[2];
+            copy_offsets(pl, i, offs);
+            put(out + offs[1], get<REPEATS>(in + offs[0]));
         }
     }
 }
@@ -91,12 +100,18 @@ int32_t launch_copy_units(hipStream_t s, NdPlan<2> &pl, const void *in, void *ou
         bool repeats = false;
         for (int d = 0; d < pl.rank; ++d)
             if (pl.stride[0][d] == 0 && pl.dim64[d] > 1) repeats = true;
-        if (repeats)
-            copy_nd_kernel<U, true><<<grid, kBlock, 0, s>>>(pl, static_cast<const U *>(in),
-                                                            static_cast<U *>(out), n);
-        else
-            copy_nd_kernel<U, false><<<grid, kBlock, 0, s>>>(pl, static_cast<const U *>(in),
-                                                             static_cast<U *>(out), n);
+        const U *pi = static_cast<const U *>(in);
+        U *po = static_cast<U *>(out);
+        grid = (n + kChunk - 1) / kChunk;      // one trip
+        NdIndex4<2> ix;
+        const int unit_shift[2] = {0, 0};
+        if (make_index4<2>(ix, pl, unit_shift, -1, 0)) {
+            if (repeats) copy_nd_kernel<U, true, NdIndex4<2>><<<grid, kBlock, 0, s>>>(ix, pi, po, n);
+            else copy_nd_kernel<U, false, NdIndex4<2>><<<grid, kBlock, 0, s>>>(ix, pi, po, n);
+        } else {
+            if (repeats) copy_nd_kernel<U, true, NdPlan<2>><<<grid, kBlock, 0, s>>>(pl, pi, po, n);
+            else copy_nd_kernel<U, false, NdPlan<2>><<<grid, kBlock, 0, s>>>(pl, pi, po, n);
+        }
     }
     return launch_status();
 }

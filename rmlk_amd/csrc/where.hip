@@ -59,36 +59,36 @@ __global__ __launch_bounds__(kEwBlock) void where_flat_kernel(const T *__restric
 // plan operands: 0 = x, 1 = y, 2 = cond, 3 = out. XM / YM: how x and y walk the innermost run
 // (VEC == 4 only; the condition walks it densely).
 template <typename T, int VEC, int UNR, int XM, int YM>
-__global__ __launch_bounds__(kEwBlock) void where_nd_kernel(NdPlan<4> pl, EwUnrollDim<4> ud,
+__global__ __launch_bounds__(kEwBlock) void where_nd_kernel(EwIndexArg<4, VEC> pl, EwUnrollDim<4> ud,
                                                             const T *__restrict__ x,
                                                             const T *__restrict__ y,
                                                             const uint8_t *__restrict__ c,
                                                             T *__restrict__ out, uint32_t n_items) {
-    const uint32_t step = gridDim.x * kEwBlock;
-    uint32_t i = blockIdx.x * kEwBlock + threadIdx.x;
     if constexpr (VEC == 1) {
-        for (; i < n_items; i += step) {
+        const uint32_t step = gridDim.x * kEwBlock;
+        for (uint32_t i = blockIdx.x * kEwBlock + threadIdx.x; i < n_items; i += step) {
             int64_t offs[4];
             nd_offsets<4>(pl, i, offs);
             out[offs[3]] = c[offs[2]] ? x[offs[0]] : y[offs[1]];
         }
     } else {
-        for (; i < n_items; i += step) {
-            int64_t offs[4];
-            nd_offsets<4>(pl, i, offs);
-            T rx[UNR][kEwVec], ry[UNR][kEwVec];
-            uint8_t rc[UNR][kEwVec];
+        // one trip: the grid covers n_items; lanes past the end work on item 0 and do not store
+        const uint32_t i_raw = blockIdx.x * kEwBlock + threadIdx.x;
+        const bool live = i_raw < n_items;
+        const uint32_t i = live ? i_raw : 0;
+        int32_t offs[4];
+        nd4_offsets<4>(pl, i, offs);
+        T rx[UNR][kEwVec], ry[UNR][kEwVec];
+        uint8_t rc[UNR][kEwVec];
 #pragma unroll
-            for (int u = 0; u < UNR; ++u) {
-                load_op<XM, false>(x + offs[0] + static_cast<int64_t>(u) * ud.stride[0], rx[u]);
-                load_op<YM, false>(y + offs[1] + static_cast<int64_t>(u) * ud.stride[1], ry[u]);
-                load_op<kEwDense, false>(c + offs[2] + static_cast<int64_t>(u) * ud.stride[2], rc[u]);
-            }
-#pragma unroll
-            for (int u = 0; u < UNR; ++u)
-                select_store(out + offs[3] + static_cast<int64_t>(u) * ud.stride[3], rx[u], ry[u],
-                             rc[u]);
+        for (int u = 0; u < UNR; ++u) {
+            load_op<XM, true>(x + (offs[0] + u * ud.stride[0]), rx[u]);
+            load_op<YM, true>(y + (offs[1] + u * ud.stride[1]), ry[u]);
+            load_op<kEwDense, true>(c + (offs[2] + u * ud.stride[2]), rc[u]);
         }
+#pragma unroll
+        for (int u = 0; u < UNR; ++u)
+            if (live) select_store(out + (offs[3] + u * ud.stride[3]), rx[u], ry[u], rc[u]);
     }
 }
 
@@ -102,13 +102,13 @@ void launch_where_mode(hipStream_t stream, const EwDecision<4> &dec, const T *x,
         where_flat_kernel<T, XM, YM><<<chunk_grid(dec.n_items / kEwVec, kEwChunk), kEwBlock, 0, stream>>>(
             x, y, c, out, dec.n_items);
     } else {
-        const unsigned grid = grid_for(dec.n_items, kEwBlock, kEwBlocksPerCu);
+        const unsigned grid = (dec.n_items + kEwBlock - 1) / kEwBlock;      // one trip
         if (dec.unrolled)
             where_nd_kernel<T, kEwVec, kEwUnroll, XM, YM><<<grid, kEwBlock, 0, stream>>>(
-                dec.plan, dec.udim, x, y, c, out, dec.n_items);
+                dec.index, dec.udim, x, y, c, out, dec.n_items);
         else
             where_nd_kernel<T, kEwVec, 1, XM, YM><<<grid, kEwBlock, 0, stream>>>(
-                dec.plan, dec.udim, x, y, c, out, dec.n_items);
+                dec.index, dec.udim, x, y, c, out, dec.n_items);
     }
 }
 
