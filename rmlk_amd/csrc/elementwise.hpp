@@ -154,10 +154,31 @@ __global__ __launch_bounds__(kEwBlock) void binary_nd_kernel(EwIndexArg<3, VEC> 
         nd4_offsets<3>(pl, i, offs);
         TA ra[UNR][kEwVec];
         TB rb[UNR][kEwVec];
+        // An operand that does not change along the lane's UNR positions is loaded once. Thousands of
+        // wavefronts asking for the same few lines of a small broadcast operand are a queue of their
+        // own in the L2, longest when the lines still have to come from HBM: four loads per lane of
+        // an 8 KB b cost the 64 MiB Add 0.4 us with b in the L2 and 1.3 us with b cold.
+        if (UNR > 1 && ud.stride[1] == 0) {
+            load_op<BM, false>(b + offs[1], rb[0]);
 #pragma unroll
-        for (int u = 0; u < UNR; ++u) {
-            load_op<AM, true>(a + (offs[0] + u * ud.stride[0]), ra[u]);
-            load_op<BM, true>(b + (offs[1] + u * ud.stride[1]), rb[u]);
+            for (int u = 0; u < UNR; ++u) load_op<AM, true>(a + (offs[0] + u * ud.stride[0]), ra[u]);
+#pragma unroll
+            for (int u = 1; u < UNR; ++u)
+#pragma unroll
+                for (int j = 0; j < kEwVec; ++j) rb[u][j] = rb[0][j];
+        } else if (UNR > 1 && ud.stride[0] == 0) {
+            load_op<AM, false>(a + offs[0], ra[0]);
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) load_op<BM, true>(b + (offs[1] + u * ud.stride[1]), rb[u]);
+#pragma unroll
+            for (int u = 1; u < UNR; ++u)
+#pragma unroll
+                for (int j = 0; j < kEwVec; ++j) ra[u][j] = ra[0][j];
+        } else {
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) load_op<AM, true>(a + (offs[0] + u * ud.stride[0]), ra[u]);
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) load_op<BM, true>(b + (offs[1] + u * ud.stride[1]), rb[u]);
         }
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {

@@ -80,11 +80,38 @@ __global__ __launch_bounds__(kEwBlock) void where_nd_kernel(EwIndexArg<4, VEC> p
         nd4_offsets<4>(pl, i, offs);
         T rx[UNR][kEwVec], ry[UNR][kEwVec];
         uint8_t rc[UNR][kEwVec];
+        // An operand that does not change along the lane's UNR positions is loaded once: thousands
+        // of wavefronts asking for the same few lines of a small broadcast operand are a queue of
+        // their own in the L2 (see binary_nd_kernel).
+        if (UNR > 1 && ud.stride[1] == 0) {
+            load_op<YM, false>(y + offs[1], ry[0]);
 #pragma unroll
-        for (int u = 0; u < UNR; ++u) {
-            load_op<XM, true>(x + (offs[0] + u * ud.stride[0]), rx[u]);
-            load_op<YM, true>(y + (offs[1] + u * ud.stride[1]), ry[u]);
-            load_op<kEwDense, true>(c + (offs[2] + u * ud.stride[2]), rc[u]);
+            for (int u = 0; u < UNR; ++u) {
+                load_op<XM, true>(x + (offs[0] + u * ud.stride[0]), rx[u]);
+                load_op<kEwDense, true>(c + (offs[2] + u * ud.stride[2]), rc[u]);
+            }
+#pragma unroll
+            for (int u = 1; u < UNR; ++u)
+#pragma unroll
+                for (int j = 0; j < kEwVec; ++j) ry[u][j] = ry[0][j];
+        } else if (UNR > 1 && ud.stride[0] == 0) {
+            load_op<XM, false>(x + offs[0], rx[0]);
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) {
+                load_op<YM, true>(y + (offs[1] + u * ud.stride[1]), ry[u]);
+                load_op<kEwDense, true>(c + (offs[2] + u * ud.stride[2]), rc[u]);
+            }
+#pragma unroll
+            for (int u = 1; u < UNR; ++u)
+#pragma unroll
+                for (int j = 0; j < kEwVec; ++j) rx[u][j] = rx[0][j];
+        } else {
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) {
+                load_op<XM, true>(x + (offs[0] + u * ud.stride[0]), rx[u]);
+                load_op<YM, true>(y + (offs[1] + u * ud.stride[1]), ry[u]);
+                load_op<kEwDense, true>(c + (offs[2] + u * ud.stride[2]), rc[u]);
+            }
         }
 #pragma unroll
         for (int u = 0; u < UNR; ++u)
