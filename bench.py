@@ -443,6 +443,8 @@ def run_ops_suite(args):
     gam = torch.rand(2048, device=dev, generator=g) + 0.5
     timed("fused_rmsnorm", lambda i: k.rmsnorm(xs[i], gam, ys[i], 4096, 2048, 1e-5), ns,
           2 * n * 4 + 8192)
+    timed("fused_rmsnorm_recip", lambda i: k.rmsnorm(xs[i], gam, ys[i], 4096, 2048, 1e-5, True), ns,
+          2 * n * 4 + 8192)
     sums = [torch.empty(n, device=dev) for _ in range(ns)]
     timed("fused_add_rmsnorm", lambda i: k.add_rmsnorm(xs[i], xs[(i + 1) % ns], gam, sums[i], ys[i],
                                                        4096, 2048, 1e-5), ns, 4 * n * 4 + 8192)
@@ -468,22 +470,17 @@ def run_ops_suite(args):
     sidx = [torch.tensor([[0, h, int(p)] for h in range(8)], device=dev, dtype=torch.int64)
             for p in np.random.default_rng(5).integers(0, 8192, size=ns)]
 
-    def scatter_copy(i):
-        j = i % nk
-        check(lib().rmlk_hip_memcpy_dtod(torch.cuda.current_stream().cuda_stream, outs[j].data_ptr(),
-                                         caches[j].data_ptr(), kv_n * 4), "rmlk_hip_memcpy_dtod")
-        k.scatter_nd(sidx[i % ns], rows[i % ns], outs[j], [1, 8, 8192, 64], 8, 3)
-    timed("scatter_nd_copy", scatter_copy, nk, 2 * kv_n * 4 + 8 * 64 * 4 + 192, kernels_per_call=2)
+    timed("scatter_nd_copy", lambda i: k.scatter_nd_copy(sidx[i % ns], rows[i % ns], caches[i % nk], outs[i % nk],
+                                                         [1, 8, 8192, 64], 8, 3), nk,
+          2 * kv_n * 4 + 8 * 64 * 4 + 192)
     timed("scatter_nd_inplace", lambda i: k.scatter_nd(sidx[i % ns], rows[i % ns], caches[i % nk],
                                                        [1, 8, 8192, 64], 8, 3), nk, 8 * 64 * 4 + 192)
     timed("slice_kv", lambda i: k.slice_(caches[i % nk], outs[i % nk], [1, 8, 8192, 64], [0, 0, 0, 0],
                                          [1, 1, 1, 1], [1, 8, 8191, 64]), nk, 2 * 8 * 8191 * 64 * 4)
 
-    def concat_kv(i):
-        j = i % nk
-        k.concat_into(caches[j][:8 * 8191 * 64], outs[j], [1, 8, 8191, 64], [1, 8, 8192, 64], 2, 0)
-        k.concat_into(rows[i % ns], outs[j], [1, 8, 1, 64], [1, 8, 8192, 64], 2, 8191)
-    timed("concat_kv", concat_kv, nk, 2 * kv_n * 4, kernels_per_call=2)
+    timed("concat_kv", lambda i: k.concat([caches[i % nk][:8 * 8191 * 64], rows[i % ns]], outs[i % nk],
+                                          [[1, 8, 8191, 64], [1, 8, 1, 64]], [1, 8, 8192, 64], 2), nk,
+          2 * kv_n * 4)
     del caches, outs
     table = torch.randn(128256, 2048, device=dev, generator=g)
     idx4 = [torch.randint(0, 128256, (4096,), device=dev, generator=g) for _ in range(ns)]

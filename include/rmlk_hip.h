@@ -203,6 +203,15 @@ int32_t rmlk_hip_concat(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *in
                         const rmlk_dims *out_shape, int32_t axis, int64_t axis_offset,
                         const void *in, void *out);
 
+/* Concat of all `n_inputs` dense inputs (shapes in_shapes[k], device pointers ins[k]; both arrays
+ * are HOST memory) along `axis` into dense `out` (out_shape, whose extent along `axis` is the sum
+ * of the inputs'). One launch for up to 8 inputs (the growing KV cache plus the new row costs one
+ * launch, not two); more inputs, or very large ones, take one strided copy per input.
+ * ref: runtime/src/providers/cuda/backend/concat.rs:28-76 (the whole host loop). */
+int32_t rmlk_hip_concat_many(rmlk_stream_t stream, int32_t dtype, int32_t n_inputs,
+                             const rmlk_dims *in_shapes, const void *const *ins,
+                             const rmlk_dims *out_shape, int32_t axis, void *out);
+
 /* Gather along `axis`: out[outer, j, inner] = data[outer, idx[j], inner], j < n_idx; negative
  * indices wrap once. idx_dtype INT32 or INT64. An index outside [-dim, dim) writes zeros for that
  * row and stores 1 to *err_flag (device int32, may be NULL); the host reads it when it chooses.
@@ -232,6 +241,18 @@ int32_t rmlk_hip_scatter_nd(rmlk_stream_t stream, int32_t reduction, int32_t dty
                             const rmlk_dims *data_shape, int64_t n_tuples, int32_t tuple_size,
                             const int64_t *idx, const void *updates, void *out,
                             int32_t *err_flag);
+
+/* ScatterND (reduction none) with the ONNX copy semantics in ONE pass: out = data with the
+ * addressed slices taken from `updates` (`out` is written everywhere, `data` is only read; they
+ * may be the same buffer). Up to 64 tuples of 16-byte aligned slices take one launch that reads
+ * data and writes out once; anything else copies data to out and calls rmlk_hip_scatter_nd. When
+ * several tuples address one slice, the last one wins. Index rules and *err_flag as above.
+ * ref: runtime/src/providers/cuda/backend/scatter_nd.rs:128-129 (memcpy_dtod of data, then the
+ * scatter kernel). */
+int32_t rmlk_hip_scatter_nd_copy(rmlk_stream_t stream, int32_t dtype, const rmlk_dims *data_shape,
+                                 int64_t n_tuples, int32_t tuple_size, const int64_t *idx,
+                                 const void *updates, const void *data, void *out,
+                                 int32_t *err_flag);
 
 /* Trilu on a dense [batch, rows, cols] view: keeps the upper (col >= row + k) or lower
  * (col <= row + k) triangle and WRITES ZERO elsewhere (the reference leaves those untouched).

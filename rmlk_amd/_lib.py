@@ -89,6 +89,10 @@ SIGNATURES = {
                                   c_void_p]),
     "rmlk_hip_gather": (c_int32, [c_void_p, c_int32, c_int32, _PD, c_int32, c_int64, c_void_p,
                                   c_void_p, c_void_p, c_void_p]),
+    "rmlk_hip_concat_many": (c_int32, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, _PD, c_int32,
+                                       c_void_p]),
+    "rmlk_hip_scatter_nd_copy": (c_int32, [c_void_p, c_int32, _PD, c_int64, c_int32, c_void_p, c_void_p,
+                                           c_void_p, c_void_p, c_void_p]),
     "rmlk_hip_scatter_nd": (c_int32, [c_void_p, c_int32, c_int32, _PD, c_int64, c_int32, c_void_p,
                                       c_void_p, c_void_p, c_void_p]),
     "rmlk_hip_trilu": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int32, c_int64,

@@ -268,13 +268,37 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const U *__restrict
     for (uint32_t base = blockIdx.x * kChunk; base < n_units; base += gridDim.x * kChunk) {
         const uint32_t i0 = base + threadIdx.x;
         if (base + kChunk <= n_units) {
+            // the index loads of all kUnroll units, then their data loads, then the stores: each
+            // group is in flight together (a fetch at a time would wait for an index, then for its
+            // data, kUnroll times over)
             U r[kUnroll];
+            I raw[kUnroll];
+            uint32_t col[kUnroll], outer[kUnroll];
 #pragma unroll
-            for (int j = 0; j < kUnroll; ++j)
-                r[j] = gather_fetch<U, I>(data, idx, i0 + j * kBlock, row_units, row_div, n_idx, idx_div,
-                                          axis_dim, err);
+            for (int j = 0; j < kUnroll; ++j) {
+                const uint32_t e = i0 + j * kBlock;
+                const uint32_t row = row_div.div(e);
+                col[j] = e - row * row_units;
+                outer[j] = idx_div.div(row);
+                raw[j] = idx[row - outer[j] * n_idx];
+            }
+            bool ok[kUnroll];
 #pragma unroll
-            for (int j = 0; j < kUnroll; ++j) put(out + i0 + j * kBlock, r[j]);
+            for (int j = 0; j < kUnroll; ++j) {
+                int64_t ix = static_cast<int64_t>(raw[j]);
+                if (ix < 0) ix += axis_dim;
+                ok[j] = ix >= 0 && ix < axis_dim;
+                if (!ok[j]) ix = 0;
+                r[j] = nt_load(data + (static_cast<int64_t>(outer[j]) * axis_dim + ix) * row_units + col[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j) {
+                if (!ok[j]) {
+                    r[j] = U{};
+                    if (err) *err = 1;
+                }
+                put(out + i0 + j * kBlock, r[j]);
+            }
         } else {
             for (uint32_t i = i0; i < n_units; i += kBlock)
                 put(out + i, gather_fetch<U, I>(data, idx, i, row_units, row_div, n_idx, idx_div, axis_dim, err));
@@ -374,6 +398,112 @@ __global__ __launch_bounds__(kBlock) void scatter_nd_kernel(ScatterPlan sp,
         } else {
             atomic_reduce<RED, T>(out + off * slice_units + c, upd[e]);
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// ScatterND with ONNX copy semantics in one launch: out = data, except for the slices the index
+// tuples address, which come from `updates`. For few tuples (at most a wavefront's lanes): every
+// wavefront lets lane t work out where tuple t lands, a ballot says which of them touch the block's
+// chunk (mostly none), and a unit inside such a slice is read from the updates instead of the data.
+// Later tuples win over earlier ones, as a sequential scatter would have it.
+constexpr uint32_t kMaxFusedTuples = kWave;
+
+__global__ __launch_bounds__(kBlock) void scatter_copy_kernel(ScatterPlan sp,
+                                                              const int64_t *__restrict__ idx,
+                                                              const U128 *__restrict__ upd,
+                                                              const U128 *__restrict__ data,
+                                                              U128 *__restrict__ out, uint32_t n,
+                                                              uint32_t n_tuples, uint32_t slice_units,
+                                                              int32_t *__restrict__ err) {
+    const uint32_t base = blockIdx.x * kChunk;
+    const uint32_t lane = threadIdx.x % kWave;
+    // lane t: first unit of the slice of tuple t
+    uint32_t start = 0;
+    bool valid = false;
+    if (lane < n_tuples) {
+        int64_t off = 0;
+        bool bad = false;
+#pragma unroll
+        for (int t = 0; t < kMaxRank; ++t) {
+            if (t < sp.tuple_size) {
+                int64_t ix = idx[static_cast<int64_t>(lane) * sp.tuple_size + t];
+                if (ix < 0) ix += sp.dim[t];
+                if (ix < 0 || ix >= sp.dim[t]) bad = true;
+                off += ix * sp.stride[t];
+            }
+        }
+        if (bad) {
+            if (err && blockIdx.x == 0 && threadIdx.x < kWave) *err = 1;
+        } else {
+            valid = true;
+            start = static_cast<uint32_t>(off) * slice_units;
+        }
+    }
+    const uint32_t chunk_end = base + kChunk < n ? base + kChunk : n;
+    const bool touches = valid && start < chunk_end && start + slice_units > base;
+    uint64_t hits = __ballot(touches);
+    U128 r[kUnroll];
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+        const uint32_t i = base + threadIdx.x + j * kBlock;
+        if (i < n) r[j] = nt_load(data + i);
+    }
+    while (hits) {       // uniform; ascending tuple order, so the last one to address a unit wins
+        const int t = __builtin_ctzll(hits);
+        hits &= hits - 1;
+        const uint32_t s0 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(start), t));
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const uint32_t i = base + threadIdx.x + j * kBlock;
+            if (i < n && i >= s0 && i - s0 < slice_units)
+                r[j] = upd[static_cast<uint64_t>(t) * slice_units + (i - s0)];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+        const uint32_t i = base + threadIdx.x + j * kBlock;
+        if (i < n) put(out + i, r[j]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Concat of up to kMaxConcatInputs inputs in one launch: blockIdx.y picks the input, blockIdx.x a
+// chunk of it (the grid is sized for the largest; blocks past the end of a smaller input leave).
+// Input k is [outer, row_units[k]] and lands at column out_off[k] of [outer, out_row_units].
+constexpr int kMaxConcatInputs = 8;
+struct ConcatArgs {
+    const void *in[kMaxConcatInputs];
+    uint32_t n_units[kMaxConcatInputs];
+    uint32_t row_units[kMaxConcatInputs];
+    uint32_t row_mul[kMaxConcatInputs], row_shr[kMaxConcatInputs];
+    uint64_t out_off[kMaxConcatInputs];
+    uint64_t out_row_units;
+};
+
+template <typename U>
+__global__ __launch_bounds__(kBlock) void concat_kernel(ConcatArgs a, U *__restrict__ out) {
+    const int k = blockIdx.y;
+    const uint32_t n = a.n_units[k];
+    const uint32_t base = blockIdx.x * kChunk;
+    if (base >= n) return;
+    const U *__restrict__ in = static_cast<const U *>(a.in[k]);
+    const uint32_t row_units = a.row_units[k], mul = a.row_mul[k], shr = a.row_shr[k];
+    const uint64_t off = a.out_off[k];
+    U r[kUnroll];
+    uint64_t dst[kUnroll];
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+        const uint32_t i = base + threadIdx.x + j * kBlock;
+        const uint32_t e = i < n ? i : n - 1;
+        const uint32_t o = row_units == 1 ? e : (__umulhi(e, mul) >> shr);
+        dst[j] = o * a.out_row_units + off + (e - o * row_units);
+        r[j] = nt_load(in + e);
+    }
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+        const uint32_t i = base + threadIdx.x + j * kBlock;
+        if (i < n) put(out + dst[j], r[j]);
     }
 }
 
@@ -641,6 +771,139 @@ extern "C" int32_t rmlk_hip_concat(rmlk_stream_t stream, int32_t dtype, const rm
     const int64_t base = axis_offset * st[1][axis];
     return strided_copy(as_stream(stream), esize, rank, in_shape->v, st, in,
                         static_cast<char *>(out) + base * esize);
+}
+
+extern "C" int32_t rmlk_hip_scatter_nd_copy(rmlk_stream_t stream, int32_t dtype,
+                                            const rmlk_dims *data_shape, int64_t n_tuples,
+                                            int32_t tuple_size, const int64_t *idx, const void *updates,
+                                            const void *data, void *out, int32_t *err_flag) {
+    if (!dims_ok(data_shape)) return RMLK_ERR_BAD_RANK;
+    const int rank = data_shape->rank;
+    if (tuple_size < 1 || tuple_size > rank) return RMLK_ERR_INVALID_ARGUMENT;
+    const int esize = dtype_size(dtype);
+    if (!esize) return RMLK_ERR_UNSUPPORTED;
+    const int64_t numel = dims_numel(data_shape);
+    if (n_tuples < 0 || numel < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (numel == 0) return RMLK_OK;
+    if (!data || !out) return RMLK_ERR_NULL_POINTER;
+    int64_t slice_len = 1;
+    for (int d = tuple_size; d < rank; ++d) slice_len *= data_shape->v[d];
+    const int64_t bytes = numel * esize, slice_bytes = slice_len * esize;
+    auto aligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    const bool fused = n_tuples >= 1 && n_tuples <= static_cast<int64_t>(kMaxFusedTuples) && idx &&
+                       updates && slice_bytes % 16 == 0 && aligned(data) && aligned(out) &&
+                       aligned(updates) && bytes / 16 < ((int64_t)1 << 31);
+    if (!fused) {
+        if (data != out) {
+            const int32_t st = rmlk_hip_memcpy_dtod(stream, out, data, static_cast<size_t>(bytes));
+            if (st) return st;
+        }
+        return rmlk_hip_scatter_nd(stream, RMLK_SCATTER_NONE, dtype, data_shape, n_tuples, tuple_size,
+                                   idx, updates, out, err_flag);
+    }
+    ScatterPlan sp{};
+    sp.tuple_size = tuple_size;
+    int64_t stride = 1;
+    for (int t = tuple_size - 1; t >= 0; --t) {
+        sp.dim[t] = data_shape->v[t];
+        sp.stride[t] = stride;
+        stride *= data_shape->v[t];
+    }
+    const uint32_t n = static_cast<uint32_t>(bytes / 16);
+    scatter_copy_kernel<<<(n + kChunk - 1) / kChunk, kBlock, 0, as_stream(stream)>>>(
+        sp, idx, static_cast<const U128 *>(updates), static_cast<const U128 *>(data),
+        static_cast<U128 *>(out), n, static_cast<uint32_t>(n_tuples),
+        static_cast<uint32_t>(slice_bytes / 16), err_flag);
+    return launch_status();
+}
+
+namespace {
+template <typename U>
+int32_t launch_concat_units(hipStream_t s, const ConcatArgs &a, int n_in, uint32_t largest, void *out) {
+    dim3 grid((largest + kChunk - 1) / kChunk, static_cast<unsigned>(n_in));
+    concat_kernel<U><<<grid, kBlock, 0, s>>>(a, static_cast<U *>(out));
+    return launch_status();
+}
+}  // namespace
+
+extern "C" int32_t rmlk_hip_concat_many(rmlk_stream_t stream, int32_t dtype, int32_t n_inputs,
+                                        const rmlk_dims *in_shapes, const void *const *ins,
+                                        const rmlk_dims *out_shape, int32_t axis, void *out) {
+    if (n_inputs < 1 || !in_shapes || !ins) return RMLK_ERR_INVALID_ARGUMENT;
+    if (!dims_ok(out_shape)) return RMLK_ERR_BAD_RANK;
+    const int rank = out_shape->rank;
+    if (axis < 0 || axis >= rank) return RMLK_ERR_INVALID_ARGUMENT;
+    const int esize = dtype_size(dtype);
+    if (!esize) return RMLK_ERR_UNSUPPORTED;
+    int64_t total = 0, outer = 1, inner = 1;
+    for (int d = 0; d < axis; ++d) outer *= out_shape->v[d];
+    for (int d = axis + 1; d < rank; ++d) inner *= out_shape->v[d];
+    for (int k = 0; k < n_inputs; ++k) {
+        if (!dims_ok(&in_shapes[k]) || in_shapes[k].rank != rank) return RMLK_ERR_SIZE_MISMATCH;
+        for (int d = 0; d < rank; ++d) {
+            if (in_shapes[k].v[d] < 0) return RMLK_ERR_INVALID_ARGUMENT;
+            if (d != axis && in_shapes[k].v[d] != out_shape->v[d]) return RMLK_ERR_SIZE_MISMATCH;
+        }
+        total += in_shapes[k].v[axis];
+    }
+    if (total != out_shape->v[axis]) return RMLK_ERR_SIZE_MISMATCH;
+    if (dims_numel(out_shape) < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (dims_numel(out_shape) == 0) return RMLK_OK;
+    if (!out) return RMLK_ERR_NULL_POINTER;
+    // one launch when every input's rows and landing columns are whole units of one width
+    int unit = 16;
+    bool one_launch = n_inputs <= kMaxConcatInputs && outer < ((int64_t)1 << 31);
+    int64_t col = 0;
+    for (int k = 0; k < n_inputs && one_launch; ++k) {
+        const int64_t row_bytes = in_shapes[k].v[axis] * inner * esize;
+        if (row_bytes == 0) continue;
+        if (!ins[k]) return RMLK_ERR_NULL_POINTER;
+        if (row_bytes * outer >= ((int64_t)1 << 31) * esize) one_launch = false;
+        while (unit > esize && (row_bytes % unit || (col * inner * esize) % unit ||
+                                reinterpret_cast<uintptr_t>(ins[k]) % unit))
+            unit >>= 1;
+        col += in_shapes[k].v[axis];
+    }
+    while (unit > esize && ((total * inner * esize) % unit || reinterpret_cast<uintptr_t>(out) % unit))
+        unit >>= 1;
+    if (!one_launch) {
+        int64_t off = 0;
+        for (int k = 0; k < n_inputs; ++k) {
+            const int32_t st = rmlk_hip_concat(stream, dtype, &in_shapes[k], out_shape, axis, off, ins[k], out);
+            if (st) return st;
+            off += in_shapes[k].v[axis];
+        }
+        return RMLK_OK;
+    }
+    ConcatArgs a{};
+    a.out_row_units = static_cast<uint64_t>(total * inner * esize / unit);
+    uint32_t largest = 0;
+    int n_in = 0;
+    col = 0;
+    for (int k = 0; k < n_inputs; ++k) {
+        const int64_t row_units = in_shapes[k].v[axis] * inner * esize / unit;
+        if (row_units > 0) {
+            const FastDiv fd(static_cast<uint32_t>(row_units));
+            a.in[n_in] = ins[k];
+            a.row_units[n_in] = static_cast<uint32_t>(row_units);
+            a.row_mul[n_in] = fd.mul;
+            a.row_shr[n_in] = fd.shr;
+            a.n_units[n_in] = static_cast<uint32_t>(row_units * outer);
+            a.out_off[n_in] = static_cast<uint64_t>(col * inner * esize / unit);
+            if (a.n_units[n_in] > largest) largest = a.n_units[n_in];
+            ++n_in;
+        }
+        col += in_shapes[k].v[axis];
+    }
+    if (n_in == 0) return RMLK_OK;
+    hipStream_t s = as_stream(stream);
+    switch (unit) {
+        case 1: return launch_concat_units<uint8_t>(s, a, n_in, largest, out);
+        case 2: return launch_concat_units<uint16_t>(s, a, n_in, largest, out);
+        case 4: return launch_concat_units<uint32_t>(s, a, n_in, largest, out);
+        case 8: return launch_concat_units<uint64_t>(s, a, n_in, largest, out);
+        default: return launch_concat_units<U128>(s, a, n_in, largest, out);
+    }
 }
 
 extern "C" int32_t rmlk_hip_gather(rmlk_stream_t stream, int32_t dtype, int32_t idx_dtype,

@@ -74,6 +74,14 @@ __device__ __forceinline__ T wave_max(T v) {
     return cd > ab ? cd : ab;
 }
 
+// sum / n in double. For n a power of two the quotient is the product with 1 / n, exactly (a change
+// of exponent), and the multiply is one instruction where the IEEE division is a chain of thirty
+// between a wavefront's last load and its first store.
+__device__ __forceinline__ double mean_of(double sum, int64_t n) {
+    if ((n & (n - 1)) == 0) return sum * (1.0 / static_cast<double>(n));
+    return sum / static_cast<double>(n);
+}
+
 // ---- ReduceMean over trailing contiguous elements: [rows, cols] -> [rows] ---------------------
 // kGroup lanes cooperate on a row: kWave (a wavefront per row) or kBlock (a block per row).
 template <typename T, int VEC, int kGroup>
@@ -123,7 +131,7 @@ __global__ __launch_bounds__(kBlock) void mean_rows_kernel(const T *__restrict__
         }
         acc = wave_sum(acc);
         if constexpr (kGroup == kWave) {
-            if (lane_in_group == 0) out[row] = static_cast<T>(acc / static_cast<double>(cols));
+            if (lane_in_group == 0) out[row] = static_cast<T>(mean_of(acc, cols));
         } else {
             const int wave = threadIdx.x / kWave;
             if ((threadIdx.x % kWave) == 0) partial[wave] = acc;
@@ -132,7 +140,7 @@ __global__ __launch_bounds__(kBlock) void mean_rows_kernel(const T *__restrict__
                 double t = 0.0;
 #pragma unroll
                 for (int w = 0; w < kWavesPerBlock; ++w) t += partial[w];
-                out[row] = static_cast<T>(t / static_cast<double>(cols));
+                out[row] = static_cast<T>(mean_of(t, cols));
             }
             __syncthreads();
         }
@@ -181,11 +189,14 @@ __device__ __forceinline__ float neg_inf<float>() {
 // the fly with exactly the roundings of the separate Div (Mul) and Add kernels.
 template <typename T>
 struct PlainRows {
+    static constexpr bool kMasked = false;
     const T *in;
     __device__ __forceinline__ Vec<T, 4> load(int64_t row, int c, int32_t cols) const {
         // (the scores are read once: streaming loads, 196 -> 190 us on 65536 rows of 2048)
         return nt_load(reinterpret_cast<const Vec<T, 4> *>(in + row * cols) + c);
     }
+    __device__ __forceinline__ Vec<T, 4> load_mask(int64_t, int) const { return Vec<T, 4>{}; }
+    __device__ __forceinline__ void combine(Vec<T, 4> &, const Vec<T, 4> &) const {}
 };
 
 // row -> offset into a mask that is broadcast over some of the leading dims
@@ -206,16 +217,20 @@ struct ScaledMaskedRows {
     const T *mask;
     T scale;
     RowMap map;
+    static constexpr bool kMasked = true;
+    // the kernel issues every load of a row (scores, then mask) before it combines the first pair
     __device__ __forceinline__ Vec<T, 4> load(int64_t row, int c, int32_t cols) const {
-        Vec<T, 4> x = nt_load(reinterpret_cast<const Vec<T, 4> *>(in + row * cols) + c);
-        Vec<T, 4> m = reinterpret_cast<const Vec<T, 4> *>(
-            mask + map.offset(static_cast<uint32_t>(row)))[c];
+        return nt_load(reinterpret_cast<const Vec<T, 4> *>(in + row * cols) + c);
+    }
+    __device__ __forceinline__ Vec<T, 4> load_mask(int64_t row, int c) const {
+        return reinterpret_cast<const Vec<T, 4> *>(mask + map.offset(static_cast<uint32_t>(row)))[c];
+    }
+    __device__ __forceinline__ void combine(Vec<T, 4> &x, const Vec<T, 4> &m) const {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const T scaled = MUL ? x.v[j] * scale : x.v[j] / scale;
             x.v[j] = scaled + m.v[j];
         }
-        return x;
     }
 };
 
@@ -231,16 +246,31 @@ __global__ __launch_bounds__(kBlock) void softmax_regs_kernel(Rows src, T *__res
     const int nv = cols / 4;
     for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock; row0 < rows;
          row0 += static_cast<int64_t>(gridDim.x) * kRowsPerBlock) {
-        const int64_t row = row0 + group;
-        const bool live = row < rows;
+        const bool live = row0 + group < rows;
+        const int64_t row = live ? row0 + group : rows - 1;    // idle groups read the last row again
         V x[NV];
         T m = neg_inf<T>();
+        // all loads of the row first (columns past the end read the last vector again and are
+        // replaced below): a branch per vector would leave one load in flight
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int c = lane_in_group + i * kGroup;
-            if (live && c < nv) {
-                x[i] = src.load(row, c, cols);
-            } else {
+            x[i] = src.load(row, c < nv ? c : nv - 1, cols);
+        }
+        if constexpr (Rows::kMasked) {
+            V mk[NV];
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int c = lane_in_group + i * kGroup;
+                mk[i] = src.load_mask(row, c < nv ? c : nv - 1);
+            }
+#pragma unroll
+            for (int i = 0; i < NV; ++i) src.combine(x[i], mk[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = lane_in_group + i * kGroup;
+            if (!(live && c < nv)) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) x[i].v[j] = neg_inf<T>();
             }
@@ -288,7 +318,7 @@ __global__ __launch_bounds__(kBlock) void softmax_regs_kernel(Rows src, T *__res
                 V y;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) y.v[j] = x[i].v[j] * inv;
-                po[c] = y;
+                nt_store(po + c, y);
             }
         }
     }
@@ -405,40 +435,71 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(RmsSource src,
     const int lane_in_group = threadIdx.x % kGroup;
     const int group = threadIdx.x / kGroup;
     const int nv = cols / 4;
-    V g[NV];
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-        const int c = lane_in_group + i * kGroup;
-        if (c < nv) g[i] = reinterpret_cast<const V *>(gamma)[c];
-    }
     for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock; row0 < rows;
          row0 += static_cast<int64_t>(gridDim.x) * kRowsPerBlock) {
-        const int64_t row = row0 + group;
-        const bool live = row < rows;
+        const bool live = row0 + group < rows;
+        const int64_t row = live ? row0 + group : rows - 1;    // idle groups read the last row again
         const V *pv = reinterpret_cast<const V *>(src.x + row * cols);
         V xv[NV];
+        // every load of the row is issued before the first use (columns past the end read the last
+        // vector again and are masked below): a branch per vector would leave one load in flight
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = lane_in_group + i * kGroup;
+            xv[i] = nt_load(pv + (c < nv ? c : nv - 1));
+        }
+        // gamma after the row: its requests (the same 8 KB from every wavefront) queue behind the
+        // row's, not in front of them
+        V g[NV];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = lane_in_group + i * kGroup;
+            g[i] = reinterpret_cast<const V *>(gamma)[c < nv ? c : nv - 1];
+        }
+        if (src.slabs > 1) {
+            for (int z = 1; z < src.slabs; ++z) {
+                const V *pz = reinterpret_cast<const V *>(src.x + z * src.slab + row * cols);
+                V more[NV];
+#pragma unroll
+                for (int i = 0; i < NV; ++i) {
+                    const int c = lane_in_group + i * kGroup;
+                    more[i] = nt_load(pz + (c < nv ? c : nv - 1));
+                }
+#pragma unroll
+                for (int i = 0; i < NV; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) xv[i].v[j] = xv[i].v[j] + more[i].v[j];
+            }
+        }
+        if (src.add) {
+            const V *pa = reinterpret_cast<const V *>(src.add + row * cols);
+            V av[NV];
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int c = lane_in_group + i * kGroup;
+                av[i] = nt_load(pa + (c < nv ? c : nv - 1));
+            }
+#pragma unroll
+            for (int i = 0; i < NV; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xv[i].v[j] = xv[i].v[j] + av[i].v[j];
+        }
+        if (src.sum_out) {
+            V *ps = reinterpret_cast<V *>(src.sum_out + row * cols);
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int c = lane_in_group + i * kGroup;
+                if (live && c < nv) ps[c] = xv[i];
+            }
+        }
         double acc = 0.0;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int c = lane_in_group + i * kGroup;
-            if (live && c < nv) {
-                xv[i] = pv[c];
-                for (int z = 1; z < src.slabs; ++z) {
-                    const V more = reinterpret_cast<const V *>(src.x + z * src.slab + row * cols)[c];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) xv[i].v[j] = xv[i].v[j] + more.v[j];
-                }
-                if (src.add) {
-                    const V av = reinterpret_cast<const V *>(src.add + row * cols)[c];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) xv[i].v[j] = xv[i].v[j] + av.v[j];
-                }
-                if (src.sum_out) reinterpret_cast<V *>(src.sum_out + row * cols)[c] = xv[i];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float sq = xv[i].v[j] * xv[i].v[j];
-                    acc += static_cast<double>(sq);
-                }
+            for (int j = 0; j < 4; ++j) {
+                const float sq = xv[i].v[j] * xv[i].v[j];
+                acc += c < nv ? static_cast<double>(sq) : 0.0;
             }
         }
         acc = wave_sum(acc);
@@ -451,7 +512,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(RmsSource src,
             for (int w = 0; w < kWavesPerBlock; ++w) acc += partial[w];
             __syncthreads();
         }
-        const float mean = static_cast<float>(acc / static_cast<double>(cols));
+        const float mean = static_cast<float>(mean_of(acc, cols));
         const float var = mean + eps;
         const float r = sqrtf(var);
         const float inv = 1.0f / r;
@@ -466,7 +527,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(RmsSource src,
                     const float normed = RECIP ? xv[i].v[j] * inv : xv[i].v[j] / r;
                     y.v[j] = normed * g[i].v[j];
                 }
-                po[c] = y;
+                nt_store(po + c, y);
             }
         }
     }

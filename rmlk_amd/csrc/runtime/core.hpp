@@ -219,7 +219,7 @@ void op_fused_softmax(OpContext &c);
 void op_fused_rotary(OpContext &c);
 void op_fused_head_rows(OpContext &c);
 // ScatterND's output: the data tensor itself where it may be updated in place, else a copy of it
-Tensor &scatter_destination(OpContext &c, int data_index, int out_index);
+Tensor &scatter_destination(OpContext &c, int data_index, int out_index, bool *copy_left_to_caller = nullptr);
 void op_fused_attn_matmul(OpContext &c);
 void op_fused_attention(OpContext &c);
 void op_fused_matmul_add_rmsnorm(OpContext &c);

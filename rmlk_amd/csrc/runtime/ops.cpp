@@ -526,16 +526,14 @@ void op_concat(OpContext &c) {
     out_shape[axis] = total;
     Tensor &y = c.alloc_output(0, first.dtype, out_shape);
     rmlk_dims od = to_dims(out_shape);
-    int64_t off = 0;
     bool hosted = all_hosted(c) && first.rank() == 1 && total <= kHostMirrorMax;
     auto h = std::make_shared<HostVal>();
+    std::vector<rmlk_dims> in_dims;
+    std::vector<const void *> in_ptrs;
     for (int i = 0; i < c.n_inputs(); ++i) {
         const Tensor &t = c.input(i);
-        rmlk_dims id = to_dims(t.shape);
-        check_status(rmlk_hip_concat(c.stream, t.dtype, &id, &od, static_cast<int32_t>(axis), off,
-                                     t.data(), y.data()),
-                     "Concat");
-        off += t.shape[axis];
+        in_dims.push_back(to_dims(t.shape));
+        in_ptrs.push_back(t.numel() ? t.data() : nullptr);
         if (hosted) {
             h->is_float = t.host->is_float;
             for (size_t k = 0; k < t.host->size(); ++k) {
@@ -544,6 +542,9 @@ void op_concat(OpContext &c) {
             }
         }
     }
+    check_status(rmlk_hip_concat_many(c.stream, first.dtype, c.n_inputs(), in_dims.data(), in_ptrs.data(),
+                                      &od, static_cast<int32_t>(axis), y.data()),
+                 "Concat");
     if (hosted) y.host = h;
 }
 
@@ -581,7 +582,8 @@ void op_gather(OpContext &c) {
 
 // Output `out_index` as the destination of a ScatterND over input `data_index`: the data tensor
 // itself when it may be updated in place (see op_scatter_nd), else a fresh copy of it.
-Tensor &scatter_destination(OpContext &c, int data_index, int out_index) {
+Tensor &scatter_destination(OpContext &c, int data_index, int out_index, bool *copy_left_to_caller) {
+    if (copy_left_to_caller) *copy_left_to_caller = false;
     const Tensor &data = c.input(data_index);
     const int vid = c.node.inputs[data_index];
     const Value &v = c.session.graph_copy.values[vid];
@@ -597,6 +599,10 @@ Tensor &scatter_destination(OpContext &c, int data_index, int out_index) {
     if (last_reader && sole_owner && may_overwrite && !read_elsewhere && !v.is_output && !v.is_initializer)
         return c.view_output(out_index, data, data.shape);
     Tensor &y = c.alloc_output(out_index, data.dtype, data.shape);
+    if (copy_left_to_caller) {
+        *copy_left_to_caller = true;     // the caller's kernel copies while it scatters
+        return y;
+    }
     check_status(rmlk_hip_memcpy_dtod(c.stream, y.data(), data.data(), data.nbytes()),
                  "ScatterND copy");
     return y;
@@ -635,8 +641,17 @@ void op_scatter_nd(OpContext &c) {
     int64_t n_tuples = 1;
     for (size_t d = 0; d + 1 < idx.shape.size(); ++d) n_tuples *= idx.shape[d];
 
-    Tensor *y = &scatter_destination(c, 0, 0);
+    bool fresh = false;
+    Tensor *y = &scatter_destination(c, 0, 0, rcode == RMLK_SCATTER_NONE ? &fresh : nullptr);
     rmlk_dims dd = to_dims(data.shape);
+    if (fresh) {
+        // a fresh output: the copy of data and the assignment of the slices in one pass
+        check_status(rmlk_hip_scatter_nd_copy(c.stream, data.dtype, &dd, n_tuples, static_cast<int32_t>(t),
+                                              static_cast<const int64_t *>(idx.data()), upd.data(),
+                                              c.input(0).data(), y->data(), c.error_flag()),
+                     "ScatterND");
+        return;
+    }
     check_status(rmlk_hip_scatter_nd(c.stream, rcode, data.dtype, &dd, n_tuples,
                                      static_cast<int32_t>(t),
                                      static_cast<const int64_t *>(idx.data()), upd.data(),

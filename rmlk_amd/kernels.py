@@ -154,6 +154,15 @@ def concat_into(x, out, in_shape, out_shape, axis: int, axis_offset: int) -> Non
                                 axis, axis_offset, _ptr(x), _ptr(out)), "rmlk_hip_concat")
 
 
+def concat(xs, out, in_shapes, out_shape, axis: int) -> None:
+    """All inputs of a Concat in one call. ref: runtime/src/providers/cuda/backend/concat.rs:28-76."""
+    assert len(xs) == len(in_shapes) and len(xs) >= 1
+    shapes = (Dims * len(xs))(*[Dims.of(s) for s in in_shapes])
+    ptrs = (ctypes.c_void_p * len(xs))(*[_ptr(x) if x.numel() else 0 for x in xs])
+    check(lib().rmlk_hip_concat_many(_stream(), dtype_of(out), len(xs), shapes, ptrs, Dims.of(out_shape),
+                                     axis, _ptr(out)), "rmlk_hip_concat_many")
+
+
 def gather(data, idx, out, data_shape, axis: int, err_flag=None) -> None:
     """ref: runtime/src/providers/cuda/backend/gather.rs:199-258."""
     check(lib().rmlk_hip_gather(_stream(), dtype_of(data), dtype_of(idx), Dims.of(data_shape),
@@ -168,6 +177,16 @@ def scatter_nd(idx, updates, out, data_shape, n_tuples: int, tuple_size: int,
     check(lib().rmlk_hip_scatter_nd(_stream(), reduction, dtype_of(out), Dims.of(data_shape),
                                     n_tuples, tuple_size, _ptr(idx), _ptr(updates), _ptr(out),
                                     _ptr(err_flag)), "rmlk_hip_scatter_nd")
+
+
+def scatter_nd_copy(idx, updates, data, out, data_shape, n_tuples: int, tuple_size: int,
+                    err_flag=None) -> None:
+    """ScatterND (reduction none) with its copy of `data` in one pass.
+    ref: runtime/src/providers/cuda/backend/scatter_nd.rs:128-129 + cuda/src/kernels/scatter_nd.rs:91-210."""
+    assert idx.dtype == torch.int64 and data.dtype == out.dtype
+    check(lib().rmlk_hip_scatter_nd_copy(_stream(), dtype_of(out), Dims.of(data_shape), n_tuples,
+                                         tuple_size, _ptr(idx), _ptr(updates), _ptr(data), _ptr(out),
+                                         _ptr(err_flag)), "rmlk_hip_scatter_nd_copy")
 
 
 def trilu(x, out, batch: int, rows: int, cols: int, upper: bool, k: int) -> None:

@@ -458,6 +458,23 @@ def test_concat(device, case, dtype):
     assert_exact(to_np(out), expected)
 
 
+@pytest.mark.parametrize("case", CONCAT_CASES + [
+    ([(1, 8, 8191, 64), (1, 8, 1, 64)], 2),                       # KV cache grown by one row
+    ([(2, 3, 4), (2, 3, 4), (2, 3, 4), (2, 3, 4), (2, 3, 4)], 1),
+    ([(5, 2)] * 9, 0),                                              # more inputs than one launch takes
+    ([(3, 1), (3, 2), (3, 5)], 1)])                                 # narrow units
+@pytest.mark.parametrize("dtype", [np.float32, np.int64, np.uint8])
+def test_concat_all_inputs_in_one_call(device, case, dtype):
+    k = _k()
+    shapes, axis = case
+    rng = np.random.default_rng(92)
+    xs = [(rng.standard_normal(s) * 100).astype(dtype) for s in shapes]
+    expected = _ops().concat(xs, axis)
+    out = torch.full(expected.shape, 7, dtype=to_dev(xs[0], device).dtype, device=device)
+    k.concat([to_dev(x, device) for x in xs], out, [list(x.shape) for x in xs], list(expected.shape), axis)
+    assert_exact(to_np(out), expected)
+
+
 GATHER_CASES = [((3, 4), 0, [0, 2]), ((3, 4), 0, [-3, -1]), ((3, 4), 1, [1, 3]), ((2, 3, 4), 1, [[1, 2], [0, -1]]),
                 ((500, 64), 0, list(range(0, 500, 7))), ((500, 2048), 0, [499, 0, 17, 17]),
                 ((4,), 0, [2]), ((6, 5), 1, [4, 0, 0]), ((3, 7, 3), 2, [2, 1])]
@@ -520,6 +537,47 @@ def test_scatter_nd_none(device, case, dtype):
                  int(np.prod(idx.shape[:-1])), idx.shape[-1], k.SCATTER_NONE, err)
     assert_exact(to_np(out), expected)
     assert int(err.item()) == 0
+
+
+@pytest.mark.parametrize("case", SCATTER_CASES + [
+    ((1, 8, 8192, 64), [[0, h, 8191 - 17 * h] for h in range(8)], None),   # the KV-cache stress shape
+    ((2, 2048, 16), [[1, 2047], [0, 0], [1, 2047], [0, 1023], [-1, -2048]], None),  # duplicates: the last wins
+    ((300, 4), [[i] for i in range(0, 300, 4)], None),              # more tuples than the one-pass kernel takes
+    ((64, 2), [[3], [9]], None),                                    # slices narrower than 16 bytes
+])
+@pytest.mark.parametrize("dtype", [np.float32, np.int64])
+def test_scatter_nd_with_its_copy_in_one_pass(device, case, dtype):
+    k = _k()
+    shape, idx, _ = case
+    rng = np.random.default_rng(103)
+    data = (rng.standard_normal(shape) * 10).astype(dtype)
+    idx = np.array(idx, dtype=np.int64)
+    upd_shape = idx.shape[:-1] + tuple(shape[idx.shape[-1]:])
+    upd = (rng.standard_normal(upd_shape) * 10).astype(dtype)
+    expected = _ops().scatter_nd(data, idx, upd)
+    src = to_dev(data, device)
+    out = torch.full(shape, 5, dtype=src.dtype, device=device)
+    err = torch.zeros(1, dtype=torch.int32, device=device)
+    k.scatter_nd_copy(to_dev(idx, device), to_dev(upd, device), src, out, list(shape),
+                      int(np.prod(idx.shape[:-1])), idx.shape[-1], err)
+    assert_exact(to_np(out), expected)
+    assert_exact(to_np(src), data)          # data is only read
+    assert int(err.item()) == 0
+
+
+def test_scatter_nd_copy_bad_index_flag(device):
+    k = _k()
+    data = np.arange(16 * 8, dtype=np.float32).reshape(16, 8)
+    idx = np.array([[1], [16], [-17], [2]], dtype=np.int64)
+    upd = -np.ones((4, 8), dtype=np.float32)
+    out = torch.zeros((16, 8), dtype=torch.float32, device=device)
+    err = torch.zeros(1, dtype=torch.int32, device=device)
+    k.scatter_nd_copy(to_dev(idx, device), to_dev(upd, device), to_dev(data, device), out, [16, 8], 4, 1, err)
+    expected = data.copy()
+    expected[1] = -1
+    expected[2] = -1
+    assert int(err.item()) == 1
+    assert_exact(to_np(out), expected)
 
 
 @pytest.mark.parametrize("red", ["add", "mul", "max", "min"])
