@@ -194,6 +194,58 @@ def test_llama_tiny_scatter_style_equals_concat_style(device):
     assert stats_e["device_syncs"] == 0 and stats_g["device_syncs"] == 0
 
 
+@pytest.mark.timeout(900)
+def test_llama_1b_full_size_prefill_and_teacher_forced_decode(device):
+    """BASELINE configs[3] at its full size: 16 layers, hidden 2048, vocab 128256. Prefill of a
+    512-token prompt, then 8 decode steps through the recorded HIP graph with the caches fed back on
+    the device, each step teacher-forced with the oracle's token and held to the reference's bar for
+    whole-model runs (logits atol = rtol = 1e-2, identical argmax: runtime/tests/e2e_ort/llama.rs:112-156,
+    cases.rs:75-85). The oracle multiplies in fp32 BLAS here (its float64 products would take minutes
+    at this size); no ONNX Runtime vectors exist for this graph (parity unpinned beyond the oracle)."""
+    graphs, runtime = _rt()
+    og = _oracle()
+    cfg = graphs.LlamaConfig()
+    prompt_len, steps = 512, 8
+    max_len = prompt_len + steps
+    graph = graphs.llama_graph(cfg, seed=4, style="scatter", max_len=max_len)
+    rng = np.random.default_rng(4)
+    prompt = rng.integers(0, cfg.vocab, size=prompt_len)
+    zeros = {f"cache.{l}.{kv}": np.zeros((1, cfg.kv_heads, max_len, cfg.head_dim), np.float32)
+             for l in range(cfg.layers) for kv in ("key", "value")}
+    inst = runtime.Builder.from_graph(graph).build()
+    feeds = _scatter_feeds(cfg, prompt, 0, zeros)
+    for name, arr in feeds.items():
+        inst.set_input(name, arr)
+    inst.execute()
+    got = inst.output("logits")[0, -1].copy()
+    exp = og.run_graph(graph, feeds, matmul_accumulate="f32")
+    pos = prompt_len
+    captured = False
+    for step in range(steps + 1):
+        ref = exp["logits"][0, -1]
+        np.testing.assert_allclose(got, ref, rtol=1e-2, atol=1e-2, err_msg=f"step {step}")
+        tok = int(np.argmax(ref))
+        assert int(np.argmax(got)) == tok, f"step {step}"
+        if step == steps:
+            break
+        caches = {f"cache.{l}.{kv}": exp[f"cache_out.{l}.{kv}"] for l in range(cfg.layers)
+                  for kv in ("key", "value")}
+        exp = og.run_graph(graph, _scatter_feeds(cfg, np.array([tok]), pos, caches), matmul_accumulate="f32")
+        inst.set_input("input_ids", np.array([[tok]], dtype=np.int64))
+        inst.set_input("position_ids", np.array([[pos]], dtype=np.int64))
+        if not captured:
+            for l in range(cfg.layers):
+                for kv in ("key", "value"):
+                    inst.feed_output(f"cache_out.{l}.{kv}", f"cache.{l}.{kv}")
+            inst.capture()
+            captured = True
+        inst.replay()
+        got = inst.output("logits")[0, -1].copy()
+        pos += 1
+    assert inst.memory_stats()["device_syncs"] == 0
+    inst.close()
+
+
 @pytest.mark.parametrize("heads,kv_heads,head_dim,hidden,ffn", [
     (6, 2, 64, 384, 640),      # head_dim 64: the attention kernels and the row-stream launch run
     (4, 2, 128, 512, 768),     # head_dim 128: the attention chain falls back to its three kernels

@@ -679,3 +679,88 @@ def test_memset_is_a_kernel_fill_and_replays_in_a_graph(device, offset, nbytes):
         graph.replay()
         torch.cuda.synchronize()
         assert_exact(to_np(buf), expected)
+
+
+# ---- the operator microbench configuration at its stated sizes -----------------------------------
+# (BASELINE configs[1]; seeded with 2 like the benchmark.) At these sizes the one-trip grids, the
+# 16 KiB chunks per block and the rows-in-registers kernels run with thousands of blocks; the small
+# cases above run them with a handful.
+
+FULL_SHAPE, FULL_B = (8, 32, 512, 64), (1, 32, 1, 64)
+
+
+@pytest.mark.parametrize("name", ["add", "mul", "div"])
+def test_full_size_broadcast_arithmetic_is_bit_exact(device, name):
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal(FULL_SHAPE).astype(np.float32)
+    b = rng.standard_normal(FULL_B).astype(np.float32)
+    assert_exact(run_binary(device, name, a, b), getattr(_ops(), name)(a, b))
+
+
+def test_full_size_where_is_bit_exact(device):
+    k = _k()
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal(FULL_SHAPE).astype(np.float32)
+    y = rng.standard_normal(FULL_B).astype(np.float32)
+    cond = rng.random(FULL_SHAPE) < 0.5
+    out = torch.empty(FULL_SHAPE, dtype=torch.float32, device=device)
+    shp = list(FULL_SHAPE)
+    k.where(to_dev(x, device), to_dev(y, device), to_dev(cond, device), out, shp,
+            bcast_strides(FULL_SHAPE, shp), bcast_strides(FULL_B, shp), bcast_strides(FULL_SHAPE, shp))
+    assert_exact(to_np(out), np.where(cond, x, y))
+
+
+def test_full_size_reduce_mean(device):
+    k = _k()
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((4096, 2048)).astype(np.float32)
+    out = torch.empty(4096, dtype=torch.float32, device=device)
+    k.reduce_mean(to_dev(x, device), out, [4096, 2048], [1])
+    expected = x.astype(np.float64).mean(axis=1).astype(np.float32)   # double accumulation, like the reference
+    assert_close(to_np(out), expected, rtol=1e-6, atol=1e-7)
+
+
+def test_full_size_transpose_is_bit_exact(device):
+    k = _k()
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((1, 2048, 32, 64)).astype(np.float32)
+    out = torch.empty((1, 32, 2048, 64), dtype=torch.float32, device=device)
+    k.transpose(to_dev(x, device), out, [1, 2048, 32, 64], [0, 2, 1, 3])
+    assert_exact(to_np(out), np.ascontiguousarray(x.transpose(0, 2, 1, 3)))
+
+
+@pytest.mark.parametrize("n_idx", [2048, 4096])
+def test_full_size_gather_is_bit_exact(device, n_idx):
+    k = _k()
+    g = torch.Generator(device=device).manual_seed(2)
+    table = torch.randn((128256, 2048), device=device, generator=g)       # 1 GB: made on the device
+    rng = np.random.default_rng(2)
+    idx = rng.integers(0, 128256, size=(1, n_idx)).astype(np.int64)
+    idx[0, :4] = [0, 128255, -1, -128256]                                   # the ends, and wrapped
+    out = torch.empty((n_idx, 2048), dtype=torch.float32, device=device)
+    err = torch.zeros(1, dtype=torch.int32, device=device)
+    k.gather(table, to_dev(idx.reshape(-1), device), out, [128256, 2048], 0, err)
+    expected = table[torch.from_numpy(idx.reshape(-1) % 128256).to(device)]
+    assert torch.equal(out, expected)
+    assert int(err.item()) == 0
+
+
+def test_full_size_masked_softmax(device):
+    """[1,32,2048,2048] with -inf above the diagonal: four heads against the float64 oracle, every
+    row of every head through what the mathematics fixes (masked entries exactly 0, rows sum to 1,
+    row 0 is exactly [1, 0, ...])."""
+    k = _k()
+    s, heads = 2048, 32
+    g = torch.Generator(device=device).manual_seed(2)
+    x = torch.randn((heads, s, s), device=device, generator=g)
+    x += torch.triu(torch.full((s, s), float("-inf"), device=device), 1)
+    out = torch.empty_like(x)
+    k.softmax(x, out, heads * s, s, 1)
+    for h in (0, 7, 19, 31):
+        xh = to_np(x[h])
+        assert_close(to_np(out[h]), _ops().softmax(xh, axis=-1))
+    upper = torch.triu(torch.ones((s, s), dtype=torch.bool, device=device), 1)
+    assert bool((out[:, upper] == 0).all())
+    sums = out.sum(dim=-1, dtype=torch.float64)
+    assert float((sums - 1.0).abs().max()) <= 2e-6
+    assert bool((out[:, 0, 0] == 1.0).all())
