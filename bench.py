@@ -14,6 +14,9 @@ GEMM) measured with HIP events, and the CPU oracle timed on the host cores on a 
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--prompt 512] [--decode 128]
     python bench.py --suite ops        # per-kernel launches of the op microbench shapes (for rocprofv3)
+    python bench.py --suite c1|c3|c5   # BASELINE configs[0], [2], [4] as graphs, fused and one kernel per node
+    python bench.py --summarize-ops JSON --kernel-trace CSV [--pmc-fetch CSV --pmc-write CSV]
+    python bench.py --summarize-graph JSON --kernel-trace CSV
 """
 import argparse
 import json
@@ -29,23 +32,40 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 CALIBRATION_COPY_BYTES = 256 << 20
 
-# HBM-side traffic of one GEMM launch per shape (batch, m, n, k[, epilogue]) of the default workload,
-# in KiB: (fetched, written). Read with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (one run
-# each) over `python3 bench.py --no-cpu --steps 1 --warmup 0 --decode 4`, scaled by what the same
-# counters read for the 256 MiB calibration copy below (FETCH_SIZE 131092 -> x2.0, WRITE_SIZE
-# 262144 -> x1.0). Split-K launches write partial sums to the workspace; what their consumer (the
-# combine kernel or the norm kernel) moves is not included.
+# HBM-side traffic of one GEMM launch per shape (batch, m, n, k[, epilogue]) of the default workload:
+# (kernel the library chose when the counters were read, KiB fetched, KiB written). RECORDED values,
+# not measured by the run that prints them: read with `rocprofv3 --pmc FETCH_SIZE` and `--pmc
+# WRITE_SIZE` (one run each) over `python3 bench.py --no-cpu --steps 1 --warmup 0 --decode 4`, scaled
+# by what the same counters read for the 256 MiB calibration copy below (FETCH_SIZE 131092 -> x2.0,
+# WRITE_SIZE 262144 -> x1.0); summary and command in PMC_TRAFFIC_SOURCE. An entry counts only while
+# the library still picks the kernel named with it. Split-K launches write partial sums to the
+# workspace; what their consumer (the combine kernel or the norm kernel) moves is not included.
+PMC_TRAFFIC_SOURCE = "profiles/gemm_mfma_llama1b_prefill512_hbm_traffic.md"
 PMC_TRAFFIC_KIB = {
-    (1, 512, 3072, 2048): (32997, 24576),                 # q/k/v (128 x 192 tiles), split-K 4
-    (1, 512, 2048, 2048): (24677, 16384),                 # o (128 x 64 tiles), split-K 4
-    (1, 512, 2048, 8192): (99094, 16384),                 # down (128 x 64 tiles), split-K 4
-    (1, 512, 16384, 2048, "swiglu"): (164044, 16384),     # gate/up with the SwiGLU epilogue
-    (1, 512, 128256, 2048): (1522548, 256512),            # lm-head
+    (1, 512, 3072, 2048): ("mfma128x192x32 direct splitk=4", 32997, 24576),               # q/k/v
+    (1, 512, 2048, 2048): ("mfma128x64x32 direct splitk=4", 24677, 16384),                # o
+    (1, 512, 2048, 8192): ("mfma128x64x32 direct splitk=4", 99094, 16384),                # down
+    (1, 512, 16384, 2048, "swiglu"): ("mfma128x128x32 direct splitk=1", 164044, 16384),   # gate/up, SwiGLU epilogue
+    (1, 512, 128256, 2048): ("mfma128x128x32 direct splitk=1", 1522548, 256512),          # lm-head
 }
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def cpu_threads():
+    """(threads the oracle's BLAS products run on, a description of the BLAS pool)."""
+    try:
+        from threadpoolctl import threadpool_info
+        pools = [p for p in threadpool_info() if p.get("user_api") == "blas"]
+        if pools:
+            n = max(int(p["num_threads"]) for p in pools)
+            return n, ", ".join(f"{p.get('internal_api', '?')} x{p['num_threads']}" for p in pools)
+    except Exception:           # threadpoolctl missing or numpy not loaded yet: fall back to the environment
+        pass
+    n = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return n, f"OMP_NUM_THREADS / cpu_count = {n}"
 
 
 def cpu_baseline(graph, cfg, graphs, prompt, n_tokens, max_len):
@@ -150,7 +170,9 @@ def run_llama(args):
             d["flops"] += flops
             d["alg_bytes"] += 4.0 * batch * (m * k + k * n + m * (n // 2 if swiglu else n))
             pmc = PMC_TRAFFIC_KIB.get(shape)
-            d["traffic"] = None if pmc is None or d["traffic"] is None else d["traffic"] + 1024.0 * sum(pmc)
+            if pmc is not None and pmc[0] != kind:
+                pmc = None                       # another kernel than the one the counters were read for
+            d["traffic"] = None if pmc is None or d["traffic"] is None else d["traffic"] + 1024.0 * sum(pmc[1:])
     for s in stats:
         if s["micros"] > 0:
             d = per_op.setdefault(s["op"], {"n": 0, "us": 0.0, "bytes": 0.0})
@@ -173,6 +195,8 @@ def run_llama(args):
         "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
         "traffic": None if dom["traffic"] is None else round(dom["traffic"] / dom["launches"]),
         "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated)",
+        "traffic_source": f"recorded table from {PMC_TRAFFIC_SOURCE} (an earlier counter run of this command), "
+                          "not measured by this run; null when the library picks another kernel than then",
         "algorithmic_bytes_per_launch": round(dom["alg_bytes"] / dom["launches"]),
         "launches": dom["launches"], "avg_launch_us": round(dom_us, 2),
         "avg_node_us_with_events": round(dom["us"] / dom["launches"], 2),
@@ -234,7 +258,7 @@ def run_llama(args):
     cpu = None
     if not args.no_cpu:
         n_cpu = min(args.cpu_tokens, prompt_len)
-        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        cores, blas = cpu_threads()
         cpu_tok_s, cpu_s, cpu_logits = cpu_baseline(graph, cfg, graphs, prompt, n_cpu, max_len)
         # the same sample through the GPU session (eager), as a check of the measured path
         inst.set_input("input_ids", prompt[:n_cpu].reshape(1, -1).astype(np.int64))
@@ -249,7 +273,8 @@ def run_llama(args):
         cpu = {"value": round(cpu_tok_s, 2), "unit": "tok/s", "cores": cores,
                "kind": "port",
                "sample": f"prefill of the first {n_cpu} prompt tokens through the same graph with the "
-                         f"numpy oracle (fp32 BLAS matmuls), {cpu_s:.1f} s; ONNX Runtime is not installed",
+                         f"numpy oracle (fp32 BLAS matmuls, {blas}), {cpu_s:.1f} s; "
+                         "ONNX Runtime is not installed",
                "gpu_vs_oracle_on_sample": {"max_abs_logit_diff": round(diff, 6), "top1_equal": same_top1,
                                            "bar": "1e-2 on logits, identical top-1"}}
         log(f"[bench] cpu oracle: {cpu_tok_s:.1f} tok/s over {n_cpu} tokens ({cpu_s:.1f}s); "
@@ -596,6 +621,134 @@ def summarize_ops(args):
         print(f"\n{label}: one counter unit = {unit:.3f} KiB (from the 256 MiB copy of the same run).")
 
 
+def run_graph_suite(args):
+    """BASELINE configs[0], [2] and [4] as graphs through the session, with pattern fusion and with
+    one kernel per node: replays of the recorded HIP graph timed on the device, and one eager pass
+    with HIP events per node for the per-operator figures. A torch `bitwise_not` launch marks the
+    start of every timed block in a kernel trace (`bench.py --summarize-graph`)."""
+    import numpy as np
+    import torch
+    from rmlk_amd import graphs, runtime
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    marker = torch.zeros(4, dtype=torch.int32, device="cuda:0")
+    if args.suite == "c1":
+        graph, feeds = graphs.rmsnorm_matmul_graph(seed=1)
+        workload = "BASELINE configs[0]: decomposed RMSNorm [1,128,2048] + MatMul [2048,8192], fp32"
+    elif args.suite == "c3":
+        graph, feeds = graphs.decoder_layer_graph(seed=3, seq=2048)
+        workload = "BASELINE configs[2]: one Llama-3.2-1B-shaped decoder layer, prefill S=2048, fp32"
+    else:
+        graph, feeds = graphs.kv_stress_graph(seed=5)
+        workload = "BASELINE configs[4]: indexing / KV-cache stress graph at length 8192"
+    mm_ops = ("MatMul", "rmlk.MatMulGroup", "rmlk.MatMulGroupSwiGLU", "rmlk.MatMulAddRMSNorm",
+              "rmlk.MatMulConst", "rmlk.AttnMatMul")
+    blocks, out = [], {"suite": args.suite, "workload": workload, "modes": {}}
+    reference = None
+    for mode, fuse in (("fused", True), ("one_kernel_per_node", False)):
+        inst = runtime.Builder.from_graph(graph).build(0, fuse=fuse)
+        got = inst.run(feeds)                      # first run fills the pool; outputs kept for the check
+        if reference is None:
+            reference = got
+        else:
+            for name in reference:
+                a, b = reference[name], got[name]
+                if a.dtype.kind == "f":
+                    np.testing.assert_allclose(a, b, rtol=2e-3, atol=2e-4, err_msg=name)
+                else:
+                    assert np.array_equal(a, b), name
+        for name, arr in feeds.items():
+            inst.set_input(name, arr)
+        inst.capture()
+        for _ in range(max(args.warmup, 3)):
+            inst.replay()
+        inst.sync()
+        marker.bitwise_not_()              # the mark in a kernel trace (the session never launches this)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            inst.replay()
+        inst.sync()
+        ms = (time.perf_counter() - t0) / args.steps * 1e3
+        marker.bitwise_not_()              # end of the timed block; what follows up to the next mark is not timed
+        torch.cuda.synchronize()
+        blocks.append({"label": mode, "replays": args.steps})
+        blocks.append(None)
+        # per-node events on one eager pass (they add a cache write-back after every node)
+        for name, arr in feeds.items():
+            inst.set_input(name, arr)
+        inst.set_profiling(True)
+        inst.execute()
+        inst.set_profiling(False)
+        per_op, mm_us, mm_flops = {}, 0.0, 0.0
+        for st in inst.node_stats():
+            if st["micros"] <= 0:
+                continue
+            d = per_op.setdefault(st["op"], {"n": 0, "us": 0.0, "bytes": 0.0})
+            d["n"] += 1
+            d["us"] += st["micros"]
+            d["bytes"] += st["bytes"]
+            if st["op"] in mm_ops:
+                mm_us += st["micros"]
+                mm_flops += st["flops"]
+        out["modes"][mode] = {
+            "ms_per_pass_device_replay": round(ms, 4), "nodes": len(graph.nodes),
+            "fused_nodes": inst.fused_nodes,
+            "matmul_us_with_events": round(mm_us, 1),
+            "matmul_tflops_with_events": round(mm_flops / mm_us / 1e6, 2) if mm_us else None,
+            "ops_with_events": {op: {"n": d["n"], "us": round(d["us"], 1),
+                                     "gbs": round(d["bytes"] / d["us"] / 1e3, 1)}
+                                for op, d in sorted(per_op.items(), key=lambda kv: -kv[1]["us"])}}
+        log(f"[{args.suite}] {mode}: {ms:.3f} ms per pass (device replay), MatMul nodes {mm_us:.1f} us with events")
+        inst.close()
+    out["trace_blocks"] = blocks[:-1]
+    print(json.dumps(out))
+
+
+GRAPH_MARKER_KERNEL = "bitwise_not"
+
+
+def summarize_graph(args):
+    """Kernels of every timed block of a graph suite (split at the marker launches), grouped by
+    kernel and grid: launches per replay, average and summed duration per replay."""
+    import csv
+    import statistics
+    res = json.loads([l for l in open(args.summarize_graph) if l.startswith("{")][-1])
+    rows = list(csv.DictReader(open(args.kernel_trace)))
+    rows.sort(key=lambda r: int(r["Start_Timestamp"]))
+    segments, cur = [], None
+    for r in rows:
+        if GRAPH_MARKER_KERNEL in r["Kernel_Name"]:
+            if cur is not None:
+                segments.append(cur)
+            cur = []
+        elif cur is not None and "rmlk::" in r["Kernel_Name"]:
+            cur.append(r)
+    blocks = res["trace_blocks"]
+    assert len(segments) == len(blocks), (len(segments), len(blocks))
+    print(f"Workload: {res['workload']}\n")
+    for blk, seg in zip(blocks, segments):
+        if blk is None:
+            continue
+        reps = blk["replays"]
+        n_launch = len(seg)
+        per_replay = n_launch // reps if n_launch % reps == 0 else None
+        timed = seg[:per_replay * reps] if per_replay else seg
+        groups = {}
+        for x in timed:
+            key = (_short_kernel_name(x["Kernel_Name"]),
+                   f"{int(x['Grid_Size_X']) // int(x['Workgroup_Size_X'])}x{int(x['Grid_Size_Y'])}x{int(x['Grid_Size_Z'])}")
+            groups.setdefault(key, []).append((int(x["End_Timestamp"]) - int(x["Start_Timestamp"])) / 1e3)
+        total = sum(sum(v) for v in groups.values()) / reps
+        mode = res["modes"][blk["label"]]
+        print(f"### {blk['label']}: {n_launch // reps} launches per pass, {total:.1f} us of kernel time per pass, "
+              f"{mode['ms_per_pass_device_replay'] * 1e3:.1f} us per replay on the host clock\n")
+        print("| kernel | blocks | launches per pass | avg us | min us | us per pass |")
+        print("|---|---|---|---|---|---|")
+        for (name, grid), v in sorted(groups.items(), key=lambda kv: -sum(kv[1])):
+            print(f"| {name} | {grid} | {len(v) / reps:g} | {statistics.mean(v):.2f} | {min(v):.2f} | {sum(v) / reps:.1f} |")
+        print()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -606,12 +759,14 @@ def main():
     ap.add_argument("--cpu-tokens", type=int, default=512)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--tiny", action="store_true", help="2-layer toy shape (plumbing check only)")
-    ap.add_argument("--suite", default="llama", choices=["llama", "ops"])
+    ap.add_argument("--suite", default="llama", choices=["llama", "ops", "c1", "c3", "c5"])
     ap.add_argument("--ops-launches", type=int, default=100, help="ops suite: launches per recorded graph")
     ap.add_argument("--ops-quick", action="store_true",
                     help="ops suite: one replay per op, no settling (for counter runs, which serialise launches)")
     ap.add_argument("--summarize-ops", metavar="JSON", help="print the per-op table from an ops-suite JSON "
                     "line and the rocprofv3 CSVs of the same command (no GPU needed)")
+    ap.add_argument("--summarize-graph", metavar="JSON", help="print the per-kernel table of a c1/c3/c5 "
+                    "suite from its JSON line and the rocprofv3 kernel trace of the same command")
     ap.add_argument("--kernel-trace", metavar="CSV")
     ap.add_argument("--pmc-fetch", metavar="CSV")
     ap.add_argument("--pmc-write", metavar="CSV")
@@ -619,12 +774,18 @@ def main():
     if args.summarize_ops:
         summarize_ops(args)
         return
+    if args.summarize_graph:
+        summarize_graph(args)
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one MI355X: the operator path has no multi-GPU part "
               "(run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
     if args.suite == "ops":
         run_ops_suite(args)
+        return
+    if args.suite in ("c1", "c3", "c5"):
+        run_graph_suite(args)
         return
     print(json.dumps(run_llama(args)))
 
