@@ -978,18 +978,23 @@ __global__ __launch_bounds__(kThreads) void gemv_dot_kernel(GemvArgs g) {
     }
 }
 
-// One-row product with K-contiguous weights, y[n] = sum_k x[k] * Wt[n][k]: a wavefront owns COLS
-// output columns and walks K in 128-bit units, eight units per lane and column in flight; the lanes'
-// partial sums meet in a shuffle tree. A column is finished inside its wavefront, so there is no
-// split-K, no workspace and no combine launch whatever the width.
-// SWIGLU: COLS is 2 and the wavefront's two rows of Wt are the gate and the up row of ONE output
-// (rows gate_row + i and up_row + i); it writes silu(gate) * up.
+// One-row product with K-contiguous weights, y[n] = sum_k x[k] * Wt[n][k]: a wavefront owns ONE output
+// and walks its row(s) of Wt in chunks of eight 128-bit units per lane (8 KiB per wavefront and row
+// in flight, streaming loads), x following the weights; the lanes' partial sums meet in a DPP
+// reduction. A column is finished inside its wavefront, so there is no split-K, no workspace and
+// no combine launch whatever the width. (Measured against two and four outputs per wavefront and
+// against wavefronts that walk several rows with the next row's loads in flight: the short-lived
+// wavefront with eight loads per lane wins at every width, 20.0 against 23.9 us on 16384 x 2048
+// and 142 against 158 us on 128256 x 2048, 7.4 TB/s.)
+// SWIGLU: the wavefront's two rows of Wt are the gate and the up row of its output (rows
+// gate_row + i and up_row + i, sharing the loads of x); it writes silu(gate) * up.
 // NORM: x is the row BEFORE an RMSNorm and the product is taken with RMSNorm(x) * gamma, which is
 // never stored in memory: every block first normalises the row into LDS exactly as the norm
 // kernel's block-per-row form does (squares rounded to float, summed in double per lane, wavefront
 // and block in that kernel's order), so the result equals the norm kernel followed by the product
-// bit for bit. (Every WAVEFRONT normalising the row for itself was tried first: the arithmetic,
-// repeated for each output column, cost more than the launch it saves.)
+// bit for bit. The block's loads of x and gamma are issued BEFORE the first weight loads (loads of a
+// wavefront return in order: behind the weights, the row - which the caches hold - would arrive
+// only after a full trip to HBM) and the arithmetic runs while the weights are in flight.
 // `residual` (may be null) is added to the outputs (the Add behind an output projection).
 struct RowNormArgs {
     const float *gamma;
@@ -997,113 +1002,154 @@ struct RowNormArgs {
     int32_t reciprocal;
 };
 
-template <int COLS, bool SWIGLU = false, bool NORM = false>
+constexpr int kGemvDepth = 8;                    // 128-bit units per lane, row and chunk
+constexpr int kGemvNormUnits = 8;                // NORM: units of x a lane holds (k <= 256 * 8 * 4)
+
+template <bool SWIGLU = false, bool NORM = false>
 __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__restrict__ x,
                                                           const float *__restrict__ wt,
                                                           float *__restrict__ y, int32_t n, int32_t k,
                                                           int64_t ldw, int32_t gate_row, int32_t up_row,
                                                           const float *__restrict__ residual,
                                                           RowNormArgs norm) {
-    static_assert(!SWIGLU || COLS == 2, "gate and up");
-    constexpr int kDepth = 8;
+    constexpr int COLS = SWIGLU ? 2 : 1;
     constexpr int kWaves = kThreads / kWave;
     // the normalised row of the block (NORM): k floats of dynamic LDS
     extern __shared__ __align__(16) float xs[];
     __shared__ double partial[kWaves];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    const int col0 = (blockIdx.x * kWaves + wave) * (SWIGLU ? 1 : COLS);
+    const int col = blockIdx.x * kWaves + wave;
     const int k4 = k / 4;
     const v4f *xv = reinterpret_cast<const v4f *>(x);
     // (a wavefront past the last column keeps valid addresses and takes part in the barriers)
-    const int col_c = min(col0, n - 1);
+    const int col_c = min(col, n - 1);
     const v4f *wv[COLS];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
-        const int64_t row = SWIGLU ? (c == 0 ? gate_row : up_row) + col_c : min(col_c + c, n - 1);
+        const int64_t row = SWIGLU ? (c == 0 ? gate_row : up_row) + col_c : col_c;
         wv[c] = reinterpret_cast<const v4f *>(wt + row * ldw);
     }
-    // NORM: the first batch of weight loads is in flight while the block normalises the row
-    [[maybe_unused]] v4f w_first[kDepth][COLS];
+    // NORM: this lane's share of the row and of gamma, requested before any weight
+    [[maybe_unused]] v4f xn[kGemvNormUnits], gn[kGemvNormUnits];
     if constexpr (NORM) {
+        const v4f *gv = reinterpret_cast<const v4f *>(norm.gamma);
 #pragma unroll
-        for (int j = 0; j < kDepth; ++j) {
-            const int u = lane + j * kWave;
-#pragma unroll
-            for (int c = 0; c < COLS; ++c)
-                w_first[j][c] = u < k4 ? __builtin_nontemporal_load(wv[c] + u) : v4f{0.f, 0.f, 0.f, 0.f};
-        }
-    }
-    if constexpr (NORM) {
-        // (two passes over the row, which the caches hold: keeping it in registers between them
-        // cost the wavefronts that stream the weights their occupancy)
-        double acc = 0.0;
-        for (int c = threadIdx.x; c < k4; c += kThreads) {
-            const v4f v = xv[c];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float sq = v[j] * v[j];
-                acc += static_cast<double>(sq);
+        for (int i = 0; i < kGemvNormUnits; ++i) {
+            const int c = threadIdx.x + i * kThreads;
+            if (i * kThreads < k4) {             // (uniform)
+                xn[i] = xv[min(c, k4 - 1)];
+                gn[i] = gv[min(c, k4 - 1)];
             }
         }
+    }
+    // Chunks of kGemvDepth * 64 units. Whole chunks are addressed as pointer + constant (the loads
+    // carry their offsets as immediates: with two wavefronts per SIMD, as on the 2048-wide outputs,
+    // address arithmetic per load is time nothing else covers - it cost the k = 8192 product 2 us);
+    // the last, partial chunk of a k that is no multiple of 2048 clamps its units and zeroes them.
+    constexpr int kChunkUnits = kWave * kGemvDepth;
+    const int full_chunks = k4 / kChunkUnits;
+    v4f wr[kGemvDepth][COLS];
+    auto load_w = [&](int chunk, bool partial_chunk) {
+        if (!partial_chunk) {
 #pragma unroll
-        for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, kWave);
+            for (int c = 0; c < COLS; ++c) {
+                const v4f *p = wv[c] + chunk * kChunkUnits + lane;
+#pragma unroll
+                for (int j = 0; j < kGemvDepth; ++j) wr[j][c] = __builtin_nontemporal_load(p + j * kWave);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < kGemvDepth; ++j) {
+                const int u = min(chunk * kChunkUnits + lane + j * kWave, k4 - 1);
+#pragma unroll
+                for (int c = 0; c < COLS; ++c) wr[j][c] = __builtin_nontemporal_load(wv[c] + u);
+            }
+        }
+    };
+    load_w(0, full_chunks == 0);      // in flight during the NORM prologue
+    if constexpr (NORM) {
+        double acc = 0.0;
+#pragma unroll
+        for (int i = 0; i < kGemvNormUnits; ++i) {
+            if (i * kThreads < k4) {
+                const bool live = threadIdx.x + i * kThreads < k4;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float sq = xn[i][j] * xn[i][j];
+                    acc += live ? static_cast<double>(sq) : 0.0;
+                }
+            }
+        }
+        acc = wave_sum(acc);
         if (lane == 0) partial[wave] = acc;
         __syncthreads();
         acc = 0.0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) acc += partial[w];
-        const float mean = static_cast<float>(acc / static_cast<double>(k));
+        const double kd = static_cast<double>(k);
+        const float mean = static_cast<float>((k & (k - 1)) == 0 ? acc * (1.0 / kd) : acc / kd);
         const float var = mean + norm.eps;
         const float r = sqrtf(var);
         const float inv = 1.0f / r;
-        const v4f *gv = reinterpret_cast<const v4f *>(norm.gamma);
-        for (int c = threadIdx.x; c < k4; c += kThreads) {
-            v4f v = xv[c];
-            const v4f g = gv[c];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float normed = norm.reciprocal ? v[j] * inv : v[j] / r;
-                v[j] = normed * g[j];
+        for (int i = 0; i < kGemvNormUnits; ++i) {
+            const int c = threadIdx.x + i * kThreads;
+            if (c < k4) {
+                v4f v = xn[i];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float normed = norm.reciprocal ? v[j] * inv : v[j] / r;
+                    v[j] = normed * gn[i][j];
+                }
+                reinterpret_cast<v4f *>(xs)[c] = v;
             }
-            reinterpret_cast<v4f *>(xs)[c] = v;
         }
         __syncthreads();
     }
-    if (col0 >= n) return;
-    auto load_x = [&](int u) { return NORM ? reinterpret_cast<const v4f *>(xs)[u] : xv[u]; };
+    if (col >= n) return;
+    const v4f *xsrc = NORM ? reinterpret_cast<const v4f *>(xs) : xv;
     float acc[COLS];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) acc[c] = 0.f;
-    for (int u0 = lane; u0 < k4; u0 += kWave * kDepth) {
-        v4f xr[kDepth], wr[kDepth][COLS];
+    for (int chunk = 0; chunk < full_chunks; ++chunk) {
+        if (chunk > 0) load_w(chunk, false);
+        const v4f *px = xsrc + chunk * kChunkUnits + lane;
+        v4f xr[kGemvDepth];
 #pragma unroll
-        for (int j = 0; j < kDepth; ++j) {
-            const int u = u0 + j * kWave;
-            const bool live = u < k4;
-            xr[j] = live ? load_x(u) : v4f{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < kGemvDepth; ++j) xr[j] = px[j * kWave];
 #pragma unroll
-            for (int c = 0; c < COLS; ++c) {
-                if (NORM && u0 == lane) wr[j][c] = w_first[j][c];
-                else wr[j][c] = live ? __builtin_nontemporal_load(wv[c] + u) : v4f{0.f, 0.f, 0.f, 0.f};
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < kDepth; ++j)
+        for (int j = 0; j < kGemvDepth; ++j)
 #pragma unroll
             for (int c = 0; c < COLS; ++c)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) acc[c] = fmaf(xr[j][e], wr[j][c][e], acc[c]);
     }
+    if (full_chunks * kChunkUnits < k4) {
+        if (full_chunks > 0) load_w(full_chunks, true);
 #pragma unroll
-    for (int c = 0; c < COLS; ++c) {
+        for (int j = 0; j < kGemvDepth; ++j) {
+            const int u = full_chunks * kChunkUnits + lane + j * kWave;
+            v4f xr = xsrc[min(u, k4 - 1)];
+            if (u >= k4) {
+                xr = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int o = kWave / 2; o > 0; o >>= 1) acc[c] += __shfl_xor(acc[c], o, kWave);
-        if (!SWIGLU && lane == 0 && col0 + c < n)
-            y[col0 + c] = residual ? acc[c] + residual[col0 + c] : acc[c];
+                for (int c = 0; c < COLS; ++c) wr[j][c] = v4f{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int c = 0; c < COLS; ++c)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[c] = fmaf(xr[e], wr[j][c][e], acc[c]);
+        }
     }
-    if (SWIGLU && lane == 0) {
-        const float silu = acc[0] * (1.0f / (1.0f + expf(-acc[0])));
-        y[col0] = silu * acc[COLS - 1];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) acc[c] = wave_sum(acc[c]);
+    if (lane == 0) {
+        if constexpr (SWIGLU) {
+            const float silu = acc[0] * (1.0f / (1.0f + expf(-acc[0])));
+            y[col] = silu * acc[COLS - 1];
+        } else {
+            y[col] = residual ? acc[0] + residual[col] : acc[0];
+        }
     }
 }
 
@@ -1816,16 +1862,9 @@ int32_t gemv_kmajor_launch(rmlk_stream_t stream, int32_t dtype, int64_t n, int64
     hipStream_t s = as_stream(stream);
     constexpr int kWaves = kThreads / kWave;
     const int32_t ni = static_cast<int32_t>(n), ki = static_cast<int32_t>(k);
-    // few columns: one per wavefront keeps every compute unit busy; many: four share the loads of x
-    if (n >= 16 * kNumCU * kWaves) {
-        const unsigned grid = static_cast<unsigned>((n + kWaves * 4 - 1) / (kWaves * 4));
-        if (norm) gemv_kmajor_kernel<4, false, true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
-        else gemv_kmajor_kernel<4><<<grid, kThreads, 0, s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, RowNormArgs{});
-    } else {
-        const unsigned grid = static_cast<unsigned>((n + kWaves - 1) / kWaves);
-        if (norm) gemv_kmajor_kernel<1, false, true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
-        else gemv_kmajor_kernel<1><<<grid, kThreads, 0, s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, RowNormArgs{});
-    }
+    const unsigned grid = static_cast<unsigned>((n + kWaves - 1) / kWaves);
+    if (norm) gemv_kmajor_kernel<false, true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
+    else gemv_kmajor_kernel<><<<grid, kThreads, 0, s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, RowNormArgs{});
     return launch_status();
 }
 
@@ -1851,11 +1890,11 @@ int32_t gemv_kmajor_swiglu_launch(rmlk_stream_t stream, int32_t dtype, int64_t n
     const int32_t ni = static_cast<int32_t>(n), ki = static_cast<int32_t>(k);
     const int32_t gr = static_cast<int32_t>(gate_row), ur = static_cast<int32_t>(up_row);
     if (norm)
-        gemv_kmajor_kernel<2, true, true><<<grid, kThreads, k * sizeof(float), as_stream(stream)>>>(
+        gemv_kmajor_kernel<true, true><<<grid, kThreads, k * sizeof(float), as_stream(stream)>>>(
             px, pw, py, ni, ki, ldw, gr, ur, nullptr, *norm);
     else
-        gemv_kmajor_kernel<2, true><<<grid, kThreads, 0, as_stream(stream)>>>(px, pw, py, ni, ki, ldw, gr, ur,
-                                                                             nullptr, RowNormArgs{});
+        gemv_kmajor_kernel<true><<<grid, kThreads, 0, as_stream(stream)>>>(px, pw, py, ni, ki, ldw, gr, ur,
+                                                                          nullptr, RowNormArgs{});
     return launch_status();
 }
 

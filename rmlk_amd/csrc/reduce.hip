@@ -17,63 +17,6 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 
-// Wavefront reductions through DPP (data-parallel primitives: an operand read from another lane of
-// the same row of 16 inside the instruction itself) instead of ds_bpermute shuffles, each of which
-// is a round trip through the LDS crossbar: quad swaps, then the two mirrors give every lane of a
-// row the row's result; the four row results meet through readlane. The order of the additions is
-// fixed (and the same for every kernel of this file).
-template <int CTRL, typename T>
-__device__ __forceinline__ T dpp_take(T v) {
-    static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- or 64-bit values");
-    if constexpr (sizeof(T) == 4) {
-        const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false);
-        return __builtin_bit_cast(T, r);
-    } else {
-        const uint64_t u = __builtin_bit_cast(uint64_t, v);
-        const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(u), CTRL, 0xf, 0xf, false));
-        const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(u >> 32), CTRL, 0xf, 0xf, false));
-        return __builtin_bit_cast(T, (static_cast<uint64_t>(hi) << 32) | lo);
-    }
-}
-template <typename T>
-__device__ __forceinline__ T lane_value(T v, int lane) {
-    if constexpr (sizeof(T) == 4) {
-        return __builtin_bit_cast(T, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
-    } else {
-        const uint64_t u = __builtin_bit_cast(uint64_t, v);
-        const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(u), lane));
-        const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(u >> 32), lane));
-        return __builtin_bit_cast(T, (static_cast<uint64_t>(hi) << 32) | lo);
-    }
-}
-constexpr int kDppQuadSwap1 = 0xB1;      // quad_perm [1,0,3,2]
-constexpr int kDppQuadSwap2 = 0x4E;      // quad_perm [2,3,0,1]
-constexpr int kDppRowHalfMirror = 0x141;
-constexpr int kDppRowMirror = 0x140;
-
-template <typename T>
-__device__ __forceinline__ T wave_sum(T v) {
-    v += dpp_take<kDppQuadSwap1>(v);
-    v += dpp_take<kDppQuadSwap2>(v);
-    v += dpp_take<kDppRowHalfMirror>(v);
-    v += dpp_take<kDppRowMirror>(v);
-    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
-}
-template <typename T>
-__device__ __forceinline__ T wave_max(T v) {
-    T w = dpp_take<kDppQuadSwap1>(v);
-    v = w > v ? w : v;
-    w = dpp_take<kDppQuadSwap2>(v);
-    v = w > v ? w : v;
-    w = dpp_take<kDppRowHalfMirror>(v);
-    v = w > v ? w : v;
-    w = dpp_take<kDppRowMirror>(v);
-    v = w > v ? w : v;
-    const T a = lane_value(v, 0), b = lane_value(v, 16), c = lane_value(v, 32), d = lane_value(v, 48);
-    const T ab = b > a ? b : a, cd = d > c ? d : c;
-    return cd > ab ? cd : ab;
-}
-
 // sum / n in double. For n a power of two the quotient is the product with 1 / n, exactly (a change
 // of exponent), and the multiply is one instruction where the IEEE division is a chain of thirty
 // between a wavefront's last load and its first store.
