@@ -367,14 +367,10 @@ __global__ __launch_bounds__(kAttnThreads) void attention_few_rows_kernel(AttnAr
             const float m = g.mask[b * g.mask_b + head * g.mask_h + srow * g.mask_s + key];
             sc = (scale_is_mul ? dot * scale : dot / scale) + m;
         }
-        float mx = sc;
-#pragma unroll
-        for (int o = kWave / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+        const float mx = wave_max(sc);
         const float m_safe = mx == -INFINITY ? 0.f : mx;
         const float p = expf(sc - m_safe);
-        float sum = p;
-#pragma unroll
-        for (int o = kWave / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+        const float sum = wave_sum(p);
         ps[r][lane] = p;   // read back by this wavefront only
         __builtin_amdgcn_wave_barrier();
         float acc = 0.f;   // lane = head dim
@@ -390,7 +386,13 @@ __global__ __launch_bounds__(kAttnThreads) void attention_few_rows_kernel(AttnAr
 }
 
 // out row = sum over chunks of the partial outputs, rescaled to the common maximum, over the
-// rescaled sums; a wavefront per (kv head, row), lane = head dim.
+// rescaled sums; a wavefront per (kv head, row), lane = head dim. The kernel is one trip to memory
+// long, so it asks for everything at once: lane c the maximum and the sum of chunk c, then every
+// lane its element of the first sixteen partial outputs, and only then reduces the maxima (loads
+// return in order: the reduction runs while the outputs are on their way). Up to 64 chunks.
+constexpr int kMergeGroup = 16;
+constexpr int kMergeMaxChunks = kWave;
+
 __global__ __launch_bounds__(kAttnThreads) void attention_merge_kernel(AttnArgs g, const float *__restrict__ ws,
                                                                        int32_t n_chunks, int32_t total_rows) {
     const int lane = threadIdx.x % kWave;
@@ -401,12 +403,49 @@ __global__ __launch_bounds__(kAttnThreads) void attention_merge_kernel(AttnArgs 
     const int b = bg / g.kv_heads, grp = bg - b * g.kv_heads;
     const float *src = ws + (static_cast<int64_t>(bg) * n_chunks * rows + r) * kPartial;
     const int64_t step = static_cast<int64_t>(rows) * kPartial;
-    // maxima and sums: a chunk per lane (all loads in flight at once), then the outputs chunk by chunk
+    const int mine = min(lane, n_chunks - 1);
+    const float m_c = src[mine * step + kHeadDim];
+    const float s_c = src[mine * step + kHeadDim + 1];
+    float part[kMergeGroup];
+#pragma unroll
+    for (int j = 0; j < kMergeGroup; ++j) part[j] = src[min(j, n_chunks - 1) * step + lane];
+    const float m = wave_max(lane < n_chunks ? m_c : -INFINITY);
+    const float m_safe = m == -INFINITY ? 0.f : m;
+    const float w = lane < n_chunks ? expf(m_c - m_safe) : 0.f;
+    const float sum = wave_sum(lane < n_chunks ? s_c * w : 0.f);
+    float acc = 0.f;
+    for (int c0 = 0; c0 < n_chunks; c0 += kMergeGroup) {
+        if (c0 > 0) {
+#pragma unroll
+            for (int j = 0; j < kMergeGroup; ++j) part[j] = src[min(c0 + j, n_chunks - 1) * step + lane];
+        }
+#pragma unroll
+        for (int j = 0; j < kMergeGroup; ++j) {
+            // (chunks past the end read the last one again with weight 0: lanes >= n_chunks hold w = 0)
+            const float wj = __shfl(w, c0 + j, kWave);
+            acc = fmaf(part[j], c0 + j < n_chunks ? wj : 0.f, acc);
+        }
+    }
+    const int head = grp * g.rep + r / g.seq, srow = r - (r / g.seq) * g.seq;
+    g.out[b * g.out_b + head * g.out_h + srow * g.out_s + lane] = acc / sum;   // nothing visible: 0 / 0
+}
+
+// The same for more chunks than a wavefront has lanes: maxima and sums a chunk per lane in rounds,
+// then the outputs chunk by chunk.
+__global__ __launch_bounds__(kAttnThreads) void attention_merge_many_kernel(AttnArgs g, const float *__restrict__ ws,
+                                                                            int32_t n_chunks, int32_t total_rows) {
+    const int lane = threadIdx.x % kWave;
+    const int item = blockIdx.x * (kAttnThreads / kWave) + threadIdx.x / kWave;
+    if (item >= total_rows) return;
+    const int rows = g.rows;
+    const int bg = item / rows, r = item - bg * rows;
+    const int b = bg / g.kv_heads, grp = bg - b * g.kv_heads;
+    const float *src = ws + (static_cast<int64_t>(bg) * n_chunks * rows + r) * kPartial;
+    const int64_t step = static_cast<int64_t>(rows) * kPartial;
     float m = -INFINITY;
     for (int c0 = 0; c0 < n_chunks; c0 += kWave)
         if (c0 + lane < n_chunks) m = fmaxf(m, src[(c0 + lane) * step + kHeadDim]);
-#pragma unroll
-    for (int o = kWave / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, kWave));
+    m = wave_max(m);
     const float m_safe = m == -INFINITY ? 0.f : m;
     float acc = 0.f, sum = 0.f;
     for (int c0 = 0; c0 < n_chunks; c0 += kWave) {
@@ -417,8 +456,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_merge_kernel(AttnArgs 
 #pragma unroll 8
         for (int j = 0; j < here; ++j) acc = fmaf(src[(c0 + j) * step + lane], __shfl(w, j, kWave), acc);
     }
-#pragma unroll
-    for (int o = kWave / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+    sum = wave_sum(sum);
     const int head = grp * g.rep + r / g.seq, srow = r - (r / g.seq) * g.seq;
     g.out[b * g.out_b + head * g.out_h + srow * g.out_s + lane] = acc / sum;   // nothing visible: 0 / 0
 }
@@ -556,7 +594,12 @@ extern "C" int32_t rmlk_hip_attention_few_rows(rmlk_stream_t stream, int32_t dty
     if (launched) return launched;
     const int64_t total_rows = batch * kv_heads * g.rows;
     constexpr int kWaves = kAttnThreads / kWave;
-    attention_merge_kernel<<<static_cast<unsigned>((total_rows + kWaves - 1) / kWaves), kAttnThreads, 0, s>>>(
-        g, ws, static_cast<int32_t>(chunks), static_cast<int32_t>(total_rows));
+    const unsigned merge_grid = static_cast<unsigned>((total_rows + kWaves - 1) / kWaves);
+    if (chunks <= kMergeMaxChunks)
+        attention_merge_kernel<<<merge_grid, kAttnThreads, 0, s>>>(g, ws, static_cast<int32_t>(chunks),
+                                                                   static_cast<int32_t>(total_rows));
+    else
+        attention_merge_many_kernel<<<merge_grid, kAttnThreads, 0, s>>>(g, ws, static_cast<int32_t>(chunks),
+                                                                        static_cast<int32_t>(total_rows));
     return launch_status();
 }
