@@ -463,6 +463,20 @@ typedef struct rmlk_row_stream {
 int32_t rmlk_hip_head_rows(rmlk_stream_t stream, int32_t dtype, int32_t n_streams,
                            const rmlk_row_stream *streams, int32_t *err_flag);
 
+/* rmlk_hip_gemv_kmajor[_normed] and rmlk_hip_head_rows in one launch, for the q/k/v projection of
+ * ONE token: the one-row product x[k] . wt[n, k]^T (over RMSNorm(x) * gamma when gamma is given;
+ * gamma NULL: over x) is not stored; stream i takes its columns [first_col[i], first_col[i] +
+ * H * D) as the H rows of a [1, H, 1, D] tensor (streams[i].shape; x and x_stride are ignored) and
+ * rotates / moves / scatters them exactly as rmlk_hip_head_rows does (same arithmetic, same index
+ * rules and *err_flag). first_col is HOST memory. RMLK_ERR_UNSUPPORTED when a stream is not one
+ * token of one sequence, for more than 4 streams, or for operands the one-row products refuse.
+ * No counterpart in the reference (gemm.rs:191-232 followed by the kernels listed above). */
+int32_t rmlk_hip_gemv_kmajor_head_rows(rmlk_stream_t stream, int32_t dtype, int64_t k, const void *x,
+                                       const void *gamma, float eps, int32_t reciprocal_form,
+                                       const void *wt, int64_t ldw, int32_t n_streams,
+                                       const rmlk_row_stream *streams, const int64_t *first_col,
+                                       int32_t *err_flag);
+
 /* Fill `n` elements of `out` with the element at host address `value` (size of dtype).
  * ref: runtime/src/providers/cuda/backend/constant_of_shape.rs:59-62 (host vector + H2D). */
 int32_t rmlk_hip_fill(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *value,

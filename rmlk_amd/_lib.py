@@ -147,6 +147,9 @@ SIGNATURES = {
     "rmlk_hip_rotary": (c_int32, [c_void_p, c_int32, _PD, _PD, _PD, _PD, c_void_p, c_void_p,
                                   c_void_p, c_void_p]),
     "rmlk_hip_head_rows": (c_int32, [c_void_p, c_int32, c_int32, POINTER(RowStream), c_void_p]),
+    "rmlk_hip_gemv_kmajor_head_rows": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, ctypes.c_float,
+                                                 c_int32, c_void_p, c_int64, c_int32, c_void_p, c_void_p,
+                                                 c_void_p]),
     "rmlk_hip_fill": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
     "rmlk_hip_range": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p]),
     "rmlk_hip_write_small": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),

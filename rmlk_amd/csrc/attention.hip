@@ -355,8 +355,15 @@ __global__ __launch_bounds__(kAttnThreads) void attention_few_rows_kernel(AttnAr
     for (int idx = tid; idx < rows * 16; idx += kAttnThreads)
         *reinterpret_cast<v4f *>(&qs[idx / 16][(idx % 16) * 4]) =
             *reinterpret_cast<const v4f *>(Qg + static_cast<int64_t>(idx) * 4);
-    __syncthreads();
+    // the mask value of the wavefront's first row: asked for now, on its way with the chunk (after
+    // the dot product it would be a trip to memory of its own)
     const int key = chunk * kChunk + lane;
+    float mask_first = 0.f;
+    if (wave < rows && key < g.len) {
+        const int head = grp * g.rep + wave / g.seq, srow = wave - (wave / g.seq) * g.seq;
+        mask_first = g.mask[b * g.mask_b + head * g.mask_h + srow * g.mask_s + key];
+    }
+    __syncthreads();
     for (int r = wave; r < rows; r += kAttnThreads / kWave) {
         const int head = grp * g.rep + r / g.seq, srow = r - (r / g.seq) * g.seq;
         float dot = 0.f;
@@ -364,7 +371,8 @@ __global__ __launch_bounds__(kAttnThreads) void attention_few_rows_kernel(AttnAr
         for (int d = 0; d < kHeadDim; ++d) dot = fmaf(qs[r][d], Ks[lane][d], dot);
         float sc = -INFINITY;
         if (key < g.len) {
-            const float m = g.mask[b * g.mask_b + head * g.mask_h + srow * g.mask_s + key];
+            const float m = r == wave ? mask_first
+                                      : g.mask[b * g.mask_b + head * g.mask_h + srow * g.mask_s + key];
             sc = (scale_is_mul ? dot * scale : dot / scale) + m;
         }
         const float mx = wave_max(sc);

@@ -191,6 +191,14 @@ __global__ __launch_bounds__(kBlock) void head_rows_kernel(RowStreams all) {
         const uint32_t b = a.div_h.div(bh), h = bh - b * a.n_h;
         const int64_t xo = b * a.xs[0] + h * a.xs[1] + s * a.xs[2];
         const uint32_t d = q * W;
+        // the index tuple of the row first: its loads are then on their way together with the row's
+        // (asked for after the arithmetic, they were a second trip to memory of a 4 us launch)
+        int64_t ix[kMaxRowTuple];
+        if (a.idx) {
+#pragma unroll
+            for (int k = 0; k < kMaxRowTuple; ++k)
+                ix[k] = k < a.tuple_size ? a.idx[static_cast<int64_t>(row) * a.tuple_size + k] : 0;
+        }
         const V x1 = *reinterpret_cast<const V *>(a.x + xo + d);
         const V x2 = *reinterpret_cast<const V *>(a.x + xo + d + all.half);
         V y1 = x1, y2 = x2;
@@ -218,10 +226,10 @@ __global__ __launch_bounds__(kBlock) void head_rows_kernel(RowStreams all) {
 #pragma unroll
             for (int k = 0; k < kMaxRowTuple; ++k)
                 if (k < a.tuple_size) {
-                    int64_t ix = a.idx[static_cast<int64_t>(row) * a.tuple_size + k];
-                    if (ix < 0) ix += a.dim[k];
-                    if (ix < 0 || ix >= a.dim[k]) bad = true;
-                    out_row += ix * a.stride[k];
+                    int64_t i = ix[k];
+                    if (i < 0) i += a.dim[k];
+                    if (i < 0 || i >= a.dim[k]) bad = true;
+                    out_row += i * a.stride[k];
                 }
             if (bad) {
                 if (all.err) *all.err = 1;

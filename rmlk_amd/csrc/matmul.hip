@@ -1005,30 +1005,25 @@ struct RowNormArgs {
 constexpr int kGemvDepth = 8;                    // 128-bit units per lane, row and chunk
 constexpr int kGemvNormUnits = 8;                // NORM: units of x a lane holds (k <= 256 * 8 * 4)
 
-template <bool SWIGLU = false, bool NORM = false>
-__global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__restrict__ x,
-                                                          const float *__restrict__ wt,
-                                                          float *__restrict__ y, int32_t n, int32_t k,
-                                                          int64_t ldw, int32_t gate_row, int32_t up_row,
-                                                          const float *__restrict__ residual,
-                                                          RowNormArgs norm) {
-    constexpr int COLS = SWIGLU ? 2 : 1;
+// The dot products of one wavefront: COLS rows of Wt (wv[c], K-contiguous) with x or, NORM, with
+// RMSNorm(x) * gamma formed by the whole block in LDS. Every wavefront of the block calls this
+// (barriers); one that is not `active` skips the products. acc[c] is valid in every lane.
+struct NoExtraLoads {
+    __device__ __forceinline__ void operator()() const {}
+};
+// `extra_loads()` is called once the first chunk of weights has been requested: loads an epilogue
+// needs, on their way with the weights but not in front of the row (loads return in order).
+template <int COLS, bool NORM, typename Extra = NoExtraLoads>
+__device__ __forceinline__ void gemv_wave_dots(const float *__restrict__ x, const v4f *const (&wv)[COLS],
+                                               int32_t k, const RowNormArgs &norm, bool active,
+                                               float (&acc)[COLS], Extra extra_loads = Extra()) {
     constexpr int kWaves = kThreads / kWave;
     // the normalised row of the block (NORM): k floats of dynamic LDS
     extern __shared__ __align__(16) float xs[];
     __shared__ double partial[kWaves];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    const int col = blockIdx.x * kWaves + wave;
     const int k4 = k / 4;
     const v4f *xv = reinterpret_cast<const v4f *>(x);
-    // (a wavefront past the last column keeps valid addresses and takes part in the barriers)
-    const int col_c = min(col, n - 1);
-    const v4f *wv[COLS];
-#pragma unroll
-    for (int c = 0; c < COLS; ++c) {
-        const int64_t row = SWIGLU ? (c == 0 ? gate_row : up_row) + col_c : col_c;
-        wv[c] = reinterpret_cast<const v4f *>(wt + row * ldw);
-    }
     // NORM: this lane's share of the row and of gamma, requested before any weight
     [[maybe_unused]] v4f xn[kGemvNormUnits], gn[kGemvNormUnits];
     if constexpr (NORM) {
@@ -1067,8 +1062,9 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__re
         }
     };
     load_w(0, full_chunks == 0);      // in flight during the NORM prologue
+    extra_loads();
     if constexpr (NORM) {
-        double acc = 0.0;
+        double sq_sum = 0.0;
 #pragma unroll
         for (int i = 0; i < kGemvNormUnits; ++i) {
             if (i * kThreads < k4) {
@@ -1076,18 +1072,18 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__re
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const float sq = xn[i][j] * xn[i][j];
-                    acc += live ? static_cast<double>(sq) : 0.0;
+                    sq_sum += live ? static_cast<double>(sq) : 0.0;
                 }
             }
         }
-        acc = wave_sum(acc);
-        if (lane == 0) partial[wave] = acc;
+        sq_sum = wave_sum(sq_sum);
+        if (lane == 0) partial[wave] = sq_sum;
         __syncthreads();
-        acc = 0.0;
+        sq_sum = 0.0;
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) acc += partial[w];
+        for (int w = 0; w < kWaves; ++w) sq_sum += partial[w];
         const double kd = static_cast<double>(k);
-        const float mean = static_cast<float>((k & (k - 1)) == 0 ? acc * (1.0 / kd) : acc / kd);
+        const float mean = static_cast<float>((k & (k - 1)) == 0 ? sq_sum * (1.0 / kd) : sq_sum / kd);
         const float var = mean + norm.eps;
         const float r = sqrtf(var);
         const float inv = 1.0f / r;
@@ -1106,11 +1102,10 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__re
         }
         __syncthreads();
     }
-    if (col >= n) return;
-    const v4f *xsrc = NORM ? reinterpret_cast<const v4f *>(xs) : xv;
-    float acc[COLS];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) acc[c] = 0.f;
+    if (!active) return;
+    const v4f *xsrc = NORM ? reinterpret_cast<const v4f *>(xs) : xv;
     for (int chunk = 0; chunk < full_chunks; ++chunk) {
         if (chunk > 0) load_w(chunk, false);
         const v4f *px = xsrc + chunk * kChunkUnits + lane;
@@ -1143,7 +1138,29 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__re
     }
 #pragma unroll
     for (int c = 0; c < COLS; ++c) acc[c] = wave_sum(acc[c]);
-    if (lane == 0) {
+}
+
+template <bool SWIGLU = false, bool NORM = false>
+__global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__restrict__ x,
+                                                          const float *__restrict__ wt,
+                                                          float *__restrict__ y, int32_t n, int32_t k,
+                                                          int64_t ldw, int32_t gate_row, int32_t up_row,
+                                                          const float *__restrict__ residual,
+                                                          RowNormArgs norm) {
+    constexpr int COLS = SWIGLU ? 2 : 1;
+    const int lane = threadIdx.x % kWave;
+    const int col = blockIdx.x * (kThreads / kWave) + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    // (a wavefront past the last column keeps valid addresses and takes part in the barriers)
+    const int col_c = min(col, n - 1);
+    const v4f *wv[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+        const int64_t row = SWIGLU ? (c == 0 ? gate_row : up_row) + col_c : col_c;
+        wv[c] = reinterpret_cast<const v4f *>(wt + row * ldw);
+    }
+    float acc[COLS];
+    gemv_wave_dots<COLS, NORM>(x, wv, k, norm, col < n, acc);
+    if (col < n && lane == 0) {
         if constexpr (SWIGLU) {
             const float silu = acc[0] * (1.0f / (1.0f + expf(-acc[0])));
             y[col] = silu * acc[COLS - 1];
@@ -1151,6 +1168,116 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__re
             y[col] = residual ? acc[0] + residual[col] : acc[0];
         }
     }
+}
+
+// The same product with its result handed on as head rows (what rmlk_hip_head_rows does to the
+// output of a q/k/v projection) instead of being stored: the columns form up to four streams of
+// heads of D columns each, [first_col, first_col + heads * D); two wavefronts compute columns d and
+// d + D / 2 of a head, which is the pair a rotation needs; one of them rotates them (cos, sin) or leaves them,
+// and writes them to a dense [heads, D] output or to the row of a ScatterND destination that the
+// head's index tuple names. The table values and the index tuple are requested before the weights.
+constexpr int kGemvMaxStreams = 4;
+constexpr int kGemvMaxTuple = 4;
+struct GemvRowStream {
+    const float *cos, *sin;          // null: the pair is not rotated
+    float *out;
+    const int64_t *idx;              // null: dense output
+    int32_t first_col, heads;
+    int32_t first_pair;              // pairs of the streams before this one
+    int32_t tuple_size;
+    int64_t cs_head, ss_head;        // element strides of cos / sin from one head to the next
+    int64_t dim[kGemvMaxTuple], stride[kGemvMaxTuple];   // leading dims of the scatter destination, in rows
+};
+struct GemvRowStreams {
+    GemvRowStream s[kGemvMaxStreams];
+    int32_t n_streams, half, total_pairs;
+    int32_t *err;
+};
+
+template <bool NORM>
+__global__ __launch_bounds__(kThreads) void gemv_kmajor_rows_kernel(const float *__restrict__ x,
+                                                                    const float *__restrict__ wt, int32_t k,
+                                                                    int64_t ldw, RowNormArgs norm,
+                                                                    GemvRowStreams rs) {
+    // A wavefront per column, like the plain product (two columns per wavefront left the SIMDs with
+    // one or two wavefronts each, 8.5 against 6.3 us on the 3072 columns of q, k and v): wavefronts
+    // 2 p and 2 p + 1 of a block take columns d and d + D / 2 of a pair and meet in LDS.
+    constexpr int kWaves = kThreads / kWave;
+    __shared__ float pair_acc[kWaves];
+    // (the wavefront's number as a scalar: everything derived from it - the stream, the head, the
+    // row of the weights - then lives in scalar registers and the stream table is read with scalar loads)
+    const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int pair = blockIdx.x * (kWaves / 2) + wave / 2;
+    const int second = wave & 1;
+    const bool active = pair < rs.total_pairs;
+    const int pair_c = min(pair, rs.total_pairs - 1);
+    int si = 0;
+#pragma unroll
+    for (int i = 1; i < kGemvMaxStreams; ++i)
+        if (i < rs.n_streams && pair_c >= rs.s[i].first_pair) si = i;
+    const GemvRowStream &st = rs.s[si];
+    const int local = pair_c - st.first_pair;
+    const int head = local / rs.half, d = local - head * rs.half;
+    const int col = st.first_col + head * (2 * rs.half) + d + second * rs.half;
+    const v4f *wv[1];
+    wv[0] = reinterpret_cast<const v4f *>(wt + static_cast<int64_t>(col) * ldw);
+    // what the epilogue needs from memory (in the wavefront that runs it), requested behind the
+    // first weights
+    float c1 = 1.f, c2 = 1.f, s1 = 0.f, s2 = 0.f;
+    int64_t ix[kGemvMaxTuple];
+    auto epilogue_loads = [&]() {
+        if (second) return;
+        if (st.cos) {
+            const float *cp = st.cos + head * st.cs_head + d, *sp = st.sin + head * st.ss_head + d;
+            c1 = cp[0];
+            c2 = cp[rs.half];
+            s1 = sp[0];
+            s2 = sp[rs.half];
+        }
+        if (st.idx) {
+#pragma unroll
+            for (int t = 0; t < kGemvMaxTuple; ++t)
+                ix[t] = t < st.tuple_size ? st.idx[static_cast<int64_t>(head) * st.tuple_size + t] : 0;
+        }
+    };
+    float acc[1];
+    gemv_wave_dots<1, NORM>(x, wv, k, norm, active, acc, epilogue_loads);
+    if (lane == 0) pair_acc[wave] = acc[0];
+    __syncthreads();
+    if (!active || lane != 0 || second) return;
+    const float x1 = acc[0], x2 = pair_acc[wave + 1];
+    float y1 = x1, y2 = x2;
+    if (st.cos) {
+        // (products and sums rounded one by one, although this file is compiled with contraction
+        // allowed: the expressions and roundings of rotary_kernel / head_rows_kernel)
+#pragma clang fp contract(off)
+        const float a1 = x1 * c1;
+        const float r1 = (-x2) * s1;
+        y1 = a1 + r1;
+        const float a2 = x2 * c2;
+        const float r2 = x1 * s2;
+        y2 = a2 + r2;
+    }
+    int64_t out_row = head;
+    if (st.idx) {
+        out_row = 0;
+        bool bad = false;
+#pragma unroll
+        for (int t = 0; t < kGemvMaxTuple; ++t)
+            if (t < st.tuple_size) {
+                int64_t i = ix[t];
+                if (i < 0) i += st.dim[t];
+                if (i < 0 || i >= st.dim[t]) bad = true;
+                out_row += i * st.stride[t];
+            }
+        if (bad) {
+            if (rs.err) *rs.err = 1;
+            return;
+        }
+    }
+    float *o = st.out + out_row * (2 * rs.half) + d;
+    o[0] = y1;
+    o[rs.half] = y2;
 }
 
 // Any-layout fallback (transposed operands with M > 1): one lane per C element.
@@ -1899,6 +2026,90 @@ int32_t gemv_kmajor_swiglu_launch(rmlk_stream_t stream, int32_t dtype, int64_t n
 }
 
 }  // namespace
+
+extern "C" int32_t rmlk_hip_gemv_kmajor_head_rows(rmlk_stream_t stream, int32_t dtype, int64_t k,
+                                                  const void *x, const void *gamma, float eps,
+                                                  int32_t reciprocal_form, const void *wt, int64_t ldw,
+                                                  int32_t n_streams, const rmlk_row_stream *streams,
+                                                  const int64_t *first_col, int32_t *err_flag) {
+    if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (n_streams < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n_streams == 0) return RMLK_OK;
+    if (n_streams > kGemvMaxStreams) return RMLK_ERR_UNSUPPORTED;
+    if (!streams || !first_col || (k > 0 && (!x || !wt))) return RMLK_ERR_NULL_POINTER;
+    if (k >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
+    if (ldw < k) return RMLK_ERR_SIZE_MISMATCH;
+    if (k == 0 || k % 4 != 0 || ldw % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(wt) % 16 != 0)
+        return RMLK_ERR_UNSUPPORTED;
+    if (gamma && (k > kThreads * 4 * kGemvNormUnits || reinterpret_cast<uintptr_t>(gamma) % 16 != 0))
+        return RMLK_ERR_UNSUPPORTED;
+    GemvRowStreams rs{};
+    rs.err = err_flag;
+    int64_t d_common = -1, pairs = 0;
+    for (int i = 0; i < n_streams; ++i) {
+        const rmlk_row_stream &in = streams[i];
+        const bool rotate = in.cos || in.sin;
+        if (!dims_ok(&in.shape) || in.shape.rank != 4) return RMLK_ERR_BAD_RANK;
+        if (rotate && (!dims_ok(&in.cos_stride) || !dims_ok(&in.sin_stride) || in.cos_stride.rank != 4 ||
+                       in.sin_stride.rank != 4))
+            return RMLK_ERR_BAD_RANK;
+        if (dims_numel(&in.shape) <= 0) return RMLK_ERR_INVALID_ARGUMENT;
+        // one row of the product: one token of one sequence
+        if (in.shape.v[0] != 1 || in.shape.v[2] != 1) return RMLK_ERR_UNSUPPORTED;
+        const int64_t heads = in.shape.v[1], d = in.shape.v[3];
+        if (d % 2 != 0 || (d_common >= 0 && d != d_common)) return RMLK_ERR_UNSUPPORTED;
+        d_common = d;
+        if (!in.out || (rotate && (!in.cos || !in.sin))) return RMLK_ERR_NULL_POINTER;
+        if (rotate && (in.cos_stride.v[3] != 1 || in.sin_stride.v[3] != 1 || in.cos_stride.v[1] < 0 ||
+                       in.sin_stride.v[1] < 0))
+            return RMLK_ERR_UNSUPPORTED;
+        if (first_col[i] < 0 || first_col[i] + heads * d >= (1ll << 31)) return RMLK_ERR_INVALID_ARGUMENT;
+        GemvRowStream &a = rs.s[i];
+        a.cos = rotate ? static_cast<const float *>(in.cos) : nullptr;
+        a.sin = rotate ? static_cast<const float *>(in.sin) : nullptr;
+        a.out = static_cast<float *>(in.out);
+        a.idx = in.idx;
+        a.first_col = static_cast<int32_t>(first_col[i]);
+        a.heads = static_cast<int32_t>(heads);
+        a.first_pair = static_cast<int32_t>(pairs);
+        a.cs_head = rotate ? in.cos_stride.v[1] : 0;
+        a.ss_head = rotate ? in.sin_stride.v[1] : 0;
+        a.tuple_size = 0;
+        if (in.idx) {
+            if (!dims_ok(&in.data_shape)) return RMLK_ERR_BAD_RANK;
+            if (in.tuple_size < 1 || in.tuple_size != in.data_shape.rank - 1) return RMLK_ERR_INVALID_ARGUMENT;
+            if (in.tuple_size > kGemvMaxTuple) return RMLK_ERR_UNSUPPORTED;
+            if (in.data_shape.v[in.tuple_size] != d || dims_numel(&in.data_shape) < 0)
+                return RMLK_ERR_INVALID_ARGUMENT;
+            if (dims_numel(&in.data_shape) >= ((int64_t)1 << 40)) return RMLK_ERR_TOO_LARGE;
+            a.tuple_size = in.tuple_size;
+            int64_t stride = 1;
+            for (int t = a.tuple_size - 1; t >= 0; --t) {
+                a.dim[t] = in.data_shape.v[t];
+                a.stride[t] = stride;
+                stride *= in.data_shape.v[t];
+            }
+        }
+        pairs += heads * (d / 2);
+        if (pairs >= (1ll << 30)) return RMLK_ERR_TOO_LARGE;
+    }
+    rs.n_streams = n_streams;
+    rs.half = static_cast<int32_t>(d_common / 2);
+    rs.total_pairs = static_cast<int32_t>(pairs);
+    constexpr int kPairsPerBlock = kThreads / kWave / 2;
+    const unsigned grid = static_cast<unsigned>((pairs + kPairsPerBlock - 1) / kPairsPerBlock);
+    const float *px = static_cast<const float *>(x), *pw = static_cast<const float *>(wt);
+    const int32_t ki = static_cast<int32_t>(k);
+    hipStream_t s = as_stream(stream);
+    if (gamma) {
+        const RowNormArgs norm{static_cast<const float *>(gamma), eps, reciprocal_form};
+        gemv_kmajor_rows_kernel<true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
+    } else {
+        gemv_kmajor_rows_kernel<false><<<grid, kThreads, 0, s>>>(px, pw, ki, ldw, RowNormArgs{}, rs);
+    }
+    return launch_status();
+}
 
 extern "C" int32_t rmlk_hip_gemv_kmajor(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
                                    const void *x, const void *wt, int64_t ldw, void *y) {

@@ -81,6 +81,7 @@ struct HostVal {
 };
 
 struct PendingNorm;
+struct PendingProduct;
 
 struct Tensor {
     int32_t dtype = 0;
@@ -92,6 +93,11 @@ struct Tensor {
     // the norm, and the one consumer (a one-row product, which the fusion pass has checked) applies
     // the norm while it loads the row, or computes it first if it cannot.
     std::shared_ptr<const PendingNorm> pending_norm;
+    // Set on the members of a one-row product over joint K-contiguous weights that was NOT computed
+    // (and on views of them): the memory is reserved but not written. The fusion pass has checked
+    // that everything that reads them is one row-stream node, which either runs the product and
+    // its own work as one launch or has the product computed first.
+    std::shared_ptr<PendingProduct> pending_product;
 
     bool defined() const { return dtype != 0; }
     int64_t numel() const {
@@ -109,6 +115,7 @@ struct Tensor {
         offset = 0;
         host.reset();
         pending_norm.reset();
+        pending_product.reset();
     }
 };
 
@@ -116,6 +123,15 @@ struct PendingNorm {
     Tensor gamma;
     float eps = 0.f;
     int32_t reciprocal = 0;
+};
+
+struct PendingProduct {
+    Tensor x;                                   // the input row (before `norm`, when there is one)
+    std::shared_ptr<const PendingNorm> norm;    // null: x as it is
+    Tensor wt;                                  // the joint weights, K-contiguous [total, k]
+    Tensor row;                                 // where the product goes when it has to be stored
+    int64_t k = 0, total = 0;
+    bool computed = false;                      // stored in `row`, or consumed by the fused launch
 };
 
 rmlk_dims to_dims(const std::vector<int64_t> &v);          // rank-0 becomes [1]

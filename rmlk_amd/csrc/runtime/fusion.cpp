@@ -630,6 +630,34 @@ struct Matcher {
         return marked;
     }
 
+    // ---- joint one-row products whose members only feed one row-stream node -----------------------
+    // (through a Reshape each: the q/k/v projection in front of rmlk.HeadRows). For a one-row input
+    // such a product is left to the row-stream node, which runs it and its own work as one launch.
+    int mark_deferred_products() {
+        int marked = 0;
+        for (size_t n = 0; n < g.nodes.size(); ++n) {
+            if (removed[n]) continue;
+            Node &p = g.nodes[n];
+            if (p.op != "rmlk.MatMulGroup" || p.inputs.size() != 3) continue;
+            int reader = -1;
+            bool ok = true;
+            for (int o : p.outputs) {
+                if (g.values[o].is_output || users[o].size() != 1) { ok = false; break; }
+                const Node &r = g.nodes[users[o][0]];
+                if (r.op != "Reshape" || r.inputs.empty() || r.inputs[0] != o || r.outputs.size() != 1) { ok = false; break; }
+                const int v = r.outputs[0];
+                if (g.values[v].is_output || users[v].size() != 1) { ok = false; break; }
+                const int h = users[v][0];
+                if (g.nodes[h].op != "rmlk.HeadRows" || (reader >= 0 && h != reader)) { ok = false; break; }
+                reader = h;
+            }
+            if (!ok || reader < 0) continue;
+            p.attrs["defer_product"] = a_int(1);
+            ++marked;
+        }
+        return marked;
+    }
+
     // ---- a producer whose split-K combine can move into the consumer -----------------------------
     // (Tried for one-row inputs as well and dropped, both slower than what they replace: MatMul ->
     // AddRMSNorm, where the norm owns a row with ONE block that then adds up 32-64 slabs by itself;
@@ -1144,6 +1172,32 @@ void op_fused_rotary(OpContext &c) {
     run_body(c);
 }
 
+// A one-row product that was left to its reader and has to be stored after all.
+void store_product(OpContext &c, PendingProduct &pp) {
+    int32_t st;
+    if (pp.norm)
+        st = rmlk_hip_gemv_kmajor_normed(c.stream, RMLK_FLOAT, pp.total, pp.k, pp.x.data(), pp.norm->gamma.data(),
+                                         pp.norm->eps, pp.norm->reciprocal, pp.wt.data(), pp.k, pp.row.data());
+    else
+        st = rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, pp.total, pp.k, pp.x.data(), pp.wt.data(), pp.k,
+                                  pp.row.data());
+    if (st == RMLK_ERR_UNSUPPORTED && pp.norm) {
+        // (a row the one-row kernels refuse to normalise: norm, then product)
+        Tensor normed;
+        std::vector<Tensor *> keep = c.out;
+        c.out = {&normed};
+        c.alloc_output(0, RMLK_FLOAT, pp.x.shape);
+        c.out = keep;
+        check_status(rmlk_hip_rmsnorm(c.stream, RMLK_FLOAT, 1, pp.k, pp.x.data(), pp.norm->gamma.data(),
+                                      pp.norm->eps, pp.norm->reciprocal, normed.data()),
+                     "rmlk.RMSNorm (deferred)");
+        st = rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, pp.total, pp.k, normed.data(), pp.wt.data(), pp.k,
+                                  pp.row.data());
+    }
+    check_status(st, "rmlk.MatMulGroup (deferred)");
+    pp.computed = true;
+}
+
 // Streams of head rows (rmlk.HeadRows): per stream, by `kinds`,
 //   0  rmlk.Rotary                                 inputs src, cos, sin
 //   1  rmlk.Rotary -> ScatterND(data, idx, .)      inputs src, cos, sin, data, idx
@@ -1189,15 +1243,48 @@ void op_fused_head_rows(OpContext &c) {
                  data.numel() > 0;
         }
     }
+    // Sources that are members of a one-row product left to this node (op_fused_matmul_group): the
+    // product and the row streams run as one launch when every source is a member of the same
+    // product and a [1, H, 1, D] tensor with its heads side by side; otherwise the product is
+    // computed first, and everything below finds its rows in memory.
+    std::shared_ptr<PendingProduct> product;
+    bool one_launch = ok;
+    {
+        std::vector<std::shared_ptr<PendingProduct>> seen;
+        int at_src = 0;
+        for (size_t i = 0; i < n; ++i) {
+            const Tensor &src = c.input(at_src);
+            at_src += kinds[i] == 2 ? 3 : (kinds[i] == 1 ? 5 : 3);
+            const std::shared_ptr<PendingProduct> &pp = src.pending_product;
+            if (!pp || pp->computed) {
+                one_launch = false;
+                continue;
+            }
+            if (std::find(seen.begin(), seen.end(), pp) == seen.end()) seen.push_back(pp);
+            if (ok) {
+                const std::vector<int64_t> &sh = lay[i].shape, &xs = lay[i].xst;
+                if (sh[0] != 1 || sh[2] != 1 || xs[1] != sh[3] || xs[3] != 1) one_launch = false;
+            }
+        }
+        if (seen.size() != 1) one_launch = false;
+        if (one_launch) {
+            product = seen[0];
+        } else {
+            for (const std::shared_ptr<PendingProduct> &pp : seen) store_product(c, *pp);
+        }
+    }
     if (!ok) {
         run_body(c);
         return;
     }
     std::vector<rmlk_row_stream> streams(n);
+    std::vector<int64_t> first_col(n, 0);
     for (size_t i = 0; i < n; ++i) {
         rmlk_row_stream &st = streams[i];
         st = rmlk_row_stream{};
         int in = first_input[i];
+        if (product)
+            first_col[i] = static_cast<int64_t>(c.input(in).offset - product->row.offset) / static_cast<int64_t>(sizeof(float));
         st.shape = to_dims(lay[i].shape);
         st.x_stride = to_dims(lay[i].xst);
         st.x = c.input(in++).data();
@@ -1216,6 +1303,19 @@ void op_fused_head_rows(OpContext &c) {
             st.idx = static_cast<const int64_t *>(idx.data());
             st.out = scatter_destination(c, in, static_cast<int>(i)).data();
         }
+    }
+    if (product) {
+        const PendingProduct &pp = *product;
+        const int32_t st = rmlk_hip_gemv_kmajor_head_rows(
+            c.stream, RMLK_FLOAT, pp.k, pp.x.data(), pp.norm ? pp.norm->gamma.data() : nullptr,
+            pp.norm ? pp.norm->eps : 0.f, pp.norm ? pp.norm->reciprocal : 0, pp.wt.data(), pp.k,
+            static_cast<int32_t>(n), streams.data(), first_col.data(), c.error_flag());
+        if (took_fast_path(st, "rmlk.HeadRows (with its projection)")) {
+            product->computed = true;   // consumed: nothing else reads its members
+            return;
+        }
+        // the one-row kernels refuse these operands: the product on its own, then the streams
+        store_product(c, *product);
     }
     if (took_fast_path(rmlk_hip_head_rows(c.stream, RMLK_FLOAT, static_cast<int32_t>(n), streams.data(),
                                           c.error_flag()),
@@ -1554,6 +1654,32 @@ void op_fused_matmul_group(OpContext &c) {
             c.alloc_output(0, RMLK_FLOAT, {total});
             c.out = keep;
         }
+        auto hand_out = [&](const std::shared_ptr<PendingProduct> &pp) {
+            int64_t off = 0;
+            for (size_t i = 0; i < widths.size(); ++i) {
+                Tensor v;
+                v.dtype = RMLK_FLOAT;
+                v.shape = out_shape(widths[i]);
+                v.buf = row.buf;
+                v.offset = row.offset + static_cast<size_t>(off) * sizeof(float);
+                v.pending_product = pp;
+                *c.out[i] = v;
+                off += widths[i];
+            }
+        };
+        if (RMLK_DEFER_NORM && c.attr_int("defer_product", 0) != 0 && c.has_input(2) && k % 4 == 0 && k > 0) {
+            // left to the row-stream node behind it (op_fused_head_rows)
+            auto pp = std::make_shared<PendingProduct>();
+            pp->x = a;
+            pp->x.pending_norm.reset();
+            pp->norm = pending;
+            pp->wt = c.input(2);
+            pp->row = row;
+            pp->k = k;
+            pp->total = total;
+            hand_out(pp);
+            return;
+        }
         // (over its K-contiguous copy when there is one: no split-K, no combine launch)
         bool done = false;
         if (pending) {
@@ -1570,16 +1696,7 @@ void op_fused_matmul_group(OpContext &c) {
                                                            c.input(2).data(), k, row.data()),
                                       "rmlk.MatMulGroup")))
             run(total, w.data(), row.data(), total);
-        int64_t off = 0;
-        for (size_t i = 0; i < widths.size(); ++i) {
-            Tensor v;
-            v.dtype = RMLK_FLOAT;
-            v.shape = out_shape(widths[i]);
-            v.buf = row.buf;
-            v.offset = row.offset + static_cast<size_t>(off) * sizeof(float);
-            *c.out[i] = v;
-            off += widths[i];
-        }
+        hand_out(nullptr);
         return;
     }
     if (widths.size() <= 4) {
@@ -1631,6 +1748,7 @@ int fuse_patterns(Session &s) {
     formed += m.form_splitk_epilogues();
     formed += m.form_const_matmuls();
     if (formed) m.mark_deferred_norms();   // an attribute on existing fused nodes, not a node of its own
+    if (formed) m.mark_deferred_products();
     if (!formed) return 0;
     std::vector<Node> kept;
     kept.reserve(m.g.nodes.size());

@@ -166,6 +166,7 @@ Tensor &OpContext::view_output(int i, const Tensor &src, const std::vector<int64
     v.shape = shape;
     v.buf = src.buf;
     v.offset = src.offset;
+    v.pending_product = src.pending_product;   // a view of a product not computed yet is not computed either
     *out[i] = v;
     return *out[i];
 }

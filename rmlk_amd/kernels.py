@@ -318,12 +318,21 @@ def head_rows(streams, err_flag=None) -> None:
     """Several streams of head rows in one launch. Each stream is a dict: x, shape [B,H,S,D],
     x_stride, out, and optionally cos, sin, cos_stride, sin_stride (rotate) and idx, data_shape
     (scatter the rows into `out` by index tuples)."""
+    arr = _row_streams(streams)
+    dt = dtype_of(streams[0]["x"]) if streams else 1
+    check(lib().rmlk_hip_head_rows(_stream(), dt, len(streams), arr,
+                                   _ptr(err_flag) if err_flag is not None else None),
+          "rmlk_hip_head_rows")
+
+
+def _row_streams(streams, with_x=True):
     from ._lib import RowStream
     arr = (RowStream * len(streams))()
     for st, d in zip(arr, streams):
         st.shape = Dims.of(d["shape"])
-        st.x_stride = Dims.of(d["x_stride"])
-        st.x = _ptr(d["x"])
+        if with_x:
+            st.x_stride = Dims.of(d["x_stride"])
+            st.x = _ptr(d["x"])
         if d.get("cos") is not None:
             st.cos, st.sin = _ptr(d["cos"]), _ptr(d["sin"])
             st.cos_stride, st.sin_stride = Dims.of(d["cos_stride"]), Dims.of(d["sin_stride"])
@@ -332,10 +341,20 @@ def head_rows(streams, err_flag=None) -> None:
             st.idx = _ptr(d["idx"])
             st.data_shape = Dims.of(d["data_shape"])
             st.tuple_size = len(d["data_shape"]) - 1
-    dt = dtype_of(streams[0]["x"]) if streams else 1
-    check(lib().rmlk_hip_head_rows(_stream(), dt, len(streams), arr,
-                                   _ptr(err_flag) if err_flag is not None else None),
-          "rmlk_hip_head_rows")
+    return arr
+
+
+def gemv_kmajor_head_rows(x, wt, k: int, streams, first_cols, gamma=None, eps: float = 0.0,
+                          reciprocal_form: bool = False, err_flag=None) -> None:
+    """The q/k/v projection of one token (x . wt^T over K-contiguous weights, over RMSNorm(x) * gamma
+    when gamma is given) with its result handed on as head rows (see head_rows; streams carry no x)
+    in one launch. first_cols[i]: first product column of stream i."""
+    arr = _row_streams(streams, with_x=False)
+    cols = (ctypes.c_int64 * len(streams))(*[int(c) for c in first_cols])
+    check(lib().rmlk_hip_gemv_kmajor_head_rows(_stream(), dtype_of(x), k, _ptr(x), _ptr(gamma), eps,
+                                               int(reciprocal_form), _ptr(wt), k, len(streams), arr, cols,
+                                               _ptr(err_flag) if err_flag is not None else None),
+          "rmlk_hip_gemv_kmajor_head_rows")
 
 
 def device_info(device: int = 0) -> dict:

@@ -255,6 +255,72 @@ def test_head_rows_flag_an_index_out_of_range_and_check_their_arguments(device):
     k.head_rows([], err)                 # nothing to do
 
 
+@pytest.mark.parametrize("hq,hk,d,k,length,normed", [(32, 8, 64, 2048, 640, True), (32, 8, 64, 2048, 640, False),
+                                                     (6, 2, 64, 384, 40, True), (4, 4, 16, 100, 9, False),
+                                                     (3, 1, 128, 520, 33, True)])
+def test_one_token_projection_with_its_head_rows_in_one_launch(device, hq, hk, d, k, length, normed):
+    """The q/k/v projection of one token, rotated / scattered behind it, in ONE launch equals the
+    one-row product followed by the row-stream launch bit for bit."""
+    import torch
+    kk = _k()
+    rng = np.random.default_rng(hq + d + k)
+    n = (hq + 2 * hk) * d
+    x = to_dev(rng.standard_normal(k, dtype=np.float32), device)
+    wt = to_dev((rng.standard_normal((n, k), dtype=np.float32) * 0.05), device)
+    gamma = to_dev(rng.uniform(0.5, 1.5, size=k).astype(np.float32), device) if normed else None
+    cos = to_dev(rng.uniform(-1, 1, size=(1, 1, 1, d)).astype(np.float32), device)
+    sin = to_dev(rng.uniform(-1, 1, size=(1, 1, 1, d)).astype(np.float32), device)
+    cache_shape = [1, hk, length, d]
+    kc = rng.standard_normal(cache_shape, dtype=np.float32)
+    vc = rng.standard_normal(cache_shape, dtype=np.float32)
+    idx = np.zeros((1, hk, 1, 3), np.int64)
+    idx[0, :, 0, 1] = np.arange(hk)
+    idx[0, :, 0, 2] = length - 2
+    idx[0, 0, 0, 2] -= length                        # a negative index wraps
+    idx_d = to_dev(idx, device)
+    tab = [0, 0, 0, 1]
+    # two launches
+    y = torch.empty(n, device=device)
+    if normed:
+        kk.gemv_kmajor_normed(x, gamma, wt, y, n, k, 1e-5)
+    else:
+        kk.gemv_kmajor(x, wt, y, n, k)
+    q_exp = torch.empty(hq * d, device=device)
+    kc_exp, vc_exp = to_dev(kc, device), to_dev(vc, device)
+    err = torch.zeros(1, dtype=torch.int32, device=device)
+    def streams(q_out, k_out, v_out, src=None):
+        def with_x(dct, first, h):
+            if src is not None:
+                dct.update(x=src[first:first + h * d], x_stride=[h * d, d, h * d, 1])
+            return dct
+        return [
+            with_x(dict(shape=[1, hq, 1, d], cos=cos, sin=sin, cos_stride=tab, sin_stride=tab, out=q_out), 0, hq),
+            with_x(dict(shape=[1, hk, 1, d], cos=cos, sin=sin, cos_stride=tab, sin_stride=tab, out=k_out,
+                        idx=idx_d, data_shape=cache_shape), hq * d, hk),
+            with_x(dict(shape=[1, hk, 1, d], out=v_out, idx=idx_d, data_shape=cache_shape), (hq + hk) * d, hk)]
+    kk.head_rows(streams(q_exp, kc_exp, vc_exp, src=y), err)
+    # one launch
+    q_got = torch.full_like(q_exp, 9.0)
+    kc_got, vc_got = to_dev(kc, device), to_dev(vc, device)
+    kk.gemv_kmajor_head_rows(x, wt, k, streams(q_got, kc_got, vc_got), [0, hq * d, (hq + hk) * d],
+                             gamma=gamma, eps=1e-5, err_flag=err)
+    assert_exact(to_np(q_got), to_np(q_exp))
+    assert_exact(to_np(kc_got), to_np(kc_exp))
+    assert_exact(to_np(vc_got), to_np(vc_exp))
+    assert int(err.item()) == 0
+    # an index past the end of the cache: the flag, and that head's row is not written
+    idx[0, hk - 1, 0, 2] = length
+    kc_bad = to_dev(kc, device)
+    st = streams(q_got, kc_bad, vc_got)[:2]
+    st[1]["idx"] = to_dev(idx, device)
+    kk.gemv_kmajor_head_rows(x, wt, k, st, [0, hq * d], gamma=gamma, eps=1e-5, err_flag=err)
+    assert int(err.item()) == 1
+    got = to_np(kc_bad)
+    assert_exact(got[0, hk - 1], kc[0, hk - 1])
+    if hk > 1:
+        assert_exact(got[0, :hk - 1], to_np(kc_exp)[0, :hk - 1])
+
+
 # ---- session level: the fusion pass ------------------------------------------------------------
 
 def _run_both(graph, feeds, outputs=None):
