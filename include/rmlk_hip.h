@@ -335,6 +335,23 @@ int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch, i
                            const void *q, const void *k, const void *v, const void *mask,
                            const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
                            int32_t out_seq_major, void *out);
+/* The same kernel with room to skip what the mask hides: with `workspace` of at least
+ * rmlk_hip_attention_workspace_size() bytes a small kernel first marks, per tile of 64 queries and
+ * chunk of 64 keys, whether the mask holds anything but -inf there, and the main kernel neither loads
+ * nor multiplies the chunks a tile cannot see (a causal mask: about half of them). Their probabilities
+ * are exact zeros, so results are those of rmlk_hip_attention bit for bit, with two exceptions: a NaN
+ * or infinity in a K or V row no query of the tile can see does not reach that tile's output
+ * (0 * NaN would), and a row with nothing visible anywhere is NaN as before. The size is 0 (and a
+ * null workspace allowed) where skipping does not apply: few blocks, q_len not a multiple of 64, or
+ * more than 128 chunks. rmlk_hip_attention is this call with a null workspace. */
+size_t rmlk_hip_attention_workspace_size(int32_t dtype, int64_t batch, int64_t kv_heads, int64_t rep,
+                                         int64_t q_len, int64_t kv_len, int64_t head_dim,
+                                         const rmlk_dims *mask_stride);
+int32_t rmlk_hip_attention_ws(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t kv_heads,
+                              int64_t rep, int64_t q_len, int64_t kv_len, int64_t head_dim,
+                              const void *q, const void *k, const void *v, const void *mask,
+                              const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
+                              int32_t out_seq_major, void *workspace, size_t workspace_bytes, void *out);
 
 /* The same attention for a handful of query rows per KV head (rep * q_len <= 16: a decode step),
  * where there is no matrix work, only K and V to read: the keys are split over blocks in chunks of

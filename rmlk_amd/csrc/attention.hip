@@ -30,10 +30,6 @@ namespace {
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-// 0: always four wavefronts per block (to compare)
-#ifndef RMLK_ATTN_WIDE_BLOCKS
-#define RMLK_ATTN_WIDE_BLOCKS 1
-#endif
 
 constexpr int kAttnThreads = 256;                 // of the few-rows kernels
 constexpr int kHeadDim = 64;
@@ -69,6 +65,18 @@ struct AttnArgs {
     int64_t mask_b, mask_h, mask_s;   // element strides of the mask over batch, head, query
     int64_t out_b, out_h, out_s;      // element strides of out over batch, head, query
     float qscale;      // score scale (folded into the query)
+    // Visibility of the mask per (64-query tile, key chunk), one byte each, or null: a chunk whose
+    // mask is -inf for all 64 queries of the block is not loaded and not multiplied (its
+    // probabilities are exact zeros). Laid out [.., tile, chunk]; tiles_b / tiles_h are the byte
+    // strides over batch and head (0 where the mask is broadcast).
+    const uint8_t *tiles;
+    int64_t tiles_b, tiles_h;
+    // With a tile map the blocks differ in work (a causal mask: 1 to L / 64 chunks), and blocks are
+    // handed out in order: the grid is then as many blocks as fit the chip at once, each taking the
+    // next (query tile, KV head) item from this counter until they run out - last query tiles first,
+    // which under a causal mask are the long ones. Null: block (x, y) is item (tile x, KV head y).
+    int32_t *queue;
+    int32_t items, tiles_per_head;
 };
 
 template <int NK>
@@ -82,12 +90,53 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     const int lane = tid % kWave, wave = tid / kWave;
     const int l32 = lane % 32, half = lane / 32;
     const int wq = wave / NK, wk = wave % NK;
-    const int bg = blockIdx.y;
+    __shared__ int next_item;
+    for (;;) {
+    int bg = blockIdx.y, tile_x = blockIdx.x;
+    if (g.queue) {
+        if (tid == 0) next_item = atomicAdd(g.queue, 1);
+        __syncthreads();
+        const int item = next_item;
+        if (item >= g.items) break;   // every block ends here: the counter only grows
+        // items by falling query tile; inside one tile index, all the heads of all the KV heads
+        const int n_bg = g.items / (g.tiles_per_head * g.rep);
+        const int per_tile = n_bg * g.rep;
+        const int t = g.tiles_per_head - 1 - item / per_tile, hb = item % per_tile;
+        bg = hb / g.rep;
+        tile_x = (hb - bg * g.rep) * g.tiles_per_head + t;
+    }
     const int b = bg / g.kv_heads, grp = bg - b * g.kv_heads;
-    const int r0 = blockIdx.x * 64;
+    const int r0 = tile_x * 64;
     const float *Kg = g.k + static_cast<int64_t>(bg) * g.len * kHeadDim;
     const float *Vg = g.v + static_cast<int64_t>(bg) * g.len * kHeadDim;
     const int n_chunks = (g.len + kKeys - 1) / kKeys;
+
+    // ---- the chunks this block visits (bit c of active[c / 64]); all of them without a tile map ------
+    uint64_t active[2];
+    active[0] = n_chunks >= 64 ? ~0ull : ((1ull << n_chunks) - 1);
+    active[1] = n_chunks >= 128 ? ~0ull : (n_chunks > 64 ? ((1ull << (n_chunks - 64)) - 1) : 0ull);
+    if (g.tiles) {   // (the launcher gives a map only for n_chunks <= 128 and seq % 64 == 0: a tile lies in one head)
+        const int head0 = grp * g.rep + r0 / g.seq, srow0 = r0 - (r0 / g.seq) * g.seq;
+        const uint8_t *tp = g.tiles + b * g.tiles_b + head0 * g.tiles_h + static_cast<int64_t>(srow0 / 64) * n_chunks;
+        const bool f0 = lane < n_chunks && tp[min(lane, n_chunks - 1)] != 0;
+        const bool f1 = lane + 64 < n_chunks && tp[min(lane + 64, n_chunks - 1)] != 0;
+        active[0] = __builtin_amdgcn_ballot_w64(f0);
+        active[1] = __builtin_amdgcn_ballot_w64(f1);
+        if ((active[0] | active[1]) == 0) active[0] = 1;   // nothing visible at all: chunk 0 gives the NaN rows
+    }
+    auto next_active = [&](int c) {   // the first visited chunk after c, -1 when there is none
+        const int from = c + 1;
+        if (from < 64) {
+            const uint64_t m = active[0] & (~0ull << from);
+            if (m) return static_cast<int>(__builtin_ctzll(m));
+        }
+        if (from < 128) {
+            const uint64_t m = from <= 64 ? active[1] : (active[1] & (~0ull << (from - 64)));
+            if (m) return 64 + static_cast<int>(__builtin_ctzll(m));
+        }
+        if (from >= 128 && from < n_chunks) return from;   // beyond the map: every chunk
+        return -1;
+    };
 
     // ---- staging: piece p * 2 NK + wave of a chunk (4 keys, 1 KiB) is this wavefront's p-th load ---
     const int lrow = wave * 4 + lane / 16;   // key of this lane inside a group of 8 NK keys
@@ -151,11 +200,12 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
         const int key0 = c * kKeys + wk * 32 + 4 * half;
         return *reinterpret_cast<const v4f *>(mrow + min(key0 + 8 * a, g.len - 4));
     };
+    const int first_chunk = next_active(-1);
     v4f mk[4], mk_next[4];
 #pragma unroll
-    for (int a = 0; a < 4; ++a) mk[a] = load_mask(a, 0);
+    for (int a = 0; a < 4; ++a) mk[a] = load_mask(a, first_chunk);
 #pragma unroll
-    for (int p = 0; p < 8; ++p) issue_piece(p, 0, 0);
+    for (int p = 0; p < 8; ++p) issue_piece(p, first_chunk, 0);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier"
                  : "+v"(mk[0]), "+v"(mk[1]), "+v"(mk[2]), "+v"(mk[3])
                  :
@@ -166,9 +216,9 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     const int v_frag0 = (wk * 32 + 4 * half) * kHeadDim + (half * 32 + l32);        // d =      l32
     const int v_frag1 = (wk * 32 + 4 * half) * kHeadDim + ((half ^ 1) * 32 + l32);  // d = 32 + l32
 
-    auto step = [&](int c, auto more_tag) {
+    // chunk c from buffer buf; MORE: chunk `next` is fetched into the other buffer meanwhile
+    auto step = [&](int c, int next, int buf, auto more_tag) {
         constexpr bool MORE = decltype(more_tag)::value;
-        const int buf = c & 1;
         const int key0 = c * kKeys + wk * 32 + 4 * half;
 
         // S^T (32 keys x 32 queries) = K . Q^T over the 64 head dims
@@ -184,8 +234,8 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
             for (int s = 0; s < 4; ++s)
                 st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[s], qf[kc][s], st, 0, 0, 0);
             if constexpr (MORE) {
-                if constexpr (kc < 4) mk_next[kc] = load_mask(kc, c + 1);
-                issue_piece(kc, c + 1, buf ^ 1);
+                if constexpr (kc < 4) mk_next[kc] = load_mask(kc, next);
+                issue_piece(kc, next, buf ^ 1);
             }
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -257,8 +307,15 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }
     };
-    for (int c = 0; c + 1 < n_chunks; ++c) step(c, std::true_type{});
-    step(n_chunks - 1, std::false_type{});
+    {
+        int c = first_chunk, buf = 0;
+        for (int next = next_active(c); next >= 0; next = next_active(c)) {
+            step(c, next, buf, std::true_type{});
+            c = next;
+            buf ^= 1;
+        }
+        step(c, -1, buf, std::false_type{});
+    }
 
     // ---- merge the NK key parts of every query tile and write -------------------------------------
     {
@@ -317,6 +374,36 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
             }
         }
     }
+    if (!g.queue) break;
+    __syncthreads();   // the merge has read its slots, and thread 0 may write next_item again
+    }
+}
+
+// ---- which (64-query tile, key chunk) pairs of a mask hold anything but -inf -----------------------
+// Block (chunk, tile, batch x head of the mask) looks at 64 x KEYS mask values; a byte per pair.
+template <int KEYS>
+__global__ __launch_bounds__(256) void attention_mask_tiles_kernel(const float *__restrict__ mask, int64_t mask_b,
+                                                                   int64_t mask_h, int64_t mask_s, int32_t heads,
+                                                                   int32_t seq, int32_t len,
+                                                                   uint8_t *__restrict__ tiles,
+                                                                   int32_t *__restrict__ queue) {
+    const int chunk = blockIdx.x, tile = blockIdx.y, bh = blockIdx.z;
+    if (chunk == 0 && tile == 0 && bh == 0 && threadIdx.x == 0) *queue = 0;   // the item counter of the kernel that follows
+    const int b = bh / heads, h = bh - b * heads;
+    const float *base = mask + b * mask_b + h * mask_h;
+    constexpr int kVecPerRow = KEYS / 4;
+    bool seen = false;
+    for (int i = threadIdx.x; i < 64 * kVecPerRow; i += 256) {
+        const int row = tile * 64 + i / kVecPerRow, key = chunk * KEYS + (i % kVecPerRow) * 4;
+        if (row < seq && key < len) {   // len % 4 == 0: a vector is inside or outside
+            const v4f m = *reinterpret_cast<const v4f *>(base + row * mask_s + key);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) seen |= !(m[e] == -INFINITY);
+        }
+    }
+    const int any = __syncthreads_or(seen ? 1 : 0);
+    if (threadIdx.x == 0)
+        tiles[(static_cast<int64_t>(bh) * gridDim.y + tile) * gridDim.x + chunk] = any ? 1 : 0;
 }
 
 // ---- a handful of query rows (a decode step): keys split over blocks ------------------------------
@@ -539,12 +626,47 @@ int32_t attention_args(int32_t dtype, int64_t batch, int64_t kv_heads, int64_t r
 
 }  // namespace
 
-extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch,
-                                      int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
-                                      int64_t head_dim, const void *q, const void *k, const void *v,
-                                      const void *mask, const rmlk_dims *mask_stride,
-                                      int32_t scale_is_mul, float scale, int32_t out_seq_major,
-                                      void *out) {
+namespace {
+// The tile map of masked-chunk skipping: dims and bytes, or 0 bytes when skipping does not apply -
+// the blocks must outnumber the compute units (otherwise the block with the most visible chunks
+// decides and nothing is gained; it is also the case that runs 64-key chunks), a query tile must
+// lie inside one head, and the chunks must fit the kernel's two 64-bit sets.
+struct TileMapDims {
+    int64_t mask_batches, mask_heads, tiles, chunks;
+    size_t map_bytes, bytes;
+};
+TileMapDims tile_map_dims(int64_t batch, int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
+                          const rmlk_dims *mask_stride) {
+    TileMapDims d{};
+    if (batch <= 0 || kv_heads <= 0 || rep <= 0 || q_len <= 0 || kv_len <= 0 || !dims_ok(mask_stride) ||
+        mask_stride->rank != 4)
+        return d;
+    const int64_t blocks = (rep * q_len + 63) / 64 * batch * kv_heads;
+    d.chunks = (kv_len + 63) / 64;
+    if (blocks <= kNumCU || q_len % 64 != 0 || d.chunks < 4 || d.chunks > 128) return d;
+    d.mask_batches = mask_stride->v[0] ? batch : 1;
+    d.mask_heads = mask_stride->v[1] ? kv_heads * rep : 1;
+    d.tiles = q_len / 64;
+    if (d.mask_batches * d.mask_heads >= 65536 || d.tiles >= 65536) return d;
+    d.map_bytes = static_cast<size_t>(d.mask_batches * d.mask_heads * d.tiles * d.chunks + 15) / 16 * 16;
+    d.bytes = d.map_bytes + 16;   // the map, then the item counter
+    return d;
+}
+}  // namespace
+
+extern "C" size_t rmlk_hip_attention_workspace_size(int32_t dtype, int64_t batch, int64_t kv_heads,
+                                                    int64_t rep, int64_t q_len, int64_t kv_len,
+                                                    int64_t head_dim, const rmlk_dims *mask_stride) {
+    if (dtype != RMLK_FLOAT || head_dim != kHeadDim) return 0;
+    return tile_map_dims(batch, kv_heads, rep, q_len, kv_len, mask_stride).bytes;
+}
+
+extern "C" int32_t rmlk_hip_attention_ws(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                         int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
+                                         int64_t head_dim, const void *q, const void *k, const void *v,
+                                         const void *mask, const rmlk_dims *mask_stride,
+                                         int32_t scale_is_mul, float scale, int32_t out_seq_major,
+                                         void *workspace, size_t workspace_bytes, void *out) {
     AttnArgs g{};
     bool empty = false;
     const int32_t st = attention_args(dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
@@ -552,7 +674,25 @@ extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64
     if (st || empty) return st;
     dim3 grid(static_cast<unsigned>((g.rows + 63) / 64), static_cast<unsigned>(batch * kv_heads), 1);
     // two blocks of four wavefronts per CU when there are that many, else one block of eight
-    if (!RMLK_ATTN_WIDE_BLOCKS || static_cast<int64_t>(grid.x) * grid.y > kNumCU) {
+    if (static_cast<int64_t>(grid.x) * grid.y > kNumCU) {
+        const TileMapDims tm = tile_map_dims(batch, kv_heads, rep, q_len, kv_len, mask_stride);
+        if (workspace && tm.bytes && workspace_bytes >= tm.bytes) {
+            uint8_t *tiles = static_cast<uint8_t *>(workspace);
+            const dim3 tgrid(static_cast<unsigned>(tm.chunks), static_cast<unsigned>(tm.tiles),
+                             static_cast<unsigned>(tm.mask_batches * tm.mask_heads));
+            attention_mask_tiles_kernel<64><<<tgrid, 256, 0, as_stream(stream)>>>(
+                g.mask, g.mask_b, g.mask_h, g.mask_s, static_cast<int32_t>(tm.mask_heads), g.seq, g.len, tiles,
+                reinterpret_cast<int32_t *>(tiles + tm.map_bytes));
+            const int32_t launched = launch_status();
+            if (launched) return launched;
+            g.tiles = tiles;
+            g.tiles_h = mask_stride->v[1] ? tm.tiles * tm.chunks : 0;
+            g.tiles_b = mask_stride->v[0] ? tm.mask_heads * tm.tiles * tm.chunks : 0;
+            g.queue = reinterpret_cast<int32_t *>(tiles + tm.map_bytes);
+            g.items = static_cast<int32_t>(static_cast<int64_t>(grid.x) * grid.y);
+            g.tiles_per_head = static_cast<int32_t>(tm.tiles);
+            grid = dim3(static_cast<unsigned>(std::min<int64_t>(g.items, 2 * kNumCU)), 1, 1);
+        }
         static DynamicLdsGrant grant;
         const int32_t granted = grant.ensure(attention_rows_kernel<2>, AttnShape<2>::kLdsBytes);
         if (granted) return granted;
@@ -564,6 +704,16 @@ extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64
         attention_rows_kernel<4><<<grid, AttnShape<4>::kThreads, AttnShape<4>::kLdsBytes, as_stream(stream)>>>(g);
     }
     return launch_status();
+}
+
+extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                      int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
+                                      int64_t head_dim, const void *q, const void *k, const void *v,
+                                      const void *mask, const rmlk_dims *mask_stride,
+                                      int32_t scale_is_mul, float scale, int32_t out_seq_major,
+                                      void *out) {
+    return rmlk_hip_attention_ws(stream, dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
+                                 mask_stride, scale_is_mul, scale, out_seq_major, nullptr, 0, out);
 }
 
 extern "C" size_t rmlk_hip_attention_few_rows_workspace_size(int32_t dtype, int64_t batch, int64_t kv_heads,

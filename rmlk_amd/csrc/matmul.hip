@@ -523,15 +523,9 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     // them and issue the loads of the next stage; the last chunk meets the block a quarter of the
     // way in and then reads chunk 0 of the next stage.
     constexpr int NM = 4 * TM * TN;                  // MFMAs per chunk
-#ifndef RMLK_GEMM_LOAD_CHUNKS
-#define RMLK_GEMM_LOAD_CHUNKS 1
-#endif
-#ifndef RMLK_GEMM_BARRIER_AT
-#define RMLK_GEMM_BARRIER_AT 2
-#endif
-    constexpr int kLoadChunks = RMLK_GEMM_LOAD_CHUNKS;   // chunks (from the first) that carry the loads
+    constexpr int kLoadChunks = 1;   // chunks (from the first) that carry the loads
     constexpr int kLoadsPerChunk = (kLoadsPerStage + kLoadChunks - 1) / kLoadChunks;
-    constexpr int kBarrierAt = NM * RMLK_GEMM_BARRIER_AT / 4 < NM - 1 ? NM * RMLK_GEMM_BARRIER_AT / 4 : NM - 2;
+    constexpr int kBarrierAt = NM * 2 / 4 < NM - 1 ? NM * 2 / 4 : NM - 2;
     auto k_step = [&](int buf, auto load_tag, auto more_tag) {
         constexpr bool LOAD = decltype(load_tag)::value;   // another stage to fetch
         constexpr bool MORE = decltype(more_tag)::value;   // another step follows
@@ -695,9 +689,7 @@ __global__ __launch_bounds__(kThreads) void splitk_reduce_vec_kernel(const float
 // ---- GEMV: y[n] = sum_k x[k] * W[k][n], W row-major -------------------------------------------
 // A block covers kThreads / 64 * ... columns: VEC columns per lane, 64 lanes per wavefront, and
 // the block's 4 wavefronts split the block's K slice; partial sums meet in LDS.
-#ifndef RMLK_GEMV_DEPTH
-#define RMLK_GEMV_DEPTH 16
-#endif
+constexpr int kGemvRowMajorDepth = 16;
 
 struct GemvArgs {
     const float *x;   // [batch][k], element stride x_inc
@@ -756,8 +748,8 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(GemvArgs g) {
                 wp += static_cast<int64_t>(U) * g.ldb;
                 kk += U;
             };
-            while (kk + RMLK_GEMV_DEPTH <= ke) rows(std::integral_constant<int, RMLK_GEMV_DEPTH>{});
-            if (RMLK_GEMV_DEPTH > 8 && kk + 8 <= ke) rows(std::integral_constant<int, 8>{});
+            while (kk + kGemvRowMajorDepth <= ke) rows(std::integral_constant<int, kGemvRowMajorDepth>{});
+            if (kGemvRowMajorDepth > 8 && kk + 8 <= ke) rows(std::integral_constant<int, 8>{});
             if (kk + 4 <= ke) rows(std::integral_constant<int, 4>{});
             for (; kk < ke; ++kk) {
                 v4f wv = *reinterpret_cast<const v4f *>(wp);
@@ -1316,13 +1308,7 @@ struct TileChoice {
     int k_per_split;
 };
 
-#ifndef RMLK_GEMM_SPLIT_TARGET
-#define RMLK_GEMM_SPLIT_TARGET 1
-#endif
-// 0: split-K products keep 128 x 128 tiles (to compare)
-#ifndef RMLK_GEMM_NARROW_SPLIT
-#define RMLK_GEMM_NARROW_SPLIT 1
-#endif
+constexpr int kGemmSplitTarget = 1;   // blocks per CU a split-K product aims for
 
 // allow_wide: the 128 x 192 and 128 x 64 tiles may be chosen (they exist for the direct-to-LDS kernel
 // only; a caller whose operands do not qualify asks again without it).
@@ -1351,7 +1337,7 @@ inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k, b
         const int64_t nt = tiles(bm, bn);
         int splits = 1;
         if (nt < kNumCU) {
-            splits = static_cast<int>((RMLK_GEMM_SPLIT_TARGET * kNumCU + nt - 1) / nt);
+            splits = static_cast<int>((kGemmSplitTarget * kNumCU + nt - 1) / nt);
             int64_t max_splits = k / (8 * t.bk);
             if (max_splits < 1) max_splits = 1;
             if (splits > max_splits) splits = static_cast<int>(max_splits);
@@ -1386,13 +1372,11 @@ inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k, b
             t.k_per_split = kps_w;
         }
     }
-#if RMLK_GEMM_NARROW_SPLIT
     // split-K products whose 128 x 128 tiles give one block per CU: 128 x 64 tiles with the same
     // split put two or three blocks on a CU, which overlap each other's first stage and epilogue
     if (allow_wide && t.bm == 128 && t.bn == 128 && t.bk == 32 && t.splits > 1 && n % 64 == 0 &&
         tiles(128, 128) * t.splits <= kNumCU)
         t.bn = 64;
-#endif
     return t;
 }
 
@@ -1406,15 +1390,11 @@ inline int max_tile_splits(int64_t batch, int64_t m, int64_t n, int64_t k) {
 inline int gemv_splits(int64_t batch, int64_t n, int64_t k, int cols_per_block, int *k_per_split) {
     int64_t blocks = (n + cols_per_block - 1) / cols_per_block * batch;
     int64_t splits = 1;
-#ifndef RMLK_GEMV_BLOCKS_PER_CU
-#define RMLK_GEMV_BLOCKS_PER_CU 6
-#endif
-    if (blocks < RMLK_GEMV_BLOCKS_PER_CU * kNumCU)
-        splits = (RMLK_GEMV_BLOCKS_PER_CU * kNumCU + blocks - 1) / blocks;
-#ifndef RMLK_GEMV_MIN_ROWS
-#define RMLK_GEMV_MIN_ROWS 64
-#endif
-    int64_t max_splits = k / RMLK_GEMV_MIN_ROWS;
+    constexpr int kGemvBlocksPerCu = 6;   // blocks per CU that keep enough loads in flight
+    constexpr int kGemvMinRows = 64;      // rows of K a split keeps at least
+    if (blocks < kGemvBlocksPerCu * kNumCU)
+        splits = (kGemvBlocksPerCu * kNumCU + blocks - 1) / blocks;
+    int64_t max_splits = k / kGemvMinRows;
     if (max_splits < 1) max_splits = 1;
     if (splits > max_splits) splits = max_splits;
     if (splits > 64) splits = 64;
@@ -1454,10 +1434,6 @@ int32_t launch_direct(hipStream_t s, const GemmArgs &g, int64_t batch, int split
     return launch_status();
 }
 
-#ifndef RMLK_GEMM_DIRECT
-#define RMLK_GEMM_DIRECT 1
-#endif
-
 // The tiled MFMA path of a product (m > 1, A not transposed). `seg`: column blocks of C with their
 // own destinations (see Segments; their rows must be 16-byte aligned) instead of c/ldc; the call
 // then answers RMLK_ERR_UNSUPPORTED unless the whole-tile kernel applies.
@@ -1471,7 +1447,7 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
     // the direct-to-LDS kernel: whole K steps and aligned rows; partial tiles in m and n are fine
     // (for row-major B as long as n is a multiple of 4); per-lane byte offsets are 32-bit
     auto direct_ok = [&](const TileChoice &c) {
-        return RMLK_GEMM_DIRECT && c.bk == 32 && aligned && c.k_per_split % c.bk == 0 &&
+        return c.bk == 32 && aligned && c.k_per_split % c.bk == 0 &&
                k % c.k_per_split == 0 && (trans_b || n % 4 == 0) && lda < (1ll << 21) && ldb < (1ll << 21);
     };
     TileChoice t = choose_tiles(batch, m, n, k);
@@ -1531,10 +1507,7 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
     (whole ? RMLK_DIRECT_E(BM_, BN_, WM_, WN_, S_, false) : RMLK_DIRECT_E(BM_, BN_, WM_, WN_, S_, true))
     // two LDS stages: a third (loads two K steps ahead) measured no faster and halves the blocks
     // that fit a CU
-#ifndef RMLK_GEMM_STAGES
-#define RMLK_GEMM_STAGES 2
-#endif
-#define RMLK_DIRECT(BM_, BN_, WM_, WN_) RMLK_DIRECT_S(BM_, BN_, WM_, WN_, RMLK_GEMM_STAGES)
+#define RMLK_DIRECT(BM_, BN_, WM_, WN_) RMLK_DIRECT_S(BM_, BN_, WM_, WN_, 2)
     const bool whole = m % t.bm == 0 && n % t.bn == 0;
     const bool direct = direct_ok(t);
     if (seg) {

@@ -943,14 +943,10 @@ bool took_fast_path(int32_t st, const char *what) {
 // row while it loads it (rmlk_hip_gemv_kmajor_normed). One launch less per norm of a decode step.
 constexpr int64_t kMaxDeferredNormCols = 8192;   // what the product kernels accept
 constexpr int64_t kMaxDeferredNormWidth = 16384; // output columns up to which a product applies the norm
-// 0: every norm runs as its own launch (to compare)
-#ifndef RMLK_DEFER_NORM
-#define RMLK_DEFER_NORM 1
-#endif
 
 bool may_defer_norm(const OpContext &c, const Tensor &row, const Tensor &gamma) {
     const int64_t cols = row.shape.empty() ? 0 : row.shape.back();
-    return RMLK_DEFER_NORM && c.attr_int("defer_norm", 0) != 0 && row.dtype == RMLK_FLOAT && gamma.dtype == RMLK_FLOAT &&
+    return c.attr_int("defer_norm", 0) != 0 && row.dtype == RMLK_FLOAT && gamma.dtype == RMLK_FLOAT &&
            cols > 0 && row.numel() == cols && cols % 4 == 0 && cols <= kMaxDeferredNormCols &&
            gamma.numel() == cols;
 }
@@ -1399,10 +1395,14 @@ void op_fused_attention(OpContext &c) {
             const bool seq_major = c.attr_int("seq_major_output", 0) != 0;
             Tensor &y = seq_major ? c.alloc_output(0, RMLK_FLOAT, {bsz, seq, heads, dim})
                                   : c.alloc_output(0, RMLK_FLOAT, {bsz, heads, seq, dim});
-            if (took_fast_path(rmlk_hip_attention(c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim,
-                                                  q.data(), k.data(), v.data(), mask.data(), &ms,
-                                                  static_cast<int32_t>(c.attr_int("scale_is_mul", 0)),
-                                                  attr_float(c, "scale"), seq_major ? 1 : 0, y.data()),
+            // room for the map of (query tile, key chunk) pairs the mask leaves visible, when it pays
+            const size_t map_bytes = rmlk_hip_attention_workspace_size(RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, &ms);
+            void *map = map_bytes ? c.scratch(map_bytes) : nullptr;
+            if (took_fast_path(rmlk_hip_attention_ws(c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim,
+                                                     q.data(), k.data(), v.data(), mask.data(), &ms,
+                                                     static_cast<int32_t>(c.attr_int("scale_is_mul", 0)),
+                                                     attr_float(c, "scale"), seq_major ? 1 : 0, map, map_bytes,
+                                                     y.data()),
                                "rmlk.Attention"))
                 return;
         }
@@ -1667,7 +1667,7 @@ void op_fused_matmul_group(OpContext &c) {
                 off += widths[i];
             }
         };
-        if (RMLK_DEFER_NORM && c.attr_int("defer_product", 0) != 0 && c.has_input(2) && k % 4 == 0 && k > 0) {
+        if (c.attr_int("defer_product", 0) != 0 && c.has_input(2) && k % 4 == 0 && k > 0) {
             // left to the row-stream node behind it (op_fused_head_rows)
             auto pp = std::make_shared<PendingProduct>();
             pp->x = a;

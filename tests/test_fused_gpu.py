@@ -1020,6 +1020,101 @@ def test_attention_matches_separate_kernels(device, b, g, rep, s, l, mask_shape,
     assert_exact(to_np(moved), to_np(got).transpose(0, 2, 1, 3))
 
 
+def _skipping_mask(kind, rng, mask_shape, l):
+    """Masks with whole (64-query, 64-key) tiles hidden, in the shapes that occur: causal with a past,
+    a sliding window (hidden tiles on both sides), random hidden tiles per batch and head (one query
+    tile sees nothing at all), one mask row shared by every query."""
+    mb, mh, ms_, _ = mask_shape
+    m = (rng.standard_normal(mask_shape, dtype=np.float32) * 0.5).astype(np.float32)
+    rows = np.arange(ms_)[:, None] + (l - ms_ if ms_ > 1 else 0)
+    keys = np.arange(l)[None, :]
+    if kind == "causal":
+        hidden = np.broadcast_to(keys > rows, mask_shape)
+    elif kind == "window":
+        hidden = np.broadcast_to((keys > rows) | (keys < rows - 300), mask_shape)
+    elif kind == "tiles":
+        t = rng.random((mb, mh, (ms_ + 63) // 64, (l + 63) // 64)) < 0.6
+        t[0, 0, 0, 0] = False
+        t[0, 0, 1, :] = True          # a tile of queries that sees nothing: NaN rows
+        t[-1, -1, 2, :] = True
+        t[-1, -1, 2, 5] = False       # and one that sees a single chunk
+        hidden = np.repeat(np.repeat(t, 64, axis=2), 64, axis=3)[:, :, :ms_, :l]
+        # single visible keys inside otherwise hidden tiles keep those chunks on the list
+        hidden = hidden.copy()
+        hidden[0, 0, 200, 777 % l] = False
+    else:                              # "row": chunks 2.. and 9 hidden for everyone
+        hidden = np.zeros(mask_shape, dtype=bool)
+        hidden[..., 128:448] = True
+        hidden[..., 576:640] = True
+    return np.where(hidden, np.float32(-np.inf), m).astype(np.float32)
+
+
+@pytest.mark.parametrize("b,g,rep,s,l,mask_shape,kind,skips", [
+    (1, 8, 4, 2048, 2048, (1, 1, 2048, 2048), "causal", True),    # the 2048-token prefill
+    (1, 8, 4, 2048, 2064, (1, 1, 2048, 2064), "causal", True),    # with a past; keys end inside a chunk
+    (1, 8, 4, 1024, 1024, (1, 1, 1024, 1024), "window", True),
+    (2, 4, 3, 1024, 1024, (2, 12, 1024, 1024), "tiles", True),    # per batch and head
+    (1, 8, 4, 1024, 1024, (1, 32, 1024, 1024), "tiles", True),    # per head only
+    (2, 8, 4, 512, 1024, (2, 1, 512, 1024), "tiles", True),       # per batch only
+    (1, 8, 4, 2048, 704, (1, 1, 1, 704), "row", True),            # one mask row for every query
+    (1, 8, 4, 512, 640, (1, 1, 512, 640), "causal", False),       # too few blocks: the 8-wavefront kernel
+    (1, 8, 4, 2000, 2048, (1, 1, 2000, 2048), "causal", False),   # tiles would straddle heads
+    (1, 8, 4, 2048, 128, (1, 1, 2048, 128), "causal", False),     # two chunks: nothing to gain
+])
+def test_attention_skipping_hidden_chunks_is_bit_identical(device, b, g, rep, s, l, mask_shape, kind, skips):
+    """Chunks of keys that a tile of 64 queries cannot see (-inf for all of them) have probabilities
+    that are exact zeros, so leaving them out changes no bit; rows that see nothing are NaN either way."""
+    import torch
+    kk = _k()
+    h, d = g * rep, 64
+    rng = np.random.default_rng(s * 7 + l + b)
+    q, k, v = (to_dev(rng.standard_normal(sh, dtype=np.float32), device)
+               for sh in ((b, h, s, d), (b, g, l, d), (b, g, l, d)))
+    m_np = _skipping_mask(kind, rng, mask_shape, l)
+    m = to_dev(m_np, device)
+    ms = bcast_strides(list(mask_shape), [b, h, s, l])
+    for seq_major in (False, True):
+        shape = (b, s, h, d) if seq_major else (b, h, s, d)
+        plain = torch.full(shape, 7.0, device=device)
+        kk.attention(q, k, v, m, plain, b, g, rep, s, l, d, ms, 8.0, False, out_seq_major=seq_major)
+        got = torch.full(shape, 9.0, device=device)
+        need = kk.attention_skipping(q, k, v, m, got, b, g, rep, s, l, d, ms, 8.0, False, out_seq_major=seq_major)
+        assert (need > 0) == skips
+        if skips:
+            mb, mh = mask_shape[0], mask_shape[1]
+            assert need == (mb * mh * (s // 64) * ((l + 63) // 64) + 15) // 16 * 16 + 16   # the map and a counter
+        a, e = to_np(got), to_np(plain)
+        assert np.array_equal(np.isnan(a), np.isnan(e))
+        assert_exact(np.nan_to_num(a, nan=0.0), np.nan_to_num(e, nan=0.0))
+    if kind == "tiles":
+        out = to_np(plain)   # [B, S, H, D] from the last pass
+        assert np.isnan(out[0, 64:128, 0]).all() and np.isfinite(out[0, :64, 0]).all()
+
+
+def test_attention_skipped_chunks_do_not_read_their_keys(device):
+    """What the skipped chunks hold never reaches the output: NaN in K and V rows no query of a tile
+    sees leaves that tile finite (the kernel without the map gives 0 * NaN there)."""
+    import torch
+    kk = _k()
+    b, g, rep, s, l, d = 1, 8, 4, 1024, 1024, 64
+    rng = np.random.default_rng(11)
+    q_np, k_np, v_np = (rng.standard_normal(sh, dtype=np.float32) for sh in ((b, g * rep, s, d), (b, g, l, d), (b, g, l, d)))
+    m_np = _skipping_mask("causal", rng, (1, 1, s, l), l)
+    k_bad, v_bad = k_np.copy(), v_np.copy()
+    k_bad[:, :, 512:] = np.nan
+    v_bad[:, :, 512:] = np.nan
+    m = to_dev(m_np, device)
+    got = torch.empty(b, g * rep, s, d, device=device)
+    need = kk.attention_skipping(to_dev(q_np, device), to_dev(k_bad, device), to_dev(v_bad, device), m, got,
+                                 b, g, rep, s, l, d, [0, 0, l, 1], 8.0)
+    assert need > 0
+    exp = torch.empty_like(got)
+    kk.attention(to_dev(q_np, device), to_dev(k_np, device), to_dev(v_np, device), m, exp, b, g, rep, s, l, d,
+                 [0, 0, l, 1], 8.0)
+    assert_exact(to_np(got)[:, :, :512], to_np(exp)[:, :, :512])
+    assert np.isnan(to_np(got)[:, :, 512:]).all()
+
+
 def test_attention_row_with_nothing_visible_is_nan_like_softmax(device):
     import torch
     kk = _k()
