@@ -343,7 +343,8 @@ int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch, i
  * or infinity in a K or V row no query of the tile can see does not reach that tile's output
  * (0 * NaN would), and a row with nothing visible anywhere is NaN as before. The size is 0 (and a
  * null workspace allowed) where skipping does not apply: few blocks, q_len not a multiple of 64, or
- * more than 128 chunks. rmlk_hip_attention is this call with a null workspace. */
+ * more than 128 chunks. The workspace is 16-byte aligned and belongs to the call until its kernels
+ * have run. rmlk_hip_attention is this call with a null workspace. */
 size_t rmlk_hip_attention_workspace_size(int32_t dtype, int64_t batch, int64_t kv_heads, int64_t rep,
                                          int64_t q_len, int64_t kv_len, int64_t head_dim,
                                          const rmlk_dims *mask_stride);
@@ -366,6 +367,19 @@ int32_t rmlk_hip_attention_few_rows(rmlk_stream_t stream, int32_t dtype, int64_t
                                     const void *mask, const rmlk_dims *mask_stride,
                                     int32_t scale_is_mul, float scale, int32_t out_seq_major,
                                     void *workspace, size_t workspace_bytes, void *out);
+/* The same in ONE launch: the block that finishes a KV head's last chunk merges that head's partial
+ * results itself. `counters` holds batch * kv_heads 32-bit counters in device memory that are zero
+ * before the first call; the kernel counts finished blocks there and leaves every counter zero again,
+ * so one zeroed buffer serves all later calls on the same stream (calls that overlap on the GPU need
+ * buffers of their own, like the workspace). Results are those of rmlk_hip_attention_few_rows bit for
+ * bit. */
+int32_t rmlk_hip_attention_few_rows_one_launch(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                               int64_t kv_heads, int64_t rep, int64_t q_len,
+                                               int64_t kv_len, int64_t head_dim, const void *q,
+                                               const void *k, const void *v, const void *mask,
+                                               const rmlk_dims *mask_stride, int32_t scale_is_mul,
+                                               float scale, int32_t out_seq_major, void *workspace,
+                                               size_t workspace_bytes, int32_t *counters, void *out);
 
 /* ---- products that share their first operand (q/k/v, gate/up) ----------------------------------
  * The weights of such MatMuls (ref: one cublasGemmStridedBatchedEx each,

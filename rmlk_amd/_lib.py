@@ -141,6 +141,10 @@ SIGNATURES = {
                                               c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
                                               _PD, c_int32, ctypes.c_float, c_int32, c_void_p, c_size_t,
                                               c_void_p]),
+    "rmlk_hip_attention_few_rows_one_launch": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64,
+                                                         c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                                         c_void_p, c_void_p, _PD, c_int32, ctypes.c_float,
+                                                         c_int32, c_void_p, c_size_t, c_void_p, c_void_p]),
     "rmlk_hip_matmul_grouped_workspace_size": (c_size_t, [c_int32, c_int64, c_int64, c_int32,
                                                           POINTER(c_int64)]),
     "rmlk_hip_matmul_grouped": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int64,

@@ -414,8 +414,24 @@ __global__ __launch_bounds__(256) void attention_mask_tiles_kernel(const float *
 constexpr int kFewRowsMax = 16;
 constexpr int kPartial = kHeadDim + 2;   // floats per (row, chunk): output, maximum, sum
 
+template <bool FRESH>
+__device__ __forceinline__ void merge_row(const AttnArgs &g, const float *__restrict__ ws, int n_chunks, int bg,
+                                          int r, int lane);
+template <bool FRESH>
+__device__ __forceinline__ void merge_row_many(const AttnArgs &g, const float *__restrict__ ws, int n_chunks,
+                                               int bg, int r, int lane);
+
+// MERGE: the block that finishes last for a KV head (a counter per KV head tells, zero before the
+// launch and zero again after it) merges the partial results of all chunks itself; otherwise a
+// second kernel does. Blocks of one launch run on different XCDs, whose L2s do not see each other's
+// lines; a device-wide fence on both sides would write back and invalidate whole L2s (measured: some
+// 6 us per launch, more than the merge launch costs). Instead the partial results alone bypass the
+// cache: device-scope stores that go through to memory, awaited before the block counts itself,
+// and device-scope loads in the merging block.
+template <bool MERGE>
 __global__ __launch_bounds__(kAttnThreads) void attention_few_rows_kernel(AttnArgs g, float *__restrict__ ws,
-                                                                          float scale, int32_t scale_is_mul) {
+                                                                          float scale, int32_t scale_is_mul,
+                                                                          int32_t *__restrict__ counters) {
     __shared__ float Ks[kChunk][kHeadDim + 1];   // +1: lanes read different rows of one column
     __shared__ __align__(16) float Vs[kChunk][kHeadDim];
     __shared__ __align__(16) float qs[kFewRowsMax][kHeadDim];
@@ -472,10 +488,33 @@ __global__ __launch_bounds__(kAttnThreads) void attention_few_rows_kernel(AttnAr
 #pragma unroll 16
         for (int j = 0; j < kChunk; ++j) acc = fmaf(ps[r][j], Vs[j][lane], acc);
         float *dst = ws + ((static_cast<int64_t>(bg) * n_chunks + chunk) * rows + r) * kPartial;
-        dst[lane] = acc;
-        if (lane == 0) {
-            dst[kHeadDim] = mx;
-            dst[kHeadDim + 1] = sum;
+        if constexpr (MERGE) {
+            __hip_atomic_store(dst + lane, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) {
+                __hip_atomic_store(dst + kHeadDim, mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(dst + kHeadDim + 1, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        } else {
+            dst[lane] = acc;
+            if (lane == 0) {
+                dst[kHeadDim] = mx;
+                dst[kHeadDim + 1] = sum;
+            }
+        }
+    }
+    if constexpr (MERGE) {
+        __shared__ int is_last;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's stores have reached memory ...
+        __syncthreads();                                    // ... and so have the block's, before it counts itself done
+        if (tid == 0)
+            is_last = __hip_atomic_fetch_add(counters + bg, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                      n_chunks - 1;
+        __syncthreads();
+        if (!is_last) return;
+        if (tid == 0) counters[bg] = 0;   // for the next launch
+        for (int r = wave; r < rows; r += kAttnThreads / kWave) {
+            if (n_chunks <= kWave) merge_row<true>(g, ws, n_chunks, bg, r, lane);
+            else merge_row_many<true>(g, ws, n_chunks, bg, r, lane);
         }
     }
 }
@@ -488,22 +527,29 @@ __global__ __launch_bounds__(kAttnThreads) void attention_few_rows_kernel(AttnAr
 constexpr int kMergeGroup = 16;
 constexpr int kMergeMaxChunks = kWave;
 
-__global__ __launch_bounds__(kAttnThreads) void attention_merge_kernel(AttnArgs g, const float *__restrict__ ws,
-                                                                       int32_t n_chunks, int32_t total_rows) {
-    const int lane = threadIdx.x % kWave;
-    const int item = blockIdx.x * (kAttnThreads / kWave) + threadIdx.x / kWave;
-    if (item >= total_rows) return;
+// FRESH: the partial results were written by other blocks of the SAME launch, possibly through
+// another XCD's L2: they are read with device-scope loads, which that cache does not answer from
+// what it holds (the writers stored them the same way, see the few-rows kernel).
+template <bool FRESH>
+__device__ __forceinline__ float partial_load(const float *p) {
+    if constexpr (FRESH) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else return *p;
+}
+
+// (kv head bg, row r) by one wavefront, n_chunks <= 64
+template <bool FRESH>
+__device__ __forceinline__ void merge_row(const AttnArgs &g, const float *__restrict__ ws, int n_chunks, int bg,
+                                          int r, int lane) {
     const int rows = g.rows;
-    const int bg = item / rows, r = item - bg * rows;
     const int b = bg / g.kv_heads, grp = bg - b * g.kv_heads;
     const float *src = ws + (static_cast<int64_t>(bg) * n_chunks * rows + r) * kPartial;
     const int64_t step = static_cast<int64_t>(rows) * kPartial;
     const int mine = min(lane, n_chunks - 1);
-    const float m_c = src[mine * step + kHeadDim];
-    const float s_c = src[mine * step + kHeadDim + 1];
+    const float m_c = partial_load<FRESH>(src + mine * step + kHeadDim);
+    const float s_c = partial_load<FRESH>(src + mine * step + kHeadDim + 1);
     float part[kMergeGroup];
 #pragma unroll
-    for (int j = 0; j < kMergeGroup; ++j) part[j] = src[min(j, n_chunks - 1) * step + lane];
+    for (int j = 0; j < kMergeGroup; ++j) part[j] = partial_load<FRESH>(src + min(j, n_chunks - 1) * step + lane);
     const float m = wave_max(lane < n_chunks ? m_c : -INFINITY);
     const float m_safe = m == -INFINITY ? 0.f : m;
     const float w = lane < n_chunks ? expf(m_c - m_safe) : 0.f;
@@ -512,7 +558,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_merge_kernel(AttnArgs 
     for (int c0 = 0; c0 < n_chunks; c0 += kMergeGroup) {
         if (c0 > 0) {
 #pragma unroll
-            for (int j = 0; j < kMergeGroup; ++j) part[j] = src[min(c0 + j, n_chunks - 1) * step + lane];
+            for (int j = 0; j < kMergeGroup; ++j) part[j] = partial_load<FRESH>(src + min(c0 + j, n_chunks - 1) * step + lane);
         }
 #pragma unroll
         for (int j = 0; j < kMergeGroup; ++j) {
@@ -527,33 +573,44 @@ __global__ __launch_bounds__(kAttnThreads) void attention_merge_kernel(AttnArgs 
 
 // The same for more chunks than a wavefront has lanes: maxima and sums a chunk per lane in rounds,
 // then the outputs chunk by chunk.
-__global__ __launch_bounds__(kAttnThreads) void attention_merge_many_kernel(AttnArgs g, const float *__restrict__ ws,
-                                                                            int32_t n_chunks, int32_t total_rows) {
-    const int lane = threadIdx.x % kWave;
-    const int item = blockIdx.x * (kAttnThreads / kWave) + threadIdx.x / kWave;
-    if (item >= total_rows) return;
+template <bool FRESH>
+__device__ __forceinline__ void merge_row_many(const AttnArgs &g, const float *__restrict__ ws, int n_chunks,
+                                               int bg, int r, int lane) {
     const int rows = g.rows;
-    const int bg = item / rows, r = item - bg * rows;
     const int b = bg / g.kv_heads, grp = bg - b * g.kv_heads;
     const float *src = ws + (static_cast<int64_t>(bg) * n_chunks * rows + r) * kPartial;
     const int64_t step = static_cast<int64_t>(rows) * kPartial;
     float m = -INFINITY;
     for (int c0 = 0; c0 < n_chunks; c0 += kWave)
-        if (c0 + lane < n_chunks) m = fmaxf(m, src[(c0 + lane) * step + kHeadDim]);
+        if (c0 + lane < n_chunks) m = fmaxf(m, partial_load<FRESH>(src + (c0 + lane) * step + kHeadDim));
     m = wave_max(m);
     const float m_safe = m == -INFINITY ? 0.f : m;
     float acc = 0.f, sum = 0.f;
     for (int c0 = 0; c0 < n_chunks; c0 += kWave) {
         const int c = c0 + lane;
-        const float w = c < n_chunks ? expf(src[c * step + kHeadDim] - m_safe) : 0.f;
-        if (c < n_chunks) sum = fmaf(src[c * step + kHeadDim + 1], w, sum);
+        const float w = c < n_chunks ? expf(partial_load<FRESH>(src + c * step + kHeadDim) - m_safe) : 0.f;
+        if (c < n_chunks) sum = fmaf(partial_load<FRESH>(src + c * step + kHeadDim + 1), w, sum);
         const int here = min(kWave, n_chunks - c0);
 #pragma unroll 8
-        for (int j = 0; j < here; ++j) acc = fmaf(src[(c0 + j) * step + lane], __shfl(w, j, kWave), acc);
+        for (int j = 0; j < here; ++j) acc = fmaf(partial_load<FRESH>(src + (c0 + j) * step + lane), __shfl(w, j, kWave), acc);
     }
     sum = wave_sum(sum);
     const int head = grp * g.rep + r / g.seq, srow = r - (r / g.seq) * g.seq;
     g.out[b * g.out_b + head * g.out_h + srow * g.out_s + lane] = acc / sum;   // nothing visible: 0 / 0
+}
+
+__global__ __launch_bounds__(kAttnThreads) void attention_merge_kernel(AttnArgs g, const float *__restrict__ ws,
+                                                                       int32_t n_chunks, int32_t total_rows) {
+    const int item = blockIdx.x * (kAttnThreads / kWave) + threadIdx.x / kWave;
+    if (item >= total_rows) return;
+    merge_row<false>(g, ws, n_chunks, item / g.rows, item % g.rows, threadIdx.x % kWave);
+}
+
+__global__ __launch_bounds__(kAttnThreads) void attention_merge_many_kernel(AttnArgs g, const float *__restrict__ ws,
+                                                                            int32_t n_chunks, int32_t total_rows) {
+    const int item = blockIdx.x * (kAttnThreads / kWave) + threadIdx.x / kWave;
+    if (item >= total_rows) return;
+    merge_row_many<false>(g, ws, n_chunks, item / g.rows, item % g.rows, threadIdx.x % kWave);
 }
 
 }  // namespace
@@ -726,13 +783,12 @@ extern "C" size_t rmlk_hip_attention_few_rows_workspace_size(int32_t dtype, int6
     return static_cast<size_t>(batch * kv_heads * chunks * rep * q_len * kPartial) * sizeof(float);
 }
 
-extern "C" int32_t rmlk_hip_attention_few_rows(rmlk_stream_t stream, int32_t dtype, int64_t batch,
-                                               int64_t kv_heads, int64_t rep, int64_t q_len,
-                                               int64_t kv_len, int64_t head_dim, const void *q,
-                                               const void *k, const void *v, const void *mask,
-                                               const rmlk_dims *mask_stride, int32_t scale_is_mul,
-                                               float scale, int32_t out_seq_major, void *workspace,
-                                               size_t workspace_bytes, void *out) {
+namespace {
+int32_t attention_few_rows_launch(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t kv_heads,
+                                  int64_t rep, int64_t q_len, int64_t kv_len, int64_t head_dim, const void *q,
+                                  const void *k, const void *v, const void *mask, const rmlk_dims *mask_stride,
+                                  int32_t scale_is_mul, float scale, int32_t out_seq_major, void *workspace,
+                                  size_t workspace_bytes, int32_t *counters, void *out) {
     AttnArgs g{};
     bool empty = false;
     const int32_t st = attention_args(dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
@@ -747,7 +803,11 @@ extern "C" int32_t rmlk_hip_attention_few_rows(rmlk_stream_t stream, int32_t dty
     hipStream_t s = as_stream(stream);
     float *ws = static_cast<float *>(workspace);
     dim3 grid(static_cast<unsigned>(chunks), static_cast<unsigned>(batch * kv_heads), 1);
-    attention_few_rows_kernel<<<grid, kAttnThreads, 0, s>>>(g, ws, scale, scale_is_mul);
+    if (counters) {
+        attention_few_rows_kernel<true><<<grid, kAttnThreads, 0, s>>>(g, ws, scale, scale_is_mul, counters);
+        return launch_status();
+    }
+    attention_few_rows_kernel<false><<<grid, kAttnThreads, 0, s>>>(g, ws, scale, scale_is_mul, nullptr);
     int32_t launched = launch_status();
     if (launched) return launched;
     const int64_t total_rows = batch * kv_heads * g.rows;
@@ -760,4 +820,30 @@ extern "C" int32_t rmlk_hip_attention_few_rows(rmlk_stream_t stream, int32_t dty
         attention_merge_many_kernel<<<merge_grid, kAttnThreads, 0, s>>>(g, ws, static_cast<int32_t>(chunks),
                                                                         static_cast<int32_t>(total_rows));
     return launch_status();
+}
+}  // namespace
+
+extern "C" int32_t rmlk_hip_attention_few_rows(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                               int64_t kv_heads, int64_t rep, int64_t q_len,
+                                               int64_t kv_len, int64_t head_dim, const void *q,
+                                               const void *k, const void *v, const void *mask,
+                                               const rmlk_dims *mask_stride, int32_t scale_is_mul,
+                                               float scale, int32_t out_seq_major, void *workspace,
+                                               size_t workspace_bytes, void *out) {
+    return attention_few_rows_launch(stream, dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
+                                     mask_stride, scale_is_mul, scale, out_seq_major, workspace, workspace_bytes,
+                                     nullptr, out);
+}
+
+extern "C" int32_t rmlk_hip_attention_few_rows_one_launch(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                                          int64_t kv_heads, int64_t rep, int64_t q_len,
+                                                          int64_t kv_len, int64_t head_dim, const void *q,
+                                                          const void *k, const void *v, const void *mask,
+                                                          const rmlk_dims *mask_stride, int32_t scale_is_mul,
+                                                          float scale, int32_t out_seq_major, void *workspace,
+                                                          size_t workspace_bytes, int32_t *counters, void *out) {
+    if (!counters) return RMLK_ERR_NULL_POINTER;
+    return attention_few_rows_launch(stream, dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
+                                     mask_stride, scale_is_mul, scale, out_seq_major, workspace, workspace_bytes,
+                                     counters, out);
 }

@@ -262,6 +262,10 @@ struct Session {
     void *workspace = nullptr;       // persistent MatMul workspace (raw allocation)
     size_t workspace_bytes = 0;
     int32_t *err_flag = nullptr;     // device
+    // Block counters of kernels whose last block finishes the job (the decode-step attention):
+    // zero when the session is built, and left zero by every kernel that uses them.
+    static constexpr int64_t kBlockCounters = 1024;
+    int32_t *block_counters = nullptr;
     int32_t *err_host = nullptr;     // pinned host
     bool capturing = false;
     bool profiling = false;

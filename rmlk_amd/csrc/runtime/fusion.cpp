@@ -1382,13 +1382,19 @@ void op_fused_attention(OpContext &c) {
             void *ws = c.scratch(few_bytes);
             Tensor &y = seq_major ? c.alloc_output(0, RMLK_FLOAT, {bsz, seq, heads, dim})
                                   : c.alloc_output(0, RMLK_FLOAT, {bsz, heads, seq, dim});
-            if (took_fast_path(rmlk_hip_attention_few_rows(
-                                   c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, q.data(), k.data(),
-                                   v.data(), mask.data(), &ms,
-                                   static_cast<int32_t>(c.attr_int("scale_is_mul", 0)), attr_float(c, "scale"),
-                                   seq_major ? 1 : 0, ws, few_bytes, y.data()),
-                               "rmlk.Attention"))
-                return;
+            const int32_t scale_is_mul = static_cast<int32_t>(c.attr_int("scale_is_mul", 0));
+            // the last block of a KV head merges its chunks when the session's counters cover the heads
+            const int32_t st =
+                bsz * grp <= Session::kBlockCounters
+                    ? rmlk_hip_attention_few_rows_one_launch(c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim,
+                                                             q.data(), k.data(), v.data(), mask.data(), &ms,
+                                                             scale_is_mul, attr_float(c, "scale"), seq_major ? 1 : 0,
+                                                             ws, few_bytes, c.session.block_counters, y.data())
+                    : rmlk_hip_attention_few_rows(c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, q.data(),
+                                                  k.data(), v.data(), mask.data(), &ms, scale_is_mul,
+                                                  attr_float(c, "scale"), seq_major ? 1 : 0, ws, few_bytes,
+                                                  y.data());
+            if (took_fast_path(st, "rmlk.Attention")) return;
         }
         ok = ok && rep_k * seq >= 32;
         if (ok) {

@@ -267,6 +267,7 @@ Session::~Session() {
     scratch_bufs.clear();
     if (workspace) (void)hipFree(workspace);
     if (err_flag) (void)hipFree(err_flag);
+    if (block_counters) (void)hipFree(block_counters);
     if (err_host) (void)hipHostFree(err_host);
     if (stream) (void)hipStreamDestroy(stream);
 }
@@ -356,6 +357,8 @@ void Session::build(const rmlk_graph &graph, int dev) {
     check_hip(hipMalloc(reinterpret_cast<void **>(&err_flag), sizeof(int32_t)), "hipMalloc");
     check_hip(hipHostMalloc(reinterpret_cast<void **>(&err_host), sizeof(int32_t)), "hipHostMalloc");
     *err_host = 0;
+    check_hip(hipMalloc(reinterpret_cast<void **>(&block_counters), kBlockCounters * sizeof(int32_t)), "hipMalloc");
+    check_hip(hipMemset(block_counters, 0, kBlockCounters * sizeof(int32_t)), "hipMemset");
     if (g->outputs.empty()) throw RtError(RMLK_ERR_GRAPH, "graph has no outputs");
     values.assign(g->values.size(), Tensor());
     for (size_t n = 0; n < g->nodes.size(); ++n) {

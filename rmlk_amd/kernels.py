@@ -270,6 +270,22 @@ def attention_few_rows(q, k, v, mask, out, batch: int, kv_heads: int, rep: int, 
           "rmlk_hip_attention_few_rows")
 
 
+def attention_few_rows_one_launch(q, k, v, mask, out, counters, batch: int, kv_heads: int, rep: int,
+                                  q_len: int, kv_len: int, head_dim: int, mask_stride, scale: float,
+                                  scale_is_mul: bool = False, out_seq_major: bool = False) -> None:
+    """`attention_few_rows` without the merge launch; `counters`: batch * kv_heads int32, zero before the
+    first call and zero again after every call."""
+    need = int(lib().rmlk_hip_attention_few_rows_workspace_size(dtype_of(q), batch, kv_heads, rep, q_len,
+                                                                kv_len, head_dim))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    check(lib().rmlk_hip_attention_few_rows_one_launch(_stream(), dtype_of(q), batch, kv_heads, rep, q_len,
+                                                       kv_len, head_dim, _ptr(q), _ptr(k), _ptr(v),
+                                                       _ptr(mask), Dims.of(mask_stride), int(scale_is_mul),
+                                                       float(scale), int(out_seq_major), _ptr(ws), need,
+                                                       _ptr(counters), _ptr(out)),
+          "rmlk_hip_attention_few_rows_one_launch")
+
+
 def gemv_kmajor(x, wt, y, n: int, k: int) -> None:
     """y[n] = sum_k x[k] * wt[n][k]: one-row product with K-contiguous weights, no combine launch."""
     check(lib().rmlk_hip_gemv_kmajor(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(wt), k, _ptr(y)),

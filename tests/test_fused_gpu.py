@@ -1435,6 +1435,40 @@ def test_attention_few_rows_matches_separate_kernels(device, b, g, rep, s, l, ma
     assert_exact(to_np(moved), to_np(got).transpose(0, 2, 1, 3))
 
 
+@pytest.mark.parametrize("b,g,rep,s,l,mask_shape", [
+    (1, 8, 4, 1, 640, (1, 1, 1, 640)),       # a decode step of the 1B shape
+    (1, 8, 4, 1, 2048, (1, 1, 1, 2048)),     # 32 chunks
+    (2, 2, 3, 2, 130, (2, 1, 2, 130)),       # ragged last chunk, per-batch mask, two query rows
+    (1, 1, 1, 1, 5, (1, 1, 1, 5)),           # one chunk: every block is the last
+    (1, 2, 16, 1, 200, (1, 32, 1, 200)),     # 16 query heads per KV head
+    (3, 8, 2, 1, 4500, (3, 1, 1, 4500)),     # more chunks than a wavefront has lanes
+])
+def test_attention_few_rows_in_one_launch_is_bit_identical(device, b, g, rep, s, l, mask_shape):
+    """The last block of a KV head merges its chunks: same numbers as the two-kernel call, and the
+    counters are zero again, call after call with the same counters."""
+    import torch
+    kk = _k()
+    h, d = g * rep, 64
+    rng = np.random.default_rng(b * 100 + s + l)
+    q, k, v = (to_dev(rng.standard_normal(sh, dtype=np.float32), device)
+               for sh in ((b, h, s, d), (b, g, l, d), (b, g, l, d)))
+    m_np = rng.standard_normal(mask_shape, dtype=np.float32)
+    m_np[..., l - l // 3:] = -np.inf
+    m = to_dev(m_np, device)
+    ms = bcast_strides(list(mask_shape), [b, h, s, l])
+    exp = torch.full((b, h, s, d), float("nan"), device=device)
+    kk.attention_few_rows(q, k, v, m, exp, b, g, rep, s, l, d, ms, 8.0)
+    counters = torch.zeros(b * g + 3, dtype=torch.int32, device=device)
+    counters[b * g:] = 77     # not the kernel's
+    for seq_major in (False, True, False):
+        got = torch.full((b, s, h, d) if seq_major else (b, h, s, d), float("nan"), device=device)
+        kk.attention_few_rows_one_launch(q, k, v, m, got, counters, b, g, rep, s, l, d, ms, 8.0,
+                                         out_seq_major=seq_major)
+        want = to_np(exp).transpose(0, 2, 1, 3) if seq_major else to_np(exp)
+        assert_exact(to_np(got), want)
+        assert to_np(counters).tolist() == [0] * (b * g) + [77] * 3
+
+
 def test_attention_few_rows_declines_many_rows(device):
     import torch
     from rmlk_amd import RmlkError
