@@ -8,6 +8,7 @@
 #include <cstdint>
 #include <cstring>
 #include <map>
+#include <deque>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -201,6 +202,9 @@ struct OpContext {
     std::vector<Tensor *> in;   // nullptr for an omitted optional input
     std::vector<Tensor *> out;
     hipStream_t stream;
+    // Tensors an op makes to stand in for an input (`in[i]` may point here): they live as long as
+    // the context, which the executor still reads after the op has returned.
+    std::deque<Tensor> temps;
 
     int n_inputs() const { return static_cast<int>(in.size()); }
     bool has_input(int i) const { return i < n_inputs() && in[i] && in[i]->defined(); }

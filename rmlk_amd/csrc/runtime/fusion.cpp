@@ -960,11 +960,13 @@ void defer_norm(OpContext &c, int out_index, const Tensor &row, const Tensor &ga
     y.pending_norm = pn;
 }
 
-// The consumer's side: input 0 with a pending norm is replaced by the computed norm (kept in
-// `store`) when the consumer is not going to apply it itself.
-void compute_pending_norm(OpContext &c, Tensor *store) {
+// The consumer's side: input 0 with a pending norm is replaced by the computed norm (a tensor of
+// the context's own) when the consumer is not going to apply it itself.
+void compute_pending_norm(OpContext &c) {
     const Tensor &row = c.input(0);
     const PendingNorm &pn = *row.pending_norm;
+    c.temps.emplace_back();
+    Tensor *store = &c.temps.back();
     {
         std::vector<Tensor *> keep = c.out;
         c.out = {store};
@@ -1508,7 +1510,6 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
 // no combine launch); anything else is the plain MatMul.
 void op_fused_matmul_const(OpContext &c) {
     const Tensor &w = c.input(1), &wt = c.input(2);
-    Tensor normed;   // of a row whose norm was left to this node and that it cannot apply itself
     const bool one_row = [&] {
         const Tensor &a = c.input(0);
         return a.dtype == RMLK_FLOAT && a.rank() >= 1 && w.rank() == 2 && a.shape.back() == w.shape[0] &&
@@ -1529,13 +1530,13 @@ void op_fused_matmul_const(OpContext &c) {
                                "rmlk.MatMulConst"))
                 return;
         }
-        if (c.input(0).pending_norm) compute_pending_norm(c, &normed);
+        if (c.input(0).pending_norm) compute_pending_norm(c);
         if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, w.shape[1], w.shape[0], c.input(0).data(),
                                                 wt.data(), w.shape[0], y.data()),
                            "rmlk.MatMulConst"))
             return;
     }
-    if (c.input(0).pending_norm) compute_pending_norm(c, &normed);
+    if (c.input(0).pending_norm) compute_pending_norm(c);
     run_body(c);
 }
 
@@ -1557,7 +1558,6 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
     const Tensor &w = c.input(1);
     const std::vector<int64_t> widths = c.attr_ints("widths");
     const int64_t k = w.shape[0];
-    Tensor normed;   // of a row whose norm was left to this node and that it cannot apply itself
     if (c.input(0).pending_norm) {
         const Tensor &row = c.input(0);
         const PendingNorm &pn = *row.pending_norm;
@@ -1574,7 +1574,7 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
                                "rmlk.MatMulGroupSwiGLU"))
                 return;
         }
-        compute_pending_norm(c, &normed);
+        compute_pending_norm(c);
     }
     const Tensor &a = c.input(0);
     const bool ok = a.dtype == RMLK_FLOAT && a.rank() >= 1 && a.shape.back() == k && a.numel() == k &&
@@ -1626,10 +1626,9 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
 void op_fused_matmul_group(OpContext &c) {
     const Tensor &w = c.input(1);
     const std::vector<int64_t> widths = c.attr_ints("widths");
-    Tensor normed;   // of a row whose norm was left to this node and that it cannot apply itself
     std::shared_ptr<const PendingNorm> pending = c.input(0).pending_norm;
     if (pending && !(c.has_input(2) && c.input(0).numel() == w.shape[0] && w.shape[1] < kMaxDeferredNormWidth)) {
-        compute_pending_norm(c, &normed);
+        compute_pending_norm(c);
         pending.reset();
     }
     const Tensor &a = c.input(0);
@@ -1694,7 +1693,7 @@ void op_fused_matmul_group(OpContext &c) {
                                                               pending->reciprocal, c.input(2).data(), k,
                                                               row.data()),
                                   "rmlk.MatMulGroup");
-            if (!done) compute_pending_norm(c, &normed);   // `run` reads input 0 through the context
+            if (!done) compute_pending_norm(c);   // `run` reads input 0 through the context
         }
         const Tensor &a1 = c.input(0);
         if (!done && !(c.has_input(2) &&
