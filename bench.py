@@ -99,8 +99,13 @@ def run_llama(args):
     graph = graphs.llama_graph(cfg, seed=4, style="scatter", max_len=max_len)
     log(f"[bench] graph built in {time.perf_counter() - t0:.1f}s: {len(graph.nodes)} nodes")
     t0 = time.perf_counter()
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(0)[0]
     inst = runtime.Builder.from_graph(graph).build(0)
-    log(f"[bench] session created (weights uploaded) in {time.perf_counter() - t0:.1f}s")
+    torch.cuda.synchronize()
+    weights_resident = free_before - torch.cuda.mem_get_info(0)[0]
+    log(f"[bench] session created (weights uploaded) in {time.perf_counter() - t0:.1f}s, "
+        f"{weights_resident / 1e9:.2f} GB of device memory")
 
     # A plain copy of known size (256 MiB read + 256 MiB written by copy_flat_kernel): the unit
     # that rocprofv3's FETCH_SIZE / WRITE_SIZE readings of the other kernels are scaled by.
@@ -141,6 +146,7 @@ def run_llama(args):
     replay_logits = inst.output("logits")[0, -1].copy()
     assert np.array_equal(first_logits, replay_logits), "replayed prefill differs from the eager run"
     mem = inst.memory_stats()
+    mem["session_device_bytes_after_build"] = int(weights_resident)
     log(f"[bench] prefill {prompt_len} tokens: {ms_per_step:.2f} ms/step, {tok_s:.0f} tok/s")
 
     # ---- roofline of the MatMul kernels: one extra eager pass with HIP events per node ----------

@@ -383,31 +383,34 @@ int32_t rmlk_hip_attention_few_rows_one_launch(rmlk_stream_t stream, int32_t dty
 
 /* ---- products that share their first operand (q/k/v, gate/up) ----------------------------------
  * The weights of such MatMuls (ref: one cublasGemmStridedBatchedEx each,
- * cuda/src/kernels/gemm.rs:191-232) lie side by side in one row-major matrix B [k, sum(widths)].
+ * cuda/src/kernels/gemm.rs:191-232) lie side by side in one matrix B: row-major [k, sum(widths)]
+ * (trans_b == 0), or K-contiguous [sum(widths), k], one row per output column (trans_b != 0), which
+ * is also what the one-row products below read - one copy of the weights serves every row count.
  *
  * rmlk_hip_matmul_grouped: outs[i] (dense [m, widths[i]]) = A[m, k] . B[:, block i], block i being
- * the next widths[i] columns. One launch covers all blocks where whole tiles allow it; otherwise
+ * the next widths[i] columns (rows of a K-contiguous B). One launch covers all blocks where whole tiles allow it; otherwise
  * the blocks are multiplied one after the other, with the same results as rmlk_hip_matmul on each.
  * groups <= 4. The workspace must hold rmlk_hip_matmul_grouped_workspace_size bytes. */
 size_t rmlk_hip_matmul_grouped_workspace_size(int32_t dtype, int64_t m, int64_t k, int32_t groups,
                                               const int64_t *widths);
 int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t k,
                                 const void *a, int64_t lda, const void *b, int64_t ldb,
-                                int32_t groups, const int64_t *widths, void *const *outs,
-                                void *workspace, size_t workspace_bytes);
+                                int32_t trans_b, int32_t groups, const int64_t *widths,
+                                void *const *outs, void *workspace, size_t workspace_bytes);
 /* out[m, n] = swiglu(A . B[:, gate_offset .. +n], A . B[:, up_offset .. +n]) (see rmlk_hip_swiglu)
- * in one launch, the activation applied to the accumulators. Covers n % 64 == 0, k % 32 == 0,
- * 16-byte aligned rows and at least one 128 x 64 tile per compute unit; RMLK_ERR_UNSUPPORTED
- * otherwise (the caller then multiplies and activates separately). */
+ * in one launch, the activation applied to the accumulators; with trans_b the offsets count rows of
+ * the K-contiguous B. Covers n % 64 == 0, k % 32 == 0, 16-byte aligned rows and at least one
+ * 128 x 64 tile per compute unit; RMLK_ERR_UNSUPPORTED otherwise (the caller then multiplies and
+ * activates separately). Results do not depend on trans_b. */
 int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n, int64_t k,
-                               const void *a, int64_t lda, const void *b, int64_t ldb,
+                               const void *a, int64_t lda, const void *b, int64_t ldb, int32_t trans_b,
                                int64_t gate_offset, int64_t up_offset, void *out, int64_t ldc);
 
 /* One-row product with K-CONTIGUOUS weights: y[n] = sum_k x[k] * wt[n][k] (wt row-major [n, k],
  * leading dimension ldw), i.e. rmlk_hip_matmul with m = 1 and trans_b. Every output column is
  * finished inside one wavefront: no workspace and no combine launch, at any width. k % 4 == 0,
- * 16-byte aligned operands; RMLK_ERR_UNSUPPORTED otherwise. The decode step of a session keeps a
- * K-contiguous copy of constant weight matrices for it (ref: cublasGemmStridedBatchedEx with
+ * 16-byte aligned operands; RMLK_ERR_UNSUPPORTED otherwise. A session stores constant weight
+ * matrices K-contiguous for it (ref: cublasGemmStridedBatchedEx with
  * CUBLAS_OP_T on a transposed operand, cuda/src/kernels/gemm.rs:191-232). */
 int32_t rmlk_hip_gemv_kmajor(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k, const void *x,
                         const void *wt, int64_t ldw, void *y);
@@ -434,8 +437,8 @@ int32_t rmlk_hip_gemv_kmajor_swiglu_normed(rmlk_stream_t stream, int32_t dtype, 
                                            int64_t gate_row, int64_t up_row, void *y);
 
 /* ---- many-row products whose split-K combine is left to the consumer ----------------------------
- * rmlk_hip_matmul_partials: the tiled kernels of rmlk_hip_matmul for A[m, k] . B[k, n] (row-major,
- * m > 8) without the combine: `workspace` receives *splits_out partial matrices [m, n] one after
+ * rmlk_hip_matmul_partials: the tiled kernels of rmlk_hip_matmul for A[m, k] . B (row-major [k, n],
+ * or K-contiguous [n, k] with trans_b; m > 8) without the combine: `workspace` receives *splits_out partial matrices [m, n] one after
  * the other (*splits_out >= 1; their sum in ascending order is the product rmlk_hip_matmul returns).
  * rmlk_hip_splitk_add_rmsnorm: rmlk_hip_add_rmsnorm whose first operand is that sum,
  * a = partials[0] + partials[1] + ..; `slab` = elements from one partial matrix to the next.
@@ -444,7 +447,8 @@ int32_t rmlk_hip_gemv_kmajor_swiglu_normed(rmlk_stream_t stream, int32_t dtype, 
 size_t rmlk_hip_matmul_partials_workspace_size(int32_t dtype, int64_t m, int64_t n, int64_t k);
 int32_t rmlk_hip_matmul_partials(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n, int64_t k,
                                  const void *a, int64_t lda, const void *b, int64_t ldb,
-                                 void *workspace, size_t workspace_bytes, int32_t *splits_out);
+                                 int32_t trans_b, void *workspace, size_t workspace_bytes,
+                                 int32_t *splits_out);
 int32_t rmlk_hip_splitk_add_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t rows, int64_t cols,
                                     const void *partials, int32_t splits, int64_t slab,
                                     const void *b, const void *gamma, float eps,

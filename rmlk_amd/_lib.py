@@ -111,7 +111,7 @@ SIGNATURES = {
                                          c_int64, c_int64, c_void_p]),
     "rmlk_hip_matmul_partials_workspace_size": (c_size_t, [c_int32, c_int64, c_int64, c_int64]),
     "rmlk_hip_matmul_partials": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p,
-                                           c_int64, c_void_p, c_int64, c_void_p, c_size_t,
+                                           c_int64, c_void_p, c_int64, c_int32, c_void_p, c_size_t,
                                            POINTER(c_int32)]),
     "rmlk_hip_splitk_add_rmsnorm": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int32,
                                               c_int64, c_void_p, c_void_p, ctypes.c_float, c_int32,
@@ -148,10 +148,10 @@ SIGNATURES = {
     "rmlk_hip_matmul_grouped_workspace_size": (c_size_t, [c_int32, c_int64, c_int64, c_int32,
                                                           POINTER(c_int64)]),
     "rmlk_hip_matmul_grouped": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int64,
-                                          c_void_p, c_int64, c_int32, POINTER(c_int64),
+                                          c_void_p, c_int64, c_int32, c_int32, POINTER(c_int64),
                                           POINTER(c_void_p), c_void_p, c_size_t]),
     "rmlk_hip_matmul_swiglu": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p,
-                                         c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p,
+                                         c_int64, c_void_p, c_int64, c_int32, c_int64, c_int64, c_void_p,
                                          c_int64]),
     "rmlk_hip_rotary": (c_int32, [c_void_p, c_int32, _PD, _PD, _PD, _PD, c_void_p, c_void_p,
                                   c_void_p, c_void_p]),

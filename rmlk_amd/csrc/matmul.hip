@@ -371,8 +371,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
 template <int BM, int BN, int WM, int WN, bool TB, int STAGES, bool SWIGLU = false, bool EDGE = false>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) {
     static_assert(STAGES == 2, "two LDS stages");
-    static_assert(!SWIGLU || (!TB && WN == 64),
-                  "SwiGLU epilogue: row-major B, two accumulator columns (EDGE: partial tiles in m only)");
+    static_assert(!SWIGLU || WN == 64,
+                  "SwiGLU epilogue: two accumulator columns (EDGE: partial tiles in m only)");
     constexpr int BK = 32;
     constexpr int KC = BK / 8;
     constexpr int kAFloats = BM * BK;   // one stage of A, floats
@@ -421,12 +421,18 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     const float *b_ptr;
     int64_t b_step_stride;
     if constexpr (TB) {
-        b_ptr = B + static_cast<int64_t>(n0) * g.ldb + k_begin;
+        b_ptr = B + (SWIGLU ? 0 : static_cast<int64_t>(n0) * g.ldb) + k_begin;
         b_step_stride = BK;
 #pragma unroll
         for (int p = 0; p < B_PASSES; ++p) {
             int row = p * 32 + wave * 8 + sw_row;
-            if constexpr (EDGE) row = min(row, g.n - 1 - n0);
+            if constexpr (SWIGLU) {
+                // LDS row r: wavefront column r / 64, accumulator (r % 64) / 32, lane r % 32
+                const int out_col = tile_n * (BN / 2) + (row / 64) * 32 + row % 32;
+                row = ((row % 64) / 32 ? g.up_offset : g.gate_offset) + out_col;
+            } else if constexpr (EDGE) {
+                row = min(row, g.n - 1 - n0);
+            }
             b_voff[p] = static_cast<uint32_t>((row * g.ldb + sw_unit * 4) * static_cast<int64_t>(4));
         }
     } else {
@@ -1560,8 +1566,8 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
 // silu(A . B[:, gate..]) * (A . B[:, up..]) in one launch: 128 x 128 tiles of 64 gate and 64 up
 // columns. Whole tiles in n and k, no split-K, enough tiles to cover the chip; otherwise UNSUPPORTED.
 int32_t gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float *pa, int64_t lda,
-                    const float *pb, int64_t ldb, int64_t gate_offset, int64_t up_offset, float *pc,
-                    int64_t ldc) {
+                    const float *pb, int64_t ldb, int32_t trans_b, int64_t gate_offset, int64_t up_offset,
+                    float *pc, int64_t ldc) {
     const bool aligned = lda % 4 == 0 && ldb % 4 == 0 && gate_offset % 4 == 0 && up_offset % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
                          reinterpret_cast<uintptr_t>(pb) % 16 == 0;
@@ -1587,6 +1593,13 @@ int32_t gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float 
     g.aligned = 1;
     g.gate_offset = static_cast<int32_t>(gate_offset);
     g.up_offset = static_cast<int32_t>(up_offset);
+    if (trans_b) {
+        // (a lane's byte offset into B covers a row number of the whole matrix here)
+        const int64_t last_row = (gate_offset > up_offset ? gate_offset : up_offset) + n;
+        if (last_row * ldb >= (1ll << 30)) return RMLK_ERR_UNSUPPORTED;
+        if (m % 128 == 0) return launch_direct<128, 128, 64, 64, true, 2, true, false>(s, g, 1, 1);
+        return launch_direct<128, 128, 64, 64, true, 2, true, true>(s, g, 1, 1);
+    }
     if (m % 128 == 0) return launch_direct<128, 128, 64, 64, false, 2, true, false>(s, g, 1, 1);
     return launch_direct<128, 128, 64, 64, false, 2, true, true>(s, g, 1, 1);
 }
@@ -1861,8 +1874,8 @@ extern "C" size_t rmlk_hip_matmul_grouped_workspace_size(int32_t dtype, int64_t 
 
 extern "C" int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t k,
                                            const void *a, int64_t lda, const void *b, int64_t ldb,
-                                           int32_t groups, const int64_t *widths, void *const *outs,
-                                           void *workspace, size_t workspace_bytes) {
+                                           int32_t trans_b, int32_t groups, const int64_t *widths,
+                                           void *const *outs, void *workspace, size_t workspace_bytes) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
     if (!widths || !outs) return RMLK_ERR_NULL_POINTER;
     if (groups <= 0 || groups > kMaxSegments || m < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
@@ -1881,7 +1894,7 @@ extern "C" int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, 
         total += widths[i];
     }
     if (total >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
-    if (ldb < total) return RMLK_ERR_SIZE_MISMATCH;
+    if (ldb < (trans_b ? k : total)) return RMLK_ERR_SIZE_MISMATCH;
     sg.begin[groups] = static_cast<int32_t>(total);
     if (m == 0 || total == 0) return RMLK_OK;
     if (!a || !b) return RMLK_ERR_NULL_POINTER;
@@ -1889,16 +1902,17 @@ extern "C" int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, 
         const size_t need = rmlk_hip_matmul_workspace_size(dtype, 1, m, total, k);
         if (need && (!workspace || workspace_bytes < need)) return RMLK_ERR_WORKSPACE;
         const int32_t st = gemm_tiled(as_stream(stream), 1, m, total, k, static_cast<const float *>(a),
-                                      lda, 0, static_cast<const float *>(b), ldb, 0, 0, sg.c[0], sg.ldc[0],
-                                      0, workspace, workspace_bytes, &sg);
+                                      lda, 0, static_cast<const float *>(b), ldb, 0, trans_b, sg.c[0],
+                                      sg.ldc[0], 0, workspace, workspace_bytes, &sg);
         if (st != RMLK_ERR_UNSUPPORTED) return st;
     }
     int64_t off = 0;
     for (int i = 0; i < groups; ++i) {
         if (widths[i] > 0) {
+            // block i: the next widths[i] columns of a row-major B, the next widths[i] rows of a K-contiguous one
             const int32_t st = rmlk_hip_matmul(stream, dtype, 1, m, widths[i], k, a, lda, 0, 0,
-                                               static_cast<const float *>(b) + off, ldb, 0, 0, outs[i],
-                                               widths[i], 0, workspace, workspace_bytes);
+                                               static_cast<const float *>(b) + (trans_b ? off * ldb : off), ldb,
+                                               0, trans_b, outs[i], widths[i], 0, workspace, workspace_bytes);
             if (st) return st;
         }
         off += widths[i];
@@ -1908,17 +1922,20 @@ extern "C" int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, 
 
 extern "C" int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n,
                                           int64_t k, const void *a, int64_t lda, const void *b,
-                                          int64_t ldb, int64_t gate_offset, int64_t up_offset, void *out,
-                                          int64_t ldc) {
+                                          int64_t ldb, int32_t trans_b, int64_t gate_offset,
+                                          int64_t up_offset, void *out, int64_t ldc) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
     if (m < 0 || n < 0 || k < 0 || gate_offset < 0 || up_offset < 0) return RMLK_ERR_INVALID_ARGUMENT;
-    if (m >= (1ll << 31) || n >= (1ll << 30) || k >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
-    if (lda < k || ldc < n || ldb < gate_offset + n || ldb < up_offset + n) return RMLK_ERR_SIZE_MISMATCH;
+    if (m >= (1ll << 31) || n >= (1ll << 30) || k >= (1ll << 31) || gate_offset >= (1ll << 30) ||
+        up_offset >= (1ll << 30))
+        return RMLK_ERR_TOO_LARGE;
+    if (lda < k || ldc < n) return RMLK_ERR_SIZE_MISMATCH;
+    if (trans_b ? ldb < k : (ldb < gate_offset + n || ldb < up_offset + n)) return RMLK_ERR_SIZE_MISMATCH;
     if (m == 0 || n == 0) return RMLK_OK;
     if (!a || !b || !out) return RMLK_ERR_NULL_POINTER;
     if (reinterpret_cast<uintptr_t>(out) % 4 != 0) return RMLK_ERR_UNSUPPORTED;
     return gemm_swiglu(as_stream(stream), m, n, k, static_cast<const float *>(a), lda,
-                       static_cast<const float *>(b), ldb, gate_offset, up_offset,
+                       static_cast<const float *>(b), ldb, trans_b, gate_offset, up_offset,
                        static_cast<float *>(out), ldc);
 }
 
@@ -1929,17 +1946,17 @@ extern "C" size_t rmlk_hip_matmul_partials_workspace_size(int32_t dtype, int64_t
 
 extern "C" int32_t rmlk_hip_matmul_partials(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n,
                                             int64_t k, const void *a, int64_t lda, const void *b,
-                                            int64_t ldb, void *workspace, size_t workspace_bytes,
-                                            int32_t *splits_out) {
+                                            int64_t ldb, int32_t trans_b, void *workspace,
+                                            size_t workspace_bytes, int32_t *splits_out) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
     if (m < 0 || n < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (m >= (1ll << 31) || n >= (1ll << 31) || k >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
     if (m <= kSkinnyRows || n == 0 || k == 0) return RMLK_ERR_UNSUPPORTED;   // not the tiled kernels' case
     if (!a || !b || !workspace || !splits_out) return RMLK_ERR_NULL_POINTER;
-    if (lda < k || ldb < n) return RMLK_ERR_SIZE_MISMATCH;
+    if (lda < k || ldb < (trans_b ? k : n)) return RMLK_ERR_SIZE_MISMATCH;
     if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return RMLK_ERR_UNSUPPORTED;
     return gemm_tiled(as_stream(stream), 1, m, n, k, static_cast<const float *>(a), lda, 0,
-                      static_cast<const float *>(b), ldb, 0, 0, nullptr, n, 0, workspace,
+                      static_cast<const float *>(b), ldb, 0, trans_b, nullptr, n, 0, workspace,
                       workspace_bytes, nullptr, splits_out);
 }
 

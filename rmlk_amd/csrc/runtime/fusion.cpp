@@ -616,13 +616,12 @@ struct Matcher {
             Node &p = g.nodes[n];
             int normed = -1;
             if (p.op == "rmlk.RMSNorm") normed = p.outputs[0];
-            else if (p.op == "rmlk.MatMulAddRMSNorm" && p.inputs.size() == 5) normed = p.outputs[1];
+            else if (p.op == "rmlk.MatMulAddRMSNorm") normed = p.outputs[1];
             if (normed < 0 || g.values[normed].is_output || users[normed].size() != 1) continue;
             const Node &cons = g.nodes[users[normed][0]];
             const bool aware = (cons.op == "rmlk.MatMulGroup" || cons.op == "rmlk.MatMulGroupSwiGLU" ||
                                 cons.op == "rmlk.MatMulConst") &&
-                               cons.inputs.size() == 3 && cons.inputs[0] == normed &&
-                               cons.inputs[1] != normed && cons.inputs[2] != normed;
+                               cons.inputs.size() == 2 && cons.inputs[0] == normed && cons.inputs[1] != normed;
             if (!aware) continue;
             p.attrs["defer_norm"] = a_int(1);
             ++marked;
@@ -638,7 +637,7 @@ struct Matcher {
         for (size_t n = 0; n < g.nodes.size(); ++n) {
             if (removed[n]) continue;
             Node &p = g.nodes[n];
-            if (p.op != "rmlk.MatMulGroup" || p.inputs.size() != 3) continue;
+            if (p.op != "rmlk.MatMulGroup") continue;
             int reader = -1;
             bool ok = true;
             for (int o : p.outputs) {
@@ -682,26 +681,30 @@ struct Matcher {
                     if (!only_used_by(mm->outputs[0], {&cons}) ||
                         cons.inputs[0] == cons.inputs[1])
                         continue;
+                    const int wt = transposed_copy(w);
+                    if (wt < 0) continue;   // (K no multiple of 4: the separate nodes stay)
                     Node f;
                     f.op = "rmlk.MatMulAddRMSNorm";
-                    f.inputs = {mm->inputs[0], w, cons.inputs[1 - side], cons.inputs[2]};
-                    const int wt = transposed_copy(w);
-                    if (wt >= 0) {
-                        f.inputs.push_back(wt);
-                        users[wt].push_back(static_cast<int>(n));
-                    }
+                    f.inputs = {mm->inputs[0], wt, cons.inputs[1 - side], cons.inputs[2]};
+                    users[wt].push_back(static_cast<int>(n));
                     f.outputs = cons.outputs;
                     f.attrs = cons.attrs;
+                    Node prod;   // the product on its own, for the cases the joint kernels decline
+                    prod.op = "rmlk.MatMulConst";
+                    prod.inputs = {mm->inputs[0], wt};
+                    prod.outputs = mm->outputs;
                     Node norm = cons;
-                    f.body = {*mm, norm};
+                    f.body = {prod, norm};
                     const int mi = index_of(mm);
+                    const int act = mm->inputs[0];
                     for (int v : mm->inputs) {
                         auto &u = users[v];
                         u.erase(std::remove(u.begin(), u.end(), mi), u.end());
-                        u.push_back(static_cast<int>(n));
                     }
+                    users[act].push_back(static_cast<int>(n));
                     removed[mi] = true;
                     g.nodes[n] = std::move(f);
+                    release_unused(w);
                     ++formed;
                     break;
                 }
@@ -736,10 +739,15 @@ struct Matcher {
         return formed;
     }
 
-    // A K-contiguous ([n][k]) device copy of the constant 2-D float matrix `w` ([k][n]) as a new
-    // initializer; -1 when w is not such a matrix. A one-row product reads it with a wavefront per
-    // output column and needs no split-K combine; the row-major original stays for the GEMM.
+    // The constant 2-D float matrix `w` ([k][n]) stored K-contiguous ([n][k]) as a new initializer;
+    // -1 when w is not such a matrix or k is no multiple of 4. Every product of a fused node reads
+    // its weights in this one form: a one-row product with a wavefront per output column and no
+    // split-K combine, the GEMMs as their transposed-B variants (same sums in the same order as
+    // over the row-major form). The row-major original is released once no node reads it.
     std::unordered_map<int, int> transposed_of;
+    void release_unused(int w) {
+        if (w >= 0 && users[w].empty() && !g.values[w].is_output && !g.values[w].is_input) s.values[w].reset();
+    }
     int transposed_copy(int w) {
         auto it = transposed_of.find(w);
         if (it != transposed_of.end()) return it->second;
@@ -775,7 +783,7 @@ struct Matcher {
         return id;
     }
 
-    // ---- remaining MatMuls with constant 2-D weights (the lm-head): a K-contiguous copy for one row ---
+    // ---- remaining MatMuls with constant 2-D weights (the lm-head) --------------------------------
     int form_const_matmuls() {
         int formed = 0;
         for (size_t n = 0; n < g.nodes.size(); ++n) {
@@ -784,24 +792,28 @@ struct Matcher {
             if (mm.inputs.size() != 2 || mm.inputs[0] < 0) continue;
             const int wt = transposed_copy(mm.inputs[1]);
             if (wt < 0) continue;
+            const int w = mm.inputs[1];
             Node f;
             f.op = "rmlk.MatMulConst";
-            f.inputs = {mm.inputs[0], mm.inputs[1], wt};
+            f.inputs = {mm.inputs[0], wt};
             f.outputs = mm.outputs;
-            f.body = {mm};
             users[wt].push_back(static_cast<int>(n));
+            auto &u = users[w];
+            u.erase(std::remove(u.begin(), u.end(), static_cast<int>(n)), u.end());
             g.nodes[n] = std::move(f);
+            release_unused(w);
             ++formed;
         }
         return formed;
     }
 
     // ---- MatMuls that share their first operand and have constant 2-D weights (q/k/v, gate/up) ----
-    // The weights are laid side by side in ONE device matrix [K, N1 + N2 + ..] while building (the
-    // separate copies are released unless something else reads them). A one-row input then takes a
-    // single weight-streaming launch whose result is handed out as views; more rows take one GEMM
-    // per member on its column block of the joint matrix (leading dimension = the joint width), i.e.
-    // exactly the separate products. Nothing is left for a fallback body.
+    // The weights are laid one below the other in ONE K-contiguous device matrix [N1 + N2 + .., K]
+    // while building (the separate matrices are released unless something else reads them). A
+    // one-row input then takes a single weight-streaming launch whose result is handed out as
+    // views; more rows take one GEMM whose tiles write to the members' outputs, or one GEMM per
+    // member on its block of rows, i.e. exactly the separate products. Nothing is left for a
+    // fallback body.
     int form_matmul_groups() {
         int formed = 0;
         const size_t n_nodes = g.nodes.size();
@@ -813,7 +825,7 @@ struct Matcher {
                 if (!g.values[w].is_initializer) return false;
                 const Tensor &t = s.values[w];
                 if (!t.defined() || t.dtype != RMLK_FLOAT || t.rank() != 2 || t.shape[1] % 4 != 0 ||
-                    t.shape[0] == 0 || t.shape[1] == 0)
+                    t.shape[0] % 4 != 0 || t.shape[0] == 0 || t.shape[1] == 0)
                     return false;
                 *k = t.shape[0];
                 *n = t.shape[1];
@@ -839,19 +851,20 @@ struct Matcher {
             // the joint weight matrix
             Tensor joint;
             joint.dtype = RMLK_FLOAT;
-            joint.shape = {k0, total};
+            joint.shape = {total, k0};
             auto buf = std::make_shared<Buffer>();
             buf->bytes = joint.nbytes();
             buf->owned_raw = true;
             check_hip(hipMalloc(&buf->ptr, buf->bytes), "hipMalloc (joint weights)");
             joint.buf = buf;
-            rmlk_dims out_shape = to_dims(joint.shape);
             int64_t off = 0;
             for (size_t i = 0; i < members.size(); ++i) {
+                // member i transposed into its block of rows
                 const Tensor &w = s.values[g.nodes[members[i]].inputs[1]];
                 rmlk_dims in_shape = to_dims(w.shape);
-                check_status(rmlk_hip_concat(s.stream, RMLK_FLOAT, &in_shape, &out_shape, 1, off,
-                                             w.data(), joint.data()),
+                const int64_t perm[2] = {1, 0};
+                check_status(rmlk_hip_transpose(s.stream, RMLK_FLOAT, &in_shape, perm, w.data(),
+                                                static_cast<float *>(joint.data()) + off * k0),
                              "joint weights");
                 off += widths[i];
             }
@@ -866,11 +879,9 @@ struct Matcher {
             g.by_name[jv.name] = joint_id;
             s.values.push_back(joint);
             users.emplace_back();
-            const int joint_t = transposed_copy(joint_id);
             Node f;
             f.op = "rmlk.MatMulGroup";
             f.inputs = {a, joint_id};
-            if (joint_t >= 0) f.inputs.push_back(joint_t);
             f.attrs["widths"] = a_ints(widths);
             for (size_t i = 0; i < members.size(); ++i) {
                 const Node &mm = g.nodes[members[i]];
@@ -888,7 +899,6 @@ struct Matcher {
             removed[first] = false;
             users[a].push_back(static_cast<int>(first));
             users[joint_id].push_back(static_cast<int>(first));
-            if (joint_t >= 0) users[joint_t].push_back(static_cast<int>(first));
             for (int v : g.nodes[first].outputs) g.values[v].producer = static_cast<int>(first);
             ++formed;
         }
@@ -1442,28 +1452,28 @@ void op_fused_add_rmsnorm(OpContext &c) {
     run_body(c);
 }
 
-// MatMul(a, W) -> Add(residual) -> RMSNorm for many rows: the GEMM leaves its split-K slabs in the
-// workspace and the norm kernel adds them up while it forms the residual row.
+// MatMul(a, W) -> Add(residual) -> RMSNorm, W constant and stored K-contiguous (wt [n, k]). Many
+// rows: the GEMM leaves its split-K slabs in the workspace and the norm kernel adds them up while it
+// forms the residual row. One row: the product with the residual added, the norm left to its reader.
 void op_fused_matmul_add_rmsnorm(OpContext &c) {
-    const Tensor &a = c.input(0), &w = c.input(1), &res = c.input(2), &gamma = c.input(3);
-    bool ok = a.dtype == RMLK_FLOAT && w.dtype == RMLK_FLOAT && res.dtype == RMLK_FLOAT &&
-              gamma.dtype == RMLK_FLOAT && a.rank() >= 2 && w.rank() == 2 && a.numel() > 0 &&
-              w.numel() > 0 && a.shape.back() == w.shape[0];
+    const Tensor &a = c.input(0), &wt = c.input(1), &res = c.input(2), &gamma = c.input(3);
+    const int64_t n = wt.shape[0], k = wt.shape[1];
+    bool ok = a.dtype == RMLK_FLOAT && res.dtype == RMLK_FLOAT && gamma.dtype == RMLK_FLOAT && a.rank() >= 2 &&
+              a.numel() > 0 && a.shape.back() == k;
     if (ok) {
         std::vector<int64_t> out_shape(a.shape.begin(), a.shape.end() - 1);
-        out_shape.push_back(w.shape[1]);
+        out_shape.push_back(n);
         const int64_t axis = c.attr_int("axis", -1);
         ok = res.shape == out_shape && (axis == -1 || axis == res.rank() - 1) && gamma.rank() >= 1 &&
-             gamma.rank() <= res.rank() && gamma.numel() == w.shape[1] && gamma.shape.back() == w.shape[1];
+             gamma.rank() <= res.rank() && gamma.numel() == n && gamma.shape.back() == n;
     }
-    if (ok && a.numel() == w.shape[0] && c.has_input(4)) {
-        // one row: the product over the K-contiguous copy (no combine launch), then Add + norm
-        const int64_t k = w.shape[0], n = w.shape[1];
+    if (ok && a.numel() == k) {
+        // one row: no combine launch, then Add + norm
         if (may_defer_norm(c, res, gamma)) {
             // the product with the residual added is the row; the norm is left to the product
             // that reads it
             Tensor &sum = c.alloc_output(0, RMLK_FLOAT, res.shape);
-            if (took_fast_path(rmlk_hip_gemv_kmajor_add(c.stream, RMLK_FLOAT, n, k, a.data(), c.input(4).data(), k,
+            if (took_fast_path(rmlk_hip_gemv_kmajor_add(c.stream, RMLK_FLOAT, n, k, a.data(), wt.data(), k,
                                                         res.data(), sum.data()),
                                "rmlk.MatMulAddRMSNorm")) {
                 defer_norm(c, 1, sum, gamma);
@@ -1471,7 +1481,7 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
             }
         }
         float *prod = static_cast<float *>(c.scratch(static_cast<size_t>(n) * sizeof(float)));
-        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, n, k, a.data(), c.input(4).data(), k, prod),
+        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, n, k, a.data(), wt.data(), k, prod),
                            "rmlk.MatMulAddRMSNorm")) {
             Tensor &sum = c.alloc_output(0, RMLK_FLOAT, res.shape);
             Tensor &y = c.alloc_output(1, RMLK_FLOAT, res.shape);
@@ -1484,13 +1494,13 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
         }
     }
     if (ok) {
-        const int64_t k = w.shape[0], n = w.shape[1], m = a.numel() / k;
+        const int64_t m = a.numel() / k;
         const size_t bytes = rmlk_hip_matmul_partials_workspace_size(RMLK_FLOAT, m, n, k);
         if (bytes) {
             void *ws = c.scratch(bytes);
             int32_t splits = 0;
-            if (took_fast_path(rmlk_hip_matmul_partials(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, w.data(),
-                                                        n, ws, bytes, &splits),
+            if (took_fast_path(rmlk_hip_matmul_partials(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, wt.data(),
+                                                        k, 1, ws, bytes, &splits),
                                "rmlk.MatMulAddRMSNorm")) {
                 Tensor &sum = c.alloc_output(0, RMLK_FLOAT, res.shape);
                 Tensor &y = c.alloc_output(1, RMLK_FLOAT, res.shape);
@@ -1503,66 +1513,68 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
             }
         }
     }
-    run_body(c);
+    run_body(c);   // the product (rmlk.MatMulConst), then rmlk.AddRMSNorm
 }
 
-// MatMul(a, W) with constant 2-D W: a one-row input reads the K-contiguous copy of W (no split-K,
-// no combine launch); anything else is the plain MatMul.
+// a [.., k] . wt^T for any number of rows: the general product with a K-contiguous second operand
+// (`wt`: n rows of k), into the dense [m, n] at `out`.
+void product_over_kmajor(OpContext &c, const void *a, int64_t m, int64_t k, const void *wt, int64_t n, void *out,
+                         const char *what) {
+    const size_t ws_bytes = rmlk_hip_matmul_workspace_size(RMLK_FLOAT, 1, m, n, k);
+    void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
+    check_status(rmlk_hip_matmul(c.stream, RMLK_FLOAT, 1, m, n, k, a, k, 0, 0, wt, k, 0, 1, out, n, 0, ws, ws_bytes),
+                 what);
+}
+
+// What MatMul checks of a first operand [.., k]; returns its rows.
+int64_t rows_of(const Tensor &a, int64_t k) {
+    require_float(a.dtype);
+    if (a.rank() == 0) fail_op("ZeroRank");
+    if (a.shape.back() != k) fail_op("IncompatibleDimForMul");
+    return k ? a.numel() / k : 0;
+}
+
+// MatMul(a, W) with constant 2-D W stored K-contiguous (wt [n, k]): a one-row input takes the kernel
+// with a wavefront per output column (no split-K, no combine launch), anything else the general
+// product with a transposed second operand.
 void op_fused_matmul_const(OpContext &c) {
-    const Tensor &w = c.input(1), &wt = c.input(2);
-    const bool one_row = [&] {
+    const Tensor &wt = c.input(1);
+    const int64_t n = wt.shape[0], k = wt.shape[1];
+    const int64_t m = rows_of(c.input(0), k);
+    std::vector<int64_t> shape(c.input(0).shape.begin(), c.input(0).shape.end() - 1);
+    shape.push_back(n);
+    Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
+    if (m == 0) return;
+    if (m == 1) {
         const Tensor &a = c.input(0);
-        return a.dtype == RMLK_FLOAT && a.rank() >= 1 && w.rank() == 2 && a.shape.back() == w.shape[0] &&
-               a.numel() == w.shape[0] && w.shape[0] > 0;
-    }();
-    if (one_row) {
-        const Tensor &a = c.input(0);
-        std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
-        shape.push_back(w.shape[1]);
-        Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
         // (a very wide product -- the lm-head -- has thousands of blocks that would each normalise
         // the row: there the separate norm launch is cheaper)
-        if (a.pending_norm && w.shape[1] < kMaxDeferredNormWidth) {
+        if (a.pending_norm && n < kMaxDeferredNormWidth) {
             const PendingNorm &pn = *a.pending_norm;
-            if (took_fast_path(rmlk_hip_gemv_kmajor_normed(c.stream, RMLK_FLOAT, w.shape[1], w.shape[0], a.data(),
-                                                           pn.gamma.data(), pn.eps, pn.reciprocal, wt.data(),
-                                                           w.shape[0], y.data()),
+            if (took_fast_path(rmlk_hip_gemv_kmajor_normed(c.stream, RMLK_FLOAT, n, k, a.data(), pn.gamma.data(),
+                                                           pn.eps, pn.reciprocal, wt.data(), k, y.data()),
                                "rmlk.MatMulConst"))
                 return;
         }
         if (c.input(0).pending_norm) compute_pending_norm(c);
-        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, w.shape[1], w.shape[0], c.input(0).data(),
-                                                wt.data(), w.shape[0], y.data()),
+        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, n, k, c.input(0).data(), wt.data(), k, y.data()),
                            "rmlk.MatMulConst"))
             return;
     }
     if (c.input(0).pending_norm) compute_pending_norm(c);
-    run_body(c);
+    product_over_kmajor(c, c.input(0).data(), m, k, wt.data(), n, y.data(), "rmlk.MatMulConst");
 }
 
-// Partial rows of a one-row product in the session workspace; false when the GEMV does not cover it.
-bool gemv_partials(OpContext &c, const Tensor &a, const Tensor &w, const void **ws_out, int32_t *splits) {
-    const int64_t k = w.shape[0], n = w.shape[1];
-    const size_t bytes = rmlk_hip_gemv_partials_workspace_size(RMLK_FLOAT, n, k);
-    if (!bytes) return false;
-    void *ws = c.scratch(bytes);
-    if (!took_fast_path(rmlk_hip_gemv_partials(c.stream, RMLK_FLOAT, n, k, a.data(), w.data(), n, ws,
-                                               bytes, splits),
-                        "one-row MatMul"))
-        return false;
-    *ws_out = ws;
-    return true;
-}
-
+// swiglu(a . Wg, a . Wu) with [Wg | Wu] constant and stored K-contiguous as one matrix (wt [2 n, k]).
 void op_fused_matmul_group_swiglu(OpContext &c) {
-    const Tensor &w = c.input(1);
+    const Tensor &wt = c.input(1);
     const std::vector<int64_t> widths = c.attr_ints("widths");
-    const int64_t k = w.shape[0];
+    const int64_t k = wt.shape[1];
     if (c.input(0).pending_norm) {
         const Tensor &row = c.input(0);
         const PendingNorm &pn = *row.pending_norm;
         if (row.dtype == RMLK_FLOAT && row.rank() >= 1 && row.shape.back() == k && row.numel() == k &&
-            widths.size() == 2 && widths[0] == widths[1] && c.has_input(2)) {
+            widths.size() == 2 && widths[0] == widths[1]) {
             const int64_t n = widths[0];
             const bool gate_first = c.attr_int("gate_first", 1) != 0;
             std::vector<int64_t> shape(row.shape.begin(), row.shape.end() - 1);
@@ -1570,15 +1582,13 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
             Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
             if (took_fast_path(rmlk_hip_gemv_kmajor_swiglu_normed(
                                    c.stream, RMLK_FLOAT, n, k, row.data(), pn.gamma.data(), pn.eps, pn.reciprocal,
-                                   c.input(2).data(), k, gate_first ? 0 : n, gate_first ? n : 0, y.data()),
+                                   wt.data(), k, gate_first ? 0 : n, gate_first ? n : 0, y.data()),
                                "rmlk.MatMulGroupSwiGLU"))
                 return;
         }
         compute_pending_norm(c);
     }
     const Tensor &a = c.input(0);
-    const bool ok = a.dtype == RMLK_FLOAT && a.rank() >= 1 && a.shape.back() == k && a.numel() == k &&
-                    widths.size() == 2 && widths[0] == widths[1];
     const bool same_width = a.dtype == RMLK_FLOAT && a.rank() >= 1 && a.shape.back() == k && k > 0 &&
                             widths.size() == 2 && widths[0] == widths[1];
     if (same_width && a.numel() / k >= 128) {
@@ -1588,68 +1598,46 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
         std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
         shape.push_back(n);
         Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
-        if (took_fast_path(rmlk_hip_matmul_swiglu(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, w.data(),
-                                                  2 * n, gate_first ? 0 : n, gate_first ? n : 0, y.data(),
-                                                  n),
+        if (took_fast_path(rmlk_hip_matmul_swiglu(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, wt.data(), k, 1,
+                                                  gate_first ? 0 : n, gate_first ? n : 0, y.data(), n),
                            "rmlk.MatMulGroupSwiGLU"))
             return;
     }
-    if (ok && c.has_input(2)) {
-        // one row, K-contiguous weights: gate, up and the activation in one launch
+    if (same_width && a.numel() == k) {
+        // one row: gate, up and the activation in one launch
         const int64_t n = widths[0];
         const bool gate_first = c.attr_int("gate_first", 1) != 0;
         std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
         shape.push_back(n);
         Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
-        if (took_fast_path(rmlk_hip_gemv_kmajor_swiglu(c.stream, RMLK_FLOAT, n, k, a.data(), c.input(2).data(), k,
-                                                  gate_first ? 0 : n, gate_first ? n : 0, y.data()),
+        if (took_fast_path(rmlk_hip_gemv_kmajor_swiglu(c.stream, RMLK_FLOAT, n, k, a.data(), wt.data(), k,
+                                                       gate_first ? 0 : n, gate_first ? n : 0, y.data()),
                            "rmlk.MatMulGroupSwiGLU"))
             return;
     }
-    const void *ws = nullptr;
-    int32_t splits = 0;
-    if (ok && gemv_partials(c, a, w, &ws, &splits)) {
-        const int64_t n = widths[0];
-        const bool gate_first = c.attr_int("gate_first", 1) != 0;
-        std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
-        shape.push_back(n);
-        Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
-        if (took_fast_path(rmlk_hip_splitk_swiglu(c.stream, RMLK_FLOAT, n, ws, splits, 2 * n,
-                                                  gate_first ? 0 : n, gate_first ? n : 0, y.data()),
-                           "rmlk.MatMulGroupSwiGLU"))
-            return;
-    }
-    run_body(c);
+    run_body(c);   // rmlk.MatMulGroup, then rmlk.SwiGLU
 }
 
-// MatMul(a, W_i) for every member of a group, W_i being column blocks of one joint matrix.
+// MatMul(a, W_i) for every member of a group, the W_i stored K-contiguous one below the other in one
+// joint matrix (wt [N1 + N2 + .., k]).
 void op_fused_matmul_group(OpContext &c) {
-    const Tensor &w = c.input(1);
+    const Tensor &wt = c.input(1);
     const std::vector<int64_t> widths = c.attr_ints("widths");
+    const int64_t k = wt.shape[1], total = wt.shape[0];
     std::shared_ptr<const PendingNorm> pending = c.input(0).pending_norm;
-    if (pending && !(c.has_input(2) && c.input(0).numel() == w.shape[0] && w.shape[1] < kMaxDeferredNormWidth)) {
+    if (pending && !(c.input(0).numel() == k && total < kMaxDeferredNormWidth)) {
         compute_pending_norm(c);
         pending.reset();
     }
     const Tensor &a = c.input(0);
-    require_float(a.dtype);
-    if (a.rank() == 0) fail_op("ZeroRank");
-    const int64_t k = w.shape[0], total = w.shape[1];
-    if (a.shape.back() != k) fail_op("IncompatibleDimForMul");
-    const int64_t m = k ? a.numel() / k : 0;
+    const int64_t m = rows_of(a, k);
     std::vector<int64_t> lead(a.shape.begin(), a.shape.end() - 1);   // 1-D a: the row dim is dropped
     auto out_shape = [&](int64_t n) {
         std::vector<int64_t> sh = lead;
         sh.push_back(n);
         return sh;
     };
-    auto run = [&](int64_t n, const void *b, void *out, int64_t ldc) {
-        const size_t ws_bytes = rmlk_hip_matmul_workspace_size(RMLK_FLOAT, 1, m, n, k);
-        void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
-        check_status(rmlk_hip_matmul(c.stream, RMLK_FLOAT, 1, m, n, k, c.input(0).data(), k, 0, 0, b, total, 0,
-                                     0, out, ldc, 0, ws, ws_bytes),
-                     "rmlk.MatMulGroup");
-    };
+    const float *rows = static_cast<const float *>(wt.data());
     if (m == 1) {
         // one launch over the joint matrix; the members' results are slices of its output row
         Tensor row;
@@ -1672,35 +1660,32 @@ void op_fused_matmul_group(OpContext &c) {
                 off += widths[i];
             }
         };
-        if (c.attr_int("defer_product", 0) != 0 && c.has_input(2) && k % 4 == 0 && k > 0) {
+        if (c.attr_int("defer_product", 0) != 0) {
             // left to the row-stream node behind it (op_fused_head_rows)
             auto pp = std::make_shared<PendingProduct>();
             pp->x = a;
             pp->x.pending_norm.reset();
             pp->norm = pending;
-            pp->wt = c.input(2);
+            pp->wt = wt;
             pp->row = row;
             pp->k = k;
             pp->total = total;
             hand_out(pp);
             return;
         }
-        // (over its K-contiguous copy when there is one: no split-K, no combine launch)
         bool done = false;
         if (pending) {
             done = took_fast_path(rmlk_hip_gemv_kmajor_normed(c.stream, RMLK_FLOAT, total, k, a.data(),
                                                               pending->gamma.data(), pending->eps,
-                                                              pending->reciprocal, c.input(2).data(), k,
-                                                              row.data()),
+                                                              pending->reciprocal, wt.data(), k, row.data()),
                                   "rmlk.MatMulGroup");
-            if (!done) compute_pending_norm(c);   // `run` reads input 0 through the context
+            if (!done) compute_pending_norm(c);   // what follows reads input 0 through the context
         }
         const Tensor &a1 = c.input(0);
-        if (!done && !(c.has_input(2) &&
-                       took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, total, k, a1.data(),
-                                                           c.input(2).data(), k, row.data()),
-                                      "rmlk.MatMulGroup")))
-            run(total, w.data(), row.data(), total);
+        if (!done && !took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, total, k, a1.data(), wt.data(), k,
+                                                          row.data()),
+                                     "rmlk.MatMulGroup"))
+            product_over_kmajor(c, a1.data(), 1, k, wt.data(), total, row.data(), "rmlk.MatMulGroup");
         hand_out(nullptr);
         return;
     }
@@ -1713,7 +1698,7 @@ void op_fused_matmul_group(OpContext &c) {
         const size_t ws_bytes = rmlk_hip_matmul_grouped_workspace_size(
             RMLK_FLOAT, m, k, static_cast<int32_t>(widths.size()), widths.data());
         void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
-        check_status(rmlk_hip_matmul_grouped(c.stream, RMLK_FLOAT, m, k, a.data(), k, w.data(), total,
+        check_status(rmlk_hip_matmul_grouped(c.stream, RMLK_FLOAT, m, k, a.data(), k, wt.data(), k, 1,
                                              static_cast<int32_t>(widths.size()), widths.data(),
                                              outs.data(), ws, ws_bytes),
                      "rmlk.MatMulGroup");
@@ -1723,7 +1708,7 @@ void op_fused_matmul_group(OpContext &c) {
     for (size_t i = 0; i < widths.size(); ++i) {
         Tensor &y = c.alloc_output(static_cast<int>(i), RMLK_FLOAT, out_shape(widths[i]));
         if (y.numel() > 0)
-            run(widths[i], static_cast<const float *>(w.data()) + off, y.data(), widths[i]);
+            product_over_kmajor(c, a.data(), m, k, rows + off * k, widths[i], y.data(), "rmlk.MatMulGroup");
         off += widths[i];
     }
 }

@@ -505,15 +505,16 @@ void Session::run_nodes() {
             for (const Tensor &t : outs) out_elems += static_cast<double>(t.numel());
             flops = 2.0 * out_elems * static_cast<double>(ctx.in[0]->shape.back());
         } else if (node.op == "rmlk.MatMulAddRMSNorm" && ctx.in[0] && ctx.in[1] && ctx.in[1]->rank() == 2) {
-            flops = 2.0 * static_cast<double>(ctx.in[0]->numel()) * static_cast<double>(ctx.in[1]->shape[1]);
+            // (weights of fused nodes are stored [n, k])
+            flops = 2.0 * static_cast<double>(ctx.in[0]->numel()) * static_cast<double>(ctx.in[1]->shape[0]);
         } else if (node.op == "rmlk.Attention" && ctx.in[0] && ctx.in[1] && ctx.in[0]->rank() == 4 &&
                    ctx.in[1]->rank() == 4) {
             // scores and context: 2 * [B, H, S, L, D] multiply-adds
             flops = 4.0 * static_cast<double>(ctx.in[0]->numel()) * static_cast<double>(ctx.in[1]->shape[2]);
         } else if (node.op == "rmlk.MatMulGroupSwiGLU" &&
-                   ctx.in[0] && ctx.in[1] && ctx.in[1]->rank() == 2 && ctx.in[1]->shape[0] > 0) {
+                   ctx.in[0] && ctx.in[1] && ctx.in[1]->rank() == 2 && ctx.in[1]->shape[1] > 0) {
             // rows of a times the whole weight matrix
-            flops = 2.0 * static_cast<double>(ctx.in[0]->numel()) / static_cast<double>(ctx.in[1]->shape[0]) *
+            flops = 2.0 * static_cast<double>(ctx.in[0]->numel()) / static_cast<double>(ctx.in[1]->shape[1]) *
                     static_cast<double>(ctx.in[1]->numel());
         }
         st.bytes = bytes;

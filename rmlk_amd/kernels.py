@@ -319,8 +319,9 @@ def gemv_kmajor_swiglu_normed(x, gamma, wt, y, n: int, k: int, gate_row: int, up
                                                    _ptr(y)), "rmlk_hip_gemv_kmajor_swiglu_normed")
 
 
-def matmul_grouped(a, b, outs, m: int, k: int, widths, workspace=None) -> None:
-    """outs[i] = a[m, k] . (the next widths[i] columns of the row-major joint matrix b)."""
+def matmul_grouped(a, b, outs, m: int, k: int, widths, workspace=None, trans_b: bool = False) -> None:
+    """outs[i] = a[m, k] . (the next widths[i] columns of the joint matrix b: row-major [k, sum], or with
+    trans_b K-contiguous [sum, k])."""
     n = len(widths)
     w = (ctypes.c_int64 * n)(*[int(x) for x in widths])
     need = int(lib().rmlk_hip_matmul_grouped_workspace_size(dtype_of(a), m, k, n, w))
@@ -329,15 +330,19 @@ def matmul_grouped(a, b, outs, m: int, k: int, widths, workspace=None) -> None:
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
     ptrs = (ctypes.c_void_p * n)(*[_ptr(o) for o in outs])
     check(lib().rmlk_hip_matmul_grouped(_stream(), dtype_of(a), m, k, _ptr(a), k, _ptr(b),
-                                        int(sum(widths)), n, w, ptrs, _ptr(workspace), ws_bytes),
+                                        k if trans_b else int(sum(widths)), int(trans_b), n, w, ptrs,
+                                        _ptr(workspace), ws_bytes),
           "rmlk_hip_matmul_grouped")
 
 
-def matmul_swiglu(a, b, out, m: int, n: int, k: int, ldb: int, gate_offset: int, up_offset: int) -> None:
-    """out[m, n] = swiglu(a . b[:, gate_offset:+n], a . b[:, up_offset:+n]); RmlkError with status
-    RMLK_ERR_UNSUPPORTED (-2) for shapes the one-launch kernel does not cover."""
+def matmul_swiglu(a, b, out, m: int, n: int, k: int, ldb: int, gate_offset: int, up_offset: int,
+                  trans_b: bool = False) -> None:
+    """out[m, n] = swiglu(a . b[:, gate_offset:+n], a . b[:, up_offset:+n]) (trans_b: b is [., k] and the
+    offsets count its rows); RmlkError with status RMLK_ERR_UNSUPPORTED (-2) for shapes the one-launch
+    kernel does not cover."""
     check(lib().rmlk_hip_matmul_swiglu(_stream(), dtype_of(a), m, n, k, _ptr(a), k, _ptr(b), ldb,
-                                       gate_offset, up_offset, _ptr(out), n), "rmlk_hip_matmul_swiglu")
+                                       int(trans_b), gate_offset, up_offset, _ptr(out), n),
+          "rmlk_hip_matmul_swiglu")
 
 
 def rotary(x, cos, sin, out, shape, x_stride, cos_stride, sin_stride) -> None:

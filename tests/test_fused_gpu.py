@@ -877,6 +877,22 @@ def test_grouped_matmul_matches_separate_products(device, m, k, widths):
             exp = a_np.astype(np.float64) @ b_np[:, off:off + w].astype(np.float64)
             assert_close(to_np(got), exp.astype(np.float32), rtol=1e-4, atol=1e-5)
         off += w
+    # the same over the K-contiguous form of the joint matrix: the members' rows instead of columns
+    if k % 4 == 0:
+        bt = to_dev(np.ascontiguousarray(b_np.T), device)
+        outs_t = [torch.full((m, w), float("nan"), device=device) for w in widths]
+        kk.matmul_grouped(a, bt, outs_t, m, k, widths, trans_b=True)
+        off = 0
+        for w, got_t, got in zip(widths, outs_t, outs):
+            if w:
+                sep = torch.empty(m, w, device=device)
+                kk.matmul(a, bt[off:off + w], sep, 1, m, w, k, k, k, w, 0, 0, 0, trans_b=True)
+                assert_close(to_np(got_t), to_np(sep), rtol=1e-4, atol=1e-5)
+                if m > 8:   # the tiled kernels add up in the same order for both forms of B
+                    assert_exact(to_np(got_t), to_np(got))
+                else:
+                    assert_close(to_np(got_t), to_np(got), rtol=1e-4, atol=1e-5)
+            off += w
 
 
 def test_grouped_matmul_argument_checks(device):
@@ -915,6 +931,11 @@ def test_matmul_swiglu_matches_separate_kernels(device, m, n, k, gate_first):
     u64 = a_np.astype(np.float64) @ b_np[:, uo:uo + n].astype(np.float64)
     exp = g64 / (1.0 + np.exp(-g64)) * u64
     assert_close(to_np(got), exp.astype(np.float32), rtol=1e-4, atol=1e-5)
+    # K-contiguous weights ([2n, k], gate and up rows): the same sums in the same order
+    bt = to_dev(np.ascontiguousarray(b_np.T), device)
+    got_t = torch.full((m, n), float("nan"), device=device)
+    kk.matmul_swiglu(a, bt, got_t, m, n, k, k, go, uo, trans_b=True)
+    assert_exact(to_np(got_t), to_np(got))
 
 
 @pytest.mark.parametrize("m,n,k", [(64, 8192, 256), (512, 8200, 256), (512, 128, 256), (512, 8192, 48),
@@ -928,6 +949,9 @@ def test_matmul_swiglu_declines_what_it_does_not_cover(device, m, n, k):
     out = torch.zeros(m, n, device=device)
     with pytest.raises(RmlkError) as e:
         kk.matmul_swiglu(a, b, out, m, n, k, 2 * n, 0, n)
+    assert e.value.status == -2
+    with pytest.raises(RmlkError) as e:
+        kk.matmul_swiglu(a, b.t().contiguous(), out, m, n, k, k, 0, n, trans_b=True)
     assert e.value.status == -2
 
 
@@ -1295,10 +1319,21 @@ def test_matmul_partials_feed_the_norm(device, m, n, k):
     assert need >= m * n * 4
     ws = torch.empty(need, dtype=torch.uint8, device=device)
     splits = ctypes.c_int32(0)
-    check(lib().rmlk_hip_matmul_partials(stream, kk.FLOAT, m, n, k, a.data_ptr(), k, w.data_ptr(), n,
+    check(lib().rmlk_hip_matmul_partials(stream, kk.FLOAT, m, n, k, a.data_ptr(), k, w.data_ptr(), n, 0,
                                          ws.data_ptr(), need, ctypes.byref(splits)),
           "rmlk_hip_matmul_partials")
     assert 1 <= splits.value and splits.value * m * n * 4 <= need
+    if k % 4 == 0:
+        # K-contiguous weights: the same slabs
+        wt = w.t().contiguous()
+        ws_t = torch.empty(need, dtype=torch.uint8, device=device)
+        splits_t = ctypes.c_int32(0)
+        check(lib().rmlk_hip_matmul_partials(stream, kk.FLOAT, m, n, k, a.data_ptr(), k, wt.data_ptr(), k, 1,
+                                             ws_t.data_ptr(), need, ctypes.byref(splits_t)),
+              "rmlk_hip_matmul_partials")
+        assert splits_t.value == splits.value
+        used = splits.value * m * n * 4
+        assert_exact(to_np(ws_t[:used]), to_np(ws[:used]))
     got_sum, got = torch.empty_like(res), torch.empty_like(res)
     check(lib().rmlk_hip_splitk_add_rmsnorm(stream, kk.FLOAT, m, n, ws.data_ptr(), splits.value, m * n,
                                             res.data_ptr(), gamma.data_ptr(), 1e-5, 0,
