@@ -1,0 +1,163 @@
+//! Chains of a decoder layer as single launches. None of them has a counterpart in the reference's
+//! kernel crate: a backend ported one to one never calls them; the session runtime of this
+//! repository (`include/rmlk_runtime.h`) forms them from the operator graph. Operands are raw
+//! device pointers here, since most of them are views into larger tensors (a KV cache, a row of a
+//! joint projection).
+use crate::device::{dims, HipStream};
+use crate::error::{check, Result};
+use crate::ffi;
+use std::os::raw::c_void;
+
+/// `out = x / sqrt(mean(x^2) + eps) * gamma` per row (`reciprocal_form`: `x * (1 / sqrt(..))`,
+/// the rounding of a graph that spells the norm with a Reciprocal-like Div).
+pub unsafe fn rmsnorm(
+    stream: &HipStream,
+    rows: usize,
+    cols: usize,
+    x: *const c_void,
+    gamma: *const c_void,
+    eps: f32,
+    reciprocal_form: bool,
+    out: *mut c_void,
+) -> Result<()> {
+    check(
+        ffi::rmlk_hip_rmsnorm(
+            stream.raw(),
+            ffi::RMLK_FLOAT,
+            rows as i64,
+            cols as i64,
+            x,
+            gamma,
+            eps,
+            reciprocal_form as i32,
+            out,
+        ),
+        "rmsnorm",
+    )
+}
+
+/// `sum_out = a + b`, `out = rmsnorm(sum_out)`.
+pub unsafe fn add_rmsnorm(
+    stream: &HipStream,
+    rows: usize,
+    cols: usize,
+    a: *const c_void,
+    b: *const c_void,
+    gamma: *const c_void,
+    eps: f32,
+    reciprocal_form: bool,
+    sum_out: *mut c_void,
+    out: *mut c_void,
+) -> Result<()> {
+    check(
+        ffi::rmlk_hip_add_rmsnorm(
+            stream.raw(),
+            ffi::RMLK_FLOAT,
+            rows as i64,
+            cols as i64,
+            a,
+            b,
+            gamma,
+            eps,
+            reciprocal_form as i32,
+            sum_out,
+            out,
+        ),
+        "add_rmsnorm",
+    )
+}
+
+/// `out = gate * sigmoid(gate) * up`.
+pub unsafe fn swiglu(stream: &HipStream, n: usize, gate: *const c_void, up: *const c_void, out: *mut c_void) -> Result<()> {
+    check(ffi::rmlk_hip_swiglu(stream.raw(), ffi::RMLK_FLOAT, n as i64, gate, up, out), "swiglu")
+}
+
+/// One-row product over K-contiguous weights: `y[n] = sum_k x[k] * wt[n][k]`.
+pub unsafe fn gemv_kmajor(
+    stream: &HipStream,
+    n: usize,
+    k: usize,
+    x: *const c_void,
+    wt: *const c_void,
+    ldw: usize,
+    y: *mut c_void,
+) -> Result<()> {
+    check(
+        ffi::rmlk_hip_gemv_kmajor(stream.raw(), ffi::RMLK_FLOAT, n as i64, k as i64, x, wt, ldw as i64, y),
+        "gemv_kmajor",
+    )
+}
+
+/// Shape of a grouped-query attention call.
+#[derive(Clone, Copy, Debug)]
+pub struct AttentionShape {
+    pub batch: usize,
+    pub kv_heads: usize,
+    /// Query heads per KV head.
+    pub rep: usize,
+    pub q_len: usize,
+    pub kv_len: usize,
+    pub head_dim: usize,
+}
+
+/// Bytes of workspace with which `attention` skips the key chunks a query tile cannot see
+/// (0: skipping does not apply to this shape and no workspace is needed).
+pub fn attention_workspace_size(shape: &AttentionShape, mask_stride: &[usize; 4]) -> Result<usize> {
+    let ms = dims(mask_stride)?;
+    Ok(unsafe {
+        ffi::rmlk_hip_attention_workspace_size(
+            ffi::RMLK_FLOAT,
+            shape.batch as i64,
+            shape.kv_heads as i64,
+            shape.rep as i64,
+            shape.q_len as i64,
+            shape.kv_len as i64,
+            shape.head_dim as i64,
+            &ms,
+        )
+    })
+}
+
+/// `Softmax(q . k^T (*|/) scale + mask) . v` over many query rows in one kernel; `workspace` may be
+/// null with 0 bytes.
+pub unsafe fn attention(
+    stream: &HipStream,
+    shape: &AttentionShape,
+    q: *const c_void,
+    k: *const c_void,
+    v: *const c_void,
+    mask: *const c_void,
+    mask_stride: &[usize; 4],
+    scale_is_mul: bool,
+    scale: f32,
+    out_seq_major: bool,
+    workspace: *mut c_void,
+    workspace_bytes: usize,
+    out: *mut c_void,
+) -> Result<()> {
+    let ms = dims(mask_stride)?;
+    check(
+        ffi::rmlk_hip_attention_ws(
+            stream.raw(),
+            ffi::RMLK_FLOAT,
+            shape.batch as i64,
+            shape.kv_heads as i64,
+            shape.rep as i64,
+            shape.q_len as i64,
+            shape.kv_len as i64,
+            shape.head_dim as i64,
+            q,
+            k,
+            v,
+            mask,
+            &ms,
+            scale_is_mul as i32,
+            scale,
+            out_seq_major as i32,
+            workspace,
+            workspace_bytes,
+            out,
+        ),
+        "attention",
+    )
+}
