@@ -42,11 +42,11 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # workspace; what their consumer (the combine kernel or the norm kernel) moves is not included.
 PMC_TRAFFIC_SOURCE = "profiles/gemm_mfma_llama1b_prefill512_hbm_traffic.md"
 PMC_TRAFFIC_KIB = {
-    (1, 512, 3072, 2048): ("mfma128x192x32 direct splitk=4", 32997, 24576),               # q/k/v
-    (1, 512, 2048, 2048): ("mfma128x64x32 direct splitk=4", 24677, 16384),                # o
-    (1, 512, 2048, 8192): ("mfma128x64x32 direct splitk=4", 99094, 16384),                # down
-    (1, 512, 16384, 2048, "swiglu"): ("mfma128x128x32 direct splitk=1", 164044, 16384),   # gate/up, SwiGLU epilogue
-    (1, 512, 128256, 2048): ("mfma128x128x32 direct splitk=1", 1522548, 256512),          # lm-head
+    (1, 512, 3072, 2048): ("mfma128x192x32 direct splitk=4", 32988, 24576),               # q/k/v
+    (1, 512, 2048, 2048): ("mfma128x64x32 direct splitk=4", 24675, 16384),                # o
+    (1, 512, 2048, 8192): ("mfma128x64x32 direct splitk=4", 98467, 16384),                # down
+    (1, 512, 16384, 2048, "swiglu"): ("mfma128x128x32 direct splitk=1", 164050, 16384),   # gate/up, SwiGLU epilogue
+    (1, 512, 128256, 2048): ("mfma128x128x32 direct splitk=1", 1493613, 256512),          # lm-head
 }
 
 
@@ -311,7 +311,7 @@ def run_llama(args):
 
 def time_matmul_launches(kernels, torch, shape_counts, reps=4, warm_reps=8):
     """Average duration (us) of rmlk_hip_matmul launches: for every (batch, m, n, k) -> count, `count`
-    launches with a broadcast 2-D weight operand taken in turn from enough distinct buffers to
+    launches with a broadcast 2-D K-contiguous weight operand taken in turn from enough distinct buffers to
     exceed the 256 MB Infinity Cache, all between one pair of HIP events on the current stream.
     `warm_reps` untimed repetitions come first: after the event-per-node pass (idle gaps) the chip
     needs some tens of milliseconds of continuous work before launch durations settle at what the
@@ -323,7 +323,7 @@ def time_matmul_launches(kernels, torch, shape_counts, reps=4, warm_reps=8):
         swiglu = len(shape) > 4
         a = torch.randn(batch, m, k, device=dev)
         nb = max(2, min(count, int(600e6 // (4 * k * n)) + 1))
-        bs = [torch.randn(k, n, device=dev) * 0.02 for _ in range(nb)]
+        bs = [torch.randn(n, k, device=dev) * 0.02 for _ in range(nb)]   # K-contiguous, as a session stores weights
         c = torch.empty(batch, m, n // 2 if swiglu else n, device=dev)
         need = kernels.matmul_workspace_size(batch, m, n, k)
         ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
@@ -334,10 +334,10 @@ def time_matmul_launches(kernels, torch, shape_counts, reps=4, warm_reps=8):
         for batch, m, n, k, swiglu, count, a, bs, c, ws in plans:
             for i in range(count):
                 if swiglu:
-                    kernels.matmul_swiglu(a, bs[i % len(bs)], c, m, n // 2, k, n, 0, n // 2)
+                    kernels.matmul_swiglu(a, bs[i % len(bs)], c, m, n // 2, k, k, 0, n // 2, trans_b=True)
                 else:
-                    kernels.matmul(a, bs[i % len(bs)], c, batch, m, n, k, k, n, n, m * k, 0, m * n,
-                                   workspace=ws)
+                    kernels.matmul(a, bs[i % len(bs)], c, batch, m, n, k, k, k, n, m * k, 0, m * n,
+                                   trans_b=True, workspace=ws)
     for _ in range(warm_reps):
         run_once()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
