@@ -433,6 +433,43 @@ def _rmsnorm_nodes(g, x, gamma, out, recip=False, axis=-1, expose_mean=False):
         g.output("mean")
 
 
+@pytest.mark.parametrize("rows", [1, 5, 200])
+def test_constant_weights_that_something_else_reads_stay_as_they_are(device, rows):
+    """Fused product nodes keep their weights K-contiguous and release the row-major initializer -
+    unless another node reads it, it is a graph output, or two products share it."""
+    from oracle import graph as og
+    k, n = 64, 128
+    rng = np.random.default_rng(rows)
+    g = _builder()
+    g.input("x", np.float32, [1, rows, k])
+    g.input("z", np.float32, [1, rows, k])
+    g.constant("w_shared", rng.standard_normal((k, n), dtype=np.float32) * np.float32(0.1))   # two products
+    g.constant("w_read", rng.standard_normal((k, n), dtype=np.float32) * np.float32(0.1))     # a product and an Add
+    g.constant("w_out", rng.standard_normal((k, n), dtype=np.float32) * np.float32(0.1))      # a product and a graph output
+    g.constant("w_q", rng.standard_normal((k, n), dtype=np.float32) * np.float32(0.1))        # a member of a group, and alone
+    g.constant("w_k", rng.standard_normal((k, 2 * n), dtype=np.float32) * np.float32(0.1))
+    g.constant("one", np.array(1.0, np.float32))
+    g.op("MatMul", ["x", "w_shared"], ["y_shared_x"])
+    g.op("MatMul", ["z", "w_shared"], ["y_shared_z"])
+    g.op("MatMul", ["x", "w_read"], ["y_read"])
+    g.op("Add", ["w_read", "one"], ["w_plus"])
+    g.op("MatMul", ["x", "w_out"], ["y_out"])
+    g.op("MatMul", ["z", "w_q"], ["y_q"])        # these two share `z` with each other and with w_shared's product
+    g.op("MatMul", ["z", "w_k"], ["y_k"])
+    g.op("MatMul", ["x", "w_q"], ["y_q_alone"])
+    for name in ("y_shared_x", "y_shared_z", "y_read", "w_plus", "y_out", "w_out", "y_q", "y_k", "y_q_alone"):
+        g.output(name)
+    feeds = {"x": rng.standard_normal((1, rows, k), dtype=np.float32),
+             "z": rng.standard_normal((1, rows, k), dtype=np.float32)}
+    a, b, nf, ops = _run_both(g.build(), feeds)
+    assert nf >= 2     # the products on x form one joint node, those on z another
+    loose = {"y_shared_x", "y_shared_z", "y_read", "y_out", "y_q", "y_k", "y_q_alone"} if rows <= 8 else set()
+    _same(a, b, loose=loose)     # many rows: the same sums in the same order over either form of the weights
+    exp = og.run_graph(g.build(), feeds)
+    for name in exp:
+        assert_close(a[name], exp[name], rtol=1e-4, atol=1e-5)
+
+
 @pytest.mark.parametrize("rows,k,n,recip", [
     (1, 256, 96, False),       # one row: the norm is left to the product's kernel
     (1, 256, 96, True),
