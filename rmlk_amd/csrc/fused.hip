@@ -109,48 +109,57 @@ __global__ __launch_bounds__(kBlock) void splitk_swiglu_kernel(const float *__re
 // Rotary embedding over x [B,H,S,D] read through element strides (the innermost stride is 1), so a
 // [B,S,H,D] projection output is rotated and laid out [B,H,S,D] in the same pass. One lane takes W
 // neighbouring elements of the first half of a row together with their partners in the second half.
+// OFF: the type of element offsets - 32-bit when every operand ends below 2^31 elements (64-bit
+// multiplies per dim and operand were most of the kernel's arithmetic). One trip: the grid covers
+// the rows; x and the result stream past the caches, the tables (shared by the heads) stay in them.
+template <typename OFF>
 struct RotaryArgs {
     const float *x, *cos, *sin;
     float *out;
     FastDiv div_s, div_h, div_q;     // S, H, lanes per row
     uint32_t n_s, n_h, n_q, half;
-    int64_t xs[3], cs[3], ss[3];     // strides of (b, h, s)
+    OFF xs[3], cs[3], ss[3];         // strides of (b, h, s)
     uint32_t total;                  // B * H * S * n_q
 };
 
-template <int W>
-__global__ __launch_bounds__(kBlock) void rotary_kernel(RotaryArgs a) {
+template <int W, typename OFF>
+__global__ __launch_bounds__(kBlock) void rotary_kernel(RotaryArgs<OFF> a) {
     using V = Vec<float, W>;
-    for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t < a.total; t += gridDim.x * kBlock) {
-        const uint32_t row = a.div_q.div(t), q = t - row * a.n_q;
-        const uint32_t bh = a.div_s.div(row), s = row - bh * a.n_s;
-        const uint32_t b = a.div_h.div(bh), h = bh - b * a.n_h;
-        const int64_t xo = b * a.xs[0] + h * a.xs[1] + s * a.xs[2];
-        const int64_t co = b * a.cs[0] + h * a.cs[1] + s * a.cs[2];
-        const int64_t so = b * a.ss[0] + h * a.ss[1] + s * a.ss[2];
-        const uint32_t d = q * W;
-        const V x1 = *reinterpret_cast<const V *>(a.x + xo + d);
-        const V x2 = *reinterpret_cast<const V *>(a.x + xo + d + a.half);
-        const V c1 = *reinterpret_cast<const V *>(a.cos + co + d);
-        const V c2 = *reinterpret_cast<const V *>(a.cos + co + d + a.half);
-        const V s1 = *reinterpret_cast<const V *>(a.sin + so + d);
-        const V s2 = *reinterpret_cast<const V *>(a.sin + so + d + a.half);
-        V y1, y2;
+    // (Four positions per lane, a quarter of the work apart, with all loads of x in front: 16.9 us
+    // against the 15.0 us of one position per lane - the index arithmetic per position outweighs
+    // what the deeper queue of loads gains.)
+    const uint32_t t0 = blockIdx.x * kBlock + threadIdx.x;
+    const bool live = t0 < a.total;
+    const uint32_t t = live ? t0 : 0;     // (a lane past the end repeats lane 0's loads and stores nothing)
+    const uint32_t row = a.div_q.div(t), q = t - row * a.n_q;
+    const uint32_t bh = a.div_s.div(row), s = row - bh * a.n_s;
+    const uint32_t b = a.div_h.div(bh), h = bh - b * a.n_h;
+    const OFF xo = b * a.xs[0] + h * a.xs[1] + s * a.xs[2];
+    const OFF co = b * a.cs[0] + h * a.cs[1] + s * a.cs[2];
+    const OFF so = b * a.ss[0] + h * a.ss[1] + s * a.ss[2];
+    const uint32_t d = q * W;
+    const V x1 = nt_load(reinterpret_cast<const V *>(a.x + xo + d));
+    const V x2 = nt_load(reinterpret_cast<const V *>(a.x + xo + d + a.half));
+    const V c1 = *reinterpret_cast<const V *>(a.cos + co + d);
+    const V c2 = *reinterpret_cast<const V *>(a.cos + co + d + a.half);
+    const V s1 = *reinterpret_cast<const V *>(a.sin + so + d);
+    const V s2 = *reinterpret_cast<const V *>(a.sin + so + d + a.half);
+    V y1, y2;
 #pragma unroll
-        for (int j = 0; j < W; ++j) {
-            const float a1 = x1.v[j] * c1.v[j];
-            const float r1 = (-x2.v[j]) * s1.v[j];
-            y1.v[j] = a1 + r1;
-            const float a2 = x2.v[j] * c2.v[j];
-            const float r2 = x1.v[j] * s2.v[j];
-            y2.v[j] = a2 + r2;
-        }
+    for (int j = 0; j < W; ++j) {
+        const float a1 = x1.v[j] * c1.v[j];
+        const float r1 = (-x2.v[j]) * s1.v[j];
+        y1.v[j] = a1 + r1;
+        const float a2 = x2.v[j] * c2.v[j];
+        const float r2 = x1.v[j] * s2.v[j];
+        y2.v[j] = a2 + r2;
+    }
+    if (live) {
         float *o = a.out + static_cast<int64_t>(row) * (2 * a.half) + d;
-        *reinterpret_cast<V *>(o) = y1;
-        *reinterpret_cast<V *>(o + a.half) = y2;
+        nt_store(reinterpret_cast<V *>(o), y1);
+        nt_store(reinterpret_cast<V *>(o + a.half), y2);
     }
 }
-
 
 // Up to kMaxRowStreams independent streams of head rows in ONE launch (blockIdx.y picks the stream):
 // each reads rows of D elements through strides over (b, h, s) like rotary_kernel, rotates them
@@ -334,29 +343,42 @@ extern "C" int32_t rmlk_hip_rotary(rmlk_stream_t stream, int32_t dtype, const rm
     const int w = ok(4) ? 4 : ok(2) ? 2 : 1;
     const int64_t total = rows * (half / w);
     if (total >= ((int64_t)1 << 31) || numel >= ((int64_t)1 << 32)) return RMLK_ERR_TOO_LARGE;
-    RotaryArgs a;
-    a.x = static_cast<const float *>(x);
-    a.cos = static_cast<const float *>(cos);
-    a.sin = static_cast<const float *>(sin);
-    a.out = static_cast<float *>(out);
-    a.n_s = static_cast<uint32_t>(shape->v[2]);
-    a.n_h = static_cast<uint32_t>(shape->v[1]);
-    a.n_q = static_cast<uint32_t>(half / w);
-    a.half = static_cast<uint32_t>(half);
-    a.div_s = FastDiv(a.n_s);
-    a.div_h = FastDiv(a.n_h);
-    a.div_q = FastDiv(a.n_q);
-    for (int i = 0; i < 3; ++i) {
-        a.xs[i] = x_stride->v[i];
-        a.cs[i] = cos_stride->v[i];
-        a.ss[i] = sin_stride->v[i];
-    }
-    a.total = static_cast<uint32_t>(total);
+    // the last element an operand's strides reach
+    auto reach = [&](const rmlk_dims *st) {
+        int64_t r = d;
+        for (int i = 0; i < 3; ++i) r += (shape->v[i] - 1) * st->v[i];
+        return r;
+    };
+    const bool narrow = reach(x_stride) < (1ll << 31) && reach(cos_stride) < (1ll << 31) &&
+                        reach(sin_stride) < (1ll << 31);
     hipStream_t s = as_stream(stream);
-    const unsigned grid = grid_for(total, kBlock, 16);
-    if (w == 4) rotary_kernel<4><<<grid, kBlock, 0, s>>>(a);
-    else if (w == 2) rotary_kernel<2><<<grid, kBlock, 0, s>>>(a);
-    else rotary_kernel<1><<<grid, kBlock, 0, s>>>(a);
+    const unsigned grid = static_cast<unsigned>((total + kBlock - 1) / kBlock);   // one trip
+    auto launch = [&](auto off_tag) {
+        using OFF = decltype(off_tag);
+        RotaryArgs<OFF> a;
+        a.x = static_cast<const float *>(x);
+        a.cos = static_cast<const float *>(cos);
+        a.sin = static_cast<const float *>(sin);
+        a.out = static_cast<float *>(out);
+        a.n_s = static_cast<uint32_t>(shape->v[2]);
+        a.n_h = static_cast<uint32_t>(shape->v[1]);
+        a.n_q = static_cast<uint32_t>(half / w);
+        a.half = static_cast<uint32_t>(half);
+        a.div_s = FastDiv(a.n_s);
+        a.div_h = FastDiv(a.n_h);
+        a.div_q = FastDiv(a.n_q);
+        for (int i = 0; i < 3; ++i) {
+            a.xs[i] = static_cast<OFF>(x_stride->v[i]);
+            a.cs[i] = static_cast<OFF>(cos_stride->v[i]);
+            a.ss[i] = static_cast<OFF>(sin_stride->v[i]);
+        }
+        a.total = static_cast<uint32_t>(total);
+        if (w == 4) rotary_kernel<4, OFF><<<grid, kBlock, 0, s>>>(a);
+        else if (w == 2) rotary_kernel<2, OFF><<<grid, kBlock, 0, s>>>(a);
+        else rotary_kernel<1, OFF><<<grid, kBlock, 0, s>>>(a);
+    };
+    if (narrow) launch(uint32_t{});
+    else launch(int64_t{});
     return launch_status();
 }
 
