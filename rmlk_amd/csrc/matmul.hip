@@ -1376,6 +1376,13 @@ inline TileChoice choose_tiles(int64_t batch, int64_t m, int64_t n, int64_t k, b
             t.bn = 192;
             t.splits = splits_w;
             t.k_per_split = kps_w;
+            // the same blocks as half-width tiles with half the split: half the partial sums to
+            // write and to add up again, twice the K steps per block behind one prologue
+            if (splits_w % 2 == 0 && n % 96 == 0 && tiles(128, 96) * (splits_w / 2) <= kNumCU) {
+                t.bn = 96;
+                t.splits = splits_w / 2;
+                t.k_per_split = kps_w * 2;
+            }
         }
     }
     // split-K products whose 128 x 128 tiles give one block per CU: 128 x 64 tiles with the same
@@ -1457,7 +1464,7 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
                k % c.k_per_split == 0 && (trans_b || n % 4 == 0) && lda < (1ll << 21) && ldb < (1ll << 21);
     };
     TileChoice t = choose_tiles(batch, m, n, k);
-    if ((t.bn == 192 || (t.bm == 128 && t.bn == 64)) && !direct_ok(t)) t = choose_tiles(batch, m, n, k, false);
+    if ((t.bn == 192 || t.bn == 96 || (t.bm == 128 && t.bn == 64)) && !direct_ok(t)) t = choose_tiles(batch, m, n, k, false);
     GemmArgs g{};
     g.a = pa;
     g.b = pb;
@@ -1524,6 +1531,7 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
     }
     if (direct && t.bm == 256) st = RMLK_DIRECT(256, 64, 64, 64);
     else if (direct && t.bn == 192) st = RMLK_DIRECT(128, 192, 64, 96);
+    else if (direct && t.bn == 96) st = RMLK_DIRECT(128, 96, 32, 96);
     else if (direct && t.bm == 128 && t.bn == 64) st = RMLK_DIRECT(128, 64, 64, 32);
     else if (direct && t.bm == 128) st = RMLK_DIRECT(128, 128, 64, 64);
     else if (direct) st = RMLK_DIRECT(64, 64, 32, 32);
@@ -1652,7 +1660,7 @@ extern "C" int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_
             return c.bk == 32 && k % 4 == 0 && n % 4 == 0 && c.k_per_split % c.bk == 0 &&
                    k % c.k_per_split == 0;
         };
-        if ((t.bn == 192 || (t.bm == 128 && t.bn == 64)) && !direct_ok(t)) t = choose_tiles(batch, m, n, k, false);
+        if ((t.bn == 192 || t.bn == 96 || (t.bm == 128 && t.bn == 64)) && !direct_ok(t)) t = choose_tiles(batch, m, n, k, false);
         const bool direct = direct_ok(t);
         snprintf(tmp, sizeof(tmp), "mfma%dx%dx%d%s splitk=%d", t.bm, t.bn, t.bk,
                  direct ? " direct" : "", t.splits);
