@@ -1011,7 +1011,10 @@ struct NoExtraLoads {
 };
 // `extra_loads()` is called once the first chunk of weights has been requested: loads an epilogue
 // needs, on their way with the weights but not in front of the row (loads return in order).
-template <int COLS, bool NORM, typename Extra = NoExtraLoads>
+// NU: 128-bit units of the row a lane holds during the NORM prologue (k <= 256 * NU * 4); the
+// common k <= 2048 takes NU = 2 and with it 48 registers less than NU = 8, i.e. five or six
+// resident wavefronts per SIMD instead of four.
+template <int COLS, bool NORM, int NU = kGemvNormUnits, typename Extra = NoExtraLoads>
 __device__ __forceinline__ void gemv_wave_dots(const float *__restrict__ x, const v4f *const (&wv)[COLS],
                                                int32_t k, const RowNormArgs &norm, bool active,
                                                float (&acc)[COLS], Extra extra_loads = Extra()) {
@@ -1023,11 +1026,11 @@ __device__ __forceinline__ void gemv_wave_dots(const float *__restrict__ x, cons
     const int k4 = k / 4;
     const v4f *xv = reinterpret_cast<const v4f *>(x);
     // NORM: this lane's share of the row and of gamma, requested before any weight
-    [[maybe_unused]] v4f xn[kGemvNormUnits], gn[kGemvNormUnits];
+    [[maybe_unused]] v4f xn[NU], gn[NU];
     if constexpr (NORM) {
         const v4f *gv = reinterpret_cast<const v4f *>(norm.gamma);
 #pragma unroll
-        for (int i = 0; i < kGemvNormUnits; ++i) {
+        for (int i = 0; i < NU; ++i) {
             const int c = threadIdx.x + i * kThreads;
             if (i * kThreads < k4) {             // (uniform)
                 xn[i] = xv[min(c, k4 - 1)];
@@ -1064,7 +1067,7 @@ __device__ __forceinline__ void gemv_wave_dots(const float *__restrict__ x, cons
     if constexpr (NORM) {
         double sq_sum = 0.0;
 #pragma unroll
-        for (int i = 0; i < kGemvNormUnits; ++i) {
+        for (int i = 0; i < NU; ++i) {
             if (i * kThreads < k4) {
                 const bool live = threadIdx.x + i * kThreads < k4;
 #pragma unroll
@@ -1086,7 +1089,7 @@ __device__ __forceinline__ void gemv_wave_dots(const float *__restrict__ x, cons
         const float r = sqrtf(var);
         const float inv = 1.0f / r;
 #pragma unroll
-        for (int i = 0; i < kGemvNormUnits; ++i) {
+        for (int i = 0; i < NU; ++i) {
             const int c = threadIdx.x + i * kThreads;
             if (c < k4) {
                 v4f v = xn[i];
@@ -1138,7 +1141,7 @@ __device__ __forceinline__ void gemv_wave_dots(const float *__restrict__ x, cons
     for (int c = 0; c < COLS; ++c) acc[c] = wave_sum(acc[c]);
 }
 
-template <bool SWIGLU = false, bool NORM = false>
+template <bool SWIGLU = false, bool NORM = false, int NU = kGemvNormUnits>
 __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__restrict__ x,
                                                           const float *__restrict__ wt,
                                                           float *__restrict__ y, int32_t n, int32_t k,
@@ -1160,7 +1163,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__re
     const v4f *wv[1];
     wv[0] = reinterpret_cast<const v4f *>(wt + row * ldw);
     float acc[1];
-    gemv_wave_dots<1, NORM>(x, wv, k, norm, col < n, acc);
+    gemv_wave_dots<1, NORM, NU>(x, wv, k, norm, col < n, acc);
     if constexpr (SWIGLU) {
         if (lane == 0) pair_acc[wave] = acc[0];
         __syncthreads();
@@ -1198,7 +1201,7 @@ struct GemvRowStreams {
     int32_t *err;
 };
 
-template <bool NORM>
+template <bool NORM, int NU = kGemvNormUnits>
 __global__ __launch_bounds__(kThreads) void gemv_kmajor_rows_kernel(const float *__restrict__ x,
                                                                     const float *__restrict__ wt, int32_t k,
                                                                     int64_t ldw, RowNormArgs norm,
@@ -1245,7 +1248,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_rows_kernel(const float 
         }
     };
     float acc[1];
-    gemv_wave_dots<1, NORM>(x, wv, k, norm, active, acc, epilogue_loads);
+    gemv_wave_dots<1, NORM, NU>(x, wv, k, norm, active, acc, epilogue_loads);
     if (lane == 0) pair_acc[wave] = acc[0];
     __syncthreads();
     if (!active || lane != 0 || second) return;
@@ -1994,7 +1997,10 @@ int32_t gemv_kmajor_launch(rmlk_stream_t stream, int32_t dtype, int64_t n, int64
     constexpr int kWaves = kThreads / kWave;
     const int32_t ni = static_cast<int32_t>(n), ki = static_cast<int32_t>(k);
     const unsigned grid = static_cast<unsigned>((n + kWaves - 1) / kWaves);
-    if (norm) gemv_kmajor_kernel<false, true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
+    if (norm && k <= kThreads * 4 * 2)
+        gemv_kmajor_kernel<false, true, 2><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
+    else if (norm)
+        gemv_kmajor_kernel<false, true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
     else gemv_kmajor_kernel<><<<grid, kThreads, 0, s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, RowNormArgs{});
     return launch_status();
 }
@@ -2020,7 +2026,10 @@ int32_t gemv_kmajor_swiglu_launch(rmlk_stream_t stream, int32_t dtype, int64_t n
     float *py = static_cast<float *>(y);
     const int32_t ni = static_cast<int32_t>(n), ki = static_cast<int32_t>(k);
     const int32_t gr = static_cast<int32_t>(gate_row), ur = static_cast<int32_t>(up_row);
-    if (norm)
+    if (norm && k <= kThreads * 4 * 2)
+        gemv_kmajor_kernel<true, true, 2><<<grid, kThreads, k * sizeof(float), as_stream(stream)>>>(
+            px, pw, py, ni, ki, ldw, gr, ur, nullptr, *norm);
+    else if (norm)
         gemv_kmajor_kernel<true, true><<<grid, kThreads, k * sizeof(float), as_stream(stream)>>>(
             px, pw, py, ni, ki, ldw, gr, ur, nullptr, *norm);
     else
@@ -2108,7 +2117,10 @@ extern "C" int32_t rmlk_hip_gemv_kmajor_head_rows(rmlk_stream_t stream, int32_t 
     hipStream_t s = as_stream(stream);
     if (gamma) {
         const RowNormArgs norm{static_cast<const float *>(gamma), eps, reciprocal_form};
-        gemv_kmajor_rows_kernel<true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
+        if (k <= kThreads * 4 * 2)
+            gemv_kmajor_rows_kernel<true, 2><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
+        else
+            gemv_kmajor_rows_kernel<true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
     } else {
         gemv_kmajor_rows_kernel<false><<<grid, kThreads, 0, s>>>(px, pw, ki, ldw, RowNormArgs{}, rs);
     }
