@@ -1152,6 +1152,46 @@ def test_attention_skipping_hidden_chunks_is_bit_identical(device, b, g, rep, s,
         assert np.isnan(out[0, 64:128, 0]).all() and np.isfinite(out[0, :64, 0]).all()
 
 
+def test_attention_workspace_that_is_too_small_is_not_used(device):
+    """A workspace below the size the library names is ignored (every chunk is visited): nothing is
+    written to it and the result is the plain kernel's."""
+    import torch
+    from rmlk_amd._lib import check, lib
+    from rmlk_amd.kernels import Dims
+    kk = _k()
+    b, g, rep, s, l, d = 1, 8, 4, 1024, 1024, 64
+    rng = np.random.default_rng(5)
+    q, k, v = (to_dev(rng.standard_normal(sh, dtype=np.float32), device)
+               for sh in ((b, g * rep, s, d), (b, g, l, d), (b, g, l, d)))
+    m = to_dev(_skipping_mask("causal", rng, (1, 1, s, l), l), device)
+    ms = Dims.of([0, 0, l, 1])
+    need = int(lib().rmlk_hip_attention_workspace_size(kk.FLOAT, b, g, rep, s, l, d, ms))
+    assert need > 16
+    exp = torch.empty(b, g * rep, s, d, device=device)
+    kk.attention(q, k, v, m, exp, b, g, rep, s, l, d, [0, 0, l, 1], 8.0)
+    ws = torch.full((need,), 7, dtype=torch.uint8, device=device)
+    got = torch.empty_like(exp)
+    stream = torch.cuda.current_stream().cuda_stream
+    check(lib().rmlk_hip_attention_ws(stream, kk.FLOAT, b, g, rep, s, l, d, q.data_ptr(), k.data_ptr(),
+                                      v.data_ptr(), m.data_ptr(), ms, 0, 8.0, 0, ws.data_ptr(), need - 1,
+                                      got.data_ptr()), "rmlk_hip_attention_ws")
+    assert_exact(to_np(got), to_np(exp))
+    assert (to_np(ws) == 7).all()
+
+
+def test_attention_few_rows_one_launch_needs_its_counters(device):
+    import torch
+    from rmlk_amd import RmlkError
+    kk = _k()
+    q = torch.zeros(1, 8, 1, 64, device=device)
+    k = torch.zeros(1, 2, 64, 64, device=device)
+    m = torch.zeros(1, 64, device=device)
+
+    with pytest.raises(RmlkError):
+        kk.attention_few_rows_one_launch(q, k, k, m, torch.zeros_like(q), None, 1, 2, 4, 1, 64, 64,
+                                         [0, 0, 0, 1], 8.0)
+
+
 def test_attention_skipped_chunks_do_not_read_their_keys(device):
     """What the skipped chunks hold never reaches the output: NaN in K and V rows no query of a tile
     sees leaves that tile finite (the kernel without the map gives 0 * NaN there)."""
