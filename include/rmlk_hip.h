@@ -494,6 +494,11 @@ typedef struct rmlk_row_stream {
     const int64_t *idx;     /* NULL: dense output */
     int32_t tuple_size;     /* read only when idx is given */
     rmlk_dims data_shape;
+    int32_t partials;       /* > 1 (rmlk_hip_head_rows only): x is the sum, in ascending order, of this
+                               many matrices that lie partial_stride elements apart, the first at x -
+                               the partial sums of a split-K product (rmlk_hip_matmul_partials) whose
+                               combine launch this saves; 0 or 1: x itself */
+    int64_t partial_stride;
 } rmlk_row_stream;
 int32_t rmlk_hip_head_rows(rmlk_stream_t stream, int32_t dtype, int32_t n_streams,
                            const rmlk_row_stream *streams, int32_t *err_flag);

@@ -43,7 +43,8 @@ class RowStream(ctypes.Structure):
     """struct rmlk_row_stream"""
     _fields_ = [("shape", Dims), ("x_stride", Dims), ("x", c_void_p), ("cos", c_void_p),
                 ("sin", c_void_p), ("cos_stride", Dims), ("sin_stride", Dims), ("out", c_void_p),
-                ("idx", c_void_p), ("tuple_size", c_int32), ("data_shape", Dims)]
+                ("idx", c_void_p), ("tuple_size", c_int32), ("data_shape", Dims),
+                ("partials", c_int32), ("partial_stride", c_int64)]
 
 
 class DeviceInfo(ctypes.Structure):

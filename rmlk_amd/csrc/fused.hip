@@ -179,6 +179,8 @@ struct RowStream {
     uint32_t n_s, n_h;
     uint32_t total;                  // B * H * S * n_q
     int32_t tuple_size;
+    int32_t partials;                // x is the sum of this many slabs (split-K partial sums); <= 1: x itself
+    int64_t partial_stride;          // elements from one slab to the next
     int64_t xs[3], cs[3], ss[3];     // strides of (b, h, s)
     int64_t dim[kMaxRowTuple], stride[kMaxRowTuple];   // leading dims of the scatter destination, in rows
 };
@@ -208,8 +210,20 @@ __global__ __launch_bounds__(kBlock) void head_rows_kernel(RowStreams all) {
             for (int k = 0; k < kMaxRowTuple; ++k)
                 ix[k] = k < a.tuple_size ? a.idx[static_cast<int64_t>(row) * a.tuple_size + k] : 0;
         }
-        const V x1 = *reinterpret_cast<const V *>(a.x + xo + d);
-        const V x2 = *reinterpret_cast<const V *>(a.x + xo + d + all.half);
+        V x1 = *reinterpret_cast<const V *>(a.x + xo + d);
+        V x2 = *reinterpret_cast<const V *>(a.x + xo + d + all.half);
+        // the rows of a split-K product that was not added up: slab 0 + slab 1 + .., in that order
+        // (the order of the combine kernel this replaces)
+        for (int z = 1; z < a.partials; ++z) {
+            const float *pz = a.x + z * a.partial_stride + xo + d;
+            const V p1 = *reinterpret_cast<const V *>(pz);
+            const V p2 = *reinterpret_cast<const V *>(pz + all.half);
+#pragma unroll
+            for (int j = 0; j < W; ++j) {
+                x1.v[j] += p1.v[j];
+                x2.v[j] += p2.v[j];
+            }
+        }
         V y1 = x1, y2 = x2;
         if (a.cos) {
             const int64_t co = b * a.cs[0] + h * a.cs[1] + s * a.cs[2];
@@ -453,6 +467,13 @@ extern "C" int32_t rmlk_hip_head_rows(rmlk_stream_t stream, int32_t dtype, int32
             a.ss[k] = rotate ? in.sin_stride.v[k] : 0;
         }
         a.tuple_size = in.idx ? in.tuple_size : 0;
+        if (in.partials < 0 || in.partials > 64 || (in.partials > 1 && in.partial_stride <= 0))
+            return RMLK_ERR_INVALID_ARGUMENT;
+        if (in.partials > 1 && in.partial_stride % w) {
+            while (w > 1 && in.partial_stride % w) w /= 2;
+        }
+        a.partials = in.partials;
+        a.partial_stride = in.partial_stride;
         int64_t stride = 1;
         for (int k = a.tuple_size - 1; k >= 0; --k) {
             a.dim[k] = in.data_shape.v[k];

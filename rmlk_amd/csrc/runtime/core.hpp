@@ -133,6 +133,17 @@ struct PendingProduct {
     Tensor row;                                 // where the product goes when it has to be stored
     int64_t k = 0, total = 0;
     bool computed = false;                      // stored in `row`, or consumed by the fused launch
+    // Many rows (m > 0): the product HAS run, but its split-K partial sums were not added up -
+    // `slabs` holds `splits` matrices [m, total], `slab` elements apart; `outs` are the members'
+    // (dense, still unwritten) outputs in the order of their column blocks `widths`. The row-stream
+    // node reads its rows from the slabs and adds them up on the way; `x` is kept for the case
+    // that the members have to be written after all.
+    int64_t m = 0;
+    Tensor slabs;
+    int32_t splits = 0;
+    int64_t slab = 0;
+    std::vector<int64_t> widths;
+    std::vector<Tensor> outs;
 };
 
 rmlk_dims to_dims(const std::vector<int64_t> &v);          // rank-0 becomes [1]

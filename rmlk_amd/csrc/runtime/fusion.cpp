@@ -1182,6 +1182,20 @@ void op_fused_rotary(OpContext &c) {
 
 // A one-row product that was left to its reader and has to be stored after all.
 void store_product(OpContext &c, PendingProduct &pp) {
+    if (pp.m > 0) {
+        // many rows, partial sums not added up: the members' outputs by the grouped product
+        std::vector<void *> outs;
+        for (Tensor &t : pp.outs) outs.push_back(t.data());
+        const size_t ws_bytes = rmlk_hip_matmul_grouped_workspace_size(
+            RMLK_FLOAT, pp.m, pp.k, static_cast<int32_t>(pp.widths.size()), pp.widths.data());
+        void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
+        check_status(rmlk_hip_matmul_grouped(c.stream, RMLK_FLOAT, pp.m, pp.k, pp.x.data(), pp.k, pp.wt.data(),
+                                             pp.k, 1, static_cast<int32_t>(pp.widths.size()), pp.widths.data(),
+                                             outs.data(), ws, ws_bytes),
+                     "rmlk.MatMulGroup (deferred)");
+        pp.computed = true;
+        return;
+    }
     int32_t st;
     if (pp.norm)
         st = rmlk_hip_gemv_kmajor_normed(c.stream, RMLK_FLOAT, pp.total, pp.k, pp.x.data(), pp.norm->gamma.data(),
@@ -1256,7 +1270,8 @@ void op_fused_head_rows(OpContext &c) {
     // product and a [1, H, 1, D] tensor with its heads side by side; otherwise the product is
     // computed first, and everything below finds its rows in memory.
     std::shared_ptr<PendingProduct> product;
-    bool one_launch = ok;
+    bool one_launch = ok, from_slabs = false;
+    std::vector<int64_t> slab_col(n, 0);
     {
         std::vector<std::shared_ptr<PendingProduct>> seen;
         int at_src = 0;
@@ -1275,7 +1290,31 @@ void op_fused_head_rows(OpContext &c) {
             }
         }
         if (seen.size() != 1) one_launch = false;
-        if (one_launch) {
+        // a many-row product whose partial sums were left in their slabs: every source is a member
+        // of it, seen as [B, S, H, D] rows of the joint matrix
+        if (ok && seen.size() == 1 && seen[0]->m > 0) {
+            const PendingProduct &pp = *seen[0];
+            from_slabs = true;
+            int at_m = 0;
+            for (size_t i = 0; i < n && from_slabs; ++i) {
+                const Tensor &src = c.input(at_m);
+                at_m += kinds[i] == 2 ? 3 : (kinds[i] == 1 ? 5 : 3);
+                int member = -1;
+                int64_t col = 0;
+                for (size_t j = 0; j < pp.outs.size(); ++j) {
+                    if (src.pending_product && pp.outs[j].buf == src.buf && pp.outs[j].offset == src.offset) {
+                        member = static_cast<int>(j);
+                        break;
+                    }
+                    col += pp.widths[j];
+                }
+                from_slabs = member >= 0 && pre[i] != 0 && src.rank() == 4 &&
+                             src.shape[0] * src.shape[1] == pp.m && src.shape[2] * src.shape[3] == pp.widths[member];
+                slab_col[i] = col;
+            }
+            one_launch = false;
+        }
+        if (one_launch || from_slabs) {
             product = seen[0];
         } else {
             for (const std::shared_ptr<PendingProduct> &pp : seen) store_product(c, *pp);
@@ -1291,11 +1330,20 @@ void op_fused_head_rows(OpContext &c) {
         rmlk_row_stream &st = streams[i];
         st = rmlk_row_stream{};
         int in = first_input[i];
-        if (product)
+        if (product && !from_slabs)
             first_col[i] = static_cast<int64_t>(c.input(in).offset - product->row.offset) / static_cast<int64_t>(sizeof(float));
         st.shape = to_dims(lay[i].shape);
         st.x_stride = to_dims(lay[i].xst);
         st.x = c.input(in++).data();
+        if (from_slabs) {
+            // logical [B, H, S, D] over the rows (b, s) of the joint matrix, `total` columns wide
+            const PendingProduct &pp = *product;
+            const int64_t seq = lay[i].shape[2], d = lay[i].shape[3];
+            st.x_stride = to_dims({seq * pp.total, d, pp.total, 1});
+            st.x = static_cast<const float *>(pp.slabs.data()) + slab_col[i];
+            st.partials = pp.splits;
+            st.partial_stride = pp.slab;
+        }
         if (kinds[i] != 2) {
             st.cos = c.input(in++).data();
             st.sin = c.input(in++).data();
@@ -1312,7 +1360,22 @@ void op_fused_head_rows(OpContext &c) {
             st.out = scatter_destination(c, in, static_cast<int>(i)).data();
         }
     }
-    if (product) {
+    if (product && from_slabs) {
+        if (took_fast_path(rmlk_hip_head_rows(c.stream, RMLK_FLOAT, static_cast<int32_t>(n), streams.data(),
+                                              c.error_flag()),
+                           "rmlk.HeadRows (over partial sums)")) {
+            product->computed = true;   // consumed: nothing else reads its members
+            return;
+        }
+        // the kernel refuses these operands: the members stored after all, then the streams over them
+        store_product(c, *product);
+        for (size_t i = 0; i < n; ++i) {
+            streams[i].x = c.input(first_input[i]).data();
+            streams[i].x_stride = to_dims(lay[i].xst);
+            streams[i].partials = 0;
+            streams[i].partial_stride = 0;
+        }
+    } else if (product) {
         const PendingProduct &pp = *product;
         const int32_t st = rmlk_hip_gemv_kmajor_head_rows(
             c.stream, RMLK_FLOAT, pp.k, pp.x.data(), pp.norm ? pp.norm->gamma.data() : nullptr,
@@ -1688,6 +1751,41 @@ void op_fused_matmul_group(OpContext &c) {
             product_over_kmajor(c, a1.data(), 1, k, wt.data(), total, row.data(), "rmlk.MatMulGroup");
         hand_out(nullptr);
         return;
+    }
+    if (widths.size() <= 4 && c.attr_int("defer_product", 0) != 0) {
+        // Everything that reads the members is one row-stream node: the product runs now, but its
+        // split-K partial sums stay where they are - that node adds them up while it reads its rows,
+        // which saves the combine launch and a round trip of the product through memory.
+        const size_t bytes = rmlk_hip_matmul_partials_workspace_size(RMLK_FLOAT, m, total, k);
+        if (bytes) {
+            auto pp = std::make_shared<PendingProduct>();
+            {
+                std::vector<Tensor *> keep = c.out;
+                c.out = {&pp->slabs};
+                c.alloc_output(0, RMLK_UINT8, {static_cast<int64_t>(bytes)});
+                c.out = keep;
+            }
+            int32_t splits = 0;
+            if (took_fast_path(rmlk_hip_matmul_partials(c.stream, RMLK_FLOAT, m, total, k, a.data(), k, wt.data(), k,
+                                                        1, pp->slabs.data(), bytes, &splits),
+                               "rmlk.MatMulGroup")) {
+                pp->x = a;
+                pp->wt = wt;
+                pp->k = k;
+                pp->total = total;
+                pp->m = m;
+                pp->splits = splits;
+                pp->slab = m * total;
+                pp->widths = widths;
+                for (size_t i = 0; i < widths.size(); ++i) {
+                    Tensor &y = c.alloc_output(static_cast<int>(i), RMLK_FLOAT, out_shape(widths[i]));
+                    y.pending_product = pp;
+                    pp->outs.push_back(y);
+                    pp->outs.back().pending_product.reset();   // (no cycle: the copies only name the memory)
+                }
+                return;
+            }
+        }
     }
     if (widths.size() <= 4) {
         // one launch whose tiles write to the members' outputs (or the members one by one, as the

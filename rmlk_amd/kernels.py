@@ -379,6 +379,8 @@ def _row_streams(streams, with_x=True):
             st.idx = _ptr(d["idx"])
             st.data_shape = Dims.of(d["data_shape"])
             st.tuple_size = len(d["data_shape"]) - 1
+        if d.get("partials"):
+            st.partials, st.partial_stride = int(d["partials"]), int(d["partial_stride"])
     return arr
 
 

@@ -230,6 +230,59 @@ def test_head_rows_match_separate_kernels(device, b, hq, hk, s, length, d):
     assert int(err.item()) == 0
 
 
+@pytest.mark.parametrize("b,hq,hk,s,length,d,splits", [(1, 32, 8, 512, 640, 64, 2), (1, 32, 8, 512, 640, 64, 4),
+                                                      (2, 4, 2, 7, 12, 16, 3), (1, 3, 1, 5, 9, 6, 2)])
+def test_head_rows_over_the_partial_sums_of_a_joint_product(device, b, hq, hk, s, length, d, splits):
+    """The rows of a joint q/k/v product read from its split-K slabs (added up in ascending order while
+    they are loaded) equal the rows of the combined product: same bits as adding the slabs first."""
+    import torch
+    k = _k()
+    rng = np.random.default_rng(hq + s + d + splits)
+    total = (hq + 2 * hk) * d
+    slabs = to_dev(rng.standard_normal((splits, b * s, total), dtype=np.float32), device)
+    joint = slabs[0].clone()
+    for z in range(1, splits):
+        joint = joint + slabs[z]          # fp32 adds in ascending order, like the combine kernel
+    cos = to_dev(rng.uniform(-1, 1, size=(1, 1, s, d)).astype(np.float32), device)
+    sin = to_dev(rng.uniform(-1, 1, size=(1, 1, s, d)).astype(np.float32), device)
+    cache_shape = [b, hk, length, d]
+    kc = rng.standard_normal(cache_shape, dtype=np.float32)
+    vc = rng.standard_normal(cache_shape, dtype=np.float32)
+    pos = rng.permutation(length)[:s]
+    idx = np.zeros((b, hk, s, 3), np.int64)
+    idx[..., 0] = np.arange(b).reshape(b, 1, 1)
+    idx[..., 1] = np.arange(hk).reshape(1, hk, 1)
+    idx[..., 2] = pos.reshape(1, 1, s)
+    idx_d = to_dev(idx, device)
+
+    def table(h):
+        cs = bcast_strides([1, 1, s, d], [b, h, s, d])
+        cs[-1] = 1
+        return cs
+    xs = [s * total, d, total, 1]          # logical [B,H,S,D] over rows of the joint matrix
+
+    def streams(src, q_out, k_out, v_out, **extra):
+        cols = (0, hq * d, (hq + hk) * d)
+        return [
+            dict(x=src.reshape(-1)[cols[0]:], shape=[b, hq, s, d], x_stride=xs, cos=cos, sin=sin,
+                 cos_stride=table(hq), sin_stride=table(hq), out=q_out, **extra),
+            dict(x=src.reshape(-1)[cols[1]:], shape=[b, hk, s, d], x_stride=xs, cos=cos, sin=sin,
+                 cos_stride=table(hk), sin_stride=table(hk), out=k_out, idx=idx_d, data_shape=cache_shape, **extra),
+            dict(x=src.reshape(-1)[cols[2]:], shape=[b, hk, s, d], x_stride=xs, out=v_out, idx=idx_d,
+                 data_shape=cache_shape, **extra)]
+    err = torch.zeros(1, dtype=torch.int32, device=device)
+    q_exp = torch.empty(b * hq * s * d, device=device)
+    kc_exp, vc_exp = to_dev(kc, device), to_dev(vc, device)
+    k.head_rows(streams(joint, q_exp, kc_exp, vc_exp), err)
+    q_got = torch.full_like(q_exp, 3.0)
+    kc_got, vc_got = to_dev(kc, device), to_dev(vc, device)
+    k.head_rows(streams(slabs, q_got, kc_got, vc_got, partials=splits, partial_stride=b * s * total), err)
+    assert_exact(to_np(q_got), to_np(q_exp))
+    assert_exact(to_np(kc_got), to_np(kc_exp))
+    assert_exact(to_np(vc_got), to_np(vc_exp))
+    assert int(err.item()) == 0
+
+
 def test_head_rows_flag_an_index_out_of_range_and_check_their_arguments(device):
     import torch
     from rmlk_amd import RmlkError
