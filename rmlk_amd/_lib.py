@@ -168,6 +168,8 @@ SIGNATURES = {
     "rmlk_hip_memcpy_htod": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "rmlk_hip_memcpy_dtoh": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "rmlk_hip_memcpy_dtod": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
+    "rmlk_hip_memcpy_dtod_many": (c_int32, [c_void_p, c_int32, POINTER(c_void_p), POINTER(c_void_p),
+                                            POINTER(c_size_t)]),
     "rmlk_hip_memset": (c_int32, [c_void_p, c_void_p, c_int32, c_size_t]),
     "rmlk_hip_stream_sync": (c_int32, [c_void_p]),
     "rmlk_hip_device_info": (c_int32, [c_int32, POINTER(DeviceInfo)]),

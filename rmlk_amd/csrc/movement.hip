@@ -89,6 +89,31 @@ __global__ __launch_bounds__(kBlock) void copy_flat_kernel(const U *__restrict__
     }
 }
 
+// several dense flat copies in one launch: blockIdx.y picks the copy
+constexpr int kMaxCopies = 8;
+struct CopyMany {
+    const U128 *in[kMaxCopies];
+    U128 *out[kMaxCopies];
+    uint32_t n[kMaxCopies];   // units
+};
+__global__ __launch_bounds__(kBlock) void copy_many_kernel(CopyMany a) {
+    const U128 *__restrict__ in = a.in[blockIdx.y];
+    U128 *__restrict__ out = a.out[blockIdx.y];
+    const uint32_t n = a.n[blockIdx.y];
+    for (uint32_t base = blockIdx.x * kChunk; base < n; base += gridDim.x * kChunk) {
+        const uint32_t i0 = base + threadIdx.x;
+        if (base + kChunk <= n) {
+            U128 r[kUnroll];
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j) r[j] = nt_load(in + i0 + j * kBlock);
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j) put(out + i0 + j * kBlock, r[j]);
+        } else {
+            for (uint32_t i = i0; i < n; i += kBlock) put(out + i, nt_load(in + i));
+        }
+    }
+}
+
 template <typename U>
 int32_t launch_copy_units(hipStream_t s, NdPlan<2> &pl, const void *in, void *out) {
     uint32_t n = static_cast<uint32_t>(pl.numel);
@@ -614,6 +639,41 @@ extern "C" int32_t rmlk_hip_memcpy_dtod(rmlk_stream_t stream, void *dst, const v
         if (st) return st;
     }
     return RMLK_OK;
+}
+
+// Up to 8 device-to-device copies as ONE launch (16-byte aligned ends and lengths, below 16 GiB
+// each); anything else one call of rmlk_hip_memcpy_dtod per copy.
+extern "C" int32_t rmlk_hip_memcpy_dtod_many(rmlk_stream_t stream, int32_t n_copies, void *const *dsts,
+                                             const void *const *srcs, const size_t *bytes) {
+    if (n_copies < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n_copies == 0) return RMLK_OK;
+    if (!dsts || !srcs || !bytes) return RMLK_ERR_NULL_POINTER;
+    bool together = n_copies <= kMaxCopies;
+    size_t longest = 0;
+    for (int i = 0; i < n_copies; ++i) {
+        if (bytes[i] && (!dsts[i] || !srcs[i])) return RMLK_ERR_NULL_POINTER;
+        if (bytes[i] % 16 || reinterpret_cast<uintptr_t>(dsts[i]) % 16 || reinterpret_cast<uintptr_t>(srcs[i]) % 16 ||
+            bytes[i] / 16 >= (static_cast<size_t>(1) << 30))
+            together = false;
+        if (bytes[i] > longest) longest = bytes[i];
+    }
+    if (!together || n_copies == 1) {
+        for (int i = 0; i < n_copies; ++i) {
+            const int32_t st = rmlk_hip_memcpy_dtod(stream, dsts[i], srcs[i], bytes[i]);
+            if (st) return st;
+        }
+        return RMLK_OK;
+    }
+    if (longest == 0) return RMLK_OK;
+    CopyMany a{};
+    for (int i = 0; i < n_copies; ++i) {
+        a.in[i] = static_cast<const U128 *>(srcs[i]);
+        a.out[i] = static_cast<U128 *>(dsts[i]);
+        a.n[i] = static_cast<uint32_t>(bytes[i] / 16);
+    }
+    dim3 grid(chunk_grid(static_cast<uint32_t>(longest / 16), kChunk), static_cast<unsigned>(n_copies), 1);
+    copy_many_kernel<<<grid, kBlock, 0, as_stream(stream)>>>(a);
+    return launch_status();
 }
 
 extern "C" int32_t rmlk_hip_transpose(rmlk_stream_t stream, int32_t dtype,

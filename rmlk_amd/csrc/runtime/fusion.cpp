@@ -1326,6 +1326,9 @@ void op_fused_head_rows(OpContext &c) {
     }
     std::vector<rmlk_row_stream> streams(n);
     std::vector<int64_t> first_col(n, 0);
+    std::vector<void *> copy_dst;
+    std::vector<const void *> copy_src;
+    std::vector<size_t> copy_bytes;
     for (size_t i = 0; i < n; ++i) {
         rmlk_row_stream &st = streams[i];
         st = rmlk_row_stream{};
@@ -1357,9 +1360,22 @@ void op_fused_head_rows(OpContext &c) {
             st.data_shape = to_dims(data.shape);
             st.tuple_size = static_cast<int32_t>(data.rank() - 1);
             st.idx = static_cast<const int64_t *>(idx.data());
-            st.out = scatter_destination(c, in, static_cast<int>(i)).data();
+            // a destination that has to be a copy of its data tensor: the copies of all streams go
+            // out as one launch below
+            bool copy_here = false;
+            Tensor &dest = scatter_destination(c, in, static_cast<int>(i), &copy_here);
+            st.out = dest.data();
+            if (copy_here && data.nbytes() > 0) {
+                copy_dst.push_back(dest.data());
+                copy_src.push_back(data.data());
+                copy_bytes.push_back(data.nbytes());
+            }
         }
     }
+    if (!copy_dst.empty())
+        check_status(rmlk_hip_memcpy_dtod_many(c.stream, static_cast<int32_t>(copy_dst.size()), copy_dst.data(),
+                                               copy_src.data(), copy_bytes.data()),
+                     "ScatterND copy");
     if (product && from_slabs) {
         if (took_fast_path(rmlk_hip_head_rows(c.stream, RMLK_FLOAT, static_cast<int32_t>(n), streams.data(),
                                               c.error_flag()),

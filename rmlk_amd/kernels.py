@@ -397,6 +397,15 @@ def gemv_kmajor_head_rows(x, wt, k: int, streams, first_cols, gamma=None, eps: f
           "rmlk_hip_gemv_kmajor_head_rows")
 
 
+def memcpy_dtod_many(dsts, srcs) -> None:
+    """dsts[i] <- srcs[i] (dense device tensors of equal byte size each), one launch for up to 8 copies."""
+    n = len(dsts)
+    d = (ctypes.c_void_p * n)(*[_ptr(t) for t in dsts])
+    s_ = (ctypes.c_void_p * n)(*[_ptr(t) for t in srcs])
+    b = (ctypes.c_size_t * n)(*[t.numel() * t.element_size() for t in srcs])
+    check(lib().rmlk_hip_memcpy_dtod_many(_stream(), n, d, s_, b), "rmlk_hip_memcpy_dtod_many")
+
+
 def device_info(device: int = 0) -> dict:
     from ._lib import DeviceInfo
     info = DeviceInfo()

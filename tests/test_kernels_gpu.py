@@ -458,6 +458,22 @@ def test_concat(device, case, dtype):
     assert_exact(to_np(out), expected)
 
 
+@pytest.mark.parametrize("sizes", [[1310720, 1310720], [16, 4096, 48, 1 << 20], [64] * 9, [20, 64]])
+def test_several_device_copies_in_one_call(device, sizes):
+    """rmlk_hip_memcpy_dtod_many: every destination gets its source, nothing past the ends is touched
+    (more than 8 copies, or lengths that are no multiple of 16, go one by one)."""
+    import torch
+    k = _k()
+    rng = np.random.default_rng(len(sizes) + sizes[0])
+    srcs = [to_dev(rng.integers(0, 255, size=n + 32, dtype=np.uint8), device) for n in sizes]
+    dsts = [torch.full((n + 32,), 7, dtype=torch.uint8, device=device) for n in sizes]
+    k.memcpy_dtod_many([d[16:16 + n] for d, n in zip(dsts, sizes)], [s_[16:16 + n] for s_, n in zip(srcs, sizes)])
+    for d, s_, n in zip(dsts, srcs, sizes):
+        got = to_np(d)
+        assert (got[:16] == 7).all() and (got[16 + n:] == 7).all()
+        assert_exact(got[16:16 + n], to_np(s_)[16:16 + n])
+
+
 @pytest.mark.parametrize("case", CONCAT_CASES + [
     ([(1, 8, 8191, 64), (1, 8, 1, 64)], 2),                       # KV cache grown by one row
     ([(2, 3, 4), (2, 3, 4), (2, 3, 4), (2, 3, 4), (2, 3, 4)], 1),
