@@ -3,8 +3,8 @@
 // The reference executes an ONNX graph node by node, one kernel each
 // (runtime/src/core/instance.rs:25-37). Decoder graphs repeat a few chains of small element-wise
 // nodes in every layer; on this GPU each launch costs ~2 us whatever it moves, so those chains
-// dominate a decode step. This pass finds four of them and replaces each by ONE node backed by a
-// fused kernel that rounds every intermediate like the separate kernels do (the attention MatMul
+// dominate a decode step. This pass finds them and replaces each by ONE node backed by a fused
+// kernel that rounds every intermediate like the separate kernels do (the attention MatMul
 // instead drops two copies: the grouped-query Expand and the K transpose become GEMM strides):
 //
 //   rmlk.RMSNorm           Pow(x,2) ReduceMean(-1) Add(eps) Sqrt Div|(Div(1,.) Mul) Mul(gamma)
@@ -12,12 +12,20 @@
 //   rmlk.SwiGLU            Sigmoid(g) Mul(g,.) Mul(.,u)
 //   rmlk.ScaleMaskSoftmax  Div|Mul(x,c) Add(mask) Softmax(-1)
 //   rmlk.Rotary            [Transpose(0,2,1,3)] Slice Slice Neg Concat Mul Mul Add
+//   rmlk.HeadRows          up to four streams of rows (rmlk.Rotary, or a ScatterND fed by one or by
+//                          a head Transpose) behind one projection, one launch
 //   rmlk.AttnMatMul        MatMul(a, [Transpose(0,1,3,2)] [Reshape Expand Unsqueeze] (kv))
+//   rmlk.Attention         rmlk.AttnMatMul -> rmlk.ScaleMaskSoftmax -> rmlk.AttnMatMul [-> Transpose]
 //   rmlk.MatMulGroup       MatMul(a, W1), MatMul(a, W2), ... on the same a with constant 2-D weights
-//   rmlk.MatMulGroupSwiGLU a [gate | up] rmlk.MatMulGroup feeding only an rmlk.SwiGLU: a one-row a
-//                          leaves its split-K slabs to the SwiGLU kernel (no combine launch)
+//   rmlk.MatMulGroupSwiGLU a [gate | up] rmlk.MatMulGroup feeding only an rmlk.SwiGLU
+//   rmlk.MatMulAddRMSNorm  MatMul(a, W) feeding the residual Add of an rmlk.AddRMSNorm
+//   rmlk.MatMulConst       any other MatMul(a, W) with constant 2-D W
 //
-// A fused node keeps the nodes it replaced as its `body`. What cannot be decided while building
+// The nodes over constant weights store them K-contiguous ([n][k]) and release the row-major
+// initializers: one-row inputs and many-row inputs read the same copy.
+//
+// A fused node keeps the nodes it replaced as its `body` (the nodes over constant weights: product
+// nodes over the K-contiguous weights, or nothing where every case is covered). What cannot be decided while building
 // (shapes are only known at run time) is checked when the node runs; if the fused kernel does not
 // cover the case, the body runs instead, node by node, so the graph's meaning never changes.
 #include <algorithm>
