@@ -343,8 +343,8 @@ int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch, i
  * or infinity in a K or V row no query of the tile can see does not reach that tile's output
  * (0 * NaN would), and a row with nothing visible anywhere is NaN as before. The size is 0 (and a
  * null workspace allowed) where skipping does not apply: few blocks, q_len not a multiple of 64, or
- * more than 128 chunks. The workspace is 16-byte aligned and belongs to the call until its kernels
- * have run. rmlk_hip_attention is this call with a null workspace. */
+ * more than 128 chunks. The workspace is 16-byte aligned (one that is not, or is too small, is
+ * ignored: every chunk is then visited) and belongs to the call until its kernels have run. rmlk_hip_attention is this call with a null workspace. */
 size_t rmlk_hip_attention_workspace_size(int32_t dtype, int64_t batch, int64_t kv_heads, int64_t rep,
                                          int64_t q_len, int64_t kv_len, int64_t head_dim,
                                          const rmlk_dims *mask_stride);

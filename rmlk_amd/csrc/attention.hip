@@ -733,7 +733,7 @@ extern "C" int32_t rmlk_hip_attention_ws(rmlk_stream_t stream, int32_t dtype, in
     // two blocks of four wavefronts per CU when there are that many, else one block of eight
     if (static_cast<int64_t>(grid.x) * grid.y > kNumCU) {
         const TileMapDims tm = tile_map_dims(batch, kv_heads, rep, q_len, kv_len, mask_stride);
-        if (workspace && tm.bytes && workspace_bytes >= tm.bytes) {
+        if (workspace && tm.bytes && workspace_bytes >= tm.bytes && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
             uint8_t *tiles = static_cast<uint8_t *>(workspace);
             const dim3 tgrid(static_cast<unsigned>(tm.chunks), static_cast<unsigned>(tm.tiles),
                              static_cast<unsigned>(tm.mask_batches * tm.mask_heads));

@@ -1230,6 +1230,14 @@ def test_attention_workspace_that_is_too_small_is_not_used(device):
                                       got.data_ptr()), "rmlk_hip_attention_ws")
     assert_exact(to_np(got), to_np(exp))
     assert (to_np(ws) == 7).all()
+    # the same for one that is large enough but not 16-byte aligned
+    ws2 = torch.full((need + 16,), 7, dtype=torch.uint8, device=device)
+    got2 = torch.empty_like(exp)
+    check(lib().rmlk_hip_attention_ws(stream, kk.FLOAT, b, g, rep, s, l, d, q.data_ptr(), k.data_ptr(),
+                                      v.data_ptr(), m.data_ptr(), ms, 0, 8.0, 0, ws2.data_ptr() + 4, need,
+                                      got2.data_ptr()), "rmlk_hip_attention_ws")
+    assert_exact(to_np(got2), to_np(exp))
+    assert (to_np(ws2) == 7).all()
 
 
 def test_attention_few_rows_one_launch_needs_its_counters(device):
