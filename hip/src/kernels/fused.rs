@@ -72,18 +72,58 @@ pub unsafe fn swiglu(stream: &HipStream, n: usize, gate: *const c_void, up: *con
     check(ffi::rmlk_hip_swiglu(stream.raw(), ffi::RMLK_FLOAT, n as i64, gate, up, out), "swiglu")
 }
 
+/// How constant weights are held in device memory; the arithmetic is fp32 in every case.
+#[derive(Clone, Copy, Debug, PartialEq, Eq)]
+pub enum WeightStorage {
+    F32,
+    F16,
+    BF16,
+}
+
+impl WeightStorage {
+    pub fn dtype(self) -> i32 {
+        match self {
+            WeightStorage::F32 => ffi::RMLK_FLOAT,
+            WeightStorage::F16 => ffi::RMLK_FLOAT16,
+            WeightStorage::BF16 => ffi::RMLK_BFLOAT16,
+        }
+    }
+}
+
+/// `dst[i] = src[i]` rounded to nearest even in a 16-bit storage type.
+pub unsafe fn store_weights(
+    stream: &HipStream,
+    storage: WeightStorage,
+    n: usize,
+    src: *const c_void,
+    dst: *mut c_void,
+) -> Result<()> {
+    check(ffi::rmlk_hip_store_weights(stream.raw(), storage.dtype(), n as i64, src, dst), "store_weights")
+}
+
 /// One-row product over K-contiguous weights: `y[n] = sum_k x[k] * wt[n][k]`.
 pub unsafe fn gemv_kmajor(
     stream: &HipStream,
     n: usize,
     k: usize,
     x: *const c_void,
+    storage: WeightStorage,
     wt: *const c_void,
     ldw: usize,
     y: *mut c_void,
 ) -> Result<()> {
     check(
-        ffi::rmlk_hip_gemv_kmajor(stream.raw(), ffi::RMLK_FLOAT, n as i64, k as i64, x, wt, ldw as i64, y),
+        ffi::rmlk_hip_gemv_kmajor(
+            stream.raw(),
+            ffi::RMLK_FLOAT,
+            n as i64,
+            k as i64,
+            x,
+            storage.dtype(),
+            wt,
+            ldw as i64,
+            y,
+        ),
         "gemv_kmajor",
     )
 }

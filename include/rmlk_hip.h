@@ -58,7 +58,8 @@ typedef enum rmlk_dtype {
     RMLK_FLOAT16 = 10,
     RMLK_DOUBLE = 11,
     RMLK_UINT32 = 12,
-    RMLK_UINT64 = 13
+    RMLK_UINT64 = 13,
+    RMLK_BFLOAT16 = 16 /* only as the storage type of constant weights (w_dtype below) */
 } rmlk_dtype;
 
 /* Shape or stride vector passed by value from the host; replaces the device `info` buffers the
@@ -381,6 +382,25 @@ int32_t rmlk_hip_attention_few_rows_one_launch(rmlk_stream_t stream, int32_t dty
                                                float scale, int32_t out_seq_major, void *workspace,
                                                size_t workspace_bytes, int32_t *counters, void *out);
 
+/* ---- constant weights stored as 16-bit values ----------------------------------------------------
+ * The products over constant weights below take the storage type of the weights as `w_dtype`:
+ * RMLK_FLOAT, or RMLK_FLOAT16 / RMLK_BFLOAT16 for weights that were rounded ONCE, when they were
+ * stored (rmlk_hip_store_weights), to half the bytes a token has to stream. The arithmetic stays
+ * fp32: a stored value is widened exactly, products and sums are formed in float, x, gamma, the
+ * residual and every output are float. A many-row product over 16-bit weights equals the fp32
+ * product over the widened weights bit for bit (same kernels behind the widening); the one-row
+ * products agree with it to rounding (other order of the sum). 16-bit weights must be K-contiguous
+ * (trans_b), rows whole 128-bit units (k % 8 == 0, ldb % 8 == 0, 16-byte aligned base); ldb / ldw
+ * and the row offsets count stored values. RMLK_ERR_UNSUPPORTED otherwise, and for any other
+ * w_dtype. (ref: the f16 kernel symbols of the reference, e.g. cuda/src/ptx/add.cu:19-25, which its
+ * provider cannot run: runtime/src/providers/cuda/data.rs:109-126; storage with fp32 accumulation
+ * has no counterpart there.)
+ *
+ * rmlk_hip_store_weights: dst[i] = src[i] (float) rounded to nearest even in `w_dtype`
+ * (RMLK_FLOAT16 or RMLK_BFLOAT16; NaN stays NaN, overflow gives infinity). */
+int32_t rmlk_hip_store_weights(rmlk_stream_t stream, int32_t w_dtype, int64_t n, const void *src,
+                               void *dst);
+
 /* ---- products that share their first operand (q/k/v, gate/up) ----------------------------------
  * The weights of such MatMuls (ref: one cublasGemmStridedBatchedEx each,
  * cuda/src/kernels/gemm.rs:191-232) lie side by side in one matrix B: row-major [k, sum(widths)]
@@ -394,7 +414,7 @@ int32_t rmlk_hip_attention_few_rows_one_launch(rmlk_stream_t stream, int32_t dty
 size_t rmlk_hip_matmul_grouped_workspace_size(int32_t dtype, int64_t m, int64_t k, int32_t groups,
                                               const int64_t *widths);
 int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t k,
-                                const void *a, int64_t lda, const void *b, int64_t ldb,
+                                const void *a, int64_t lda, int32_t w_dtype, const void *b, int64_t ldb,
                                 int32_t trans_b, int32_t groups, const int64_t *widths,
                                 void *const *outs, void *workspace, size_t workspace_bytes);
 /* out[m, n] = swiglu(A . B[:, gate_offset .. +n], A . B[:, up_offset .. +n]) (see rmlk_hip_swiglu)
@@ -403,8 +423,9 @@ int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, int64_t m, 
  * 128 x 64 tile per compute unit; RMLK_ERR_UNSUPPORTED otherwise (the caller then multiplies and
  * activates separately). Results do not depend on trans_b. */
 int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n, int64_t k,
-                               const void *a, int64_t lda, const void *b, int64_t ldb, int32_t trans_b,
-                               int64_t gate_offset, int64_t up_offset, void *out, int64_t ldc);
+                               const void *a, int64_t lda, int32_t w_dtype, const void *b, int64_t ldb,
+                               int32_t trans_b, int64_t gate_offset, int64_t up_offset, void *out,
+                               int64_t ldc);
 
 /* One-row product with K-CONTIGUOUS weights: y[n] = sum_k x[k] * wt[n][k] (wt row-major [n, k],
  * leading dimension ldw), i.e. rmlk_hip_matmul with m = 1 and trans_b. Every output column is
@@ -413,28 +434,29 @@ int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t m, i
  * matrices K-contiguous for it (ref: cublasGemmStridedBatchedEx with
  * CUBLAS_OP_T on a transposed operand, cuda/src/kernels/gemm.rs:191-232). */
 int32_t rmlk_hip_gemv_kmajor(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k, const void *x,
-                        const void *wt, int64_t ldw, void *y);
+                        int32_t w_dtype, const void *wt, int64_t ldw, void *y);
 /* y[i] = swiglu(x . wt[gate_row + i, :], x . wt[up_row + i, :]) for i < n (see rmlk_hip_swiglu): the
  * gate and the up projection of a one-row input and the activation in one launch. */
 int32_t rmlk_hip_gemv_kmajor_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
-                               const void *x, const void *wt, int64_t ldw, int64_t gate_row,
-                               int64_t up_row, void *y);
+                               const void *x, int32_t w_dtype, const void *wt, int64_t ldw,
+                               int64_t gate_row, int64_t up_row, void *y);
 /* rmlk_hip_gemv_kmajor with a residual row added to the result: y = x . wt^T + residual (the Add
  * behind an output projection; ref kernels: gemm.rs:191-232, binary.rs:58-100). */
 int32_t rmlk_hip_gemv_kmajor_add(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k, const void *x,
-                                 const void *wt, int64_t ldw, const void *residual, void *y);
+                                 int32_t w_dtype, const void *wt, int64_t ldw, const void *residual,
+                                 void *y);
 /* The same products over RMSNorm(x) * gamma instead of x, the normalised row never stored: every
  * wavefront works out the row's statistics with rmlk_hip_rmsnorm's arithmetic, so the results equal
  * rmlk_hip_rmsnorm followed by the product bit for bit. k <= 8192, gamma 16-byte aligned, else
  * RMLK_ERR_UNSUPPORTED. Chain: Pow, ReduceMean, Add, Sqrt, Div | Div(1,.) Mul, Mul, MatMul
  * (ref kernels: unary.rs:10-42, reduce_mean.rs:5-36, binary.rs:58-100, gemm.rs:191-232). */
 int32_t rmlk_hip_gemv_kmajor_normed(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k, const void *x,
-                                    const void *gamma, float eps, int32_t reciprocal_form, const void *wt,
-                                    int64_t ldw, void *y);
+                                    const void *gamma, float eps, int32_t reciprocal_form,
+                                    int32_t w_dtype, const void *wt, int64_t ldw, void *y);
 int32_t rmlk_hip_gemv_kmajor_swiglu_normed(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
                                            const void *x, const void *gamma, float eps,
-                                           int32_t reciprocal_form, const void *wt, int64_t ldw,
-                                           int64_t gate_row, int64_t up_row, void *y);
+                                           int32_t reciprocal_form, int32_t w_dtype, const void *wt,
+                                           int64_t ldw, int64_t gate_row, int64_t up_row, void *y);
 
 /* ---- many-row products whose split-K combine is left to the consumer ----------------------------
  * rmlk_hip_matmul_partials: the tiled kernels of rmlk_hip_matmul for A[m, k] . B (row-major [k, n],
@@ -446,7 +468,7 @@ int32_t rmlk_hip_gemv_kmajor_swiglu_normed(rmlk_stream_t stream, int32_t dtype, 
  * No counterpart in the reference. */
 size_t rmlk_hip_matmul_partials_workspace_size(int32_t dtype, int64_t m, int64_t n, int64_t k);
 int32_t rmlk_hip_matmul_partials(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n, int64_t k,
-                                 const void *a, int64_t lda, const void *b, int64_t ldb,
+                                 const void *a, int64_t lda, int32_t w_dtype, const void *b, int64_t ldb,
                                  int32_t trans_b, void *workspace, size_t workspace_bytes,
                                  int32_t *splits_out);
 int32_t rmlk_hip_splitk_add_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t rows, int64_t cols,
@@ -513,7 +535,7 @@ int32_t rmlk_hip_head_rows(rmlk_stream_t stream, int32_t dtype, int32_t n_stream
  * No counterpart in the reference (gemm.rs:191-232 followed by the kernels listed above). */
 int32_t rmlk_hip_gemv_kmajor_head_rows(rmlk_stream_t stream, int32_t dtype, int64_t k, const void *x,
                                        const void *gamma, float eps, int32_t reciprocal_form,
-                                       const void *wt, int64_t ldw, int32_t n_streams,
+                                       int32_t w_dtype, const void *wt, int64_t ldw, int32_t n_streams,
                                        const rmlk_row_stream *streams, const int64_t *first_col,
                                        int32_t *err_flag);
 

@@ -88,6 +88,14 @@ int32_t rmlk_session_create(const rmlk_graph *g, int32_t device, rmlk_session **
  * RMLK_SESSION_NO_FUSION keeps one kernel per ONNX node as the reference executes it
  * (runtime/src/core/instance.rs:25-37). rmlk_session_create passes flags = 0. */
 #define RMLK_SESSION_NO_FUSION 1u
+/* Constant 2-D weights that only MatMuls of fused nodes read are stored as IEEE half or bfloat16
+ * values (rounded to nearest even once, while the session is built) instead of floats: half the
+ * bytes per decode step, half the device memory. Activations, accumulation and every other tensor
+ * stay fp32; the results are those of the same session over a graph whose weights were rounded
+ * beforehand (many-row products bit for bit, one-row products to rounding). At most one of the two;
+ * ignored with RMLK_SESSION_NO_FUSION. Off by default: the reference computes in fp32 only. */
+#define RMLK_SESSION_WEIGHTS_F16 2u
+#define RMLK_SESSION_WEIGHTS_BF16 4u
 int32_t rmlk_session_create_ex(const rmlk_graph *g, int32_t device, uint32_t flags,
                                rmlk_session **out);
 /* Number of fused nodes the session formed while it was built. */

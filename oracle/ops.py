@@ -443,3 +443,23 @@ def constant_of_shape(shape, value=None):
         value = np.zeros((1,), dtype=np.float32)
     value = np.asarray(value).reshape(-1)
     return np.full(shape, value[0], dtype=value.dtype)
+
+
+def store_weights(w, storage: str):
+    """Constant weights rounded once to a 16-bit storage type and widened again: what a product over
+    stored weights multiplies with. `storage`: "f16" (IEEE binary16, numpy's own conversion) or
+    "bf16" (the upper 16 bits of the float after rounding to nearest, ties to even; NaN stays NaN).
+    No counterpart in the reference, whose provider holds fp32 only
+    (runtime/src/providers/cuda/data.rs:109-126). Pinned in tests/test_oracle_golden.py: ties,
+    overflow and special values in closed form, and torch's CPU conversion on random floats."""
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    if storage == "f16":
+        with np.errstate(over="ignore"):
+            return w.astype(np.float16).astype(np.float32)
+    if storage != "bf16":
+        raise OracleError(f"unknown weight storage {storage!r}")
+    u = w.view(np.uint32).astype(np.uint64)
+    rounded = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    rounded = np.where(nan, ((u >> 16) | 0x40) << 16, rounded)
+    return (rounded & 0xFFFFFFFF).astype(np.uint32).view(np.float32).reshape(w.shape)

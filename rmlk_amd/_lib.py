@@ -112,22 +112,24 @@ SIGNATURES = {
                                          c_int64, c_int64, c_void_p]),
     "rmlk_hip_matmul_partials_workspace_size": (c_size_t, [c_int32, c_int64, c_int64, c_int64]),
     "rmlk_hip_matmul_partials": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p,
-                                           c_int64, c_void_p, c_int64, c_int32, c_void_p, c_size_t,
+                                           c_int64, c_int32, c_void_p, c_int64, c_int32, c_void_p, c_size_t,
                                            POINTER(c_int32)]),
     "rmlk_hip_splitk_add_rmsnorm": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int32,
                                               c_int64, c_void_p, c_void_p, ctypes.c_float, c_int32,
                                               c_void_p, c_void_p]),
-    "rmlk_hip_gemv_kmajor": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p, c_int64,
-                                  c_void_p]),
-    "rmlk_hip_gemv_kmajor_swiglu": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p,
-                                         c_int64, c_int64, c_int64, c_void_p]),
-    "rmlk_hip_gemv_kmajor_add": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p, c_int64,
-                                           c_void_p, c_void_p]),
+    "rmlk_hip_store_weights": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
+    "rmlk_hip_gemv_kmajor": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int32, c_void_p,
+                                       c_int64, c_void_p]),
+    "rmlk_hip_gemv_kmajor_swiglu": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int32,
+                                              c_void_p, c_int64, c_int64, c_int64, c_void_p]),
+    "rmlk_hip_gemv_kmajor_add": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int32, c_void_p,
+                                           c_int64, c_void_p, c_void_p]),
     "rmlk_hip_gemv_kmajor_normed": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p,
-                                              ctypes.c_float, c_int32, c_void_p, c_int64, c_void_p]),
+                                              ctypes.c_float, c_int32, c_int32, c_void_p, c_int64,
+                                              c_void_p]),
     "rmlk_hip_gemv_kmajor_swiglu_normed": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p,
-                                                     ctypes.c_float, c_int32, c_void_p, c_int64, c_int64,
-                                                     c_int64, c_void_p]),
+                                                     ctypes.c_float, c_int32, c_int32, c_void_p, c_int64,
+                                                     c_int64, c_int64, c_void_p]),
     "rmlk_hip_attention": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64,
                                      c_int64, c_void_p, c_void_p, c_void_p, c_void_p, _PD, c_int32,
                                      ctypes.c_float, c_int32, c_void_p]),
@@ -149,17 +151,17 @@ SIGNATURES = {
     "rmlk_hip_matmul_grouped_workspace_size": (c_size_t, [c_int32, c_int64, c_int64, c_int32,
                                                           POINTER(c_int64)]),
     "rmlk_hip_matmul_grouped": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int64,
-                                          c_void_p, c_int64, c_int32, c_int32, POINTER(c_int64),
+                                          c_int32, c_void_p, c_int64, c_int32, c_int32, POINTER(c_int64),
                                           POINTER(c_void_p), c_void_p, c_size_t]),
     "rmlk_hip_matmul_swiglu": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p,
-                                         c_int64, c_void_p, c_int64, c_int32, c_int64, c_int64, c_void_p,
-                                         c_int64]),
+                                         c_int64, c_int32, c_void_p, c_int64, c_int32, c_int64, c_int64,
+                                         c_void_p, c_int64]),
     "rmlk_hip_rotary": (c_int32, [c_void_p, c_int32, _PD, _PD, _PD, _PD, c_void_p, c_void_p,
                                   c_void_p, c_void_p]),
     "rmlk_hip_head_rows": (c_int32, [c_void_p, c_int32, c_int32, POINTER(RowStream), c_void_p]),
     "rmlk_hip_gemv_kmajor_head_rows": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, ctypes.c_float,
-                                                 c_int32, c_void_p, c_int64, c_int32, c_void_p, c_void_p,
-                                                 c_void_p]),
+                                                 c_int32, c_int32, c_void_p, c_int64, c_int32, c_void_p,
+                                                 c_void_p, c_void_p]),
     "rmlk_hip_fill": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
     "rmlk_hip_range": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p]),
     "rmlk_hip_write_small": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),

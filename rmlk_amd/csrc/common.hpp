@@ -27,7 +27,8 @@ inline int dtype_size(int32_t dt) {
         case RMLK_INT8: return 1;
         case RMLK_UINT16:
         case RMLK_INT16:
-        case RMLK_FLOAT16: return 2;
+        case RMLK_FLOAT16:
+        case RMLK_BFLOAT16: return 2;
         case RMLK_FLOAT:
         case RMLK_INT32:
         case RMLK_UINT32: return 4;

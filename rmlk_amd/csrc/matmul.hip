@@ -28,6 +28,63 @@ namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+
+// How the second operand of a product over constant weights is held in memory: as floats, or as
+// IEEE half or bfloat16 values (half the bytes to stream). The arithmetic is fp32 whatever the
+// storage: both 16-bit formats are subsets of float, a stored value is widened exactly before it
+// is multiplied, and every sum is formed in float - the result is that of the fp32 product over the
+// weights rounded once, when they were stored.
+struct StoredF32 {
+    using elem = float;
+    static constexpr int kUnit = 4;      // weights per 128-bit unit
+};
+struct StoredF16 {
+    using elem = uint16_t;
+    static constexpr int kUnit = 8;
+    static __device__ __forceinline__ float widen(uint16_t v) {
+        return static_cast<float>(__builtin_bit_cast(_Float16, v));
+    }
+    // two neighbours of a row, the one at the lower address in the low half
+    static __device__ __forceinline__ void widen2(uint32_t pair, float &lo, float &hi) {
+        const v2h h = __builtin_bit_cast(v2h, pair);
+        lo = static_cast<float>(h[0]);
+        hi = static_cast<float>(h[1]);
+    }
+};
+struct StoredBF16 {
+    using elem = uint16_t;
+    static constexpr int kUnit = 8;
+    static __device__ __forceinline__ float widen(uint16_t v) {
+        return __uint_as_float(static_cast<uint32_t>(v) << 16);
+    }
+    static __device__ __forceinline__ void widen2(uint32_t pair, float &lo, float &hi) {
+        lo = __uint_as_float(pair << 16);
+        hi = __uint_as_float(pair & 0xffff0000u);
+    }
+};
+template <typename WS>
+constexpr bool kStored16 = !std::is_same<WS, StoredF32>::value;
+
+// The eight weights of one 128-bit unit of a 16-bit row, in row order.
+template <typename WS>
+__device__ __forceinline__ void widen_unit(const v4u &raw, float (&w)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) WS::widen2(raw[i], w[2 * i], w[2 * i + 1]);
+}
+
+// f(storage tag) for the storage type `w_dtype` names; UNSUPPORTED for any other type.
+template <typename F>
+int32_t with_storage(int32_t w_dtype, F &&f) {
+    switch (w_dtype) {
+        case RMLK_FLOAT: return f(StoredF32{});
+        case RMLK_FLOAT16: return f(StoredF16{});
+        case RMLK_BFLOAT16: return f(StoredBF16{});
+        default: return RMLK_ERR_UNSUPPORTED;
+    }
+}
 
 constexpr int kMaxSegments = 4;
 
@@ -105,9 +162,34 @@ __device__ __forceinline__ void tile_coords(const GemmArgs &g, int &tm, int &tn,
 // loads where a whole vector is in range.
 // TB == true: B is given as [N][K] rows (C = A . B^T); both operands are then K-contiguous and the
 // B fragment is one 128-bit LDS read like A's.
-template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool TB = false>
+// WS: B (K-contiguous only) may be stored as 16-bit values; they are widened on their way from
+// global memory to LDS, which holds floats either way.
+template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool TB = false, typename WS = StoredF32>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
     using L = SmemLayout<BM, BN, BK, TB>;
+    using BE = typename WS::elem;
+    static_assert(!kStored16<WS> || TB, "16-bit weights are K-contiguous");
+    // four consecutive values of a row of B as floats
+    auto load_b4 = [](const BE *src) -> v4f {
+        if constexpr (kStored16<WS>) {
+            const v2u raw = *reinterpret_cast<const v2u *>(src);
+            v4f v;
+            float lo, hi;
+            WS::widen2(raw[0], lo, hi);
+            v[0] = lo;
+            v[1] = hi;
+            WS::widen2(raw[1], lo, hi);
+            v[2] = lo;
+            v[3] = hi;
+            return v;
+        } else {
+            return *reinterpret_cast<const v4f *>(src);
+        }
+    };
+    auto load_b1 = [](const BE *src) -> float {
+        if constexpr (kStored16<WS>) return WS::widen(*src);
+        else return *src;
+    };
     extern __shared__ __align__(16) float smem[];
     float *As = smem;                     // [2][BM][kAStride]
     float *Bs = smem + 2 * L::kAFloats;   // [2][BK][kBStride]
@@ -134,7 +216,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
     const int k_end = min(g.k, k_begin + g.k_per_split);
 
     const float *A = g.a + batch * g.stride_a;
-    const float *B = g.b + batch * g.stride_b;
+    const BE *B = reinterpret_cast<const BE *>(g.b) + batch * g.stride_b;
     float *C = g.c + (static_cast<int64_t>(split) * gridDim.y + batch) * g.stride_c;
 
     const int tid = threadIdx.x;
@@ -150,8 +232,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
 
     // per-lane source pointers of the first K step; they advance by BK (A) and BK rows (B)
     const float *a_src = A + static_cast<int64_t>(m0 + a_row) * g.lda + k_begin + a_vec * 4;
-    const float *b_src = TB ? B + static_cast<int64_t>(n0 + b_row) * g.ldb + k_begin + b_vec * 4
-                            : B + static_cast<int64_t>(k_begin + b_row) * g.ldb + n0 + b_vec * 4;
+    const BE *b_src = TB ? B + static_cast<int64_t>(n0 + b_row) * g.ldb + k_begin + b_vec * 4
+                         : B + static_cast<int64_t>(k_begin + b_row) * g.ldb + n0 + b_vec * 4;
     const int64_t a_pass_stride = static_cast<int64_t>(A_ROWS_PER_PASS) * g.lda;
     const int64_t b_pass_stride = static_cast<int64_t>(B_ROWS_PER_PASS) * g.ldb;
     const int64_t b_step_stride = TB ? BK : static_cast<int64_t>(BK) * g.ldb;
@@ -163,8 +245,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
             for (int p = 0; p < A_PASSES; ++p)
                 a_reg[p] = *reinterpret_cast<const v4f *>(a_src + p * a_pass_stride);
 #pragma unroll
-            for (int p = 0; p < B_PASSES; ++p)
-                b_reg[p] = *reinterpret_cast<const v4f *>(b_src + p * b_pass_stride);
+            for (int p = 0; p < B_PASSES; ++p) b_reg[p] = load_b4(b_src + p * b_pass_stride);
         } else {
 #pragma unroll
             for (int p = 0; p < A_PASSES; ++p) {
@@ -190,13 +271,13 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
                     const int kk = k0 + b_vec * 4;
                     v4f v = {0.f, 0.f, 0.f, 0.f};
                     if (r < g.n) {
-                        const float *src = b_src + p * b_pass_stride;
+                        const BE *src = b_src + p * b_pass_stride;
                         if (vec_ok && kk + 3 < k_end) {
-                            v = *reinterpret_cast<const v4f *>(src);
+                            v = load_b4(src);
                         } else {
 #pragma unroll
                             for (int j = 0; j < 4; ++j)
-                                if (kk + j < k_end) v[j] = src[j];
+                                if (kk + j < k_end) v[j] = load_b1(src + j);
                         }
                     }
                     b_reg[p] = v;
@@ -206,13 +287,13 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
                 const int c = n0 + b_vec * 4;
                 v4f v = {0.f, 0.f, 0.f, 0.f};
                 if (kk < k_end) {
-                    const float *src = b_src + p * b_pass_stride;
+                    const BE *src = b_src + p * b_pass_stride;
                     if (vec_ok && c + 3 < g.n) {
-                        v = *reinterpret_cast<const v4f *>(src);
+                        v = load_b4(src);
                     } else {
 #pragma unroll
                         for (int j = 0; j < 4; ++j)
-                            if (c + j < g.n) v[j] = src[j];
+                            if (c + j < g.n) v[j] = load_b1(src + j);
                     }
                 }
                 b_reg[p] = v;
@@ -368,9 +449,19 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
 // EDGE: m and n need not be whole tiles (K steps stay whole, rows 16-byte aligned). Rows and columns
 // past the end are fetched from the last valid row / 16-byte unit instead -- what they feed is
 // never stored -- so the main loop is the same; only the stores are guarded.
-template <int BM, int BN, int WM, int WN, bool TB, int STAGES, bool SWIGLU = false, bool EDGE = false>
+//
+// WS: a K-contiguous B stored as 16-bit values. LDS holds floats in the same swizzled layout, so
+// fragments, MFMAs and epilogue are those of the fp32 kernel and the result equals the fp32 product
+// over the widened weights bit for bit. Only B's way into LDS differs: every lane fetches 128-bit
+// units of eight weights into registers one K step ahead of A's direct loads, and widens and stores
+// them as two units of four floats at the start of the next step (dealt out between the MFMAs like
+// every other instruction of a step).
+template <int BM, int BN, int WM, int WN, bool TB, int STAGES, bool SWIGLU = false, bool EDGE = false,
+          typename WS = StoredF32>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) {
     static_assert(STAGES == 2, "two LDS stages");
+    constexpr bool B16 = kStored16<WS>;
+    static_assert(!B16 || TB, "16-bit weights are K-contiguous");
     static_assert(!SWIGLU || WN == 64,
                   "SwiGLU epilogue: two accumulator columns (EDGE: partial tiles in m only)");
     constexpr int BK = 32;
@@ -385,8 +476,12 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     constexpr int WAVES_N = BN / WN;
     static_assert((BM / WM) * (BN / WN) == kThreads / kWave, "four wavefronts per block");
     constexpr int A_PASSES = BM / 32;   // 1 KiB pieces (8 rows of A) per wavefront and stage
-    constexpr int B_PASSES = BN / 32;
+    constexpr int B_PASSES = B16 ? 0 : BN / 32;
     constexpr int B_ROW_UNITS = BN / 4;             // 16-byte units per K-row of a row-major B tile
+    // 16-bit B: 128-bit units of eight weights per stage (four per row), dealt to the 256 lanes
+    constexpr int B16_UNITS = BN * 4;
+    constexpr int B16_PASSES = B16 ? (B16_UNITS + kThreads - 1) / kThreads : 0;
+    constexpr int kB16Slots = B16_PASSES > 0 ? B16_PASSES : 1;
 
     int tile_m, tile_n, split;
     tile_coords(g, tile_m, tile_n, split);
@@ -410,7 +505,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     // wave-uniform base (scalar registers, advanced by one K step with scalar adds) plus a per-lane
     // byte offset per piece that never changes, so the loads cost no vector ALU work.
     const int sw_row = lane / 8, sw_unit = (lane % 8) ^ sw_row;
-    uint32_t a_voff[A_PASSES], b_voff[B_PASSES];
+    uint32_t a_voff[A_PASSES], b_voff[B_PASSES > 0 ? B_PASSES : 1];
     const float *a_ptr = A + static_cast<int64_t>(m0) * g.lda + k_begin;
 #pragma unroll
     for (int p = 0; p < A_PASSES; ++p) {
@@ -418,9 +513,34 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
         if constexpr (EDGE) row = min(row, g.m - 1 - m0);
         a_voff[p] = static_cast<uint32_t>((row * g.lda + sw_unit * 4) * static_cast<int64_t>(4));
     }
-    const float *b_ptr;
-    int64_t b_step_stride;
-    if constexpr (TB) {
+    const float *b_ptr = nullptr;
+    int64_t b_step_stride = 0;
+    // 16-bit B: the unit this lane fetches in pass p, as a byte offset from b16_ptr (which walks K),
+    // and the float index of the first of the two LDS units it becomes (stage 0)
+    [[maybe_unused]] const uint16_t *b16_ptr = nullptr;
+    [[maybe_unused]] uint32_t b16_voff[kB16Slots];
+    [[maybe_unused]] int b16_lds[kB16Slots][2];
+    [[maybe_unused]] v4u b_raw[kB16Slots];
+    if constexpr (B16) {
+        b16_ptr = reinterpret_cast<const uint16_t *>(g.b) + batch * g.stride_b +
+                  (SWIGLU ? 0 : static_cast<int64_t>(n0) * g.ldb) + k_begin;
+#pragma unroll
+        for (int p = 0; p < B16_PASSES; ++p) {
+            const int id = min(p * kThreads + tid, B16_UNITS - 1);
+            const int lrow = id / 4, u = id % 4;       // row of the tile, unit of eight weights in it
+            int row = lrow;
+            if constexpr (SWIGLU) {
+                // LDS row r: wavefront column r / 64, accumulator (r % 64) / 32, lane r % 32
+                const int out_col = tile_n * (BN / 2) + (row / 64) * 32 + row % 32;
+                row = ((row % 64) / 32 ? g.up_offset : g.gate_offset) + out_col;
+            } else if constexpr (EDGE) {
+                row = min(row, g.n - 1 - n0);
+            }
+            b16_voff[p] = static_cast<uint32_t>((row * g.ldb + u * 8) * static_cast<int64_t>(2));
+            b16_lds[p][0] = lrow * BK + ((2 * u) ^ (lrow & 7)) * 4;
+            b16_lds[p][1] = lrow * BK + ((2 * u + 1) ^ (lrow & 7)) * 4;
+        }
+    } else if constexpr (TB) {
         b_ptr = B + (SWIGLU ? 0 : static_cast<int64_t>(n0) * g.ldb) + k_begin;
         b_step_stride = BK;
 #pragma unroll
@@ -480,6 +600,25 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
         a_ptr += BK;
         b_ptr += b_step_stride;
     };
+    // 16-bit B: request pass p of the stage b16_ptr stands at; widen and store pass p of the stage in
+    // the registers to LDS buffer `buf`
+    [[maybe_unused]] auto b16_load = [&](int p) {
+        if constexpr (B16) {
+            if (B16_UNITS % kThreads == 0 || p * kThreads + tid < B16_UNITS)
+                b_raw[p] = *reinterpret_cast<const v4u *>(reinterpret_cast<const char *>(b16_ptr) + b16_voff[p]);
+        }
+    };
+    [[maybe_unused]] auto b16_store = [&](int buf, int p) {
+        if constexpr (B16) {
+            if (B16_UNITS % kThreads == 0 || p * kThreads + tid < B16_UNITS) {
+                float w[8];
+                widen_unit<WS>(b_raw[p], w);
+                float *bs = Bs + buf * kBFloats;
+                *reinterpret_cast<v4f *>(bs + b16_lds[p][0]) = v4f{w[0], w[1], w[2], w[3]};
+                *reinterpret_cast<v4f *>(bs + b16_lds[p][1]) = v4f{w[4], w[5], w[6], w[7]};
+            }
+        }
+    };
 
     // fragment addressing
     const int xr = l32 & 7;
@@ -532,9 +671,10 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     constexpr int kLoadChunks = 1;   // chunks (from the first) that carry the loads
     constexpr int kLoadsPerChunk = (kLoadsPerStage + kLoadChunks - 1) / kLoadChunks;
     constexpr int kBarrierAt = NM * 2 / 4 < NM - 1 ? NM * 2 / 4 : NM - 2;
-    auto k_step = [&](int buf, auto load_tag, auto more_tag) {
+    auto k_step = [&](int buf, auto load_tag, auto more_tag, auto load2_tag) {
         constexpr bool LOAD = decltype(load_tag)::value;   // another stage to fetch
         constexpr bool MORE = decltype(more_tag)::value;   // another step follows
+        constexpr bool LOAD2 = decltype(load2_tag)::value; // 16-bit B: a stage after that one to request
         const int other = buf ^ 1;
         static_for<KC>([&](auto kc_tag) {
             constexpr int kc = decltype(kc_tag)::value;
@@ -549,7 +689,12 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
                                                                          : kLoadsPerStage)
                            : 0;
             constexpr int n_frag = last ? (MORE ? kFragOps : 0) : kFragOps;
-            constexpr int n_ops = n_frag + (load_hi - load_lo);
+            // 16-bit B, first chunk: the stage in the registers goes to LDS before the loads of this
+            // step are issued, the stage after it is requested behind them
+            constexpr int n_store = B16 && LOAD && kc == 0 ? B16_PASSES : 0;
+            constexpr int n_direct = load_hi - load_lo;
+            constexpr int n_b16 = B16 && LOAD2 && kc == 0 ? B16_PASSES : 0;
+            constexpr int n_ops = n_frag + n_store + n_direct + n_b16;
             constexpr int first = last ? kBarrierAt + 1 : 0;     // first MFMA that carries an op
             constexpr int room = NM - first;
             static_for<NM>([&](auto q_tag) {
@@ -565,14 +710,19 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
                         if constexpr (o < n_frag) {
                             if constexpr (last) frag_op(other, 0, slot ^ 1, o);
                             else frag_op(buf, kc + 1, slot ^ 1, o);
+                        } else if constexpr (o < n_frag + n_store) {
+                            b16_store(other, o - n_frag);
+                        } else if constexpr (o < n_frag + n_store + n_direct) {
+                            load_op(other, load_lo + o - n_frag - n_store);
                         } else {
-                            load_op(other, load_lo + o - n_frag);
+                            b16_load(o - n_frag - n_store - n_direct);
                         }
                     }
                 });
                 __builtin_amdgcn_sched_barrier(0);
             });
             if constexpr (LOAD && kc == kLoadChunks - 1) advance_sources();
+            if constexpr (B16 && LOAD2 && kc == 0) b16_ptr += BK;
         });
     };
 
@@ -580,15 +730,39 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
 #pragma unroll
         for (int o = 0; o < kLoadsPerStage; ++o) load_op(0, o);
         advance_sources();
+        if constexpr (B16) {
+            // stage 0 of B through the registers, then stage 1 requested
+#pragma unroll
+            for (int p = 0; p < B16_PASSES; ++p) b16_load(p);
+            b16_ptr += BK;
+#pragma unroll
+            for (int p = 0; p < B16_PASSES; ++p) b16_store(0, p);
+            if (n_steps > 1) {
+#pragma unroll
+                for (int p = 0; p < B16_PASSES; ++p) b16_load(p);
+                b16_ptr += BK;
+            }
+        }
         stage_barrier();
 #pragma unroll
         for (int o = 0; o < kFragOps; ++o) frag_op(0, 0, 0, o);
         int buf = 0;
-        for (int step = 0; step + 1 < n_steps; ++step) {
-            k_step(buf, std::true_type{}, std::true_type{});
-            buf ^= 1;
+        if constexpr (B16) {
+            for (int step = 0; step + 2 < n_steps; ++step) {
+                k_step(buf, std::true_type{}, std::true_type{}, std::true_type{});
+                buf ^= 1;
+            }
+            if (n_steps > 1) {
+                k_step(buf, std::true_type{}, std::true_type{}, std::false_type{});
+                buf ^= 1;
+            }
+        } else {
+            for (int step = 0; step + 1 < n_steps; ++step) {
+                k_step(buf, std::true_type{}, std::true_type{}, std::false_type{});
+                buf ^= 1;
+            }
         }
-        k_step(buf, std::false_type{}, std::false_type{});
+        k_step(buf, std::false_type{}, std::false_type{}, std::false_type{});
     }
 
     if constexpr (SWIGLU) {
@@ -927,24 +1101,28 @@ __global__ __launch_bounds__(kThreads) void skinny_kernel(SkinnyArgs g) {
 }
 
 // B stored [n][k] (C = A . B^T): a wavefront per output column, ROWS dots along contiguous k.
-template <int ROWS>
+// (WS: B may be stored as 16-bit values, see StoredF16; g.w, ldb and stride_w then count those.)
+template <int ROWS, typename WS = StoredF32>
 __global__ __launch_bounds__(kThreads) void skinny_dot_kernel(SkinnyArgs g) {
+    using E = typename WS::elem;
     const int lane = threadIdx.x % kWave;
     const int batch = blockIdx.y;
     const float *x = g.x + batch * g.stride_x;
-    const float *w = g.w + batch * g.stride_w;
+    const E *w = reinterpret_cast<const E *>(g.w) + batch * g.stride_w;
     float *y = g.y + batch * g.stride_y;
     const float *xr[ROWS];
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) xr[r] = x + static_cast<int64_t>(min(r, g.m - 1)) * g.lda;
     for (int n = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave; n < g.n;
          n += gridDim.x * (kThreads / kWave)) {
-        const float *wr = w + static_cast<int64_t>(n) * g.ldb;
+        const E *wr = w + static_cast<int64_t>(n) * g.ldb;
         float acc[ROWS];
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) acc[r] = 0.f;
         for (int kk = lane; kk < g.k; kk += kWave) {
-            const float wv = wr[kk];
+            float wv;
+            if constexpr (kStored16<WS>) wv = WS::widen(wr[kk]);
+            else wv = wr[kk];
 #pragma unroll
             for (int r = 0; r < ROWS; ++r) acc[r] = fmaf(xr[r][kk], wv, acc[r]);
         }
@@ -958,18 +1136,24 @@ __global__ __launch_bounds__(kThreads) void skinny_dot_kernel(SkinnyArgs g) {
 }
 
 // GEMV with W stored [n][k] (trans_b): a wavefront per output column, dot along contiguous k.
+template <typename WS = StoredF32>
 __global__ __launch_bounds__(kThreads) void gemv_dot_kernel(GemvArgs g) {
+    using E = typename WS::elem;
     const int lane = threadIdx.x % kWave;
     const int batch = blockIdx.y;
     const float *x = g.x + batch * g.stride_x;
-    const float *w = g.w + batch * g.stride_w;
+    const E *w = reinterpret_cast<const E *>(g.w) + batch * g.stride_w;
     float *y = g.y + batch * g.stride_y;
     for (int n = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave; n < g.n;
          n += gridDim.x * (kThreads / kWave)) {
-        const float *wr = w + static_cast<int64_t>(n) * g.ldb;
+        const E *wr = w + static_cast<int64_t>(n) * g.ldb;
         float acc = 0.f;
-        for (int kk = lane; kk < g.k; kk += kWave)
-            acc = fmaf(x[static_cast<int64_t>(kk) * g.x_inc], wr[kk], acc);
+        for (int kk = lane; kk < g.k; kk += kWave) {
+            float wv;
+            if constexpr (kStored16<WS>) wv = WS::widen(wr[kk]);
+            else wv = wr[kk];
+            acc = fmaf(x[static_cast<int64_t>(kk) * g.x_inc], wv, acc);
+        }
 #pragma unroll
         for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, kWave);
         if (lane == 0) y[n] = acc;
@@ -1014,16 +1198,22 @@ struct NoExtraLoads {
 // NU: 128-bit units of the row a lane holds during the NORM prologue (k <= 256 * NU * 4); the
 // common k <= 2048 takes NU = 2 and with it 48 registers less than NU = 8, i.e. five or six
 // resident wavefronts per SIMD instead of four.
-template <int COLS, bool NORM, int NU = kGemvNormUnits, typename Extra = NoExtraLoads>
+// WS, DEPTH: how the weights are stored and how many 128-bit units of a row a lane requests per
+// chunk. A unit of 16-bit weights meets two units of x; rows of up to 2048 such weights are one
+// chunk of four units per lane, longer ones chunks of eight.
+template <int COLS, bool NORM, int NU = kGemvNormUnits, typename WS = StoredF32, int DEPTH = kGemvDepth,
+          typename Extra = NoExtraLoads>
 __device__ __forceinline__ void gemv_wave_dots(const float *__restrict__ x, const v4f *const (&wv)[COLS],
                                                int32_t k, const RowNormArgs &norm, bool active,
                                                float (&acc)[COLS], Extra extra_loads = Extra()) {
     constexpr int kWaves = kThreads / kWave;
+    constexpr int kX = WS::kUnit / 4;          // units of x one unit of weights meets
     // the normalised row of the block (NORM): k floats of dynamic LDS
     extern __shared__ __align__(16) float xs[];
     __shared__ double partial[kWaves];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    const int k4 = k / 4;
+    const int k4 = k / 4;                      // units of x
+    const int kw = k / WS::kUnit;              // units of a row of weights
     const v4f *xv = reinterpret_cast<const v4f *>(x);
     // NORM: this lane's share of the row and of gamma, requested before any weight
     [[maybe_unused]] v4f xn[NU], gn[NU];
@@ -1038,28 +1228,41 @@ __device__ __forceinline__ void gemv_wave_dots(const float *__restrict__ x, cons
             }
         }
     }
-    // Chunks of kGemvDepth * 64 units. Whole chunks are addressed as pointer + constant (the loads
+    // Chunks of DEPTH * 64 units. Whole chunks are addressed as pointer + constant (the loads
     // carry their offsets as immediates: with two wavefronts per SIMD, as on the 2048-wide outputs,
     // address arithmetic per load is time nothing else covers - it cost the k = 8192 product 2 us);
-    // the last, partial chunk of a k that is no multiple of 2048 clamps its units and zeroes them.
-    constexpr int kChunkUnits = kWave * kGemvDepth;
-    const int full_chunks = k4 / kChunkUnits;
-    v4f wr[kGemvDepth][COLS];
+    // the last, partial chunk of a row that is no whole number of chunks clamps its units and
+    // zeroes them.
+    constexpr int kChunkUnits = kWave * DEPTH;
+    const int full_chunks = kw / kChunkUnits;
+    v4f wr[DEPTH][COLS];
     auto load_w = [&](int chunk, bool partial_chunk) {
         if (!partial_chunk) {
 #pragma unroll
             for (int c = 0; c < COLS; ++c) {
                 const v4f *p = wv[c] + chunk * kChunkUnits + lane;
 #pragma unroll
-                for (int j = 0; j < kGemvDepth; ++j) wr[j][c] = __builtin_nontemporal_load(p + j * kWave);
+                for (int j = 0; j < DEPTH; ++j) wr[j][c] = __builtin_nontemporal_load(p + j * kWave);
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < kGemvDepth; ++j) {
-                const int u = min(chunk * kChunkUnits + lane + j * kWave, k4 - 1);
+            for (int j = 0; j < DEPTH; ++j) {
+                const int u = min(chunk * kChunkUnits + lane + j * kWave, kw - 1);
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) wr[j][c] = __builtin_nontemporal_load(wv[c] + u);
             }
+        }
+    };
+    // one unit of weights against the units of x under it
+    auto unit_fma = [&](const v4f (&xu)[kX], const v4f &w, float &sum) {
+        if constexpr (kStored16<WS>) {
+            float wf[8];
+            widen_unit<WS>(__builtin_bit_cast(v4u, w), wf);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sum = fmaf(xu[e / 4][e % 4], wf[e], sum);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum = fmaf(xu[0][e], w[e], sum);
         }
     };
     load_w(0, full_chunks == 0);      // in flight during the NORM prologue
@@ -1109,41 +1312,43 @@ __device__ __forceinline__ void gemv_wave_dots(const float *__restrict__ x, cons
     const v4f *xsrc = NORM ? reinterpret_cast<const v4f *>(xs) : xv;
     for (int chunk = 0; chunk < full_chunks; ++chunk) {
         if (chunk > 0) load_w(chunk, false);
-        const v4f *px = xsrc + chunk * kChunkUnits + lane;
-        v4f xr[kGemvDepth];
+        const v4f *px = xsrc + (chunk * kChunkUnits + lane) * kX;
+        v4f xr[DEPTH][kX];
 #pragma unroll
-        for (int j = 0; j < kGemvDepth; ++j) xr[j] = px[j * kWave];
+        for (int j = 0; j < DEPTH; ++j)
 #pragma unroll
-        for (int j = 0; j < kGemvDepth; ++j)
+            for (int h = 0; h < kX; ++h) xr[j][h] = px[j * kWave * kX + h];
 #pragma unroll
-            for (int c = 0; c < COLS; ++c)
+        for (int j = 0; j < DEPTH; ++j)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[c] = fmaf(xr[j][e], wr[j][c][e], acc[c]);
+            for (int c = 0; c < COLS; ++c) unit_fma(xr[j], wr[j][c], acc[c]);
     }
-    if (full_chunks * kChunkUnits < k4) {
+    if (full_chunks * kChunkUnits < kw) {
         if (full_chunks > 0) load_w(full_chunks, true);
 #pragma unroll
-        for (int j = 0; j < kGemvDepth; ++j) {
+        for (int j = 0; j < DEPTH; ++j) {
             const int u = full_chunks * kChunkUnits + lane + j * kWave;
-            v4f xr = xsrc[min(u, k4 - 1)];
-            if (u >= k4) {
-                xr = v4f{0.f, 0.f, 0.f, 0.f};
+            v4f xr[kX];
+#pragma unroll
+            for (int h = 0; h < kX; ++h) xr[h] = xsrc[min(u, kw - 1) * kX + h];
+            if (u >= kw) {
+#pragma unroll
+                for (int h = 0; h < kX; ++h) xr[h] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) wr[j][c] = v4f{0.f, 0.f, 0.f, 0.f};
             }
 #pragma unroll
-            for (int c = 0; c < COLS; ++c)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc[c] = fmaf(xr[e], wr[j][c][e], acc[c]);
+            for (int c = 0; c < COLS; ++c) unit_fma(xr, wr[j][c], acc[c]);
         }
     }
 #pragma unroll
     for (int c = 0; c < COLS; ++c) acc[c] = wave_sum(acc[c]);
 }
 
-template <bool SWIGLU = false, bool NORM = false, int NU = kGemvNormUnits>
+template <bool SWIGLU = false, bool NORM = false, int NU = kGemvNormUnits, typename WS = StoredF32,
+          int DEPTH = kGemvDepth>
 __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__restrict__ x,
-                                                          const float *__restrict__ wt,
+                                                          const typename WS::elem *__restrict__ wt,
                                                           float *__restrict__ y, int32_t n, int32_t k,
                                                           int64_t ldw, int32_t gate_row, int32_t up_row,
                                                           const float *__restrict__ residual,
@@ -1163,7 +1368,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__re
     const v4f *wv[1];
     wv[0] = reinterpret_cast<const v4f *>(wt + row * ldw);
     float acc[1];
-    gemv_wave_dots<1, NORM, NU>(x, wv, k, norm, col < n, acc);
+    gemv_wave_dots<1, NORM, NU, WS, DEPTH>(x, wv, k, norm, col < n, acc);
     if constexpr (SWIGLU) {
         if (lane == 0) pair_acc[wave] = acc[0];
         __syncthreads();
@@ -1201,9 +1406,10 @@ struct GemvRowStreams {
     int32_t *err;
 };
 
-template <bool NORM, int NU = kGemvNormUnits>
+template <bool NORM, int NU = kGemvNormUnits, typename WS = StoredF32, int DEPTH = kGemvDepth>
 __global__ __launch_bounds__(kThreads) void gemv_kmajor_rows_kernel(const float *__restrict__ x,
-                                                                    const float *__restrict__ wt, int32_t k,
+                                                                    const typename WS::elem *__restrict__ wt,
+                                                                    int32_t k,
                                                                     int64_t ldw, RowNormArgs norm,
                                                                     GemvRowStreams rs) {
     // A wavefront per column, like the plain product (two columns per wavefront left the SIMDs with
@@ -1248,7 +1454,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_rows_kernel(const float 
         }
     };
     float acc[1];
-    gemv_wave_dots<1, NORM, NU>(x, wv, k, norm, active, acc, epilogue_loads);
+    gemv_wave_dots<1, NORM, NU, WS, DEPTH>(x, wv, k, norm, active, acc, epilogue_loads);
     if (lane == 0) pair_acc[wave] = acc[0];
     __syncthreads();
     if (!active || lane != 0 || second) return;
@@ -1420,10 +1626,10 @@ inline int gemv_splits(int64_t batch, int64_t n, int64_t k, int cols_per_block, 
     return static_cast<int>((k + kps - 1) / kps);
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool TB = false>
+template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool TB = false, typename WS = StoredF32>
 int32_t launch_mfma(hipStream_t s, const GemmArgs &g, int64_t batch, int splits) {
     using L = SmemLayout<BM, BN, BK, TB>;
-    auto kern = gemm_mfma_kernel<BM, BN, BK, WM, WN, EDGE, TB>;
+    auto kern = gemm_mfma_kernel<BM, BN, BK, WM, WN, EDGE, TB, WS>;
     if (L::kBytes > 64 * 1024) {
         static DynamicLdsGrant grant;   // one per instantiation, i.e. per kernel
         const int32_t st = grant.ensure(kern, L::kBytes);
@@ -1435,10 +1641,11 @@ int32_t launch_mfma(hipStream_t s, const GemmArgs &g, int64_t batch, int splits)
     return launch_status();
 }
 
-template <int BM, int BN, int WM, int WN, bool TB, int STAGES, bool SWIGLU = false, bool EDGE = false>
+template <int BM, int BN, int WM, int WN, bool TB, int STAGES, bool SWIGLU = false, bool EDGE = false,
+          typename WS = StoredF32>
 int32_t launch_direct(hipStream_t s, const GemmArgs &g, int64_t batch, int splits) {
     constexpr int kBytes = STAGES * (BM * 32 + 32 * BN) * 4;
-    auto kern = gemm_mfma_direct_kernel<BM, BN, WM, WN, TB, STAGES, SWIGLU, EDGE>;
+    auto kern = gemm_mfma_direct_kernel<BM, BN, WM, WN, TB, STAGES, SWIGLU, EDGE, WS>;
     if (kBytes > 64 * 1024) {
         static DynamicLdsGrant grant;   // one per instantiation, i.e. per kernel
         const int32_t st = grant.ensure(kern, kBytes);
@@ -1453,11 +1660,18 @@ int32_t launch_direct(hipStream_t s, const GemmArgs &g, int64_t batch, int split
 // The tiled MFMA path of a product (m > 1, A not transposed). `seg`: column blocks of C with their
 // own destinations (see Segments; their rows must be 16-byte aligned) instead of c/ldc; the call
 // then answers RMLK_ERR_UNSUPPORTED unless the whole-tile kernel applies.
+// b_dtype: how B is stored (RMLK_FLOAT, or a 16-bit type for a K-contiguous B; ldb and stride_b
+// count stored values).
 int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k, const float *pa,
-                   int64_t lda, int64_t stride_a, const float *pb, int64_t ldb, int64_t stride_b,
-                   int32_t trans_b, float *pc, int64_t ldc, int64_t stride_c, void *workspace,
-                   size_t workspace_bytes, const Segments *seg, int32_t *partial_splits = nullptr) {
-    const bool aligned = lda % 4 == 0 && ldb % 4 == 0 && stride_a % 4 == 0 && stride_b % 4 == 0 &&
+                   int64_t lda, int64_t stride_a, int32_t b_dtype, const void *pb, int64_t ldb,
+                   int64_t stride_b, int32_t trans_b, float *pc, int64_t ldc, int64_t stride_c,
+                   void *workspace, size_t workspace_bytes, const Segments *seg,
+                   int32_t *partial_splits = nullptr) {
+    const bool b16 = b_dtype != RMLK_FLOAT;
+    if (b16 && !trans_b) return RMLK_ERR_UNSUPPORTED;
+    // (rows of 16-bit values: whole 128-bit units)
+    const int64_t b_unit = b16 ? 8 : 4;
+    const bool aligned = lda % 4 == 0 && ldb % b_unit == 0 && stride_a % 4 == 0 && stride_b % b_unit == 0 &&
                          reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
                          reinterpret_cast<uintptr_t>(pb) % 16 == 0;
     // the direct-to-LDS kernel: whole K steps and aligned rows; partial tiles in m and n are fine
@@ -1470,7 +1684,7 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
     if ((t.bn == 192 || t.bn == 96 || (t.bm == 128 && t.bn == 64)) && !direct_ok(t)) t = choose_tiles(batch, m, n, k, false);
     GemmArgs g{};
     g.a = pa;
-    g.b = pb;
+    g.b = static_cast<const float *>(pb);   // (the kernels of a 16-bit B read it as such)
     g.m = static_cast<int32_t>(m);
     g.n = static_cast<int32_t>(n);
     g.k = static_cast<int32_t>(k);
@@ -1507,23 +1721,6 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
     g.aligned = aligned ? 1 : 0;
     const bool full = aligned && m % t.bm == 0 && n % t.bn == 0 && t.k_per_split % t.bk == 0 &&
                       k % t.k_per_split == 0;
-    int32_t st;
-#define RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, TB_)                                                   \
-    (t.bk == 32                                                                                  \
-         ? (full ? launch_mfma<BM_, BN_, 32, WM_, WN_, false, TB_>(s, g, batch, t.splits)        \
-                 : launch_mfma<BM_, BN_, 32, WM_, WN_, true, TB_>(s, g, batch, t.splits))        \
-         : (full ? launch_mfma<BM_, BN_, 16, WM_, WN_, false, TB_>(s, g, batch, t.splits)        \
-                 : launch_mfma<BM_, BN_, 16, WM_, WN_, true, TB_>(s, g, batch, t.splits)))
-#define RMLK_LAUNCH(BM_, BN_, WM_, WN_)                                                          \
-    (trans_b ? RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, true) : RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, false))
-#define RMLK_DIRECT_E(BM_, BN_, WM_, WN_, S_, E_)                                                \
-    (trans_b ? launch_direct<BM_, BN_, WM_, WN_, true, S_, false, E_>(s, g, batch, t.splits)     \
-             : launch_direct<BM_, BN_, WM_, WN_, false, S_, false, E_>(s, g, batch, t.splits))
-#define RMLK_DIRECT_S(BM_, BN_, WM_, WN_, S_)                                                    \
-    (whole ? RMLK_DIRECT_E(BM_, BN_, WM_, WN_, S_, false) : RMLK_DIRECT_E(BM_, BN_, WM_, WN_, S_, true))
-    // two LDS stages: a third (loads two K steps ahead) measured no faster and halves the blocks
-    // that fit a CU
-#define RMLK_DIRECT(BM_, BN_, WM_, WN_) RMLK_DIRECT_S(BM_, BN_, WM_, WN_, 2)
     const bool whole = m % t.bm == 0 && n % t.bn == 0;
     const bool direct = direct_ok(t);
     if (seg) {
@@ -1532,19 +1729,38 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
         for (int i = 0; i <= seg->n_seg; ++i)
             if (seg->begin[i] % 32 != 0) return RMLK_ERR_UNSUPPORTED;
     }
-    if (direct && t.bm == 256) st = RMLK_DIRECT(256, 64, 64, 64);
-    else if (direct && t.bn == 192) st = RMLK_DIRECT(128, 192, 64, 96);
-    else if (direct && t.bn == 96) st = RMLK_DIRECT(128, 96, 32, 96);
-    else if (direct && t.bm == 128 && t.bn == 64) st = RMLK_DIRECT(128, 64, 64, 32);
-    else if (direct && t.bm == 128) st = RMLK_DIRECT(128, 128, 64, 64);
-    else if (direct) st = RMLK_DIRECT(64, 64, 32, 32);
-    else if (t.bm == 256) st = RMLK_LAUNCH(256, 64, 64, 64);
-    else if (t.bm == 128) st = RMLK_LAUNCH(128, 128, 64, 64);
-    else st = RMLK_LAUNCH(64, 64, 32, 32);
+#define RMLK_LAUNCH_TB(BM_, BN_, WM_, WN_, TB_, WS_)                                              \
+    (t.bk == 32                                                                                  \
+         ? (full ? launch_mfma<BM_, BN_, 32, WM_, WN_, false, TB_, WS_>(s, g, batch, t.splits)   \
+                 : launch_mfma<BM_, BN_, 32, WM_, WN_, true, TB_, WS_>(s, g, batch, t.splits))   \
+         : (full ? launch_mfma<BM_, BN_, 16, WM_, WN_, false, TB_, WS_>(s, g, batch, t.splits)   \
+                 : launch_mfma<BM_, BN_, 16, WM_, WN_, true, TB_, WS_>(s, g, batch, t.splits)))
+#define RMLK_DIRECT_E(BM_, BN_, WM_, WN_, TB_, E_, WS_)                                           \
+    launch_direct<BM_, BN_, WM_, WN_, TB_, 2, false, E_, WS_>(s, g, batch, t.splits)
+    // two LDS stages: a third (loads two K steps ahead) measured no faster and halves the blocks
+    // that fit a CU
+#define RMLK_DIRECT(BM_, BN_, WM_, WN_, TB_, WS_)                                                 \
+    (whole ? RMLK_DIRECT_E(BM_, BN_, WM_, WN_, TB_, false, WS_) : RMLK_DIRECT_E(BM_, BN_, WM_, WN_, TB_, true, WS_))
+    // every tile shape for one layout and storage of B
+    auto launch_layout = [&](auto tb_tag, auto ws) -> int32_t {
+        constexpr bool TB_ = decltype(tb_tag)::value;
+        using WS_ = decltype(ws);
+        if (direct && t.bm == 256) return RMLK_DIRECT(256, 64, 64, 64, TB_, WS_);
+        if (direct && t.bn == 192) return RMLK_DIRECT(128, 192, 64, 96, TB_, WS_);
+        if (direct && t.bn == 96) return RMLK_DIRECT(128, 96, 32, 96, TB_, WS_);
+        if (direct && t.bm == 128 && t.bn == 64) return RMLK_DIRECT(128, 64, 64, 32, TB_, WS_);
+        if (direct && t.bm == 128) return RMLK_DIRECT(128, 128, 64, 64, TB_, WS_);
+        if (direct) return RMLK_DIRECT(64, 64, 32, 32, TB_, WS_);
+        if (t.bm == 256) return RMLK_LAUNCH_TB(256, 64, 64, 64, TB_, WS_);
+        if (t.bm == 128) return RMLK_LAUNCH_TB(128, 128, 64, 64, TB_, WS_);
+        return RMLK_LAUNCH_TB(64, 64, 32, 32, TB_, WS_);
+    };
+    int32_t st = with_storage(b_dtype, [&](auto ws) -> int32_t {
+        if constexpr (kStored16<decltype(ws)>) return launch_layout(std::true_type{}, ws);
+        else return trans_b ? launch_layout(std::true_type{}, ws) : launch_layout(std::false_type{}, ws);
+    });
 #undef RMLK_DIRECT
-#undef RMLK_DIRECT_S
 #undef RMLK_DIRECT_E
-#undef RMLK_LAUNCH
 #undef RMLK_LAUNCH_TB
     if (st) return st;
     if (partial_splits) {
@@ -1577,9 +1793,11 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
 // silu(A . B[:, gate..]) * (A . B[:, up..]) in one launch: 128 x 128 tiles of 64 gate and 64 up
 // columns. Whole tiles in n and k, no split-K, enough tiles to cover the chip; otherwise UNSUPPORTED.
 int32_t gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float *pa, int64_t lda,
-                    const float *pb, int64_t ldb, int32_t trans_b, int64_t gate_offset, int64_t up_offset,
-                    float *pc, int64_t ldc) {
-    const bool aligned = lda % 4 == 0 && ldb % 4 == 0 && gate_offset % 4 == 0 && up_offset % 4 == 0 &&
+                    int32_t b_dtype, const void *pb, int64_t ldb, int32_t trans_b, int64_t gate_offset,
+                    int64_t up_offset, float *pc, int64_t ldc) {
+    const bool b16 = b_dtype != RMLK_FLOAT;
+    if (b16 && !trans_b) return RMLK_ERR_UNSUPPORTED;
+    const bool aligned = lda % 4 == 0 && ldb % (b16 ? 8 : 4) == 0 && gate_offset % 4 == 0 && up_offset % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
                          reinterpret_cast<uintptr_t>(pb) % 16 == 0;
     if (!aligned || n % 64 != 0 || k % 32 != 0 || k < 32 || lda >= (1ll << 21) || ldb >= (1ll << 21))
@@ -1590,7 +1808,7 @@ int32_t gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float 
     if (tiles < kNumCU || tiles >= (1ll << 31)) return RMLK_ERR_UNSUPPORTED;
     GemmArgs g{};
     g.a = pa;
-    g.b = pb;
+    g.b = static_cast<const float *>(pb);
     g.c = pc;
     g.m = static_cast<int32_t>(m);
     g.n = static_cast<int32_t>(2 * n);
@@ -1608,8 +1826,11 @@ int32_t gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float 
         // (a lane's byte offset into B covers a row number of the whole matrix here)
         const int64_t last_row = (gate_offset > up_offset ? gate_offset : up_offset) + n;
         if (last_row * ldb >= (1ll << 30)) return RMLK_ERR_UNSUPPORTED;
-        if (m % 128 == 0) return launch_direct<128, 128, 64, 64, true, 2, true, false>(s, g, 1, 1);
-        return launch_direct<128, 128, 64, 64, true, 2, true, true>(s, g, 1, 1);
+        return with_storage(b_dtype, [&](auto ws) -> int32_t {
+            using WS = decltype(ws);
+            if (m % 128 == 0) return launch_direct<128, 128, 64, 64, true, 2, true, false, WS>(s, g, 1, 1);
+            return launch_direct<128, 128, 64, 64, true, 2, true, true, WS>(s, g, 1, 1);
+        });
     }
     if (m % 128 == 0) return launch_direct<128, 128, 64, 64, false, 2, true, false>(s, g, 1, 1);
     return launch_direct<128, 128, 64, 64, false, 2, true, true>(s, g, 1, 1);
@@ -1676,12 +1897,52 @@ extern "C" int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_
     return len + 1;
 }
 
-extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t m,
-                                   int64_t n, int64_t k, const void *a, int64_t lda,
-                                   int64_t stride_a, int32_t trans_a, const void *b, int64_t ldb,
-                                   int64_t stride_b, int32_t trans_b, void *c, int64_t ldc,
-                                   int64_t stride_c, void *workspace, size_t workspace_bytes) {
+namespace {
+// float -> 16-bit storage, round to nearest even
+template <typename WS>
+__global__ __launch_bounds__(kThreads) void store_weights_kernel(const float *__restrict__ src,
+                                                                 uint16_t *__restrict__ dst, int64_t n) {
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n;
+         i += static_cast<int64_t>(gridDim.x) * kThreads) {
+        const float v = src[i];
+        if constexpr (std::is_same<WS, StoredF16>::value) {
+            dst[i] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
+        } else {
+            uint32_t u = __float_as_uint(v);
+            if ((u & 0x7fffffffu) > 0x7f800000u) u = (u >> 16) | 0x40u;            // NaN stays (quiet) NaN
+            else u = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;                        // ties to even
+            dst[i] = static_cast<uint16_t>(u);
+        }
+    }
+}
+}  // namespace
+
+extern "C" int32_t rmlk_hip_store_weights(rmlk_stream_t stream, int32_t w_dtype, int64_t n, const void *src,
+                                          void *dst) {
+    if (w_dtype != RMLK_FLOAT16 && w_dtype != RMLK_BFLOAT16) return RMLK_ERR_UNSUPPORTED;
+    if (n < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n == 0) return RMLK_OK;
+    if (n >= kMaxElems) return RMLK_ERR_TOO_LARGE;
+    if (!src || !dst) return RMLK_ERR_NULL_POINTER;
+    const unsigned grid = grid_for(n, kThreads, 8);
+    const float *ps = static_cast<const float *>(src);
+    uint16_t *pd = static_cast<uint16_t *>(dst);
+    if (w_dtype == RMLK_FLOAT16) store_weights_kernel<StoredF16><<<grid, kThreads, 0, as_stream(stream)>>>(ps, pd, n);
+    else store_weights_kernel<StoredBF16><<<grid, kThreads, 0, as_stream(stream)>>>(ps, pd, n);
+    return launch_status();
+}
+
+namespace {
+// rmlk_hip_matmul with the storage type of B as an argument: a B of 16-bit values must be
+// K-contiguous (trans_b) under a row-major A; ldb and stride_b count stored values.
+int32_t matmul_stored(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t m, int64_t n, int64_t k,
+                      const void *a, int64_t lda, int64_t stride_a, int32_t trans_a, int32_t b_dtype,
+                      const void *b, int64_t ldb, int64_t stride_b, int32_t trans_b, void *c, int64_t ldc,
+                      int64_t stride_c, void *workspace, size_t workspace_bytes) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    const bool b16 = b_dtype != RMLK_FLOAT;
+    if (b16 && b_dtype != RMLK_FLOAT16 && b_dtype != RMLK_BFLOAT16) return RMLK_ERR_UNSUPPORTED;
+    if (b16 && (!trans_b || trans_a)) return RMLK_ERR_UNSUPPORTED;
     if (batch < 0 || m < 0 || n < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (batch == 0 || m == 0 || n == 0) return RMLK_OK;
     if (m >= (1ll << 31) || n >= (1ll << 31) || k >= (1ll << 31) || batch >= 65536)
@@ -1693,7 +1954,7 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
     if (stride_a < 0 || stride_b < 0 || stride_c < 0) return RMLK_ERR_INVALID_ARGUMENT;
     hipStream_t s = as_stream(stream);
     const float *pa = static_cast<const float *>(a);
-    const float *pb = static_cast<const float *>(b);
+    const float *pb = static_cast<const float *>(b);   // (a 16-bit B is only handed on, never read here)
     float *pc = static_cast<float *>(c);
 
     if (k == 0) {
@@ -1725,8 +1986,10 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
             int64_t blocks = (n + 3) / 4;
             if (blocks > 8 * kNumCU) blocks = 8 * kNumCU;
             dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch), 1);
-            gemv_dot_kernel<<<grid, kThreads, 0, s>>>(g);
-            return launch_status();
+            return with_storage(b_dtype, [&](auto ws) -> int32_t {
+                gemv_dot_kernel<decltype(ws)><<<grid, kThreads, 0, s>>>(g);
+                return launch_status();
+            });
         }
         const bool vec = n % 4 == 0 && ldb % 4 == 0 && stride_b % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(pb) % 16 == 0;
@@ -1777,10 +2040,13 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
             int64_t blocks = (n + 3) / 4;
             if (blocks > 8 * kNumCU) blocks = 8 * kNumCU;
             dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch), 1);
-            if (m <= 2) skinny_dot_kernel<2><<<grid, kThreads, 0, s>>>(g);
-            else if (m <= 4) skinny_dot_kernel<4><<<grid, kThreads, 0, s>>>(g);
-            else skinny_dot_kernel<8><<<grid, kThreads, 0, s>>>(g);
-            return launch_status();
+            return with_storage(b_dtype, [&](auto ws) -> int32_t {
+                using WS = decltype(ws);
+                if (m <= 2) skinny_dot_kernel<2, WS><<<grid, kThreads, 0, s>>>(g);
+                else if (m <= 4) skinny_dot_kernel<4, WS><<<grid, kThreads, 0, s>>>(g);
+                else skinny_dot_kernel<8, WS><<<grid, kThreads, 0, s>>>(g);
+                return launch_status();
+            });
         }
         const bool vec = n % 4 == 0 && ldb % 4 == 0 && stride_b % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(pb) % 16 == 0;
@@ -1827,8 +2093,18 @@ extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t 
         return launch_status();
     }
 
-    return gemm_tiled(s, batch, m, n, k, pa, lda, stride_a, pb, ldb, stride_b, trans_b, pc, ldc, stride_c,
-                      workspace, workspace_bytes, nullptr);
+    return gemm_tiled(s, batch, m, n, k, pa, lda, stride_a, b_dtype, b, ldb, stride_b, trans_b, pc, ldc,
+                      stride_c, workspace, workspace_bytes, nullptr);
+}
+}  // namespace
+
+extern "C" int32_t rmlk_hip_matmul(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t m,
+                                   int64_t n, int64_t k, const void *a, int64_t lda,
+                                   int64_t stride_a, int32_t trans_a, const void *b, int64_t ldb,
+                                   int64_t stride_b, int32_t trans_b, void *c, int64_t ldc,
+                                   int64_t stride_c, void *workspace, size_t workspace_bytes) {
+    return matmul_stored(stream, dtype, batch, m, n, k, a, lda, stride_a, trans_a, dtype, b, ldb, stride_b,
+                         trans_b, c, ldc, stride_c, workspace, workspace_bytes);
 }
 
 extern "C" size_t rmlk_hip_gemv_partials_workspace_size(int32_t dtype, int64_t n, int64_t k) {
@@ -1884,10 +2160,13 @@ extern "C" size_t rmlk_hip_matmul_grouped_workspace_size(int32_t dtype, int64_t 
 }
 
 extern "C" int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t k,
-                                           const void *a, int64_t lda, const void *b, int64_t ldb,
-                                           int32_t trans_b, int32_t groups, const int64_t *widths,
-                                           void *const *outs, void *workspace, size_t workspace_bytes) {
+                                           const void *a, int64_t lda, int32_t w_dtype, const void *b,
+                                           int64_t ldb, int32_t trans_b, int32_t groups,
+                                           const int64_t *widths, void *const *outs, void *workspace,
+                                           size_t workspace_bytes) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (w_dtype != RMLK_FLOAT && w_dtype != RMLK_FLOAT16 && w_dtype != RMLK_BFLOAT16) return RMLK_ERR_UNSUPPORTED;
+    if (w_dtype != RMLK_FLOAT && !trans_b) return RMLK_ERR_UNSUPPORTED;
     if (!widths || !outs) return RMLK_ERR_NULL_POINTER;
     if (groups <= 0 || groups > kMaxSegments || m < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
     int64_t total = 0;
@@ -1913,17 +2192,18 @@ extern "C" int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, 
         const size_t need = rmlk_hip_matmul_workspace_size(dtype, 1, m, total, k);
         if (need && (!workspace || workspace_bytes < need)) return RMLK_ERR_WORKSPACE;
         const int32_t st = gemm_tiled(as_stream(stream), 1, m, total, k, static_cast<const float *>(a),
-                                      lda, 0, static_cast<const float *>(b), ldb, 0, trans_b, sg.c[0],
-                                      sg.ldc[0], 0, workspace, workspace_bytes, &sg);
+                                      lda, 0, w_dtype, b, ldb, 0, trans_b, sg.c[0], sg.ldc[0], 0, workspace,
+                                      workspace_bytes, &sg);
         if (st != RMLK_ERR_UNSUPPORTED) return st;
     }
     int64_t off = 0;
     for (int i = 0; i < groups; ++i) {
         if (widths[i] > 0) {
             // block i: the next widths[i] columns of a row-major B, the next widths[i] rows of a K-contiguous one
-            const int32_t st = rmlk_hip_matmul(stream, dtype, 1, m, widths[i], k, a, lda, 0, 0,
-                                               static_cast<const float *>(b) + (trans_b ? off * ldb : off), ldb,
-                                               0, trans_b, outs[i], widths[i], 0, workspace, workspace_bytes);
+            const int64_t first = trans_b ? off * ldb : off;   // in stored values
+            const char *bi = static_cast<const char *>(b) + first * (w_dtype == RMLK_FLOAT ? 4 : 2);
+            const int32_t st = matmul_stored(stream, dtype, 1, m, widths[i], k, a, lda, 0, 0, w_dtype, bi, ldb,
+                                             0, trans_b, outs[i], widths[i], 0, workspace, workspace_bytes);
             if (st) return st;
         }
         off += widths[i];
@@ -1932,10 +2212,11 @@ extern "C" int32_t rmlk_hip_matmul_grouped(rmlk_stream_t stream, int32_t dtype, 
 }
 
 extern "C" int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n,
-                                          int64_t k, const void *a, int64_t lda, const void *b,
-                                          int64_t ldb, int32_t trans_b, int64_t gate_offset,
+                                          int64_t k, const void *a, int64_t lda, int32_t w_dtype,
+                                          const void *b, int64_t ldb, int32_t trans_b, int64_t gate_offset,
                                           int64_t up_offset, void *out, int64_t ldc) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (w_dtype != RMLK_FLOAT && w_dtype != RMLK_FLOAT16 && w_dtype != RMLK_BFLOAT16) return RMLK_ERR_UNSUPPORTED;
     if (m < 0 || n < 0 || k < 0 || gate_offset < 0 || up_offset < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (m >= (1ll << 31) || n >= (1ll << 30) || k >= (1ll << 31) || gate_offset >= (1ll << 30) ||
         up_offset >= (1ll << 30))
@@ -1945,9 +2226,8 @@ extern "C" int32_t rmlk_hip_matmul_swiglu(rmlk_stream_t stream, int32_t dtype, i
     if (m == 0 || n == 0) return RMLK_OK;
     if (!a || !b || !out) return RMLK_ERR_NULL_POINTER;
     if (reinterpret_cast<uintptr_t>(out) % 4 != 0) return RMLK_ERR_UNSUPPORTED;
-    return gemm_swiglu(as_stream(stream), m, n, k, static_cast<const float *>(a), lda,
-                       static_cast<const float *>(b), ldb, trans_b, gate_offset, up_offset,
-                       static_cast<float *>(out), ldc);
+    return gemm_swiglu(as_stream(stream), m, n, k, static_cast<const float *>(a), lda, w_dtype, b, ldb,
+                       trans_b, gate_offset, up_offset, static_cast<float *>(out), ldc);
 }
 
 extern "C" size_t rmlk_hip_matmul_partials_workspace_size(int32_t dtype, int64_t m, int64_t n, int64_t k) {
@@ -1956,58 +2236,82 @@ extern "C" size_t rmlk_hip_matmul_partials_workspace_size(int32_t dtype, int64_t
 }
 
 extern "C" int32_t rmlk_hip_matmul_partials(rmlk_stream_t stream, int32_t dtype, int64_t m, int64_t n,
-                                            int64_t k, const void *a, int64_t lda, const void *b,
-                                            int64_t ldb, int32_t trans_b, void *workspace,
+                                            int64_t k, const void *a, int64_t lda, int32_t w_dtype,
+                                            const void *b, int64_t ldb, int32_t trans_b, void *workspace,
                                             size_t workspace_bytes, int32_t *splits_out) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
+    if (w_dtype != RMLK_FLOAT && w_dtype != RMLK_FLOAT16 && w_dtype != RMLK_BFLOAT16) return RMLK_ERR_UNSUPPORTED;
     if (m < 0 || n < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (m >= (1ll << 31) || n >= (1ll << 31) || k >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
     if (m <= kSkinnyRows || n == 0 || k == 0) return RMLK_ERR_UNSUPPORTED;   // not the tiled kernels' case
     if (!a || !b || !workspace || !splits_out) return RMLK_ERR_NULL_POINTER;
     if (lda < k || ldb < (trans_b ? k : n)) return RMLK_ERR_SIZE_MISMATCH;
     if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return RMLK_ERR_UNSUPPORTED;
-    return gemm_tiled(as_stream(stream), 1, m, n, k, static_cast<const float *>(a), lda, 0,
-                      static_cast<const float *>(b), ldb, 0, trans_b, nullptr, n, 0, workspace,
-                      workspace_bytes, nullptr, splits_out);
+    return gemm_tiled(as_stream(stream), 1, m, n, k, static_cast<const float *>(a), lda, 0, w_dtype, b, ldb,
+                      0, trans_b, nullptr, n, 0, workspace, workspace_bytes, nullptr, splits_out);
 }
 
 namespace {
 
 // Shared argument checks and launches of the K-major one-row products. `norm`: x is normalised on
 // the fly (see gemv_kmajor_kernel); `residual`: added to the outputs.
+// What every K-major one-row product checks of its weights: rows of whole 128-bit units that
+// start on 16-byte boundaries.
+template <typename WS>
+bool kmajor_rows_ok(int64_t k, const void *wt, int64_t ldw) {
+    return k % WS::kUnit == 0 && ldw % WS::kUnit == 0 && reinterpret_cast<uintptr_t>(wt) % 16 == 0;
+}
+
+// f(storage tag, units per lane and chunk) for a row of k weights stored as `w_dtype`.
+template <typename F>
+int32_t with_storage_depth(int32_t w_dtype, int64_t k, F &&f) {
+    return with_storage(w_dtype, [&](auto ws) -> int32_t {
+        using WS = decltype(ws);
+        if constexpr (kStored16<WS>) {
+            if (k < 64 * 8 * WS::kUnit) return f(ws, std::integral_constant<int, 4>{});
+        }
+        return f(ws, std::integral_constant<int, kGemvDepth>{});
+    });
+}
+
 int32_t gemv_kmajor_launch(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k, const void *x,
-                           const void *wt, int64_t ldw, const void *residual, const RowNormArgs *norm,
-                           void *y) {
+                           int32_t w_dtype, const void *wt, int64_t ldw, const void *residual,
+                           const RowNormArgs *norm, void *y) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
     if (n < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (n >= (1ll << 31) || k >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
     if (n == 0) return RMLK_OK;
     if (!y || (k > 0 && (!x || !wt)) || (norm && !norm->gamma)) return RMLK_ERR_NULL_POINTER;
     if (ldw < k) return RMLK_ERR_SIZE_MISMATCH;
-    if (k % 4 != 0 || ldw % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
-        reinterpret_cast<uintptr_t>(wt) % 16 != 0)
-        return RMLK_ERR_UNSUPPORTED;
+    if (k % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0) return RMLK_ERR_UNSUPPORTED;
     // the widths the norm kernel gives one block
     if (norm && (k == 0 || k > kThreads * 4 * 8 || reinterpret_cast<uintptr_t>(norm->gamma) % 16 != 0))
         return RMLK_ERR_UNSUPPORTED;
-    const float *px = static_cast<const float *>(x), *pw = static_cast<const float *>(wt);
+    const float *px = static_cast<const float *>(x);
     const float *pr = static_cast<const float *>(residual);
     float *py = static_cast<float *>(y);
     hipStream_t s = as_stream(stream);
     constexpr int kWaves = kThreads / kWave;
     const int32_t ni = static_cast<int32_t>(n), ki = static_cast<int32_t>(k);
     const unsigned grid = static_cast<unsigned>((n + kWaves - 1) / kWaves);
-    if (norm && k <= kThreads * 4 * 2)
-        gemv_kmajor_kernel<false, true, 2><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
-    else if (norm)
-        gemv_kmajor_kernel<false, true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
-    else gemv_kmajor_kernel<><<<grid, kThreads, 0, s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, RowNormArgs{});
-    return launch_status();
+    return with_storage_depth(w_dtype, k, [&](auto ws, auto depth) -> int32_t {
+        using WS = decltype(ws);
+        constexpr int D = decltype(depth)::value;
+        if (!kmajor_rows_ok<WS>(k, wt, ldw)) return RMLK_ERR_UNSUPPORTED;
+        const typename WS::elem *pw = static_cast<const typename WS::elem *>(wt);
+        if (norm && k <= kThreads * 4 * 2)
+            gemv_kmajor_kernel<false, true, 2, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
+        else if (norm)
+            gemv_kmajor_kernel<false, true, kGemvNormUnits, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
+        else
+            gemv_kmajor_kernel<false, false, kGemvNormUnits, WS, D><<<grid, kThreads, 0, s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, RowNormArgs{});
+        return launch_status();
+    });
 }
 
 int32_t gemv_kmajor_swiglu_launch(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k, const void *x,
-                                  const void *wt, int64_t ldw, int64_t gate_row, int64_t up_row,
-                                  const RowNormArgs *norm, void *y) {
+                                  int32_t w_dtype, const void *wt, int64_t ldw, int64_t gate_row,
+                                  int64_t up_row, const RowNormArgs *norm, void *y) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
     if (n < 0 || k < 0 || gate_row < 0 || up_row < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (n >= (1ll << 30) || k >= (1ll << 31) || gate_row >= (1ll << 30) || up_row >= (1ll << 30))
@@ -2015,36 +2319,42 @@ int32_t gemv_kmajor_swiglu_launch(rmlk_stream_t stream, int32_t dtype, int64_t n
     if (n == 0) return RMLK_OK;
     if (!y || (k > 0 && (!x || !wt)) || (norm && !norm->gamma)) return RMLK_ERR_NULL_POINTER;
     if (ldw < k) return RMLK_ERR_SIZE_MISMATCH;
-    if (k % 4 != 0 || ldw % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
-        reinterpret_cast<uintptr_t>(wt) % 16 != 0)
-        return RMLK_ERR_UNSUPPORTED;
+    if (k % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0) return RMLK_ERR_UNSUPPORTED;
     if (norm && (k == 0 || k > kThreads * 4 * 8 || reinterpret_cast<uintptr_t>(norm->gamma) % 16 != 0))
         return RMLK_ERR_UNSUPPORTED;
     constexpr int kOutputsPerBlock = kThreads / kWave / 2;   // a wavefront per gate row and per up row
     const unsigned grid = static_cast<unsigned>((n + kOutputsPerBlock - 1) / kOutputsPerBlock);
-    const float *px = static_cast<const float *>(x), *pw = static_cast<const float *>(wt);
+    const float *px = static_cast<const float *>(x);
     float *py = static_cast<float *>(y);
     const int32_t ni = static_cast<int32_t>(n), ki = static_cast<int32_t>(k);
     const int32_t gr = static_cast<int32_t>(gate_row), ur = static_cast<int32_t>(up_row);
-    if (norm && k <= kThreads * 4 * 2)
-        gemv_kmajor_kernel<true, true, 2><<<grid, kThreads, k * sizeof(float), as_stream(stream)>>>(
-            px, pw, py, ni, ki, ldw, gr, ur, nullptr, *norm);
-    else if (norm)
-        gemv_kmajor_kernel<true, true><<<grid, kThreads, k * sizeof(float), as_stream(stream)>>>(
-            px, pw, py, ni, ki, ldw, gr, ur, nullptr, *norm);
-    else
-        gemv_kmajor_kernel<true><<<grid, kThreads, 0, as_stream(stream)>>>(px, pw, py, ni, ki, ldw, gr, ur,
-                                                                          nullptr, RowNormArgs{});
-    return launch_status();
+    hipStream_t s = as_stream(stream);
+    return with_storage_depth(w_dtype, k, [&](auto ws, auto depth) -> int32_t {
+        using WS = decltype(ws);
+        constexpr int D = decltype(depth)::value;
+        if (!kmajor_rows_ok<WS>(k, wt, ldw)) return RMLK_ERR_UNSUPPORTED;
+        const typename WS::elem *pw = static_cast<const typename WS::elem *>(wt);
+        if (norm && k <= kThreads * 4 * 2)
+            gemv_kmajor_kernel<true, true, 2, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(
+                px, pw, py, ni, ki, ldw, gr, ur, nullptr, *norm);
+        else if (norm)
+            gemv_kmajor_kernel<true, true, kGemvNormUnits, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(
+                px, pw, py, ni, ki, ldw, gr, ur, nullptr, *norm);
+        else
+            gemv_kmajor_kernel<true, false, kGemvNormUnits, WS, D><<<grid, kThreads, 0, s>>>(
+                px, pw, py, ni, ki, ldw, gr, ur, nullptr, RowNormArgs{});
+        return launch_status();
+    });
 }
 
 }  // namespace
 
 extern "C" int32_t rmlk_hip_gemv_kmajor_head_rows(rmlk_stream_t stream, int32_t dtype, int64_t k,
                                                   const void *x, const void *gamma, float eps,
-                                                  int32_t reciprocal_form, const void *wt, int64_t ldw,
-                                                  int32_t n_streams, const rmlk_row_stream *streams,
-                                                  const int64_t *first_col, int32_t *err_flag) {
+                                                  int32_t reciprocal_form, int32_t w_dtype, const void *wt,
+                                                  int64_t ldw, int32_t n_streams,
+                                                  const rmlk_row_stream *streams, const int64_t *first_col,
+                                                  int32_t *err_flag) {
     if (dtype != RMLK_FLOAT) return RMLK_ERR_UNSUPPORTED;
     if (n_streams < 0 || k < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (n_streams == 0) return RMLK_OK;
@@ -2052,9 +2362,7 @@ extern "C" int32_t rmlk_hip_gemv_kmajor_head_rows(rmlk_stream_t stream, int32_t 
     if (!streams || !first_col || (k > 0 && (!x || !wt))) return RMLK_ERR_NULL_POINTER;
     if (k >= (1ll << 31)) return RMLK_ERR_TOO_LARGE;
     if (ldw < k) return RMLK_ERR_SIZE_MISMATCH;
-    if (k == 0 || k % 4 != 0 || ldw % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
-        reinterpret_cast<uintptr_t>(wt) % 16 != 0)
-        return RMLK_ERR_UNSUPPORTED;
+    if (k == 0 || k % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0) return RMLK_ERR_UNSUPPORTED;
     if (gamma && (k > kThreads * 4 * kGemvNormUnits || reinterpret_cast<uintptr_t>(gamma) % 16 != 0))
         return RMLK_ERR_UNSUPPORTED;
     GemvRowStreams rs{};
@@ -2112,56 +2420,62 @@ extern "C" int32_t rmlk_hip_gemv_kmajor_head_rows(rmlk_stream_t stream, int32_t 
     rs.total_pairs = static_cast<int32_t>(pairs);
     constexpr int kPairsPerBlock = kThreads / kWave / 2;
     const unsigned grid = static_cast<unsigned>((pairs + kPairsPerBlock - 1) / kPairsPerBlock);
-    const float *px = static_cast<const float *>(x), *pw = static_cast<const float *>(wt);
+    const float *px = static_cast<const float *>(x);
     const int32_t ki = static_cast<int32_t>(k);
     hipStream_t s = as_stream(stream);
-    if (gamma) {
-        const RowNormArgs norm{static_cast<const float *>(gamma), eps, reciprocal_form};
-        if (k <= kThreads * 4 * 2)
-            gemv_kmajor_rows_kernel<true, 2><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
-        else
-            gemv_kmajor_rows_kernel<true><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
-    } else {
-        gemv_kmajor_rows_kernel<false><<<grid, kThreads, 0, s>>>(px, pw, ki, ldw, RowNormArgs{}, rs);
-    }
-    return launch_status();
+    return with_storage_depth(w_dtype, k, [&](auto ws, auto depth) -> int32_t {
+        using WS = decltype(ws);
+        constexpr int D = decltype(depth)::value;
+        if (!kmajor_rows_ok<WS>(k, wt, ldw)) return RMLK_ERR_UNSUPPORTED;
+        const typename WS::elem *pw = static_cast<const typename WS::elem *>(wt);
+        if (gamma) {
+            const RowNormArgs norm{static_cast<const float *>(gamma), eps, reciprocal_form};
+            if (k <= kThreads * 4 * 2)
+                gemv_kmajor_rows_kernel<true, 2, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
+            else
+                gemv_kmajor_rows_kernel<true, kGemvNormUnits, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
+        } else {
+            gemv_kmajor_rows_kernel<false, kGemvNormUnits, WS, D><<<grid, kThreads, 0, s>>>(px, pw, ki, ldw, RowNormArgs{}, rs);
+        }
+        return launch_status();
+    });
 }
 
 extern "C" int32_t rmlk_hip_gemv_kmajor(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
-                                   const void *x, const void *wt, int64_t ldw, void *y) {
-    return gemv_kmajor_launch(stream, dtype, n, k, x, wt, ldw, nullptr, nullptr, y);
+                                   const void *x, int32_t w_dtype, const void *wt, int64_t ldw, void *y) {
+    return gemv_kmajor_launch(stream, dtype, n, k, x, w_dtype, wt, ldw, nullptr, nullptr, y);
 }
 
 extern "C" int32_t rmlk_hip_gemv_kmajor_add(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
-                                            const void *x, const void *wt, int64_t ldw,
+                                            const void *x, int32_t w_dtype, const void *wt, int64_t ldw,
                                             const void *residual, void *y) {
     if (n > 0 && !residual) return RMLK_ERR_NULL_POINTER;
-    return gemv_kmajor_launch(stream, dtype, n, k, x, wt, ldw, residual, nullptr, y);
+    return gemv_kmajor_launch(stream, dtype, n, k, x, w_dtype, wt, ldw, residual, nullptr, y);
 }
 
 extern "C" int32_t rmlk_hip_gemv_kmajor_normed(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
                                                const void *x, const void *gamma, float eps,
-                                               int32_t reciprocal_form, const void *wt, int64_t ldw,
-                                               void *y) {
+                                               int32_t reciprocal_form, int32_t w_dtype, const void *wt,
+                                               int64_t ldw, void *y) {
     const RowNormArgs norm{static_cast<const float *>(gamma), eps, reciprocal_form};
     if (n > 0 && !gamma) return RMLK_ERR_NULL_POINTER;
-    return gemv_kmajor_launch(stream, dtype, n, k, x, wt, ldw, nullptr, &norm, y);
+    return gemv_kmajor_launch(stream, dtype, n, k, x, w_dtype, wt, ldw, nullptr, &norm, y);
 }
 
 extern "C" int32_t rmlk_hip_gemv_kmajor_swiglu(rmlk_stream_t stream, int32_t dtype, int64_t n, int64_t k,
-                                          const void *x, const void *wt, int64_t ldw, int64_t gate_row,
-                                          int64_t up_row, void *y) {
-    return gemv_kmajor_swiglu_launch(stream, dtype, n, k, x, wt, ldw, gate_row, up_row, nullptr, y);
+                                          const void *x, int32_t w_dtype, const void *wt, int64_t ldw,
+                                          int64_t gate_row, int64_t up_row, void *y) {
+    return gemv_kmajor_swiglu_launch(stream, dtype, n, k, x, w_dtype, wt, ldw, gate_row, up_row, nullptr, y);
 }
 
 extern "C" int32_t rmlk_hip_gemv_kmajor_swiglu_normed(rmlk_stream_t stream, int32_t dtype, int64_t n,
                                                       int64_t k, const void *x, const void *gamma,
-                                                      float eps, int32_t reciprocal_form, const void *wt,
-                                                      int64_t ldw, int64_t gate_row, int64_t up_row,
-                                                      void *y) {
+                                                      float eps, int32_t reciprocal_form, int32_t w_dtype,
+                                                      const void *wt, int64_t ldw, int64_t gate_row,
+                                                      int64_t up_row, void *y) {
     const RowNormArgs norm{static_cast<const float *>(gamma), eps, reciprocal_form};
     if (n > 0 && !gamma) return RMLK_ERR_NULL_POINTER;
-    return gemv_kmajor_swiglu_launch(stream, dtype, n, k, x, wt, ldw, gate_row, up_row, &norm, y);
+    return gemv_kmajor_swiglu_launch(stream, dtype, n, k, x, w_dtype, wt, ldw, gate_row, up_row, &norm, y);
 }
 
 // ---- MatMul for callers that cannot allocate ----------------------------------------------------

@@ -255,6 +255,10 @@ int32_t rmlk_session_create_ex(const rmlk_graph *g, int32_t device, uint32_t fla
         if (!g || !out) throw RtError(RMLK_ERR_NULL_POINTER, "null argument");
         auto s = std::make_unique<rmlk_session>();
         s->impl.fuse = (flags & RMLK_SESSION_NO_FUSION) == 0;
+        if ((flags & RMLK_SESSION_WEIGHTS_F16) && (flags & RMLK_SESSION_WEIGHTS_BF16))
+            throw RtError(RMLK_ERR_INVALID_ARGUMENT, "one storage type for the weights at most");
+        if (flags & RMLK_SESSION_WEIGHTS_F16) s->impl.weight_storage = RMLK_FLOAT16;
+        if (flags & RMLK_SESSION_WEIGHTS_BF16) s->impl.weight_storage = RMLK_BFLOAT16;
         s->impl.build(*g, device);
         *out = s.release();
     });

@@ -285,6 +285,7 @@ struct Session {
     bool capturing = false;
     bool profiling = false;
     bool fuse = true;                // form fused nodes while building
+    int32_t weight_storage = RMLK_FLOAT;   // how the K-contiguous copies of constant weights are held
     int fused_nodes = 0;
     int folded_nodes = 0;            // constant nodes evaluated while building
     int64_t device_syncs = 0;            // blocking reads of shape-like tensors

@@ -756,6 +756,36 @@ struct Matcher {
     void release_unused(int w) {
         if (w >= 0 && users[w].empty() && !g.values[w].is_output && !g.values[w].is_input) s.values[w].reset();
     }
+    // A float matrix [rows, k] in its own allocation.
+    Tensor weight_matrix(int64_t rows, int64_t k, const char *what) {
+        Tensor tt;
+        tt.dtype = RMLK_FLOAT;
+        tt.shape = {rows, k};
+        auto buf = std::make_shared<Buffer>();
+        buf->bytes = tt.nbytes();
+        buf->owned_raw = true;
+        check_hip(hipMalloc(&buf->ptr, buf->bytes), what);
+        tt.buf = buf;
+        return tt;
+    }
+    // The K-contiguous float matrix `tt` as the session holds it: itself, or (a session built with
+    // 16-bit weight storage, rows of whole 128-bit units) rounded once to that type, the float form
+    // released.
+    Tensor as_stored(const Tensor &tt) {
+        check_hip(hipStreamSynchronize(s.stream), "hipStreamSynchronize");
+        if (s.weight_storage == RMLK_FLOAT || tt.shape[1] % 8 != 0) return tt;
+        Tensor st;
+        st.dtype = s.weight_storage;
+        st.shape = tt.shape;
+        auto buf = std::make_shared<Buffer>();
+        buf->bytes = st.nbytes();
+        buf->owned_raw = true;
+        check_hip(hipMalloc(&buf->ptr, buf->bytes), "hipMalloc (16-bit weights)");
+        st.buf = buf;
+        check_status(rmlk_hip_store_weights(s.stream, st.dtype, tt.numel(), tt.data(), st.data()), "16-bit weights");
+        check_hip(hipStreamSynchronize(s.stream), "hipStreamSynchronize");
+        return st;
+    }
     int transposed_copy(int w) {
         auto it = transposed_of.find(w);
         if (it != transposed_of.end()) return it->second;
@@ -764,23 +794,16 @@ struct Matcher {
         if (!t.defined() || t.dtype != RMLK_FLOAT || t.rank() != 2 || t.shape[0] == 0 || t.shape[1] == 0 ||
             t.shape[0] % 4 != 0)
             return -1;
-        Tensor tt;
-        tt.dtype = RMLK_FLOAT;
-        tt.shape = {t.shape[1], t.shape[0]};
-        auto buf = std::make_shared<Buffer>();
-        buf->bytes = tt.nbytes();
-        buf->owned_raw = true;
-        check_hip(hipMalloc(&buf->ptr, buf->bytes), "hipMalloc (K-contiguous weights)");
-        tt.buf = buf;
+        Tensor tt = weight_matrix(t.shape[1], t.shape[0], "hipMalloc (K-contiguous weights)");
         rmlk_dims in_shape = to_dims(t.shape);
         const int64_t perm[2] = {1, 0};
         check_status(rmlk_hip_transpose(s.stream, RMLK_FLOAT, &in_shape, perm, t.data(), tt.data()),
                      "K-contiguous weights");
-        check_hip(hipStreamSynchronize(s.stream), "hipStreamSynchronize");
+        tt = as_stored(tt);
         const int id = static_cast<int>(g.values.size());
         Value v;
         v.name = "rmlk.k_contiguous." + std::to_string(w);
-        v.dtype = RMLK_FLOAT;
+        v.dtype = tt.dtype;
         v.shape = tt.shape;
         v.is_initializer = true;
         g.values.push_back(v);
@@ -857,14 +880,7 @@ struct Matcher {
             int64_t total = 0;
             for (int64_t w : widths) total += w;
             // the joint weight matrix
-            Tensor joint;
-            joint.dtype = RMLK_FLOAT;
-            joint.shape = {total, k0};
-            auto buf = std::make_shared<Buffer>();
-            buf->bytes = joint.nbytes();
-            buf->owned_raw = true;
-            check_hip(hipMalloc(&buf->ptr, buf->bytes), "hipMalloc (joint weights)");
-            joint.buf = buf;
+            Tensor joint = weight_matrix(total, k0, "hipMalloc (joint weights)");
             int64_t off = 0;
             for (size_t i = 0; i < members.size(); ++i) {
                 // member i transposed into its block of rows
@@ -876,11 +892,11 @@ struct Matcher {
                              "joint weights");
                 off += widths[i];
             }
-            check_hip(hipStreamSynchronize(s.stream), "hipStreamSynchronize");
+            joint = as_stored(joint);
             const int joint_id = static_cast<int>(g.values.size());
             Value jv;
             jv.name = "rmlk.joint_weights." + std::to_string(first);
-            jv.dtype = RMLK_FLOAT;
+            jv.dtype = joint.dtype;
             jv.shape = joint.shape;
             jv.is_initializer = true;
             g.values.push_back(jv);
@@ -1197,7 +1213,7 @@ void store_product(OpContext &c, PendingProduct &pp) {
         const size_t ws_bytes = rmlk_hip_matmul_grouped_workspace_size(
             RMLK_FLOAT, pp.m, pp.k, static_cast<int32_t>(pp.widths.size()), pp.widths.data());
         void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
-        check_status(rmlk_hip_matmul_grouped(c.stream, RMLK_FLOAT, pp.m, pp.k, pp.x.data(), pp.k, pp.wt.data(),
+        check_status(rmlk_hip_matmul_grouped(c.stream, RMLK_FLOAT, pp.m, pp.k, pp.x.data(), pp.k, pp.wt.dtype, pp.wt.data(),
                                              pp.k, 1, static_cast<int32_t>(pp.widths.size()), pp.widths.data(),
                                              outs.data(), ws, ws_bytes),
                      "rmlk.MatMulGroup (deferred)");
@@ -1207,9 +1223,9 @@ void store_product(OpContext &c, PendingProduct &pp) {
     int32_t st;
     if (pp.norm)
         st = rmlk_hip_gemv_kmajor_normed(c.stream, RMLK_FLOAT, pp.total, pp.k, pp.x.data(), pp.norm->gamma.data(),
-                                         pp.norm->eps, pp.norm->reciprocal, pp.wt.data(), pp.k, pp.row.data());
+                                         pp.norm->eps, pp.norm->reciprocal, pp.wt.dtype, pp.wt.data(), pp.k, pp.row.data());
     else
-        st = rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, pp.total, pp.k, pp.x.data(), pp.wt.data(), pp.k,
+        st = rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, pp.total, pp.k, pp.x.data(), pp.wt.dtype, pp.wt.data(), pp.k,
                                   pp.row.data());
     if (st == RMLK_ERR_UNSUPPORTED && pp.norm) {
         // (a row the one-row kernels refuse to normalise: norm, then product)
@@ -1221,7 +1237,7 @@ void store_product(OpContext &c, PendingProduct &pp) {
         check_status(rmlk_hip_rmsnorm(c.stream, RMLK_FLOAT, 1, pp.k, pp.x.data(), pp.norm->gamma.data(),
                                       pp.norm->eps, pp.norm->reciprocal, normed.data()),
                      "rmlk.RMSNorm (deferred)");
-        st = rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, pp.total, pp.k, normed.data(), pp.wt.data(), pp.k,
+        st = rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, pp.total, pp.k, normed.data(), pp.wt.dtype, pp.wt.data(), pp.k,
                                   pp.row.data());
     }
     check_status(st, "rmlk.MatMulGroup (deferred)");
@@ -1403,7 +1419,7 @@ void op_fused_head_rows(OpContext &c) {
         const PendingProduct &pp = *product;
         const int32_t st = rmlk_hip_gemv_kmajor_head_rows(
             c.stream, RMLK_FLOAT, pp.k, pp.x.data(), pp.norm ? pp.norm->gamma.data() : nullptr,
-            pp.norm ? pp.norm->eps : 0.f, pp.norm ? pp.norm->reciprocal : 0, pp.wt.data(), pp.k,
+            pp.norm ? pp.norm->eps : 0.f, pp.norm ? pp.norm->reciprocal : 0, pp.wt.dtype, pp.wt.data(), pp.k,
             static_cast<int32_t>(n), streams.data(), first_col.data(), c.error_flag());
         if (took_fast_path(st, "rmlk.HeadRows (with its projection)")) {
             product->computed = true;   // consumed: nothing else reads its members
@@ -1560,7 +1576,7 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
             // the product with the residual added is the row; the norm is left to the product
             // that reads it
             Tensor &sum = c.alloc_output(0, RMLK_FLOAT, res.shape);
-            if (took_fast_path(rmlk_hip_gemv_kmajor_add(c.stream, RMLK_FLOAT, n, k, a.data(), wt.data(), k,
+            if (took_fast_path(rmlk_hip_gemv_kmajor_add(c.stream, RMLK_FLOAT, n, k, a.data(), wt.dtype, wt.data(), k,
                                                         res.data(), sum.data()),
                                "rmlk.MatMulAddRMSNorm")) {
                 defer_norm(c, 1, sum, gamma);
@@ -1568,7 +1584,7 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
             }
         }
         float *prod = static_cast<float *>(c.scratch(static_cast<size_t>(n) * sizeof(float)));
-        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, n, k, a.data(), wt.data(), k, prod),
+        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, n, k, a.data(), wt.dtype, wt.data(), k, prod),
                            "rmlk.MatMulAddRMSNorm")) {
             Tensor &sum = c.alloc_output(0, RMLK_FLOAT, res.shape);
             Tensor &y = c.alloc_output(1, RMLK_FLOAT, res.shape);
@@ -1586,8 +1602,8 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
         if (bytes) {
             void *ws = c.scratch(bytes);
             int32_t splits = 0;
-            if (took_fast_path(rmlk_hip_matmul_partials(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, wt.data(),
-                                                        k, 1, ws, bytes, &splits),
+            if (took_fast_path(rmlk_hip_matmul_partials(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, wt.dtype,
+                                                        wt.data(), k, 1, ws, bytes, &splits),
                                "rmlk.MatMulAddRMSNorm")) {
                 Tensor &sum = c.alloc_output(0, RMLK_FLOAT, res.shape);
                 Tensor &y = c.alloc_output(1, RMLK_FLOAT, res.shape);
@@ -1605,11 +1621,21 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
 
 // a [.., k] . wt^T for any number of rows: the general product with a K-contiguous second operand
 // (`wt`: n rows of k), into the dense [m, n] at `out`.
-void product_over_kmajor(OpContext &c, const void *a, int64_t m, int64_t k, const void *wt, int64_t n, void *out,
-                         const char *what) {
+// `w_dtype`: how the weights are stored (float, or the 16-bit type the session was built with).
+void product_over_kmajor(OpContext &c, const void *a, int64_t m, int64_t k, int32_t w_dtype, const void *wt,
+                         int64_t n, void *out, const char *what) {
     const size_t ws_bytes = rmlk_hip_matmul_workspace_size(RMLK_FLOAT, 1, m, n, k);
     void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
-    check_status(rmlk_hip_matmul(c.stream, RMLK_FLOAT, 1, m, n, k, a, k, 0, 0, wt, k, 0, 1, out, n, 0, ws, ws_bytes),
+    if (w_dtype == RMLK_FLOAT) {
+        check_status(rmlk_hip_matmul(c.stream, RMLK_FLOAT, 1, m, n, k, a, k, 0, 0, wt, k, 0, 1, out, n, 0, ws,
+                                     ws_bytes),
+                     what);
+        return;
+    }
+    // (the grouped product with one member is the general product over stored weights)
+    void *outs[1] = {out};
+    check_status(rmlk_hip_matmul_grouped(c.stream, RMLK_FLOAT, m, k, a, k, w_dtype, wt, k, 1, 1, &n, outs, ws,
+                                         ws_bytes),
                  what);
 }
 
@@ -1639,17 +1665,17 @@ void op_fused_matmul_const(OpContext &c) {
         if (a.pending_norm && n < kMaxDeferredNormWidth) {
             const PendingNorm &pn = *a.pending_norm;
             if (took_fast_path(rmlk_hip_gemv_kmajor_normed(c.stream, RMLK_FLOAT, n, k, a.data(), pn.gamma.data(),
-                                                           pn.eps, pn.reciprocal, wt.data(), k, y.data()),
+                                                           pn.eps, pn.reciprocal, wt.dtype, wt.data(), k, y.data()),
                                "rmlk.MatMulConst"))
                 return;
         }
         if (c.input(0).pending_norm) compute_pending_norm(c);
-        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, n, k, c.input(0).data(), wt.data(), k, y.data()),
+        if (took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, n, k, c.input(0).data(), wt.dtype, wt.data(), k, y.data()),
                            "rmlk.MatMulConst"))
             return;
     }
     if (c.input(0).pending_norm) compute_pending_norm(c);
-    product_over_kmajor(c, c.input(0).data(), m, k, wt.data(), n, y.data(), "rmlk.MatMulConst");
+    product_over_kmajor(c, c.input(0).data(), m, k, wt.dtype, wt.data(), n, y.data(), "rmlk.MatMulConst");
 }
 
 // swiglu(a . Wg, a . Wu) with [Wg | Wu] constant and stored K-contiguous as one matrix (wt [2 n, k]).
@@ -1669,7 +1695,7 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
             Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
             if (took_fast_path(rmlk_hip_gemv_kmajor_swiglu_normed(
                                    c.stream, RMLK_FLOAT, n, k, row.data(), pn.gamma.data(), pn.eps, pn.reciprocal,
-                                   wt.data(), k, gate_first ? 0 : n, gate_first ? n : 0, y.data()),
+                                   wt.dtype, wt.data(), k, gate_first ? 0 : n, gate_first ? n : 0, y.data()),
                                "rmlk.MatMulGroupSwiGLU"))
                 return;
         }
@@ -1685,7 +1711,7 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
         std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
         shape.push_back(n);
         Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
-        if (took_fast_path(rmlk_hip_matmul_swiglu(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, wt.data(), k, 1,
+        if (took_fast_path(rmlk_hip_matmul_swiglu(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, wt.dtype, wt.data(), k, 1,
                                                   gate_first ? 0 : n, gate_first ? n : 0, y.data(), n),
                            "rmlk.MatMulGroupSwiGLU"))
             return;
@@ -1697,7 +1723,7 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
         std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
         shape.push_back(n);
         Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
-        if (took_fast_path(rmlk_hip_gemv_kmajor_swiglu(c.stream, RMLK_FLOAT, n, k, a.data(), wt.data(), k,
+        if (took_fast_path(rmlk_hip_gemv_kmajor_swiglu(c.stream, RMLK_FLOAT, n, k, a.data(), wt.dtype, wt.data(), k,
                                                        gate_first ? 0 : n, gate_first ? n : 0, y.data()),
                            "rmlk.MatMulGroupSwiGLU"))
             return;
@@ -1724,7 +1750,8 @@ void op_fused_matmul_group(OpContext &c) {
         sh.push_back(n);
         return sh;
     };
-    const float *rows = static_cast<const float *>(wt.data());
+    const char *rows = static_cast<const char *>(wt.data());
+    const int64_t row_bytes = k * static_cast<int64_t>(dtype_size(wt.dtype));
     if (m == 1) {
         // one launch over the joint matrix; the members' results are slices of its output row
         Tensor row;
@@ -1764,15 +1791,16 @@ void op_fused_matmul_group(OpContext &c) {
         if (pending) {
             done = took_fast_path(rmlk_hip_gemv_kmajor_normed(c.stream, RMLK_FLOAT, total, k, a.data(),
                                                               pending->gamma.data(), pending->eps,
-                                                              pending->reciprocal, wt.data(), k, row.data()),
+                                                              pending->reciprocal, wt.dtype, wt.data(), k,
+                                                              row.data()),
                                   "rmlk.MatMulGroup");
             if (!done) compute_pending_norm(c);   // what follows reads input 0 through the context
         }
         const Tensor &a1 = c.input(0);
-        if (!done && !took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, total, k, a1.data(), wt.data(), k,
+        if (!done && !took_fast_path(rmlk_hip_gemv_kmajor(c.stream, RMLK_FLOAT, total, k, a1.data(), wt.dtype, wt.data(), k,
                                                           row.data()),
                                      "rmlk.MatMulGroup"))
-            product_over_kmajor(c, a1.data(), 1, k, wt.data(), total, row.data(), "rmlk.MatMulGroup");
+            product_over_kmajor(c, a1.data(), 1, k, wt.dtype, wt.data(), total, row.data(), "rmlk.MatMulGroup");
         hand_out(nullptr);
         return;
     }
@@ -1790,7 +1818,7 @@ void op_fused_matmul_group(OpContext &c) {
                 c.out = keep;
             }
             int32_t splits = 0;
-            if (took_fast_path(rmlk_hip_matmul_partials(c.stream, RMLK_FLOAT, m, total, k, a.data(), k, wt.data(), k,
+            if (took_fast_path(rmlk_hip_matmul_partials(c.stream, RMLK_FLOAT, m, total, k, a.data(), k, wt.dtype, wt.data(), k,
                                                         1, pp->slabs.data(), bytes, &splits),
                                "rmlk.MatMulGroup")) {
                 pp->x = a;
@@ -1820,7 +1848,7 @@ void op_fused_matmul_group(OpContext &c) {
         const size_t ws_bytes = rmlk_hip_matmul_grouped_workspace_size(
             RMLK_FLOAT, m, k, static_cast<int32_t>(widths.size()), widths.data());
         void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
-        check_status(rmlk_hip_matmul_grouped(c.stream, RMLK_FLOAT, m, k, a.data(), k, wt.data(), k, 1,
+        check_status(rmlk_hip_matmul_grouped(c.stream, RMLK_FLOAT, m, k, a.data(), k, wt.dtype, wt.data(), k, 1,
                                              static_cast<int32_t>(widths.size()), widths.data(),
                                              outs.data(), ws, ws_bytes),
                      "rmlk.MatMulGroup");
@@ -1830,7 +1858,7 @@ void op_fused_matmul_group(OpContext &c) {
     for (size_t i = 0; i < widths.size(); ++i) {
         Tensor &y = c.alloc_output(static_cast<int>(i), RMLK_FLOAT, out_shape(widths[i]));
         if (y.numel() > 0)
-            product_over_kmajor(c, a.data(), m, k, rows + off * k, widths[i], y.data(), "rmlk.MatMulGroup");
+            product_over_kmajor(c, a.data(), m, k, wt.dtype, rows + off * row_bytes, widths[i], y.data(), "rmlk.MatMulGroup");
         off += widths[i];
     }
 }

@@ -32,7 +32,7 @@ const char *dtype_name(int32_t dt) {
 size_t dtype_size(int32_t dt) {
     switch (dt) {
         case RMLK_BOOL: case RMLK_UINT8: case RMLK_INT8: return 1;
-        case RMLK_UINT16: case RMLK_INT16: case RMLK_FLOAT16: return 2;
+        case RMLK_UINT16: case RMLK_INT16: case RMLK_FLOAT16: case RMLK_BFLOAT16: return 2;
         case RMLK_FLOAT: case RMLK_INT32: case RMLK_UINT32: return 4;
         case RMLK_DOUBLE: case RMLK_INT64: case RMLK_UINT64: return 8;
         default: return 0;

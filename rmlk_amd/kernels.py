@@ -17,6 +17,7 @@ from ._lib import Dims, RmlkError, check, lib
 # ONNX TensorProto.DataType numbers (include/rmlk_hip.h rmlk_dtype)
 FLOAT, UINT8, INT8, UINT16, INT16, INT32, INT64, BOOL, FLOAT16, DOUBLE, UINT32, UINT64 = (
     1, 2, 3, 4, 5, 6, 7, 9, 10, 11, 12, 13)
+BFLOAT16 = 16   # only as the storage type of constant weights
 
 TORCH_TO_DTYPE = {
     torch.float32: FLOAT, torch.uint8: UINT8, torch.int8: INT8, torch.int16: INT16,
@@ -43,6 +44,19 @@ def _ptr(t) -> int:
 
 def dtype_of(t: torch.Tensor) -> int:
     return TORCH_TO_DTYPE[t.dtype]
+
+
+def storage_of(w: torch.Tensor) -> int:
+    """Storage type of a weight matrix handed to the products over constant weights."""
+    return BFLOAT16 if w.dtype == torch.bfloat16 else TORCH_TO_DTYPE[w.dtype]
+
+
+def store_weights(w: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """The float tensor w rounded (to nearest even) to torch.float16 or torch.bfloat16 on the device."""
+    out = torch.empty(w.shape, dtype=dtype, device=w.device)
+    wd = BFLOAT16 if dtype == torch.bfloat16 else TORCH_TO_DTYPE[dtype]
+    check(lib().rmlk_hip_store_weights(_stream(), wd, w.numel(), _ptr(w), _ptr(out)), "rmlk_hip_store_weights")
+    return out
 
 
 def binary(op: int, a, b, out, out_shape, a_stride, b_stride) -> None:
@@ -288,26 +302,26 @@ def attention_few_rows_one_launch(q, k, v, mask, out, counters, batch: int, kv_h
 
 def gemv_kmajor(x, wt, y, n: int, k: int) -> None:
     """y[n] = sum_k x[k] * wt[n][k]: one-row product with K-contiguous weights, no combine launch."""
-    check(lib().rmlk_hip_gemv_kmajor(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(wt), k, _ptr(y)),
+    check(lib().rmlk_hip_gemv_kmajor(_stream(), dtype_of(x), n, k, _ptr(x), storage_of(wt), _ptr(wt), k, _ptr(y)),
           "rmlk_hip_gemv_kmajor")
 
 
 def gemv_kmajor_swiglu(x, wt, y, n: int, k: int, gate_row: int, up_row: int) -> None:
     """y[i] = swiglu(x . wt[gate_row + i], x . wt[up_row + i]) in one launch (K-contiguous weights)."""
-    check(lib().rmlk_hip_gemv_kmajor_swiglu(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(wt), k, gate_row,
-                                       up_row, _ptr(y)), "rmlk_hip_gemv_kmajor_swiglu")
+    check(lib().rmlk_hip_gemv_kmajor_swiglu(_stream(), dtype_of(x), n, k, _ptr(x), storage_of(wt), _ptr(wt), k,
+                                            gate_row, up_row, _ptr(y)), "rmlk_hip_gemv_kmajor_swiglu")
 
 
 def gemv_kmajor_add(x, wt, residual, y, n: int, k: int) -> None:
     """y = x . wt^T + residual (K-contiguous weights, one launch)."""
-    check(lib().rmlk_hip_gemv_kmajor_add(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(wt), k, _ptr(residual),
-                                         _ptr(y)), "rmlk_hip_gemv_kmajor_add")
+    check(lib().rmlk_hip_gemv_kmajor_add(_stream(), dtype_of(x), n, k, _ptr(x), storage_of(wt), _ptr(wt), k,
+                                         _ptr(residual), _ptr(y)), "rmlk_hip_gemv_kmajor_add")
 
 
 def gemv_kmajor_normed(x, gamma, wt, y, n: int, k: int, eps: float, reciprocal_form: bool = False) -> None:
     """y = (RMSNorm(x) * gamma) . wt^T, the normalised row never stored."""
     check(lib().rmlk_hip_gemv_kmajor_normed(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(gamma), eps,
-                                            int(reciprocal_form), _ptr(wt), k, _ptr(y)),
+                                            int(reciprocal_form), storage_of(wt), _ptr(wt), k, _ptr(y)),
           "rmlk_hip_gemv_kmajor_normed")
 
 
@@ -315,8 +329,8 @@ def gemv_kmajor_swiglu_normed(x, gamma, wt, y, n: int, k: int, gate_row: int, up
                               reciprocal_form: bool = False) -> None:
     """gemv_kmajor_swiglu over RMSNorm(x) * gamma."""
     check(lib().rmlk_hip_gemv_kmajor_swiglu_normed(_stream(), dtype_of(x), n, k, _ptr(x), _ptr(gamma), eps,
-                                                   int(reciprocal_form), _ptr(wt), k, gate_row, up_row,
-                                                   _ptr(y)), "rmlk_hip_gemv_kmajor_swiglu_normed")
+                                                   int(reciprocal_form), storage_of(wt), _ptr(wt), k, gate_row,
+                                                   up_row, _ptr(y)), "rmlk_hip_gemv_kmajor_swiglu_normed")
 
 
 def matmul_grouped(a, b, outs, m: int, k: int, widths, workspace=None, trans_b: bool = False) -> None:
@@ -329,7 +343,7 @@ def matmul_grouped(a, b, outs, m: int, k: int, widths, workspace=None, trans_b: 
         workspace = torch.empty(need, dtype=torch.uint8, device=a.device)
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
     ptrs = (ctypes.c_void_p * n)(*[_ptr(o) for o in outs])
-    check(lib().rmlk_hip_matmul_grouped(_stream(), dtype_of(a), m, k, _ptr(a), k, _ptr(b),
+    check(lib().rmlk_hip_matmul_grouped(_stream(), dtype_of(a), m, k, _ptr(a), k, storage_of(b), _ptr(b),
                                         k if trans_b else int(sum(widths)), int(trans_b), n, w, ptrs,
                                         _ptr(workspace), ws_bytes),
           "rmlk_hip_matmul_grouped")
@@ -340,7 +354,7 @@ def matmul_swiglu(a, b, out, m: int, n: int, k: int, ldb: int, gate_offset: int,
     """out[m, n] = swiglu(a . b[:, gate_offset:+n], a . b[:, up_offset:+n]) (trans_b: b is [., k] and the
     offsets count its rows); RmlkError with status RMLK_ERR_UNSUPPORTED (-2) for shapes the one-launch
     kernel does not cover."""
-    check(lib().rmlk_hip_matmul_swiglu(_stream(), dtype_of(a), m, n, k, _ptr(a), k, _ptr(b), ldb,
+    check(lib().rmlk_hip_matmul_swiglu(_stream(), dtype_of(a), m, n, k, _ptr(a), k, storage_of(b), _ptr(b), ldb,
                                        int(trans_b), gate_offset, up_offset, _ptr(out), n),
           "rmlk_hip_matmul_swiglu")
 
@@ -392,7 +406,8 @@ def gemv_kmajor_head_rows(x, wt, k: int, streams, first_cols, gamma=None, eps: f
     arr = _row_streams(streams, with_x=False)
     cols = (ctypes.c_int64 * len(streams))(*[int(c) for c in first_cols])
     check(lib().rmlk_hip_gemv_kmajor_head_rows(_stream(), dtype_of(x), k, _ptr(x), _ptr(gamma), eps,
-                                               int(reciprocal_form), _ptr(wt), k, len(streams), arr, cols,
+                                               int(reciprocal_form), storage_of(wt), _ptr(wt), k, len(streams),
+                                               arr, cols,
                                                _ptr(err_flag) if err_flag is not None else None),
           "rmlk_hip_gemv_kmajor_head_rows")
 

@@ -179,10 +179,11 @@ class GraphBuilder:
 class ModelInstance:
     """ref: runtime/src/core/instance.rs:20-119"""
 
-    def __init__(self, graph: Graph, device: int = 0, fuse: bool = True):
+    def __init__(self, graph: Graph, device: int = 0, fuse: bool = True, weights: str = "f32"):
         self.graph = graph
         h = ctypes.c_void_p()
-        _check(lib().rmlk_session_create_ex(graph.handle, device, 0 if fuse else 1, ctypes.byref(h)),
+        flags = (0 if fuse else 1) | {"f32": 0, "f16": 2, "bf16": 4}[weights]
+        _check(lib().rmlk_session_create_ex(graph.handle, device, flags, ctypes.byref(h)),
                "Builder.build")
         self._h = h
 
@@ -309,6 +310,8 @@ class Builder:
         from .onnx_io import load_onnx_bytes
         return Builder(load_onnx_bytes(data, base_dir))
 
-    def build(self, device: int = 0, fuse: bool = True) -> ModelInstance:
-        """fuse=False keeps one kernel per node, as the reference executes a graph."""
-        return ModelInstance(self._graph, device, fuse)
+    def build(self, device: int = 0, fuse: bool = True, weights: str = "f32") -> ModelInstance:
+        """fuse=False keeps one kernel per node, as the reference executes a graph. weights="f16" or
+        "bf16": the constant weights of fused MatMuls are stored rounded to that type (half the bytes
+        to stream per token); the arithmetic stays fp32."""
+        return ModelInstance(self._graph, device, fuse, weights)

@@ -1457,7 +1457,7 @@ def test_matmul_partials_feed_the_norm(device, m, n, k):
     assert need >= m * n * 4
     ws = torch.empty(need, dtype=torch.uint8, device=device)
     splits = ctypes.c_int32(0)
-    check(lib().rmlk_hip_matmul_partials(stream, kk.FLOAT, m, n, k, a.data_ptr(), k, w.data_ptr(), n, 0,
+    check(lib().rmlk_hip_matmul_partials(stream, kk.FLOAT, m, n, k, a.data_ptr(), k, kk.FLOAT, w.data_ptr(), n, 0,
                                          ws.data_ptr(), need, ctypes.byref(splits)),
           "rmlk_hip_matmul_partials")
     assert 1 <= splits.value and splits.value * m * n * 4 <= need
@@ -1466,7 +1466,7 @@ def test_matmul_partials_feed_the_norm(device, m, n, k):
         wt = w.t().contiguous()
         ws_t = torch.empty(need, dtype=torch.uint8, device=device)
         splits_t = ctypes.c_int32(0)
-        check(lib().rmlk_hip_matmul_partials(stream, kk.FLOAT, m, n, k, a.data_ptr(), k, wt.data_ptr(), k, 1,
+        check(lib().rmlk_hip_matmul_partials(stream, kk.FLOAT, m, n, k, a.data_ptr(), k, kk.FLOAT, wt.data_ptr(), k, 1,
                                              ws_t.data_ptr(), need, ctypes.byref(splits_t)),
               "rmlk_hip_matmul_partials")
         assert splits_t.value == splits.value

@@ -262,3 +262,37 @@ def test_pow_and_cast_and_intdiv_semantics():
     assert np.array_equal(ops.range_(np.int64(10), np.int64(1), np.int64(-4)), [10, 6, 2])
     assert ops.range_(np.float32(0), np.float32(1), np.float32(0.25)).tolist() == [0, 0.25, 0.5, 0.75]
     assert np.array_equal(ops.reduce_mean(np.full((3, 4), 2.5, np.float32), [1]), np.full((3, 1), 2.5))
+
+
+def test_weight_storage_rounding_closed_forms_and_torch():
+    """oracle.ops.store_weights: closed forms a wrong rounding rule fails (ties to even in both
+    directions, carry into the exponent, overflow to infinity, NaN kept, signed zero), then torch's
+    own CPU conversions on random floats of every magnitude."""
+    import torch
+
+    def f32(bits):
+        return np.array(bits, dtype=np.uint32).view(np.float32)
+
+    # bfloat16 keeps the upper 16 bits: 0x3F80_8000 is the tie between 0x3F80 (even) and 0x3F81
+    got = ops.store_weights(f32([0x3F808000, 0x3F818000, 0x3F808001, 0x3F807FFF, 0x3FFF8000, 0x7F7FFFFF,
+                                 0x80000000, 0x00000001, 0xFF800000]), "bf16").view(np.uint32)
+    assert [hex(v) for v in got] == [hex(v) for v in
+                                     [0x3F800000, 0x3F820000, 0x3F810000, 0x3F800000, 0x40000000, 0x7F800000,
+                                      0x80000000, 0x00000000, 0xFF800000]]
+    assert np.isnan(ops.store_weights(f32([0x7FC00001, 0x7F800001, 0xFFFFFFFF]), "bf16")).all()
+    # binary16: 11 significant bits, so 2049 is the tie between 2048 (even) and 2050, 2051 between
+    # 2050 and 2052 (even); 65520 is the tie that overflows; 2^-25 is the tie between 0 and the
+    # smallest subnormal 2^-24
+    np.testing.assert_array_equal(
+        ops.store_weights(np.array([2049.0, 2051.0, 65519.0, 65520.0, 2.0 ** -25, 1.5 * 2.0 ** -25, -0.0],
+                                   dtype=np.float32), "f16"),
+        np.array([2048.0, 2052.0, 65504.0, np.inf, 0.0, 2.0 ** -24, -0.0], dtype=np.float32))
+    rng = np.random.default_rng(16)
+    bits = rng.integers(0, 2 ** 32, size=200000, dtype=np.uint64).astype(np.uint32)
+    x = bits.view(np.float32)
+    x = x[np.isfinite(x)]
+    for name, tdt in (("f16", torch.float16), ("bf16", torch.bfloat16)):
+        exp = torch.from_numpy(x.copy()).to(tdt).to(torch.float32).numpy()
+        np.testing.assert_array_equal(ops.store_weights(x, name).view(np.uint32), exp.view(np.uint32))
+    with pytest.raises(ops.OracleError):
+        ops.store_weights(x[:4], "fp8")
