@@ -101,7 +101,7 @@ def run_llama(args):
     t0 = time.perf_counter()
     torch.cuda.synchronize()
     free_before = torch.cuda.mem_get_info(0)[0]
-    inst = runtime.Builder.from_graph(graph).build(0)
+    inst = runtime.Builder.from_graph(graph).build(0, weights=args.weights)
     torch.cuda.synchronize()
     weights_resident = free_before - torch.cuda.mem_get_info(0)[0]
     log(f"[bench] session created (weights uploaded) in {time.perf_counter() - t0:.1f}s, "
@@ -174,8 +174,9 @@ def run_llama(args):
             flops = 2.0 * batch * m * n * k
             d["us"] += s["micros"] * flops / node_flops     # a node of several launches: by flops
             d["flops"] += flops
-            d["alg_bytes"] += 4.0 * batch * (m * k + k * n + m * (n // 2 if swiglu else n))
-            pmc = PMC_TRAFFIC_KIB.get(shape)
+            w_bytes = 4.0 if args.weights == "f32" else 2.0
+            d["alg_bytes"] += batch * (4.0 * m * k + w_bytes * k * n + 4.0 * m * (n // 2 if swiglu else n))
+            pmc = PMC_TRAFFIC_KIB.get(shape) if args.weights == "f32" else None
             if pmc is not None and pmc[0] != kind:
                 pmc = None                       # another kernel than the one the counters were read for
             d["traffic"] = None if pmc is None or d["traffic"] is None else d["traffic"] + 1024.0 * sum(pmc[1:])
@@ -192,7 +193,7 @@ def run_llama(args):
     # same counts, weights rotated so that they come from HBM as in the model), issued back to back
     # through the C ABI between ONE pair of HIP events on the stream they run on. (The per-node
     # events above add a cache write-back after every node, ~10 us on a 16 MiB output.)
-    dom_us = time_matmul_launches(kernels, torch, dom["shapes"])
+    dom_us = time_matmul_launches(kernels, torch, dom["shapes"], storage=args.weights)
     achieved = dom["flops"] / dom["launches"] / (dom_us * 1e-6) / 1e12
     roofline = {
         "bound": "mfma",
@@ -254,15 +255,15 @@ def run_llama(args):
             inst.replay()
         inst.sync()
         decode_dev_ms = (time.perf_counter() - t0) / 20 * 1e3
-        weight_bytes = decode_weight_bytes(cfg)
+        weight_bytes = decode_weight_bytes(cfg, args.weights)
         log(f"[bench] decode: {decode_ms:.3f} ms/token end to end, {decode_dev_ms:.3f} ms/token "
             f"device replay ({weight_bytes / decode_dev_ms / 1e6:.0f} GB/s of weights)")
     else:
-        decode_dev_ms, weight_bytes = None, decode_weight_bytes(cfg)
+        decode_dev_ms, weight_bytes = None, decode_weight_bytes(cfg, args.weights)
 
     # ---- CPU baseline: the oracle on a bounded sample -------------------------------------------
     cpu = None
-    if not args.no_cpu:
+    if not args.no_cpu and args.weights == "f32":
         n_cpu = min(args.cpu_tokens, prompt_len)
         cores, blas = cpu_threads()
         cpu_tok_s, cpu_s, cpu_logits = cpu_baseline(graph, cfg, graphs, prompt, n_cpu, max_len)
@@ -291,6 +292,7 @@ def run_llama(args):
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "weight_storage": args.weights,
         "config": {"workload": "BASELINE configs[3]: full Llama-3.2-1B-shaped ONNX-op graph, fp32, "
                                f"prefill {prompt_len} tokens + {decode_steps} greedy decode steps, batch 1, "
                                "KV cache updated by ScatterND, random-init weights N(0,0.02)",
@@ -309,7 +311,7 @@ def run_llama(args):
     return result
 
 
-def time_matmul_launches(kernels, torch, shape_counts, reps=4, warm_reps=8):
+def time_matmul_launches(kernels, torch, shape_counts, reps=4, warm_reps=8, storage="f32"):
     """Average duration (us) of rmlk_hip_matmul launches: for every (batch, m, n, k) -> count, `count`
     launches with a broadcast 2-D K-contiguous weight operand taken in turn from enough distinct buffers to
     exceed the 256 MB Infinity Cache, all between one pair of HIP events on the current stream.
@@ -324,6 +326,8 @@ def time_matmul_launches(kernels, torch, shape_counts, reps=4, warm_reps=8):
         a = torch.randn(batch, m, k, device=dev)
         nb = max(2, min(count, int(600e6 // (4 * k * n)) + 1))
         bs = [torch.randn(n, k, device=dev) * 0.02 for _ in range(nb)]   # K-contiguous, as a session stores weights
+        if storage != "f32":
+            bs = [kernels.store_weights(b, {"f16": torch.float16, "bf16": torch.bfloat16}[storage]) for b in bs]
         c = torch.empty(batch, m, n // 2 if swiglu else n, device=dev)
         need = kernels.matmul_workspace_size(batch, m, n, k)
         ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
@@ -335,6 +339,9 @@ def time_matmul_launches(kernels, torch, shape_counts, reps=4, warm_reps=8):
             for i in range(count):
                 if swiglu:
                     kernels.matmul_swiglu(a, bs[i % len(bs)], c, m, n // 2, k, k, 0, n // 2, trans_b=True)
+                elif storage != "f32":
+                    # (the product over stored weights: the grouped entry point with one member)
+                    kernels.matmul_grouped(a, bs[i % len(bs)], [c], m, k, [n], workspace=ws, trans_b=True)
                 else:
                     kernels.matmul(a, bs[i % len(bs)], c, batch, m, n, k, k, k, n, m * k, 0, m * n,
                                    trans_b=True, workspace=ws)
@@ -349,12 +356,13 @@ def time_matmul_launches(kernels, torch, shape_counts, reps=4, warm_reps=8):
     return e0.elapsed_time(e1) * 1e3 / (reps * total)
 
 
-def decode_weight_bytes(cfg):
-    """Weights streamed once per decoded token (fp32): per layer q,o,k,v,gate,up,down + lm-head."""
+def decode_weight_bytes(cfg, storage="f32"):
+    """Weights streamed once per decoded token: per layer q,o,k,v,gate,up,down + lm-head, 4 bytes
+    each as the reference holds them, 2 with 16-bit weight storage."""
     kvd = cfg.kv_heads * cfg.head_dim
     per_layer = (2 * cfg.hidden * cfg.heads * cfg.head_dim + 2 * cfg.hidden * kvd +
                  3 * cfg.hidden * cfg.ffn)
-    return 4.0 * (cfg.layers * per_layer + cfg.hidden * cfg.vocab)
+    return (4.0 if storage == "f32" else 2.0) * (cfg.layers * per_layer + cfg.hidden * cfg.vocab)
 
 
 def matmul_launches(cfg, s, max_len):
@@ -764,6 +772,10 @@ def main():
     ap.add_argument("--decode", type=int, default=128)
     ap.add_argument("--cpu-tokens", type=int, default=512)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--weights", default="f32", choices=["f32", "f16", "bf16"],
+                    help="llama suite: how the session stores the constant MatMul weights (arithmetic is "
+                         "fp32 in every case). The reference and the headline figure are f32; with a 16-bit "
+                         "storage the oracle leg is skipped (it walks the unrounded graph)")
     ap.add_argument("--tiny", action="store_true", help="2-layer toy shape (plumbing check only)")
     ap.add_argument("--suite", default="llama", choices=["llama", "ops", "c1", "c3", "c5"])
     ap.add_argument("--ops-launches", type=int, default=100, help="ops suite: launches per recorded graph")

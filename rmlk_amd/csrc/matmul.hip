@@ -1345,8 +1345,12 @@ __device__ __forceinline__ void gemv_wave_dots(const float *__restrict__ x, cons
     for (int c = 0; c < COLS; ++c) acc[c] = wave_sum(acc[c]);
 }
 
+// COLS == 2 (rows of 16-bit weights that are one chunk of four units per lane): a wavefront takes
+// two rows of Wt, so that it has eight loads per lane in flight like a wavefront over one row of
+// floats - two neighbouring outputs, or SWIGLU the gate and the up row of its output, which then
+// meet in registers.
 template <bool SWIGLU = false, bool NORM = false, int NU = kGemvNormUnits, typename WS = StoredF32,
-          int DEPTH = kGemvDepth>
+          int DEPTH = kGemvDepth, int COLS = 1>
 __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__restrict__ x,
                                                           const typename WS::elem *__restrict__ wt,
                                                           float *__restrict__ y, int32_t n, int32_t k,
@@ -1355,30 +1359,51 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_kernel(const float *__re
                                                           RowNormArgs norm) {
     // A wavefront per row of Wt. SWIGLU: wavefronts 2 p and 2 p + 1 of a block take the gate and
     // the up row of one output and meet in LDS (both rows in one wavefront, sixteen loads per lane
-    // in flight, was 22.0 against 20.5 us on 2 x 8192 rows).
+    // in flight, was 22.0 against 20.5 us on 2 x 8192 rows of floats).
     constexpr int kWaves = kThreads / kWave;
-    constexpr int kOutputs = SWIGLU ? kWaves / 2 : kWaves;    // per block
+    constexpr int kOutputs = SWIGLU ? kWaves * COLS / 2 : kWaves * COLS;    // per block
     [[maybe_unused]] __shared__ float pair_acc[kWaves];
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int col = blockIdx.x * kOutputs + (SWIGLU ? wave / 2 : wave);
-    // (a wavefront past the last column keeps valid addresses and takes part in the barriers)
-    const int col_c = min(col, n - 1);
-    const int64_t row = SWIGLU ? ((wave & 1) ? up_row : gate_row) + col_c : col_c;
-    const v4f *wv[1];
-    wv[0] = reinterpret_cast<const v4f *>(wt + row * ldw);
-    float acc[1];
-    gemv_wave_dots<1, NORM, NU, WS, DEPTH>(x, wv, k, norm, col < n, acc);
-    if constexpr (SWIGLU) {
-        if (lane == 0) pair_acc[wave] = acc[0];
-        __syncthreads();
-        if (col < n && lane == 0 && !(wave & 1)) {
-            const float gate = acc[0], up = pair_acc[wave + 1];
+    if constexpr (COLS == 2) {
+        const int col = blockIdx.x * kOutputs + (SWIGLU ? wave : 2 * wave);
+        // (a wavefront past the last column keeps valid addresses and takes part in the barriers)
+        const int col_c = min(col, n - 1);
+        const int64_t row0 = SWIGLU ? gate_row + col_c : col_c;
+        const int64_t row1 = SWIGLU ? up_row + col_c : min(col + 1, n - 1);
+        const v4f *wv[2];
+        wv[0] = reinterpret_cast<const v4f *>(wt + row0 * ldw);
+        wv[1] = reinterpret_cast<const v4f *>(wt + row1 * ldw);
+        float acc[2];
+        gemv_wave_dots<2, NORM, NU, WS, DEPTH>(x, wv, k, norm, col < n, acc);
+        if (col >= n || lane != 0) return;
+        if constexpr (SWIGLU) {
+            const float gate = acc[0], up = acc[1];
             const float silu = gate * (1.0f / (1.0f + expf(-gate)));
             y[col] = silu * up;
+        } else {
+            y[col] = residual ? acc[0] + residual[col] : acc[0];
+            if (col + 1 < n) y[col + 1] = residual ? acc[1] + residual[col + 1] : acc[1];
         }
     } else {
-        if (col < n && lane == 0) y[col] = residual ? acc[0] + residual[col] : acc[0];
+        const int col = blockIdx.x * kOutputs + (SWIGLU ? wave / 2 : wave);
+        const int col_c = min(col, n - 1);
+        const int64_t row = SWIGLU ? ((wave & 1) ? up_row : gate_row) + col_c : col_c;
+        const v4f *wv[1];
+        wv[0] = reinterpret_cast<const v4f *>(wt + row * ldw);
+        float acc[1];
+        gemv_wave_dots<1, NORM, NU, WS, DEPTH>(x, wv, k, norm, col < n, acc);
+        if constexpr (SWIGLU) {
+            if (lane == 0) pair_acc[wave] = acc[0];
+            __syncthreads();
+            if (col < n && lane == 0 && !(wave & 1)) {
+                const float gate = acc[0], up = pair_acc[wave + 1];
+                const float silu = gate * (1.0f / (1.0f + expf(-gate)));
+                y[col] = silu * up;
+            }
+        } else {
+            if (col < n && lane == 0) y[col] = residual ? acc[0] + residual[col] : acc[0];
+        }
     }
 }
 
@@ -1406,7 +1431,7 @@ struct GemvRowStreams {
     int32_t *err;
 };
 
-template <bool NORM, int NU = kGemvNormUnits, typename WS = StoredF32, int DEPTH = kGemvDepth>
+template <bool NORM, int NU = kGemvNormUnits, typename WS = StoredF32, int DEPTH = kGemvDepth, int COLS = 1>
 __global__ __launch_bounds__(kThreads) void gemv_kmajor_rows_kernel(const float *__restrict__ x,
                                                                     const typename WS::elem *__restrict__ wt,
                                                                     int32_t k,
@@ -1415,13 +1440,14 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_rows_kernel(const float 
     // A wavefront per column, like the plain product (two columns per wavefront left the SIMDs with
     // one or two wavefronts each, 8.5 against 6.3 us on the 3072 columns of q, k and v): wavefronts
     // 2 p and 2 p + 1 of a block take columns d and d + D / 2 of a pair and meet in LDS.
+    // COLS == 2 (see gemv_kmajor_kernel): one wavefront takes both columns of a pair.
     constexpr int kWaves = kThreads / kWave;
-    __shared__ float pair_acc[kWaves];
+    [[maybe_unused]] __shared__ float pair_acc[kWaves];
     // (the wavefront's number as a scalar: everything derived from it - the stream, the head, the
     // row of the weights - then lives in scalar registers and the stream table is read with scalar loads)
     const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int pair = blockIdx.x * (kWaves / 2) + wave / 2;
-    const int second = wave & 1;
+    const int pair = COLS == 2 ? blockIdx.x * kWaves + wave : blockIdx.x * (kWaves / 2) + wave / 2;
+    const int second = COLS == 2 ? 0 : wave & 1;
     const bool active = pair < rs.total_pairs;
     const int pair_c = min(pair, rs.total_pairs - 1);
     int si = 0;
@@ -1432,8 +1458,9 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_rows_kernel(const float 
     const int local = pair_c - st.first_pair;
     const int head = local / rs.half, d = local - head * rs.half;
     const int col = st.first_col + head * (2 * rs.half) + d + second * rs.half;
-    const v4f *wv[1];
+    const v4f *wv[COLS];
     wv[0] = reinterpret_cast<const v4f *>(wt + static_cast<int64_t>(col) * ldw);
+    if constexpr (COLS == 2) wv[1] = reinterpret_cast<const v4f *>(wt + static_cast<int64_t>(col + rs.half) * ldw);
     // what the epilogue needs from memory (in the wavefront that runs it), requested behind the
     // first weights
     float c1 = 1.f, c2 = 1.f, s1 = 0.f, s2 = 0.f;
@@ -1453,12 +1480,18 @@ __global__ __launch_bounds__(kThreads) void gemv_kmajor_rows_kernel(const float 
                 ix[t] = t < st.tuple_size ? st.idx[static_cast<int64_t>(head) * st.tuple_size + t] : 0;
         }
     };
-    float acc[1];
-    gemv_wave_dots<1, NORM, NU, WS, DEPTH>(x, wv, k, norm, active, acc, epilogue_loads);
-    if (lane == 0) pair_acc[wave] = acc[0];
-    __syncthreads();
+    float acc[COLS];
+    gemv_wave_dots<COLS, NORM, NU, WS, DEPTH>(x, wv, k, norm, active, acc, epilogue_loads);
+    float x2;
+    if constexpr (COLS == 2) {
+        x2 = acc[1];
+    } else {
+        if (lane == 0) pair_acc[wave] = acc[0];
+        __syncthreads();
+        x2 = second ? 0.f : pair_acc[wave + 1];
+    }
     if (!active || lane != 0 || second) return;
-    const float x1 = acc[0], x2 = pair_acc[wave + 1];
+    const float x1 = acc[0];
     float y1 = x1, y2 = x2;
     if (st.cos) {
         // (products and sums rounded one by one, although this file is compiled with contraction
@@ -2262,15 +2295,17 @@ bool kmajor_rows_ok(int64_t k, const void *wt, int64_t ldw) {
     return k % WS::kUnit == 0 && ldw % WS::kUnit == 0 && reinterpret_cast<uintptr_t>(wt) % 16 == 0;
 }
 
-// f(storage tag, units per lane and chunk) for a row of k weights stored as `w_dtype`.
+// f(storage tag, units per lane and chunk, rows per wavefront) for a row of k weights stored as
+// `w_dtype`: short rows of 16-bit weights are walked four units at a time, two rows per wavefront.
 template <typename F>
 int32_t with_storage_depth(int32_t w_dtype, int64_t k, F &&f) {
     return with_storage(w_dtype, [&](auto ws) -> int32_t {
         using WS = decltype(ws);
         if constexpr (kStored16<WS>) {
-            if (k < 64 * 8 * WS::kUnit) return f(ws, std::integral_constant<int, 4>{});
+            if (k < 64 * 8 * WS::kUnit)
+                return f(ws, std::integral_constant<int, 4>{}, std::integral_constant<int, 2>{});
         }
-        return f(ws, std::integral_constant<int, kGemvDepth>{});
+        return f(ws, std::integral_constant<int, kGemvDepth>{}, std::integral_constant<int, 1>{});
     });
 }
 
@@ -2293,18 +2328,18 @@ int32_t gemv_kmajor_launch(rmlk_stream_t stream, int32_t dtype, int64_t n, int64
     hipStream_t s = as_stream(stream);
     constexpr int kWaves = kThreads / kWave;
     const int32_t ni = static_cast<int32_t>(n), ki = static_cast<int32_t>(k);
-    const unsigned grid = static_cast<unsigned>((n + kWaves - 1) / kWaves);
-    return with_storage_depth(w_dtype, k, [&](auto ws, auto depth) -> int32_t {
+    return with_storage_depth(w_dtype, k, [&](auto ws, auto depth, auto cols) -> int32_t {
         using WS = decltype(ws);
-        constexpr int D = decltype(depth)::value;
+        constexpr int D = decltype(depth)::value, C = decltype(cols)::value;
         if (!kmajor_rows_ok<WS>(k, wt, ldw)) return RMLK_ERR_UNSUPPORTED;
         const typename WS::elem *pw = static_cast<const typename WS::elem *>(wt);
+        const unsigned grid = static_cast<unsigned>((n + kWaves * C - 1) / (kWaves * C));
         if (norm && k <= kThreads * 4 * 2)
-            gemv_kmajor_kernel<false, true, 2, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
+            gemv_kmajor_kernel<false, true, 2, WS, D, C><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
         else if (norm)
-            gemv_kmajor_kernel<false, true, kGemvNormUnits, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
+            gemv_kmajor_kernel<false, true, kGemvNormUnits, WS, D, C><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, *norm);
         else
-            gemv_kmajor_kernel<false, false, kGemvNormUnits, WS, D><<<grid, kThreads, 0, s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, RowNormArgs{});
+            gemv_kmajor_kernel<false, false, kGemvNormUnits, WS, D, C><<<grid, kThreads, 0, s>>>(px, pw, py, ni, ki, ldw, 0, 0, pr, RowNormArgs{});
         return launch_status();
     });
 }
@@ -2323,25 +2358,26 @@ int32_t gemv_kmajor_swiglu_launch(rmlk_stream_t stream, int32_t dtype, int64_t n
     if (norm && (k == 0 || k > kThreads * 4 * 8 || reinterpret_cast<uintptr_t>(norm->gamma) % 16 != 0))
         return RMLK_ERR_UNSUPPORTED;
     constexpr int kOutputsPerBlock = kThreads / kWave / 2;   // a wavefront per gate row and per up row
-    const unsigned grid = static_cast<unsigned>((n + kOutputsPerBlock - 1) / kOutputsPerBlock);
     const float *px = static_cast<const float *>(x);
     float *py = static_cast<float *>(y);
     const int32_t ni = static_cast<int32_t>(n), ki = static_cast<int32_t>(k);
     const int32_t gr = static_cast<int32_t>(gate_row), ur = static_cast<int32_t>(up_row);
     hipStream_t s = as_stream(stream);
-    return with_storage_depth(w_dtype, k, [&](auto ws, auto depth) -> int32_t {
+    return with_storage_depth(w_dtype, k, [&](auto ws, auto depth, auto cols) -> int32_t {
         using WS = decltype(ws);
-        constexpr int D = decltype(depth)::value;
+        constexpr int D = decltype(depth)::value, C = decltype(cols)::value;
         if (!kmajor_rows_ok<WS>(k, wt, ldw)) return RMLK_ERR_UNSUPPORTED;
         const typename WS::elem *pw = static_cast<const typename WS::elem *>(wt);
+        // (two rows per wavefront: the gate and the up row of one output)
+        const unsigned grid = static_cast<unsigned>((n + kOutputsPerBlock * C - 1) / (kOutputsPerBlock * C));
         if (norm && k <= kThreads * 4 * 2)
-            gemv_kmajor_kernel<true, true, 2, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(
+            gemv_kmajor_kernel<true, true, 2, WS, D, C><<<grid, kThreads, k * sizeof(float), s>>>(
                 px, pw, py, ni, ki, ldw, gr, ur, nullptr, *norm);
         else if (norm)
-            gemv_kmajor_kernel<true, true, kGemvNormUnits, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(
+            gemv_kmajor_kernel<true, true, kGemvNormUnits, WS, D, C><<<grid, kThreads, k * sizeof(float), s>>>(
                 px, pw, py, ni, ki, ldw, gr, ur, nullptr, *norm);
         else
-            gemv_kmajor_kernel<true, false, kGemvNormUnits, WS, D><<<grid, kThreads, 0, s>>>(
+            gemv_kmajor_kernel<true, false, kGemvNormUnits, WS, D, C><<<grid, kThreads, 0, s>>>(
                 px, pw, py, ni, ki, ldw, gr, ur, nullptr, RowNormArgs{});
         return launch_status();
     });
@@ -2419,23 +2455,23 @@ extern "C" int32_t rmlk_hip_gemv_kmajor_head_rows(rmlk_stream_t stream, int32_t 
     rs.half = static_cast<int32_t>(d_common / 2);
     rs.total_pairs = static_cast<int32_t>(pairs);
     constexpr int kPairsPerBlock = kThreads / kWave / 2;
-    const unsigned grid = static_cast<unsigned>((pairs + kPairsPerBlock - 1) / kPairsPerBlock);
     const float *px = static_cast<const float *>(x);
     const int32_t ki = static_cast<int32_t>(k);
     hipStream_t s = as_stream(stream);
-    return with_storage_depth(w_dtype, k, [&](auto ws, auto depth) -> int32_t {
+    return with_storage_depth(w_dtype, k, [&](auto ws, auto depth, auto cols) -> int32_t {
         using WS = decltype(ws);
-        constexpr int D = decltype(depth)::value;
+        constexpr int D = decltype(depth)::value, C = decltype(cols)::value;
         if (!kmajor_rows_ok<WS>(k, wt, ldw)) return RMLK_ERR_UNSUPPORTED;
         const typename WS::elem *pw = static_cast<const typename WS::elem *>(wt);
+        const unsigned grid = static_cast<unsigned>((pairs + kPairsPerBlock * C - 1) / (kPairsPerBlock * C));
         if (gamma) {
             const RowNormArgs norm{static_cast<const float *>(gamma), eps, reciprocal_form};
             if (k <= kThreads * 4 * 2)
-                gemv_kmajor_rows_kernel<true, 2, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
+                gemv_kmajor_rows_kernel<true, 2, WS, D, C><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
             else
-                gemv_kmajor_rows_kernel<true, kGemvNormUnits, WS, D><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
+                gemv_kmajor_rows_kernel<true, kGemvNormUnits, WS, D, C><<<grid, kThreads, k * sizeof(float), s>>>(px, pw, ki, ldw, norm, rs);
         } else {
-            gemv_kmajor_rows_kernel<false, kGemvNormUnits, WS, D><<<grid, kThreads, 0, s>>>(px, pw, ki, ldw, RowNormArgs{}, rs);
+            gemv_kmajor_rows_kernel<false, kGemvNormUnits, WS, D, C><<<grid, kThreads, 0, s>>>(px, pw, ki, ldw, RowNormArgs{}, rs);
         }
         return launch_status();
     });
