@@ -608,14 +608,15 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
                 b_raw[p] = *reinterpret_cast<const v4u *>(reinterpret_cast<const char *>(b16_ptr) + b16_voff[p]);
         }
     };
-    [[maybe_unused]] auto b16_store = [&](int buf, int p) {
+    // (one half of a unit per call: four values widened, one 128-bit LDS store - a short enough run
+    // of instructions to fit between two MFMAs)
+    [[maybe_unused]] auto b16_store = [&](int buf, int p, int h) {
         if constexpr (B16) {
             if (B16_UNITS % kThreads == 0 || p * kThreads + tid < B16_UNITS) {
-                float w[8];
-                widen_unit<WS>(b_raw[p], w);
-                float *bs = Bs + buf * kBFloats;
-                *reinterpret_cast<v4f *>(bs + b16_lds[p][0]) = v4f{w[0], w[1], w[2], w[3]};
-                *reinterpret_cast<v4f *>(bs + b16_lds[p][1]) = v4f{w[4], w[5], w[6], w[7]};
+                float w0, w1, w2, w3;
+                WS::widen2(b_raw[p][2 * h], w0, w1);
+                WS::widen2(b_raw[p][2 * h + 1], w2, w3);
+                *reinterpret_cast<v4f *>(Bs + buf * kBFloats + b16_lds[p][h]) = v4f{w0, w1, w2, w3};
             }
         }
     };
@@ -691,7 +692,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
             constexpr int n_frag = last ? (MORE ? kFragOps : 0) : kFragOps;
             // 16-bit B, first chunk: the stage in the registers goes to LDS before the loads of this
             // step are issued, the stage after it is requested behind them
-            constexpr int n_store = B16 && LOAD && kc == 0 ? B16_PASSES : 0;
+            constexpr int n_store = B16 && LOAD && kc == 0 ? 2 * B16_PASSES : 0;
             constexpr int n_direct = load_hi - load_lo;
             constexpr int n_b16 = B16 && LOAD2 && kc == 0 ? B16_PASSES : 0;
             constexpr int n_ops = n_frag + n_store + n_direct + n_b16;
@@ -711,7 +712,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
                             if constexpr (last) frag_op(other, 0, slot ^ 1, o);
                             else frag_op(buf, kc + 1, slot ^ 1, o);
                         } else if constexpr (o < n_frag + n_store) {
-                            b16_store(other, o - n_frag);
+                            b16_store(other, (o - n_frag) / 2, (o - n_frag) % 2);
                         } else if constexpr (o < n_frag + n_store + n_direct) {
                             load_op(other, load_lo + o - n_frag - n_store);
                         } else {
@@ -736,7 +737,10 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
             for (int p = 0; p < B16_PASSES; ++p) b16_load(p);
             b16_ptr += BK;
 #pragma unroll
-            for (int p = 0; p < B16_PASSES; ++p) b16_store(0, p);
+            for (int p = 0; p < B16_PASSES; ++p) {
+                b16_store(0, p, 0);
+                b16_store(0, p, 1);
+            }
             if (n_steps > 1) {
 #pragma unroll
                 for (int p = 0; p < B16_PASSES; ++p) b16_load(p);
