@@ -539,6 +539,24 @@ int32_t rmlk_hip_gemv_kmajor_head_rows(rmlk_stream_t stream, int32_t dtype, int6
                                        const rmlk_row_stream *streams, const int64_t *first_col,
                                        int32_t *err_flag);
 
+/* ---- launches over tiny tensors collected into one ------------------------------------------------
+ * Between rmlk_hip_batch_begin and rmlk_hip_batch_end on a stream, calls of rmlk_hip_binary (not
+ * Pow), rmlk_hip_unary, rmlk_hip_cast, rmlk_hip_where, rmlk_hip_expand and rmlk_hip_concat_many whose
+ * output has at most 4096 elements (FLOAT, DOUBLE, INT32, INT64, BOOL operands; any element size for
+ * the moves) do not launch: they are recorded, and one single-block launch runs up to 24 records in
+ * order with the element arithmetic of the kernels they replace (same bits). Every other call of
+ * this library on the stream, rmlk_hip_batch_flush and rmlk_hip_batch_end send the recorded calls
+ * out first, so effects keep the order of the calls; the operands of a recorded call must stay
+ * valid until then. A caller that issues work on the stream by other means (its own kernels,
+ * hipMemcpyAsync, events) calls rmlk_hip_batch_flush before it does. A decode step spends a dozen
+ * launches on such tensors (a position turned into rotary tables, scatter indices, a mask).
+ * rmlk_hip_batch_end returns the status of the launches the batch made. Recordable into a HIP
+ * graph. No counterpart in the reference (one kernel per operator,
+ * runtime/src/core/instance.rs:100-112). */
+int32_t rmlk_hip_batch_begin(rmlk_stream_t stream);
+int32_t rmlk_hip_batch_flush(rmlk_stream_t stream);
+int32_t rmlk_hip_batch_end(rmlk_stream_t stream);
+
 /* Fill `n` elements of `out` with the element at host address `value` (size of dtype).
  * ref: runtime/src/providers/cuda/backend/constant_of_shape.rs:59-62 (host vector + H2D). */
 int32_t rmlk_hip_fill(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *value,

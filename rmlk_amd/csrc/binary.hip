@@ -4,92 +4,12 @@
 // (cuda/src/ptx/headers/binary_op_macros.cuh:14-42).
 #include <type_traits>
 
+#include "batch.hpp"
 #include "elementwise.hpp"
+#include "functors.hpp"
 
 namespace rmlk {
 namespace {
-
-template <typename T>
-struct AddF {
-    static __device__ __forceinline__ T apply(T x, T y) {
-        if constexpr (std::is_integral<T>::value) {
-            using U = typename std::make_unsigned<T>::type;
-            return static_cast<T>(static_cast<U>(x) + static_cast<U>(y));
-        } else {
-            return x + y;
-        }
-    }
-};
-template <typename T>
-struct SubF {
-    static __device__ __forceinline__ T apply(T x, T y) {
-        if constexpr (std::is_integral<T>::value) {
-            using U = typename std::make_unsigned<T>::type;
-            return static_cast<T>(static_cast<U>(x) - static_cast<U>(y));
-        } else {
-            return x - y;
-        }
-    }
-};
-template <typename T>
-struct MulF {
-    static __device__ __forceinline__ T apply(T x, T y) {
-        if constexpr (std::is_integral<T>::value) {
-            using U = typename std::make_unsigned<T>::type;
-            return static_cast<T>(static_cast<U>(x) * static_cast<U>(y));
-        } else {
-            return x * y;
-        }
-    }
-};
-// Integer division truncates toward zero (cuda/src/ptx/div.cu:9-12). The reference leaves x/0 and
-// MIN/-1 undefined; here x/0 = 0 and MIN/-1 wraps to MIN so that no input can trap.
-template <typename T>
-struct DivF {
-    static __device__ __forceinline__ T apply(T x, T y) {
-        if constexpr (std::is_integral<T>::value) {
-            using U = typename std::make_unsigned<T>::type;
-            if (y == 0) return 0;
-            if (y == static_cast<T>(-1)) return static_cast<T>(U(0) - static_cast<U>(x));
-            return x / y;
-        } else {
-            return x / y;
-        }
-    }
-};
-template <typename T>
-struct EqualF {
-    static __device__ __forceinline__ uint8_t apply(T x, T y) { return x == y ? 1 : 0; }
-};
-template <typename T>
-struct GreaterF {
-    static __device__ __forceinline__ uint8_t apply(T x, T y) { return x > y ? 1 : 0; }
-};
-
-// Pow (cuda/src/ptx/pow.cu:18-65): float base -> powf(x, (float)y); double base -> pow; integer
-// base -> llround(pow((double)x, (double)y)). Exponents 2, 3 and 0.5 take the product / sqrt
-// forms, which are the correctly rounded results the CPU oracle produces for them.
-template <typename TX, typename TY>
-struct PowF {
-    static __device__ __forceinline__ TX apply(TX x, TY y) {
-        if constexpr (std::is_same<TX, float>::value) {
-            float e = static_cast<float>(y);
-            if (e == 2.0f) return x * x;
-            if (e == 3.0f) return x * x * x;
-            if (e == 0.5f) return sqrtf(x);
-            return powf(x, e);
-        } else if constexpr (std::is_same<TX, double>::value) {
-            double e = static_cast<double>(y);
-            if (e == 2.0) return x * x;
-            if (e == 3.0) return x * x * x;
-            if (e == 0.5) return sqrt(x);
-            return pow(x, e);
-        } else {
-            double r = pow(static_cast<double>(x), static_cast<double>(y));
-            return static_cast<TX>(llround(r));
-        }
-    }
-};
 
 template <template <typename> class F, typename T, typename TO>
 int32_t run_same(hipStream_t s, int rank, const int64_t *shape, const int64_t (*st)[kMaxRank],
@@ -175,8 +95,21 @@ extern "C" int32_t rmlk_hip_binary(rmlk_stream_t stream, int32_t op, int32_t dty
         st[1][d] = b_stride->v[d];
     }
     dense_strides(rank, out_shape->v, st[2]);
-    hipStream_t s = as_stream(stream);
     if (op != RMLK_POW && dtype_a != dtype_b) return RMLK_ERR_UNSUPPORTED;
+    // a tiny operator on a stream that is collecting its launches: handed over as a record
+    if (numel <= kBatchMaxElems && batch_collecting() && op >= RMLK_ADD && op <= RMLK_GREATER && op != RMLK_POW &&
+        (dtype_a == RMLK_FLOAT || dtype_a == RMLK_DOUBLE || dtype_a == RMLK_INT32 || dtype_a == RMLK_INT64)) {
+        SmallOp so{};
+        so.kind = kSmallBinary;
+        so.op = op;
+        so.dt = dtype_a;
+        so.in[0] = a;
+        so.in[1] = b;
+        so.out = out;
+        if (small_op_layout(so, rank, out_shape->v, 2, st) && batch_take(as_stream_collecting(stream), so))
+            return RMLK_OK;
+    }
+    hipStream_t s = as_stream(stream);
     switch (op) {
         case RMLK_ADD: return dispatch_same<AddF, false>(s, dtype_a, rank, out_shape->v, st, a, b, out);
         case RMLK_SUB: return dispatch_same<SubF, false>(s, dtype_a, rank, out_shape->v, st, a, b, out);

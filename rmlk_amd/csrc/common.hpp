@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "../../include/rmlk_hip.h"
@@ -15,7 +16,18 @@ constexpr int kWave = 64;         // CDNA wavefront width
 constexpr int kNumCU = 256;       // MI355X compute units (8 XCDs x 32)
 constexpr int64_t kMaxElems = (int64_t)1 << 62;
 
-inline hipStream_t as_stream(rmlk_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+// Streams on which small launches are being collected (batch.hip), and the call that sends the
+// collected ones of a stream out. Every entry point turns its stream handle into a hipStream_t
+// through as_stream before it issues anything, so whatever was collected is in the stream first.
+extern std::atomic<int> g_open_batches;
+int32_t batch_flush_stream(hipStream_t s);
+inline hipStream_t as_stream(rmlk_stream_t s) {
+    hipStream_t h = reinterpret_cast<hipStream_t>(s);
+    if (g_open_batches.load(std::memory_order_relaxed) > 0) (void)batch_flush_stream(h);
+    return h;
+}
+// (for the entry points that may hand their work to the batch instead)
+inline hipStream_t as_stream_collecting(rmlk_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 // Status of the launch just issued (hipError_t as a positive int, 0 when fine).
 inline int32_t launch_status() { return static_cast<int32_t>(hipGetLastError()); }

@@ -5,6 +5,7 @@
 //
 // Replaces cuda/src/ptx/{transpose,expand,slice,scatter_nd,trilu}.cu and the host memcpy loops of
 // runtime/src/providers/cuda/backend/{gather,concat}.rs in the reference.
+#include "batch.hpp"
 #include "nd_index.hpp"
 
 namespace rmlk {
@@ -765,6 +766,16 @@ extern "C" int32_t rmlk_hip_expand(rmlk_stream_t stream, int32_t dtype, const rm
     if (numel == 0) return RMLK_OK;
     if (!in || !out) return RMLK_ERR_NULL_POINTER;
     dense_strides(rank, out_shape->v, st[1]);
+    if (numel <= kBatchMaxElems && batch_collecting()) {
+        // (a tiny broadcast copy on a stream that is collecting its launches)
+        SmallOp so{};
+        so.kind = kSmallCopy;
+        so.dt = esize;
+        so.in[0] = in;
+        so.out = out;
+        if (small_op_layout(so, rank, out_shape->v, 1, st) && batch_take(as_stream_collecting(stream), so))
+            return RMLK_OK;
+    }
     return strided_copy(as_stream(stream), esize, rank, out_shape->v, st, in, out);
 }
 
@@ -910,6 +921,40 @@ extern "C" int32_t rmlk_hip_concat_many(rmlk_stream_t stream, int32_t dtype, int
     if (dims_numel(out_shape) < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (dims_numel(out_shape) == 0) return RMLK_OK;
     if (!out) return RMLK_ERR_NULL_POINTER;
+    if (dims_numel(out_shape) <= kBatchMaxElems && batch_collecting() && n_inputs <= kBatchMaxOps) {
+        // a tiny Concat on a stream that is collecting its launches: a copy record per input, each
+        // into its columns of the output
+        SmallOp recs[kBatchMaxOps];
+        int n_rec = 0;
+        bool fits = true;
+        int64_t out_st[kMaxRank], at = 0;
+        dense_strides(rank, out_shape->v, out_st);
+        for (int k = 0; k < n_inputs && fits; ++k) {
+            const int64_t len = in_shapes[k].v[axis];
+            if (len > 0 && outer * inner > 0) {
+                if (!ins[k]) return RMLK_ERR_NULL_POINTER;
+                int64_t st2[2][kMaxRank];
+                dense_strides(rank, in_shapes[k].v, st2[0]);
+                for (int d = 0; d < rank; ++d) st2[1][d] = out_st[d];
+                SmallOp &so = recs[n_rec];
+                so = SmallOp{};
+                so.kind = kSmallCopy;
+                so.dt = esize;
+                so.in[0] = ins[k];
+                so.out = static_cast<char *>(out) + at * inner * esize;
+                fits = small_op_layout(so, rank, in_shapes[k].v, 1, st2);
+                ++n_rec;
+            }
+            at += len;
+        }
+        if (fits) {
+            hipStream_t sc = as_stream_collecting(stream);
+            bool taken = true;
+            for (int r = 0; r < n_rec && taken; ++r) taken = batch_take(sc, recs[r]);
+            if (taken) return RMLK_OK;
+            // (no batch on this stream after all: nothing was taken, the launch below does the work)
+        }
+    }
     // one launch when every input's rows and landing columns are whole units of one width
     int unit = 16;
     bool one_launch = n_inputs <= kMaxConcatInputs && outer < ((int64_t)1 << 31);

@@ -49,8 +49,16 @@ public:
     int64_t pool_bytes = 0;
     int64_t hip_mallocs = 0;
     bool forbid_malloc = false;  // set while a HIP graph is being captured
+    // While the launches over tiny tensors of a run are being collected, the buffers such tensors
+    // give back are kept aside until let_go(): handed out again at once, a buffer would make two
+    // collected operators that have nothing to do with each other look dependent (one overwrites
+    // what the other read), and they could not run side by side.
+    bool hold_small = false;
+    static constexpr size_t kSmallBytes = 32 * 1024;   // the largest output a collected operator has
+    void let_go();
 
 private:
+    std::vector<std::pair<void *, size_t>> held_;
     std::map<size_t, std::vector<void *>> free_;
     std::vector<void *> all_;
 };

@@ -118,7 +118,16 @@ void *Pool::alloc(size_t bytes) {
     return p;
 }
 
-void Pool::release(void *p, size_t bytes) { free_[bucket(bytes)].push_back(p); }
+void Pool::release(void *p, size_t bytes) {
+    const size_t b = bucket(bytes);
+    if (hold_small && b <= kSmallBytes) held_.emplace_back(p, b);
+    else free_[b].push_back(p);
+}
+
+void Pool::let_go() {
+    for (const auto &h : held_) free_[h.second].push_back(h.first);
+    held_.clear();
+}
 
 Pool::~Pool() {
     for (void *p : all_) (void)hipFree(p);
@@ -228,6 +237,7 @@ HostVal OpContext::host_values(int i) const {
     if (n > (1u << 20)) fail_op(node.op + ": shape-like input is too large");
     std::vector<uint8_t> tmp(t.nbytes());
     if (!tmp.empty()) {
+        check_status(rmlk_hip_batch_flush(stream), "collected launches");   // (what wrote t may still be collected)
         check_hip(hipMemcpyAsync(tmp.data(), t.data(), tmp.size(), hipMemcpyDeviceToHost, stream),
                   "hipMemcpyAsync D2H");
         check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
@@ -433,6 +443,29 @@ void Session::build(const rmlk_graph &graph, int dev) {
 
 void Session::run_nodes() {
     const rmlk_graph &gr = graph_copy;
+    // Operators over tiny tensors (the per-step set-up of a decoder graph: tables, indices, masks) are
+    // collected by the kernel library and go out as one launch in front of the next larger one. Not
+    // with one kernel per node (no fusion), and not while nodes are timed one by one.
+    struct Collecting {
+        rmlk_stream_t stream;
+        Pool &pool;
+        bool on = false;
+        void stop() {
+            on = false;
+            pool.hold_small = false;
+            pool.let_go();
+        }
+        ~Collecting() {
+            if (!on) return;
+            (void)rmlk_hip_batch_end(stream);   // (an exception is on its way)
+            stop();
+        }
+    } collecting{stream, pool};
+    if (fuse && !profiling) {
+        check_status(rmlk_hip_batch_begin(stream), "collected launches");
+        collecting.on = true;
+        pool.hold_small = true;
+    }
     for (size_t n = 0; n < gr.nodes.size(); ++n) {
         const Node &node = gr.nodes[n];
         if (node.op == "Constant") continue;
@@ -532,6 +565,10 @@ void Session::run_nodes() {
             int v = node.outputs[o];
             if (last_use[v] < 0 && !gr.values[v].is_output) values[v].reset();
         }
+    }
+    if (collecting.on) {
+        collecting.stop();
+        check_status(rmlk_hip_batch_end(stream), "collected launches");
     }
     scratch_bufs.clear();
 }

@@ -5,7 +5,9 @@
 #include <limits>
 #include <type_traits>
 
+#include "batch.hpp"
 #include "elementwise.hpp"
+#include "functors.hpp"
 
 namespace rmlk {
 namespace {
@@ -74,47 +76,6 @@ int32_t launch_map(hipStream_t s, int64_t n, const void *in, void *out) {
     return RMLK_OK;
 }
 
-template <typename T>
-struct SqrtF {
-    static __device__ __forceinline__ T apply(T x) {
-        if constexpr (std::is_same<T, float>::value) return sqrtf(x);
-        else return sqrt(x);
-    }
-};
-// The reference multiplies by -1 (cuda/src/ptx/neg.cu:6); a sign flip gives the same bits.
-template <typename T>
-struct NegF {
-    static __device__ __forceinline__ T apply(T x) {
-        if constexpr (std::is_integral<T>::value) {
-            using U = typename std::make_unsigned<T>::type;
-            return static_cast<T>(U(0) - static_cast<U>(x));
-        } else {
-            return -x;
-        }
-    }
-};
-template <typename T>
-struct SinF {
-    static __device__ __forceinline__ T apply(T x) {
-        if constexpr (std::is_same<T, float>::value) return sinf(x);
-        else return sin(x);
-    }
-};
-template <typename T>
-struct CosF {
-    static __device__ __forceinline__ T apply(T x) {
-        if constexpr (std::is_same<T, float>::value) return cosf(x);
-        else return cos(x);
-    }
-};
-template <typename T>
-struct SigmoidF {
-    static __device__ __forceinline__ T apply(T x) {
-        if constexpr (std::is_same<T, float>::value) return 1.0f / (1.0f + expf(-x));
-        else return 1.0 / (1.0 + exp(-x));
-    }
-};
-
 template <template <typename> class F>
 int32_t dispatch_float(hipStream_t s, int32_t dt, int64_t n, const void *in, void *out) {
     switch (dt) {
@@ -125,37 +86,6 @@ int32_t dispatch_float(hipStream_t s, int32_t dt, int64_t n, const void *in, voi
 }
 
 // ---- cast ------------------------------------------------------------------------------------
-struct BoolTag {
-    uint8_t b;
-};
-
-template <typename TI, typename TO>
-struct CastF {
-    static __device__ __forceinline__ TO apply(TI x) {
-        constexpr bool in_bool = std::is_same<TI, BoolTag>::value;
-        constexpr bool out_bool = std::is_same<TO, BoolTag>::value;
-        if constexpr (in_bool && out_bool) {
-            return BoolTag{static_cast<uint8_t>(x.b ? 1 : 0)};
-        } else if constexpr (in_bool) {
-            return static_cast<TO>(x.b ? 1 : 0);
-        } else if constexpr (out_bool) {
-            return BoolTag{static_cast<uint8_t>(x != static_cast<TI>(0) ? 1 : 0)};
-        } else if constexpr (std::is_integral<TO>::value && !std::is_integral<TI>::value) {
-            // float -> int: truncate toward zero; NaN -> 0; out of range saturates.
-            double v = static_cast<double>(x);
-            if (v != v) return 0;
-            constexpr double lo = static_cast<double>(std::numeric_limits<TO>::min());
-            // max() of 64-bit types is not a double; 2^63 / 2^64 is the first value out of range.
-            constexpr double hi = static_cast<double>(std::numeric_limits<TO>::max());
-            if (v <= lo) return std::numeric_limits<TO>::min();
-            if (v >= hi) return std::numeric_limits<TO>::max();
-            return static_cast<TO>(v);
-        } else {
-            return static_cast<TO>(x);
-        }
-    }
-};
-
 template <typename TI>
 int32_t dispatch_cast_dst(hipStream_t s, int32_t dst, int64_t n, const void *in, void *out) {
     switch (dst) {
@@ -249,12 +179,23 @@ extern "C" int32_t rmlk_hip_unary(rmlk_stream_t stream, int32_t op, int32_t dtyp
     if (n >= kMaxElems) return RMLK_ERR_TOO_LARGE;
     if (op < RMLK_SQRT || op > RMLK_SIGMOID) return RMLK_ERR_INVALID_ARGUMENT;
     if (dtype_size(dtype) == 0) return RMLK_ERR_UNSUPPORTED;
-    hipStream_t s = as_stream(stream);
     bool is_float = dtype == RMLK_FLOAT || dtype == RMLK_DOUBLE;
     bool neg_int = op == RMLK_NEG && (dtype == RMLK_INT32 || dtype == RMLK_INT64);
     if (!is_float && !neg_int) return RMLK_ERR_UNSUPPORTED;
     if (n == 0) return RMLK_OK;
     if (!in || !out) return RMLK_ERR_NULL_POINTER;
+    if (n <= kBatchMaxElems && batch_collecting() && is_float) {
+        // (a tiny map on a stream that is collecting its launches)
+        SmallOp so{};
+        so.kind = kSmallUnary;
+        so.op = op;
+        so.dt = dtype;
+        so.in[0] = in;
+        so.out = out;
+        const int64_t flat[2][kMaxRank] = {{1}, {1}};
+        if (small_op_layout(so, 1, &n, 1, flat) && batch_take(as_stream_collecting(stream), so)) return RMLK_OK;
+    }
+    hipStream_t s = as_stream(stream);
     switch (op) {
         case RMLK_SQRT: return dispatch_float<SqrtF>(s, dtype, n, in, out);
         case RMLK_SIN: return dispatch_float<SinF>(s, dtype, n, in, out);
@@ -275,6 +216,19 @@ extern "C" int32_t rmlk_hip_cast(rmlk_stream_t stream, int32_t src, int32_t dst,
     if (dtype_size(src) == 0 || dtype_size(dst) == 0) return RMLK_ERR_UNSUPPORTED;
     if (n == 0) return RMLK_OK;
     if (!in || !out) return RMLK_ERR_NULL_POINTER;
+    auto collectable = [](int32_t dt) {
+        return dt == RMLK_FLOAT || dt == RMLK_DOUBLE || dt == RMLK_INT32 || dt == RMLK_INT64 || dt == RMLK_BOOL;
+    };
+    if (n <= kBatchMaxElems && batch_collecting() && collectable(src) && collectable(dst)) {
+        SmallOp so{};
+        so.kind = kSmallCast;
+        so.dt = src;
+        so.dt2 = dst;
+        so.in[0] = in;
+        so.out = out;
+        const int64_t flat[2][kMaxRank] = {{1}, {1}};
+        if (small_op_layout(so, 1, &n, 1, flat) && batch_take(as_stream_collecting(stream), so)) return RMLK_OK;
+    }
     hipStream_t s = as_stream(stream);
     switch (src) {
         case RMLK_FLOAT: return dispatch_cast_dst<float>(s, dst, n, in, out);

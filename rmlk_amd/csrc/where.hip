@@ -1,6 +1,7 @@
 // Where: out = cond ? x : y with three-way broadcast. A pure move, so it is instantiated per
 // element size, not per dtype. Replaces cuda/src/ptx/where.cu:4-12
 // (cuda/src/ptx/headers/ternary_op_macro.cuh:1-34).
+#include "batch.hpp"
 #include "elementwise.hpp"
 
 namespace rmlk {
@@ -202,6 +203,18 @@ extern "C" int32_t rmlk_hip_where(rmlk_stream_t stream, int32_t dtype, const rml
         st[2][d] = cond_stride->v[d];
     }
     dense_strides(rank, out_shape->v, st[3]);
+    if (numel <= kBatchMaxElems && batch_collecting() && dtype_size(dtype) != 0) {
+        // (a tiny select on a stream that is collecting its launches)
+        SmallOp so{};
+        so.kind = kSmallWhere;
+        so.dt = dtype_size(dtype);
+        so.in[0] = x;
+        so.in[1] = y;
+        so.in[2] = cond;
+        so.out = out;
+        if (small_op_layout(so, rank, out_shape->v, 3, st) && batch_take(as_stream_collecting(stream), so))
+            return RMLK_OK;
+    }
     hipStream_t s = as_stream(stream);
     switch (dtype_size(dtype)) {
         case 1: return run_where<uint8_t>(s, rank, out_shape->v, st, x, y, cond, out);

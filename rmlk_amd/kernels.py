@@ -421,6 +421,23 @@ def memcpy_dtod_many(dsts, srcs) -> None:
     check(lib().rmlk_hip_memcpy_dtod_many(_stream(), n, d, s_, b), "rmlk_hip_memcpy_dtod_many")
 
 
+class collected_launches:
+    """Context manager: operators over tiny tensors issued inside it on the current stream are
+    collected and run as one launch (rmlk_hip_batch_begin / rmlk_hip_batch_end)."""
+
+    def __enter__(self):
+        self._stream = _stream()
+        check(lib().rmlk_hip_batch_begin(self._stream), "rmlk_hip_batch_begin")
+        return self
+
+    def flush(self) -> None:
+        check(lib().rmlk_hip_batch_flush(self._stream), "rmlk_hip_batch_flush")
+
+    def __exit__(self, *exc):
+        check(lib().rmlk_hip_batch_end(self._stream), "rmlk_hip_batch_end")
+        return False
+
+
 def device_info(device: int = 0) -> dict:
     from ._lib import DeviceInfo
     info = DeviceInfo()

@@ -332,6 +332,45 @@ def test_llama_prefill_and_decode_with_stored_weights(device, storage, style):
     ref.close()
 
 
+def test_rows_that_are_no_whole_units_stay_float(device):
+    """Weights whose K is no multiple of 8 are not stored as 16-bit values (their rows would not be
+    whole 128-bit units): a session over such a graph gives the fp32 session's bits, and a graph
+    that mixes both kinds what the fp32 session gives when only the storable weights are rounded."""
+    from oracle import ops
+    from rmlk_amd import graphs, runtime
+    rng = np.random.default_rng(5)
+    # hidden 60, ffn 100: no MatMul has K % 8 == 0
+    cfg = graphs.LlamaConfig(layers=2, hidden=60, heads=15, kv_heads=3, head_dim=4, ffn=100, vocab=50)
+    graph = graphs.llama_graph(cfg, seed=2, style="concat")
+    feeds = graphs.llama_concat_inputs(cfg, rng.integers(0, cfg.vocab, size=9), None, 0)
+    got = runtime.Builder.from_graph(graph).build(0, weights="bf16").run(feeds)
+    exp = runtime.Builder.from_graph(graph).build(0).run(feeds)
+    for name in exp:
+        assert_exact(got[name], exp[name])
+    # hidden 80 (storable), ffn 100 (the down projection stays float)
+    cfg = graphs.LlamaConfig(layers=1, hidden=80, heads=20, kv_heads=4, head_dim=4, ffn=100, vocab=1000)
+    graph = graphs.llama_graph(cfg, seed=3, style="concat")
+    feeds = graphs.llama_concat_inputs(cfg, rng.integers(0, cfg.vocab, size=130), None, 0)
+    weights = {n.inputs[1] for n in graph.nodes if n.op == "MatMul" and len(n.inputs) == 2}
+    gb = runtime.GraphBuilder()
+    for name, (dt, dims) in graph.inputs.items():
+        gb.input(name, dt, dims)
+    for name, arr in graph.initializers.items():
+        if name in weights and arr.ndim == 2 and arr.shape[0] % 8 == 0:
+            arr = ops.store_weights(arr, "f16")
+        gb.constant(name, arr)
+    for node in graph.nodes:
+        ob = gb.op(node.op, [i or None for i in node.inputs], node.outputs)
+        for key, value in node.attrs.items():
+            ob.attr(key, value)
+    for name in graph.outputs:
+        gb.output(name)
+    got = runtime.Builder.from_graph(graph).build(0, weights="f16").run(feeds)
+    exp = runtime.Builder.from_graph(gb.build()).build(0).run(feeds)
+    for name in exp:
+        assert_exact(got[name], exp[name])
+
+
 def test_both_storage_flags_at_once_are_refused(device):
     from rmlk_amd import graphs, runtime
     from rmlk_amd._lib import lib
