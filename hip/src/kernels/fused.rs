@@ -201,3 +201,34 @@ pub unsafe fn attention(
         "attention",
     )
 }
+
+/// While a value of this type lives, operators over tiny tensors issued on `stream` through this
+/// crate are recorded and go out as one launch, in call order (`rmlk_hip_batch_begin` / `_end`).
+/// Work put on the stream by other means must be preceded by `flush`.
+pub struct CollectedLaunches<'a> {
+    stream: &'a HipStream,
+}
+
+impl<'a> CollectedLaunches<'a> {
+    pub fn begin(stream: &'a HipStream) -> Result<Self> {
+        check(unsafe { ffi::rmlk_hip_batch_begin(stream.raw()) }, "batch_begin")?;
+        Ok(CollectedLaunches { stream })
+    }
+
+    pub fn flush(&self) -> Result<()> {
+        check(unsafe { ffi::rmlk_hip_batch_flush(self.stream.raw()) }, "batch_flush")
+    }
+
+    /// Sends the recorded calls out and reports the status of the launches the batch made.
+    pub fn end(self) -> Result<()> {
+        let status = unsafe { ffi::rmlk_hip_batch_end(self.stream.raw()) };
+        std::mem::forget(self);
+        check(status, "batch_end")
+    }
+}
+
+impl Drop for CollectedLaunches<'_> {
+    fn drop(&mut self) {
+        let _ = unsafe { ffi::rmlk_hip_batch_end(self.stream.raw()) };
+    }
+}
