@@ -96,7 +96,7 @@ def run_llama(args):
     prompt_len, decode_steps = args.prompt, args.decode
     max_len = prompt_len + decode_steps
     t0 = time.perf_counter()
-    graph = graphs.llama_graph(cfg, seed=4, style="scatter", max_len=max_len)
+    graph = graphs.llama_graph(cfg, seed=4, style="scatter", max_len=max_len, bf16_values=args.bf16_values)
     log(f"[bench] graph built in {time.perf_counter() - t0:.1f}s: {len(graph.nodes)} nodes")
     t0 = time.perf_counter()
     torch.cuda.synchronize()
@@ -104,6 +104,8 @@ def run_llama(args):
     inst = runtime.Builder.from_graph(graph).build(0, weights=args.weights)
     torch.cuda.synchronize()
     weights_resident = free_before - torch.cuda.mem_get_info(0)[0]
+    # how the session ended up holding the weights: as asked, or ("auto") 16-bit where nothing is lost
+    stored = args.weights if args.weights in ("f16", "bf16") else ("bf16" if inst.weights_16bit else "f32")
     log(f"[bench] session created (weights uploaded) in {time.perf_counter() - t0:.1f}s, "
         f"{weights_resident / 1e9:.2f} GB of device memory")
 
@@ -174,9 +176,9 @@ def run_llama(args):
             flops = 2.0 * batch * m * n * k
             d["us"] += s["micros"] * flops / node_flops     # a node of several launches: by flops
             d["flops"] += flops
-            w_bytes = 4.0 if args.weights == "f32" else 2.0
+            w_bytes = 4.0 if stored == "f32" else 2.0
             d["alg_bytes"] += batch * (4.0 * m * k + w_bytes * k * n + 4.0 * m * (n // 2 if swiglu else n))
-            pmc = PMC_TRAFFIC_KIB.get(shape) if args.weights == "f32" else None
+            pmc = PMC_TRAFFIC_KIB.get(shape) if stored == "f32" else None
             if pmc is not None and pmc[0] != kind:
                 pmc = None                       # another kernel than the one the counters were read for
             d["traffic"] = None if pmc is None or d["traffic"] is None else d["traffic"] + 1024.0 * sum(pmc[1:])
@@ -193,7 +195,7 @@ def run_llama(args):
     # same counts, weights rotated so that they come from HBM as in the model), issued back to back
     # through the C ABI between ONE pair of HIP events on the stream they run on. (The per-node
     # events above add a cache write-back after every node, ~10 us on a 16 MiB output.)
-    dom_us = time_matmul_launches(kernels, torch, dom["shapes"], storage=args.weights)
+    dom_us = time_matmul_launches(kernels, torch, dom["shapes"], storage=stored)
     achieved = dom["flops"] / dom["launches"] / (dom_us * 1e-6) / 1e12
     roofline = {
         "bound": "mfma",
@@ -255,15 +257,15 @@ def run_llama(args):
             inst.replay()
         inst.sync()
         decode_dev_ms = (time.perf_counter() - t0) / 20 * 1e3
-        weight_bytes = decode_weight_bytes(cfg, args.weights)
+        weight_bytes = decode_weight_bytes(cfg, stored)
         log(f"[bench] decode: {decode_ms:.3f} ms/token end to end, {decode_dev_ms:.3f} ms/token "
             f"device replay ({weight_bytes / decode_dev_ms / 1e6:.0f} GB/s of weights)")
     else:
-        decode_dev_ms, weight_bytes = None, decode_weight_bytes(cfg, args.weights)
+        decode_dev_ms, weight_bytes = None, decode_weight_bytes(cfg, stored)
 
     # ---- CPU baseline: the oracle on a bounded sample -------------------------------------------
     cpu = None
-    if not args.no_cpu and args.weights == "f32":
+    if not args.no_cpu and args.weights in ("f32", "auto"):
         n_cpu = min(args.cpu_tokens, prompt_len)
         cores, blas = cpu_threads()
         cpu_tok_s, cpu_s, cpu_logits = cpu_baseline(graph, cfg, graphs, prompt, n_cpu, max_len)
@@ -292,7 +294,8 @@ def run_llama(args):
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "weight_storage": args.weights,
+        "weight_storage": stored, "weight_storage_asked": args.weights,
+        "weights_are_bfloat16_values": bool(args.bf16_values),
         "config": {"workload": "BASELINE configs[3]: full Llama-3.2-1B-shaped ONNX-op graph, fp32, "
                                f"prefill {prompt_len} tokens + {decode_steps} greedy decode steps, batch 1, "
                                "KV cache updated by ScatterND, random-init weights N(0,0.02)",
@@ -772,10 +775,15 @@ def main():
     ap.add_argument("--decode", type=int, default=128)
     ap.add_argument("--cpu-tokens", type=int, default=512)
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--weights", default="f32", choices=["f32", "f16", "bf16"],
+    ap.add_argument("--weights", default="f32", choices=["f32", "auto", "f16", "bf16"],
                     help="llama suite: how the session stores the constant MatMul weights (arithmetic is "
-                         "fp32 in every case). The reference and the headline figure are f32; with a 16-bit "
-                         "storage the oracle leg is skipped (it walks the unrounded graph)")
+                         "fp32 in every case). The reference and the headline figure are f32; auto: 16-bit "
+                         "where every float of a matrix is a bfloat16 / half value already (nothing lost); "
+                         "f16 / bf16: rounded to that type (the oracle leg is skipped: it walks the "
+                         "unrounded graph)")
+    ap.add_argument("--bf16-values", action="store_true",
+                    help="llama suite: synthetic weights that are bfloat16 values held as floats, as a "
+                         "checkpoint trained in bfloat16 and exported as float has them")
     ap.add_argument("--tiny", action="store_true", help="2-layer toy shape (plumbing check only)")
     ap.add_argument("--suite", default="llama", choices=["llama", "ops", "c1", "c3", "c5"])
     ap.add_argument("--ops-launches", type=int, default=100, help="ops suite: launches per recorded graph")

@@ -400,6 +400,12 @@ int32_t rmlk_hip_attention_few_rows_one_launch(rmlk_stream_t stream, int32_t dty
  * (RMLK_FLOAT16 or RMLK_BFLOAT16; NaN stays NaN, overflow gives infinity). */
 int32_t rmlk_hip_store_weights(rmlk_stream_t stream, int32_t w_dtype, int64_t n, const void *src,
                                void *dst);
+/* Stores 0 to *fits (device memory, set to 1 by the caller beforehand) when one of the n floats at
+ * `src` would come back from `w_dtype` storage with other bits (a NaN never fits); leaves it alone
+ * otherwise. Weights that fit - every checkpoint trained in bfloat16 and exported as float does -
+ * can be held as 16-bit values at no loss. */
+int32_t rmlk_hip_weights_fit(rmlk_stream_t stream, int32_t w_dtype, int64_t n, const void *src,
+                             int32_t *fits);
 
 /* ---- products that share their first operand (q/k/v, gate/up) ----------------------------------
  * The weights of such MatMuls (ref: one cublasGemmStridedBatchedEx each,

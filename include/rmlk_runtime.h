@@ -96,10 +96,18 @@ int32_t rmlk_session_create(const rmlk_graph *g, int32_t device, rmlk_session **
  * ignored with RMLK_SESSION_NO_FUSION. Off by default: the reference computes in fp32 only. */
 #define RMLK_SESSION_WEIGHTS_F16 2u
 #define RMLK_SESSION_WEIGHTS_BF16 4u
+/* Without either of them a session still holds such a weight matrix as 16-bit values when that loses
+ * nothing: when every one of its floats is a bfloat16 (or half) value already, as in a checkpoint
+ * trained in bfloat16 and exported as float. The products then multiply exactly the numbers of the
+ * graph (many-row products bit for bit as over float storage, one-row products with their sums in
+ * another order) from half the bytes. RMLK_SESSION_WEIGHTS_F32 keeps float storage regardless. */
+#define RMLK_SESSION_WEIGHTS_F32 8u
 int32_t rmlk_session_create_ex(const rmlk_graph *g, int32_t device, uint32_t flags,
                                rmlk_session **out);
 /* Number of fused nodes the session formed while it was built. */
 int32_t rmlk_session_fused_nodes(const rmlk_session *s);
+/* Number of constant weight matrices the session holds as 16-bit values. */
+int32_t rmlk_session_weights_16bit(const rmlk_session *s);
 void rmlk_session_destroy(rmlk_session *s);
 
 /* Feed a graph input from host memory (copied to a session-owned device buffer, H2D on the

@@ -1937,22 +1937,52 @@ extern "C" int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_
 namespace {
 // float -> 16-bit storage, round to nearest even
 template <typename WS>
+__device__ __forceinline__ uint16_t round_to_storage(float v) {
+    if constexpr (std::is_same<WS, StoredF16>::value) {
+        return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
+    } else {
+        uint32_t u = __float_as_uint(v);
+        if ((u & 0x7fffffffu) > 0x7f800000u) u = (u >> 16) | 0x40u;            // NaN stays (quiet) NaN
+        else u = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;                        // ties to even
+        return static_cast<uint16_t>(u);
+    }
+}
+
+template <typename WS>
 __global__ __launch_bounds__(kThreads) void store_weights_kernel(const float *__restrict__ src,
                                                                  uint16_t *__restrict__ dst, int64_t n) {
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n;
+         i += static_cast<int64_t>(gridDim.x) * kThreads)
+        dst[i] = round_to_storage<WS>(src[i]);
+}
+
+// *fits = 0 when storing a value would change it (compared as bits: a NaN never fits).
+template <typename WS>
+__global__ __launch_bounds__(kThreads) void weights_fit_kernel(const float *__restrict__ src, int64_t n,
+                                                               int32_t *__restrict__ fits) {
+    bool same = true;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n;
          i += static_cast<int64_t>(gridDim.x) * kThreads) {
         const float v = src[i];
-        if constexpr (std::is_same<WS, StoredF16>::value) {
-            dst[i] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
-        } else {
-            uint32_t u = __float_as_uint(v);
-            if ((u & 0x7fffffffu) > 0x7f800000u) u = (u >> 16) | 0x40u;            // NaN stays (quiet) NaN
-            else u = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;                        // ties to even
-            dst[i] = static_cast<uint16_t>(u);
-        }
+        same = same && __float_as_uint(WS::widen(round_to_storage<WS>(v))) == __float_as_uint(v) && v == v;
     }
+    if (!same) *fits = 0;
 }
 }  // namespace
+
+extern "C" int32_t rmlk_hip_weights_fit(rmlk_stream_t stream, int32_t w_dtype, int64_t n, const void *src,
+                                        int32_t *fits) {
+    if (w_dtype != RMLK_FLOAT16 && w_dtype != RMLK_BFLOAT16) return RMLK_ERR_UNSUPPORTED;
+    if (n < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (n == 0) return RMLK_OK;
+    if (n >= kMaxElems) return RMLK_ERR_TOO_LARGE;
+    if (!src || !fits) return RMLK_ERR_NULL_POINTER;
+    const unsigned grid = grid_for(n, kThreads, 8);
+    const float *ps = static_cast<const float *>(src);
+    if (w_dtype == RMLK_FLOAT16) weights_fit_kernel<StoredF16><<<grid, kThreads, 0, as_stream(stream)>>>(ps, n, fits);
+    else weights_fit_kernel<StoredBF16><<<grid, kThreads, 0, as_stream(stream)>>>(ps, n, fits);
+    return launch_status();
+}
 
 extern "C" int32_t rmlk_hip_store_weights(rmlk_stream_t stream, int32_t w_dtype, int64_t n, const void *src,
                                           void *dst) {

@@ -259,12 +259,18 @@ int32_t rmlk_session_create_ex(const rmlk_graph *g, int32_t device, uint32_t fla
             throw RtError(RMLK_ERR_INVALID_ARGUMENT, "one storage type for the weights at most");
         if (flags & RMLK_SESSION_WEIGHTS_F16) s->impl.weight_storage = RMLK_FLOAT16;
         if (flags & RMLK_SESSION_WEIGHTS_BF16) s->impl.weight_storage = RMLK_BFLOAT16;
+        if (flags & RMLK_SESSION_WEIGHTS_F32) {
+            if (s->impl.weight_storage != RMLK_FLOAT)
+                throw RtError(RMLK_ERR_INVALID_ARGUMENT, "one storage type for the weights at most");
+            s->impl.lossless_16bit = false;
+        }
         s->impl.build(*g, device);
         *out = s.release();
     });
 }
 
 int32_t rmlk_session_fused_nodes(const rmlk_session *s) { return s ? s->impl.fused_nodes : 0; }
+int32_t rmlk_session_weights_16bit(const rmlk_session *s) { return s ? s->impl.weights_16bit : 0; }
 
 void rmlk_session_destroy(rmlk_session *s) {
     if (!s) return;

@@ -294,6 +294,8 @@ struct Session {
     bool profiling = false;
     bool fuse = true;                // form fused nodes while building
     int32_t weight_storage = RMLK_FLOAT;   // how the K-contiguous copies of constant weights are held
+    bool lossless_16bit = true;            // float storage gives way to 16 bits where no value changes
+    int weights_16bit = 0;                 // weight matrices held as 16-bit values
     int fused_nodes = 0;
     int folded_nodes = 0;            // constant nodes evaluated while building
     int64_t device_syncs = 0;            // blocking reads of shape-like tensors

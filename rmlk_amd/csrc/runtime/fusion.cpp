@@ -771,11 +771,33 @@ struct Matcher {
     // The K-contiguous float matrix `tt` as the session holds it: itself, or (a session built with
     // 16-bit weight storage, rows of whole 128-bit units) rounded once to that type, the float form
     // released.
+    // True when every value of the float matrix comes back from `storage` with the bits it has.
+    int32_t *fit_flag = nullptr;   // device
+    ~Matcher() {
+        if (fit_flag) (void)hipFree(fit_flag);
+    }
+    bool fits(const Tensor &tt, int32_t storage) {
+        if (!fit_flag) check_hip(hipMalloc(reinterpret_cast<void **>(&fit_flag), sizeof(int32_t)), "hipMalloc");
+        int32_t one = 1;
+        check_hip(hipMemcpy(fit_flag, &one, sizeof(one), hipMemcpyHostToDevice), "hipMemcpy");
+        check_status(rmlk_hip_weights_fit(s.stream, storage, tt.numel(), tt.data(), fit_flag), "16-bit weights");
+        check_hip(hipStreamSynchronize(s.stream), "hipStreamSynchronize");
+        check_hip(hipMemcpy(&one, fit_flag, sizeof(one), hipMemcpyDeviceToHost), "hipMemcpy");
+        return one != 0;
+    }
     Tensor as_stored(const Tensor &tt) {
         check_hip(hipStreamSynchronize(s.stream), "hipStreamSynchronize");
-        if (s.weight_storage == RMLK_FLOAT || tt.shape[1] % 8 != 0) return tt;
+        if (tt.shape[1] % 8 != 0) return tt;
+        int32_t storage = s.weight_storage;
+        if (storage == RMLK_FLOAT && s.lossless_16bit) {
+            // (bfloat16 first: what checkpoints of this model family are trained and released in)
+            if (fits(tt, RMLK_BFLOAT16)) storage = RMLK_BFLOAT16;
+            else if (fits(tt, RMLK_FLOAT16)) storage = RMLK_FLOAT16;
+        }
+        if (storage == RMLK_FLOAT) return tt;
+        ++s.weights_16bit;
         Tensor st;
-        st.dtype = s.weight_storage;
+        st.dtype = storage;
         st.shape = tt.shape;
         auto buf = std::make_shared<Buffer>();
         buf->bytes = st.nbytes();

@@ -109,9 +109,18 @@ def rmsnorm_matmul_graph(seed=1, seq=128, hidden=2048, n_out=8192):
     return b.g.build(), {"x": x}
 
 
-def _weights(rng, cfg: LlamaConfig, layer: int):
+def as_bfloat16_values(x: np.ndarray) -> np.ndarray:
+    """x (float32) rounded to the nearest bfloat16 value, ties to even, still float32: weights as a
+    checkpoint trained in bfloat16 and exported as float holds them."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    return (u & 0xFFFFFFFF).astype(np.uint32).view(np.float32).reshape(x.shape)
+
+
+def _weights(rng, cfg: LlamaConfig, layer: int, bf16_values: bool = False):
     def w(shape):
-        return rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02)
+        x = rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02)
+        return as_bfloat16_values(x) if bf16_values else x
     h, kvd = cfg.hidden, cfg.kv_heads * cfg.head_dim
     return {
         "ln1": np.ones((h,), np.float32), "ln2": np.ones((h,), np.float32),
@@ -259,7 +268,7 @@ def decoder_layer_graph(seed=3, seq=2048, cfg: LlamaConfig | None = None):
     return b.g.build(), {"x": x}
 
 
-def llama_graph(cfg: LlamaConfig | None = None, seed=4, style="scatter", max_len=640):
+def llama_graph(cfg: LlamaConfig | None = None, seed=4, style="scatter", max_len=640, bf16_values=False):
     """Config 4: the full Llama-shaped graph (tied embedding: Gather on `embed`, final MatMul with
     the same values laid out [hidden, vocab]). Returns the Graph; inputs are built by the callers
     (llama_inputs_*)."""
@@ -267,6 +276,8 @@ def llama_graph(cfg: LlamaConfig | None = None, seed=4, style="scatter", max_len
     rng = np.random.default_rng(seed)
     b = _B()
     embed = rng.standard_normal((cfg.vocab, cfg.hidden), dtype=np.float32) * np.float32(0.02)
+    if bf16_values:     # every weight a bfloat16 value held as float (see as_bfloat16_values)
+        embed = as_bfloat16_values(embed)
     embed_n = b.const(embed, "embed")
     lm_head_n = b.const(np.ascontiguousarray(embed.T), "lm_head")
     del embed
@@ -309,7 +320,7 @@ def llama_graph(cfg: LlamaConfig | None = None, seed=4, style="scatter", max_len
 
     outputs = []
     for l in range(cfg.layers):
-        wn = _layer_consts(b, _weights(rng, cfg, l), l)
+        wn = _layer_consts(b, _weights(rng, cfg, l, bf16_values), l)
         if style == "concat":
             def kv_update(k, v, l=l):
                 k_all = b.op("Concat", [f"past_key_values.{l}.key", k], out=f"present.{l}.key", axis=2)

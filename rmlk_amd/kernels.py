@@ -59,6 +59,14 @@ def store_weights(w: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
+def weights_fit(w: torch.Tensor, dtype: torch.dtype) -> bool:
+    """True when every value of the float tensor w survives storage as torch.float16 / torch.bfloat16."""
+    flag = torch.ones(1, dtype=torch.int32, device=w.device)
+    wd = BFLOAT16 if dtype == torch.bfloat16 else TORCH_TO_DTYPE[dtype]
+    check(lib().rmlk_hip_weights_fit(_stream(), wd, w.numel(), _ptr(w), _ptr(flag)), "rmlk_hip_weights_fit")
+    return bool(flag.item())
+
+
 def binary(op: int, a, b, out, out_shape, a_stride, b_stride) -> None:
     """ref: cuda/src/kernels/binary.rs:58-100 (compute_with_types). Strides are per output dim,
     0 on broadcast dims."""

@@ -179,13 +179,18 @@ class GraphBuilder:
 class ModelInstance:
     """ref: runtime/src/core/instance.rs:20-119"""
 
-    def __init__(self, graph: Graph, device: int = 0, fuse: bool = True, weights: str = "f32"):
+    def __init__(self, graph: Graph, device: int = 0, fuse: bool = True, weights: str = "auto"):
         self.graph = graph
         h = ctypes.c_void_p()
-        flags = (0 if fuse else 1) | {"f32": 0, "f16": 2, "bf16": 4}[weights]
+        flags = (0 if fuse else 1) | {"auto": 0, "f16": 2, "bf16": 4, "f32": 8}[weights]
         _check(lib().rmlk_session_create_ex(graph.handle, device, flags, ctypes.byref(h)),
                "Builder.build")
         self._h = h
+
+    @property
+    def weights_16bit(self) -> int:
+        """Constant weight matrices the session holds as 16-bit values."""
+        return int(lib().rmlk_session_weights_16bit(self._h))
 
     @property
     def fused_nodes(self) -> int:
@@ -310,8 +315,10 @@ class Builder:
         from .onnx_io import load_onnx_bytes
         return Builder(load_onnx_bytes(data, base_dir))
 
-    def build(self, device: int = 0, fuse: bool = True, weights: str = "f32") -> ModelInstance:
-        """fuse=False keeps one kernel per node, as the reference executes a graph. weights="f16" or
-        "bf16": the constant weights of fused MatMuls are stored rounded to that type (half the bytes
-        to stream per token); the arithmetic stays fp32."""
+    def build(self, device: int = 0, fuse: bool = True, weights: str = "auto") -> ModelInstance:
+        """fuse=False keeps one kernel per node, as the reference executes a graph. weights: how the
+        constant weights of fused MatMuls are stored (the arithmetic is fp32 in every case): "auto"
+        as floats, or as 16-bit values where every float of a matrix is a bfloat16 / half value
+        already (nothing is lost); "f32" as floats regardless; "f16" / "bf16" rounded to that type
+        (half the bytes to stream per token)."""
         return ModelInstance(self._graph, device, fuse, weights)

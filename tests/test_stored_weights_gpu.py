@@ -271,13 +271,13 @@ def test_decoder_layer_with_stored_weights_equals_fp32_over_rounded_weights(devi
     graph, feeds = graphs.decoder_layer_graph(seed=3, seq=256)
     rounded = _with_rounded_weights(graph, storage)
     inst = runtime.Builder.from_graph(graph).build(0, weights=storage)
-    ref = runtime.Builder.from_graph(rounded).build(0)
+    ref = runtime.Builder.from_graph(rounded).build(0, weights="f32")
     assert inst.fused_nodes == ref.fused_nodes > 0
     got, exp = inst.run(feeds), ref.run(feeds)
     for name in exp:
         assert_exact(got[name], exp[name])
     # and the fp32 session on the ORIGINAL weights is a different (nearby) result: the storage is on
-    full = runtime.Builder.from_graph(graph).build(0).run(feeds)
+    full = runtime.Builder.from_graph(graph).build(0, weights="f32").run(feeds)
     first = next(iter(exp))
     assert not np.array_equal(full[first], got[first])
     oracle = og.run_graph(rounded, feeds)
@@ -300,7 +300,7 @@ def test_llama_prefill_and_decode_with_stored_weights(device, storage, style):
     graph = graphs.llama_graph(cfg, seed=4, style=style, max_len=max_len)
     rounded = _with_rounded_weights(graph, storage)
     inst = runtime.Builder.from_graph(graph).build(0, weights=storage)
-    ref = runtime.Builder.from_graph(rounded).build(0)
+    ref = runtime.Builder.from_graph(rounded).build(0, weights="f32")
     rng = np.random.default_rng(1)
     prompt = rng.integers(0, cfg.vocab, size=12)
 
@@ -366,9 +366,76 @@ def test_rows_that_are_no_whole_units_stay_float(device):
     for name in graph.outputs:
         gb.output(name)
     got = runtime.Builder.from_graph(graph).build(0, weights="f16").run(feeds)
-    exp = runtime.Builder.from_graph(gb.build()).build(0).run(feeds)
+    exp = runtime.Builder.from_graph(gb.build()).build(0, weights="f32").run(feeds)
     for name in exp:
         assert_exact(got[name], exp[name])
+
+
+def test_weights_fit_tells_what_storage_would_change(device):
+    import torch
+    from oracle import ops
+    kk = _k()
+    rng = np.random.default_rng(8)
+    w = (rng.standard_normal(100000) * 0.02).astype(np.float32)
+    for storage, other in (("bf16", "f16"), ("f16", "bf16")):
+        fitting = to_dev(ops.store_weights(w, storage), device)
+        assert kk.weights_fit(fitting, _torch_dtype(storage))
+        assert not kk.weights_fit(fitting, _torch_dtype(other))        # 8 against 11 significant bits, other ranges
+        spoiled = fitting.clone()
+        spoiled[77777] = float(np.nextafter(np.float32(0.02), np.float32(1)))
+        assert not kk.weights_fit(spoiled, _torch_dtype(storage))
+    assert not kk.weights_fit(to_dev(w, device), torch.bfloat16)
+    special = to_dev(np.array([0.0, -0.0, np.inf, -np.inf, 1.0, -2.5], dtype=np.float32), device)
+    assert kk.weights_fit(special, torch.bfloat16) and kk.weights_fit(special, torch.float16)
+    assert not kk.weights_fit(to_dev(np.array([1.0, np.nan], dtype=np.float32), device), torch.bfloat16)
+    assert kk.weights_fit(torch.empty(0, device=device), torch.float16)
+
+
+@pytest.mark.parametrize("style", ["scatter", "concat"])
+def test_weights_that_are_bfloat16_values_are_held_as_such(device, style):
+    """A graph whose float weights are bfloat16 values already (a checkpoint trained in bfloat16): the
+    session stores them in 16 bits without being asked, since nothing is lost. Against the session
+    that keeps floats: the prefill (tiled products) bit for bit, decode steps to rounding, same
+    tokens. Ordinary float weights stay floats."""
+    from rmlk_amd import graphs, runtime
+    cfg = graphs.LlamaConfig.tiny()
+    max_len = 32
+    graph = graphs.llama_graph(cfg, seed=4, style=style, max_len=max_len, bf16_values=True)
+    auto = runtime.Builder.from_graph(graph).build(0)
+    floats = runtime.Builder.from_graph(graph).build(0, weights="f32")
+    assert auto.weights_16bit == 4 * cfg.layers + 1     # joint q/k/v, joint gate/up, o, down per layer; the lm-head
+    assert floats.weights_16bit == 0
+    plain = runtime.Builder.from_graph(graphs.llama_graph(cfg, seed=4, style=style, max_len=max_len)).build(0)
+    assert plain.weights_16bit == 0
+    plain.close()
+    rng = np.random.default_rng(2)
+    ids, past_len, outs = rng.integers(0, cfg.vocab, size=12), 0, {"auto": None, "floats": None}
+
+    def feeds_for(ids, past, past_len):
+        if style == "concat":
+            return graphs.llama_concat_inputs(cfg, ids, past, past_len)
+        f = {"input_ids": ids.reshape(1, -1).astype(np.int64),
+             "position_ids": np.arange(past_len, past_len + ids.size, dtype=np.int64).reshape(1, -1)}
+        for l in range(cfg.layers):
+            for kv in ("key", "value"):
+                f[f"cache.{l}.{kv}"] = (past[f"cache_out.{l}.{kv}"] if past is not None else
+                                        np.zeros((1, cfg.kv_heads, max_len, cfg.head_dim), np.float32))
+        return f
+
+    for step in range(4):
+        outs["auto"] = auto.run(feeds_for(ids, outs["auto"], past_len))
+        outs["floats"] = floats.run(feeds_for(ids, outs["floats"], past_len))
+        got, exp = outs["auto"]["logits"], outs["floats"]["logits"]
+        if step == 0:
+            assert_exact(got, exp)
+        else:
+            assert_close(got, exp, rtol=1e-4, atol=1e-5)
+        tok = int(np.argmax(got[0, -1]))
+        assert tok == int(np.argmax(exp[0, -1]))
+        past_len += ids.size
+        ids = np.array([tok])
+    auto.close()
+    floats.close()
 
 
 def test_both_storage_flags_at_once_are_refused(device):
@@ -376,5 +443,6 @@ def test_both_storage_flags_at_once_are_refused(device):
     from rmlk_amd._lib import lib
     graph = graphs.llama_graph(graphs.LlamaConfig.tiny(), seed=4, style="scatter", max_len=16)
     h = ctypes.c_void_p()
-    assert lib().rmlk_session_create_ex(graph.handle, 0, 2 | 4, ctypes.byref(h)) != 0
-    assert not h
+    for flags in (2 | 4, 2 | 8, 4 | 8):
+        assert lib().rmlk_session_create_ex(graph.handle, 0, flags, ctypes.byref(h)) != 0
+        assert not h
