@@ -16,6 +16,10 @@
 //     global memory straight into LDS (global_load_lds_dwordx4), see gemm_mfma_direct_kernel;
 //   - split-K (grid z) writes partial tiles to the workspace, a second kernel adds them in a
 //     fixed order, so results do not depend on scheduling.
+//   - a K-contiguous B of constant weights may be STORED as IEEE half or bfloat16 values (StoredF16,
+//     StoredBF16): they are widened exactly and everything is computed in fp32 as before, from half
+//     the bytes. The tiled kernels widen on the way into LDS (same MFMAs, same bits as over the
+//     widened weights), the one-row kernels in registers.
 #include <atomic>
 #include <cstdio>
 #include <cstring>
