@@ -690,6 +690,7 @@ namespace {
 // lie inside one head, and the chunks must fit the kernel's two 64-bit sets.
 struct TileMapDims {
     int64_t mask_batches, mask_heads, tiles, chunks;
+    int keys;   // keys of a chunk: what the kernel that will run takes per step
     size_t map_bytes, bytes;
 };
 TileMapDims tile_map_dims(int64_t batch, int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
@@ -699,8 +700,13 @@ TileMapDims tile_map_dims(int64_t batch, int64_t kv_heads, int64_t rep, int64_t 
         mask_stride->rank != 4)
         return d;
     const int64_t blocks = (rep * q_len + 63) / 64 * batch * kv_heads;
-    d.chunks = (kv_len + 63) / 64;
-    if (blocks <= kNumCU || q_len % 64 != 0 || d.chunks < 4 || d.chunks > 128) return d;
+    // More blocks than compute units: the kernel with 64-key steps, its items handed out from a
+    // counter. Otherwise the kernel with 128-key steps and one block per tile, which keeps its tile and
+    // only skips the chunks it cannot see: that pays where a prompt is much shorter than its cache.
+    const bool many_blocks = blocks > kNumCU;
+    d.keys = many_blocks ? AttnShape<2>::kKeys : AttnShape<4>::kKeys;
+    d.chunks = (kv_len + d.keys - 1) / d.keys;
+    if (q_len % 64 != 0 || d.chunks < (many_blocks ? 4 : 6) || d.chunks > 128) return d;
     d.mask_batches = mask_stride->v[0] ? batch : 1;
     d.mask_heads = mask_stride->v[1] ? kv_heads * rep : 1;
     d.tiles = q_len / 64;
@@ -730,26 +736,37 @@ extern "C" int32_t rmlk_hip_attention_ws(rmlk_stream_t stream, int32_t dtype, in
                                       mask_stride, scale_is_mul, scale, out_seq_major, out, true, &g, &empty);
     if (st || empty) return st;
     dim3 grid(static_cast<unsigned>((g.rows + 63) / 64), static_cast<unsigned>(batch * kv_heads), 1);
-    // two blocks of four wavefronts per CU when there are that many, else one block of eight
-    if (static_cast<int64_t>(grid.x) * grid.y > kNumCU) {
+    const bool many_blocks = static_cast<int64_t>(grid.x) * grid.y > kNumCU;
+    {
         const TileMapDims tm = tile_map_dims(batch, kv_heads, rep, q_len, kv_len, mask_stride);
         if (workspace && tm.bytes && workspace_bytes >= tm.bytes && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
             uint8_t *tiles = static_cast<uint8_t *>(workspace);
             const dim3 tgrid(static_cast<unsigned>(tm.chunks), static_cast<unsigned>(tm.tiles),
                              static_cast<unsigned>(tm.mask_batches * tm.mask_heads));
-            attention_mask_tiles_kernel<64><<<tgrid, 256, 0, as_stream(stream)>>>(
-                g.mask, g.mask_b, g.mask_h, g.mask_s, static_cast<int32_t>(tm.mask_heads), g.seq, g.len, tiles,
-                reinterpret_cast<int32_t *>(tiles + tm.map_bytes));
+            if (tm.keys == 64)
+                attention_mask_tiles_kernel<64><<<tgrid, 256, 0, as_stream(stream)>>>(
+                    g.mask, g.mask_b, g.mask_h, g.mask_s, static_cast<int32_t>(tm.mask_heads), g.seq, g.len, tiles,
+                    reinterpret_cast<int32_t *>(tiles + tm.map_bytes));
+            else
+                attention_mask_tiles_kernel<128><<<tgrid, 256, 0, as_stream(stream)>>>(
+                    g.mask, g.mask_b, g.mask_h, g.mask_s, static_cast<int32_t>(tm.mask_heads), g.seq, g.len, tiles,
+                    reinterpret_cast<int32_t *>(tiles + tm.map_bytes));
             const int32_t launched = launch_status();
             if (launched) return launched;
             g.tiles = tiles;
             g.tiles_h = mask_stride->v[1] ? tm.tiles * tm.chunks : 0;
             g.tiles_b = mask_stride->v[0] ? tm.mask_heads * tm.tiles * tm.chunks : 0;
-            g.queue = reinterpret_cast<int32_t *>(tiles + tm.map_bytes);
-            g.items = static_cast<int32_t>(static_cast<int64_t>(grid.x) * grid.y);
-            g.tiles_per_head = static_cast<int32_t>(tm.tiles);
-            grid = dim3(static_cast<unsigned>(std::min<int64_t>(g.items, 2 * kNumCU)), 1, 1);
+            if (many_blocks) {
+                // (tile, KV head) items handed to a resident grid from a counter, longest first
+                g.queue = reinterpret_cast<int32_t *>(tiles + tm.map_bytes);
+                g.items = static_cast<int32_t>(static_cast<int64_t>(grid.x) * grid.y);
+                g.tiles_per_head = static_cast<int32_t>(tm.tiles);
+                grid = dim3(static_cast<unsigned>(std::min<int64_t>(g.items, 2 * kNumCU)), 1, 1);
+            }
         }
+    }
+    // two blocks of four wavefronts per CU when there are that many, else one block of eight
+    if (many_blocks) {
         static DynamicLdsGrant grant;
         const int32_t granted = grant.ensure(attention_rows_kernel<2>, AttnShape<2>::kLdsBytes);
         if (granted) return granted;

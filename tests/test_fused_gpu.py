@@ -1171,7 +1171,11 @@ def _skipping_mask(kind, rng, mask_shape, l):
     (1, 8, 4, 1024, 1024, (1, 32, 1024, 1024), "tiles", True),    # per head only
     (2, 8, 4, 512, 1024, (2, 1, 512, 1024), "tiles", True),       # per batch only
     (1, 8, 4, 2048, 704, (1, 1, 1, 704), "row", True),            # one mask row for every query
-    (1, 8, 4, 512, 640, (1, 1, 512, 640), "causal", False),       # too few blocks: the 8-wavefront kernel
+    (1, 8, 4, 512, 640, (1, 1, 512, 640), "causal", False),       # a block per compute unit and five chunks of 128
+    (1, 8, 4, 512, 2048, (1, 1, 512, 2048), "causal", True),      # the same prompt in a longer cache: 16 chunks
+    (1, 8, 4, 512, 2000, (1, 1, 1, 2000), "row", True),           # keys end inside a chunk of 128
+    (2, 2, 2, 256, 1024, (2, 4, 256, 1024), "tiles", True),       # a few blocks, per batch and head
+    (1, 1, 1, 192, 900, (1, 1, 192, 900), "window", True),        # three blocks
     (1, 8, 4, 2000, 2048, (1, 1, 2000, 2048), "causal", False),   # tiles would straddle heads
     (1, 8, 4, 2048, 128, (1, 1, 2048, 128), "causal", False),     # two chunks: nothing to gain
 ])
@@ -1196,7 +1200,9 @@ def test_attention_skipping_hidden_chunks_is_bit_identical(device, b, g, rep, s,
         assert (need > 0) == skips
         if skips:
             mb, mh = mask_shape[0], mask_shape[1]
-            assert need == (mb * mh * (s // 64) * ((l + 63) // 64) + 15) // 16 * 16 + 16   # the map and a counter
+            # chunks of 64 keys for the kernel that has more blocks than compute units, of 128 otherwise
+            keys = 64 if b * g * (rep * s // 64) > 256 else 128
+            assert need == (mb * mh * (s // 64) * ((l + keys - 1) // keys) + 15) // 16 * 16 + 16   # the map and a counter
         a, e = to_np(got), to_np(plain)
         assert np.array_equal(np.isnan(a), np.isnan(e))
         assert_exact(np.nan_to_num(a, nan=0.0), np.nan_to_num(e, nan=0.0))
