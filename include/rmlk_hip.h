@@ -338,12 +338,12 @@ int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch, i
                            int32_t out_seq_major, void *out);
 /* The same kernel with room to skip what the mask hides: with `workspace` of at least
  * rmlk_hip_attention_workspace_size() bytes a small kernel first marks, per tile of 64 queries and
- * chunk of 64 keys, whether the mask holds anything but -inf there, and the main kernel neither loads
+ * chunk of 64 keys (of 128 where the launch has no more blocks than compute units), whether the mask holds anything but -inf there, and the main kernel neither loads
  * nor multiplies the chunks a tile cannot see (a causal mask: about half of them). Their probabilities
  * are exact zeros, so results are those of rmlk_hip_attention bit for bit, with two exceptions: a NaN
  * or infinity in a K or V row no query of the tile can see does not reach that tile's output
  * (0 * NaN would), and a row with nothing visible anywhere is NaN as before. The size is 0 (and a
- * null workspace allowed) where skipping does not apply: few blocks, q_len not a multiple of 64, or
+ * null workspace allowed) where skipping does not apply: q_len not a multiple of 64, fewer than 4 chunks (6 of 128), or
  * more than 128 chunks. The workspace is 16-byte aligned (one that is not, or is too small, is
  * ignored: every chunk is then visited) and belongs to the call until its kernels have run. rmlk_hip_attention is this call with a null workspace. */
 size_t rmlk_hip_attention_workspace_size(int32_t dtype, int64_t batch, int64_t kv_heads, int64_t rep,
