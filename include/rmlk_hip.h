@@ -548,7 +548,7 @@ int32_t rmlk_hip_gemv_kmajor_head_rows(rmlk_stream_t stream, int32_t dtype, int6
 /* ---- launches over tiny tensors collected into one ------------------------------------------------
  * Between rmlk_hip_batch_begin and rmlk_hip_batch_end on a stream, calls of rmlk_hip_binary (not
  * Pow), rmlk_hip_unary, rmlk_hip_cast, rmlk_hip_where, rmlk_hip_expand and rmlk_hip_concat_many whose
- * output has at most 4096 elements (FLOAT, DOUBLE, INT32, INT64, BOOL operands; any element size for
+ * output has at most 1024 elements (FLOAT, DOUBLE, INT32, INT64, BOOL operands; any element size for
  * the moves) do not launch: they are recorded, and one single-block launch runs up to 24 records in
  * order with the element arithmetic of the kernels they replace (same bits). Every other call of
  * this library on the stream, rmlk_hip_batch_flush and rmlk_hip_batch_end send the recorded calls

@@ -54,7 +54,7 @@ public:
     // collected operators that have nothing to do with each other look dependent (one overwrites
     // what the other read), and they could not run side by side.
     bool hold_small = false;
-    static constexpr size_t kSmallBytes = 32 * 1024;   // the largest output a collected operator has
+    static constexpr size_t kSmallBytes = 8 * 1024;   // the largest output a collected operator has
     void let_go();
 
 private:

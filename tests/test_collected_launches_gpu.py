@@ -30,8 +30,8 @@ SHAPES = [
     ((1,), (7,)),                        # scalar against a row
     ((2, 3, 4, 5, 1, 2), (2, 3, 4, 5, 1, 2)),   # six dims that merge into one
     ((2, 1, 3, 1, 2, 1, 3), (1, 2, 1, 3, 1, 2, 1)),   # seven dims that do not merge: the operator's own kernel
-    ((64, 64), (64, 1)),                 # 4096 elements: the largest collected
-    ((65, 64), (1, 64)),                 # one row more: not collected
+    ((16, 64), (16, 1)),                 # 1024 elements: the largest collected
+    ((17, 64), (1, 64)),                 # one row more: not collected
 ]
 
 
