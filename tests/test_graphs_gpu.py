@@ -195,8 +195,13 @@ def test_llama_tiny_scatter_style_equals_concat_style(device):
 
 
 @pytest.mark.timeout(900)
-def test_llama_1b_full_size_prefill_and_teacher_forced_decode(device):
-    """BASELINE configs[3] at its full size: 16 layers, hidden 2048, vocab 128256. Prefill of a
+@pytest.mark.parametrize("bf16_values", [False, True])
+def test_llama_1b_full_size_prefill_and_teacher_forced_decode(device, bf16_values):
+    """(bf16_values: the same graph with weights that are bfloat16 values held as floats, which the
+    session stores in 16 bits by itself: the products over stored weights at the full widths -
+    lm-head over 128256 rows, gate / up / down at 8192 - against the oracle on the same graph.)
+
+    BASELINE configs[3] at its full size: 16 layers, hidden 2048, vocab 128256. Prefill of a
     512-token prompt, then 8 decode steps through the recorded HIP graph with the caches fed back on
     the device, each step teacher-forced with the oracle's token and held to the reference's bar for
     whole-model runs (logits atol = rtol = 1e-2, identical argmax: runtime/tests/e2e_ort/llama.rs:112-156,
@@ -207,12 +212,13 @@ def test_llama_1b_full_size_prefill_and_teacher_forced_decode(device):
     cfg = graphs.LlamaConfig()
     prompt_len, steps = 512, 8
     max_len = prompt_len + steps
-    graph = graphs.llama_graph(cfg, seed=4, style="scatter", max_len=max_len)
+    graph = graphs.llama_graph(cfg, seed=4, style="scatter", max_len=max_len, bf16_values=bf16_values)
     rng = np.random.default_rng(4)
     prompt = rng.integers(0, cfg.vocab, size=prompt_len)
     zeros = {f"cache.{l}.{kv}": np.zeros((1, cfg.kv_heads, max_len, cfg.head_dim), np.float32)
              for l in range(cfg.layers) for kv in ("key", "value")}
     inst = runtime.Builder.from_graph(graph).build()
+    assert inst.weights_16bit == (4 * cfg.layers + 1 if bf16_values else 0)
     feeds = _scatter_feeds(cfg, prompt, 0, zeros)
     for name, arr in feeds.items():
         inst.set_input(name, arr)
