@@ -101,7 +101,7 @@ def run_llama(args):
     t0 = time.perf_counter()
     torch.cuda.synchronize()
     free_before = torch.cuda.mem_get_info(0)[0]
-    inst = runtime.Builder.from_graph(graph).build(0, weights=args.weights)
+    inst = runtime.Builder.from_graph(graph).build(0, weights=args.weights, bf16_pieces=args.bf16_pieces)
     torch.cuda.synchronize()
     weights_resident = free_before - torch.cuda.mem_get_info(0)[0]
     # how the session ended up holding the weights: as asked, or ("auto") 16-bit where nothing is lost
@@ -132,6 +132,7 @@ def run_llama(args):
     feed_prefill()
     inst.execute()                       # first run: fills the buffer pool
     first_logits = inst.output("logits")[0, -1].copy()
+    prefill_products_bf16 = inst.products_bf16_pieces
     inst.capture()
     for _ in range(args.warmup):
         inst.replay()
@@ -296,6 +297,7 @@ def run_llama(args):
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "weight_storage": stored, "weight_storage_asked": args.weights,
         "weights_are_bfloat16_values": bool(args.bf16_values),
+        "prefill_products_on_bf16_matrix_cores": prefill_products_bf16,
         "config": {"workload": "BASELINE configs[3]: full Llama-3.2-1B-shaped ONNX-op graph, fp32, "
                                f"prefill {prompt_len} tokens + {decode_steps} greedy decode steps, batch 1, "
                                "KV cache updated by ScatterND, random-init weights N(0,0.02)",
@@ -786,6 +788,10 @@ def main():
     ap.add_argument("--bf16-values", action="store_true",
                     help="llama suite: synthetic weights that are bfloat16 values held as floats, as a "
                          "checkpoint trained in bfloat16 and exported as float has them")
+    ap.add_argument("--bf16-pieces", action="store_true",
+                    help="llama suite: many-row products over weights held as bfloat16 values split their "
+                         "fp32 operand into three bfloat16 pieces (exactly) and run on the bf16 matrix cores "
+                         "(fp32 results; needs --bf16-values with --weights auto, or --weights bf16)")
     ap.add_argument("--tiny", action="store_true", help="2-layer toy shape (plumbing check only)")
     ap.add_argument("--suite", default="llama", choices=["llama", "ops", "c1", "c3", "c5"])
     ap.add_argument("--ops-launches", type=int, default=100, help="ops suite: launches per recorded graph")
@@ -832,6 +838,14 @@ def main():
             "decode_device_ms_per_token": r["decode_device_ms_per_token"],
             "decode_weight_gbs": r["decode_weight_gbs"],
             "session_device_bytes_after_build": r["memory"]["session_device_bytes_after_build"]}
+        # ... and with the prefill's products on the bf16 matrix cores: the fp32 operand as three
+        # bfloat16 pieces whose sum it is exactly, exact products, fp32 accumulation
+        v.bf16_pieces = True
+        r = run_llama(v)
+        result["variant_bf16_valued_weights"]["prefill_tok_s_products_as_bf16_pieces"] = r["value"]
+        result["variant_bf16_valued_weights"]["prefill_ms_products_as_bf16_pieces"] = r["ms_per_step"]
+        result["variant_bf16_valued_weights"]["prefill_products_on_bf16_matrix_cores"] = \
+            r["prefill_products_on_bf16_matrix_cores"]
     print(json.dumps(result))
 
 

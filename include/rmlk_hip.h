@@ -482,6 +482,39 @@ int32_t rmlk_hip_splitk_add_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t
                                     const void *b, const void *gamma, float eps,
                                     int32_t reciprocal_form, void *sum_out, void *out);
 
+/* ---- many-row products over bfloat16 weights on the bf16 matrix cores ----------------------------
+ * c[m, n] = a[m, k] . wt[n, k]^T with a fp32, wt bfloat16 values (K-contiguous, as
+ * rmlk_hip_store_weights writes them) and fp32 results, multiplied by v_mfma_f32_32x32x16_bf16
+ * without rounding a: a float is the exact sum of three bfloat16 pieces (8 + 8 + 8 significant
+ * bits), a product of two bfloat16 values is exact in fp32, so three MFMAs per tile and K chunk
+ * over the three pieces add up exactly the products a[i, k] * wt[j, k] - what remains is the
+ * rounding of fp32 accumulation, as in any fp32 product with its sums in another order. About 2.5x
+ * the rate of the fp32 MFMA kernels. No counterpart in the reference (fp32 cuBLAS,
+ * cuda/src/kernels/gemm.rs:191-232).
+ *
+ * rmlk_hip_bf16x3_split writes the pieces of a as three planes [3][m_pad][k] of bfloat16 (m_pad = m
+ * rounded up to a multiple of 128, the padding rows zero) into `pieces`, which must hold
+ * rmlk_hip_bf16x3_pieces_size(m, k) bytes; k % 8 == 0, lda % 4 == 0, 16-byte aligned pointers.
+ * Infinities and NaNs of a arrive in the result as they would from an fp32 product.
+ * rmlk_hip_matmul_bf16x3 multiplies the pieces by wt: with splits == 1 into c (leading dimension
+ * ldc); with splits > 1 slab s of K (k / splits values) goes to c + s * slab elements, for a reader
+ * that adds the slabs up itself (rmlk_hip_splitk_add_rmsnorm, rmlk_hip_head_rows).
+ * rmlk_hip_bf16x3_splits is the number of slabs that fills the GPU for a size (1 for wide products;
+ * 0 for sizes the kernel does not take). rmlk_hip_matmul_bf16x3_swiglu is rmlk_hip_matmul_swiglu over
+ * the pieces: out[m, n] = swiglu(a . wt[gate_row .. +n]^T, a . wt[up_row .. +n]^T).
+ * Covered: k % 32 == 0 (per slab), n % 128 == 0 (swiglu: n % 64 == 0), ldw % 8 == 0, operands below
+ * 4 GiB; RMLK_ERR_UNSUPPORTED otherwise. */
+size_t rmlk_hip_bf16x3_pieces_size(int64_t m, int64_t k);
+int32_t rmlk_hip_bf16x3_split(rmlk_stream_t stream, int64_t m, int64_t k, const void *a, int64_t lda,
+                              void *pieces);
+int32_t rmlk_hip_bf16x3_splits(int64_t m, int64_t n, int64_t k);
+int32_t rmlk_hip_matmul_bf16x3(rmlk_stream_t stream, int64_t m, int64_t n, int64_t k, const void *pieces,
+                               const void *wt, int64_t ldw, int32_t splits, void *c, int64_t ldc,
+                               int64_t slab);
+int32_t rmlk_hip_matmul_bf16x3_swiglu(rmlk_stream_t stream, int64_t m, int64_t n, int64_t k,
+                                      const void *pieces, const void *wt, int64_t ldw, int64_t gate_row,
+                                      int64_t up_row, void *out, int64_t ldc);
+
 /* Rotary position embedding, half-rotation form, over x of logical shape [B, H, S, D]:
  * out = x * cos + concat(-x[..., D/2:], x[..., :D/2]) * sin, out dense [B, H, S, D].
  * x, cos and sin are read through element strides per dim of `shape` (innermost stride 1; 0 on

@@ -102,8 +102,18 @@ int32_t rmlk_session_create(const rmlk_graph *g, int32_t device, rmlk_session **
  * graph (many-row products bit for bit as over float storage, one-row products with their sums in
  * another order) from half the bytes. RMLK_SESSION_WEIGHTS_F32 keeps float storage regardless. */
 #define RMLK_SESSION_WEIGHTS_F32 8u
+/* Products of many rows (64 and more) over weight matrices held as bfloat16 values run on the bf16
+ * matrix cores: the fp32 first operand is split into three bfloat16 pieces whose sum it is exactly,
+ * every product of a piece and a weight is exact in fp32, accumulation is fp32
+ * (rmlk_hip_matmul_bf16x3). The results are fp32 products with their sums in another order - not
+ * the bits of the fp32 MFMA kernels - at about 2.5x their rate. Concerns prefill over checkpoints
+ * whose floats are bfloat16 values (stored in 16 bits without loss by default) or over
+ * RMLK_SESSION_WEIGHTS_BF16; one-row products (decode) are unchanged. Off by default. */
+#define RMLK_SESSION_BF16_PIECES 16u
 int32_t rmlk_session_create_ex(const rmlk_graph *g, int32_t device, uint32_t flags,
                                rmlk_session **out);
+/* Number of products the session's last run multiplied that way. */
+int32_t rmlk_session_products_bf16_pieces(const rmlk_session *s);
 /* Number of fused nodes the session formed while it was built. */
 int32_t rmlk_session_fused_nodes(const rmlk_session *s);
 /* Number of constant weight matrices the session holds as 16-bit values. */

@@ -117,6 +117,13 @@ SIGNATURES = {
     "rmlk_hip_splitk_add_rmsnorm": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int32,
                                               c_int64, c_void_p, c_void_p, ctypes.c_float, c_int32,
                                               c_void_p, c_void_p]),
+    "rmlk_hip_bf16x3_pieces_size": (c_size_t, [c_int64, c_int64]),
+    "rmlk_hip_bf16x3_split": (c_int32, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p]),
+    "rmlk_hip_bf16x3_splits": (c_int32, [c_int64, c_int64, c_int64]),
+    "rmlk_hip_matmul_bf16x3": (c_int32, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int64,
+                                         c_int32, c_void_p, c_int64, c_int64]),
+    "rmlk_hip_matmul_bf16x3_swiglu": (c_int32, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                                c_int64, c_int64, c_int64, c_void_p, c_int64]),
     "rmlk_hip_store_weights": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
     "rmlk_hip_weights_fit": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
     "rmlk_hip_gemv_kmajor": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int32, c_void_p,
@@ -206,6 +213,7 @@ SIGNATURES = {
     "rmlk_session_create_ex": (c_int32, [c_void_p, c_int32, ctypes.c_uint32, POINTER(c_void_p)]),
     "rmlk_session_fused_nodes": (c_int32, [c_void_p]),
     "rmlk_session_weights_16bit": (c_int32, [c_void_p]),
+    "rmlk_session_products_bf16_pieces": (c_int32, [c_void_p]),
     "rmlk_session_destroy": (None, [c_void_p]),
     "rmlk_session_set_input": (c_int32, [c_void_p, c_char_p, c_int32, POINTER(c_int64), c_int32,
                                          c_void_p]),

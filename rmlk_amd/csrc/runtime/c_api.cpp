@@ -264,6 +264,7 @@ int32_t rmlk_session_create_ex(const rmlk_graph *g, int32_t device, uint32_t fla
                 throw RtError(RMLK_ERR_INVALID_ARGUMENT, "one storage type for the weights at most");
             s->impl.lossless_16bit = false;
         }
+        s->impl.bf16_pieces = (flags & RMLK_SESSION_BF16_PIECES) != 0;
         s->impl.build(*g, device);
         *out = s.release();
     });
@@ -271,6 +272,7 @@ int32_t rmlk_session_create_ex(const rmlk_graph *g, int32_t device, uint32_t fla
 
 int32_t rmlk_session_fused_nodes(const rmlk_session *s) { return s ? s->impl.fused_nodes : 0; }
 int32_t rmlk_session_weights_16bit(const rmlk_session *s) { return s ? s->impl.weights_16bit : 0; }
+int32_t rmlk_session_products_bf16_pieces(const rmlk_session *s) { return s ? s->impl.products_bf16_pieces : 0; }
 
 void rmlk_session_destroy(rmlk_session *s) {
     if (!s) return;

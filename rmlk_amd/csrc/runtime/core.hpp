@@ -296,6 +296,8 @@ struct Session {
     int32_t weight_storage = RMLK_FLOAT;   // how the K-contiguous copies of constant weights are held
     bool lossless_16bit = true;            // float storage gives way to 16 bits where no value changes
     int weights_16bit = 0;                 // weight matrices held as 16-bit values
+    bool bf16_pieces = false;              // many-row products over bfloat16 weights on the bf16 matrix cores
+    int products_bf16_pieces = 0;          // products the last run multiplied that way
     int fused_nodes = 0;
     int folded_nodes = 0;            // constant nodes evaluated while building
     int64_t device_syncs = 0;            // blocking reads of shape-like tensors

@@ -992,6 +992,26 @@ bool took_fast_path(int32_t st, const char *what) {
     return true;
 }
 
+// ---- many-row products over bfloat16 weights on the bf16 matrix cores ----------------------------
+// With Session::bf16_pieces a product of 64 and more rows over a weight matrix held as bfloat16
+// values splits its first operand into three bfloat16 pieces (exactly) and multiplies those
+// (rmlk_hip_matmul_bf16x3). The pieces live in the session workspace, behind `own` bytes that the
+// caller wants there for itself.
+bool wants_pieces(const OpContext &c, int64_t m, int64_t k, int32_t w_dtype) {
+    return c.session.bf16_pieces && w_dtype == RMLK_BFLOAT16 && m >= 64 && k % 32 == 0;
+}
+
+// Splits a [m, k] (dense rows); returns the pieces, null when the split does not take the operand.
+// *own_out: the caller's part of the workspace.
+void *split_pieces(OpContext &c, const void *a, int64_t m, int64_t k, size_t own, void **own_out,
+                   const char *what) {
+    const size_t own_bytes = (own + 255) / 256 * 256;
+    char *ws = static_cast<char *>(c.scratch(own_bytes + rmlk_hip_bf16x3_pieces_size(m, k)));
+    if (own_out) *own_out = ws;
+    void *pieces = ws + own_bytes;
+    return took_fast_path(rmlk_hip_bf16x3_split(c.stream, m, k, a, k, pieces), what) ? pieces : nullptr;
+}
+
 // ---- one-row RMSNorm left to the product that reads it ------------------------------------------
 // A norm node marked `defer_norm` (its result feeds exactly one product over K-contiguous constant
 // weights) does not run for a one-row input: its output is a view of the row BEFORE the norm that
@@ -1618,6 +1638,28 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
                 return;
         }
     }
+    if (ok && wants_pieces(c, a.numel() / k, k, wt.dtype)) {
+        const int64_t m = a.numel() / k;
+        const int32_t splits = rmlk_hip_bf16x3_splits(m, n, k);
+        void *slabs = nullptr;
+        void *pieces = splits > 0 ? split_pieces(c, a.data(), m, k, static_cast<size_t>(splits) * m * n * sizeof(float),
+                                                 &slabs, "rmlk.MatMulAddRMSNorm")
+                                  : nullptr;
+        if (pieces && took_fast_path(rmlk_hip_matmul_bf16x3(c.stream, m, n, k, pieces, wt.data(), k, splits, slabs, n,
+                                                            m * n),
+                                     "rmlk.MatMulAddRMSNorm")) {
+            Tensor &sum = c.alloc_output(0, RMLK_FLOAT, res.shape);
+            Tensor &y = c.alloc_output(1, RMLK_FLOAT, res.shape);
+            if (took_fast_path(rmlk_hip_splitk_add_rmsnorm(c.stream, RMLK_FLOAT, m, n, slabs, splits, m * n, res.data(),
+                                                           gamma.data(), attr_float(c, "epsilon"),
+                                                           static_cast<int32_t>(c.attr_int("reciprocal", 0)),
+                                                           sum.data(), y.data()),
+                               "rmlk.MatMulAddRMSNorm")) {
+                ++c.session.products_bf16_pieces;
+                return;
+            }
+        }
+    }
     if (ok) {
         const int64_t m = a.numel() / k;
         const size_t bytes = rmlk_hip_matmul_partials_workspace_size(RMLK_FLOAT, m, n, k);
@@ -1646,6 +1688,13 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
 // `w_dtype`: how the weights are stored (float, or the 16-bit type the session was built with).
 void product_over_kmajor(OpContext &c, const void *a, int64_t m, int64_t k, int32_t w_dtype, const void *wt,
                          int64_t n, void *out, const char *what) {
+    if (wants_pieces(c, m, k, w_dtype) && rmlk_hip_bf16x3_splits(m, n, k) > 0) {
+        void *pieces = split_pieces(c, a, m, k, 0, nullptr, what);
+        if (pieces && took_fast_path(rmlk_hip_matmul_bf16x3(c.stream, m, n, k, pieces, wt, k, 1, out, n, 0), what)) {
+            ++c.session.products_bf16_pieces;
+            return;
+        }
+    }
     const size_t ws_bytes = rmlk_hip_matmul_workspace_size(RMLK_FLOAT, 1, m, n, k);
     void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;
     if (w_dtype == RMLK_FLOAT) {
@@ -1733,6 +1782,16 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
         std::vector<int64_t> shape(a.shape.begin(), a.shape.end() - 1);
         shape.push_back(n);
         Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
+        if (wants_pieces(c, m, k, wt.dtype)) {
+            void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroupSwiGLU");
+            if (pieces && took_fast_path(rmlk_hip_matmul_bf16x3_swiglu(c.stream, m, n, k, pieces, wt.data(), k,
+                                                                       gate_first ? 0 : n, gate_first ? n : 0,
+                                                                       y.data(), n),
+                                         "rmlk.MatMulGroupSwiGLU")) {
+                ++c.session.products_bf16_pieces;
+                return;
+            }
+        }
         if (took_fast_path(rmlk_hip_matmul_swiglu(c.stream, RMLK_FLOAT, m, n, k, a.data(), k, wt.dtype, wt.data(), k, 1,
                                                   gate_first ? 0 : n, gate_first ? n : 0, y.data(), n),
                            "rmlk.MatMulGroupSwiGLU"))
@@ -1830,7 +1889,9 @@ void op_fused_matmul_group(OpContext &c) {
         // Everything that reads the members is one row-stream node: the product runs now, but its
         // split-K partial sums stay where they are - that node adds them up while it reads its rows,
         // which saves the combine launch and a round trip of the product through memory.
-        const size_t bytes = rmlk_hip_matmul_partials_workspace_size(RMLK_FLOAT, m, total, k);
+        const int32_t x3_splits = wants_pieces(c, m, k, wt.dtype) ? rmlk_hip_bf16x3_splits(m, total, k) : 0;
+        const size_t bytes = x3_splits > 0 ? static_cast<size_t>(x3_splits) * m * total * sizeof(float)
+                                           : rmlk_hip_matmul_partials_workspace_size(RMLK_FLOAT, m, total, k);
         if (bytes) {
             auto pp = std::make_shared<PendingProduct>();
             {
@@ -1840,9 +1901,25 @@ void op_fused_matmul_group(OpContext &c) {
                 c.out = keep;
             }
             int32_t splits = 0;
-            if (took_fast_path(rmlk_hip_matmul_partials(c.stream, RMLK_FLOAT, m, total, k, a.data(), k, wt.dtype, wt.data(), k,
-                                                        1, pp->slabs.data(), bytes, &splits),
-                               "rmlk.MatMulGroup")) {
+            bool multiplied = false;
+            if (x3_splits > 0) {
+                void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroup");
+                multiplied = pieces && took_fast_path(rmlk_hip_matmul_bf16x3(c.stream, m, total, k, pieces, wt.data(), k,
+                                                                             x3_splits, pp->slabs.data(), total,
+                                                                             m * total),
+                                                      "rmlk.MatMulGroup");
+                if (multiplied) {
+                    splits = x3_splits;
+                    ++c.session.products_bf16_pieces;
+                }
+            }
+            // (should the pieces be refused after all, the fp32 kernels take over where the slabs
+            // allocated for them are large enough for theirs)
+            if (multiplied ||
+                (bytes >= rmlk_hip_matmul_partials_workspace_size(RMLK_FLOAT, m, total, k) &&
+                 took_fast_path(rmlk_hip_matmul_partials(c.stream, RMLK_FLOAT, m, total, k, a.data(), k, wt.dtype,
+                                                         wt.data(), k, 1, pp->slabs.data(), bytes, &splits),
+                                "rmlk.MatMulGroup"))) {
                 pp->x = a;
                 pp->wt = wt;
                 pp->k = k;
@@ -1867,6 +1944,23 @@ void op_fused_matmul_group(OpContext &c) {
         std::vector<void *> outs;
         for (size_t i = 0; i < widths.size(); ++i)
             outs.push_back(c.alloc_output(static_cast<int>(i), RMLK_FLOAT, out_shape(widths[i])).data());
+        bool as_pieces = wants_pieces(c, m, k, wt.dtype);
+        for (size_t i = 0; as_pieces && i < widths.size(); ++i)
+            as_pieces = rmlk_hip_bf16x3_splits(m, widths[i], k) > 0;
+        if (as_pieces) {
+            // one split of the operand, a product per member over its rows of the joint matrix
+            if (void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroup")) {
+                int64_t first = 0;
+                for (size_t i = 0; i < widths.size(); ++i) {
+                    check_status(rmlk_hip_matmul_bf16x3(c.stream, m, widths[i], k, pieces, rows + first * row_bytes, k, 1,
+                                                        outs[i], widths[i], 0),
+                                 "rmlk.MatMulGroup");
+                    first += widths[i];
+                }
+                ++c.session.products_bf16_pieces;
+                return;
+            }
+        }
         const size_t ws_bytes = rmlk_hip_matmul_grouped_workspace_size(
             RMLK_FLOAT, m, k, static_cast<int32_t>(widths.size()), widths.data());
         void *ws = ws_bytes ? c.scratch(ws_bytes) : nullptr;

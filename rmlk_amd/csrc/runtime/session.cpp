@@ -443,6 +443,7 @@ void Session::build(const rmlk_graph &graph, int dev) {
 
 void Session::run_nodes() {
     const rmlk_graph &gr = graph_copy;
+    products_bf16_pieces = 0;
     // Operators over tiny tensors (the per-step set-up of a decoder graph: tables, indices, masks) are
     // collected by the kernel library and go out as one launch in front of the next larger one. Not
     // with one kernel per node (no fusion), and not while nodes are timed one by one.

@@ -367,6 +367,35 @@ def matmul_swiglu(a, b, out, m: int, n: int, k: int, ldb: int, gate_offset: int,
           "rmlk_hip_matmul_swiglu")
 
 
+def bf16x3_split(a: torch.Tensor) -> torch.Tensor:
+    """The three bfloat16 pieces of the dense float matrix a [m, k] (a = hi + mid + lo exactly), as the
+    planes [3][m rounded up to 128][k] that matmul_bf16x3 reads (an int16 tensor)."""
+    m, k = a.shape
+    pieces = torch.empty(lib().rmlk_hip_bf16x3_pieces_size(m, k) // 2, dtype=torch.int16, device=a.device)
+    check(lib().rmlk_hip_bf16x3_split(_stream(), m, k, _ptr(a), k, _ptr(pieces)), "rmlk_hip_bf16x3_split")
+    return pieces
+
+
+def bf16x3_splits(m: int, n: int, k: int) -> int:
+    """Slabs of K with which matmul_bf16x3 fills the GPU for this size; 0: a size it does not take."""
+    return int(lib().rmlk_hip_bf16x3_splits(m, n, k))
+
+
+def matmul_bf16x3(pieces, wt, out, m: int, n: int, k: int, splits: int = 1) -> None:
+    """out[m, n] (splits == 1) or out[splits, m, n] (one partial product per slab of K) = a . wt^T over
+    the pieces of a (bf16x3_split) and bfloat16 weights wt [n, k], on the bf16 matrix cores."""
+    assert wt.dtype == torch.bfloat16
+    check(lib().rmlk_hip_matmul_bf16x3(_stream(), m, n, k, _ptr(pieces), _ptr(wt), k, splits, _ptr(out), n, m * n),
+          "rmlk_hip_matmul_bf16x3")
+
+
+def matmul_bf16x3_swiglu(pieces, wt, out, m: int, n: int, k: int, gate_row: int, up_row: int) -> None:
+    """out[m, n] = swiglu(a . wt[gate_row:+n]^T, a . wt[up_row:+n]^T) over the pieces of a."""
+    assert wt.dtype == torch.bfloat16
+    check(lib().rmlk_hip_matmul_bf16x3_swiglu(_stream(), m, n, k, _ptr(pieces), _ptr(wt), k, gate_row, up_row,
+                                              _ptr(out), n), "rmlk_hip_matmul_bf16x3_swiglu")
+
+
 def rotary(x, cos, sin, out, shape, x_stride, cos_stride, sin_stride) -> None:
     """Fused half-rotation rotary embedding over a strided [B,H,S,D] view of x."""
     check(lib().rmlk_hip_rotary(_stream(), dtype_of(x), Dims.of(shape), Dims.of(x_stride),

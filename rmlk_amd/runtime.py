@@ -179,10 +179,11 @@ class GraphBuilder:
 class ModelInstance:
     """ref: runtime/src/core/instance.rs:20-119"""
 
-    def __init__(self, graph: Graph, device: int = 0, fuse: bool = True, weights: str = "auto"):
+    def __init__(self, graph: Graph, device: int = 0, fuse: bool = True, weights: str = "auto",
+                 bf16_pieces: bool = False):
         self.graph = graph
         h = ctypes.c_void_p()
-        flags = (0 if fuse else 1) | {"auto": 0, "f16": 2, "bf16": 4, "f32": 8}[weights]
+        flags = (0 if fuse else 1) | {"auto": 0, "f16": 2, "bf16": 4, "f32": 8}[weights] | (16 if bf16_pieces else 0)
         _check(lib().rmlk_session_create_ex(graph.handle, device, flags, ctypes.byref(h)),
                "Builder.build")
         self._h = h
@@ -191,6 +192,11 @@ class ModelInstance:
     def weights_16bit(self) -> int:
         """Constant weight matrices the session holds as 16-bit values."""
         return int(lib().rmlk_session_weights_16bit(self._h))
+
+    @property
+    def products_bf16_pieces(self) -> int:
+        """Products of the last run that went to the bf16 matrix cores (bf16_pieces=True)."""
+        return int(lib().rmlk_session_products_bf16_pieces(self._h))
 
     @property
     def fused_nodes(self) -> int:
@@ -315,10 +321,13 @@ class Builder:
         from .onnx_io import load_onnx_bytes
         return Builder(load_onnx_bytes(data, base_dir))
 
-    def build(self, device: int = 0, fuse: bool = True, weights: str = "auto") -> ModelInstance:
+    def build(self, device: int = 0, fuse: bool = True, weights: str = "auto",
+              bf16_pieces: bool = False) -> ModelInstance:
         """fuse=False keeps one kernel per node, as the reference executes a graph. weights: how the
         constant weights of fused MatMuls are stored (the arithmetic is fp32 in every case): "auto"
         as floats, or as 16-bit values where every float of a matrix is a bfloat16 / half value
         already (nothing is lost); "f32" as floats regardless; "f16" / "bf16" rounded to that type
-        (half the bytes to stream per token)."""
-        return ModelInstance(self._graph, device, fuse, weights)
+        (half the bytes to stream per token). bf16_pieces: products of 64 and more rows over
+        weights held as bfloat16 values split their fp32 operand into three bfloat16 pieces (exactly)
+        and run on the bf16 matrix cores - fp32 results, sums in another order, about 2.5x the rate."""
+        return ModelInstance(self._graph, device, fuse, weights, bf16_pieces)
