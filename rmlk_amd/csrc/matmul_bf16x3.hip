@@ -17,10 +17,23 @@
 // against 3 x 2 fragments of A, 6 * TN MFMAs.
 //
 // No counterpart in the reference (its products are fp32 cuBLAS calls, cuda/src/kernels/gemm.rs:191-232).
+#include <utility>
+
 #include "common.hpp"
 
 namespace rmlk {
 namespace {
+
+// f(integral_constant<int, 0>) .. f(integral_constant<int, N - 1>): a loop whose index is a constant
+// expression in the body.
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(std::forward<F>(f), std::make_integer_sequence<int, N>{});
+}
 
 typedef __attribute__((ext_vector_type(8))) __bf16 v8bf;
 typedef __attribute__((ext_vector_type(16))) float v16f;
@@ -86,16 +99,19 @@ struct X3Args {
 };
 
 // Block tile 128 x (64 * TN), four wavefronts (2 x 2) of 64 x (32 * TN). LDS rows are 64 bytes (32
-// bfloat16): two rows make a 128-byte super-row of eight 16-byte units, and unit q of super-row R
-// lives at position q ^ (R & 7) - applied on the global side when a unit is fetched (each lane of a
-// direct load picks its own source) and again when it is read back, which spreads the eight lanes of
-// a 128-bit fragment read over all banks.
+// bfloat16, four 16-byte units), unpadded - a direct load writes 64 lanes x 16 bytes as one
+// contiguous KiB - and unit u of row r lives at position u ^ ((r >> 2) & 3) of its row, applied on
+// the global side when a unit is fetched (each lane of a direct load picks its own source) and again
+// when it is read back: the sixteen lanes that a 128-bit fragment read serves together (sixteen
+// consecutive rows, one unit each) then cover all 64 banks once.
 //
-// The stage for K step s + STAGES - 1 is requested at the start of step s, into the LDS stage that
-// was read in step s - 1; a wavefront's loads complete in order, so "all but the loads of the
-// STAGES - 2 newest stages have landed" (vmcnt) says that the next stage is there. One block-wide
-// barrier per K step, halfway through it: before it every wavefront has read the step's second
-// chunk into registers, after it the first chunk of the next step is read.
+// The stage for K step s + STAGES - 1 is requested during step s, into the LDS stage that was read
+// in step s - 1; a wavefront's loads complete in order, so "all but the loads of the STAGES - 2
+// newest stages have landed" (vmcnt) says that the next stage is there. One block-wide barrier per K
+// step, a quarter into its second chunk: before it every wavefront has read the step's second chunk
+// into registers, after it the first chunk of the next step is read. The matrix pipe takes a new
+// MFMA every 32 cycles and a wavefront issues in order, so the LDS reads and the direct loads are
+// dealt out between the MFMAs one at a time (loads and reads alternating) instead of in bursts.
 //
 // SWIGLU: the tile's rows of W are half gate rows, half up rows, arranged so that a wavefront's
 // accumulator columns j and j + TN / 2 hold the gate and the up value of the same output column; the
@@ -129,9 +145,8 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16x3_kernel(X3Args g) {
     const int wm = wave / 2, wn = wave % 2;
     const int l32 = lane % 32, half = lane / 32;
 
-    // Sources. Lane l of a piece fills LDS unit l of the piece: super-row l / 8, position l % 8.
-    const int src_v = (lane % 8) ^ (lane / 8);
-    const int src_row = 2 * (lane / 8) + src_v / 4, src_unit = src_v % 4;
+    // Sources. Lane l of a piece fills LDS unit l of the piece: row l / 4, position l % 4.
+    const int src_row = lane / 4, src_unit = (lane % 4) ^ ((lane / 16) & 3);
     uint32_t a_voff[A_LOADS], b_voff[B_LOADS];
 #pragma unroll
     for (int j = 0; j < A_LOADS; ++j) {
@@ -171,25 +186,32 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16x3_kernel(X3Args g) {
         a_ptr += BK;
         b_ptr += BK;
     };
+    auto load_op = [&](int buf, auto o_tag) {
+        constexpr int o = decltype(o_tag)::value;
+        const uint32_t base = lds0 + static_cast<uint32_t>(buf * kStage);
+        if constexpr (o < A_LOADS) direct_load(base + o * 4096, a_ptr, a_voff[o]);
+        else direct_load(base + kAStage + (o - A_LOADS) * 4096, b_ptr, b_voff[o - A_LOADS]);
+    };
 
     // Fragments: for K chunk c lane (l32, half) reads unit c * 2 + half of its row - eight
     // consecutive K values, the same eight for A and W.
     int frag_off[2];
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
-        frag_off[c] = (l32 / 2) * 128 + ((((l32 % 2) * 4 + c * 2 + half) ^ ((l32 / 2) & 7)) * 16);
-    const int a_base = wm * 32 * 128, b_base = kAStage + wn * (WN / 2) * 128;
+    for (int c = 0; c < 2; ++c) frag_off[c] = l32 * 64 + ((c * 2 + half) ^ ((l32 / 4) & 3)) * 16;
+    const int a_base = wm * 64 * 64, b_base = kAStage + wn * WN * 64;
     v4u af[2][3][TM], bfr[2][TN];
-    auto read_frags = [&](int buf, int c, int s) {
+    // read number o of a chunk, in the order the MFMAs want them: W's column blocks, then the lo,
+    // the mid and the hi piece of A's row blocks
+    constexpr int kFragOps = TN + 3 * TM;
+    auto frag_op = [&](int buf, int c, auto s_tag, auto o_tag) {
+        constexpr int s = decltype(s_tag)::value, o = decltype(o_tag)::value;
         const unsigned char *st = smem + buf * kStage;
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-            bfr[s][j] = *reinterpret_cast<const v4u *>(st + b_base + j * 2048 + frag_off[c]);
-#pragma unroll
-        for (int p = 0; p < 3; ++p)
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                af[s][p][i] = *reinterpret_cast<const v4u *>(st + p * kPlane + a_base + i * 2048 + frag_off[c]);
+        if constexpr (o < TN) {
+            bfr[s][o] = *reinterpret_cast<const v4u *>(st + b_base + o * 2048 + frag_off[c]);
+        } else {
+            constexpr int q = o - TN, p = 2 - q / TM, i = q % TM;
+            af[s][p][i] = *reinterpret_cast<const v4u *>(st + p * kPlane + a_base + i * 2048 + frag_off[c]);
+        }
     };
 
     v16f acc[TM][TN];
@@ -200,53 +222,86 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16x3_kernel(X3Args g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // (pieces outermost: TM * TN independent accumulators between two MFMAs on the same one; the
-    // small pieces first)
-    auto mfmas = [&](int s) {
-#pragma unroll
-        for (int p = 2; p >= 0; --p)
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(v8bf, af[s][p][i]), __builtin_bit_cast(v8bf, bfr[s][j]), acc[i][j], 0,
-                        0, 0);
+    // MFMA number q of a chunk: pieces outermost (TM * TN independent accumulators between two MFMAs
+    // on the same one), the small pieces first
+    constexpr int NM = 3 * TM * TN;
+    auto mfma_at = [&](auto s_tag, auto q_tag) {
+        constexpr int s = decltype(s_tag)::value, q = decltype(q_tag)::value;
+        constexpr int p = 2 - q / (TM * TN), i = (q / TN) % TM, j = q % TN;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, af[s][p][i]),
+                                                            __builtin_bit_cast(v8bf, bfr[s][j]), acc[i][j], 0, 0, 0);
+    };
+    using Slot0 = std::integral_constant<int, 0>;
+    using Slot1 = std::integral_constant<int, 1>;
+    constexpr int kBarrierAt = NM / 4;
+    // One K step over LDS stage `buf`: chunk 0 from fragment slot 0 while chunk 1 is read into slot 1
+    // and (LOAD) the stage `fill` is requested; chunk 1 from slot 1, the block meets, chunk 0 of
+    // stage `next` is read into slot 0 (MORE).
+    auto k_step = [&](int buf, int next, int fill, auto load_tag, auto more_tag) {
+        constexpr bool LOAD = decltype(load_tag)::value, MORE = decltype(more_tag)::value;
+        constexpr int n_loads = LOAD ? kLoads : 0;
+        static_for<NM>([&](auto q_tag) {
+            constexpr int q = decltype(q_tag)::value;
+            mfma_at(Slot0{}, q_tag);
+            static_for<kFragOps>([&](auto o_tag) {
+                constexpr int o = decltype(o_tag)::value;
+                if constexpr ((2 * kFragOps <= NM ? 2 * o + 1 : o * (NM - 2) / kFragOps) == q)
+                    frag_op(buf, 1, Slot1{}, o_tag);
+            });
+            static_for<n_loads>([&](auto o_tag) {
+                constexpr int o = decltype(o_tag)::value;
+                if constexpr (o * NM / (n_loads > 0 ? n_loads : 1) == q) load_op(fill, o_tag);
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if constexpr (LOAD) {
+            a_ptr += BK;
+            b_ptr += BK;
+        }
+        constexpr int room = NM - kBarrierAt - 1;
+        static_for<NM>([&](auto q_tag) {
+            constexpr int q = decltype(q_tag)::value;
+            mfma_at(Slot1{}, q_tag);
+            if constexpr (MORE && q == kBarrierAt) {
+                // this wavefront has read all of this stage and the next stage has landed; then the
+                // block meets
+                if constexpr (LOAD)
+                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((STAGES - 2) * kLoads) : "memory");
+                else
+                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                asm volatile("s_barrier" ::: "memory");
+            }
+            if constexpr (MORE) {
+                static_for<kFragOps>([&](auto o_tag) {
+                    constexpr int o = decltype(o_tag)::value;
+                    if constexpr (kBarrierAt + 1 + (kFragOps <= room ? o : o * room / kFragOps) == q)
+                        frag_op(next, 0, Slot0{}, o_tag);
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
     };
 
     if (n_steps > 0) {
-        int issued = 0;
-#pragma unroll
-        for (int s = 0; s < STAGES - 1; ++s)
-            if (issued < n_steps) {
-                load_stage(s);
-                ++issued;
-            }
-        if (issued == STAGES - 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * kLoads) : "memory");
+        const int pre = n_steps < STAGES - 1 ? n_steps : STAGES - 1;
+        for (int s = 0; s < pre; ++s) load_stage(s);
+        // stage 0 has landed: everything but the stages requested after it
+        if (pre == STAGES - 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * kLoads) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         asm volatile("s_barrier" ::: "memory");
-        read_frags(0, 0, 0);
-        int buf = 0, fill = STAGES - 1;            // fill: the LDS stage the next loads go to
-        for (int step = 0; step < n_steps; ++step) {
-            const bool more = step + 1 < n_steps;
-            const bool load = issued < n_steps;
-            if (load) {
-                load_stage(fill);
-                ++issued;
-                fill = fill + 1 == STAGES ? 0 : fill + 1;
-            }
-            read_frags(buf, 1, 1);
-            mfmas(0);
-            const int next = buf + 1 == STAGES ? 0 : buf + 1;
-            if (more) {
-                if (load) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((STAGES - 2) * kLoads) : "memory");
-                else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-                asm volatile("s_barrier" ::: "memory");
-                read_frags(next, 0, 0);
-            }
-            mfmas(1);
-            buf = next;
+        static_for<kFragOps>([&](auto o_tag) { frag_op(0, 0, Slot0{}, o_tag); });
+        int buf = 0, fill = STAGES - 1, step = 0;   // fill: the LDS stage the next loads go to
+        auto after = [](int stage) { return stage + 1 == STAGES ? 0 : stage + 1; };
+        for (; step + STAGES - 1 < n_steps; ++step) {
+            k_step(buf, after(buf), fill, std::true_type{}, std::true_type{});
+            buf = after(buf);
+            fill = after(fill);
         }
+        for (; step + 1 < n_steps; ++step) {      // nothing left to request
+            k_step(buf, after(buf), fill, std::false_type{}, std::true_type{});
+            buf = after(buf);
+        }
+        k_step(buf, 0, fill, std::false_type{}, std::false_type{});
     }
 
     float *C = g.c + split * g.slab;
