@@ -128,6 +128,98 @@ pub unsafe fn gemv_kmajor(
     )
 }
 
+/// Bytes that the three bfloat16 pieces of a dense float matrix `[m, k]` take (`bf16x3_split`).
+pub fn bf16x3_pieces_size(m: usize, k: usize) -> usize {
+    unsafe { ffi::rmlk_hip_bf16x3_pieces_size(m as i64, k as i64) }
+}
+
+/// Splits the float matrix `a` `[m, k]` into three bfloat16 pieces whose sum it is exactly, as
+/// the planes `[3][m rounded up to 128][k]` that `matmul_bf16x3` reads.
+pub unsafe fn bf16x3_split(
+    stream: &HipStream,
+    m: usize,
+    k: usize,
+    a: *const c_void,
+    lda: usize,
+    pieces: *mut c_void,
+) -> Result<()> {
+    check(ffi::rmlk_hip_bf16x3_split(stream.raw(), m as i64, k as i64, a, lda as i64, pieces), "bf16x3_split")
+}
+
+/// Slabs of K with which `matmul_bf16x3` fills the GPU for a size; `None`: a size it does not take.
+pub fn bf16x3_splits(m: usize, n: usize, k: usize) -> Option<usize> {
+    match unsafe { ffi::rmlk_hip_bf16x3_splits(m as i64, n as i64, k as i64) } {
+        s if s > 0 => Some(s as usize),
+        _ => None,
+    }
+}
+
+/// `c[m, n] = a . wt^T` over the pieces of `a` and bfloat16 weights `wt` `[n, k]` on the bf16
+/// matrix cores, fp32 results. `splits > 1`: one partial product per slab of K, `slab` elements
+/// apart, for a reader that adds them up.
+pub unsafe fn matmul_bf16x3(
+    stream: &HipStream,
+    m: usize,
+    n: usize,
+    k: usize,
+    pieces: *const c_void,
+    wt: *const c_void,
+    ldw: usize,
+    splits: usize,
+    c: *mut c_void,
+    ldc: usize,
+    slab: usize,
+) -> Result<()> {
+    check(
+        ffi::rmlk_hip_matmul_bf16x3(
+            stream.raw(),
+            m as i64,
+            n as i64,
+            k as i64,
+            pieces,
+            wt,
+            ldw as i64,
+            splits as i32,
+            c,
+            ldc as i64,
+            slab as i64,
+        ),
+        "matmul_bf16x3",
+    )
+}
+
+/// `out[m, n] = swiglu(a . wt[gate_row..+n]^T, a . wt[up_row..+n]^T)` over the pieces of `a`.
+pub unsafe fn matmul_bf16x3_swiglu(
+    stream: &HipStream,
+    m: usize,
+    n: usize,
+    k: usize,
+    pieces: *const c_void,
+    wt: *const c_void,
+    ldw: usize,
+    gate_row: usize,
+    up_row: usize,
+    out: *mut c_void,
+    ldc: usize,
+) -> Result<()> {
+    check(
+        ffi::rmlk_hip_matmul_bf16x3_swiglu(
+            stream.raw(),
+            m as i64,
+            n as i64,
+            k as i64,
+            pieces,
+            wt,
+            ldw as i64,
+            gate_row as i64,
+            up_row as i64,
+            out,
+            ldc as i64,
+        ),
+        "matmul_bf16x3_swiglu",
+    )
+}
+
 /// Shape of a grouped-query attention call.
 #[derive(Clone, Copy, Debug)]
 pub struct AttentionShape {

@@ -442,9 +442,12 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(GemmArgs g) {
 // writes 64 lanes x 16 bytes as one contiguous 1 KiB piece of LDS while every lane picks its own
 // global address. Rows of 32 floats are therefore unpadded in LDS; bank conflicts on the
 // fragment reads of K-contiguous operands are avoided by a swizzle instead: the 16-byte unit q of
-// row r lives in unit q ^ (r & 7), applied on the global side when the unit is fetched and again
-// when it is read back. The loads are opaque to the compiler (inline asm), so completion is
-// awaited by hand (vmcnt) before the block-wide barrier that publishes a stage.
+// row r lives in unit q ^ ((r >> 1) & 7), applied on the global side when the unit is fetched and
+// again when it is read back. (A 128-bit read serves sixteen lanes together - sixteen consecutive
+// rows, one unit each; rows of 128 bytes alternate between the two halves of the 64 banks, and the
+// eight rows of one parity take eight different units: every bank once.) The loads are opaque to
+// the compiler (inline asm), so completion is awaited by hand (vmcnt) before the block-wide barrier
+// that publishes a stage.
 //
 // SWIGLU: the block's B tile is half gate columns, half up columns of one joint weight matrix,
 // arranged so that a wavefront's first accumulator column holds gate values and its second the up
@@ -508,7 +511,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     // Global sources of a stage: piece (p * 4 + wave) goes to this wavefront. The address is a
     // wave-uniform base (scalar registers, advanced by one K step with scalar adds) plus a per-lane
     // byte offset per piece that never changes, so the loads cost no vector ALU work.
-    const int sw_row = lane / 8, sw_unit = (lane % 8) ^ sw_row;
+    const int sw_row = lane / 8, sw_unit = (lane % 8) ^ ((wave * 4 + sw_row / 2) & 7);
     uint32_t a_voff[A_PASSES], b_voff[B_PASSES > 0 ? B_PASSES : 1];
     const float *a_ptr = A + static_cast<int64_t>(m0) * g.lda + k_begin;
 #pragma unroll
@@ -541,8 +544,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
                 row = min(row, g.n - 1 - n0);
             }
             b16_voff[p] = static_cast<uint32_t>((row * g.ldb + u * 8) * static_cast<int64_t>(2));
-            b16_lds[p][0] = lrow * BK + ((2 * u) ^ (lrow & 7)) * 4;
-            b16_lds[p][1] = lrow * BK + ((2 * u + 1) ^ (lrow & 7)) * 4;
+            b16_lds[p][0] = lrow * BK + ((2 * u) ^ ((lrow >> 1) & 7)) * 4;
+            b16_lds[p][1] = lrow * BK + ((2 * u + 1) ^ ((lrow >> 1) & 7)) * 4;
         }
     } else if constexpr (TB) {
         b_ptr = B + (SWIGLU ? 0 : static_cast<int64_t>(n0) * g.ldb) + k_begin;
@@ -626,7 +629,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     };
 
     // fragment addressing
-    const int xr = l32 & 7;
+    const int xr = (l32 >> 1) & 7;
     const int a_row = (wm * WM + l32) * BK;
     const int b_base = TB ? (wn * WN + l32) * BK : (half * 4) * BN + wn * WN + l32;
     v4f af[2][TM];
