@@ -86,6 +86,39 @@ def test_products_of_small_integers_are_exact(device, m, n, k, splits):
         assert np.array_equal(got[s].astype(np.float64), exp), f"slab {s}"
 
 
+def test_random_sizes_of_small_integers_are_exact(device):
+    """Forty random sizes (any m, n in whole 128-column tiles, K in whole steps, any slab count that
+    cuts K into whole steps), plain and SwiGLU form: every tile shape, stage count, step count below
+    and above the number of stages, padded rows."""
+    import torch
+    kk = _k()
+    rng = np.random.default_rng(77)
+    for case in range(40):
+        m = int(rng.integers(1, 700))
+        n = 128 * int(rng.integers(1, 40)) if case % 4 else 256 * int(rng.integers(100, 300))
+        steps = int(rng.integers(1, 60))
+        splits = int(rng.choice([s for s in (1, 2, 3, 4, 8) if steps % s == 0]))
+        k = 32 * steps
+        if m * n > 40e6:
+            m = max(1, int(40e6 // n))
+        a = rng.integers(-8, 9, size=(m, k)).astype(np.float32)
+        w = rng.integers(-4, 5, size=(n, k)).astype(np.float32)
+        a_d, w_d = to_dev(a, device), _bf16_weights(w, device)
+        pieces = kk.bf16x3_split(a_d)
+        out = torch.full((splits, m, n), np.nan, dtype=torch.float32, device=device)
+        kk.matmul_bf16x3(pieces, w_d, out, m, n, k, splits)
+        got = out.to(torch.float64).sum(0)
+        exp = a_d.to(torch.float64) @ w_d.to(torch.float64).T
+        assert torch.equal(got, exp), (case, m, n, k, splits)
+        if n % 256 == 0:
+            half = n // 2
+            act = torch.full((m, half), np.nan, dtype=torch.float32, device=device)
+            kk.matmul_bf16x3_swiglu(pieces, w_d, act, m, half, k, half, 0)
+            gate, up = exp[:, half:], exp[:, :half]
+            ref = (gate / (1 + torch.exp(-gate)) * up).to(torch.float32)
+            assert torch.allclose(act, ref, rtol=1e-5, atol=1e-5), (case, m, n, k, "swiglu")
+
+
 @pytest.mark.parametrize("m,n,k", [(512, 2048, 2048), (100, 640, 8192), (512, 16384, 256)])
 def test_full_mantissa_products_have_the_error_of_fp32_accumulation(device, m, n, k):
     import torch
