@@ -17,23 +17,10 @@
 // against 3 x 2 fragments of A, 6 * TN MFMAs.
 //
 // No counterpart in the reference (its products are fp32 cuBLAS calls, cuda/src/kernels/gemm.rs:191-232).
-#include <utility>
-
 #include "common.hpp"
 
 namespace rmlk {
 namespace {
-
-// f(integral_constant<int, 0>) .. f(integral_constant<int, N - 1>): a loop whose index is a constant
-// expression in the body.
-template <typename F, int... I>
-__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
-    (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F &&f) {
-    static_for_impl(std::forward<F>(f), std::make_integer_sequence<int, N>{});
-}
 
 typedef __attribute__((ext_vector_type(8))) __bf16 v8bf;
 typedef __attribute__((ext_vector_type(16))) float v16f;
@@ -344,13 +331,8 @@ int32_t launch_x3(hipStream_t st, X3Args g, int splits) {
     const int64_t tiles = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
     g.per_xcd = static_cast<int32_t>((tiles + 7) / 8);
     auto kern = gemm_bf16x3_kernel<TN, STAGES, SWIGLU>;
-    static std::atomic<bool> raised{false};        // (per device in principle; one limit for all is fine)
-    if (!raised.load(std::memory_order_acquire)) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return static_cast<int32_t>(e);
-        raised.store(true, std::memory_order_release);
-    }
+    static DynamicLdsGrant grant;
+    if (const int32_t st_grant = grant.ensure(kern, lds); st_grant != RMLK_OK) return st_grant;
     kern<<<dim3(g.per_xcd * 8, splits), kThreads, lds, st>>>(g);
     return launch_status();
 }
