@@ -29,6 +29,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_BF16_MFMA_TFLOPS = 2500.0   # dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 CALIBRATION_COPY_BYTES = 256 << 20
 
@@ -196,7 +197,8 @@ def run_llama(args):
     # same counts, weights rotated so that they come from HBM as in the model), issued back to back
     # through the C ABI between ONE pair of HIP events on the stream they run on. (The per-node
     # events above add a cache write-back after every node, ~10 us on a 16 MiB output.)
-    dom_us = time_matmul_launches(kernels, torch, dom["shapes"], storage=stored)
+    pieces = bool(prefill_products_bf16)   # the products ran as bfloat16 pieces on the bf16 matrix cores
+    dom_us = time_matmul_launches(kernels, torch, dom["shapes"], storage=stored, pieces=pieces)
     achieved = dom["flops"] / dom["launches"] / (dom_us * 1e-6) / 1e12
     roofline = {
         "bound": "mfma",
@@ -216,6 +218,16 @@ def run_llama(args):
         "measured": "one HIP event pair around the kernel's launches of one prefill pass (same shapes "
                     "and counts, cold weights), 4 repetitions after 8 untimed ones, on the launching stream",
     }
+    if pieces:
+        # three bf16 MFMAs per product: priced against the bf16 peak at three times the fp32 flops
+        roofline.update({
+            "kernel": f"gemm_bf16x3_kernel (the launches that the fp32 path would give to: {dom_kind})",
+            "achieved": round(3 * achieved, 2), "peak": PEAK_BF16_MFMA_TFLOPS,
+            "frac": round(3 * achieved / PEAK_BF16_MFMA_TFLOPS, 4),
+            "fp32_equivalent_tflops": round(achieved, 2), "traffic": None,
+            "flops_per_launch": 3 * dom["flops"] / dom["launches"],
+            "note": "bf16 flops = 3 x 2 M N K (hi, mid and lo piece of the fp32 operand); the split of the "
+                    "operand into pieces is a launch of its own and not part of this duration"})
     all_mm_flops = sum(d["flops"] for d in by_kind.values())
     all_mm_us = sum(d["us"] for d in by_kind.values())
     matmul_all = {"tflops": round(all_mm_flops / (all_mm_us * 1e-6) / 1e12, 2),
@@ -294,7 +306,9 @@ def run_llama(args):
         "metric": "llama3.2-1b-shape fp32 prefill tok/s (decode ms/tok alongside)",
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if not prefill_products_bf16 else "f32 (many-row products: exact products of bf16 pieces, f32 accumulation)",
+        "data": "synthetic",
         "weight_storage": stored, "weight_storage_asked": args.weights,
         "weights_are_bfloat16_values": bool(args.bf16_values),
         "prefill_products_on_bf16_matrix_cores": prefill_products_bf16,
@@ -316,7 +330,7 @@ def run_llama(args):
     return result
 
 
-def time_matmul_launches(kernels, torch, shape_counts, reps=4, warm_reps=8, storage="f32"):
+def time_matmul_launches(kernels, torch, shape_counts, reps=4, warm_reps=8, storage="f32", pieces=False):
     """Average duration (us) of rmlk_hip_matmul launches: for every (batch, m, n, k) -> count, `count`
     launches with a broadcast 2-D K-contiguous weight operand taken in turn from enough distinct buffers to
     exceed the 256 MB Infinity Cache, all between one pair of HIP events on the current stream.
@@ -336,13 +350,19 @@ def time_matmul_launches(kernels, torch, shape_counts, reps=4, warm_reps=8, stor
         c = torch.empty(batch, m, n // 2 if swiglu else n, device=dev)
         need = kernels.matmul_workspace_size(batch, m, n, k)
         ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
-        plans.append((batch, m, n, k, swiglu, count, a, bs, c, ws))
+        # pieces: the launches of rmlk_hip_matmul_bf16x3 over the operand split beforehand
+        a3 = kernels.bf16x3_split(a[0]) if pieces else None
+        plans.append((batch, m, n, k, swiglu, count, a, bs, c, ws, a3))
         total += count
 
     def run_once():
-        for batch, m, n, k, swiglu, count, a, bs, c, ws in plans:
+        for batch, m, n, k, swiglu, count, a, bs, c, ws, a3 in plans:
             for i in range(count):
-                if swiglu:
+                if pieces and swiglu:
+                    kernels.matmul_bf16x3_swiglu(a3, bs[i % len(bs)], c, m, n // 2, k, 0, n // 2)
+                elif pieces:
+                    kernels.matmul_bf16x3(a3, bs[i % len(bs)], c, m, n, k)
+                elif swiglu:
                     kernels.matmul_swiglu(a, bs[i % len(bs)], c, m, n // 2, k, k, 0, n // 2, trans_b=True)
                 elif storage != "f32":
                     # (the product over stored weights: the grouped entry point with one member)
@@ -846,6 +866,9 @@ def main():
         result["variant_bf16_valued_weights"]["prefill_ms_products_as_bf16_pieces"] = r["ms_per_step"]
         result["variant_bf16_valued_weights"]["prefill_products_on_bf16_matrix_cores"] = \
             r["prefill_products_on_bf16_matrix_cores"]
+        result["variant_bf16_valued_weights"]["roofline_products_as_bf16_pieces"] = {
+            k_: r["roofline"][k_] for k_ in ("bound", "kernel", "achieved", "peak", "unit", "frac", "avg_launch_us",
+                                             "fp32_equivalent_tflops", "note")}
     print(json.dumps(result))
 
 
