@@ -998,7 +998,9 @@ bool took_fast_path(int32_t st, const char *what) {
 // (rmlk_hip_matmul_bf16x3). The pieces live in the session workspace, behind `own` bytes that the
 // caller wants there for itself.
 bool wants_pieces(const OpContext &c, int64_t m, int64_t k, int32_t w_dtype) {
-    return c.session.bf16_pieces && w_dtype == RMLK_BFLOAT16 && m >= 64 && k % 32 == 0;
+    // (the kernels address the pieces with 32 bits: no workspace is asked for an operand they refuse)
+    return c.session.bf16_pieces && w_dtype == RMLK_BFLOAT16 && m >= 64 && k % 32 == 0 &&
+           rmlk_hip_bf16x3_pieces_size(m, k) < (static_cast<size_t>(1) << 32);
 }
 
 // Splits a [m, k] (dense rows); returns the pieces, null when the split does not take the operand.
