@@ -674,8 +674,12 @@ def run_graph_suite(args):
         graph, feeds = graphs.rmsnorm_matmul_graph(seed=1)
         workload = "BASELINE configs[0]: decomposed RMSNorm [1,128,2048] + MatMul [2048,8192], fp32"
     elif args.suite == "c3":
-        graph, feeds = graphs.decoder_layer_graph(seed=3, seq=2048)
+        graph, feeds = graphs.decoder_layer_graph(seed=3, seq=2048, bf16_values=args.bf16_values)
         workload = "BASELINE configs[2]: one Llama-3.2-1B-shaped decoder layer, prefill S=2048, fp32"
+        if args.bf16_values:
+            workload += ("; weights that are bfloat16 values held as floats (16-bit storage where lossless)" +
+                         (", many-row products of the fused session as bfloat16 pieces on the bf16 matrix cores"
+                          if args.bf16_pieces else ""))
     else:
         graph, feeds = graphs.kv_stress_graph(seed=5)
         workload = "BASELINE configs[4]: indexing / KV-cache stress graph at length 8192"
@@ -684,7 +688,7 @@ def run_graph_suite(args):
     blocks, out = [], {"suite": args.suite, "workload": workload, "modes": {}}
     reference = None
     for mode, fuse in (("fused", True), ("one_kernel_per_node", False)):
-        inst = runtime.Builder.from_graph(graph).build(0, fuse=fuse)
+        inst = runtime.Builder.from_graph(graph).build(0, fuse=fuse, bf16_pieces=fuse and args.bf16_pieces)
         got = inst.run(feeds)                      # first run fills the pool; outputs kept for the check
         if reference is None:
             reference = got

@@ -227,12 +227,13 @@ def _causal_mask_trilu(b: _B, scores_like_q, k_len_source, past_len_1d):
     return b.op("Unsqueeze", [tri, b.i64([0, 1])], "mask4")
 
 
-def decoder_layer_graph(seed=3, seq=2048, cfg: LlamaConfig | None = None):
+def decoder_layer_graph(seed=3, seq=2048, cfg: LlamaConfig | None = None, bf16_values=False):
     """Config 3: one Llama-3.2-1B-shaped decoder layer, prefill at batch 1 (token embeddings
-    ~ N(0,1) are the graph input `x` [1,S,hidden]; no cache)."""
+    ~ N(0,1) are the graph input `x` [1,S,hidden]; no cache). bf16_values: every weight a bfloat16
+    value held as float (see as_bfloat16_values)."""
     cfg = cfg or LlamaConfig()
     rng = np.random.default_rng(seed)
-    w = _weights(rng, cfg, 0)
+    w = _weights(rng, cfg, 0, bf16_values)
     x = rng.standard_normal((1, seq, cfg.hidden), dtype=np.float32)
     b = _B()
     b.g.input("x", FLOAT, [1, 0, cfg.hidden])
