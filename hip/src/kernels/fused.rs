@@ -188,6 +188,35 @@ pub unsafe fn matmul_bf16x3(
     )
 }
 
+/// `outs[i]` (dense `[m, widths[i]]`) `= a . (the next widths[i] rows of wt)^T` over the pieces of
+/// `a`, one launch over the joint matrix. At most 4 members, widths multiples of 32.
+pub unsafe fn matmul_bf16x3_grouped(
+    stream: &HipStream,
+    m: usize,
+    k: usize,
+    pieces: *const c_void,
+    wt: *const c_void,
+    ldw: usize,
+    widths: &[i64],
+    outs: &[*mut c_void],
+) -> Result<()> {
+    assert_eq!(widths.len(), outs.len());
+    check(
+        ffi::rmlk_hip_matmul_bf16x3_grouped(
+            stream.raw(),
+            m as i64,
+            k as i64,
+            pieces,
+            wt,
+            ldw as i64,
+            widths.len() as i32,
+            widths.as_ptr(),
+            outs.as_ptr(),
+        ),
+        "matmul_bf16x3_grouped",
+    )
+}
+
 /// `out[m, n] = swiglu(a . wt[gate_row..+n]^T, a . wt[up_row..+n]^T)` over the pieces of `a`.
 pub unsafe fn matmul_bf16x3_swiglu(
     stream: &HipStream,

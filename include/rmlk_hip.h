@@ -514,6 +514,12 @@ int32_t rmlk_hip_matmul_bf16x3(rmlk_stream_t stream, int64_t m, int64_t n, int64
 int32_t rmlk_hip_matmul_bf16x3_swiglu(rmlk_stream_t stream, int64_t m, int64_t n, int64_t k,
                                       const void *pieces, const void *wt, int64_t ldw, int64_t gate_row,
                                       int64_t up_row, void *out, int64_t ldc);
+/* rmlk_hip_matmul_grouped over the pieces: outs[i] (dense [m, widths[i]]) = a . (the next widths[i]
+ * rows of wt)^T, one launch over the joint matrix whose 32-column blocks go to their member's
+ * output. groups <= 4, every width a multiple of 32, their sum of 128. */
+int32_t rmlk_hip_matmul_bf16x3_grouped(rmlk_stream_t stream, int64_t m, int64_t k, const void *pieces,
+                                       const void *wt, int64_t ldw, int32_t groups, const int64_t *widths,
+                                       void *const *outs);
 
 /* Rotary position embedding, half-rotation form, over x of logical shape [B, H, S, D]:
  * out = x * cos + concat(-x[..., D/2:], x[..., :D/2]) * sin, out dense [B, H, S, D].

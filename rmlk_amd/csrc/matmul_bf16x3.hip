@@ -29,6 +29,7 @@ typedef __attribute__((ext_vector_type(4))) float v4f;
 
 constexpr int kThreads = 256;
 constexpr int kTileRows = 128;   // rows of A per block tile
+constexpr int kMaxGroups = 4;    // members of a grouped product
 
 inline int64_t padded_rows(int64_t m) { return (m + kTileRows - 1) / kTileRows * kTileRows; }
 
@@ -83,6 +84,13 @@ struct X3Args {
     int64_t ldb, ldc, slab;
     int32_t k_per_split, tiles_m, tiles_n, per_xcd;
     int64_t gate_row, up_row;   // SWIGLU: the rows of b that hold the gate and the up weights
+    // Destinations per block of columns (n_seg > 0, one slab): columns [seg_begin[i], seg_begin[i+1])
+    // go to seg_c[i] (leading dimension seg_ldc[i], column 0 = seg_begin[i]); boundaries are
+    // multiples of 32, so a 32-column accumulator block has one destination.
+    int32_t n_seg;
+    int32_t seg_begin[kMaxGroups + 1];
+    float *seg_c[kMaxGroups];
+    int64_t seg_ldc[kMaxGroups];
 };
 
 // Block tile 128 x (64 * TN), four wavefronts (2 x 2) of 64 x (32 * TN). LDS rows are 64 bytes (32
@@ -309,13 +317,28 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16x3_kernel(X3Args g) {
     } else {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const int col = n0 + wn * WN + j * 32 + l32;
+            const int cb = n0 + wn * WN + j * 32;      // first column of this accumulator block
+            float *dst = C;
+            int64_t ldc = g.ldc;
+            int col = cb + l32;
+            if (g.n_seg > 0) {
+                // (constant indices only: the argument struct stays in scalar registers)
+                dst = g.seg_c[0];
+                ldc = g.seg_ldc[0];
+#pragma unroll
+                for (int sgm = 1; sgm < kMaxGroups; ++sgm)
+                    if (sgm < g.n_seg && cb >= g.seg_begin[sgm]) {
+                        dst = g.seg_c[sgm];
+                        ldc = g.seg_ldc[sgm];
+                        col = cb - g.seg_begin[sgm] + l32;
+                    }
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int row = m0 + wm * 64 + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                    if (row < g.m) C[static_cast<int64_t>(row) * g.ldc + col] = acc[i][j][r];
+                    if (row < g.m) dst[static_cast<int64_t>(row) * ldc + col] = acc[i][j][r];
                 }
         }
     }
@@ -351,6 +374,19 @@ int32_t splits_for(int64_t tiles, int64_t k) {
     int32_t s = 1;
     while (s < 8 && tiles * s * 2 <= kNumCU + kNumCU / 4 && k % (64 * s) == 0 && k / (2 * s) >= 256) s *= 2;
     return s;
+}
+
+// The plain product: the tile by how many blocks it makes.
+int32_t launch_plain(hipStream_t st, const X3Args &g, int32_t splits) {
+    const int64_t tiles_m = g.m_pad / kTileRows, n = g.n;
+    const bool wide = n % 256 == 0 && tiles_m * (n / 256) * splits >= kNumCU - kNumCU / 8;
+    if (wide) {
+        // more blocks than compute units: two of them per unit (two stages each) hide more latency
+        // than one with three
+        if (tiles_m * (n / 256) * splits > 2 * kNumCU) return launch_x3<4, 2, false>(st, g, splits);
+        return launch_x3<4, 3, false>(st, g, splits);
+    }
+    return launch_x3<2, 3, false>(st, g, splits);
 }
 
 }  // namespace
@@ -415,15 +451,46 @@ int32_t rmlk_hip_matmul_bf16x3(rmlk_stream_t stream, int64_t m, int64_t n, int64
     g.ldc = ldc;
     g.slab = slab;
     g.k_per_split = static_cast<int32_t>(k / splits);
-    const int64_t tiles_m = g.m_pad / kTileRows;
-    const bool wide = n % 256 == 0 && tiles_m * (n / 256) * splits >= kNumCU - kNumCU / 8;
-    if (wide) {
-        // more blocks than compute units: two of them per unit (two stages each) hide more latency
-        // than one with three
-        if (tiles_m * (n / 256) * splits > 2 * kNumCU) return launch_x3<4, 2, false>(st, g, splits);
-        return launch_x3<4, 3, false>(st, g, splits);
+    return launch_plain(st, g, splits);
+}
+
+int32_t rmlk_hip_matmul_bf16x3_grouped(rmlk_stream_t stream, int64_t m, int64_t k, const void *pieces,
+                                       const void *wt, int64_t ldw, int32_t groups, const int64_t *widths,
+                                       void *const *outs) {
+    hipStream_t st = as_stream(stream);
+    if (m < 0 || k < 0 || groups < 1 || groups > kMaxGroups || !widths || !outs) return RMLK_ERR_INVALID_ARGUMENT;
+    int64_t n = 0;
+    for (int i = 0; i < groups; ++i) {
+        if (widths[i] < 0) return RMLK_ERR_INVALID_ARGUMENT;
+        if (widths[i] % 32 != 0 || widths[i] == 0) return RMLK_ERR_UNSUPPORTED;
+        if (m > 0 && !outs[i]) return RMLK_ERR_NULL_POINTER;
+        n += widths[i];
     }
-    return launch_x3<2, 3, false>(st, g, splits);
+    if (m == 0) return RMLK_OK;
+    if (!pieces || !wt) return RMLK_ERR_NULL_POINTER;
+    if (k == 0 || n % 128 != 0 || n >= ((int64_t)1 << 30) || !operands_ok(m, k, pieces, wt, ldw, n))
+        return RMLK_ERR_UNSUPPORTED;
+    X3Args g{};
+    g.a3 = static_cast<const uint16_t *>(pieces);
+    g.b = static_cast<const uint16_t *>(wt);
+    g.m = static_cast<int32_t>(m);
+    g.n = static_cast<int32_t>(n);
+    g.k = static_cast<int32_t>(k);
+    g.m_pad = static_cast<int32_t>(padded_rows(m));
+    g.ldb = ldw;
+    g.k_per_split = g.k;
+    g.n_seg = groups;
+    int64_t first = 0;
+    for (int i = 0; i < groups; ++i) {
+        g.seg_begin[i] = static_cast<int32_t>(first);
+        g.seg_c[i] = static_cast<float *>(outs[i]);
+        g.seg_ldc[i] = widths[i];
+        first += widths[i];
+    }
+    g.seg_begin[groups] = static_cast<int32_t>(first);
+    g.c = g.seg_c[0];
+    g.ldc = g.seg_ldc[0];
+    return launch_plain(st, g, 1);
 }
 
 int32_t rmlk_hip_matmul_bf16x3_swiglu(rmlk_stream_t stream, int64_t m, int64_t n, int64_t k,

@@ -1946,19 +1946,14 @@ void op_fused_matmul_group(OpContext &c) {
         std::vector<void *> outs;
         for (size_t i = 0; i < widths.size(); ++i)
             outs.push_back(c.alloc_output(static_cast<int>(i), RMLK_FLOAT, out_shape(widths[i])).data());
-        bool as_pieces = wants_pieces(c, m, k, wt.dtype);
-        for (size_t i = 0; as_pieces && i < widths.size(); ++i)
-            as_pieces = rmlk_hip_bf16x3_splits(m, widths[i], k) > 0;
-        if (as_pieces) {
-            // one split of the operand, a product per member over its rows of the joint matrix
-            if (void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroup")) {
-                int64_t first = 0;
-                for (size_t i = 0; i < widths.size(); ++i) {
-                    check_status(rmlk_hip_matmul_bf16x3(c.stream, m, widths[i], k, pieces, rows + first * row_bytes, k, 1,
-                                                        outs[i], widths[i], 0),
-                                 "rmlk.MatMulGroup");
-                    first += widths[i];
-                }
+        if (wants_pieces(c, m, k, wt.dtype) && rmlk_hip_bf16x3_splits(m, total, k) > 0) {
+            // one split of the operand, one product over the joint matrix whose column blocks go to
+            // the members' outputs
+            void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroup");
+            if (pieces && took_fast_path(rmlk_hip_matmul_bf16x3_grouped(c.stream, m, k, pieces, wt.data(), k,
+                                                                        static_cast<int32_t>(widths.size()),
+                                                                        widths.data(), outs.data()),
+                                         "rmlk.MatMulGroup")) {
                 ++c.session.products_bf16_pieces;
                 return;
             }

@@ -389,6 +389,15 @@ def matmul_bf16x3(pieces, wt, out, m: int, n: int, k: int, splits: int = 1) -> N
           "rmlk_hip_matmul_bf16x3")
 
 
+def matmul_bf16x3_grouped(pieces, wt, outs, m: int, k: int, widths) -> None:
+    """outs[i] [m, widths[i]] = a . (the next widths[i] rows of wt)^T over the pieces of a, one launch."""
+    assert wt.dtype == torch.bfloat16 and len(outs) == len(widths)
+    w = (ctypes.c_int64 * len(widths))(*widths)
+    o = (ctypes.c_void_p * len(outs))(*[_ptr(t) for t in outs])
+    check(lib().rmlk_hip_matmul_bf16x3_grouped(_stream(), m, k, _ptr(pieces), _ptr(wt), k, len(widths), w, o),
+          "rmlk_hip_matmul_bf16x3_grouped")
+
+
 def matmul_bf16x3_swiglu(pieces, wt, out, m: int, n: int, k: int, gate_row: int, up_row: int) -> None:
     """out[m, n] = swiglu(a . wt[gate_row:+n]^T, a . wt[up_row:+n]^T) over the pieces of a."""
     assert wt.dtype == torch.bfloat16

@@ -173,6 +173,43 @@ def test_swiglu_form_equals_the_two_products_and_the_activation(device, m, n, k,
     assert_close(to_np(got), exp64.astype(np.float32), rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("m,k,widths", [(300, 256, (2048, 512, 512)), (64, 64, (96, 32)), (2048, 128, (256,)),
+                                        (130, 96, (32, 32, 32, 160))])
+def test_grouped_product_sends_column_blocks_to_their_members(device, m, k, widths):
+    """One launch over the joint matrix [sum(widths), k]; every member's output equals the plain
+    product over its rows of the matrix bit for bit (same K order), small integers exactly."""
+    import torch
+    from rmlk_amd._lib import RmlkError
+    kk = _k()
+    rng = np.random.default_rng(sum(widths) + m)
+    n = sum(widths)
+    a = rng.integers(-8, 9, size=(m, k)).astype(np.float32)
+    w = rng.integers(-4, 5, size=(n, k)).astype(np.float32)
+    a_d, w_d = to_dev(a, device), _bf16_weights(w, device)
+    pieces = kk.bf16x3_split(a_d)
+    outs = [torch.full((m, wd), np.nan, dtype=torch.float32, device=device) for wd in widths]
+    kk.matmul_bf16x3_grouped(pieces, w_d, outs, m, k, list(widths))
+    first = 0
+    for wd, out in zip(widths, outs):
+        exp = a.astype(np.float64) @ w[first:first + wd].astype(np.float64).T
+        assert np.array_equal(to_np(out).astype(np.float64), exp), (first, wd)
+        first += wd
+    # full-mantissa operands: the joint launch against the plain product over the joint matrix
+    a_d = to_dev(rng.standard_normal((m, k)).astype(np.float32), device)
+    w_d = _bf16_weights(rng.standard_normal((n, k)) * 0.05, device)
+    pieces = kk.bf16x3_split(a_d)
+    kk.matmul_bf16x3_grouped(pieces, w_d, outs, m, k, list(widths))
+    whole = torch.zeros((m, n), dtype=torch.float32, device=device)
+    kk.matmul_bf16x3(pieces, w_d, whole, m, n, k)
+    first = 0
+    for wd, out in zip(widths, outs):
+        assert_exact(to_np(out), to_np(whole[:, first:first + wd].contiguous()))
+        first += wd
+    with pytest.raises(RmlkError) as e:       # a boundary inside a 32-column block
+        kk.matmul_bf16x3_grouped(pieces, w_d, outs[:1] * 2, m, k, [48, n - 48])
+    assert e.value.status == -2
+
+
 def test_infinities_and_nans_arrive_as_from_an_fp32_product(device):
     import torch
     kk = _k()
