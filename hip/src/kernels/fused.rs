@@ -146,6 +146,43 @@ pub unsafe fn bf16x3_split(
     check(ffi::rmlk_hip_bf16x3_split(stream.raw(), m as i64, k as i64, a, lda as i64, pieces), "bf16x3_split")
 }
 
+/// RMSNorm (over `partials[0] + .. + partials[splits-1]`, plus `b` when given, the formed rows then
+/// also stored to `sum_out`) whose result goes to `out` and, as by `bf16x3_split`, to `pieces`.
+pub unsafe fn rmsnorm_pieces(
+    stream: &HipStream,
+    rows: usize,
+    cols: usize,
+    partials: *const c_void,
+    splits: usize,
+    slab: usize,
+    b: *const c_void,
+    gamma: *const c_void,
+    eps: f32,
+    reciprocal_form: bool,
+    sum_out: *mut c_void,
+    out: *mut c_void,
+    pieces: *mut c_void,
+) -> Result<()> {
+    check(
+        ffi::rmlk_hip_rmsnorm_pieces(
+            stream.raw(),
+            rows as i64,
+            cols as i64,
+            partials,
+            splits as i32,
+            slab as i64,
+            b,
+            gamma,
+            eps,
+            reciprocal_form as i32,
+            sum_out,
+            out,
+            pieces,
+        ),
+        "rmsnorm_pieces",
+    )
+}
+
 /// Slabs of K with which `matmul_bf16x3` fills the GPU for a size; `None`: a size it does not take.
 pub fn bf16x3_splits(m: usize, n: usize, k: usize) -> Option<usize> {
     match unsafe { ffi::rmlk_hip_bf16x3_splits(m as i64, n as i64, k as i64) } {

@@ -514,6 +514,14 @@ int32_t rmlk_hip_matmul_bf16x3(rmlk_stream_t stream, int64_t m, int64_t n, int64
 int32_t rmlk_hip_matmul_bf16x3_swiglu(rmlk_stream_t stream, int64_t m, int64_t n, int64_t k,
                                       const void *pieces, const void *wt, int64_t ldw, int64_t gate_row,
                                       int64_t up_row, void *out, int64_t ldc);
+/* rmlk_hip_rmsnorm / rmlk_hip_add_rmsnorm / rmlk_hip_splitk_add_rmsnorm (b NULL: no Add, sum_out
+ * unused; splits == 1: `partials` is the row matrix itself) whose result goes to `out` AND, split
+ * as by rmlk_hip_bf16x3_split, to `pieces` (rmlk_hip_bf16x3_pieces_size(rows, cols) bytes; the
+ * padding rows are left as they are: no row of a product depends on them): a norm in front of a
+ * product over the pieces needs no split launch. cols % 8 == 0. */
+int32_t rmlk_hip_rmsnorm_pieces(rmlk_stream_t stream, int64_t rows, int64_t cols, const void *partials,
+                                int32_t splits, int64_t slab, const void *b, const void *gamma, float eps,
+                                int32_t reciprocal_form, void *sum_out, void *out, void *pieces);
 /* rmlk_hip_matmul_grouped over the pieces: outs[i] (dense [m, widths[i]]) = a . (the next widths[i]
  * rows of wt)^T, one launch over the joint matrix whose 32-column blocks go to their member's
  * output. groups <= 4, every width a multiple of 32, their sum of 128. */

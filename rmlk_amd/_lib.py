@@ -122,6 +122,8 @@ SIGNATURES = {
     "rmlk_hip_bf16x3_splits": (c_int32, [c_int64, c_int64, c_int64]),
     "rmlk_hip_matmul_bf16x3": (c_int32, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int64,
                                          c_int32, c_void_p, c_int64, c_int64]),
+    "rmlk_hip_rmsnorm_pieces": (c_int32, [c_void_p, c_int64, c_int64, c_void_p, c_int32, c_int64, c_void_p, c_void_p,
+                                          ctypes.c_float, c_int32, c_void_p, c_void_p, c_void_p]),
     "rmlk_hip_matmul_bf16x3_grouped": (c_int32, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int32,
                                                  POINTER(c_int64), POINTER(c_void_p)]),
     "rmlk_hip_matmul_bf16x3_swiglu": (c_int32, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p,

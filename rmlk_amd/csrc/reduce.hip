@@ -365,6 +365,11 @@ struct RmsSource {
     float *sum_out;       // where the formed row goes (null: nowhere)
     int32_t slabs;        // x is the first of this many partial matrices (split-K), summed in order
     int64_t slab;         // elements from one partial matrix to the next
+    // The result also as three bfloat16 pieces whose sum it is exactly (hi, mid, lo: truncate,
+    // subtract, truncate, subtract; Inf / NaN in hi alone), the operand form of rmlk_hip_matmul_bf16x3:
+    // planes of `plane` elements each, rows of `cols`. Null: not wanted.
+    uint16_t *pieces;
+    int64_t plane;
 };
 
 template <int NV, int kGroup, bool RECIP>
@@ -471,6 +476,27 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(RmsSource src,
                     y.v[j] = normed * g[i].v[j];
                 }
                 nt_store(po + c, y);
+                if (src.pieces) {
+                    uint32_t hi[4], mid[4], lo[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t xb = __float_as_uint(y.v[j]);
+                        const uint32_t hb = xb & 0xffff0000u;
+                        const bool finite = (xb & 0x7f800000u) != 0x7f800000u;
+                        const float r1 = finite ? y.v[j] - __uint_as_float(hb) : 0.f;
+                        const uint32_t mb = __float_as_uint(r1) & 0xffff0000u;
+                        const float r2 = r1 - __uint_as_float(mb);
+                        hi[j] = hb >> 16;
+                        mid[j] = mb >> 16;
+                        lo[j] = __float_as_uint(r2) >> 16;
+                    }
+                    uint16_t *pp = src.pieces + row * cols + c * 4;
+                    *reinterpret_cast<uint2 *>(pp) = uint2{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16)};
+                    *reinterpret_cast<uint2 *>(pp + src.plane) =
+                        uint2{mid[0] | (mid[1] << 16), mid[2] | (mid[3] << 16)};
+                    *reinterpret_cast<uint2 *>(pp + 2 * src.plane) =
+                        uint2{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16)};
+                }
             }
         }
     }
@@ -636,7 +662,7 @@ extern "C" int32_t rmlk_hip_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t
     if (rows == 0 || cols == 0) return RMLK_OK;
     if (!x || !gamma || !out) return RMLK_ERR_NULL_POINTER;
     if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
-    RmsSource src{static_cast<const float *>(x), nullptr, nullptr, 1, 0};
+    RmsSource src{static_cast<const float *>(x), nullptr, nullptr, 1, 0, nullptr, 0};
     return rmsnorm_dispatch(as_stream(stream), src, static_cast<const float *>(gamma),
                             static_cast<float *>(out), rows, cols, eps, reciprocal_form != 0);
 }
@@ -651,7 +677,7 @@ extern "C" int32_t rmlk_hip_add_rmsnorm(rmlk_stream_t stream, int32_t dtype, int
     if (!a || !b || !gamma || !sum_out || !out) return RMLK_ERR_NULL_POINTER;
     if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
     RmsSource src{static_cast<const float *>(a), static_cast<const float *>(b),
-                  static_cast<float *>(sum_out), 1, 0};
+                  static_cast<float *>(sum_out), 1, 0, nullptr, 0};
     return rmsnorm_dispatch(as_stream(stream), src, static_cast<const float *>(gamma),
                             static_cast<float *>(out), rows, cols, eps, reciprocal_form != 0);
 }
@@ -668,7 +694,25 @@ extern "C" int32_t rmlk_hip_splitk_add_rmsnorm(rmlk_stream_t stream, int32_t dty
     if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
     if (splits > 1 && (slab < rows * cols || slab % 4 != 0)) return RMLK_ERR_SIZE_MISMATCH;
     RmsSource src{static_cast<const float *>(partials), static_cast<const float *>(b),
-                  static_cast<float *>(sum_out), splits, slab};
+                  static_cast<float *>(sum_out), splits, slab, nullptr, 0};
+    return rmsnorm_dispatch(as_stream(stream), src, static_cast<const float *>(gamma),
+                            static_cast<float *>(out), rows, cols, eps, reciprocal_form != 0);
+}
+
+extern "C" int32_t rmlk_hip_rmsnorm_pieces(rmlk_stream_t stream, int64_t rows, int64_t cols,
+                                           const void *partials, int32_t splits, int64_t slab, const void *b,
+                                           const void *gamma, float eps, int32_t reciprocal_form,
+                                           void *sum_out, void *out, void *pieces) {
+    if (rows < 0 || cols < 0 || splits < 1 || slab < 0) return RMLK_ERR_INVALID_ARGUMENT;
+    if (rows == 0 || cols == 0) return RMLK_OK;
+    if (!partials || !gamma || !out || !pieces || (b && !sum_out)) return RMLK_ERR_NULL_POINTER;
+    if (rows > kMaxElems / cols) return RMLK_ERR_TOO_LARGE;
+    if (splits > 1 && (slab < rows * cols || slab % 4 != 0)) return RMLK_ERR_SIZE_MISMATCH;
+    if (cols % 8 != 0 || reinterpret_cast<uintptr_t>(pieces) % 16 != 0) return RMLK_ERR_UNSUPPORTED;
+    const int64_t m_pad = (rows + 127) / 128 * 128;      // (the planes of rmlk_hip_bf16x3_split)
+    RmsSource src{static_cast<const float *>(partials), static_cast<const float *>(b),
+                  b ? static_cast<float *>(sum_out) : nullptr, splits, slab,
+                  static_cast<uint16_t *>(pieces), m_pad * cols};
     return rmsnorm_dispatch(as_stream(stream), src, static_cast<const float *>(gamma),
                             static_cast<float *>(out), rows, cols, eps, reciprocal_form != 0);
 }

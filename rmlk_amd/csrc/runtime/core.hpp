@@ -107,6 +107,10 @@ struct Tensor {
     // that everything that reads them is one row-stream node, which either runs the product and
     // its own work as one launch or has the product computed first.
     std::shared_ptr<PendingProduct> pending_product;
+    // Set on the result of a many-row norm whose one reader is a product over bfloat16 weights on the
+    // bf16 matrix cores: the same rows as three bfloat16 pieces (the planes rmlk_hip_bf16x3_split would
+    // write), stored by the norm kernel itself.
+    std::shared_ptr<const Tensor> pieces;
 
     bool defined() const { return dtype != 0; }
     int64_t numel() const {
@@ -125,6 +129,7 @@ struct Tensor {
         host.reset();
         pending_norm.reset();
         pending_product.reset();
+        pieces.reset();
     }
 };
 

@@ -1004,14 +1004,36 @@ bool wants_pieces(const OpContext &c, int64_t m, int64_t k, int32_t w_dtype) {
 }
 
 // Splits a [m, k] (dense rows); returns the pieces, null when the split does not take the operand.
-// *own_out: the caller's part of the workspace.
+// *own_out: the caller's part of the workspace. `src`: the tensor a belongs to, which may carry its
+// pieces already (a norm that stored them for this reader).
 void *split_pieces(OpContext &c, const void *a, int64_t m, int64_t k, size_t own, void **own_out,
-                   const char *what) {
+                   const char *what, const Tensor *src = nullptr) {
+    if (src && src->pieces && src->data() == a && src->pieces->nbytes() == rmlk_hip_bf16x3_pieces_size(m, k)) {
+        if (own_out) *own_out = own ? c.scratch(own) : nullptr;
+        return src->pieces->data();
+    }
     const size_t own_bytes = (own + 255) / 256 * 256;
     char *ws = static_cast<char *>(c.scratch(own_bytes + rmlk_hip_bf16x3_pieces_size(m, k)));
     if (own_out) *own_out = ws;
     void *pieces = ws + own_bytes;
     return took_fast_path(rmlk_hip_bf16x3_split(c.stream, m, k, a, k, pieces), what) ? pieces : nullptr;
+}
+
+// A many-row norm whose result has one reader, a product (the `defer_norm` mark of the fusion pass),
+// in a session that multiplies over bfloat16 weights on the bf16 matrix cores: room for the pieces of
+// its [rows, cols] result, which the norm kernel then writes itself. Undefined when not wanted.
+Tensor room_for_pieces(OpContext &c, int64_t rows, int64_t cols) {
+    Tensor t;
+    if (!c.session.bf16_pieces || c.session.weights_16bit == 0 || c.attr_int("defer_norm", 0) == 0 || rows < 64 ||
+        cols % 32 != 0)
+        return t;
+    const size_t bytes = rmlk_hip_bf16x3_pieces_size(rows, cols);
+    if (bytes >= (static_cast<size_t>(1) << 32)) return t;
+    std::vector<Tensor *> keep = c.out;
+    c.out = {&t};
+    c.alloc_output(0, RMLK_UINT8, {static_cast<int64_t>(bytes)});
+    c.out = keep;
+    return t;
 }
 
 // ---- one-row RMSNorm left to the product that reads it ------------------------------------------
@@ -1137,6 +1159,16 @@ void op_fused_rmsnorm(OpContext &c) {
     if (ok) {
         const int64_t cols = x.shape.back(), rows = x.numel() / cols;
         Tensor &y = c.alloc_output(0, RMLK_FLOAT, x.shape);
+        if (Tensor pieces = room_for_pieces(c, rows, cols); pieces.defined()) {
+            if (took_fast_path(rmlk_hip_rmsnorm_pieces(c.stream, rows, cols, x.data(), 1, 0, nullptr, gamma.data(),
+                                                       attr_float(c, "epsilon"),
+                                                       static_cast<int32_t>(c.attr_int("reciprocal", 0)), nullptr,
+                                                       y.data(), pieces.data()),
+                               "rmlk.RMSNorm")) {
+                y.pieces = std::make_shared<const Tensor>(std::move(pieces));
+                return;
+            }
+        }
         if (took_fast_path(rmlk_hip_rmsnorm(c.stream, RMLK_FLOAT, rows, cols, x.data(), gamma.data(),
                                             attr_float(c, "epsilon"),
                                             static_cast<int32_t>(c.attr_int("reciprocal", 0)),
@@ -1645,13 +1677,24 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
         const int32_t splits = rmlk_hip_bf16x3_splits(m, n, k);
         void *slabs = nullptr;
         void *pieces = splits > 0 ? split_pieces(c, a.data(), m, k, static_cast<size_t>(splits) * m * n * sizeof(float),
-                                                 &slabs, "rmlk.MatMulAddRMSNorm")
+                                                 &slabs, "rmlk.MatMulAddRMSNorm", &a)
                                   : nullptr;
         if (pieces && took_fast_path(rmlk_hip_matmul_bf16x3(c.stream, m, n, k, pieces, wt.data(), k, splits, slabs, n,
                                                             m * n),
                                      "rmlk.MatMulAddRMSNorm")) {
             Tensor &sum = c.alloc_output(0, RMLK_FLOAT, res.shape);
             Tensor &y = c.alloc_output(1, RMLK_FLOAT, res.shape);
+            if (Tensor normed = room_for_pieces(c, m, n); normed.defined()) {
+                if (took_fast_path(rmlk_hip_rmsnorm_pieces(c.stream, m, n, slabs, splits, m * n, res.data(), gamma.data(),
+                                                           attr_float(c, "epsilon"),
+                                                           static_cast<int32_t>(c.attr_int("reciprocal", 0)),
+                                                           sum.data(), y.data(), normed.data()),
+                                   "rmlk.MatMulAddRMSNorm")) {
+                    y.pieces = std::make_shared<const Tensor>(std::move(normed));
+                    ++c.session.products_bf16_pieces;
+                    return;
+                }
+            }
             if (took_fast_path(rmlk_hip_splitk_add_rmsnorm(c.stream, RMLK_FLOAT, m, n, slabs, splits, m * n, res.data(),
                                                            gamma.data(), attr_float(c, "epsilon"),
                                                            static_cast<int32_t>(c.attr_int("reciprocal", 0)),
@@ -1689,9 +1732,9 @@ void op_fused_matmul_add_rmsnorm(OpContext &c) {
 // (`wt`: n rows of k), into the dense [m, n] at `out`.
 // `w_dtype`: how the weights are stored (float, or the 16-bit type the session was built with).
 void product_over_kmajor(OpContext &c, const void *a, int64_t m, int64_t k, int32_t w_dtype, const void *wt,
-                         int64_t n, void *out, const char *what) {
+                         int64_t n, void *out, const char *what, const Tensor *a_tensor = nullptr) {
     if (wants_pieces(c, m, k, w_dtype) && rmlk_hip_bf16x3_splits(m, n, k) > 0) {
-        void *pieces = split_pieces(c, a, m, k, 0, nullptr, what);
+        void *pieces = split_pieces(c, a, m, k, 0, nullptr, what, a_tensor);
         if (pieces && took_fast_path(rmlk_hip_matmul_bf16x3(c.stream, m, n, k, pieces, wt, k, 1, out, n, 0), what)) {
             ++c.session.products_bf16_pieces;
             return;
@@ -1748,7 +1791,7 @@ void op_fused_matmul_const(OpContext &c) {
             return;
     }
     if (c.input(0).pending_norm) compute_pending_norm(c);
-    product_over_kmajor(c, c.input(0).data(), m, k, wt.dtype, wt.data(), n, y.data(), "rmlk.MatMulConst");
+    product_over_kmajor(c, c.input(0).data(), m, k, wt.dtype, wt.data(), n, y.data(), "rmlk.MatMulConst", &c.input(0));
 }
 
 // swiglu(a . Wg, a . Wu) with [Wg | Wu] constant and stored K-contiguous as one matrix (wt [2 n, k]).
@@ -1785,7 +1828,7 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
         shape.push_back(n);
         Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
         if (wants_pieces(c, m, k, wt.dtype)) {
-            void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroupSwiGLU");
+            void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroupSwiGLU", &a);
             if (pieces && took_fast_path(rmlk_hip_matmul_bf16x3_swiglu(c.stream, m, n, k, pieces, wt.data(), k,
                                                                        gate_first ? 0 : n, gate_first ? n : 0,
                                                                        y.data(), n),
@@ -1905,7 +1948,7 @@ void op_fused_matmul_group(OpContext &c) {
             int32_t splits = 0;
             bool multiplied = false;
             if (x3_splits > 0) {
-                void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroup");
+                void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroup", &a);
                 multiplied = pieces && took_fast_path(rmlk_hip_matmul_bf16x3(c.stream, m, total, k, pieces, wt.data(), k,
                                                                              x3_splits, pp->slabs.data(), total,
                                                                              m * total),
@@ -1949,7 +1992,7 @@ void op_fused_matmul_group(OpContext &c) {
         if (wants_pieces(c, m, k, wt.dtype) && rmlk_hip_bf16x3_splits(m, total, k) > 0) {
             // one split of the operand, one product over the joint matrix whose column blocks go to
             // the members' outputs
-            void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroup");
+            void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroup", &a);
             if (pieces && took_fast_path(rmlk_hip_matmul_bf16x3_grouped(c.stream, m, k, pieces, wt.data(), k,
                                                                         static_cast<int32_t>(widths.size()),
                                                                         widths.data(), outs.data()),

@@ -376,6 +376,18 @@ def bf16x3_split(a: torch.Tensor) -> torch.Tensor:
     return pieces
 
 
+def rmsnorm_pieces(x, gamma, eps: float, out, pieces, add=None, sum_out=None, splits: int = 1,
+                   reciprocal_form: bool = False) -> None:
+    """RMSNorm of the rows of x [rows, cols] (of x[0] + .. + x[splits-1] for x [splits, rows, cols]; plus
+    `add`, the formed rows then also stored to sum_out) into out and, as three bfloat16 pieces, into
+    `pieces` (the tensor bf16x3_split would return)."""
+    rows, cols = out.shape
+    check(lib().rmlk_hip_rmsnorm_pieces(_stream(), rows, cols, _ptr(x), splits, rows * cols,
+                                        _ptr(add) if add is not None else None, _ptr(gamma), eps,
+                                        int(reciprocal_form), _ptr(sum_out) if sum_out is not None else None,
+                                        _ptr(out), _ptr(pieces)), "rmlk_hip_rmsnorm_pieces")
+
+
 def bf16x3_splits(m: int, n: int, k: int) -> int:
     """Slabs of K with which matmul_bf16x3 fills the GPU for this size; 0: a size it does not take."""
     return int(lib().rmlk_hip_bf16x3_splits(m, n, k))

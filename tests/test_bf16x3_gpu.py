@@ -210,6 +210,36 @@ def test_grouped_product_sends_column_blocks_to_their_members(device, m, k, widt
     assert e.value.status == -2
 
 
+@pytest.mark.parametrize("rows,cols,splits,with_add", [(512, 2048, 4, True), (70, 256, 1, False), (130, 8192, 2, True),
+                                                        (2048, 512, 1, True)])
+def test_norm_that_stores_its_result_as_pieces(device, rows, cols, splits, with_add):
+    """rmlk_hip_rmsnorm_pieces: `out` and `sum_out` are the bits of the norm entry points, and the
+    pieces are those that rmlk_hip_bf16x3_split makes of `out` (padding rows aside)."""
+    import torch
+    kk = _k()
+    rng = np.random.default_rng(rows + cols)
+    x = to_dev(rng.standard_normal((splits, rows, cols)).astype(np.float32), device)
+    add = to_dev(rng.standard_normal((rows, cols)).astype(np.float32), device) if with_add else None
+    gamma = to_dev((1 + 0.1 * rng.standard_normal(cols)).astype(np.float32), device)
+    out, exp = torch.zeros((rows, cols), device=device), torch.zeros((rows, cols), device=device)
+    total, exp_total = torch.zeros((rows, cols), device=device), torch.zeros((rows, cols), device=device)
+    m_pad = (rows + 127) // 128 * 128
+    pieces = torch.zeros(3 * m_pad * cols, dtype=torch.int16, device=device)
+    kk.rmsnorm_pieces(x, gamma, 1e-5, out, pieces, add=add, sum_out=total if with_add else None, splits=splits)
+    if with_add:
+        from rmlk_amd._lib import check, lib
+        check(lib().rmlk_hip_splitk_add_rmsnorm(torch.cuda.current_stream().cuda_stream, kk.FLOAT, rows, cols,
+                                                x.data_ptr(), splits, rows * cols, add.data_ptr(), gamma.data_ptr(),
+                                                1e-5, 0, exp_total.data_ptr(), exp.data_ptr()),
+              "rmlk_hip_splitk_add_rmsnorm")
+        assert_exact(to_np(total), to_np(exp_total))
+    else:
+        kk.rmsnorm(x[0], gamma, exp, rows, cols, 1e-5)
+    assert_exact(to_np(out), to_np(exp))
+    want = kk.bf16x3_split(exp).reshape(3, m_pad, cols)[:, :rows]
+    assert torch.equal(pieces.reshape(3, m_pad, cols)[:, :rows], want)
+
+
 def test_infinities_and_nans_arrive_as_from_an_fp32_product(device):
     import torch
     kk = _k()
