@@ -195,11 +195,13 @@ def test_llama_tiny_scatter_style_equals_concat_style(device):
 
 
 @pytest.mark.timeout(900)
-@pytest.mark.parametrize("bf16_values", [False, True])
-def test_llama_1b_full_size_prefill_and_teacher_forced_decode(device, bf16_values):
+@pytest.mark.parametrize("bf16_values,bf16_pieces", [(False, False), (True, False), (True, True)])
+def test_llama_1b_full_size_prefill_and_teacher_forced_decode(device, bf16_values, bf16_pieces):
     """(bf16_values: the same graph with weights that are bfloat16 values held as floats, which the
     session stores in 16 bits by itself: the products over stored weights at the full widths -
-    lm-head over 128256 rows, gate / up / down at 8192 - against the oracle on the same graph.)
+    lm-head over 128256 rows, gate / up / down at 8192 - against the oracle on the same graph.
+    bf16_pieces: the prefill's products on the bf16 matrix cores, the fp32 operand as three exact
+    bfloat16 pieces - every one of the 65 products, none of the decode steps'.)
 
     BASELINE configs[3] at its full size: 16 layers, hidden 2048, vocab 128256. Prefill of a
     512-token prompt, then 8 decode steps through the recorded HIP graph with the caches fed back on
@@ -217,12 +219,13 @@ def test_llama_1b_full_size_prefill_and_teacher_forced_decode(device, bf16_value
     prompt = rng.integers(0, cfg.vocab, size=prompt_len)
     zeros = {f"cache.{l}.{kv}": np.zeros((1, cfg.kv_heads, max_len, cfg.head_dim), np.float32)
              for l in range(cfg.layers) for kv in ("key", "value")}
-    inst = runtime.Builder.from_graph(graph).build()
+    inst = runtime.Builder.from_graph(graph).build(bf16_pieces=bf16_pieces)
     assert inst.weights_16bit == (4 * cfg.layers + 1 if bf16_values else 0)
     feeds = _scatter_feeds(cfg, prompt, 0, zeros)
     for name, arr in feeds.items():
         inst.set_input(name, arr)
     inst.execute()
+    assert inst.products_bf16_pieces == (4 * cfg.layers + 1 if bf16_pieces else 0)
     got = inst.output("logits")[0, -1].copy()
     exp = og.run_graph(graph, feeds, matmul_accumulate="f32")
     pos = prompt_len
@@ -249,6 +252,7 @@ def test_llama_1b_full_size_prefill_and_teacher_forced_decode(device, bf16_value
         got = inst.output("logits")[0, -1].copy()
         pos += 1
     assert inst.memory_stats()["device_syncs"] == 0
+    assert inst.products_bf16_pieces == 0      # (one-row products stream their weights as before)
     inst.close()
 
 
