@@ -254,7 +254,8 @@ pub unsafe fn matmul_bf16x3_grouped(
     )
 }
 
-/// `out[m, n] = swiglu(a . wt[gate_row..+n]^T, a . wt[up_row..+n]^T)` over the pieces of `a`.
+/// `out[m, n] = swiglu(a . wt[gate_row..+n]^T, a . wt[up_row..+n]^T)` over the pieces of `a`;
+/// `out_pieces` (null: not wanted): where the same launch also stores the pieces of `out`.
 pub unsafe fn matmul_bf16x3_swiglu(
     stream: &HipStream,
     m: usize,
@@ -267,6 +268,7 @@ pub unsafe fn matmul_bf16x3_swiglu(
     up_row: usize,
     out: *mut c_void,
     ldc: usize,
+    out_pieces: *mut c_void,
 ) -> Result<()> {
     check(
         ffi::rmlk_hip_matmul_bf16x3_swiglu(
@@ -281,6 +283,7 @@ pub unsafe fn matmul_bf16x3_swiglu(
             up_row as i64,
             out,
             ldc as i64,
+            out_pieces,
         ),
         "matmul_bf16x3_swiglu",
     )

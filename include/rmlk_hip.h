@@ -501,7 +501,9 @@ int32_t rmlk_hip_splitk_add_rmsnorm(rmlk_stream_t stream, int32_t dtype, int64_t
  * that adds the slabs up itself (rmlk_hip_splitk_add_rmsnorm, rmlk_hip_head_rows).
  * rmlk_hip_bf16x3_splits is the number of slabs that fills the GPU for a size (1 for wide products;
  * 0 for sizes the kernel does not take). rmlk_hip_matmul_bf16x3_swiglu is rmlk_hip_matmul_swiglu over
- * the pieces: out[m, n] = swiglu(a . wt[gate_row .. +n]^T, a . wt[up_row .. +n]^T).
+ * the pieces: out[m, n] = swiglu(a . wt[gate_row .. +n]^T, a . wt[up_row .. +n]^T); with out_pieces
+ * (NULL: not wanted; else rmlk_hip_bf16x3_pieces_size(m, n) bytes) the same launch also stores the
+ * pieces of out, as rmlk_hip_bf16x3_split would, for a product that reads it.
  * Covered: k % 32 == 0 (per slab), n % 128 == 0 (swiglu: n % 64 == 0), ldw % 8 == 0, operands below
  * 4 GiB; RMLK_ERR_UNSUPPORTED otherwise. */
 size_t rmlk_hip_bf16x3_pieces_size(int64_t m, int64_t k);
@@ -513,7 +515,7 @@ int32_t rmlk_hip_matmul_bf16x3(rmlk_stream_t stream, int64_t m, int64_t n, int64
                                int64_t slab);
 int32_t rmlk_hip_matmul_bf16x3_swiglu(rmlk_stream_t stream, int64_t m, int64_t n, int64_t k,
                                       const void *pieces, const void *wt, int64_t ldw, int64_t gate_row,
-                                      int64_t up_row, void *out, int64_t ldc);
+                                      int64_t up_row, void *out, int64_t ldc, void *out_pieces);
 /* rmlk_hip_rmsnorm / rmlk_hip_add_rmsnorm / rmlk_hip_splitk_add_rmsnorm (b NULL: no Add, sum_out
  * unused; splits == 1: `partials` is the row matrix itself) whose result goes to `out` AND, split
  * as by rmlk_hip_bf16x3_split, to `pieces` (rmlk_hip_bf16x3_pieces_size(rows, cols) bytes; the

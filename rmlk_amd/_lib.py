@@ -127,7 +127,7 @@ SIGNATURES = {
     "rmlk_hip_matmul_bf16x3_grouped": (c_int32, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int32,
                                                  POINTER(c_int64), POINTER(c_void_p)]),
     "rmlk_hip_matmul_bf16x3_swiglu": (c_int32, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p,
-                                                c_int64, c_int64, c_int64, c_void_p, c_int64]),
+                                                c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p]),
     "rmlk_hip_store_weights": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
     "rmlk_hip_weights_fit": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
     "rmlk_hip_gemv_kmajor": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_int32, c_void_p,

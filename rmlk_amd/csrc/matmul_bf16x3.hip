@@ -87,6 +87,10 @@ struct X3Args {
     // Destinations per block of columns (n_seg > 0, one slab): columns [seg_begin[i], seg_begin[i+1])
     // go to seg_c[i] (leading dimension seg_ldc[i], column 0 = seg_begin[i]); boundaries are
     // multiples of 32, so a 32-column accumulator block has one destination.
+    // SWIGLU: the result also as three bfloat16 pieces (planes of `act_plane` elements, rows of n), for
+    // a product that reads it; null: not wanted
+    uint16_t *act_pieces;
+    int64_t act_plane;
     int32_t n_seg;
     int32_t seg_begin[kMaxGroups + 1];
     float *seg_c[kMaxGroups];
@@ -311,7 +315,22 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16x3_kernel(X3Args g) {
                     const int row = m0 + wm * 64 + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
                     const float gate = acc[i][j][r];
                     const float silu = gate * (1.0f / (1.0f + expf(-gate)));
-                    if (row < g.m) C[static_cast<int64_t>(row) * g.ldc + col] = silu * acc[i][j + TN / 2][r];
+                    const float act = silu * acc[i][j + TN / 2][r];
+                    if (row < g.m) {
+                        C[static_cast<int64_t>(row) * g.ldc + col] = act;
+                        if (g.act_pieces) {
+                            const uint32_t xb = __float_as_uint(act);
+                            const uint32_t hb = xb & 0xffff0000u;
+                            const bool finite = (xb & 0x7f800000u) != 0x7f800000u;
+                            const float r1 = finite ? act - __uint_as_float(hb) : 0.f;
+                            const uint32_t mb = __float_as_uint(r1) & 0xffff0000u;
+                            const float r2 = r1 - __uint_as_float(mb);
+                            uint16_t *pp = g.act_pieces + static_cast<int64_t>(row) * g.n + col;
+                            pp[0] = static_cast<uint16_t>(hb >> 16);
+                            pp[g.act_plane] = static_cast<uint16_t>(mb >> 16);
+                            pp[2 * g.act_plane] = static_cast<uint16_t>(__float_as_uint(r2) >> 16);
+                        }
+                    }
                 }
         }
     } else {
@@ -495,7 +514,7 @@ int32_t rmlk_hip_matmul_bf16x3_grouped(rmlk_stream_t stream, int64_t m, int64_t 
 
 int32_t rmlk_hip_matmul_bf16x3_swiglu(rmlk_stream_t stream, int64_t m, int64_t n, int64_t k,
                                       const void *pieces, const void *wt, int64_t ldw, int64_t gate_row,
-                                      int64_t up_row, void *out, int64_t ldc) {
+                                      int64_t up_row, void *out, int64_t ldc, void *out_pieces) {
     hipStream_t st = as_stream(stream);
     if (m < 0 || n < 0 || k < 0 || gate_row < 0 || up_row < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (m == 0 || n == 0) return RMLK_OK;
@@ -517,6 +536,11 @@ int32_t rmlk_hip_matmul_bf16x3_swiglu(rmlk_stream_t stream, int64_t m, int64_t n
     g.k_per_split = g.k;
     g.gate_row = gate_row;
     g.up_row = up_row;
+    if (out_pieces) {
+        if (n % 8 != 0 || reinterpret_cast<uintptr_t>(out_pieces) % 16 != 0) return RMLK_ERR_UNSUPPORTED;
+        g.act_pieces = static_cast<uint16_t *>(out_pieces);
+        g.act_plane = static_cast<int64_t>(g.m_pad) * n;
+    }
     const int64_t tiles_m = g.m_pad / kTileRows;
     if (n % 128 == 0 && tiles_m * (n / 128) >= kNumCU - kNumCU / 8) {
         if (tiles_m * (n / 128) > 2 * kNumCU) return launch_x3<4, 2, true>(st, g, 1);

@@ -634,6 +634,19 @@ struct Matcher {
             p.attrs["defer_norm"] = a_int(1);
             ++marked;
         }
+        // (the same question for the gate / up product with its activation: does its result only feed
+        // one product, the down projection? Then it may store that result as bfloat16 pieces as well.)
+        for (size_t n = 0; n < g.nodes.size(); ++n) {
+            if (removed[n]) continue;
+            Node &p = g.nodes[n];
+            if (p.op != "rmlk.MatMulGroupSwiGLU") continue;
+            const int act = p.outputs[0];
+            if (g.values[act].is_output || users[act].size() != 1) continue;
+            const Node &cons = g.nodes[users[act][0]];
+            const bool product = (cons.op == "rmlk.MatMulAddRMSNorm" || cons.op == "rmlk.MatMulConst") &&
+                                 cons.inputs.size() >= 2 && cons.inputs[0] == act && cons.inputs[1] != act;
+            if (product) p.attrs["reader_is_product"] = a_int(1);
+        }
         return marked;
     }
 
@@ -1019,12 +1032,12 @@ void *split_pieces(OpContext &c, const void *a, int64_t m, int64_t k, size_t own
     return took_fast_path(rmlk_hip_bf16x3_split(c.stream, m, k, a, k, pieces), what) ? pieces : nullptr;
 }
 
-// A many-row norm whose result has one reader, a product (the `defer_norm` mark of the fusion pass),
-// in a session that multiplies over bfloat16 weights on the bf16 matrix cores: room for the pieces of
+// A many-row norm (or gate / up product: mark `reader_is_product`) whose result has one reader, a
+// product (the `defer_norm` mark of the fusion pass), in a session that multiplies over bfloat16 weights on the bf16 matrix cores: room for the pieces of
 // its [rows, cols] result, which the norm kernel then writes itself. Undefined when not wanted.
-Tensor room_for_pieces(OpContext &c, int64_t rows, int64_t cols) {
+Tensor room_for_pieces(OpContext &c, int64_t rows, int64_t cols, const char *mark = "defer_norm") {
     Tensor t;
-    if (!c.session.bf16_pieces || c.session.weights_16bit == 0 || c.attr_int("defer_norm", 0) == 0 || rows < 64 ||
+    if (!c.session.bf16_pieces || c.session.weights_16bit == 0 || c.attr_int(mark, 0) == 0 || rows < 64 ||
         cols % 32 != 0)
         return t;
     const size_t bytes = rmlk_hip_bf16x3_pieces_size(rows, cols);
@@ -1829,10 +1842,13 @@ void op_fused_matmul_group_swiglu(OpContext &c) {
         Tensor &y = c.alloc_output(0, RMLK_FLOAT, shape);
         if (wants_pieces(c, m, k, wt.dtype)) {
             void *pieces = split_pieces(c, a.data(), m, k, 0, nullptr, "rmlk.MatMulGroupSwiGLU", &a);
+            // (the activation's pieces for the down projection behind it, stored by the same launch)
+            Tensor act = pieces ? room_for_pieces(c, m, n, "reader_is_product") : Tensor();
             if (pieces && took_fast_path(rmlk_hip_matmul_bf16x3_swiglu(c.stream, m, n, k, pieces, wt.data(), k,
                                                                        gate_first ? 0 : n, gate_first ? n : 0,
-                                                                       y.data(), n),
+                                                                       y.data(), n, act.defined() ? act.data() : nullptr),
                                          "rmlk.MatMulGroupSwiGLU")) {
+                if (act.defined()) y.pieces = std::make_shared<const Tensor>(std::move(act));
                 ++c.session.products_bf16_pieces;
                 return;
             }

@@ -410,11 +410,14 @@ def matmul_bf16x3_grouped(pieces, wt, outs, m: int, k: int, widths) -> None:
           "rmlk_hip_matmul_bf16x3_grouped")
 
 
-def matmul_bf16x3_swiglu(pieces, wt, out, m: int, n: int, k: int, gate_row: int, up_row: int) -> None:
-    """out[m, n] = swiglu(a . wt[gate_row:+n]^T, a . wt[up_row:+n]^T) over the pieces of a."""
+def matmul_bf16x3_swiglu(pieces, wt, out, m: int, n: int, k: int, gate_row: int, up_row: int,
+                         out_pieces=None) -> None:
+    """out[m, n] = swiglu(a . wt[gate_row:+n]^T, a . wt[up_row:+n]^T) over the pieces of a; out_pieces:
+    where the same launch also stores the pieces of out (the tensor bf16x3_split(out) would return)."""
     assert wt.dtype == torch.bfloat16
     check(lib().rmlk_hip_matmul_bf16x3_swiglu(_stream(), m, n, k, _ptr(pieces), _ptr(wt), k, gate_row, up_row,
-                                              _ptr(out), n), "rmlk_hip_matmul_bf16x3_swiglu")
+                                              _ptr(out), n, _ptr(out_pieces) if out_pieces is not None else None),
+          "rmlk_hip_matmul_bf16x3_swiglu")
 
 
 def rotary(x, cos, sin, out, shape, x_stride, cos_stride, sin_stride) -> None:

@@ -155,6 +155,13 @@ def test_swiglu_form_equals_the_two_products_and_the_activation(device, m, n, k,
     pieces = kk.bf16x3_split(a_d)
     got = torch.zeros((m, n), dtype=torch.float32, device=device)
     kk.matmul_bf16x3_swiglu(pieces, w_d, got, m, n, k, gate_row, up_row)
+    # the same launch storing the pieces of its result: the same floats, and the pieces of those
+    m_pad = (m + 127) // 128 * 128
+    again = torch.zeros((m, n), dtype=torch.float32, device=device)
+    act = torch.zeros(3 * m_pad * n, dtype=torch.int16, device=device)
+    kk.matmul_bf16x3_swiglu(pieces, w_d, again, m, n, k, gate_row, up_row, out_pieces=act)
+    assert_exact(to_np(again), to_np(got))
+    assert torch.equal(act.reshape(3, m_pad, n)[:, :m], kk.bf16x3_split(got).reshape(3, m_pad, n)[:, :m])
     exp64 = None
     if n % 128 == 0:
         # the same accumulation order in the plain product: bit for bit
