@@ -363,6 +363,50 @@ pub unsafe fn attention(
     )
 }
 
+/// `attention` with a `[batch, q_len, heads, head_dim]` result that is also stored as the three
+/// bfloat16 pieces `bf16x3_split` would make of it (`out_pieces`), for an output projection over them.
+pub unsafe fn attention_with_pieces(
+    stream: &HipStream,
+    shape: &AttentionShape,
+    q: *const c_void,
+    k: *const c_void,
+    v: *const c_void,
+    mask: *const c_void,
+    mask_stride: &[usize; 4],
+    scale_is_mul: bool,
+    scale: f32,
+    workspace: *mut c_void,
+    workspace_bytes: usize,
+    out: *mut c_void,
+    out_pieces: *mut c_void,
+) -> Result<()> {
+    let ms = dims(mask_stride)?;
+    check(
+        ffi::rmlk_hip_attention_ws_pieces(
+            stream.raw(),
+            ffi::RMLK_FLOAT,
+            shape.batch as i64,
+            shape.kv_heads as i64,
+            shape.rep as i64,
+            shape.q_len as i64,
+            shape.kv_len as i64,
+            shape.head_dim as i64,
+            q,
+            k,
+            v,
+            mask,
+            &ms,
+            scale_is_mul as i32,
+            scale,
+            workspace,
+            workspace_bytes,
+            out,
+            out_pieces,
+        ),
+        "attention_with_pieces",
+    )
+}
+
 /// While a value of this type lives, operators over tiny tensors issued on `stream` through this
 /// crate are recorded and go out as one launch, in call order (`rmlk_hip_batch_begin` / `_end`).
 /// Work put on the stream by other means must be preceded by `flush`.

@@ -354,6 +354,16 @@ int32_t rmlk_hip_attention_ws(rmlk_stream_t stream, int32_t dtype, int64_t batch
                               const void *q, const void *k, const void *v, const void *mask,
                               const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
                               int32_t out_seq_major, void *workspace, size_t workspace_bytes, void *out);
+/* rmlk_hip_attention_ws with a [batch, q_len, heads, head_dim] result (out_seq_major) that is also
+ * stored as three bfloat16 pieces, as rmlk_hip_bf16x3_split would split the [batch * q_len, heads *
+ * head_dim] matrix it is: `out_pieces` holds rmlk_hip_bf16x3_pieces_size(batch * q_len, heads *
+ * head_dim) bytes. For an output projection over the pieces (rmlk_hip_matmul_bf16x3) that then needs
+ * no split launch. The same values in `out`, bit for bit. */
+int32_t rmlk_hip_attention_ws_pieces(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t kv_heads,
+                                     int64_t rep, int64_t q_len, int64_t kv_len, int64_t head_dim,
+                                     const void *q, const void *k, const void *v, const void *mask,
+                                     const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
+                                     void *workspace, size_t workspace_bytes, void *out, void *out_pieces);
 
 /* The same attention for a handful of query rows per KV head (rep * q_len <= 16: a decode step),
  * where there is no matrix work, only K and V to read: the keys are split over blocks in chunks of

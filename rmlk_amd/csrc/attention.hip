@@ -77,7 +77,33 @@ struct AttnArgs {
     // which under a causal mask are the long ones. Null: block (x, y) is item (tile x, KV head y).
     int32_t *queue;
     int32_t items, tiles_per_head;
+    // The output also as three bfloat16 pieces whose sum it is exactly (the operand form of
+    // rmlk_hip_matmul_bf16x3, for the output projection behind a [B, S, H, D] result): planes of `plane`
+    // elements, laid out like `out`. Null: not wanted.
+    uint16_t *pieces;
+    int64_t plane;
 };
+
+// Four floats as three times four bfloat16 (hi, mid, lo: truncate, subtract, truncate, subtract; Inf
+// and NaN in hi alone), one 64-bit store per plane.
+__device__ __forceinline__ void store_pieces(const v4f &w, uint16_t *at, int64_t plane) {
+    uint32_t hi[4], mid[4], lo[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const uint32_t xb = __float_as_uint(w[e]);
+        const uint32_t hb = xb & 0xffff0000u;
+        const bool finite = (xb & 0x7f800000u) != 0x7f800000u;
+        const float r1 = finite ? w[e] - __uint_as_float(hb) : 0.f;
+        const uint32_t mb = __float_as_uint(r1) & 0xffff0000u;
+        const float r2 = r1 - __uint_as_float(mb);
+        hi[e] = hb >> 16;
+        mid[e] = mb >> 16;
+        lo[e] = __float_as_uint(r2) >> 16;
+    }
+    *reinterpret_cast<uint2 *>(at) = uint2{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16)};
+    *reinterpret_cast<uint2 *>(at + plane) = uint2{mid[0] | (mid[1] << 16), mid[2] | (mid[3] << 16)};
+    *reinterpret_cast<uint2 *>(at + 2 * plane) = uint2{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16)};
+}
 
 template <int NK>
 __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel(AttnArgs g) {
@@ -371,6 +397,11 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
                 }
                 *reinterpret_cast<v4f *>(op + 8 * a) = w0;
                 *reinterpret_cast<v4f *>(op + 32 + 8 * a) = w1;
+                if (g.pieces) {
+                    uint16_t *pp = g.pieces + (op - g.out);
+                    store_pieces(w0, pp + 8 * a, g.plane);
+                    store_pieces(w1, pp + 32 + 8 * a, g.plane);
+                }
             }
         }
     }
@@ -724,17 +755,24 @@ extern "C" size_t rmlk_hip_attention_workspace_size(int32_t dtype, int64_t batch
     return tile_map_dims(batch, kv_heads, rep, q_len, kv_len, mask_stride).bytes;
 }
 
-extern "C" int32_t rmlk_hip_attention_ws(rmlk_stream_t stream, int32_t dtype, int64_t batch,
-                                         int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
-                                         int64_t head_dim, const void *q, const void *k, const void *v,
-                                         const void *mask, const rmlk_dims *mask_stride,
-                                         int32_t scale_is_mul, float scale, int32_t out_seq_major,
-                                         void *workspace, size_t workspace_bytes, void *out) {
+namespace {
+int32_t attention_many_rows(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t kv_heads, int64_t rep,
+                            int64_t q_len, int64_t kv_len, int64_t head_dim, const void *q, const void *k,
+                            const void *v, const void *mask, const rmlk_dims *mask_stride, int32_t scale_is_mul,
+                            float scale, int32_t out_seq_major, void *workspace, size_t workspace_bytes, void *out,
+                            void *out_pieces) {
     AttnArgs g{};
     bool empty = false;
     const int32_t st = attention_args(dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
                                       mask_stride, scale_is_mul, scale, out_seq_major, out, true, &g, &empty);
     if (st || empty) return st;
+    if (out_pieces) {
+        // the pieces of the [batch * q_len, heads * head_dim] matrix that a [B, S, H, D] result is
+        if (!out_seq_major || reinterpret_cast<uintptr_t>(out_pieces) % 16 != 0) return RMLK_ERR_UNSUPPORTED;
+        const int64_t rows = batch * q_len, m_pad = (rows + 127) / 128 * 128;
+        g.pieces = static_cast<uint16_t *>(out_pieces);
+        g.plane = m_pad * kv_heads * rep * head_dim;
+    }
     dim3 grid(static_cast<unsigned>((g.rows + 63) / 64), static_cast<unsigned>(batch * kv_heads), 1);
     const bool many_blocks = static_cast<int64_t>(grid.x) * grid.y > kNumCU;
     {
@@ -778,6 +816,29 @@ extern "C" int32_t rmlk_hip_attention_ws(rmlk_stream_t stream, int32_t dtype, in
         attention_rows_kernel<4><<<grid, AttnShape<4>::kThreads, AttnShape<4>::kLdsBytes, as_stream(stream)>>>(g);
     }
     return launch_status();
+}
+}  // namespace
+
+extern "C" int32_t rmlk_hip_attention_ws(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                         int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
+                                         int64_t head_dim, const void *q, const void *k, const void *v,
+                                         const void *mask, const rmlk_dims *mask_stride,
+                                         int32_t scale_is_mul, float scale, int32_t out_seq_major,
+                                         void *workspace, size_t workspace_bytes, void *out) {
+    return attention_many_rows(stream, dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
+                               mask_stride, scale_is_mul, scale, out_seq_major, workspace, workspace_bytes, out,
+                               nullptr);
+}
+
+extern "C" int32_t rmlk_hip_attention_ws_pieces(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                                int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
+                                                int64_t head_dim, const void *q, const void *k, const void *v,
+                                                const void *mask, const rmlk_dims *mask_stride,
+                                                int32_t scale_is_mul, float scale, void *workspace,
+                                                size_t workspace_bytes, void *out, void *out_pieces) {
+    if (!out_pieces) return RMLK_ERR_NULL_POINTER;
+    return attention_many_rows(stream, dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
+                               mask_stride, scale_is_mul, scale, 1, workspace, workspace_bytes, out, out_pieces);
 }
 
 extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch,

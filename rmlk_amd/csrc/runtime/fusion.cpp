@@ -647,6 +647,28 @@ struct Matcher {
                                  cons.inputs.size() >= 2 && cons.inputs[0] == act && cons.inputs[1] != act;
             if (product) p.attrs["reader_is_product"] = a_int(1);
         }
+        // (and for the attention node whose [B, S, H, D] result reaches the output projection through
+        // a Reshape)
+        for (size_t n = 0; n < g.nodes.size(); ++n) {
+            if (removed[n]) continue;
+            Node &p = g.nodes[n];
+            if (p.op != "rmlk.Attention") continue;
+            const auto major = p.attrs.find("seq_major_output");
+            if (major == p.attrs.end() || major->second.i == 0) continue;
+            int value = p.outputs[0];
+            for (int hop = 0; hop < 2; ++hop) {
+                if (g.values[value].is_output || users[value].size() != 1) break;
+                const Node &cons = g.nodes[users[value][0]];
+                if (cons.op == "Reshape" && cons.inputs[0] == value) {
+                    value = cons.outputs[0];
+                    continue;
+                }
+                if ((cons.op == "rmlk.MatMulAddRMSNorm" || cons.op == "rmlk.MatMulConst") && cons.inputs.size() >= 2 &&
+                    cons.inputs[0] == value && cons.inputs[1] != value)
+                    p.attrs["reader_is_product"] = a_int(1);
+                break;
+            }
+        }
         return marked;
     }
 
@@ -1608,6 +1630,19 @@ void op_fused_attention(OpContext &c) {
             // room for the map of (query tile, key chunk) pairs the mask leaves visible, when it pays
             const size_t map_bytes = rmlk_hip_attention_workspace_size(RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, &ms);
             void *map = map_bytes ? c.scratch(map_bytes) : nullptr;
+            // (the result's pieces for the output projection behind it, stored by the same launch)
+            if (Tensor pieces = seq_major ? room_for_pieces(c, bsz * seq, heads * dim, "reader_is_product") : Tensor();
+                pieces.defined()) {
+                if (took_fast_path(rmlk_hip_attention_ws_pieces(c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim,
+                                                                q.data(), k.data(), v.data(), mask.data(), &ms,
+                                                                static_cast<int32_t>(c.attr_int("scale_is_mul", 0)),
+                                                                attr_float(c, "scale"), map, map_bytes, y.data(),
+                                                                pieces.data()),
+                                   "rmlk.Attention")) {
+                    y.pieces = std::make_shared<const Tensor>(std::move(pieces));
+                    return;
+                }
+            }
             if (took_fast_path(rmlk_hip_attention_ws(c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim,
                                                      q.data(), k.data(), v.data(), mask.data(), &ms,
                                                      static_cast<int32_t>(c.attr_int("scale_is_mul", 0)),

@@ -176,6 +176,7 @@ Tensor &OpContext::view_output(int i, const Tensor &src, const std::vector<int64
     v.buf = src.buf;
     v.offset = src.offset;
     v.pending_product = src.pending_product;   // a view of a product not computed yet is not computed either
+    v.pieces = src.pieces;                     // (the same dense elements in the same order)
     *out[i] = v;
     return *out[i];
 }

@@ -263,13 +263,21 @@ def attention(q, k, v, mask, out, batch: int, kv_heads: int, rep: int, q_len: in
 
 def attention_skipping(q, k, v, mask, out, batch: int, kv_heads: int, rep: int, q_len: int, kv_len: int,
                        head_dim: int, mask_stride, scale: float, scale_is_mul: bool = False,
-                       out_seq_major: bool = False) -> int:
+                       out_seq_major: bool = False, out_pieces=None) -> int:
     """`attention` with the workspace that lets it skip the key chunks a query tile cannot see; returns
-    the workspace size the library asked for (0: skipping does not apply to this shape)."""
+    the workspace size the library asked for (0: skipping does not apply to this shape). out_pieces
+    (with out_seq_major): the result also as the three bfloat16 pieces bf16x3_split would make of it."""
     ms = Dims.of(mask_stride)
     need = int(lib().rmlk_hip_attention_workspace_size(dtype_of(q), batch, kv_heads, rep, q_len, kv_len,
                                                        head_dim, ms))
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    if out_pieces is not None:
+        assert out_seq_major
+        check(lib().rmlk_hip_attention_ws_pieces(_stream(), dtype_of(q), batch, kv_heads, rep, q_len, kv_len,
+                                                 head_dim, _ptr(q), _ptr(k), _ptr(v), _ptr(mask), ms,
+                                                 int(scale_is_mul), float(scale), _ptr(ws) if need else None, need,
+                                                 _ptr(out), _ptr(out_pieces)), "rmlk_hip_attention_ws_pieces")
+        return need
     check(lib().rmlk_hip_attention_ws(_stream(), dtype_of(q), batch, kv_heads, rep, q_len, kv_len,
                                       head_dim, _ptr(q), _ptr(k), _ptr(v), _ptr(mask), ms,
                                       int(scale_is_mul), float(scale), int(out_seq_major),

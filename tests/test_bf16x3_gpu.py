@@ -247,6 +247,33 @@ def test_norm_that_stores_its_result_as_pieces(device, rows, cols, splits, with_
     assert torch.equal(pieces.reshape(3, m_pad, cols)[:, :rows], want)
 
 
+@pytest.mark.parametrize("b,g,rep,s,l", [(1, 8, 4, 512, 640),      # the 512-token prefill into a 640-long cache
+                                         (2, 2, 2, 192, 256),      # two sequences, tiles of the last rows half empty
+                                         (1, 8, 4, 2048, 2048)])   # more blocks than compute units, chunks skipped
+def test_attention_that_stores_its_result_as_pieces(device, b, g, rep, s, l):
+    """rmlk_hip_attention_ws_pieces: the [B, S, H, D] result bit for bit as without the pieces, and the
+    pieces those that rmlk_hip_bf16x3_split makes of the [B * S, H * D] matrix it is."""
+    import torch
+    kk = _k()
+    h, d = g * rep, 64
+    rng = np.random.default_rng(s + l)
+    q, k, v = (to_dev(rng.standard_normal(sh, dtype=np.float32), device)
+               for sh in ((b, h, s, d), (b, g, l, d), (b, g, l, d)))
+    mask = np.where(np.arange(l)[None, :] <= np.arange(s)[:, None] + (l - s) // 2, 0.0, -np.inf).astype(np.float32)
+    m = to_dev(mask.reshape(1, 1, s, l), device)
+    ms = [0, 0, l, 1]
+    plain = torch.full((b, s, h, d), 7.0, device=device)
+    kk.attention_skipping(q, k, v, m, plain, b, g, rep, s, l, d, ms, 8.0, False, out_seq_major=True)
+    rows, cols = b * s, h * d
+    m_pad = (rows + 127) // 128 * 128
+    got = torch.full((b, s, h, d), 9.0, device=device)
+    pieces = torch.zeros(3 * m_pad * cols, dtype=torch.int16, device=device)
+    kk.attention_skipping(q, k, v, m, got, b, g, rep, s, l, d, ms, 8.0, False, out_seq_major=True, out_pieces=pieces)
+    assert_exact(to_np(got), to_np(plain))
+    want = kk.bf16x3_split(plain.reshape(rows, cols)).reshape(3, m_pad, cols)[:, :rows]
+    assert torch.equal(pieces.reshape(3, m_pad, cols)[:, :rows], want)
+
+
 def test_infinities_and_nans_arrive_as_from_an_fp32_product(device):
     import torch
     kk = _k()
