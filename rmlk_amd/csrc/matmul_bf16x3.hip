@@ -14,7 +14,9 @@
 // tiles read it afterwards; the product kernel streams K steps of 32 of the three planes' tile rows
 // and of W's tile rows straight from global memory into LDS (global_load_lds_dwordx4) through two to
 // four stages, and every wavefront multiplies a 64 x (32 * TN) tile: per K chunk TN fragments of W
-// against 3 x 2 fragments of A, 6 * TN MFMAs.
+// against 3 x 2 fragments of A, 6 * TN MFMAs. Kernels that produce an operand of such a product can
+// store its pieces themselves and save the split launch: the RMSNorm kernels (reduce.hip), the
+// attention kernel (attention.hip) and the SwiGLU epilogue below do.
 //
 // No counterpart in the reference (its products are fp32 cuBLAS calls, cuda/src/kernels/gemm.rs:191-232).
 #include "common.hpp"
