@@ -120,7 +120,10 @@ typedef enum rmlk_unary_op {
 int32_t rmlk_hip_unary(rmlk_stream_t stream, int32_t op, int32_t dtype, int64_t n, const void *in,
                        void *out);
 
-/* Cast: C static_cast semantics (float -> int truncates toward zero and saturates; to BOOL is
+/* Cast: C static_cast semantics (float -> int truncates toward zero, NaN gives 0, values out of
+ * range saturate at the limits of the 32-bit type of the target's signedness — 64-bit for a 64-bit
+ * target — and an 8- or 16-bit target keeps the low bits of that, as the reference's kernels do:
+ * half 32768.0 -> INT16 is -32768, cuda/src/kernels/cast.rs:524-539; to BOOL is
  * x != 0; from BOOL is 0/1). Any pair over {FLOAT, DOUBLE, FLOAT16, INT8..INT64, UINT8..UINT64,
  * BOOL}. ref: cuda/src/kernels/unary.rs:47-80, cuda/src/ptx/cast.cu:6-124. */
 int32_t rmlk_hip_cast(rmlk_stream_t stream, int32_t src_dtype, int32_t dst_dtype, int64_t n,
@@ -621,6 +624,13 @@ int32_t rmlk_hip_gemv_kmajor_head_rows(rmlk_stream_t stream, int32_t dtype, int6
 int32_t rmlk_hip_batch_begin(rmlk_stream_t stream);
 int32_t rmlk_hip_batch_flush(rmlk_stream_t stream);
 int32_t rmlk_hip_batch_end(rmlk_stream_t stream);
+/* 1 when a call whose output iterates `shape`, its n_in (1..3) inputs walking that space with the
+ * element strides strides[0 .. n_in - 1] and its output with strides[n_in], is one an open batch
+ * records; 0 when it is launched as usual: more than 1024 elements, more than four dims left after
+ * size-1 dims are dropped and jointly contiguous dims merged, or an operand whose farthest element
+ * lies 2^31 elements or more from its first (a record's offsets are 32-bit). Host arithmetic only,
+ * no GPU needed. No counterpart in the reference. */
+int32_t rmlk_hip_batch_collects(const rmlk_dims *shape, int32_t n_in, const rmlk_dims *strides);
 
 /* Fill `n` elements of `out` with the element at host address `value` (size of dtype).
  * ref: runtime/src/providers/cuda/backend/constant_of_shape.rs:59-62 (host vector + H2D). */

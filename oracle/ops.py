@@ -170,7 +170,8 @@ def sigmoid(x):
 
 
 def cast(x, to: int):
-    """cuda/src/ptx/cast.cu:6-124: C static_cast. float -> int truncates toward zero."""
+    """cuda/src/ptx/cast.cu:6-124: C static_cast. float -> int truncates toward zero; values the
+    target cannot hold follow the rule stated below."""
     x = np.asarray(x)
     dst = np.dtype(ONNX_DTYPES[int(to)])
     if dst == np.bool_:
@@ -178,8 +179,19 @@ def cast(x, to: int):
     if x.dtype == np.bool_:
         return x.astype(dst)
     if np.issubdtype(x.dtype, np.floating) and np.issubdtype(dst, np.integer):
+        # NaN -> 0; out of range saturates at the limits of the 32-bit type of the same signedness
+        # (64-bit for 64-bit targets); 8- and 16-bit targets keep the low bits of that 32-bit value
+        # (the reference's vector half 32768.0 -> int16 -32768, cuda/src/kernels/cast.rs:524-539)
+        wide = dst if dst.itemsize == 8 else np.dtype(np.int32 if dst.kind == "i" else np.uint32)
+        info = np.iinfo(wide)
         with np.errstate(all="ignore"):
-            return np.trunc(x.astype(np.float64)).astype(dst)
+            v = np.trunc(x.astype(np.float64))
+            v = np.where(np.isnan(v), 0.0, v)
+            big = v >= float(info.max)
+            small = v <= float(info.min)
+            mid = np.where(big | small, 0.0, v).astype(wide)
+            w = np.where(big, info.max, np.where(small, info.min, mid)).astype(wide)
+        return w.astype(dst)
     with np.errstate(all="ignore"):
         return x.astype(dst)
 

@@ -343,6 +343,16 @@ bool small_op_layout(SmallOp &op, int rank, const int64_t *shape, int n_in, cons
         for (int p = 0; p < 4; ++p) st[p][0] = 0;
     }
     if (r > kBatchMaxRank) return false;
+    // the kernel adds offsets up in 32 bits: the farthest element of every operand must stay below 2^31
+    for (int p = 0; p < 4; ++p) {
+        int64_t reach = 0;
+        for (int d = 0; d < r; ++d) {
+            const int64_t a = st[p][d] < 0 ? -st[p][d] : st[p][d];
+            if (a > (1ll << 30)) return false;
+            reach += (dim[d] - 1) * a;
+        }
+        if (reach >= (1ll << 31)) return false;
+    }
     op.n = static_cast<int32_t>(n);
     op.rank = r;
     for (int d = 0; d < kBatchMaxRank; ++d) {
@@ -359,6 +369,18 @@ bool small_op_layout(SmallOp &op, int rank, const int64_t *shape, int n_in, cons
 }  // namespace rmlk
 
 using namespace rmlk;
+
+extern "C" int32_t rmlk_hip_batch_collects(const rmlk_dims *shape, int32_t n_in, const rmlk_dims *strides) {
+    if (!shape || !strides || n_in < 1 || n_in > 3) return 0;
+    if (shape->rank < 1 || shape->rank > kMaxRank) return 0;
+    int64_t st[4][kMaxRank] = {};
+    for (int p = 0; p <= n_in; ++p) {
+        if (strides[p].rank != shape->rank) return 0;
+        for (int d = 0; d < shape->rank; ++d) st[p][d] = strides[p].v[d];
+    }
+    SmallOp op{};
+    return small_op_layout(op, shape->rank, shape->v, n_in, st) ? 1 : 0;
+}
 
 extern "C" int32_t rmlk_hip_batch_begin(rmlk_stream_t stream) {
     hipStream_t s = as_stream_collecting(stream);

@@ -149,15 +149,22 @@ struct CastF {
         } else if constexpr (out_bool) {
             return BoolTag{static_cast<uint8_t>(x != static_cast<TI>(0) ? 1 : 0)};
         } else if constexpr (std::is_integral<TO>::value && !std::is_integral<TI>::value) {
-            // float -> int: truncate toward zero; NaN -> 0; out of range saturates.
+            // float -> int: truncate toward zero; NaN -> 0; out of range saturates at the limits of
+            // the 32-bit type of the same signedness (64-bit for 64-bit targets), and an 8- or
+            // 16-bit target keeps the low bits of that: what the reference's `static_cast` compiles
+            // to (a 32-bit conversion, then a narrowing move), pinned by its own vector
+            // half 32768.0 -> int16 -32768 (cuda/src/kernels/cast.rs:524-539).
+            using Wide = std::conditional_t<(sizeof(TO) > 4),
+                                            TO,
+                                            std::conditional_t<std::is_signed<TO>::value, int32_t, uint32_t>>;
             double v = static_cast<double>(x);
             if (v != v) return 0;
-            constexpr double lo = static_cast<double>(std::numeric_limits<TO>::min());
+            constexpr double lo = static_cast<double>(std::numeric_limits<Wide>::min());
             // max() of 64-bit types is not a double; 2^63 / 2^64 is the first value out of range.
-            constexpr double hi = static_cast<double>(std::numeric_limits<TO>::max());
-            if (v <= lo) return std::numeric_limits<TO>::min();
-            if (v >= hi) return std::numeric_limits<TO>::max();
-            return static_cast<TO>(v);
+            constexpr double hi = static_cast<double>(std::numeric_limits<Wide>::max());
+            if (v <= lo) return static_cast<TO>(std::numeric_limits<Wide>::min());
+            if (v >= hi) return static_cast<TO>(std::numeric_limits<Wide>::max());
+            return static_cast<TO>(static_cast<Wide>(v));
         } else {
             return static_cast<TO>(x);
         }

@@ -444,10 +444,15 @@ void op_expand(OpContext &c) {
 void op_slice(OpContext &c) {
     const Tensor &x = c.input(0);
     require_dtype(x.dtype, {RMLK_FLOAT16, RMLK_FLOAT, RMLK_DOUBLE, RMLK_INT32, RMLK_INT64});
-    if (x.rank() == 0) fail_op("Slice needs rank >= 1");
     if (x.rank() > RMLK_MAX_RANK) fail_op("Slice supports rank <= 8");
     HostVal starts = c.host_values(1), ends = c.host_values(2);
     if (starts.size() != ends.size()) fail_op("Slice starts and ends must have the same length");
+    if (x.rank() == 0) {
+        // nothing to slice along: the scalar itself (cuda/src/kernels/slice.rs:200-222)
+        if (starts.size() != 0) fail_op("AxisOutOfRange");
+        c.view_output(0, x, {});
+        return;
+    }
     const int rank = x.rank();
     std::vector<int64_t> axes, steps;
     if (c.has_input(3)) {

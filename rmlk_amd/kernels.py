@@ -152,6 +152,7 @@ def matmul_noalloc(a, b, c, batch, m, n, k, lda, ldb, ldc, stride_a, stride_b, s
 
 def transpose(x, out, in_shape, perm) -> None:
     """ref: cuda/src/kernels/transpose.rs:38-80."""
+    assert len(perm) == len(in_shape), "perm.len() must match rank"
     arr = (ctypes.c_int64 * len(perm))(*[int(p) for p in perm])
     check(lib().rmlk_hip_transpose(_stream(), dtype_of(x), Dims.of(in_shape), arr, _ptr(x),
                                    _ptr(out)), "rmlk_hip_transpose")

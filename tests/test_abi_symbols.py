@@ -59,3 +59,30 @@ def test_version_and_status_strings_without_gpu(handle):
     handle.rmlk_hip_status_string.argtypes = [ctypes.c_int32]
     assert "dtype" in handle.rmlk_hip_status_string(-2).decode().lower() or \
         handle.rmlk_hip_status_string(-2).decode()
+
+
+def _collects(handle, shape, strides):
+    from rmlk_amd._lib import Dims
+    handle.rmlk_hip_batch_collects.restype = ctypes.c_int32
+    handle.rmlk_hip_batch_collects.argtypes = [ctypes.POINTER(Dims), ctypes.c_int32, ctypes.POINTER(Dims)]
+    arr = (Dims * len(strides))(*[Dims.of(s) for s in strides])
+    return handle.rmlk_hip_batch_collects(Dims.of(shape), len(strides) - 1, arr)
+
+
+def test_collected_launches_refuse_offsets_beyond_32_bits(handle):
+    """A record of the collected launch keeps 32-bit element strides and the kernel adds offsets up
+    in 32 bits: a tiny tensor whose operand strides reach 2^31 elements must be launched as usual
+    (host arithmetic only, nothing runs)."""
+    dense = [32, 1]
+    assert _collects(handle, [32, 32], [dense, dense, dense]) == 1
+    assert _collects(handle, [32, 32], [dense, [0, 1], dense]) == 1            # broadcast operand
+    assert _collects(handle, [1024, 1024], [[1024, 1]] * 3) == 0               # too many elements
+    # 1024 elements, each stride below 2^30, but the last element lies 31 * 2^27 + 31 * 2^21 > 2^31 away
+    far = [1 << 27, 1 << 21]
+    assert (32 - 1) * far[0] + 31 * far[1] >= 1 << 31
+    assert _collects(handle, [32, 32], [far, dense, dense]) == 0
+    assert _collects(handle, [32, 32], [dense, dense, far]) == 0               # the output too
+    near = [1 << 25, 1 << 20]                                                  # reach just under 2^30
+    assert _collects(handle, [32, 32], [near, dense, dense]) == 1
+    assert _collects(handle, [2, 2], [[1 << 31, 1], [2, 1], [2, 1]]) == 0      # one stride beyond 2^30
+    assert _collects(handle, [2, 2], [[-(1 << 30), 1], [2, 1], [2, 1]]) == 1   # negative strides count by size

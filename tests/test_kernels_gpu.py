@@ -228,6 +228,26 @@ def test_cast_pairs(device, src, dst):
     assert_exact(to_np(out), expected)
 
 
+@pytest.mark.parametrize("src", [np.float32, np.float64, np.float16])
+@pytest.mark.parametrize("dst", [np.int8, np.int16, np.int32, np.int64, np.uint8, np.uint16, np.uint32,
+                                 np.uint64])
+def test_cast_values_the_target_cannot_hold(device, src, dst):
+    """Float values outside the target's range: the 32-bit (64-bit) limits, then the low bits for
+    narrow targets, NaN -> 0 — the rule the reference's vector half 32768.0 -> int16 -32768 pins
+    (cuda/src/kernels/cast.rs:524-539); the oracle states it, the kernel must agree bit for bit."""
+    k = _k()
+    from oracle.ops import NP_TO_ONNX
+    vals = [0.0, -0.9, 127.9, 128.0, 255.0, 256.0, 300.5, -129.0, -200.0, 32767.0, 32768.0, 40000.0,
+            65535.0, 65536.0, 65541.0, -32769.0, 2147483647.0, 2147483648.0, 4294967296.0,
+            -2147483649.0, 9.3e18, 1.9e19, -9.3e18, 1e30, -1e30, np.inf, -np.inf, np.nan]
+    with np.errstate(all="ignore"):
+        x = np.array(vals, dtype=np.float64).astype(src)
+    expected = _ops().cast(x, NP_TO_ONNX[np.dtype(dst)])
+    out = torch.empty(x.size, dtype=to_dev(expected, device).dtype, device=device)
+    k.cast(to_dev(x, device), out)
+    assert_exact(to_np(out), expected)
+
+
 REDUCE_CASES = [
     ((4, 8), [1]), ((4, 8), [0]), ((4, 8), [0, 1]),
     ((2, 3, 4), [2]), ((2, 3, 4), [1]), ((2, 3, 4), [0, 2]), ((2, 3, 4), [1, 2]),

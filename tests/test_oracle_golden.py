@@ -296,3 +296,149 @@ def test_weight_storage_rounding_closed_forms_and_torch():
         np.testing.assert_array_equal(ops.store_weights(x, name).view(np.uint32), exp.view(np.uint32))
     with pytest.raises(ops.OracleError):
         ops.store_weights(x[:4], "fp8")
+
+
+# ---- the kernel crate's own known-answer tests (cuda/src/kernels/<op>.rs) ---------------------
+import kernel_vectors as kv  # noqa: E402
+
+KC = kv.KERNEL_CASES
+ORACLE_BINARY = {"add": ops.add, "sub": ops.sub, "mul": ops.mul, "div": ops.div,
+                 "equal": ops.equal, "greater": ops.greater}
+ORACLE_UNARY = {"sqrt": ops.sqrt, "neg": ops.neg, "sin": ops.sin, "cos": ops.cos,
+                "sigmoid": ops.sigmoid}
+
+
+def test_kernel_vector_counts():
+    """Every kernel-crate file whose tests hold literal vectors is represented."""
+    want = {"reduce_mean": 10, "binary": 6, "pow": 35, "where": 1, "unary": 7, "cast": 101,
+            "expand": 7, "transpose": 5, "trilu": 6, "scatter_nd": 5, "slice": 20, "gemm": 1}
+    assert {k: len(v) for k, v in KC.items()} == want
+    assert sorted(s["test"] for s in CASES["kernel_skipped"]) == [
+        "test_expand_same_mid_axis", "test_transpose_arbitrary_3d"]
+
+
+@pytest.mark.parametrize("case", KC["binary"], ids=kv.ids(KC["binary"]))
+def test_kernel_binary_vectors(case):
+    a, b = (kv.arr(case, k, shape=case["shape"]) for k in "ab")
+    got = ORACLE_BINARY[case["op"]](a, b)
+    exp = decode(case["expected"], got.dtype)
+    kv.check(got, exp, case["compare"], case["epsilon"])
+
+
+@pytest.mark.parametrize("case", KC["pow"], ids=kv.ids(KC["pow"]))
+def test_kernel_pow_vectors(case):
+    """cuda/src/kernels/pow.rs:248-775: all 35 (base, exponent) element-type pairs the crate tests,
+    including the pairs the provider leaves disabled (backend/pow.rs:133-160)."""
+    a = kv.arr(case, "a", "a_dtype", case["shape"])
+    b = kv.arr(case, "b", "b_dtype", case["shape"])
+    got = ops.pow_(a, b)
+    assert got.dtype == a.dtype
+    kv.check(got, decode(case["expected"], a.dtype), case["compare"], case["epsilon"])
+
+
+@pytest.mark.parametrize("case", KC["where"], ids=kv.ids(KC["where"]))
+def test_kernel_where_vectors(case):
+    x, y = (kv.arr(case, k, shape=case["shape"]) for k in "xy")
+    cond = np.array(case["cond"], dtype=bool).reshape(case["shape"])
+    kv.check(ops.where(cond, x, y), decode(case["expected"], x.dtype))
+
+
+@pytest.mark.parametrize("case", KC["unary"], ids=kv.ids(KC["unary"]))
+def test_kernel_unary_vectors(case):
+    x = kv.arr(case, "input")
+    kv.check(ORACLE_UNARY[case["op"]](x), decode(case["expected"], x.dtype), case["compare"],
+             case["epsilon"])
+
+
+@pytest.mark.parametrize("case", KC["cast"], ids=kv.ids(KC["cast"]))
+def test_kernel_cast_vectors(case):
+    """cuda/src/kernels/cast.rs:372-1415."""
+    x = kv.arr(case, "input", "src_dtype")
+    got = ops.cast(x, ops.NP_TO_ONNX[np.dtype(case["dst_dtype"])])
+    assert got.dtype == np.dtype(case["dst_dtype"])
+    kv.check(got, decode(case["expected"], got.dtype))
+
+
+@pytest.mark.parametrize("case", KC["expand"], ids=kv.ids(KC["expand"]))
+def test_kernel_expand_vectors(case):
+    x = kv.arr(case, "input", shape=case["input_shape"])
+    got = ops.expand(x, case["output_shape"])
+    assert list(got.shape) == case["output_shape"]
+    kv.check(got, decode(case["expected"], x.dtype))
+    flat = loops.expand_loop(case["input_shape"], case["output_shape"], x.reshape(-1).tolist()) \
+        if hasattr(loops, "expand_loop") and x.size else None
+    if flat is not None:
+        kv.check(np.array(flat, dtype=x.dtype), decode(case["expected"], x.dtype))
+
+
+def test_kernel_expand_mid_axis_stand_in():
+    """cuda/src/kernels/expand.rs:174-189 builds its expectation with loops (each of the three
+    values repeated four times, the whole twice); restated here."""
+    x = np.array([1.0, 2.0, 3.0]).reshape(1, 3, 1)
+    exp = np.tile(np.repeat(np.array([1.0, 2.0, 3.0]), 4), 2)
+    kv.check(ops.expand(x, [2, 3, 4]), exp)
+
+
+@pytest.mark.parametrize("case", KC["transpose"], ids=kv.ids(KC["transpose"]))
+def test_kernel_transpose_vectors(case):
+    x = kv.arr(case, "input", shape=case["input_shape"])
+    if case.get("expect_error"):
+        with pytest.raises(Exception):
+            ops.transpose(x, case["perm"])
+        return
+    kv.check(ops.transpose(x, case["perm"]), decode(case["expected"], x.dtype))
+
+
+def test_kernel_transpose_3d_stand_in():
+    """cuda/src/kernels/transpose.rs:181-198: [2,3,4] with perm [2,0,1]; its loops say
+    out[o0,o1,o2] = in[o1,o2,o0]."""
+    x = np.arange(24, dtype=np.int32).reshape(2, 3, 4)
+    got = ops.transpose(x, [2, 0, 1])
+    exp = np.array([x[o1, o2, o0] for o0 in range(4) for o1 in range(2) for o2 in range(3)],
+                   dtype=np.int32)
+    kv.check(got, exp)
+
+
+@pytest.mark.parametrize("case", KC["trilu"], ids=kv.ids(KC["trilu"]))
+def test_kernel_trilu_vectors(case):
+    """cuda/src/kernels/trilu.rs:138-196. The reference kernel leaves what lies outside the triangle
+    unwritten and its tests rely on a zero-filled output; the oracle writes the zeros."""
+    x = kv.arr(case, "input", shape=case["shape"])
+    kv.check(ops.trilu(x, k=case["k"], upper=int(case["upper"])), decode(case["expected"], x.dtype))
+
+
+@pytest.mark.parametrize("case", KC["scatter_nd"], ids=kv.ids(KC["scatter_nd"]))
+def test_kernel_scatter_nd_vectors(case):
+    """cuda/src/kernels/scatter_nd.rs:318-417 over zero data (where the reference's `in + 0*out`
+    and plain assignment agree)."""
+    data = np.zeros(case["data_shape"], dtype=case["dtype"])
+    idx = np.array(case["indices"], dtype=np.int64).reshape(case["indices_shape"])
+    upd = kv.arr(case, "updates", shape=case["updates_shape"])
+    kv.check(ops.scatter_nd(data, idx, upd), decode(case["expected"], data.dtype))
+
+
+@pytest.mark.parametrize("case", KC["slice"], ids=kv.ids(KC["slice"]))
+def test_kernel_slice_vectors(case):
+    """cuda/src/kernels/slice.rs:200-700: negative steps, INT64 sentinels, clamping, absent axes /
+    steps (empty slices in the reference's kernel tests)."""
+    x = kv.arr(case, "input", shape=case["input_shape"])
+    got = ops.slice_(x, case["starts"], case["ends"], case["axes"] or None, case["steps"] or None)
+    # operator level: the shape rule of backend/slice.rs:417-452 decides the output shape
+    assert list(got.shape) == case.get("onnx_output_shape", case["output_shape"])
+    kv.check(got, decode(case.get("onnx_expected", case["expected"]), x.dtype))
+    # kernel level: the caller gives the output shape, element i of a dim is input element
+    # start + i * step (slice_op_macros.cuh:38-75)
+    res = ops.slice_resolve(case["input_shape"], case["starts"], case["ends"], case["axes"] or None,
+                            case["steps"] or None)
+    idx = tuple(s0 + np.arange(n) * st for (s0, st, _), n in zip(res, case["output_shape"]))
+    kernel_level = x[np.ix_(*idx)] if x.ndim else x
+    kv.check(kernel_level, decode(case["expected"], x.dtype))
+
+
+@pytest.mark.parametrize("case", KC["gemm"], ids=kv.ids(KC["gemm"]))
+def test_kernel_gemm_vectors(case):
+    a = kv.arr(case, "lhs", shape=case["lhs_shape"])
+    b = kv.arr(case, "rhs", shape=case["rhs_shape"])
+    assert not case["trans_a"] and not case["trans_b"]
+    kv.check(ops.matmul(a, b), decode(case["expected"], a.dtype))
+    kv.check(ops.matmul(a, b, "f32"), decode(case["expected"], a.dtype))
