@@ -90,6 +90,27 @@ def test_config3_full_sequence_properties(device):
     assert_close(y[:, :96], exp, rtol=1e-4, atol=2e-5)
 
 
+@pytest.mark.parametrize("fuse", [True, False], ids=["fused", "one_kernel_per_node"])
+def test_config3_full_sequence_every_row_against_the_oracle(device, fuse):
+    """S = 2048, the sequence length the configuration names: every one of the 2048 output rows of
+    the layer against the oracle walking the same graph (fp32 BLAS, one [1,32,2048,2048] softmax:
+    seconds on the host). With fusion this is where the resident-grid attention kernel that skips
+    hidden key chunks and the 128 x 192 q/k/v tiles run; without it, one kernel per node as the
+    reference executes a graph. The bar of the short-sequence test: rtol 1e-4 / atol 2e-5
+    (multi-op graphs in the reference: abs 1e-5 at toy sizes, runtime/tests/graphs/main.rs:28-40)."""
+    graphs, runtime = _rt()
+    graph, feeds = graphs.decoder_layer_graph(seed=3, seq=2048)
+    exp = _oracle().run_graph(graph, feeds, "f32")["y"]
+    inst = runtime.Builder.from_graph(graph).build(fuse=fuse)
+    try:
+        assert (inst.fused_nodes > 0) == fuse
+        got = inst.run(feeds)["y"]
+    finally:
+        inst.close()
+    assert got.shape == exp.shape == (1, 2048, 2048)
+    assert_close(got, exp, rtol=1e-4, atol=2e-5)
+
+
 def _greedy_concat(inst, graphs, cfg, prompt, steps):
     feeds = graphs.llama_concat_inputs(cfg, prompt, None, 0)
     out = inst.run(feeds)
