@@ -468,10 +468,43 @@ def run_ops_suite(args):
         us = e0.elapsed_time(e1) / (n_timed * reps) * 1e3
         results[name] = {"us_per_call_with_launch_gaps": round(us, 2), "algorithmic_bytes": bytes_,
                          "calls_timed": n_timed * reps, "kernels_per_call": kernels_per_call,
-                         "buffer_sets": nset}
+                         "buffer_sets": nset, "launches_per_graph": reps}
         log(f"[ops] {name}: {us:.2f} us/call with launch gaps, {bytes_ / us / 1e6:.2f} TB/s")
         del graph
 
+    # (before the first marker launch, so that a kernel trace split at the markers does not see them)
+    half = n * 2
+    sink = torch.zeros(4096, dtype=torch.int32, device=dev)
+    clock = {}
+    for name, kind, nbytes, blocks in (("read_33MB", k.YARDSTICK_READ, n * 4, n * 4 // 32768),
+                                       ("copy_17MB_17MB", k.YARDSTICK_COPY, half, half // 16384),
+                                       ("copy_33MB_33MB", k.YARDSTICK_COPY, n * 4, n * 4 // 16384)):
+        stamps = torch.zeros(reps, blocks, 2, dtype=torch.int64, device=dev)
+        with torch.cuda.stream(side):
+            fn = lambda i: k.stream_yardstick(kind, xs[i % ns], sink if kind == k.YARDSTICK_READ else ys[i % ns],  # noqa: E731
+                                              nbytes, stamps=stamps[i % reps], stream=side.cuda_stream)
+            for i in range(ns):
+                fn(i)
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(reps):
+                    fn(i)
+            for _ in range(20 if args.ops_quick else 200):
+                graph.replay()
+            side.synchronize()
+        st = stamps.cpu().numpy().astype(np.int64)          # 100 MHz: 10 ns per tick
+        first, last_start, last_end = st[:, :, 0].min(1), st[:, :, 0].max(1), st[:, :, 1].max(1)
+        span = (last_end - first) * 0.01
+        gap = (first[1:] - last_end[:-1]) * 0.01
+        clock[name] = {"launches": int(reps), "first_start_to_last_end_us": round(float(span.mean()), 2),
+                       "min": round(float(span.min()), 2), "max": round(float(span.max()), 2),
+                       "first_start_to_last_start_us": round(float(((last_start - first) * 0.01).mean()), 2),
+                       "last_end_to_next_first_start_us": round(float(gap.mean()), 2),
+                       "start_to_start_us": round(float(((first[1:] - first[:-1]) * 0.01).mean()), 2),
+                       "by_buffer_set_us": [round(float(span[np.arange(reps) % ns == j].mean()), 2) for j in range(ns)]}
+        log(f"[ops] in-kernel clock, {name}: {clock[name]}")
+        del graph, stamps
     # ---- yardsticks: an almost empty launch and a plain 256 MiB copy -------------------------------
     timed("launch_floor", lambda i: check(lib().rmlk_hip_fill(side.cuda_stream, k.INT32, 1, ctypes.byref(one),
                                                               marker.data_ptr()), "rmlk_hip_fill"), 1, 4)
@@ -482,6 +515,16 @@ def run_ops_suite(args):
         side.cuda_stream, big[2 + i % 2].data_ptr(), big[i % 2].data_ptr(), CALIBRATION_COPY_BYTES),
         "rmlk_hip_memcpy_dtod"), 2, 2 * CALIBRATION_COPY_BYTES)
     del big
+    # minimal streaming kernels over the same rotating buffers as the operators below: what this chip
+    # does with 33.5 MB read, 16.8 + 16.8 MB copied and 33.5 + 33.5 MB copied when a kernel does
+    # nothing else. yardstick_clock adds, from clocks read inside those kernels, how a launch's time
+    # splits into the memory system's part and what lies between two launches.
+    timed("yardstick_read_33MB", lambda i: k.stream_yardstick(k.YARDSTICK_READ, xs[i], sink, n * 4,
+                                                              stream=side.cuda_stream), ns, n * 4)
+    timed("yardstick_copy_17MB_17MB", lambda i: k.stream_yardstick(k.YARDSTICK_COPY, xs[i], ys[i], half,
+                                                                   stream=side.cuda_stream), ns, 2 * half)
+    timed("yardstick_copy_33MB_33MB", lambda i: k.stream_yardstick(k.YARDSTICK_COPY, xs[i], ys[i], n * 4,
+                                                                   stream=side.cuda_stream), ns, 2 * n * 4)
     # ---- configs[1] ---------------------------------------------------------------------------------
     timed("add", lambda i: k.binary(k.ADD, xs[i], bs[i], ys[i], shp, dense, bst), ns, 2 * n * 4 + 8192)
     timed("mul", lambda i: k.binary(k.MUL, xs[i], bs[i], ys[i], shp, dense, bst), ns, 2 * n * 4 + 8192)
@@ -573,6 +616,9 @@ def run_ops_suite(args):
     print(json.dumps({"suite": "ops", "note": "us_per_call_with_launch_gaps: HIP events around replays of a "
                       "recorded graph of rotating launches; kernel durations come from rocprofv3 "
                       "--kernel-trace of this command (bench.py --summarize-ops)",
+                      "yardstick_clock": {"note": "the yardstick launches once more, 100 per recorded graph over the "
+                                          "rotating buffers, each block noting the 100 MHz clock at its start "
+                                          "and end: times of the last replay, per launch", **clock},
                       "results": results}))
 
 
@@ -658,6 +704,27 @@ def summarize_ops(args):
         print(line + " |")
     for label, (_, unit) in pmc.items():
         print(f"\n{label}: one counter unit = {unit:.3f} KiB (from the 256 MiB copy of the same run).")
+    # which launches are the fast ones: by place in the recorded graph and by buffer set
+    import numpy as np
+    print("\n| op | p10 us | p50 us | p90 us | first launch of a replay | other launches | launches on buffer set 0 "
+          "| on other sets | start-to-start p50 us |")
+    print("|---|---|---|---|---|---|---|---|---|")
+    for nm, seg in zip(names, segs):
+        r = res[nm]
+        kpc, nset = r["kernels_per_call"], r["buffer_sets"]
+        if kpc != 1 or r["algorithmic_bytes"] <= 4096:
+            continue
+        rows = seg[-r["calls_timed"]:]
+        st = np.array([int(x["Start_Timestamp"]) for x in rows])
+        d = np.array([int(x["End_Timestamp"]) for x in rows]) - st
+        d = d / 1e3
+        per_graph = int(r.get("launches_per_graph", 100))
+        pos = np.arange(len(d)) % per_graph
+        bset = pos % nset
+        p10, p50, p90 = np.percentile(d, [10, 50, 90])
+        s2s = np.diff(st) / 1e3
+        print(f"| {nm} | {p10:.2f} | {p50:.2f} | {p90:.2f} | {d[pos == 0].mean():.2f} | {d[pos != 0].mean():.2f} | "
+              f"{d[bset == 0].mean():.2f} | {d[bset != 0].mean():.2f} | {np.median(s2s):.2f} |")
 
 
 def run_graph_suite(args):

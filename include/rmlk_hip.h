@@ -643,6 +643,19 @@ int32_t rmlk_hip_fill(rmlk_stream_t stream, int32_t dtype, int64_t n, const void
 int32_t rmlk_hip_range(rmlk_stream_t stream, int32_t dtype, int64_t n, const void *start,
                        const void *delta, void *out);
 
+/* Streaming yardsticks for benchmarks: the least a kernel can do with `bytes` on this chip, to be
+ * timed next to the operators of the same traffic. READ: `bytes` of `src` are loaded (streaming
+ * 128-bit loads, 32 KiB per block of 256 lanes, all requested up front, one trip) and reduced to
+ * nothing; `dst` (>= 4 * bytes / 32768 bytes) is practically never written. COPY: `bytes` of `src`
+ * go to `dst` (16 KiB per block, streaming loads and stores). `bytes` must be a multiple of the
+ * block's share, `src` / `dst` 16-byte aligned. With `stamps` non-null (2 * number of blocks 64-bit
+ * words of device memory) block b stores the constant 100 MHz clock (s_memrealtime) at its start in
+ * stamps[2b] and at its end in stamps[2b + 1]: last end - first start is the time the memory system
+ * needed, which a kernel trace cannot separate from dispatch. No counterpart in the reference. */
+enum { RMLK_YARDSTICK_READ = 0, RMLK_YARDSTICK_COPY = 1 };
+int32_t rmlk_hip_stream_yardstick(rmlk_stream_t stream, int32_t kind, size_t bytes, const void *src,
+                                  void *dst, uint64_t *stamps);
+
 /* Write up to 256 bytes from host memory `src` to device memory `dst`. The bytes travel as kernel
  * arguments: no staging copy, nothing to keep alive, recordable into a HIP graph.
  * ref: runtime/src/providers/cuda/backend/shape.rs:67-72 (host vector + H2D for tiny tensors). */

@@ -58,6 +58,69 @@ extern "C" int32_t rmlk_hip_memset(rmlk_stream_t stream, void *dst, int32_t byte
     return st;
 }
 
+// ---- streaming yardsticks --------------------------------------------------------------------------
+// The least a kernel can do with N bytes on this chip: every lane requests all its 128-bit units up
+// front (streaming loads), the grid covers the bytes in one trip. Benchmarks time these next to the
+// operators of the same traffic; with `stamps` a block also notes the constant 100 MHz clock when it
+// starts and when it ends, so that the time between the first block's start and the last block's
+// end (what the memory system needs) can be told from what a trace adds around it (dispatch).
+namespace rmlk {
+namespace {
+using U128 = Vec<uint32_t, 4>;
+
+__device__ __forceinline__ void note(uint64_t *stamps, uint64_t t0) {
+    if (stamps && threadIdx.x == 0) {
+        stamps[2 * blockIdx.x] = t0;
+        stamps[2 * blockIdx.x + 1] = wall_clock64();
+    }
+}
+
+// 32 KiB per block: 8 units per lane
+__global__ __launch_bounds__(256) void yardstick_read_kernel(const U128 *__restrict__ in, uint32_t *__restrict__ out,
+                                                             uint64_t *stamps) {
+    const uint64_t t0 = stamps ? wall_clock64() : 0;
+    const size_t base = static_cast<size_t>(blockIdx.x) * 2048 + threadIdx.x;
+    U128 r[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) r[u] = nt_load(in + base + u * 256);
+    uint32_t acc = 0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc += r[u].v[0] ^ r[u].v[1] ^ r[u].v[2] ^ r[u].v[3];
+    if (acc == 0x9e3779b9u && out) out[blockIdx.x] = acc;   // keeps the loads alive; writes next to nothing
+    note(stamps, t0);
+}
+
+// 16 KiB in and 16 KiB out per block: 4 units per lane
+__global__ __launch_bounds__(256) void yardstick_copy_kernel(const U128 *__restrict__ in, U128 *__restrict__ out,
+                                                             uint64_t *stamps) {
+    const uint64_t t0 = stamps ? wall_clock64() : 0;
+    const size_t base = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
+    U128 r[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) r[u] = nt_load(in + base + u * 256);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) nt_store(out + base + u * 256, r[u]);
+    note(stamps, t0);
+}
+}  // namespace
+}  // namespace rmlk
+
+extern "C" int32_t rmlk_hip_stream_yardstick(rmlk_stream_t stream, int32_t kind, size_t bytes, const void *src,
+                                             void *dst, uint64_t *stamps) {
+    if (kind != RMLK_YARDSTICK_READ && kind != RMLK_YARDSTICK_COPY) return RMLK_ERR_INVALID_ARGUMENT;
+    const size_t chunk = kind == RMLK_YARDSTICK_READ ? 32768 : 16384;
+    if (bytes == 0 || bytes % chunk != 0 || bytes / chunk > 0x7fffffffu) return RMLK_ERR_INVALID_ARGUMENT;
+    if (!src || !dst) return RMLK_ERR_NULL_POINTER;
+    if (reinterpret_cast<uintptr_t>(src) % 16 || reinterpret_cast<uintptr_t>(dst) % 16) return RMLK_ERR_INVALID_ARGUMENT;
+    const unsigned grid = static_cast<unsigned>(bytes / chunk);
+    hipStream_t s = as_stream(stream);
+    if (kind == RMLK_YARDSTICK_READ)
+        yardstick_read_kernel<<<grid, 256, 0, s>>>(static_cast<const U128 *>(src), static_cast<uint32_t *>(dst), stamps);
+    else
+        yardstick_copy_kernel<<<grid, 256, 0, s>>>(static_cast<const U128 *>(src), static_cast<U128 *>(dst), stamps);
+    return launch_status();
+}
+
 extern "C" int32_t rmlk_hip_stream_sync(rmlk_stream_t stream) {
     return static_cast<int32_t>(hipStreamSynchronize(as_stream(stream)));
 }

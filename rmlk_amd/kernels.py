@@ -508,6 +508,18 @@ class collected_launches:
         return False
 
 
+YARDSTICK_READ, YARDSTICK_COPY = 0, 1
+
+
+def stream_yardstick(kind: int, src, dst, nbytes: int, stamps=None, stream=None) -> None:
+    """The minimal streaming read (kind YARDSTICK_READ) or copy (YARDSTICK_COPY) of `nbytes`, for
+    benchmarks; `stamps` (int64, 2 per block) receives each block's start and end on the 100 MHz
+    clock. No counterpart in the reference."""
+    st = lib().rmlk_hip_stream_yardstick(_stream() if stream is None else stream, kind, nbytes, _ptr(src),
+                                         _ptr(dst), _ptr(stamps))
+    check(st, "rmlk_hip_stream_yardstick")
+
+
 def device_info(device: int = 0) -> dict:
     from ._lib import DeviceInfo
     info = DeviceInfo()

@@ -800,3 +800,24 @@ def test_full_size_masked_softmax(device):
     sums = out.sum(dim=-1, dtype=torch.float64)
     assert float((sums - 1.0).abs().max()) <= 2e-6
     assert bool((out[:, 0, 0] == 1.0).all())
+
+
+def test_stream_yardstick(device):
+    """The benchmark yardsticks: the copy copies, the read leaves its sink alone, and the clock
+    stamps of a block are ordered (start <= end, all within one launch's few microseconds)."""
+    k = _k()
+    n = 1 << 20                                   # 4 MiB of floats
+    src = torch.arange(n, dtype=torch.float32, device=device)
+    dst = torch.zeros_like(src)
+    blocks = n * 4 // 16384
+    stamps = torch.zeros(blocks, 2, dtype=torch.int64, device=device)
+    k.stream_yardstick(k.YARDSTICK_COPY, src, dst, n * 4, stamps=stamps)
+    assert torch.equal(src, dst)
+    st = stamps.cpu().numpy()
+    assert (st[:, 0] > 0).all() and (st[:, 1] >= st[:, 0]).all()
+    assert (st[:, 1].max() - st[:, 0].min()) * 0.01 < 1000.0       # 100 MHz clock: well under a millisecond
+    sink = torch.zeros(n * 4 // 32768, dtype=torch.int32, device=device)
+    k.stream_yardstick(k.YARDSTICK_READ, src, sink, n * 4)
+    assert int(sink.abs().sum().item()) == 0
+    with pytest.raises(k.RmlkError):
+        k.stream_yardstick(k.YARDSTICK_COPY, src, dst, 1000)     # not whole 16 KiB blocks
