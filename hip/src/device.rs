@@ -83,6 +83,26 @@ impl<T: Copy> DeviceBuffer<T> {
         Ok(host)
     }
 
+    /// Device-to-device copy of `src` into this buffer (what Reshape and Unsqueeze do in the
+    /// reference, runtime/src/providers/cuda/backend/reshape.rs:46), ordered on `stream`.
+    pub fn copy_from_device(&mut self, stream: &HipStream, src: &DeviceBuffer<T>) -> Result<()> {
+        if src.len != self.len {
+            return Err(crate::Error::InvalidArguments("copy_from_device: lengths differ".into()));
+        }
+        check(
+            unsafe { ffi::rmlk_hip_memcpy_dtod(stream.raw(), self.ptr, src.ptr, self.len * std::mem::size_of::<T>()) },
+            "memcpy_dtod",
+        )
+    }
+
+    /// Every byte of the buffer becomes `byte` (a fill kernel: safe to record into a HIP graph).
+    pub fn memset(&mut self, stream: &HipStream, byte: u8) -> Result<()> {
+        check(
+            unsafe { ffi::rmlk_hip_memset(stream.raw(), self.ptr, byte as i32, self.len * std::mem::size_of::<T>()) },
+            "memset",
+        )
+    }
+
     pub fn len(&self) -> usize {
         self.len
     }
@@ -106,6 +126,13 @@ impl<T> Drop for DeviceBuffer<T> {
             unsafe { ffi::rmlk_hip_free(self.ptr) };
         }
     }
+}
+
+/// Name, architecture, compute units, wavefront size, LDS per block, clock and memory of a GPU.
+pub fn device_info(device: i32) -> Result<ffi::rmlk_device_info> {
+    let mut info = std::mem::MaybeUninit::<ffi::rmlk_device_info>::zeroed();
+    check(unsafe { ffi::rmlk_hip_device_info(device, info.as_mut_ptr()) }, "device_info")?;
+    Ok(unsafe { info.assume_init() })
 }
 
 /// A shape or stride vector as the kernels take it (by value, at most 8 dims).

@@ -39,3 +39,39 @@ pub fn compute<T: HipType>(
         "concat",
     )
 }
+
+/// One input written into its place along `axis` of the output, `axis_offset` elements in: the
+/// per-input step of runtime/src/providers/cuda/backend/concat.rs:28-76 for callers that hold their
+/// inputs one at a time.
+pub fn compute_one<T: HipType>(
+    stream: &HipStream,
+    in_shape: &[usize],
+    input: &DeviceBuffer<T>,
+    out_shape: &[usize],
+    axis: usize,
+    axis_offset: usize,
+    output: &mut DeviceBuffer<T>,
+) -> Result<()> {
+    if axis >= out_shape.len() || in_shape.len() != out_shape.len() {
+        return Err(Error::InvalidArguments("concat: axis or rank does not match the output".into()));
+    }
+    if input.len() != in_shape.iter().product::<usize>() || output.len() != out_shape.iter().product::<usize>() {
+        return Err(Error::InvalidArguments("concat: buffer lengths do not match the shapes".into()));
+    }
+    let (is, os) = (dims(in_shape)?, dims(out_shape)?);
+    check(
+        unsafe {
+            ffi::rmlk_hip_concat(
+                stream.raw(),
+                T::DTYPE,
+                &is,
+                &os,
+                axis as i32,
+                axis_offset as i64,
+                input.as_ptr(),
+                output.as_mut_ptr(),
+            )
+        },
+        "concat",
+    )
+}

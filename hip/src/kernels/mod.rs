@@ -9,6 +9,7 @@ pub mod cos;
 pub mod div;
 pub mod equal;
 pub mod expand;
+pub mod fill;
 pub mod fused;
 pub mod gather;
 pub mod gemm;

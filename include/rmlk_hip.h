@@ -15,7 +15,13 @@
  *     (the memory helpers at the end are the exception and say so).
  *   - Tensors are dense row-major unless a stride argument says otherwise. Strides are in ELEMENTS.
  *   - A call whose output has zero elements returns 0 without launching.
- *   - No global mutable state: calls on distinct streams may be made from distinct threads.
+ *   - Thread safety: calls on distinct streams may be made from distinct threads. The library keeps
+ *     three pieces of process-wide state, each safe under that rule: a per-device note that a
+ *     kernel's dynamic LDS limit has been raised (written once); the list of open batches of
+ *     rmlk_hip_batch_begin / _flush / _end, guarded by a mutex and keyed by stream (two threads must
+ *     not drive ONE stream while it has a batch open); and the per-device address of the fixed
+ *     32 MiB scratch array of rmlk_hip_matmul_noalloc, looked up once per device — calls of THAT
+ *     entry point which overlap in time on one GPU share the array and race, whatever their streams.
  */
 #ifndef RMLK_HIP_H
 #define RMLK_HIP_H
@@ -170,7 +176,10 @@ int32_t rmlk_hip_matmul_describe(int32_t dtype, int64_t batch, int64_t m, int64_
  * tight serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same
  * arguments and results as rmlk_hip_matmul (bit for bit) without the workspace: the split-K partials
  * go to a fixed device array of RMLK_HIP_MATMUL_NOALLOC_SCRATCH_BYTES that is part of the library's
- * code object (every GPU the library runs on holds its copy until the process ends). A problem whose
+ * code object (every GPU the library runs on holds its copy until the process ends: 32 MiB of
+ * device memory per GPU and per process that loads the library, whether or not this entry point is
+ * ever called). The first call on a device looks the array's address up (hipGetSymbolAddress) and
+ * must therefore be made OUTSIDE stream capture; every later call on that device does not. A problem whose
  * rmlk_hip_matmul_workspace_size exceeds that returns RMLK_ERR_SCRATCH_LIMIT and launches nothing.
  * The call allocates nothing and frees nothing. All calls on one GPU share the array: calls that may
  * overlap in time on one GPU (different streams, different threads) race on it and must be ordered

@@ -587,6 +587,15 @@ void Session::check_error_flag() {
     }
 }
 
+// The one-launch decode attention counts the blocks that have finished a KV head in
+// `block_counters` and expects them zero on entry; it leaves them zero when it completes. A run that
+// fails between launches may not have completed one: put the zeros back (a fill kernel, best effort
+// — the error that is being reported wins) so that later runs of the session still merge.
+static void rezero_block_counters(Session &s) {
+    if (s.block_counters)
+        (void)rmlk_hip_memset(s.stream, s.block_counters, 0, Session::kBlockCounters * sizeof(int32_t));
+}
+
 static void clear_flag(Session &s) {
     int32_t zero = 0;
     check_status(rmlk_hip_write_small(s.stream, s.err_flag, &zero, sizeof(zero)), "clear flag");
@@ -601,7 +610,12 @@ void Session::run() {
         if (!val.is_initializer && !val.is_input) values[v].reset();
     }
     clear_flag(*this);
-    run_nodes();
+    try {
+        run_nodes();
+    } catch (...) {
+        rezero_block_counters(*this);
+        throw;
+    }
     check_error_flag();
     if (profiling) {
         for (auto &st : stats) {
@@ -647,6 +661,7 @@ void Session::capture() {
         if (dead) (void)hipGraphDestroy(dead);
         capturing = false;
         pool.forbid_malloc = false;
+        rezero_block_counters(*this);
         throw;
     }
     capturing = false;

@@ -71,3 +71,68 @@ def test_kernel_modules_exist_for_the_reference_layout():
               "sigmoid", "cast", "expand", "gemm", "reduce_mean", "scatter_nd", "slice", "softmax", "transpose",
               "trilu", "whereop"):
         assert m in mods, m
+
+
+def _call_sites():
+    """(entry point, number of arguments, file) of every `ffi::rmlk_hip_*( .. )` call under hip/src."""
+    out = []
+    src_dir = os.path.join(ROOT, "hip", "src")
+    for base, _, files in os.walk(src_dir):
+        for fn in files:
+            if not fn.endswith(".rs") or fn == "ffi.rs":
+                continue
+            text = open(os.path.join(base, fn)).read()
+            text = re.sub(r"//[^\n]*", "", text)
+            for m in re.finditer(r"ffi::(rmlk_hip_\w+)\s*\(", text):
+                depth, i, args, cur = 1, m.end(), [], ""
+                while depth and i < len(text):
+                    ch = text[i]
+                    if ch in "([{":
+                        depth += 1
+                    elif ch in ")]}":
+                        depth -= 1
+                        if depth == 0:
+                            break
+                    if ch == "," and depth == 1:
+                        args.append(cur)
+                        cur = ""
+                    else:
+                        cur += ch
+                    i += 1
+                if cur.strip():
+                    args.append(cur)
+                out.append((m.group(1), len(args), os.path.relpath(os.path.join(base, fn), ROOT)))
+    return out
+
+
+def _bound():
+    with open(FFI) as f:
+        ffi = f.read()
+    return {m.group(1): len([a for a in m.group(2).split(",") if a.strip()])
+            for m in re.finditer(r"pub fn (rmlk_hip_\w+)\(([^)]*)\)", ffi, flags=re.S)}
+
+
+def test_every_call_site_passes_the_declared_number_of_arguments():
+    """The crate cannot be compiled here; this is the part of the compiler's job that text can do."""
+    bound = _bound()
+    sites = _call_sites()
+    assert len(sites) >= 45
+    wrong = [(name, n, bound.get(name), path) for name, n, path in sites if bound.get(name) != n]
+    assert not wrong, wrong
+
+
+def test_entry_points_the_reference_backends_need_are_wrapped():
+    """Operators of the reference whose backends have no kernel-crate module (they move or build data
+    through cudarc: backend/reshape.rs:46, constant_of_shape.rs:59-62, range.rs:140-151, shape.rs:67-72,
+    concat.rs:28-76) still need these entry points from the Rust side."""
+    called = {name for name, _, _ in _call_sites()}
+    for need in ("rmlk_hip_fill", "rmlk_hip_range", "rmlk_hip_memcpy_dtod", "rmlk_hip_concat",
+                 "rmlk_hip_concat_many", "rmlk_hip_device_info", "rmlk_hip_write_small", "rmlk_hip_memset",
+                 "rmlk_hip_malloc", "rmlk_hip_free", "rmlk_hip_memcpy_htod", "rmlk_hip_memcpy_dtoh",
+                 "rmlk_hip_stream_sync", "rmlk_hip_status_string"):
+        assert need in called, need
+    # one wrapper per kernel row of the operator path
+    for need in ("rmlk_hip_binary", "rmlk_hip_where", "rmlk_hip_unary", "rmlk_hip_cast", "rmlk_hip_reduce_mean",
+                 "rmlk_hip_softmax", "rmlk_hip_matmul", "rmlk_hip_transpose", "rmlk_hip_expand", "rmlk_hip_slice",
+                 "rmlk_hip_gather", "rmlk_hip_scatter_nd", "rmlk_hip_trilu"):
+        assert need in called, need
