@@ -366,6 +366,28 @@ int32_t rmlk_hip_attention_ws(rmlk_stream_t stream, int32_t dtype, int64_t batch
                               const void *q, const void *k, const void *v, const void *mask,
                               const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
                               int32_t out_seq_major, void *workspace, size_t workspace_bytes, void *out);
+/* The map of rmlk_hip_attention_ws made once and used by several launches over ONE mask (the layers
+ * of a model share theirs): rmlk_hip_attention_map marks in `map` (rmlk_hip_attention_map_size()
+ * bytes, 16-byte aligned) which (query tile, key chunk) pairs of `mask` hold anything but -inf;
+ * rmlk_hip_attention_mapped is rmlk_hip_attention_ws over such a map, without making it again - the
+ * same results bit for bit. The map belongs to the mask, its strides and the sizes it was made for;
+ * between two launches that use it it must not change (each launch leaves the item counter behind
+ * the map zero, as it found it), and launches that share it are ordered by one stream. Since the
+ * cost of the map is shared, two chunks are enough for it to exist: the size is 0 where skipping
+ * does not apply at all (q_len not a multiple of 64, fewer than 2 or more than 128 chunks), and the
+ * calls then answer RMLK_ERR_UNSUPPORTED. No counterpart in the reference. */
+size_t rmlk_hip_attention_map_size(int32_t dtype, int64_t batch, int64_t kv_heads, int64_t rep,
+                                   int64_t q_len, int64_t kv_len, int64_t head_dim,
+                                   const rmlk_dims *mask_stride);
+int32_t rmlk_hip_attention_map(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t kv_heads,
+                               int64_t rep, int64_t q_len, int64_t kv_len, int64_t head_dim,
+                               const void *mask, const rmlk_dims *mask_stride, void *map,
+                               size_t map_bytes);
+int32_t rmlk_hip_attention_mapped(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t kv_heads,
+                                  int64_t rep, int64_t q_len, int64_t kv_len, int64_t head_dim,
+                                  const void *q, const void *k, const void *v, const void *mask,
+                                  const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
+                                  int32_t out_seq_major, const void *map, size_t map_bytes, void *out);
 /* rmlk_hip_attention_ws with a [batch, q_len, heads, head_dim] result (out_seq_major) that is also
  * stored as three bfloat16 pieces, as rmlk_hip_bf16x3_split would split the [batch * q_len, heads *
  * head_dim] matrix it is: `out_pieces` holds rmlk_hip_bf16x3_pieces_size(batch * q_len, heads *

@@ -150,6 +150,12 @@ SIGNATURES = {
     "rmlk_hip_attention_ws": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64,
                                         c_int64, c_void_p, c_void_p, c_void_p, c_void_p, _PD, c_int32,
                                         ctypes.c_float, c_int32, c_void_p, c_size_t, c_void_p]),
+    "rmlk_hip_attention_map_size": (c_size_t, [c_int32, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, _PD]),
+    "rmlk_hip_attention_map": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                         c_int64, c_void_p, _PD, c_void_p, c_size_t]),
+    "rmlk_hip_attention_mapped": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                            c_int64, c_void_p, c_void_p, c_void_p, c_void_p, _PD, c_int32,
+                                            ctypes.c_float, c_int32, c_void_p, c_size_t, c_void_p]),
     "rmlk_hip_attention_ws_pieces": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64,
                                                c_int64, c_void_p, c_void_p, c_void_p, c_void_p, _PD, c_int32,
                                                ctypes.c_float, c_void_p, c_size_t, c_void_p, c_void_p]),

@@ -123,7 +123,14 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
         if (tid == 0) next_item = atomicAdd(g.queue, 1);
         __syncthreads();
         const int item = next_item;
-        if (item >= g.items) break;   // every block ends here: the counter only grows
+        if (item >= g.items) {
+            // every block ends here, with a ticket of its own: the counter only grows, and the block
+            // that draws the last ticket of the launch leaves the counter as it found it (zero), so
+            // that the map and its counter serve another launch without being made again
+            if (tid == 0 && item == g.items + static_cast<int>(gridDim.x) - 1)
+                __hip_atomic_store(g.queue, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
         // items by falling query tile; inside one tile index, all the heads of all the KV heads
         const int n_bg = g.items / (g.tiles_per_head * g.rep);
         const int per_tile = n_bg * g.rep;
@@ -724,8 +731,10 @@ struct TileMapDims {
     int keys;   // keys of a chunk: what the kernel that will run takes per step
     size_t map_bytes, bytes;
 };
+// shared: the map serves several launches over one mask (the layers of a model), so making it is
+// no cost to weigh against what one launch skips: two chunks are enough.
 TileMapDims tile_map_dims(int64_t batch, int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
-                          const rmlk_dims *mask_stride) {
+                          const rmlk_dims *mask_stride, bool shared = false) {
     TileMapDims d{};
     if (batch <= 0 || kv_heads <= 0 || rep <= 0 || q_len <= 0 || kv_len <= 0 || !dims_ok(mask_stride) ||
         mask_stride->rank != 4)
@@ -737,7 +746,7 @@ TileMapDims tile_map_dims(int64_t batch, int64_t kv_heads, int64_t rep, int64_t 
     const bool many_blocks = blocks > kNumCU;
     d.keys = many_blocks ? AttnShape<2>::kKeys : AttnShape<4>::kKeys;
     d.chunks = (kv_len + d.keys - 1) / d.keys;
-    if (q_len % 64 != 0 || d.chunks < (many_blocks ? 4 : 6) || d.chunks > 128) return d;
+    if (q_len % 64 != 0 || d.chunks < (shared ? 2 : many_blocks ? 4 : 6) || d.chunks > 128) return d;
     d.mask_batches = mask_stride->v[0] ? batch : 1;
     d.mask_heads = mask_stride->v[1] ? kv_heads * rep : 1;
     d.tiles = q_len / 64;
@@ -760,12 +769,20 @@ int32_t attention_many_rows(rmlk_stream_t stream, int32_t dtype, int64_t batch, 
                             int64_t q_len, int64_t kv_len, int64_t head_dim, const void *q, const void *k,
                             const void *v, const void *mask, const rmlk_dims *mask_stride, int32_t scale_is_mul,
                             float scale, int32_t out_seq_major, void *workspace, size_t workspace_bytes, void *out,
-                            void *out_pieces) {
+                            void *out_pieces, int map_state = 0) {
+    // map_state 0: the workspace is room for a map that this call makes and uses; 1: only make the
+    // shared map (no attention launch); 2: the workspace holds a shared map made by state 1
     AttnArgs g{};
     bool empty = false;
     const int32_t st = attention_args(dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
                                       mask_stride, scale_is_mul, scale, out_seq_major, out, true, &g, &empty);
     if (st || empty) return st;
+    if (map_state != 0) {
+        const TileMapDims tm = tile_map_dims(batch, kv_heads, rep, q_len, kv_len, mask_stride, true);
+        if (!tm.bytes) return RMLK_ERR_UNSUPPORTED;
+        if (!workspace || workspace_bytes < tm.bytes || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+            return RMLK_ERR_WORKSPACE;
+    }
     if (out_pieces) {
         // the pieces of the [batch * q_len, heads * head_dim] matrix that a [B, S, H, D] result is
         if (!out_seq_major || reinterpret_cast<uintptr_t>(out_pieces) % 16 != 0) return RMLK_ERR_UNSUPPORTED;
@@ -776,12 +793,14 @@ int32_t attention_many_rows(rmlk_stream_t stream, int32_t dtype, int64_t batch, 
     dim3 grid(static_cast<unsigned>((g.rows + 63) / 64), static_cast<unsigned>(batch * kv_heads), 1);
     const bool many_blocks = static_cast<int64_t>(grid.x) * grid.y > kNumCU;
     {
-        const TileMapDims tm = tile_map_dims(batch, kv_heads, rep, q_len, kv_len, mask_stride);
+        const TileMapDims tm = tile_map_dims(batch, kv_heads, rep, q_len, kv_len, mask_stride, map_state != 0);
         if (workspace && tm.bytes && workspace_bytes >= tm.bytes && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
             uint8_t *tiles = static_cast<uint8_t *>(workspace);
             const dim3 tgrid(static_cast<unsigned>(tm.chunks), static_cast<unsigned>(tm.tiles),
                              static_cast<unsigned>(tm.mask_batches * tm.mask_heads));
-            if (tm.keys == 64)
+            if (map_state == 2) {
+                // made by an earlier call; its counter is zero again
+            } else if (tm.keys == 64)
                 attention_mask_tiles_kernel<64><<<tgrid, 256, 0, as_stream(stream)>>>(
                     g.mask, g.mask_b, g.mask_h, g.mask_s, static_cast<int32_t>(tm.mask_heads), g.seq, g.len, tiles,
                     reinterpret_cast<int32_t *>(tiles + tm.map_bytes));
@@ -790,7 +809,7 @@ int32_t attention_many_rows(rmlk_stream_t stream, int32_t dtype, int64_t batch, 
                     g.mask, g.mask_b, g.mask_h, g.mask_s, static_cast<int32_t>(tm.mask_heads), g.seq, g.len, tiles,
                     reinterpret_cast<int32_t *>(tiles + tm.map_bytes));
             const int32_t launched = launch_status();
-            if (launched) return launched;
+            if (launched || map_state == 1) return launched;
             g.tiles = tiles;
             g.tiles_h = mask_stride->v[1] ? tm.tiles * tm.chunks : 0;
             g.tiles_b = mask_stride->v[0] ? tm.mask_heads * tm.tiles * tm.chunks : 0;
@@ -839,6 +858,32 @@ extern "C" int32_t rmlk_hip_attention_ws_pieces(rmlk_stream_t stream, int32_t dt
     if (!out_pieces) return RMLK_ERR_NULL_POINTER;
     return attention_many_rows(stream, dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
                                mask_stride, scale_is_mul, scale, 1, workspace, workspace_bytes, out, out_pieces);
+}
+
+extern "C" size_t rmlk_hip_attention_map_size(int32_t dtype, int64_t batch, int64_t kv_heads, int64_t rep,
+                                              int64_t q_len, int64_t kv_len, int64_t head_dim,
+                                              const rmlk_dims *mask_stride) {
+    if (dtype != RMLK_FLOAT || head_dim != kHeadDim) return 0;
+    return tile_map_dims(batch, kv_heads, rep, q_len, kv_len, mask_stride, true).bytes;
+}
+
+extern "C" int32_t rmlk_hip_attention_map(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t kv_heads,
+                                          int64_t rep, int64_t q_len, int64_t kv_len, int64_t head_dim,
+                                          const void *mask, const rmlk_dims *mask_stride, void *map,
+                                          size_t map_bytes) {
+    // (q, k, v and out only have to pass the argument checks: the map is made of the mask alone)
+    return attention_many_rows(stream, dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, mask, mask, mask, mask,
+                               mask_stride, 1, 1.0f, 0, map, map_bytes, const_cast<void *>(mask), nullptr, 1);
+}
+
+extern "C" int32_t rmlk_hip_attention_mapped(rmlk_stream_t stream, int32_t dtype, int64_t batch, int64_t kv_heads,
+                                             int64_t rep, int64_t q_len, int64_t kv_len, int64_t head_dim,
+                                             const void *q, const void *k, const void *v, const void *mask,
+                                             const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
+                                             int32_t out_seq_major, const void *map, size_t map_bytes, void *out) {
+    return attention_many_rows(stream, dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
+                               mask_stride, scale_is_mul, scale, out_seq_major, const_cast<void *>(map), map_bytes,
+                               out, nullptr, 2);
 }
 
 extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch,

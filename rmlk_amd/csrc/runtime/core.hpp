@@ -295,6 +295,15 @@ struct Session {
     static constexpr int64_t kBlockCounters = 1024;
     int32_t *block_counters = nullptr;
     int32_t *err_host = nullptr;     // pinned host
+    // The attention kernel's map of the (query tile, key chunk) pairs a mask leaves visible, made by
+    // the first attention node of a run that reads a mask and used by the later ones that read the
+    // same value with the same sizes (the layers of a model share their mask); dropped when the run ends.
+    struct AttentionMap {
+        int mask_value = -1;           // graph value id of the mask
+        int64_t sizes[6] = {0, 0, 0, 0, 0, 0};   // batch, kv heads, rep, q_len, kv_len, head dim
+        rmlk_dims strides{};
+        Tensor map;
+    } attention_map;
     bool capturing = false;
     bool profiling = false;
     bool fuse = true;                // form fused nodes while building

@@ -1627,6 +1627,43 @@ void op_fused_attention(OpContext &c) {
             const bool seq_major = c.attr_int("seq_major_output", 0) != 0;
             Tensor &y = seq_major ? c.alloc_output(0, RMLK_FLOAT, {bsz, seq, heads, dim})
                                   : c.alloc_output(0, RMLK_FLOAT, {bsz, heads, seq, dim});
+            // The map of (query tile, key chunk) pairs the mask leaves visible, kept for the other
+            // attention nodes of this run that read the same mask (a pool buffer that lives until the
+            // run ends; the session's workspace is overwritten by the products in between).
+            const int mask_value = c.node.inputs.size() > 2 ? c.node.inputs[2] : -1;
+            const size_t shared_bytes =
+                mask_value >= 0 && !c.session.bf16_pieces   // (the launch that also stores pieces makes its own map)
+                    ? rmlk_hip_attention_map_size(RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, &ms)
+                    : 0;
+            if (shared_bytes) {
+                Session::AttentionMap &am = c.session.attention_map;
+                const int64_t sizes[6] = {bsz, grp, rep_k, seq, len, dim};
+                bool same = am.map.defined() && am.mask_value == mask_value && am.strides.rank == ms.rank &&
+                            am.map.nbytes() == shared_bytes;
+                for (int i = 0; i < 6 && same; ++i) same = am.sizes[i] == sizes[i];
+                for (int i = 0; i < ms.rank && same; ++i) same = am.strides.v[i] == ms.v[i];
+                int32_t st = RMLK_OK;
+                if (!same) {
+                    am.map.reset();
+                    std::vector<Tensor *> keep = c.out;
+                    c.out = {&am.map};
+                    c.alloc_output(0, RMLK_UINT8, {static_cast<int64_t>(shared_bytes)});
+                    c.out = keep;
+                    am.mask_value = mask_value;
+                    am.strides = ms;
+                    for (int i = 0; i < 6; ++i) am.sizes[i] = sizes[i];
+                    st = rmlk_hip_attention_map(c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, mask.data(), &ms,
+                                                am.map.data(), shared_bytes);
+                    if (st) am.map.reset();
+                }
+                if (!st && took_fast_path(rmlk_hip_attention_mapped(
+                                              c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, q.data(), k.data(),
+                                              v.data(), mask.data(), &ms,
+                                              static_cast<int32_t>(c.attr_int("scale_is_mul", 0)), attr_float(c, "scale"),
+                                              seq_major ? 1 : 0, am.map.data(), shared_bytes, y.data()),
+                                          "rmlk.Attention"))
+                    return;
+            }
             // room for the map of (query tile, key chunk) pairs the mask leaves visible, when it pays
             const size_t map_bytes = rmlk_hip_attention_workspace_size(RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, &ms);
             void *map = map_bytes ? c.scratch(map_bytes) : nullptr;

@@ -445,6 +445,8 @@ void Session::build(const rmlk_graph &graph, int dev) {
 void Session::run_nodes() {
     const rmlk_graph &gr = graph_copy;
     products_bf16_pieces = 0;
+    attention_map.map.reset();   // (a run that ended in an error may have left one)
+    attention_map.mask_value = -1;
     // Operators over tiny tensors (the per-step set-up of a decoder graph: tables, indices, masks) are
     // collected by the kernel library and go out as one launch in front of the next larger one. Not
     // with one kernel per node (no fusion), and not while nodes are timed one by one.
@@ -573,6 +575,8 @@ void Session::run_nodes() {
         check_status(rmlk_hip_batch_end(stream), "collected launches");
     }
     scratch_bufs.clear();
+    attention_map.map.reset();
+    attention_map.mask_value = -1;
 }
 
 void Session::check_error_flag() {

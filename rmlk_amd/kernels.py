@@ -287,6 +287,30 @@ def attention_skipping(q, k, v, mask, out, batch: int, kv_heads: int, rep: int, 
     return need
 
 
+def attention_map(mask, batch: int, kv_heads: int, rep: int, q_len: int, kv_len: int, head_dim: int,
+                  mask_stride):
+    """The map of visible (query tile, key chunk) pairs of `mask`, made once for several launches of
+    `attention_mapped` over that mask; None where skipping does not apply to the shape."""
+    ms = Dims.of(mask_stride)
+    need = int(lib().rmlk_hip_attention_map_size(dtype_of(mask), batch, kv_heads, rep, q_len, kv_len, head_dim, ms))
+    if need == 0:
+        return None
+    m = torch.empty(need, dtype=torch.uint8, device=mask.device)
+    check(lib().rmlk_hip_attention_map(_stream(), dtype_of(mask), batch, kv_heads, rep, q_len, kv_len, head_dim,
+                                       _ptr(mask), ms, _ptr(m), need), "rmlk_hip_attention_map")
+    return m
+
+
+def attention_mapped(q, k, v, mask, out, tile_map, batch: int, kv_heads: int, rep: int, q_len: int, kv_len: int,
+                     head_dim: int, mask_stride, scale: float, scale_is_mul: bool = False,
+                     out_seq_major: bool = False) -> None:
+    """`attention_skipping` over a map that `attention_map` made for this mask and these sizes."""
+    check(lib().rmlk_hip_attention_mapped(_stream(), dtype_of(q), batch, kv_heads, rep, q_len, kv_len, head_dim,
+                                          _ptr(q), _ptr(k), _ptr(v), _ptr(mask), Dims.of(mask_stride),
+                                          int(scale_is_mul), float(scale), int(out_seq_major), _ptr(tile_map),
+                                          tile_map.numel(), _ptr(out)), "rmlk_hip_attention_mapped")
+
+
 def attention_few_rows(q, k, v, mask, out, batch: int, kv_heads: int, rep: int, q_len: int, kv_len: int,
                        head_dim: int, mask_stride, scale: float, scale_is_mul: bool = False,
                        out_seq_major: bool = False) -> None:

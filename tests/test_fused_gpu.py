@@ -1211,6 +1211,62 @@ def test_attention_skipping_hidden_chunks_is_bit_identical(device, b, g, rep, s,
         assert np.isnan(out[0, 64:128, 0]).all() and np.isfinite(out[0, :64, 0]).all()
 
 
+@pytest.mark.parametrize("b,g,rep,s,l,mask_shape,kind", [
+    (1, 8, 4, 2048, 2048, (1, 1, 2048, 2048), "causal"),    # items handed out from the counter
+    (1, 8, 4, 512, 640, (1, 1, 512, 640), "causal"),        # a block per compute unit, five chunks of 128
+    (1, 8, 4, 2048, 128, (1, 1, 2048, 128), "causal"),      # two chunks of 64
+    (2, 4, 3, 1024, 1024, (2, 12, 1024, 1024), "tiles"),    # per batch and head, tiles that see nothing
+    (1, 1, 1, 192, 900, (1, 1, 192, 900), "window"),
+    (1, 8, 4, 512, 256, (1, 1, 1, 256), "row"),             # two chunks of 128
+])
+def test_attention_over_a_shared_map_is_bit_identical(device, b, g, rep, s, l, mask_shape, kind):
+    """One map of the mask, made once, serves several launches with different q, k, v (the layers of a
+    model): each equals the kernel that visits every chunk bit for bit, the counter behind the map is
+    zero again after every launch, and the map itself is left alone."""
+    import torch
+    kk = _k()
+    h, d = g * rep, 64
+    rng = np.random.default_rng(s + 3 * l + b)
+    m = to_dev(_skipping_mask(kind, rng, mask_shape, l), device)
+    ms = bcast_strides(list(mask_shape), [b, h, s, l])
+    tile_map = kk.attention_map(m, b, g, rep, s, l, d, ms)
+    assert tile_map is not None
+    before = to_np(tile_map).copy()
+    keys = 64 if b * g * (rep * s // 64) > 256 else 128
+    entries = mask_shape[0] * mask_shape[1] * (s // 64) * ((l + keys - 1) // keys)   # (then padding to 16 bytes)
+    assert before.size == (entries + 15) // 16 * 16 + 16
+    assert before[-16:-12].view(np.int32)[0] == 0 and set(np.unique(before[:entries])) <= {0, 1}
+    assert 0 < before[:entries].sum() < entries
+    for layer in range(3):
+        q, k, v = (to_dev(rng.standard_normal(sh, dtype=np.float32), device)
+                   for sh in ((b, h, s, d), (b, g, l, d), (b, g, l, d)))
+        seq_major = layer == 1
+        shape = (b, s, h, d) if seq_major else (b, h, s, d)
+        plain = torch.full(shape, 7.0, device=device)
+        kk.attention(q, k, v, m, plain, b, g, rep, s, l, d, ms, 8.0, False, out_seq_major=seq_major)
+        got = torch.full(shape, 9.0, device=device)
+        kk.attention_mapped(q, k, v, m, got, tile_map, b, g, rep, s, l, d, ms, 8.0, False, out_seq_major=seq_major)
+        a, e = to_np(got), to_np(plain)
+        assert np.array_equal(np.isnan(a), np.isnan(e))
+        assert_exact(np.nan_to_num(a, nan=0.0), np.nan_to_num(e, nan=0.0))
+        assert np.array_equal(to_np(tile_map), before)
+
+
+def test_attention_map_refusals(device):
+    import torch
+    kk = _k()
+    m = torch.zeros(1, 1, 100, 256, device=device)                  # q_len not a multiple of 64
+    assert kk.attention_map(m, 1, 8, 4, 100, 256, 64, [0, 0, 256, 1]) is None
+    m = torch.zeros(1, 1, 512, 64, device=device)                   # a single chunk
+    assert kk.attention_map(m, 1, 8, 4, 512, 64, 64, [0, 0, 64, 1]) is None
+    m = torch.zeros(1, 1, 512, 640, device=device)
+    q = torch.zeros(1, 32, 512, 64, device=device)
+    kv = torch.zeros(1, 8, 640, 64, device=device)
+    small = torch.zeros(16, dtype=torch.uint8, device=device)
+    with pytest.raises(kk.RmlkError):                               # a map that is too small
+        kk.attention_mapped(q, kv, kv, m, torch.empty_like(q), small, 1, 8, 4, 512, 640, 64, [0, 0, 640, 1], 8.0)
+
+
 def test_attention_workspace_that_is_too_small_is_not_used(device):
     """A workspace below the size the library names is ignored (every chunk is visited): nothing is
     written to it and the result is the plain kernel's."""
