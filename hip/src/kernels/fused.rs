@@ -363,6 +363,97 @@ pub unsafe fn attention(
     )
 }
 
+/// Bytes of a map of the mask's visible (query tile, key chunk) pairs that several `attention_mapped`
+/// calls over one mask share (0: skipping does not apply to this shape).
+pub fn attention_map_size(shape: &AttentionShape, mask_stride: &[usize; 4]) -> Result<usize> {
+    let ms = dims(mask_stride)?;
+    Ok(unsafe {
+        ffi::rmlk_hip_attention_map_size(
+            ffi::RMLK_FLOAT,
+            shape.batch as i64,
+            shape.kv_heads as i64,
+            shape.rep as i64,
+            shape.q_len as i64,
+            shape.kv_len as i64,
+            shape.head_dim as i64,
+            &ms,
+        )
+    })
+}
+
+/// Makes the map of `mask` in `map` (`attention_map_size` bytes, 16-byte aligned), once for all the
+/// layers that read the mask.
+pub unsafe fn attention_map(
+    stream: &HipStream,
+    shape: &AttentionShape,
+    mask: *const c_void,
+    mask_stride: &[usize; 4],
+    map: *mut c_void,
+    map_bytes: usize,
+) -> Result<()> {
+    let ms = dims(mask_stride)?;
+    check(
+        ffi::rmlk_hip_attention_map(
+            stream.raw(),
+            ffi::RMLK_FLOAT,
+            shape.batch as i64,
+            shape.kv_heads as i64,
+            shape.rep as i64,
+            shape.q_len as i64,
+            shape.kv_len as i64,
+            shape.head_dim as i64,
+            mask,
+            &ms,
+            map,
+            map_bytes,
+        ),
+        "attention_map",
+    )
+}
+
+/// `attention` over a map made by `attention_map` for this mask and these sizes (same bits).
+pub unsafe fn attention_mapped(
+    stream: &HipStream,
+    shape: &AttentionShape,
+    q: *const c_void,
+    k: *const c_void,
+    v: *const c_void,
+    mask: *const c_void,
+    mask_stride: &[usize; 4],
+    scale_is_mul: bool,
+    scale: f32,
+    out_seq_major: bool,
+    map: *const c_void,
+    map_bytes: usize,
+    out: *mut c_void,
+) -> Result<()> {
+    let ms = dims(mask_stride)?;
+    check(
+        ffi::rmlk_hip_attention_mapped(
+            stream.raw(),
+            ffi::RMLK_FLOAT,
+            shape.batch as i64,
+            shape.kv_heads as i64,
+            shape.rep as i64,
+            shape.q_len as i64,
+            shape.kv_len as i64,
+            shape.head_dim as i64,
+            q,
+            k,
+            v,
+            mask,
+            &ms,
+            scale_is_mul as i32,
+            scale,
+            out_seq_major as i32,
+            map,
+            map_bytes,
+            out,
+        ),
+        "attention_mapped",
+    )
+}
+
 /// `attention` with a `[batch, q_len, heads, head_dim]` result that is also stored as the three
 /// bfloat16 pieces `bf16x3_split` would make of it (`out_pieces`), for an output projection over them.
 pub unsafe fn attention_with_pieces(
