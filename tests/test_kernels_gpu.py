@@ -40,6 +40,12 @@ BCAST_CASES = [
     ((3, 1, 4), (1, 6, 1)),
     ((2, 2, 2, 2, 2, 2, 2, 2), (2, 1, 2, 1, 2, 1, 2, 1)),  # rank 8
     ((0, 4), (4,)),                  # empty
+    # one operand broadcast over a long outer dim above a long dense run (a mask under every head)
+    ((8, 65536), (65536,)),
+    ((65540,), (12, 65540)),                   # the broadcast operand first
+    ((1, 16, 256, 512), (1, 1, 256, 512)),
+    ((8, 65538), (65538,)),                    # inner run not in whole vectors
+    ((6, 65536), (65536,)),
 ]
 
 
