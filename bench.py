@@ -475,7 +475,39 @@ def run_ops_suite(args):
     # (before the first marker launch, so that a kernel trace split at the markers does not see them)
     half = n * 2
     sink = torch.zeros(4096, dtype=torch.int32, device=dev)
+    big = [torch.empty(CALIBRATION_COPY_BYTES // 4, device=dev) for _ in range(4)]
+    for t in big:
+        t.normal_(generator=g)
     clock = {}
+    # read-only launches of the sizes a decode step's one-row products stream (o 16 MiB, q/k/v 24,
+    # down 64, gate/up 128), rotating through 1 GiB: what a chain of such launches costs at the least
+    for mib in (16, 24, 64, 128):
+        nbytes = mib << 20
+        per_buf = CALIBRATION_COPY_BYTES // nbytes
+        pieces = [b_[j * (nbytes // 4):(j + 1) * (nbytes // 4)] for b_ in big for j in range(per_buf)]
+        blocks = nbytes // 32768
+        n_l = 48
+        stamps = torch.zeros(n_l, blocks, 2, dtype=torch.int64, device=dev)
+        with torch.cuda.stream(side):
+            fn = lambda i: k.stream_yardstick(k.YARDSTICK_READ, pieces[i % len(pieces)], sink, nbytes,  # noqa: E731
+                                              stamps=stamps[i % n_l], stream=side.cuda_stream)
+            for i in range(len(pieces)):
+                fn(i)
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(n_l):
+                    fn(i)
+            for _ in range(10 if args.ops_quick else 60):
+                graph.replay()
+            side.synchronize()
+        st = stamps.cpu().numpy().astype(np.int64)
+        first, last_end = st[:, :, 0].min(1), st[:, :, 1].max(1)
+        clock[f"read_{mib}MiB"] = {"launches": n_l,
+                                   "first_start_to_last_end_us": round(float(((last_end - first) * 0.01).mean()), 2),
+                                   "start_to_start_us": round(float(np.median((first[1:] - first[:-1]) * 0.01)), 2)}
+        log(f"[ops] in-kernel clock, read {mib} MiB: {clock[f'read_{mib}MiB']}")
+        del graph, stamps
     for name, kind, nbytes, blocks in (("read_33MB", k.YARDSTICK_READ, n * 4, n * 4 // 32768),
                                        ("copy_17MB_17MB", k.YARDSTICK_COPY, half, half // 16384),
                                        ("copy_33MB_33MB", k.YARDSTICK_COPY, n * 4, n * 4 // 16384)):
@@ -508,9 +540,6 @@ def run_ops_suite(args):
     # ---- yardsticks: an almost empty launch and a plain 256 MiB copy -------------------------------
     timed("launch_floor", lambda i: check(lib().rmlk_hip_fill(side.cuda_stream, k.INT32, 1, ctypes.byref(one),
                                                               marker.data_ptr()), "rmlk_hip_fill"), 1, 4)
-    big = [torch.empty(CALIBRATION_COPY_BYTES // 4, device=dev) for _ in range(4)]
-    for t in big:
-        t.normal_(generator=g)
     timed("copy_256MiB", lambda i: check(lib().rmlk_hip_memcpy_dtod(
         side.cuda_stream, big[2 + i % 2].data_ptr(), big[i % 2].data_ptr(), CALIBRATION_COPY_BYTES),
         "rmlk_hip_memcpy_dtod"), 2, 2 * CALIBRATION_COPY_BYTES)
