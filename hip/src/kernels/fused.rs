@@ -128,6 +128,179 @@ pub unsafe fn gemv_kmajor(
     )
 }
 
+/// `gemv_kmajor` with a residual row added to the outputs (the Add behind an output projection).
+pub unsafe fn gemv_kmajor_add(
+    stream: &HipStream,
+    n: usize,
+    k: usize,
+    x: *const c_void,
+    storage: WeightStorage,
+    wt: *const c_void,
+    ldw: usize,
+    residual: *const c_void,
+    y: *mut c_void,
+) -> Result<()> {
+    check(
+        ffi::rmlk_hip_gemv_kmajor_add(
+            stream.raw(),
+            ffi::RMLK_FLOAT,
+            n as i64,
+            k as i64,
+            x,
+            storage.dtype(),
+            wt,
+            ldw as i64,
+            residual,
+            y,
+        ),
+        "gemv_kmajor_add",
+    )
+}
+
+/// RMSNorm parameters of the products that normalise their input row themselves.
+#[derive(Clone, Copy, Debug)]
+pub struct RowNorm {
+    pub gamma: *const c_void,
+    pub eps: f32,
+    /// `x * (1 / rms)` instead of `x / rms` (the two decompositions exported graphs use).
+    pub reciprocal_form: bool,
+}
+
+/// `gemv_kmajor` over `RMSNorm(x) * gamma`, the norm formed by the kernel (the bits of the norm kernel
+/// followed by the product).
+pub unsafe fn gemv_kmajor_normed(
+    stream: &HipStream,
+    n: usize,
+    k: usize,
+    x: *const c_void,
+    norm: &RowNorm,
+    storage: WeightStorage,
+    wt: *const c_void,
+    ldw: usize,
+    y: *mut c_void,
+) -> Result<()> {
+    check(
+        ffi::rmlk_hip_gemv_kmajor_normed(
+            stream.raw(),
+            ffi::RMLK_FLOAT,
+            n as i64,
+            k as i64,
+            x,
+            norm.gamma,
+            norm.eps,
+            norm.reciprocal_form as i32,
+            storage.dtype(),
+            wt,
+            ldw as i64,
+            y,
+        ),
+        "gemv_kmajor_normed",
+    )
+}
+
+/// `y[i] = silu(wt[gate_row + i] . x) * (wt[up_row + i] . x)` over a joint [gate | up] matrix; with
+/// `norm` the input row is normalised first.
+pub unsafe fn gemv_kmajor_swiglu(
+    stream: &HipStream,
+    n: usize,
+    k: usize,
+    x: *const c_void,
+    norm: Option<&RowNorm>,
+    storage: WeightStorage,
+    wt: *const c_void,
+    ldw: usize,
+    gate_row: usize,
+    up_row: usize,
+    y: *mut c_void,
+) -> Result<()> {
+    match norm {
+        Some(nm) => check(
+            ffi::rmlk_hip_gemv_kmajor_swiglu_normed(
+                stream.raw(),
+                ffi::RMLK_FLOAT,
+                n as i64,
+                k as i64,
+                x,
+                nm.gamma,
+                nm.eps,
+                nm.reciprocal_form as i32,
+                storage.dtype(),
+                wt,
+                ldw as i64,
+                gate_row as i64,
+                up_row as i64,
+                y,
+            ),
+            "gemv_kmajor_swiglu_normed",
+        ),
+        None => check(
+            ffi::rmlk_hip_gemv_kmajor_swiglu(
+                stream.raw(),
+                ffi::RMLK_FLOAT,
+                n as i64,
+                k as i64,
+                x,
+                storage.dtype(),
+                wt,
+                ldw as i64,
+                gate_row as i64,
+                up_row as i64,
+                y,
+            ),
+            "gemv_kmajor_swiglu",
+        ),
+    }
+}
+
+/// Sets `*fits` (device memory, 1 before the call) to 0 when one of the `n` floats at `src` would not
+/// survive storage as `storage`.
+pub unsafe fn weights_fit(
+    stream: &HipStream,
+    storage: WeightStorage,
+    n: usize,
+    src: *const c_void,
+    fits: *mut i32,
+) -> Result<()> {
+    check(ffi::rmlk_hip_weights_fit(stream.raw(), storage.dtype(), n as i64, src, fits), "weights_fit")
+}
+
+/// Rotary embedding of `x` read through strides: `out = x * cos + rotate_half(x) * sin`.
+pub unsafe fn rotary(
+    stream: &HipStream,
+    shape: &[usize],
+    x_stride: &[usize],
+    cos_stride: &[usize],
+    sin_stride: &[usize],
+    x: *const c_void,
+    cos: *const c_void,
+    sin: *const c_void,
+    out: *mut c_void,
+) -> Result<()> {
+    let (sh, xs, cs, ss) = (dims(shape)?, dims(x_stride)?, dims(cos_stride)?, dims(sin_stride)?);
+    check(
+        ffi::rmlk_hip_rotary(stream.raw(), ffi::RMLK_FLOAT, &sh, &xs, &cs, &ss, x, cos, sin, out),
+        "rotary",
+    )
+}
+
+/// `Softmax(x (*|/) scale + mask)` along the last axis in one pass.
+pub unsafe fn scale_mask_softmax(
+    stream: &HipStream,
+    shape: &[usize],
+    mask_stride: &[usize],
+    scale_is_mul: bool,
+    scale: f32,
+    x: *const c_void,
+    mask: *const c_void,
+    out: *mut c_void,
+) -> Result<()> {
+    let (sh, ms) = (dims(shape)?, dims(mask_stride)?);
+    check(
+        ffi::rmlk_hip_scale_mask_softmax(stream.raw(), ffi::RMLK_FLOAT, &sh, &ms, scale_is_mul as i32, scale, x, mask, out),
+        "scale_mask_softmax",
+    )
+}
+
 /// Bytes that the three bfloat16 pieces of a dense float matrix `[m, k]` take (`bf16x3_split`).
 pub fn bf16x3_pieces_size(m: usize, k: usize) -> usize {
     unsafe { ffi::rmlk_hip_bf16x3_pieces_size(m as i64, k as i64) }
@@ -361,6 +534,94 @@ pub unsafe fn attention(
         ),
         "attention",
     )
+}
+
+/// Bytes of workspace of `attention_few_rows` (0: more than 16 query rows per KV head, not its case).
+pub fn attention_few_rows_workspace_size(shape: &AttentionShape) -> usize {
+    unsafe {
+        ffi::rmlk_hip_attention_few_rows_workspace_size(
+            ffi::RMLK_FLOAT,
+            shape.batch as i64,
+            shape.kv_heads as i64,
+            shape.rep as i64,
+            shape.q_len as i64,
+            shape.kv_len as i64,
+            shape.head_dim as i64,
+        )
+    }
+}
+
+/// The attention of a decode step (at most 16 query rows per KV head): the keys split over blocks,
+/// the chunks merged by the block that finishes a KV head last when `counters` (one `i32` per
+/// batch x KV head, zero before the first call and left zero) is given, by a second launch otherwise.
+pub unsafe fn attention_few_rows(
+    stream: &HipStream,
+    shape: &AttentionShape,
+    q: *const c_void,
+    k: *const c_void,
+    v: *const c_void,
+    mask: *const c_void,
+    mask_stride: &[usize; 4],
+    scale_is_mul: bool,
+    scale: f32,
+    out_seq_major: bool,
+    workspace: *mut c_void,
+    workspace_bytes: usize,
+    counters: Option<*mut i32>,
+    out: *mut c_void,
+) -> Result<()> {
+    let ms = dims(mask_stride)?;
+    match counters {
+        Some(cnt) => check(
+            ffi::rmlk_hip_attention_few_rows_one_launch(
+                stream.raw(),
+                ffi::RMLK_FLOAT,
+                shape.batch as i64,
+                shape.kv_heads as i64,
+                shape.rep as i64,
+                shape.q_len as i64,
+                shape.kv_len as i64,
+                shape.head_dim as i64,
+                q,
+                k,
+                v,
+                mask,
+                &ms,
+                scale_is_mul as i32,
+                scale,
+                out_seq_major as i32,
+                workspace,
+                workspace_bytes,
+                cnt,
+                out,
+            ),
+            "attention_few_rows_one_launch",
+        ),
+        None => check(
+            ffi::rmlk_hip_attention_few_rows(
+                stream.raw(),
+                ffi::RMLK_FLOAT,
+                shape.batch as i64,
+                shape.kv_heads as i64,
+                shape.rep as i64,
+                shape.q_len as i64,
+                shape.kv_len as i64,
+                shape.head_dim as i64,
+                q,
+                k,
+                v,
+                mask,
+                &ms,
+                scale_is_mul as i32,
+                scale,
+                out_seq_major as i32,
+                workspace,
+                workspace_bytes,
+                out,
+            ),
+            "attention_few_rows",
+        ),
+    }
 }
 
 /// Bytes of a map of the mask's visible (query tile, key chunk) pairs that several `attention_mapped`
