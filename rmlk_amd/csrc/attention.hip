@@ -117,20 +117,14 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     const int l32 = lane % 32, half = lane / 32;
     const int wq = wave / NK, wk = wave % NK;
     __shared__ int next_item;
+    // With a queue a block starts with the item of its own number (no ticket, so the blocks do not
+    // all meet at the counter when the kernel starts) and draws a ticket under the last step of
+    // every item it works on: ticket t stands for item t + gridDim.x. One ticket per item, so the
+    // tickets of a launch are 0 .. items - 1, the last gridDim.x of them for nothing.
+    int item = blockIdx.x, drawn = 0;
     for (;;) {
     int bg = blockIdx.y, tile_x = blockIdx.x;
     if (g.queue) {
-        if (tid == 0) next_item = atomicAdd(g.queue, 1);
-        __syncthreads();
-        const int item = next_item;
-        if (item >= g.items) {
-            // every block ends here, with a ticket of its own: the counter only grows, and the block
-            // that draws the last ticket of the launch leaves the counter as it found it (zero), so
-            // that the map and its counter serve another launch without being made again
-            if (tid == 0 && item == g.items + static_cast<int>(gridDim.x) - 1)
-                __hip_atomic_store(g.queue, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            break;
-        }
         // items by falling query tile; inside one tile index, all the heads of all the KV heads
         const int n_bg = g.items / (g.tiles_per_head * g.rep);
         const int per_tile = n_bg * g.rep;
@@ -253,6 +247,9 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     auto step = [&](int c, int next, int buf, auto more_tag) {
         constexpr bool MORE = decltype(more_tag)::value;
         const int key0 = c * kKeys + wk * 32 + 4 * half;
+        if constexpr (!MORE) {   // the ticket for the item after this one comes back under this step
+            if (g.queue && tid == 0) drawn = atomicAdd(g.queue, 1);
+        }
 
         // S^T (32 keys x 32 queries) = K . Q^T over the 64 head dims
         v16f st = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -370,7 +367,9 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
             mine[(18 + r) * kWave + lane] = o1[r];
         }
     }
+    if (g.queue && tid == 0) next_item = drawn + static_cast<int>(gridDim.x);
     __syncthreads();
+    const int following = next_item;
     if (wk == 0) {
         float m_f = m_run;
 #pragma unroll
@@ -413,6 +412,14 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
         }
     }
     if (!g.queue) break;
+    if (following >= g.items) {
+        // the counter only grows; the block that drew the last ticket of the launch leaves it as it
+        // found it (zero), so that the map and its counter serve another launch without being made again
+        if (tid == 0 && drawn == g.items - 1)
+            __hip_atomic_store(g.queue, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+    }
+    item = following;
     __syncthreads();   // the merge has read its slots, and thread 0 may write next_item again
     }
 }
