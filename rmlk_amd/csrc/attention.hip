@@ -105,7 +105,8 @@ __device__ __forceinline__ void store_pieces(const v4f &w, uint16_t *at, int64_t
     *reinterpret_cast<uint2 *>(at + 2 * plane) = uint2{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16)};
 }
 
-template <int NK>
+// WHOLE: the keys are a multiple of the step's, so every chunk lies inside them.
+template <int NK, bool WHOLE>
 __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel(AttnArgs g) {
     constexpr int kKeys = AttnShape<NK>::kKeys, kTile = AttnShape<NK>::kTile;
     extern __shared__ __align__(16) float smem[];
@@ -122,6 +123,12 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     // every item it works on: ticket t stands for item t + gridDim.x. One ticket per item, so the
     // tickets of a launch are 0 .. items - 1, the last gridDim.x of them for nothing.
     int item = blockIdx.x, drawn = 0;
+    // With a queue two blocks share a compute unit, a wavefront of each on every SIMD, and between
+    // wavefronts of equal priority the SIMD serves the older one first: left alone, the block that
+    // arrived first runs a sixth faster than its neighbour, and the slower blocks decide when the
+    // kernel ends. The wavefronts therefore change their priority with every step, the two
+    // neighbours (told apart by the wave slot they sit in, bits 3:0 of HW_ID) in opposite phase.
+    const int slot_bit = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (3 << 11)) & 1;
     for (;;) {
     int bg = blockIdx.y, tile_x = blockIdx.x;
     if (g.queue) {
@@ -181,14 +188,28 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
                      : "s"(lds_addr), "v"(voff), "s"(base)
                      : "memory", "m0");
     };
-    // piece p (0..3: K, 4..7: V) of chunk c into buffer buf
+    // Piece p (0..3: K, 4..7: V) of chunk c into buffer buf. WHOLE: the chunk and the piece move
+    // only the scalar base address, the lane's offset is the same for all of them, and no vector
+    // instruction is spent on addresses (fp32 MFMAs and vector ALU work share the SIMD's lanes on
+    // this chip: every such instruction costs matrix time). Otherwise rows past the end are read
+    // from the last row.
+    const uint32_t k_lane = static_cast<uint32_t>(lrow * kHeadDim + k_col) * 4u;
+    const uint32_t v_lane = static_cast<uint32_t>(lrow * kHeadDim + v_col) * 4u;
     auto issue_piece = [&](int p, int c, int buf) {
-        const int key = min(c * kKeys + (p & 3) * 8 * NK + lrow, g.len - 1);   // past the end: any valid row
         const uint32_t lds_at = static_cast<uint32_t>(buf * kTile * 4 + (p & 3) * 2048 * NK);
-        if (p < 4)
-            direct_load(lds_k + lds_at, Kg, static_cast<uint32_t>(key * kHeadDim + k_col) * 4u);
-        else
-            direct_load(lds_v + lds_at, Vg, static_cast<uint32_t>(key * kHeadDim + v_col) * 4u);
+        if constexpr (WHOLE) {
+            const int64_t first = static_cast<int64_t>(c * kKeys + (p & 3) * 8 * NK) * kHeadDim;
+            if (p < 4)
+                direct_load(lds_k + lds_at, Kg + first, k_lane);
+            else
+                direct_load(lds_v + lds_at, Vg + first, v_lane);
+        } else {
+            const int key = min(c * kKeys + (p & 3) * 8 * NK + lrow, g.len - 1);
+            if (p < 4)
+                direct_load(lds_k + lds_at, Kg, static_cast<uint32_t>(key * kHeadDim + k_col) * 4u);
+            else
+                direct_load(lds_v + lds_at, Vg, static_cast<uint32_t>(key * kHeadDim + v_col) * 4u);
+        }
     };
 
     // ---- this lane's query: B operand of S^T, scaled once --------------------------------------
@@ -223,9 +244,14 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     // registers are still in flight. (Issued from inline assembly they looked ready at once, and
     // the register allocator copied them to other registers BEFORE the wait, which now and then
     // picked up what the registers held before the data arrived.)
+    const float *mlane = mrow + wk * 32 + 4 * half;   // this lane's first key of chunk 0
     auto load_mask = [&](int a, int c) {
-        const int key0 = c * kKeys + wk * 32 + 4 * half;
-        return *reinterpret_cast<const v4f *>(mrow + min(key0 + 8 * a, g.len - 4));
+        if constexpr (WHOLE) {
+            return *reinterpret_cast<const v4f *>(mlane + (c * kKeys + 8 * a));
+        } else {
+            const int key0 = c * kKeys + wk * 32 + 4 * half;
+            return *reinterpret_cast<const v4f *>(mrow + min(key0 + 8 * a, g.len - 4));
+        }
     };
     const int first_chunk = next_active(-1);
     v4f mk[4], mk_next[4];
@@ -247,6 +273,12 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     auto step = [&](int c, int next, int buf, auto more_tag) {
         constexpr bool MORE = decltype(more_tag)::value;
         const int key0 = c * kKeys + wk * 32 + 4 * half;
+        if (g.queue) {
+            if ((c ^ slot_bit) & 1)
+                __builtin_amdgcn_s_setprio(1);
+            else
+                __builtin_amdgcn_s_setprio(0);
+        }
         if constexpr (!MORE) {   // the ticket for the item after this one comes back under this step
             if (g.queue && tid == 0) drawn = atomicAdd(g.queue, 1);
         }
@@ -279,7 +311,7 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
         for (int a = 0; a < 4; ++a)
 #pragma unroll
             for (int e = 0; e < 4; ++e) t[4 * a + e] = st[4 * a + e] + mk[a][e];
-        if ((c + 1) * kKeys > g.len) {
+        if (!WHOLE && (c + 1) * kKeys > g.len) {
             // keys past the end (their rows and mask values were read from valid but unrelated places)
 #pragma unroll
             for (int a = 0; a < 4; ++a)
@@ -830,18 +862,21 @@ int32_t attention_many_rows(rmlk_stream_t stream, int32_t dtype, int64_t batch, 
         }
     }
     // two blocks of four wavefronts per CU when there are that many, else one block of eight
-    if (many_blocks) {
+    auto launch = [&](auto nk_tag, auto whole_tag) -> int32_t {
+        constexpr int NK = decltype(nk_tag)::value;
+        constexpr bool WHOLE = decltype(whole_tag)::value;
         static DynamicLdsGrant grant;
-        const int32_t granted = grant.ensure(attention_rows_kernel<2>, AttnShape<2>::kLdsBytes);
+        const int32_t granted = grant.ensure(attention_rows_kernel<NK, WHOLE>, AttnShape<NK>::kLdsBytes);
         if (granted) return granted;
-        attention_rows_kernel<2><<<grid, AttnShape<2>::kThreads, AttnShape<2>::kLdsBytes, as_stream(stream)>>>(g);
-    } else {
-        static DynamicLdsGrant grant;
-        const int32_t granted = grant.ensure(attention_rows_kernel<4>, AttnShape<4>::kLdsBytes);
-        if (granted) return granted;
-        attention_rows_kernel<4><<<grid, AttnShape<4>::kThreads, AttnShape<4>::kLdsBytes, as_stream(stream)>>>(g);
-    }
-    return launch_status();
+        attention_rows_kernel<NK, WHOLE>
+            <<<grid, AttnShape<NK>::kThreads, AttnShape<NK>::kLdsBytes, as_stream(stream)>>>(g);
+        return launch_status();
+    };
+    using Two = std::integral_constant<int, 2>;
+    using Four = std::integral_constant<int, 4>;
+    if (many_blocks)
+        return kv_len % AttnShape<2>::kKeys == 0 ? launch(Two{}, std::true_type{}) : launch(Two{}, std::false_type{});
+    return kv_len % AttnShape<4>::kKeys == 0 ? launch(Four{}, std::true_type{}) : launch(Four{}, std::false_type{});
 }
 }  // namespace
 
