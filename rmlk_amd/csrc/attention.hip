@@ -106,7 +106,13 @@ __device__ __forceinline__ void store_pieces(const v4f &w, uint16_t *at, int64_t
 }
 
 // WHOLE: the keys are a multiple of the step's, so every chunk lies inside them.
-template <int NK, bool WHOLE>
+// PAIRED (with a tile map, one block per compute unit): the two halves of a block's wavefronts take
+// 32 rows each of two DIFFERENT query tiles of a head, tile i and tile T - 1 - i. Under a causal mask
+// one of them sees many chunks and the other few, and a SIMD holds a wavefront of either half: every
+// SIMD of the chip then has the same work, where whole tiles leave the last tile's block to decide
+// when the kernel ends. The block walks the chunks that either tile sees; a wavefront sits out the
+// ones its own tile does not see (it still fetches its share of them).
+template <int NK, bool WHOLE, bool PAIRED>
 __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel(AttnArgs g) {
     constexpr int kKeys = AttnShape<NK>::kKeys, kTile = AttnShape<NK>::kTile;
     extern __shared__ __align__(16) float smem[];
@@ -141,6 +147,16 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     }
     const int b = bg / g.kv_heads, grp = bg - b * g.kv_heads;
     const int r0 = tile_x * 64;
+    // the first of this wavefront's 32 query rows, and of the rows of the block's other half
+    int rbase = r0 + wq * 32, rbase_other = r0 + (wq ^ 1) * 32;
+    if constexpr (PAIRED) {
+        // blocks 2 i and 2 i + 1 of a head: rows 0..31 and 32..63 of the tiles T - 1 - i and i
+        const int hd = tile_x / g.tiles_per_head, j = tile_x - hd * g.tiles_per_head;
+        const int far = (hd * g.tiles_per_head + g.tiles_per_head - 1 - j / 2) * 64 + (j & 1) * 32;
+        const int near = (hd * g.tiles_per_head + j / 2) * 64 + (j & 1) * 32;
+        rbase = wq == 0 ? far : near;
+        rbase_other = wq == 0 ? near : far;
+    }
     const float *Kg = g.k + static_cast<int64_t>(bg) * g.len * kHeadDim;
     const float *Vg = g.v + static_cast<int64_t>(bg) * g.len * kHeadDim;
     const int n_chunks = (g.len + kKeys - 1) / kKeys;
@@ -149,14 +165,27 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     uint64_t active[2];
     active[0] = n_chunks >= 64 ? ~0ull : ((1ull << n_chunks) - 1);
     active[1] = n_chunks >= 128 ? ~0ull : (n_chunks > 64 ? ((1ull << (n_chunks - 64)) - 1) : 0ull);
+    uint64_t mine[2] = {active[0], active[1]};   // PAIRED: the chunks this wavefront's own tile sees
     if (g.tiles) {   // (the launcher gives a map only for n_chunks <= 128 and seq % 64 == 0: a tile lies in one head)
-        const int head0 = grp * g.rep + r0 / g.seq, srow0 = r0 - (r0 / g.seq) * g.seq;
-        const uint8_t *tp = g.tiles + b * g.tiles_b + head0 * g.tiles_h + static_cast<int64_t>(srow0 / 64) * n_chunks;
-        const bool f0 = lane < n_chunks && tp[min(lane, n_chunks - 1)] != 0;
-        const bool f1 = lane + 64 < n_chunks && tp[min(lane + 64, n_chunks - 1)] != 0;
-        active[0] = __builtin_amdgcn_ballot_w64(f0);
-        active[1] = __builtin_amdgcn_ballot_w64(f1);
-        if ((active[0] | active[1]) == 0) active[0] = 1;   // nothing visible at all: chunk 0 gives the NaN rows
+        auto seen_from = [&](int row, uint64_t (&out)[2]) {   // the map's row of the tile that holds query row `row`
+            const int head0 = grp * g.rep + row / g.seq, srow0 = row - (row / g.seq) * g.seq;
+            const uint8_t *tp =
+                g.tiles + b * g.tiles_b + head0 * g.tiles_h + static_cast<int64_t>(srow0 / 64) * n_chunks;
+            const bool f0 = lane < n_chunks && tp[min(lane, n_chunks - 1)] != 0;
+            const bool f1 = lane + 64 < n_chunks && tp[min(lane + 64, n_chunks - 1)] != 0;
+            out[0] = __builtin_amdgcn_ballot_w64(f0);
+            out[1] = __builtin_amdgcn_ballot_w64(f1);
+            if ((out[0] | out[1]) == 0) out[0] = 1;   // nothing visible at all: chunk 0 gives the NaN rows
+        };
+        seen_from(rbase, mine);
+        active[0] = mine[0];
+        active[1] = mine[1];
+        if constexpr (PAIRED) {
+            uint64_t other[2];
+            seen_from(rbase_other, other);
+            active[0] |= other[0];
+            active[1] |= other[1];
+        }
     }
     auto next_active = [&](int c) {   // the first visited chunk after c, -1 when there is none
         const int from = c + 1;
@@ -213,7 +242,7 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     };
 
     // ---- this lane's query: B operand of S^T, scaled once --------------------------------------
-    const int qrow = min(r0 + wq * 32 + l32, g.rows - 1);
+    const int qrow = min(rbase + l32, g.rows - 1);
     const float *qp = g.q + (static_cast<int64_t>(bg) * g.rows + qrow) * kHeadDim + half * 4;
     v4f qf[8];
 #pragma unroll
@@ -283,6 +312,9 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
             if (g.queue && tid == 0) drawn = atomicAdd(g.queue, 1);
         }
 
+        bool here = true;
+        if constexpr (PAIRED) here = c >= 128 || ((mine[c >> 6] >> (c & 63)) & 1) != 0;
+        if (here) {
         // S^T (32 keys x 32 queries) = K . Q^T over the 64 head dims
         v16f st = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         const float *ks = Ks + buf * kTile + k_frag;
@@ -357,6 +389,12 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
             o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[v_frag0 + key_off], p[r], o0, 0, 0, 0);
             o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[v_frag1 + key_off], p[r], o1, 0, 0, 0);
         }
+        } else if constexpr (MORE) {   // not this wavefront's chunk: only its share of the next one's loads
+#pragma unroll
+            for (int a = 0; a < 4; ++a) mk_next[a] = load_mask(a, next);
+#pragma unroll
+            for (int pc = 0; pc < 8; ++pc) issue_piece(pc, next, buf ^ 1);
+        }
         // the next chunk and its mask have landed and nobody reads this chunk any more
         if constexpr (MORE) {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier"
@@ -415,7 +453,7 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
             total += cb[j * kSlot + kWave + lane] * aj[j];
         }
         const float inv = 1.0f / total;   // nothing visible at all: 0 * inf = NaN, as Softmax
-        const int row = r0 + wq * 32 + l32;
+        const int row = rbase + l32;
         if (row < g.rows) {
             float *op = g.out + b * g.out_b + head * g.out_h + srow * g.out_s + 4 * half;   // row == qrow here
 #pragma unroll
@@ -862,21 +900,27 @@ int32_t attention_many_rows(rmlk_stream_t stream, int32_t dtype, int64_t batch, 
         }
     }
     // two blocks of four wavefronts per CU when there are that many, else one block of eight
-    auto launch = [&](auto nk_tag, auto whole_tag) -> int32_t {
+    auto launch = [&](auto nk_tag, auto whole_tag, auto paired_tag) -> int32_t {
         constexpr int NK = decltype(nk_tag)::value;
-        constexpr bool WHOLE = decltype(whole_tag)::value;
+        constexpr bool WHOLE = decltype(whole_tag)::value, PAIRED = decltype(paired_tag)::value;
         static DynamicLdsGrant grant;
-        const int32_t granted = grant.ensure(attention_rows_kernel<NK, WHOLE>, AttnShape<NK>::kLdsBytes);
+        const int32_t granted = grant.ensure(attention_rows_kernel<NK, WHOLE, PAIRED>, AttnShape<NK>::kLdsBytes);
         if (granted) return granted;
-        attention_rows_kernel<NK, WHOLE>
+        attention_rows_kernel<NK, WHOLE, PAIRED>
             <<<grid, AttnShape<NK>::kThreads, AttnShape<NK>::kLdsBytes, as_stream(stream)>>>(g);
         return launch_status();
     };
     using Two = std::integral_constant<int, 2>;
     using Four = std::integral_constant<int, 4>;
-    if (many_blocks)
-        return kv_len % AttnShape<2>::kKeys == 0 ? launch(Two{}, std::true_type{}) : launch(Two{}, std::false_type{});
-    return kv_len % AttnShape<4>::kKeys == 0 ? launch(Four{}, std::true_type{}) : launch(Four{}, std::false_type{});
+    const std::true_type yes{};
+    const std::false_type no{};
+    if (many_blocks) return kv_len % AttnShape<2>::kKeys == 0 ? launch(Two{}, yes, no) : launch(Two{}, no, no);
+    // one block per tile and a map: the blocks take halves of two tiles each (an even number of tiles per head)
+    if (g.tiles && !g.queue && q_len % 128 == 0) {
+        g.tiles_per_head = static_cast<int32_t>(q_len / 64);
+        return kv_len % AttnShape<4>::kKeys == 0 ? launch(Four{}, yes, yes) : launch(Four{}, no, yes);
+    }
+    return kv_len % AttnShape<4>::kKeys == 0 ? launch(Four{}, yes, no) : launch(Four{}, no, no);
 }
 }  // namespace
 
