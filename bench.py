@@ -537,6 +537,25 @@ def run_ops_suite(args):
                        "by_buffer_set_us": [round(float(span[np.arange(reps) % ns == j].mean()), 2) for j in range(ns)]}
         log(f"[ops] in-kernel clock, {name}: {clock[name]}")
         del graph, stamps
+    # What a SIMD does with vector ALU instructions beside fp32 MFMAs (one block per compute unit,
+    # two wavefronts per SIMD): cycles per MFMA of a chain with 0..16 independent v_fma_f32 behind
+    # each, and what a second wavefront's chain of dependent v_fma_f32 gets done meanwhile.
+    issue = {}
+    iters = 2000
+    cyc = torch.zeros(256, 8, dtype=torch.int64, device=dev)
+    for nv in (0, 4, 8, 12, 16):
+        for second in (False, True):
+            cyc.zero_()
+            k.issue_yardstick(nv, second, iters, cyc)
+            torch.cuda.synchronize()
+            c = cyc.cpu().numpy().astype(np.float64)
+            row = {"cycles_per_mfma": round(float(c[:, :4].mean() / (16 * iters)), 1)}
+            if second:
+                row["second_wavefront_cycles_per_64_fma"] = round(float(c[:, 4:].mean() / iters), 1)
+            issue[f"{nv}_fma_per_mfma" + ("_with_second_wavefront" if second else "")] = row
+    cyc.zero_()
+    log(f"[ops] issue yardstick: {issue}")
+    clock["issue"] = issue
     # ---- yardsticks: an almost empty launch and a plain 256 MiB copy -------------------------------
     timed("launch_floor", lambda i: check(lib().rmlk_hip_fill(side.cuda_stream, k.INT32, 1, ctypes.byref(one),
                                                               marker.data_ptr()), "rmlk_hip_fill"), 1, 4)

@@ -687,6 +687,17 @@ enum { RMLK_YARDSTICK_READ = 0, RMLK_YARDSTICK_COPY = 1 };
 int32_t rmlk_hip_stream_yardstick(rmlk_stream_t stream, int32_t kind, size_t bytes, const void *src,
                                   void *dst, uint64_t *stamps);
 
+/* Issue yardstick for benchmarks: what a SIMD does with vector ALU instructions beside fp32 MFMAs.
+ * `blocks` blocks of eight wavefronts (two per SIMD of a compute unit): wavefronts 0..3 issue
+ * 16 * iterations v_mfma_f32_32x32x2_f32 in a chain, each followed by `valu_per_mfma` (0, 4, 8, 12
+ * or 16) independent v_fma_f32; with `second_wavefront` non-zero wavefronts 4..7 run 64 * iterations
+ * dependent v_fma_f32 at the same time. cycles[8 b + w] (device memory, 8 * blocks 64-bit words)
+ * receives the shader clock cycles wavefront w of block b took, 0 for one that had nothing to do.
+ * A kernel's vector instructions either hide behind its MFMAs or add to them: this tells which.
+ * No counterpart in the reference. */
+int32_t rmlk_hip_issue_yardstick(rmlk_stream_t stream, int32_t valu_per_mfma, int32_t second_wavefront,
+                                 int32_t iterations, int32_t blocks, uint64_t *cycles);
+
 /* Write up to 256 bytes from host memory `src` to device memory `dst`. The bytes travel as kernel
  * arguments: no staging copy, nothing to keep alive, recordable into a HIP graph.
  * ref: runtime/src/providers/cuda/backend/shape.rs:67-72 (host vector + H2D for tiny tensors). */

@@ -190,6 +190,7 @@ SIGNATURES = {
     "rmlk_hip_fill": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
     "rmlk_hip_range": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_void_p]),
     "rmlk_hip_stream_yardstick": (c_int32, [c_void_p, c_int32, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "rmlk_hip_issue_yardstick": (c_int32, [c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p]),
     "rmlk_hip_write_small": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "rmlk_hip_malloc": (c_int32, [POINTER(c_void_p), c_size_t]),
     "rmlk_hip_free": (c_int32, [c_void_p]),

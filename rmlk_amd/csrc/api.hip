@@ -121,6 +121,77 @@ extern "C" int32_t rmlk_hip_stream_yardstick(rmlk_stream_t stream, int32_t kind,
     return launch_status();
 }
 
+// ---- issue yardstick -------------------------------------------------------------------------------
+// What a SIMD does with vector ALU instructions beside fp32 MFMAs. A block of eight wavefronts, two
+// per SIMD: wavefronts 0..3 issue a chain of v_mfma_f32_32x32x2_f32, each followed by NV independent
+// v_fma_f32; wavefronts 4..7 (when asked) run a chain of dependent v_fma_f32 meanwhile. Every
+// wavefront notes the shader clock cycles it took. Benchmarks read from it whether the vector
+// instructions of a kernel run in the shadow of its MFMAs or add to them.
+namespace rmlk {
+namespace {
+typedef float IssueAcc __attribute__((ext_vector_type(16)));
+
+template <int NV>
+__global__ __launch_bounds__(512) void yardstick_issue_kernel(int second, int iterations, uint64_t *cycles) {
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    long long t0 = 0, t1 = 0;
+    float res = 0.f;
+    const float m = 0.999f, c = 0.0001f;
+    if (wave < 4) {
+        IssueAcc acc;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+        const float a = lane * 0.001f, b = 1.0f + lane * 0.002f;
+        float x[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) x[j] = lane * 0.01f + j;
+        t0 = clock64();
+        for (int i = 0; i < iterations; ++i) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+#pragma unroll
+                for (int v = 0; v < NV; ++v) x[v % 16] = __builtin_fmaf(x[v % 16], m, c);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 16; ++j) res += acc[j] + x[j];
+        asm volatile("" : "+v"(res));
+        t1 = clock64();
+    } else if (second) {
+        float x0 = lane * 0.001f;
+        t0 = clock64();
+        for (int i = 0; i < iterations; ++i) {
+#pragma unroll
+            for (int j = 0; j < 64; ++j) x0 = __builtin_fmaf(x0, m, c);
+        }
+        res = x0;
+        asm volatile("" : "+v"(res));
+        t1 = clock64();
+    }
+    if (lane == 0) cycles[blockIdx.x * 8 + wave] = static_cast<uint64_t>(t1 - t0) + (res == 12345.678f ? 1 : 0);
+}
+}  // namespace
+}  // namespace rmlk
+
+extern "C" int32_t rmlk_hip_issue_yardstick(rmlk_stream_t stream, int32_t valu_per_mfma, int32_t second_wavefront,
+                                            int32_t iterations, int32_t blocks, uint64_t *cycles) {
+    if (iterations <= 0 || iterations > (1 << 20) || blocks <= 0 || blocks > 65535) return RMLK_ERR_INVALID_ARGUMENT;
+    if (!cycles) return RMLK_ERR_NULL_POINTER;
+    hipStream_t s = as_stream(stream);
+    const int second = second_wavefront ? 1 : 0;
+    switch (valu_per_mfma) {
+        case 0: yardstick_issue_kernel<0><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
+        case 4: yardstick_issue_kernel<4><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
+        case 8: yardstick_issue_kernel<8><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
+        case 12: yardstick_issue_kernel<12><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
+        case 16: yardstick_issue_kernel<16><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
+        default: return RMLK_ERR_INVALID_ARGUMENT;
+    }
+    return launch_status();
+}
+
 extern "C" int32_t rmlk_hip_stream_sync(rmlk_stream_t stream) {
     return static_cast<int32_t>(hipStreamSynchronize(as_stream(stream)));
 }

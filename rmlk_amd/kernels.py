@@ -544,6 +544,17 @@ def stream_yardstick(kind: int, src, dst, nbytes: int, stamps=None, stream=None)
     check(st, "rmlk_hip_stream_yardstick")
 
 
+def issue_yardstick(valu_per_mfma: int, second_wavefront: bool, iterations: int, cycles) -> None:
+    """A chain of fp32 MFMAs with `valu_per_mfma` independent vector ALU instructions behind each, in
+    wavefronts 0..3 of every block, and (second_wavefront) a chain of dependent ones in wavefronts
+    4..7 beside them; `cycles` (int64, 8 per block) receives every wavefront's shader clock cycles.
+    For benchmarks; no counterpart in the reference."""
+    blocks = cycles.numel() // 8
+    st = lib().rmlk_hip_issue_yardstick(_stream(), int(valu_per_mfma), int(bool(second_wavefront)), int(iterations),
+                                        blocks, _ptr(cycles))
+    check(st, "rmlk_hip_issue_yardstick")
+
+
 def device_info(device: int = 0) -> dict:
     from ._lib import DeviceInfo
     info = DeviceInfo()

@@ -827,3 +827,23 @@ def test_stream_yardstick(device):
     assert int(sink.abs().sum().item()) == 0
     with pytest.raises(k.RmlkError):
         k.stream_yardstick(k.YARDSTICK_COPY, src, dst, 1000)     # not whole 16 KiB blocks
+
+
+def test_issue_yardstick(device):
+    """The MFMA / vector ALU yardstick: a chain of v_mfma_f32_32x32x2_f32 takes its 64 cycles apiece, a
+    wavefront with nothing to do reports 0, and the arguments are checked."""
+    k = _k()
+    cyc = torch.zeros(4, 8, dtype=torch.int64, device=device)
+    iters = 200
+    k.issue_yardstick(0, False, iters, cyc)
+    c = cyc.cpu().numpy()
+    per_mfma = c[:, :4] / (16.0 * iters)
+    assert (per_mfma > 60).all() and (per_mfma < 80).all(), per_mfma
+    assert (c[:, 4:] == 0).all()
+    k.issue_yardstick(8, True, iters, cyc)
+    c = cyc.cpu().numpy()
+    assert (c[:, :4] / (16.0 * iters) > 64).all() and (c[:, 4:] > 0).all()
+    with pytest.raises(k.RmlkError):
+        k.issue_yardstick(5, False, iters, cyc)
+    with pytest.raises(k.RmlkError):
+        k.issue_yardstick(4, False, 0, cyc)
