@@ -42,6 +42,7 @@ struct AttnShape {
     static constexpr int kLdsBytes = 2 * 2 * kTile * 4;    // K and V, two buffers each
 };
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kSlack = 8.0f / kLog2e;   // how far a score may lie above the point its exponent is taken from
 
 // max / sum of a value over the two lanes (l, l + 32) that share a query, on all 64 lanes: one
 // v_permlane32_swap turns x into (lower half twice, upper half twice).
@@ -360,26 +361,33 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
             half_pair(mx, lo, hi);
             mx = fmaxf(lo, hi);
         }
-        const float m_new = fmaxf(m_run, mx);
-        const float m_safe = m_new == kNegInf ? 0.f : m_new;   // a row with nothing visible so far
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * kLog2e);
+        // m_run is the point the exponents are taken from, not the maximum itself: it follows the
+        // maximum only when a score of this chunk lies more than kSlack above it (probabilities then
+        // stay below 2^8, far inside the range of a float), so that the 32 accumulator registers
+        // and the sum are rescaled in the first chunks of a row and hardly ever afterwards - under a
+        // causal mask some query of a wavefront meets a new maximum in most chunks. The quotient
+        // of output and sum does not depend on the point. (-inf + kSlack is -inf: the first finite
+        // score moves it; a NaN moves nothing and reaches the output through its probability.)
+        if (__builtin_amdgcn_ballot_w64(mx > m_run + kSlack) != 0) {
+            const float m_new = fmaxf(m_run, mx);
+            const float m_to = m_new == kNegInf ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_to) * kLog2e);   // exactly 1 where m_new == m_run
+            l_run *= alpha;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                o0[r] *= alpha;
+                o1[r] *= alpha;
+            }
+            m_run = m_new;
+        }
+        const float m_safe = m_run == kNegInf ? 0.f : m_run;   // a row with nothing visible so far
         float p[16], psum = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             p[r] = __builtin_amdgcn_exp2f((t[r] - m_safe) * kLog2e);
             psum += p[r];
         }
-        l_run = l_run * alpha + psum;
-        // the output so far is rescaled only when some query of this wavefront met a new maximum
-        // (alpha is exactly 1 otherwise)
-        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                o0[r] *= alpha;
-                o1[r] *= alpha;
-            }
-        }
-        m_run = m_new;
+        l_run += psum;
 
         // O^T (64 dims x 32 queries) += V^T . P^T over this wavefront's 32 keys
         const float *vs = Vs + buf * kTile;
