@@ -679,11 +679,17 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     constexpr int kLoadChunks = 1;   // chunks (from the first) that carry the loads
     constexpr int kLoadsPerChunk = (kLoadsPerStage + kLoadChunks - 1) / kLoadChunks;
     constexpr int kBarrierAt = NM * 2 / 4 < NM - 1 ? NM * 2 / 4 : NM - 2;
-    auto k_step = [&](int buf, auto load_tag, auto more_tag, auto load2_tag) {
+    // (The LDS buffer of a step is fixed in its code, two steps per trip of the loop: the addresses
+    // of the fragment reads are then a lane offset that never changes plus an immediate. With the
+    // buffer in a register every read had a vector add in front of it, and a vector ALU
+    // instruction between two MFMAs whose result an LDS read waits for holds the next MFMA back
+    // by some 30 cycles.)
+    auto k_step = [&](auto buf_tag, auto load_tag, auto more_tag, auto load2_tag) {
+        constexpr int buf = decltype(buf_tag)::value;
         constexpr bool LOAD = decltype(load_tag)::value;   // another stage to fetch
         constexpr bool MORE = decltype(more_tag)::value;   // another step follows
         constexpr bool LOAD2 = decltype(load2_tag)::value; // 16-bit B: a stage after that one to request
-        const int other = buf ^ 1;
+        constexpr int other = buf ^ 1;
         static_for<KC>([&](auto kc_tag) {
             constexpr int kc = decltype(kc_tag)::value;
             constexpr int slot = kc & 1;
@@ -757,23 +763,39 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
         stage_barrier();
 #pragma unroll
         for (int o = 0; o < kFragOps; ++o) frag_op(0, 0, 0, o);
-        int buf = 0;
+        const std::integral_constant<int, 0> even{};
+        const std::integral_constant<int, 1> odd{};
+        const std::true_type yes{};
+        const std::false_type no{};
+        int left = n_steps;   // steps to go; the next one reads buffer 0
         if constexpr (B16) {
-            for (int step = 0; step + 2 < n_steps; ++step) {
-                k_step(buf, std::true_type{}, std::true_type{}, std::true_type{});
-                buf ^= 1;
+            // the last step fetches nothing, the one before it requests no stage behind the one it fetches
+            for (; left > 3; left -= 2) {
+                k_step(even, yes, yes, yes);
+                k_step(odd, yes, yes, yes);
             }
-            if (n_steps > 1) {
-                k_step(buf, std::true_type{}, std::true_type{}, std::false_type{});
-                buf ^= 1;
+            if (left == 3) {
+                k_step(even, yes, yes, yes);
+                k_step(odd, yes, yes, no);
+                k_step(even, no, no, no);
+            } else if (left == 2) {
+                k_step(even, yes, yes, no);
+                k_step(odd, no, no, no);
+            } else {
+                k_step(even, no, no, no);
             }
         } else {
-            for (int step = 0; step + 1 < n_steps; ++step) {
-                k_step(buf, std::true_type{}, std::true_type{}, std::false_type{});
-                buf ^= 1;
+            for (; left > 2; left -= 2) {
+                k_step(even, yes, yes, no);
+                k_step(odd, yes, yes, no);
+            }
+            if (left == 2) {
+                k_step(even, yes, yes, no);
+                k_step(odd, no, no, no);
+            } else {
+                k_step(even, no, no, no);
             }
         }
-        k_step(buf, std::false_type{}, std::false_type{}, std::false_type{});
     }
 
     if constexpr (SWIGLU) {
