@@ -298,6 +298,23 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     const int k_swz = l32 & 15;
     const int v_frag0 = (wk * 32 + 4 * half) * kHeadDim + (half * 32 + l32);        // d =      l32
     const int v_frag1 = (wk * 32 + 4 * half) * kHeadDim + ((half ^ 1) * 32 + l32);  // d = 32 + l32
+    // The LDS byte addresses of this lane's fragment reads, for the buffer the next step reads: kept
+    // in registers and moved to the other buffer by ten adds in a row at the end of a step. (Formed
+    // from the buffer number in front of every read, each was a vector add that an LDS read waited
+    // for between two MFMAs, and such a pair holds the next MFMA back by some 30 cycles.)
+    using LdsV4 = const v4f __attribute__((address_space(3))) *;
+    using LdsF = const float __attribute__((address_space(3))) *;
+    uint32_t k_at[8], v_at[2];
+    {
+        const uint32_t ks0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(Ks));
+        const uint32_t vs0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(Vs));
+#pragma unroll
+        for (int kc = 0; kc < 8; ++kc)
+            k_at[kc] = ks0 + static_cast<uint32_t>(k_frag + (((kc * 2 + half) ^ k_swz) * 4)) * 4u;
+        v_at[0] = vs0 + static_cast<uint32_t>(v_frag0) * 4u;
+        v_at[1] = vs0 + static_cast<uint32_t>(v_frag1) * 4u;
+    }
+    int32_t to_other = kTile * 4;   // to the other buffer: +, -, +, ...
 
     // chunk c from buffer buf; MORE: chunk `next` is fetched into the other buffer meanwhile
     auto step = [&](int c, int next, int buf, auto more_tag) {
@@ -318,13 +335,12 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
         if (here) {
         // S^T (32 keys x 32 queries) = K . Q^T over the 64 head dims
         v16f st = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        const float *ks = Ks + buf * kTile + k_frag;
         // The next chunk's eight pieces and its mask are requested one after each group of four
         // MFMAs (all at the top of the step they kept the matrix pipe idle for some 1200 cycles of
         // address arithmetic and load issue per step).
         static_for<8>([&](auto kc_tag) {
             constexpr int kc = decltype(kc_tag)::value;
-            const v4f kf = *reinterpret_cast<const v4f *>(ks + (((kc * 2 + half) ^ k_swz) * 4));
+            const v4f kf = *(LdsV4)(k_at[kc]);
 #pragma unroll
             for (int s = 0; s < 4; ++s)
                 st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[s], qf[kc][s], st, 0, 0, 0);
@@ -390,18 +406,24 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
         l_run += psum;
 
         // O^T (64 dims x 32 queries) += V^T . P^T over this wavefront's 32 keys
-        const float *vs = Vs + buf * kTile;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int key_off = (8 * (r / 4) + (r % 4)) * kHeadDim;
-            o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[v_frag0 + key_off], p[r], o0, 0, 0, 0);
-            o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[v_frag1 + key_off], p[r], o1, 0, 0, 0);
+            o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(*(LdsF)(v_at[0] + key_off * 4), p[r], o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(*(LdsF)(v_at[1] + key_off * 4), p[r], o1, 0, 0, 0);
         }
         } else if constexpr (MORE) {   // not this wavefront's chunk: only its share of the next one's loads
 #pragma unroll
             for (int a = 0; a < 4; ++a) mk_next[a] = load_mask(a, next);
 #pragma unroll
             for (int pc = 0; pc < 8; ++pc) issue_piece(pc, next, buf ^ 1);
+        }
+        if constexpr (MORE) {   // the next step reads the other buffer
+#pragma unroll
+            for (int kc = 0; kc < 8; ++kc) asm volatile("v_add_u32 %0, %0, %1" : "+v"(k_at[kc]) : "s"(to_other));
+            asm volatile("v_add_u32 %0, %0, %1" : "+v"(v_at[0]) : "s"(to_other));
+            asm volatile("v_add_u32 %0, %0, %1" : "+v"(v_at[1]) : "s"(to_other));
+            to_other = -to_other;
         }
         // the next chunk and its mask have landed and nobody reads this chunk any more
         if constexpr (MORE) {
