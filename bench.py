@@ -537,9 +537,10 @@ def run_ops_suite(args):
                        "by_buffer_set_us": [round(float(span[np.arange(reps) % ns == j].mean()), 2) for j in range(ns)]}
         log(f"[ops] in-kernel clock, {name}: {clock[name]}")
         del graph, stamps
-    # What a SIMD does with vector ALU instructions beside fp32 MFMAs (one block per compute unit,
-    # two wavefronts per SIMD): cycles per MFMA of a chain with 0..16 independent v_fma_f32 behind
-    # each, and what a second wavefront's chain of dependent v_fma_f32 gets done meanwhile.
+    # What a SIMD does with other instructions beside fp32 MFMAs (one block per compute unit, two
+    # wavefronts per SIMD): cycles per MFMA of a chain with 0..16 independent v_fma_f32 behind each,
+    # what a second wavefront's chain of dependent v_fma_f32 gets done meanwhile, and cycles per
+    # MFMA of independent MFMAs with an instruction behind every fourth.
     issue = {}
     iters = 2000
     cyc = torch.zeros(256, 8, dtype=torch.int64, device=dev)
@@ -553,6 +554,15 @@ def run_ops_suite(args):
             if second:
                 row["second_wavefront_cycles_per_64_fma"] = round(float(c[:, 4:].mean() / iters), 1)
             issue[f"{nv}_fma_per_mfma" + ("_with_second_wavefront" if second else "")] = row
+    for kind, what in ((100, "nothing"), (101, "v_add_u32"), (102, "ds_read_b128"),
+                       (103, "v_add_u32_then_the_ds_read_b128_that_waits_for_it")):
+        cyc.zero_()
+        k.issue_yardstick(kind, False, iters, cyc)
+        torch.cuda.synchronize()
+        c = cyc.cpu().numpy().astype(np.float64)
+        per = float(c[:, :4].mean() / (16 * iters))
+        issue[f"independent_mfmas_{what}_behind_every_4th"] = {"cycles_per_mfma": round(per, 2),
+                                                              "cycles_per_occurrence": round((per - 64.0) * 4, 1)}
     cyc.zero_()
     log(f"[ops] issue yardstick: {issue}")
     clock["issue"] = issue

@@ -687,15 +687,17 @@ enum { RMLK_YARDSTICK_READ = 0, RMLK_YARDSTICK_COPY = 1 };
 int32_t rmlk_hip_stream_yardstick(rmlk_stream_t stream, int32_t kind, size_t bytes, const void *src,
                                   void *dst, uint64_t *stamps);
 
-/* Issue yardstick for benchmarks: what a SIMD does with vector ALU instructions beside fp32 MFMAs.
+/* Issue yardstick for benchmarks: what a SIMD does with other instructions beside fp32 MFMAs.
  * `blocks` blocks of eight wavefronts (two per SIMD of a compute unit): wavefronts 0..3 issue
- * 16 * iterations v_mfma_f32_32x32x2_f32 in a chain, each followed by `valu_per_mfma` (0, 4, 8, 12
- * or 16) independent v_fma_f32; with `second_wavefront` non-zero wavefronts 4..7 run 64 * iterations
- * dependent v_fma_f32 at the same time. cycles[8 b + w] (device memory, 8 * blocks 64-bit words)
- * receives the shader clock cycles wavefront w of block b took, 0 for one that had nothing to do.
- * A kernel's vector instructions either hide behind its MFMAs or add to them: this tells which.
- * No counterpart in the reference. */
-int32_t rmlk_hip_issue_yardstick(rmlk_stream_t stream, int32_t valu_per_mfma, int32_t second_wavefront,
+ * 16 * iterations v_mfma_f32_32x32x2_f32 with something between them (`kind`), and with
+ * `second_wavefront` non-zero wavefronts 4..7 run 64 * iterations dependent v_fma_f32 at the same
+ * time. Kinds 0, 4, 8, 12, 16: one chain of MFMAs, that many independent v_fma_f32 behind each.
+ * Kinds 100..103: four accumulators in turn (independent MFMAs, as in a GEMM step) and behind every
+ * fourth MFMA nothing (100), one v_add_u32 (101), one ds_read_b128 (102), a v_add_u32 and the
+ * ds_read_b128 that takes its result as the address (103). cycles[8 b + w] (device memory,
+ * 8 * blocks 64-bit words) receives the shader clock cycles wavefront w of block b took, 0 for one
+ * that had nothing to do. No counterpart in the reference. */
+int32_t rmlk_hip_issue_yardstick(rmlk_stream_t stream, int32_t kind, int32_t second_wavefront,
                                  int32_t iterations, int32_t blocks, uint64_t *cycles);
 
 /* Write up to 256 bytes from host memory `src` to device memory `dst`. The bytes travel as kernel

@@ -122,41 +122,66 @@ extern "C" int32_t rmlk_hip_stream_yardstick(rmlk_stream_t stream, int32_t kind,
 }
 
 // ---- issue yardstick -------------------------------------------------------------------------------
-// What a SIMD does with vector ALU instructions beside fp32 MFMAs. A block of eight wavefronts, two
-// per SIMD: wavefronts 0..3 issue a chain of v_mfma_f32_32x32x2_f32, each followed by NV independent
-// v_fma_f32; wavefronts 4..7 (when asked) run a chain of dependent v_fma_f32 meanwhile. Every
-// wavefront notes the shader clock cycles it took. Benchmarks read from it whether the vector
-// instructions of a kernel run in the shadow of its MFMAs or add to them.
+// What a SIMD does with other instructions beside fp32 MFMAs. A block of eight wavefronts, two per
+// SIMD: wavefronts 0..3 issue v_mfma_f32_32x32x2_f32 with something between them, wavefronts 4..7
+// (when asked) run a chain of dependent v_fma_f32 meanwhile; every wavefront notes the shader clock
+// cycles it took. Kinds 0, 4, 8, 12, 16: ONE chain of MFMAs, that many independent v_fma_f32 behind
+// each. Kinds 100..103: four accumulators in turn (independent MFMAs, as in a GEMM step) and behind
+// every fourth MFMA nothing / one v_add_u32 / one ds_read_b128 / a v_add_u32 and the ds_read_b128
+// that takes its result as the address. Benchmarks read from it which instructions of a kernel run
+// in the shadow of its MFMAs and which add to them.
 namespace rmlk {
 namespace {
 typedef float IssueAcc __attribute__((ext_vector_type(16)));
+typedef float IssueFrag __attribute__((ext_vector_type(4)));
 
-template <int NV>
+template <int KIND>
 __global__ __launch_bounds__(512) void yardstick_issue_kernel(int second, int iterations, uint64_t *cycles) {
+    __shared__ float lds[4096];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if constexpr (KIND >= 102) {
+        for (int i = threadIdx.x; i < 4096; i += 512) lds[i] = i * 0.001f;
+        __syncthreads();
+    }
     long long t0 = 0, t1 = 0;
     float res = 0.f;
     const float m = 0.999f, c = 0.0001f;
     if (wave < 4) {
-        IssueAcc acc;
+        IssueAcc acc[4];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+        for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[k][j] = 0.f;
         const float a = lane * 0.001f, b = 1.0f + lane * 0.002f;
         float x[16];
 #pragma unroll
         for (int j = 0; j < 16; ++j) x[j] = lane * 0.01f + j;
+        uint32_t addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + lane * 16;
+        const uint32_t step = 1024;
+        IssueFrag frag = {0.f, 0.f, 0.f, 0.f};
         t0 = clock64();
         for (int i = 0; i < iterations; ++i) {
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+                constexpr int kAccs = KIND >= 100 ? 4 : 1;
+                acc[j % kAccs] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[j % kAccs], 0, 0, 0);
+                if constexpr (KIND < 100) {
 #pragma unroll
-                for (int v = 0; v < NV; ++v) x[v % 16] = __builtin_fmaf(x[v % 16], m, c);
+                    for (int v = 0; v < KIND; ++v) x[v % 16] = __builtin_fmaf(x[v % 16], m, c);
+                } else if (j % 4 == 0) {
+                    // (the address walks over 4 KiB of the 16 KiB array and comes back)
+                    if constexpr (KIND == 101 || KIND == 103)
+                        asm volatile("v_add_u32 %0, %0, %1" : "+v"(addr) : "s"(j == 12 ? 0u - 3u * step : step));
+                    if constexpr (KIND == 102 || KIND == 103)
+                        asm volatile("ds_read_b128 %0, %1" : "=v"(frag) : "v"(addr));
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        res = frag[0] + frag[3];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) res += acc[j] + x[j];
+        for (int j = 0; j < 16; ++j) res += acc[0][j] + acc[1][j] + acc[2][j] + acc[3][j] + x[j];
         asm volatile("" : "+v"(res));
         t1 = clock64();
     } else if (second) {
@@ -175,18 +200,22 @@ __global__ __launch_bounds__(512) void yardstick_issue_kernel(int second, int it
 }  // namespace
 }  // namespace rmlk
 
-extern "C" int32_t rmlk_hip_issue_yardstick(rmlk_stream_t stream, int32_t valu_per_mfma, int32_t second_wavefront,
+extern "C" int32_t rmlk_hip_issue_yardstick(rmlk_stream_t stream, int32_t kind, int32_t second_wavefront,
                                             int32_t iterations, int32_t blocks, uint64_t *cycles) {
     if (iterations <= 0 || iterations > (1 << 20) || blocks <= 0 || blocks > 65535) return RMLK_ERR_INVALID_ARGUMENT;
     if (!cycles) return RMLK_ERR_NULL_POINTER;
     hipStream_t s = as_stream(stream);
     const int second = second_wavefront ? 1 : 0;
-    switch (valu_per_mfma) {
+    switch (kind) {
         case 0: yardstick_issue_kernel<0><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
         case 4: yardstick_issue_kernel<4><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
         case 8: yardstick_issue_kernel<8><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
         case 12: yardstick_issue_kernel<12><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
         case 16: yardstick_issue_kernel<16><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
+        case 100: yardstick_issue_kernel<100><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
+        case 101: yardstick_issue_kernel<101><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
+        case 102: yardstick_issue_kernel<102><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
+        case 103: yardstick_issue_kernel<103><<<blocks, 512, 0, s>>>(second, iterations, cycles); break;
         default: return RMLK_ERR_INVALID_ARGUMENT;
     }
     return launch_status();

@@ -301,7 +301,7 @@ __global__ __launch_bounds__(AttnShape<NK>::kThreads) void attention_rows_kernel
     // The LDS byte addresses of this lane's fragment reads, for the buffer the next step reads: kept
     // in registers and moved to the other buffer by ten adds in a row at the end of a step. (Formed
     // from the buffer number in front of every read, each was a vector add that an LDS read waited
-    // for between two MFMAs, and such a pair holds the next MFMA back by some 30 cycles.)
+    // for between two MFMAs, and such a pair holds the next MFMA back by some 25 cycles.)
     using LdsV4 = const v4f __attribute__((address_space(3))) *;
     using LdsF = const float __attribute__((address_space(3))) *;
     uint32_t k_at[8], v_at[2];

@@ -683,7 +683,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_direct_kernel(GemmArgs g) 
     // of the fragment reads are then a lane offset that never changes plus an immediate. With the
     // buffer in a register every read had a vector add in front of it, and a vector ALU
     // instruction between two MFMAs whose result an LDS read waits for holds the next MFMA back
-    // by some 30 cycles.)
+    // by some 25 cycles.)
     auto k_step = [&](auto buf_tag, auto load_tag, auto more_tag, auto load2_tag) {
         constexpr int buf = decltype(buf_tag)::value;
         constexpr bool LOAD = decltype(load_tag)::value;   // another stage to fetch

@@ -544,13 +544,15 @@ def stream_yardstick(kind: int, src, dst, nbytes: int, stamps=None, stream=None)
     check(st, "rmlk_hip_stream_yardstick")
 
 
-def issue_yardstick(valu_per_mfma: int, second_wavefront: bool, iterations: int, cycles) -> None:
-    """A chain of fp32 MFMAs with `valu_per_mfma` independent vector ALU instructions behind each, in
-    wavefronts 0..3 of every block, and (second_wavefront) a chain of dependent ones in wavefronts
-    4..7 beside them; `cycles` (int64, 8 per block) receives every wavefront's shader clock cycles.
-    For benchmarks; no counterpart in the reference."""
+def issue_yardstick(kind: int, second_wavefront: bool, iterations: int, cycles) -> None:
+    """fp32 MFMAs with something between them in wavefronts 0..3 of every block (kind 0/4/8/12/16: a
+    chain with that many independent v_fma_f32 behind each MFMA; 100..103: independent MFMAs with
+    nothing / a v_add_u32 / a ds_read_b128 / both, the read waiting for the add, behind every fourth)
+    and (second_wavefront) a chain of dependent v_fma_f32 in wavefronts 4..7 beside them; `cycles`
+    (int64, 8 per block) receives every wavefront's shader clock cycles. For benchmarks; no
+    counterpart in the reference."""
     blocks = cycles.numel() // 8
-    st = lib().rmlk_hip_issue_yardstick(_stream(), int(valu_per_mfma), int(bool(second_wavefront)), int(iterations),
+    st = lib().rmlk_hip_issue_yardstick(_stream(), int(kind), int(bool(second_wavefront)), int(iterations),
                                         blocks, _ptr(cycles))
     check(st, "rmlk_hip_issue_yardstick")
 

@@ -843,6 +843,10 @@ def test_issue_yardstick(device):
     k.issue_yardstick(8, True, iters, cyc)
     c = cyc.cpu().numpy()
     assert (c[:, :4] / (16.0 * iters) > 64).all() and (c[:, 4:] > 0).all()
+    k.issue_yardstick(103, False, iters, cyc)      # independent MFMAs, an add and the LDS read behind it
+    c = cyc.cpu().numpy()
+    per = c[:, :4] / (16.0 * iters)
+    assert (per >= 63).all() and (per < 90).all(), per
     with pytest.raises(k.RmlkError):
         k.issue_yardstick(5, False, iters, cyc)
     with pytest.raises(k.RmlkError):
