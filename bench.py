@@ -43,11 +43,11 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # workspace; what their consumer (the combine kernel or the norm kernel) moves is not included.
 PMC_TRAFFIC_SOURCE = "profiles/gemm_mfma_llama1b_prefill512_hbm_traffic.md"
 PMC_TRAFFIC_KIB = {
-    (1, 512, 3072, 2048): ("mfma128x96x32 direct splitk=2", 41096, 12288),                # q/k/v
-    (1, 512, 2048, 2048): ("mfma128x64x32 direct splitk=4", 24675, 16384),                # o
-    (1, 512, 2048, 8192): ("mfma128x64x32 direct splitk=4", 98467, 16384),                # down
-    (1, 512, 16384, 2048, "swiglu"): ("mfma128x128x32 direct splitk=1", 164050, 16384),   # gate/up, SwiGLU epilogue
-    (1, 512, 128256, 2048): ("mfma128x128x32 direct splitk=1", 1493613, 256512),          # lm-head
+    (1, 512, 3072, 2048): ("mfma128x96x32 direct splitk=2", 41142, 12288),                # q/k/v
+    (1, 512, 2048, 2048): ("mfma128x64x32 direct splitk=4", 24709, 16384),                # o
+    (1, 512, 2048, 8192): ("mfma128x64x32 direct splitk=4", 130473, 16384),                # down
+    (1, 512, 16384, 2048, "swiglu"): ("mfma128x128x32 direct splitk=1", 207740, 16384),   # gate/up, SwiGLU epilogue
+    (1, 512, 128256, 2048): ("mfma128x128x32 direct splitk=1", 1844647, 256512),          # lm-head
 }
 
 
