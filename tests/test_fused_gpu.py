@@ -1134,6 +1134,44 @@ def test_attention_matches_separate_kernels(device, b, g, rep, s, l, mask_shape,
     assert_exact(to_np(moved), to_np(got).transpose(0, 2, 1, 3))
 
 
+@pytest.mark.parametrize("rise", [0.02, 0.3, 4.0])
+@pytest.mark.parametrize("s,l", [(512, 640), (2048, 1024)])
+def test_attention_scores_that_rise_along_the_keys(device, s, l, rise):
+    """The point the exponents are taken from follows the running maximum only past a slack: scores
+    that climb slowly (a few hundredths per key: the point trails the maximum for many chunks),
+    steadily (it moves in every chunk) and steeply (by hundreds per chunk) all give the softmax of
+    the float64 reference - to what fp32 scores allow: a score of size x carries an error of about
+    x * 2^-24, which its probability inherits as a relative error."""
+    import torch
+    kk = _k()
+    b, g, rep, d = 1, 8, 4, 64
+    h = g * rep
+    rng = np.random.default_rng(s + l + int(rise * 100))
+    q_np = np.zeros((b, h, s, d), dtype=np.float32)
+    k_np = np.zeros((b, g, l, d), dtype=np.float32)
+    # q . k = 8 * rise * key index (+ noise): after the division by the scale 8 a climb of `rise` per key
+    q_np[..., 0] = 8.0
+    k_np[..., 0] = (rise * np.arange(l, dtype=np.float32))[None, None, :]
+    q_np[..., 1:] = 0.1 * rng.standard_normal((b, h, s, d - 1), dtype=np.float32)
+    k_np[..., 1:] = rng.standard_normal((b, g, l, d - 1), dtype=np.float32)
+    v_np = rng.standard_normal((b, g, l, d), dtype=np.float32)
+    m_np = np.zeros((1, 1, s, l), dtype=np.float32)
+    qi = np.arange(s)[:, None] + (l - s) if l >= s else np.arange(s)[:, None] * l // s
+    m_np[0, 0][np.arange(l)[None, :] > np.maximum(qi, 0)] = -np.inf
+    q, k, v, m = (to_dev(x, device) for x in (q_np, k_np, v_np, m_np))
+    ms = [0, 0, l, 1]
+    want = _attention_reference(q_np, k_np, v_np, m_np, 8.0, False)
+    atol = 1e-5 + 1e-6 * rise * l
+    got = torch.full((b, h, s, d), float("nan"), device=device)
+    kk.attention(q, k, v, m, got, b, g, rep, s, l, d, ms, 8.0)
+    assert_close(to_np(got), want, rtol=1e-4, atol=atol)
+    skipped = torch.full((b, h, s, d), float("nan"), device=device)
+    tile_map = kk.attention_map(m, b, g, rep, s, l, d, ms)
+    assert tile_map is not None
+    kk.attention_mapped(q, k, v, m, skipped, tile_map, b, g, rep, s, l, d, ms, 8.0)
+    assert_close(to_np(skipped), want, rtol=1e-4, atol=atol)
+
+
 def _skipping_mask(kind, rng, mask_shape, l):
     """Masks with whole (64-query, 64-key) tiles hidden, in the shapes that occur: causal with a past,
     a sliding window (hidden tiles on both sides), random hidden tiles per batch and head (one query
