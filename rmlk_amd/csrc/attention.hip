@@ -8,11 +8,13 @@
 // One block owns 64 query rows of one KV head (the rep query heads that share it lie one after the
 // other, so they are rows of ONE matrix) and walks the keys in chunks of 32 * NK, staged in LDS by
 // direct global -> LDS loads, two buffers. Wavefront (wq, wk) of the 2 * NK takes query rows
-// wq*32.. and keys wk*32.. of every chunk, with its own running maximum, sum and output
-// accumulator (the NK key parts are merged once, at the end, through LDS). NK = 2 (four
+// wq*32.. and keys wk*32.. of every chunk, with its own reference point of the exponents (which
+// follows the running maximum), sum and output accumulator (the NK key parts are merged once, at
+// the end, through LDS). NK = 2 (four
 // wavefronts, 64 KB of LDS, two blocks per CU) when there are blocks enough to fill the chip that
-// way; NK = 4 (eight wavefronts, 128 KB) otherwise, so that every SIMD still holds two wavefronts
-// and one's softmax arithmetic runs under the other's MFMAs.
+// way; NK = 4 (eight wavefronts, 128 KB) otherwise, so that every SIMD still holds two wavefronts:
+// a wavefront's vector instructions do not run under its own MFMAs on this chip, only (in part)
+// under another wavefront's.
 //
 // Everything is computed TRANSPOSED so that a query stays in one lane from the scores to the
 // output: S^T = K . Q^T puts query l32 into lane column l32 of the 32x32 MFMA result, with 16 keys
