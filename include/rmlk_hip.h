@@ -388,6 +388,14 @@ int32_t rmlk_hip_attention_mapped(rmlk_stream_t stream, int32_t dtype, int64_t b
                                   const void *q, const void *k, const void *v, const void *mask,
                                   const rmlk_dims *mask_stride, int32_t scale_is_mul, float scale,
                                   int32_t out_seq_major, const void *map, size_t map_bytes, void *out);
+/* rmlk_hip_attention_mapped with the [batch, q_len, heads, head_dim] result also stored as the three
+ * bfloat16 pieces of rmlk_hip_attention_ws_pieces (same layout of `out_pieces`, same bits). */
+int32_t rmlk_hip_attention_mapped_pieces(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                         int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
+                                         int64_t head_dim, const void *q, const void *k, const void *v,
+                                         const void *mask, const rmlk_dims *mask_stride,
+                                         int32_t scale_is_mul, float scale, const void *map,
+                                         size_t map_bytes, void *out, void *out_pieces);
 /* rmlk_hip_attention_ws with a [batch, q_len, heads, head_dim] result (out_seq_major) that is also
  * stored as three bfloat16 pieces, as rmlk_hip_bf16x3_split would split the [batch * q_len, heads *
  * head_dim] matrix it is: `out_pieces` holds rmlk_hip_bf16x3_pieces_size(batch * q_len, heads *

@@ -156,6 +156,9 @@ SIGNATURES = {
     "rmlk_hip_attention_mapped": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64,
                                             c_int64, c_void_p, c_void_p, c_void_p, c_void_p, _PD, c_int32,
                                             ctypes.c_float, c_int32, c_void_p, c_size_t, c_void_p]),
+    "rmlk_hip_attention_mapped_pieces": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                                   c_int64, c_void_p, c_void_p, c_void_p, c_void_p, _PD, c_int32,
+                                                   ctypes.c_float, c_void_p, c_size_t, c_void_p, c_void_p]),
     "rmlk_hip_attention_ws_pieces": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64,
                                                c_int64, c_void_p, c_void_p, c_void_p, c_void_p, _PD, c_int32,
                                                ctypes.c_float, c_void_p, c_size_t, c_void_p, c_void_p]),

@@ -1004,6 +1004,18 @@ extern "C" int32_t rmlk_hip_attention_mapped(rmlk_stream_t stream, int32_t dtype
                                out, nullptr, 2);
 }
 
+extern "C" int32_t rmlk_hip_attention_mapped_pieces(rmlk_stream_t stream, int32_t dtype, int64_t batch,
+                                                    int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
+                                                    int64_t head_dim, const void *q, const void *k, const void *v,
+                                                    const void *mask, const rmlk_dims *mask_stride,
+                                                    int32_t scale_is_mul, float scale, const void *map,
+                                                    size_t map_bytes, void *out, void *out_pieces) {
+    if (!out_pieces) return RMLK_ERR_NULL_POINTER;
+    return attention_many_rows(stream, dtype, batch, kv_heads, rep, q_len, kv_len, head_dim, q, k, v, mask,
+                               mask_stride, scale_is_mul, scale, 1, const_cast<void *>(map), map_bytes, out,
+                               out_pieces, 2);
+}
+
 extern "C" int32_t rmlk_hip_attention(rmlk_stream_t stream, int32_t dtype, int64_t batch,
                                       int64_t kv_heads, int64_t rep, int64_t q_len, int64_t kv_len,
                                       int64_t head_dim, const void *q, const void *k, const void *v,

@@ -1632,9 +1632,9 @@ void op_fused_attention(OpContext &c) {
             // run ends; the session's workspace is overwritten by the products in between).
             const int mask_value = c.node.inputs.size() > 2 ? c.node.inputs[2] : -1;
             const size_t shared_bytes =
-                mask_value >= 0 && !c.session.bf16_pieces   // (the launch that also stores pieces makes its own map)
-                    ? rmlk_hip_attention_map_size(RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, &ms)
-                    : 0;
+                mask_value >= 0 ? rmlk_hip_attention_map_size(RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, &ms) : 0;
+            // (the result's pieces for the output projection behind it, stored by the same launch)
+            Tensor pieces = seq_major ? room_for_pieces(c, bsz * seq, heads * dim, "reader_is_product") : Tensor();
             if (shared_bytes) {
                 Session::AttentionMap &am = c.session.attention_map;
                 const int64_t sizes[6] = {bsz, grp, rep_k, seq, len, dim};
@@ -1656,20 +1656,30 @@ void op_fused_attention(OpContext &c) {
                                                 am.map.data(), shared_bytes);
                     if (st) am.map.reset();
                 }
-                if (!st && took_fast_path(rmlk_hip_attention_mapped(
-                                              c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, q.data(), k.data(),
-                                              v.data(), mask.data(), &ms,
-                                              static_cast<int32_t>(c.attr_int("scale_is_mul", 0)), attr_float(c, "scale"),
-                                              seq_major ? 1 : 0, am.map.data(), shared_bytes, y.data()),
-                                          "rmlk.Attention"))
+                if (!st && pieces.defined()) {
+                    if (took_fast_path(rmlk_hip_attention_mapped_pieces(
+                                           c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, q.data(), k.data(),
+                                           v.data(), mask.data(), &ms,
+                                           static_cast<int32_t>(c.attr_int("scale_is_mul", 0)), attr_float(c, "scale"),
+                                           am.map.data(), shared_bytes, y.data(), pieces.data()),
+                                       "rmlk.Attention")) {
+                        y.pieces = std::make_shared<const Tensor>(std::move(pieces));
+                        return;
+                    }
+                } else if (!st && took_fast_path(rmlk_hip_attention_mapped(
+                                                     c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, q.data(),
+                                                     k.data(), v.data(), mask.data(), &ms,
+                                                     static_cast<int32_t>(c.attr_int("scale_is_mul", 0)),
+                                                     attr_float(c, "scale"), seq_major ? 1 : 0, am.map.data(),
+                                                     shared_bytes, y.data()),
+                                                 "rmlk.Attention")) {
                     return;
+                }
             }
             // room for the map of (query tile, key chunk) pairs the mask leaves visible, when it pays
             const size_t map_bytes = rmlk_hip_attention_workspace_size(RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim, &ms);
             void *map = map_bytes ? c.scratch(map_bytes) : nullptr;
-            // (the result's pieces for the output projection behind it, stored by the same launch)
-            if (Tensor pieces = seq_major ? room_for_pieces(c, bsz * seq, heads * dim, "reader_is_product") : Tensor();
-                pieces.defined()) {
+            if (pieces.defined()) {
                 if (took_fast_path(rmlk_hip_attention_ws_pieces(c.stream, RMLK_FLOAT, bsz, grp, rep_k, seq, len, dim,
                                                                 q.data(), k.data(), v.data(), mask.data(), &ms,
                                                                 static_cast<int32_t>(c.attr_int("scale_is_mul", 0)),

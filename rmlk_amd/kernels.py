@@ -303,8 +303,16 @@ def attention_map(mask, batch: int, kv_heads: int, rep: int, q_len: int, kv_len:
 
 def attention_mapped(q, k, v, mask, out, tile_map, batch: int, kv_heads: int, rep: int, q_len: int, kv_len: int,
                      head_dim: int, mask_stride, scale: float, scale_is_mul: bool = False,
-                     out_seq_major: bool = False) -> None:
+                     out_seq_major: bool = False, out_pieces=None) -> None:
     """`attention_skipping` over a map that `attention_map` made for this mask and these sizes."""
+    if out_pieces is not None:
+        assert out_seq_major
+        check(lib().rmlk_hip_attention_mapped_pieces(_stream(), dtype_of(q), batch, kv_heads, rep, q_len, kv_len,
+                                                     head_dim, _ptr(q), _ptr(k), _ptr(v), _ptr(mask),
+                                                     Dims.of(mask_stride), int(scale_is_mul), float(scale),
+                                                     _ptr(tile_map), tile_map.numel(), _ptr(out), _ptr(out_pieces)),
+              "rmlk_hip_attention_mapped_pieces")
+        return
     check(lib().rmlk_hip_attention_mapped(_stream(), dtype_of(q), batch, kv_heads, rep, q_len, kv_len, head_dim,
                                           _ptr(q), _ptr(k), _ptr(v), _ptr(mask), Dims.of(mask_stride),
                                           int(scale_is_mul), float(scale), int(out_seq_major), _ptr(tile_map),

@@ -272,6 +272,16 @@ def test_attention_that_stores_its_result_as_pieces(device, b, g, rep, s, l):
     assert_exact(to_np(got), to_np(plain))
     want = kk.bf16x3_split(plain.reshape(rows, cols)).reshape(3, m_pad, cols)[:, :rows]
     assert torch.equal(pieces.reshape(3, m_pad, cols)[:, :rows], want)
+    # the same over a map of the mask made beforehand (rmlk_hip_attention_mapped_pieces), twice
+    tile_map = kk.attention_map(m, b, g, rep, s, l, d, ms)
+    assert tile_map is not None
+    for _ in range(2):
+        again = torch.full((b, s, h, d), 9.0, device=device)
+        pieces2 = torch.zeros(3 * m_pad * cols, dtype=torch.int16, device=device)
+        kk.attention_mapped(q, k, v, m, again, tile_map, b, g, rep, s, l, d, ms, 8.0, False, out_seq_major=True,
+                            out_pieces=pieces2)
+        assert_exact(to_np(again), to_np(plain))
+        assert torch.equal(pieces2.reshape(3, m_pad, cols)[:, :rows], want)
 
 
 def test_infinities_and_nans_arrive_as_from_an_fp32_product(device):
