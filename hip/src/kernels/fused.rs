@@ -715,6 +715,50 @@ pub unsafe fn attention_mapped(
     )
 }
 
+/// `attention_mapped` with the `[batch, q_len, heads, head_dim]` result also stored as the three
+/// bfloat16 pieces `bf16x3_split` would make of it (`out_pieces`).
+pub unsafe fn attention_mapped_with_pieces(
+    stream: &HipStream,
+    shape: &AttentionShape,
+    q: *const c_void,
+    k: *const c_void,
+    v: *const c_void,
+    mask: *const c_void,
+    mask_stride: &[usize; 4],
+    scale_is_mul: bool,
+    scale: f32,
+    map: *const c_void,
+    map_bytes: usize,
+    out: *mut c_void,
+    out_pieces: *mut c_void,
+) -> Result<()> {
+    let ms = dims(mask_stride)?;
+    check(
+        ffi::rmlk_hip_attention_mapped_pieces(
+            stream.raw(),
+            ffi::RMLK_FLOAT,
+            shape.batch as i64,
+            shape.kv_heads as i64,
+            shape.rep as i64,
+            shape.q_len as i64,
+            shape.kv_len as i64,
+            shape.head_dim as i64,
+            q,
+            k,
+            v,
+            mask,
+            &ms,
+            scale_is_mul as i32,
+            scale,
+            map,
+            map_bytes,
+            out,
+            out_pieces,
+        ),
+        "attention_mapped_with_pieces",
+    )
+}
+
 /// `attention` with a `[batch, q_len, heads, head_dim]` result that is also stored as the three
 /// bfloat16 pieces `bf16x3_split` would make of it (`out_pieces`), for an output projection over them.
 pub unsafe fn attention_with_pieces(
