@@ -27,7 +27,23 @@
 
 #include "common.hpp"
 
+// This file is compiled twice, so that the two halves of its many tiled-GEMM instantiations build
+// side by side: as it stands (everything but the tiled products over 16-bit weights), and included
+// by matmul_stored16.hip with RMLK_MATMUL_PART 2 (only those, behind the two functions below).
+#ifndef RMLK_MATMUL_PART
+#define RMLK_MATMUL_PART 1
+#endif
+
 namespace rmlk {
+// the tiled products over weights stored as 16-bit values (`seg`: a Segments of this file, or null)
+int32_t stored16_gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k, const float *pa,
+                            int64_t lda, int64_t stride_a, int32_t b_dtype, const void *pb, int64_t ldb,
+                            int64_t stride_b, int32_t trans_b, float *pc, int64_t ldc, int64_t stride_c,
+                            void *workspace, size_t workspace_bytes, const void *seg, int32_t *partial_splits);
+int32_t stored16_gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float *pa, int64_t lda,
+                             int32_t b_dtype, const void *pb, int64_t ldb, int32_t trans_b, int64_t gate_offset,
+                             int64_t up_offset, float *pc, int64_t ldc);
+
 namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -86,6 +102,20 @@ int32_t with_storage(int32_t w_dtype, F &&f) {
         case RMLK_FLOAT: return f(StoredF32{});
         case RMLK_FLOAT16: return f(StoredF16{});
         case RMLK_BFLOAT16: return f(StoredBF16{});
+        default: return RMLK_ERR_UNSUPPORTED;
+    }
+}
+
+// The same for the tiled MFMA kernels: each compilation of this file instantiates its share.
+template <typename F>
+int32_t with_storage_tiled(int32_t w_dtype, F &&f) {
+    switch (w_dtype) {
+#if RMLK_MATMUL_PART == 1
+        case RMLK_FLOAT: return f(StoredF32{});
+#else
+        case RMLK_FLOAT16: return f(StoredF16{});
+        case RMLK_BFLOAT16: return f(StoredBF16{});
+#endif
         default: return RMLK_ERR_UNSUPPORTED;
     }
 }
@@ -1735,6 +1765,11 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
                    int32_t *partial_splits = nullptr) {
     const bool b16 = b_dtype != RMLK_FLOAT;
     if (b16 && !trans_b) return RMLK_ERR_UNSUPPORTED;
+#if RMLK_MATMUL_PART == 1
+    if (b16)
+        return stored16_gemm_tiled(s, batch, m, n, k, pa, lda, stride_a, b_dtype, pb, ldb, stride_b, trans_b, pc, ldc,
+                                   stride_c, workspace, workspace_bytes, seg, partial_splits);
+#endif
     // (rows of 16-bit values: whole 128-bit units)
     const int64_t b_unit = b16 ? 8 : 4;
     const bool aligned = lda % 4 == 0 && ldb % b_unit == 0 && stride_a % 4 == 0 && stride_b % b_unit == 0 &&
@@ -1821,7 +1856,7 @@ int32_t gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k
         if (t.bm == 128) return RMLK_LAUNCH_TB(128, 128, 64, 64, TB_, WS_);
         return RMLK_LAUNCH_TB(64, 64, 32, 32, TB_, WS_);
     };
-    int32_t st = with_storage(b_dtype, [&](auto ws) -> int32_t {
+    int32_t st = with_storage_tiled(b_dtype, [&](auto ws) -> int32_t {
         if constexpr (kStored16<decltype(ws)>) return launch_layout(std::true_type{}, ws);
         else return trans_b ? launch_layout(std::true_type{}, ws) : launch_layout(std::false_type{}, ws);
     });
@@ -1863,6 +1898,10 @@ int32_t gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float 
                     int64_t up_offset, float *pc, int64_t ldc) {
     const bool b16 = b_dtype != RMLK_FLOAT;
     if (b16 && !trans_b) return RMLK_ERR_UNSUPPORTED;
+#if RMLK_MATMUL_PART == 1
+    if (b16)
+        return stored16_gemm_swiglu(s, m, n, k, pa, lda, b_dtype, pb, ldb, trans_b, gate_offset, up_offset, pc, ldc);
+#endif
     const bool aligned = lda % 4 == 0 && ldb % (b16 ? 8 : 4) == 0 && gate_offset % 4 == 0 && up_offset % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
                          reinterpret_cast<uintptr_t>(pb) % 16 == 0;
@@ -1892,19 +1931,39 @@ int32_t gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float 
         // (a lane's byte offset into B covers a row number of the whole matrix here)
         const int64_t last_row = (gate_offset > up_offset ? gate_offset : up_offset) + n;
         if (last_row * ldb >= (1ll << 30)) return RMLK_ERR_UNSUPPORTED;
-        return with_storage(b_dtype, [&](auto ws) -> int32_t {
+        return with_storage_tiled(b_dtype, [&](auto ws) -> int32_t {
             using WS = decltype(ws);
             if (m % 128 == 0) return launch_direct<128, 128, 64, 64, true, 2, true, false, WS>(s, g, 1, 1);
             return launch_direct<128, 128, 64, 64, true, 2, true, true, WS>(s, g, 1, 1);
         });
     }
+#if RMLK_MATMUL_PART == 1
     if (m % 128 == 0) return launch_direct<128, 128, 64, 64, false, 2, true, false>(s, g, 1, 1);
     return launch_direct<128, 128, 64, 64, false, 2, true, true>(s, g, 1, 1);
+#else
+    return RMLK_ERR_UNSUPPORTED;
+#endif
 }
 
 }  // namespace
+
+#if RMLK_MATMUL_PART == 2
+int32_t stored16_gemm_tiled(hipStream_t s, int64_t batch, int64_t m, int64_t n, int64_t k, const float *pa,
+                            int64_t lda, int64_t stride_a, int32_t b_dtype, const void *pb, int64_t ldb,
+                            int64_t stride_b, int32_t trans_b, float *pc, int64_t ldc, int64_t stride_c,
+                            void *workspace, size_t workspace_bytes, const void *seg, int32_t *partial_splits) {
+    return gemm_tiled(s, batch, m, n, k, pa, lda, stride_a, b_dtype, pb, ldb, stride_b, trans_b, pc, ldc, stride_c,
+                      workspace, workspace_bytes, static_cast<const Segments *>(seg), partial_splits);
+}
+int32_t stored16_gemm_swiglu(hipStream_t s, int64_t m, int64_t n, int64_t k, const float *pa, int64_t lda,
+                             int32_t b_dtype, const void *pb, int64_t ldb, int32_t trans_b, int64_t gate_offset,
+                             int64_t up_offset, float *pc, int64_t ldc) {
+    return gemm_swiglu(s, m, n, k, pa, lda, b_dtype, pb, ldb, trans_b, gate_offset, up_offset, pc, ldc);
+}
+#endif
 }  // namespace rmlk
 
+#if RMLK_MATMUL_PART == 1
 using namespace rmlk;
 
 extern "C" size_t rmlk_hip_matmul_workspace_size(int32_t dtype, int64_t batch, int64_t m,
@@ -2626,3 +2685,4 @@ extern "C" int32_t rmlk_hip_matmul_noalloc(rmlk_stream_t stream, int32_t dtype, 
     return rmlk_hip_matmul(stream, dtype, batch, m, n, k, a, lda, stride_a, trans_a, b, ldb, stride_b,
                            trans_b, c, ldc, stride_c, ws, need);
 }
+#endif   // RMLK_MATMUL_PART == 1
