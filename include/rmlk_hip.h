@@ -722,9 +722,9 @@ int32_t rmlk_hip_free(void *ptr);
 int32_t rmlk_hip_memcpy_htod(rmlk_stream_t stream, void *dst, const void *src, size_t bytes);
 int32_t rmlk_hip_memcpy_dtoh(rmlk_stream_t stream, void *dst, const void *src, size_t bytes);
 int32_t rmlk_hip_memcpy_dtod(rmlk_stream_t stream, void *dst, const void *src, size_t bytes);
-/* n_copies device-to-device copies (dsts, srcs and bytes are HOST arrays) in one launch for up to 8
- * copies with 16-byte aligned ends and lengths; one rmlk_hip_memcpy_dtod each otherwise. The two
- * cache copies a decoder layer needs when its cache inputs may not be overwritten are one launch. */
+/* n_copies device-to-device copies (dsts, srcs and bytes are HOST arrays), 32 per launch when all
+ * of them have 16-byte aligned ends and lengths; one rmlk_hip_memcpy_dtod each otherwise. The cache
+ * copies the layers of a decoder need when their cache inputs may not be overwritten are one launch. */
 int32_t rmlk_hip_memcpy_dtod_many(rmlk_stream_t stream, int32_t n_copies, void *const *dsts,
                                   const void *const *srcs, const size_t *bytes);
 int32_t rmlk_hip_memset(rmlk_stream_t stream, void *dst, int32_t byte, size_t bytes);

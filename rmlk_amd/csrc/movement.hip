@@ -91,7 +91,7 @@ __global__ __launch_bounds__(kBlock) void copy_flat_kernel(const U *__restrict__
 }
 
 // several dense flat copies in one launch: blockIdx.y picks the copy
-constexpr int kMaxCopies = 8;
+constexpr int kMaxCopies = 32;
 struct CopyMany {
     const U128 *in[kMaxCopies];
     U128 *out[kMaxCopies];
@@ -642,39 +642,44 @@ extern "C" int32_t rmlk_hip_memcpy_dtod(rmlk_stream_t stream, void *dst, const v
     return RMLK_OK;
 }
 
-// Up to 8 device-to-device copies as ONE launch (16-byte aligned ends and lengths, below 16 GiB
-// each); anything else one call of rmlk_hip_memcpy_dtod per copy.
+// Up to 32 device-to-device copies as ONE launch (16-byte aligned ends and lengths, below 16 GiB
+// each; more of them 32 per launch); anything else one call of rmlk_hip_memcpy_dtod per copy.
 extern "C" int32_t rmlk_hip_memcpy_dtod_many(rmlk_stream_t stream, int32_t n_copies, void *const *dsts,
                                              const void *const *srcs, const size_t *bytes) {
     if (n_copies < 0) return RMLK_ERR_INVALID_ARGUMENT;
     if (n_copies == 0) return RMLK_OK;
     if (!dsts || !srcs || !bytes) return RMLK_ERR_NULL_POINTER;
-    bool together = n_copies <= kMaxCopies;
-    size_t longest = 0;
+    bool together = n_copies > 1;
     for (int i = 0; i < n_copies; ++i) {
         if (bytes[i] && (!dsts[i] || !srcs[i])) return RMLK_ERR_NULL_POINTER;
         if (bytes[i] % 16 || reinterpret_cast<uintptr_t>(dsts[i]) % 16 || reinterpret_cast<uintptr_t>(srcs[i]) % 16 ||
             bytes[i] / 16 >= (static_cast<size_t>(1) << 30))
             together = false;
-        if (bytes[i] > longest) longest = bytes[i];
     }
-    if (!together || n_copies == 1) {
+    if (!together) {
         for (int i = 0; i < n_copies; ++i) {
             const int32_t st = rmlk_hip_memcpy_dtod(stream, dsts[i], srcs[i], bytes[i]);
             if (st) return st;
         }
         return RMLK_OK;
     }
-    if (longest == 0) return RMLK_OK;
-    CopyMany a{};
-    for (int i = 0; i < n_copies; ++i) {
-        a.in[i] = static_cast<const U128 *>(srcs[i]);
-        a.out[i] = static_cast<U128 *>(dsts[i]);
-        a.n[i] = static_cast<uint32_t>(bytes[i] / 16);
+    for (int first = 0; first < n_copies; first += kMaxCopies) {
+        const int count = n_copies - first < kMaxCopies ? n_copies - first : kMaxCopies;
+        CopyMany a{};
+        size_t longest = 0;
+        for (int i = 0; i < count; ++i) {
+            a.in[i] = static_cast<const U128 *>(srcs[first + i]);
+            a.out[i] = static_cast<U128 *>(dsts[first + i]);
+            a.n[i] = static_cast<uint32_t>(bytes[first + i] / 16);
+            if (bytes[first + i] > longest) longest = bytes[first + i];
+        }
+        if (longest == 0) continue;
+        dim3 grid(chunk_grid(static_cast<uint32_t>(longest / 16), kChunk), static_cast<unsigned>(count), 1);
+        copy_many_kernel<<<grid, kBlock, 0, as_stream(stream)>>>(a);
+        const int32_t st = launch_status();
+        if (st) return st;
     }
-    dim3 grid(chunk_grid(static_cast<uint32_t>(longest / 16), kChunk), static_cast<unsigned>(n_copies), 1);
-    copy_many_kernel<<<grid, kBlock, 0, as_stream(stream)>>>(a);
-    return launch_status();
+    return RMLK_OK;
 }
 
 extern "C" int32_t rmlk_hip_transpose(rmlk_stream_t stream, int32_t dtype,

@@ -304,6 +304,13 @@ struct Session {
         rmlk_dims strides{};
         Tensor map;
     } attention_map;
+    // A ScatterND destination that has to be a copy of a graph input (a cache input the caller did
+    // not donate) depends on nothing the run computes: all such copies go out as ONE launch in front
+    // of the first node, and the nodes find them here. `scatter_inputs` lists (node index, value id)
+    // of every place where a graph input is the data of a ScatterND; found when the session is built.
+    std::vector<std::pair<int, int>> scatter_inputs;
+    std::multimap<std::pair<int, int>, Tensor> early_copies;
+    void copy_scatter_inputs_early();
     bool capturing = false;
     bool profiling = false;
     bool fuse = true;                // form fused nodes while building

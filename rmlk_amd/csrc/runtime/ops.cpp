@@ -603,6 +603,15 @@ Tensor &scatter_destination(OpContext &c, int data_index, int out_index, bool *c
         if (static_cast<int>(i) != data_index && c.node.inputs[i] == vid) read_elsewhere = true;
     if (last_reader && sole_owner && may_overwrite && !read_elsewhere && !v.is_output && !v.is_initializer)
         return c.view_output(out_index, data, data.shape);
+    // a copy of a graph input made in front of the first node of the run
+    auto early = c.session.early_copies.find(std::make_pair(c.node_index, vid));
+    if (early != c.session.early_copies.end() && early->second.dtype == data.dtype &&
+        early->second.shape == data.shape) {
+        if (out_index >= static_cast<int>(c.out.size()) || !c.out[out_index]) fail_op(c.node.op + ": missing output");
+        *c.out[out_index] = std::move(early->second);
+        c.session.early_copies.erase(early);
+        return *c.out[out_index];
+    }
     Tensor &y = c.alloc_output(out_index, data.dtype, data.shape);
     if (copy_left_to_caller) {
         *copy_left_to_caller = true;     // the caller's kernel copies while it scatters

@@ -440,6 +440,60 @@ void Session::build(const rmlk_graph &graph, int dev) {
     for (size_t n = 0; n < g->nodes.size(); ++n)
         for (int v : g->nodes[n].inputs)
             if (v >= 0) last_use[v] = static_cast<int>(n);
+    // where a graph input is the data of a ScatterND (alone, or as a stream of a row-stream node)
+    scatter_inputs.clear();
+    for (size_t n = 0; n < g->nodes.size(); ++n) {
+        const Node &node = g->nodes[n];
+        auto note = [&](size_t i) {
+            if (i >= node.inputs.size() || node.inputs[i] < 0) return;
+            const Value &val = g->values[node.inputs[i]];
+            if (val.is_input && !val.is_initializer) scatter_inputs.emplace_back(static_cast<int>(n), node.inputs[i]);
+        };
+        if (node.op == "ScatterND") {
+            note(0);
+        } else if (node.op == "rmlk.HeadRows") {
+            auto kinds = node.attrs.find("kinds");
+            if (kinds == node.attrs.end()) continue;
+            size_t at = 0;
+            for (int64_t kind : kinds->second.ints) {   // (input lists by kind: op_fused_head_rows)
+                if (kind == 1) note(at + 3);
+                else if (kind == 2) note(at + 1);
+                at += kind == 1 ? 5 : 3;
+            }
+        }
+    }
+}
+
+// The copies of graph inputs that ScatterND nodes of this run will need as their destinations, all
+// in one launch (the reference copies data -> output in front of every scatter,
+// backend/scatter_nd.rs:128-129). Only inputs the caller did not donate: a donated one is
+// updated in place, or copied by its node when something else still reads it.
+void Session::copy_scatter_inputs_early() {
+    early_copies.clear();
+    if (!fuse || scatter_inputs.empty()) return;
+    std::vector<void *> dsts;
+    std::vector<const void *> srcs;
+    std::vector<size_t> sizes;
+    for (const std::pair<int, int> &site : scatter_inputs) {
+        const Tensor &data = values[site.second];
+        if (!data.defined() || !data.buf || data.buf->donated || data.nbytes() == 0) continue;
+        Tensor y;
+        y.dtype = data.dtype;
+        y.shape = data.shape;
+        auto b = std::make_shared<Buffer>();
+        b->bytes = data.nbytes();
+        b->pool = &pool;
+        b->ptr = pool.alloc(b->bytes);
+        y.buf = b;
+        dsts.push_back(y.data());
+        srcs.push_back(data.data());
+        sizes.push_back(data.nbytes());
+        early_copies.emplace(site, std::move(y));
+    }
+    if (!dsts.empty())
+        check_status(rmlk_hip_memcpy_dtod_many(stream, static_cast<int32_t>(dsts.size()), dsts.data(), srcs.data(),
+                                               sizes.data()),
+                     "ScatterND copies");
 }
 
 void Session::run_nodes() {
@@ -465,6 +519,7 @@ void Session::run_nodes() {
             stop();
         }
     } collecting{stream, pool};
+    copy_scatter_inputs_early();
     if (fuse && !profiling) {
         check_status(rmlk_hip_batch_begin(stream), "collected launches");
         collecting.on = true;
@@ -575,6 +630,7 @@ void Session::run_nodes() {
         check_status(rmlk_hip_batch_end(stream), "collected launches");
     }
     scratch_bufs.clear();
+    early_copies.clear();
     attention_map.map.reset();
     attention_map.mask_value = -1;
 }

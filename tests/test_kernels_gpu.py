@@ -81,6 +81,22 @@ def test_arith_broadcast(device, name, dtype, shapes):
     assert_exact(got, expected)
 
 
+@pytest.mark.parametrize("name,shapes", [
+    ("add", ((1, 32, 1024, 512), (1, 1, 1024, 512))),     # a mask added to every head
+    ("sub", ((1, 1, 1024, 512), (2, 16, 1024, 512))),     # the broadcast operand first
+    ("greater", ((16, 1024, 1024), (1, 1024, 1024))),
+    ("mul", ((48, 1024, 512), (1, 1024, 512)))])
+def test_large_operand_against_one_repeated_along_an_outer_dim(device, name, shapes):
+    """Large dense operands against one that repeats along an outer dim (a lane takes several
+    positions along that dim and fetches the repeated operand once for all of them)."""
+    rng = np.random.default_rng(zlib.crc32(repr((name, shapes)).encode()))
+    a = rng.standard_normal(shapes[0], dtype=np.float32)
+    b = rng.standard_normal(shapes[1], dtype=np.float32)
+    if name == "greater":
+        b = np.broadcast_to(a[3:4], shapes[1]).copy()   # (equal in places)
+    assert_exact(run_binary(device, name, a, b), getattr(_ops(), name)(a, b))
+
+
 def test_int_division_edges(device):
     a = np.array([7, -7, 7, -7, 0, 5, np.iinfo(np.int32).min], dtype=np.int32)
     b = np.array([2, 2, -2, -2, 3, 0, -1], dtype=np.int32)
@@ -484,10 +500,11 @@ def test_concat(device, case, dtype):
     assert_exact(to_np(out), expected)
 
 
-@pytest.mark.parametrize("sizes", [[1310720, 1310720], [16, 4096, 48, 1 << 20], [64] * 9, [20, 64]])
+@pytest.mark.parametrize("sizes", [[1310720, 1310720], [16, 4096, 48, 1 << 20], [64] * 9, [20, 64],
+                                   [1310720] * 32, [256 * (i + 1) for i in range(70)]])
 def test_several_device_copies_in_one_call(device, sizes):
     """rmlk_hip_memcpy_dtod_many: every destination gets its source, nothing past the ends is touched
-    (more than 8 copies, or lengths that are no multiple of 16, go one by one)."""
+    (32 copies per launch; lengths that are no multiple of 16 go one by one)."""
     import torch
     k = _k()
     rng = np.random.default_rng(len(sizes) + sizes[0])
