@@ -515,7 +515,7 @@ def gemv_kmajor_head_rows(x, wt, k: int, streams, first_cols, gamma=None, eps: f
 
 
 def memcpy_dtod_many(dsts, srcs) -> None:
-    """dsts[i] <- srcs[i] (dense device tensors of equal byte size each), one launch for up to 8 copies."""
+    """dsts[i] <- srcs[i] (dense device tensors of equal byte size each), 32 copies per launch."""
     n = len(dsts)
     d = (ctypes.c_void_p * n)(*[_ptr(t) for t in dsts])
     s_ = (ctypes.c_void_p * n)(*[_ptr(t) for t in srcs])
