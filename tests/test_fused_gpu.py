@@ -737,6 +737,39 @@ def test_scatter_destinations_copied_in_front_of_the_run(device, fuse):
     sess.close()
 
 
+@pytest.mark.parametrize("fuse", [True, False])
+def test_kernel_error_is_reported_once_and_the_session_goes_on(device, fuse):
+    """An index out of range makes the run (or the replay of the recorded graph) that holds it fail
+    with "kernel failed" (ref: KernelFailed{code}, backend/scatter_nd.rs:198-203); the runs and
+    replays after it, over good indices, succeed: the kernels' error flag is put back when it has
+    been reported, not cleared by every run."""
+    from rmlk_amd import runtime
+    g = _builder()
+    g.input("table", np.float32, [40, 4])
+    g.input("rows", np.int64, [3])
+    g.op("Gather", ["table", "rows"], ["picked"]).attr("axis", 0)
+    g.op("Neg", ["picked"], ["y"])
+    g.output("y")
+    sess = runtime.Builder.from_graph(g.build()).build(fuse=fuse)
+    table = np.arange(160, dtype=np.float32).reshape(40, 4)
+    good, bad = np.array([39, 0, 3], np.int64), np.array([1, 40, 2], np.int64)
+    assert_exact(sess.run({"table": table, "rows": good})["y"], -table[good])
+    with pytest.raises(Exception, match="kernel failed"):
+        sess.run({"table": table, "rows": bad})
+    assert_exact(sess.run({"table": table, "rows": good})["y"], -table[good])
+    sess.capture()
+    for rows in (good, bad, good[::-1].copy(), bad, good):
+        sess.set_input("rows", rows)
+        if rows is bad:
+            with pytest.raises(Exception, match="kernel failed"):
+                sess.replay()
+        else:
+            sess.replay()
+            sess.sync()
+            assert_exact(sess.output("y"), -table[rows])
+    sess.close()
+
+
 @pytest.mark.parametrize("s,early_reader", [(5, False), (1, False), (5, True)])
 def test_rows_behind_the_projections_become_one_node(device, s, early_reader):
     """Rotary(q), Rotary(k) -> ScatterND and Transpose(v) -> ScatterND merge into one rmlk.HeadRows
