@@ -141,8 +141,8 @@ def run_llama(args):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        inst.replay()
-    inst.sync()
+        inst.replay_enqueue()            # the passes queue up behind one another: no host round trip between them
+    inst.check()                         # waits for all of them; a kernel failure of any pass is reported here
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
     ms_per_step = prefill_s / args.steps * 1e3
@@ -267,8 +267,8 @@ def run_llama(args):
         inst.sync()
         t0 = time.perf_counter()
         for _ in range(20):
-            inst.replay()
-        inst.sync()
+            inst.replay_enqueue()
+        inst.check()
         decode_dev_ms = (time.perf_counter() - t0) / 20 * 1e3
         weight_bytes = decode_weight_bytes(cfg, stored)
         log(f"[bench] decode: {decode_ms:.3f} ms/token end to end, {decode_dev_ms:.3f} ms/token "
@@ -834,8 +834,8 @@ def run_graph_suite(args):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.steps):
-            inst.replay()
-        inst.sync()
+            inst.replay_enqueue()
+        inst.check()
         ms = (time.perf_counter() - t0) / args.steps * 1e3
         marker.bitwise_not_()              # end of the timed block; what follows up to the next mark is not timed
         torch.cuda.synchronize()

@@ -154,6 +154,14 @@ int32_t rmlk_session_read_output(rmlk_session *s, const char *name, void *host_d
  * must not depend on input VALUES between replays. */
 int32_t rmlk_session_capture(rmlk_session *s);
 int32_t rmlk_session_replay(rmlk_session *s);
+/* rmlk_session_replay in two halves, for a caller that keeps the GPU fed: _replay_enqueue launches
+ * the recorded graph and returns without waiting (several may be enqueued back to back; each reads
+ * the inputs as they are when it executes), _check waits for the session's stream and reports a
+ * kernel failure (an index out of range) of any run or replay since the last report - the
+ * kernels' error flag stays set until it has been reported. rmlk_session_replay is one of each.
+ * No counterpart in the reference, whose ModelInstance::run (instance.rs:89-119) is synchronous. */
+int32_t rmlk_session_replay_enqueue(rmlk_session *s);
+int32_t rmlk_session_check(rmlk_session *s);
 
 int32_t rmlk_session_sync(rmlk_session *s);
 /* hipStream_t the session enqueues on */

@@ -245,6 +245,8 @@ SIGNATURES = {
     "rmlk_session_read_output": (c_int32, [c_void_p, c_char_p, c_void_p, c_size_t]),
     "rmlk_session_capture": (c_int32, [c_void_p]),
     "rmlk_session_replay": (c_int32, [c_void_p]),
+    "rmlk_session_replay_enqueue": (c_int32, [c_void_p]),
+    "rmlk_session_check": (c_int32, [c_void_p]),
     "rmlk_session_sync": (c_int32, [c_void_p]),
     "rmlk_session_stream": (c_void_p, [c_void_p]),
     "rmlk_session_set_profiling": (c_int32, [c_void_p, c_int32]),

@@ -435,6 +435,20 @@ int32_t rmlk_session_replay(rmlk_session *s) {
     });
 }
 
+int32_t rmlk_session_replay_enqueue(rmlk_session *s) {
+    return guarded([&] {
+        if (!s) throw RtError(RMLK_ERR_NULL_POINTER, "null session");
+        s->impl.replay_enqueue();
+    });
+}
+
+int32_t rmlk_session_check(rmlk_session *s) {
+    return guarded([&] {
+        if (!s) throw RtError(RMLK_ERR_NULL_POINTER, "null session");
+        s->impl.check_error_flag();
+    });
+}
+
 int32_t rmlk_session_sync(rmlk_session *s) {
     return guarded([&] {
         if (!s) throw RtError(RMLK_ERR_NULL_POINTER, "null session");

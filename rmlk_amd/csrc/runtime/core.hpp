@@ -336,6 +336,7 @@ struct Session {
     void run();
     void capture();
     void replay();
+    void replay_enqueue();           // the recorded graph launched, nothing awaited
     void check_error_flag();
 };
 

@@ -366,6 +366,7 @@ void Session::build(const rmlk_graph &graph, int dev) {
     check_hip(hipSetDevice(dev), "hipSetDevice");
     check_hip(hipStreamCreate(&stream), "hipStreamCreate");  // default priority
     check_hip(hipMalloc(reinterpret_cast<void **>(&err_flag), sizeof(int32_t)), "hipMalloc");
+    check_hip(hipMemset(err_flag, 0, sizeof(int32_t)), "hipMemset");
     check_hip(hipHostMalloc(reinterpret_cast<void **>(&err_host), sizeof(int32_t)), "hipHostMalloc");
     *err_host = 0;
     check_hip(hipMalloc(reinterpret_cast<void **>(&block_counters), kBlockCounters * sizeof(int32_t)), "hipMalloc");
@@ -635,13 +636,24 @@ void Session::run_nodes() {
     attention_map.mask_value = -1;
 }
 
+// The error flag of the kernels is zero when the session is built and is put back to zero when it
+// has been reported (or when a run has failed for another reason). A run that succeeds leaves it
+// untouched, so it stays set across the replays that are enqueued without a wait in between
+// (replay_enqueue) until check_error_flag reports it, and no run spends a launch on clearing it.
+static void clear_flag(Session &s) {
+    int32_t zero = 0;
+    (void)rmlk_hip_write_small(s.stream, s.err_flag, &zero, sizeof(zero));
+}
+
 void Session::check_error_flag() {
+    check_hip(hipSetDevice(device), "hipSetDevice");
     check_hip(hipMemcpyAsync(err_host, err_flag, sizeof(int32_t), hipMemcpyDeviceToHost, stream),
               "hipMemcpyAsync D2H (error flag)");
     check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
     if (*err_host != 0) {
         int32_t code = *err_host;
         *err_host = 0;
+        clear_flag(*this);
         throw RtError(RMLK_ERR_KERNEL,
                       "kernel failed: index out of range (code " + std::to_string(code) + ")");
     }
@@ -656,11 +668,6 @@ static void rezero_block_counters(Session &s) {
         (void)rmlk_hip_memset(s.stream, s.block_counters, 0, Session::kBlockCounters * sizeof(int32_t));
 }
 
-static void clear_flag(Session &s) {
-    int32_t zero = 0;
-    check_status(rmlk_hip_write_small(s.stream, s.err_flag, &zero, sizeof(zero)), "clear flag");
-}
-
 void Session::run() {
     check_hip(hipSetDevice(device), "hipSetDevice");
     plan.reset();  // an eager run with (possibly) other shapes invalidates a recorded graph
@@ -669,11 +676,11 @@ void Session::run() {
         const Value &val = graph_copy.values[v];
         if (!val.is_initializer && !val.is_input) values[v].reset();
     }
-    clear_flag(*this);
     try {
         run_nodes();
     } catch (...) {
         rezero_block_counters(*this);
+        clear_flag(*this);
         throw;
     }
     check_error_flag();
@@ -713,7 +720,6 @@ void Session::capture() {
         check_hip(e, "hipStreamBeginCapture");
     }
     try {
-        clear_flag(*this);
         run_nodes();
     } catch (...) {
         hipGraph_t dead = nullptr;
@@ -736,10 +742,14 @@ void Session::capture() {
     plan = std::move(p);
 }
 
-void Session::replay() {
+void Session::replay_enqueue() {
     if (!plan) throw RtError(RMLK_ERR_OP, "no recorded graph: call rmlk_session_capture first");
     check_hip(hipSetDevice(device), "hipSetDevice");
     check_hip(hipGraphLaunch(plan->exec, stream), "hipGraphLaunch");
+}
+
+void Session::replay() {
+    replay_enqueue();
     check_error_flag();
 }
 

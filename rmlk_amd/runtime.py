@@ -231,6 +231,15 @@ class ModelInstance:
     def replay(self) -> None:
         _check(lib().rmlk_session_replay(self._h), "ModelInstance.replay")
 
+    def replay_enqueue(self) -> None:
+        """Launch the recorded graph without waiting for it (several may be enqueued back to back)."""
+        _check(lib().rmlk_session_replay_enqueue(self._h), "ModelInstance.replay_enqueue")
+
+    def check(self) -> None:
+        """Wait for the session's stream; raises if a kernel of any run or replay since the last
+        report failed (an index out of range)."""
+        _check(lib().rmlk_session_check(self._h), "ModelInstance.check")
+
     def sync(self) -> None:
         _check(lib().rmlk_session_sync(self._h), "ModelInstance.sync")
 

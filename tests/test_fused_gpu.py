@@ -767,6 +767,21 @@ def test_kernel_error_is_reported_once_and_the_session_goes_on(device, fuse):
             sess.replay()
             sess.sync()
             assert_exact(sess.output("y"), -table[rows])
+    # replays enqueued without a wait in between: the failure of the first is still reported when the
+    # caller checks, once; the second ran over good indices and its result stands
+    sess.set_input("rows", bad)
+    sess.replay_enqueue()
+    sess.set_input("rows", good)
+    sess.replay_enqueue()
+    with pytest.raises(Exception, match="kernel failed"):
+        sess.check()
+    sess.check()
+    assert_exact(sess.output("y"), -table[good])
+    for rows in (good[::-1].copy(), good):
+        sess.set_input("rows", rows)
+        sess.replay_enqueue()
+    sess.check()
+    assert_exact(sess.output("y"), -table[good])
     sess.close()
 
 
