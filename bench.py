@@ -317,7 +317,7 @@ def run_llama(args):
                                "KV cache updated by ScatterND, random-init weights N(0,0.02)",
                    "layers": cfg.layers, "hidden": cfg.hidden, "vocab": cfg.vocab,
                    "prompt_tokens": prompt_len, "graph_nodes": len(graph.nodes),
-                   "execution": "recorded HIP graph replay per step"},
+                   "execution": "recorded HIP graph replay per step; the timed replays are enqueued back to back and awaited once"},
         "decode_ms_per_token": None if decode_ms is None else round(decode_ms, 4),
         "decode_device_ms_per_token": None if decode_dev_ms is None else round(decode_dev_ms, 4),
         "decode_weight_gbs": None if decode_dev_ms is None else round(weight_bytes / decode_dev_ms / 1e6, 1),
